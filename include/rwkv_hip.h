@@ -1,0 +1,151 @@
+/*
+ * rwkv_hip.h -- C ABI of librwkv_hip.so: the WKV recurrence family and depthwise_conv1d
+ * for AMD MI355X (gfx950).
+ *
+ * Every entry point replaces one plain-pointer launcher of BlinkDL/RWKV-CUDA (the
+ * `cuda_forward` / `cuda_backward` prototypes that each `*_op.cpp` shim declares) and keeps
+ * that launcher's argument ORDER and meaning.  Differences, the same for all of them:
+ *   - a leading `stream` (a hipStream_t passed as void*; NULL = the null stream); the
+ *     reference launches on the legacy default stream;
+ *   - an `int` status is returned (RWKV_OK or a negative RWKV_ERR_*); the reference only
+ *     asserts.  Nothing is launched when a status other than RWKV_OK is returned;
+ *   - backward passes that need device scratch take it from the caller as a trailing
+ *     (workspace, workspace_bytes) pair whose size the matching *_workspace_bytes()
+ *     function reports.  No entry point allocates or frees device memory, and none
+ *     synchronises: work is enqueued on `stream` and the call returns.
+ *   - T is a run-time argument (the reference bakes -D_T_ into wkv6 / wkv6_state);
+ *     the head size N = C / H must be 64.
+ *
+ * bf16 tensors are passed as uint16_t* (raw bfloat16 bits).  All tensors are dense and
+ * contiguous in the layouts named per function and must be 16-byte aligned.
+ * Pointers are device pointers on the current HIP device.
+ */
+#ifndef RWKV_HIP_H
+#define RWKV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t rwkv_bf16;
+
+enum {
+    RWKV_OK = 0,
+    RWKV_ERR_SHAPE = -1,     /* a dimension is <= 0, C != H*64, T not a multiple of the chunk, ... */
+    RWKV_ERR_NULL = -2,      /* a required pointer is NULL */
+    RWKV_ERR_ALIGN = -3,     /* a pointer is not 16-byte aligned */
+    RWKV_ERR_WORKSPACE = -4, /* workspace missing or smaller than *_workspace_bytes() */
+    RWKV_ERR_LAUNCH = -5     /* the HIP runtime refused a launch (see rwkv_last_hip_error) */
+};
+
+/* Text for a status code; never NULL. */
+const char* rwkv_strerror(int status);
+/* hipError_t value of the last failed launch in this thread (0 if none). */
+int rwkv_last_hip_error(void);
+/* ABI version of this header (bumped when a signature changes). */
+int rwkv_abi_version(void);
+
+/* ---------------------------------------------------------------------------------------
+ * RWKV-4 wkv, fp32.  Replaces cuda_forward / cuda_backward of wkv/cuda/wkv_op.cpp:3-4
+ * (kernels: wkv/cuda/wkv_cuda_v2.cu:4-130).
+ *   w[C]  = -exp(w_raw) (the wrapper's pre-transform, wkv/run.py:95), u[C], k,v,y,gy,gk,gv[B,T,C].
+ *   gw,gu[B,C] are per-batch partials that the kernel ADDS into (caller zero-fills, as
+ *   wkv/run.py:110-111 does); gw already carries the factor w of the w_raw chain rule.
+ * ------------------------------------------------------------------------------------- */
+int rwkv_wkv4_forward(void* stream, int B, int T, int C,
+                      const float* w, const float* u, const float* k, const float* v, float* y);
+int rwkv_wkv4_backward(void* stream, int B, int T, int C,
+                       const float* w, const float* u, const float* k, const float* v, const float* gy,
+                       float* gw, float* gu, float* gk, float* gv);
+
+/* ---------------------------------------------------------------------------------------
+ * depthwise_conv1d ("TimeX"), fp32.  Replaces cuda_forward / cuda_backward of
+ * depthwise_conv1d/cuda/timex_op.cpp:3-4 (kernels: timex_cuda_v3.cu:7-150).
+ *   w[C,T], k,x,gwk,gk[B,C,T];  x[b,c,t] = eps + sum_{u<=t} w[c,T-1-(t-u)] k[b,c,u].
+ *   gw[B,C,T] is per batch (the wrapper sums over B, depthwise_conv1d/run.py:102).
+ *   T must be a multiple of 4 (same as the reference); B is unrestricted.
+ * ------------------------------------------------------------------------------------- */
+int rwkv_timex_forward(void* stream, const float* w, const float* k, float* x, float eps, int B, int C, int T);
+int rwkv_timex_backward(void* stream, const float* w, const float* k, const float* gwk,
+                        float* gw, float* gk, int B, int C, int T);
+
+/* ---------------------------------------------------------------------------------------
+ * RWKV-5 wkv, bf16 I/O.  Replaces cuda_forward / cuda_backward of
+ * wkv5_bf16/cuda/wkv5_op.cpp:5-6 (kernels: wkv5_cuda_v1b.cu:6-191).
+ *   r,k,v,y,gy,gr,gk,gv[B,T,C] bf16; eew = exp(-exp(w_raw)) and ew = -exp(w_raw), fp32 [H,N]
+ *   (wkv5_bf16/run.py:63-64); u[H,N] bf16; gw,gu[B,C] bf16 per-batch partials (fully written).
+ * ------------------------------------------------------------------------------------- */
+int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H,
+                      const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                      const float* eew, const rwkv_bf16* u, rwkv_bf16* y);
+size_t rwkv_wkv5_backward_workspace_bytes(int B, int T, int C, int H);
+int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H,
+                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                       const float* eew, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
+                       rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                       void* workspace, size_t workspace_bytes);
+
+/* ---------------------------------------------------------------------------------------
+ * RWKV-6 wkv, bf16 I/O, per-token decay.  Replaces cuda_forward / cuda_backward of
+ * wkv6/cuda/wkv6_op.cpp:5-6 (kernels: wkv6_cuda_v1.cu:6-223).
+ *   w = ew = -exp(w_raw), fp32 [B,T,C] (wkv6/run.py:147); the kernel applies exp(ew).
+ *   gw[B,T,C] bf16 is the gradient w.r.t. w_raw and is fully written (rows 0 and T-1 are
+ *   exact zeros, which is what the reference leaves in its pre-zeroed buffer); gu[B,C].
+ * ------------------------------------------------------------------------------------- */
+int rwkv_wkv6_forward(void* stream, int B, int T, int C, int H,
+                      const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                      const float* ew, const rwkv_bf16* u, rwkv_bf16* y);
+size_t rwkv_wkv6_backward_workspace_bytes(int B, int T, int C, int H);
+int rwkv_wkv6_backward(void* stream, int B, int T, int C, int H,
+                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                       const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
+                       rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                       void* workspace, size_t workspace_bytes);
+
+/* ---------------------------------------------------------------------------------------
+ * RWKV-6 wkv with initial state.  Replaces cuda_forward / cuda_backward of
+ * wkv6_state/cuda/wkv6state_op.cpp:5-6 (kernels: wkv6state_cuda_v1a.cu:6-308).
+ *   w[B,T,C] is the RAW bf16 decay parameter; the kernel applies exp(-exp(w)).
+ *   s,gs[B,H,N,N] bf16, indexed [value channel][key channel]; every output is fully written.
+ * ------------------------------------------------------------------------------------- */
+int rwkv_wkv6state_forward(void* stream, int B, int T, int C, int H,
+                           const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                           const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, rwkv_bf16* y);
+size_t rwkv_wkv6state_backward_workspace_bytes(int B, int T, int C, int H);
+int rwkv_wkv6state_backward(void* stream, int B, int T, int C, int H,
+                            const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                            const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, const rwkv_bf16* gy,
+                            rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                            rwkv_bf16* gs, void* workspace, size_t workspace_bytes);
+
+/* ---------------------------------------------------------------------------------------
+ * RWKV-7 "clamp-w" with state passing, bf16 I/O, fp32 states.  Replaces cuda_forward /
+ * cuda_backward of rwkv7_fast_fused/cuda/rwkv7_statepassing_clampw.cpp:10,17
+ * (kernels: rwkv7_statepassing_clampw.cu:20-193).
+ *   r,w,k,v,a,b,y,dy,dr,dw,dk,dv,da,db [B,T,H,N] bf16 (w raw; decay = exp(-e^-0.5 * sigmoid(w)));
+ *   s0,sT,dsT,ds0 [B,H,N,N] fp32 indexed [value][key];
+ *   s  [B,H,T/16,N,N] fp32 : state checkpoints written by forward, read by backward;
+ *   sa [B,T,H,N]      fp32 : S_t a_t written by forward, read by backward.
+ *   T must be a multiple of RWKV7_CHUNK_LEN (16), as rwkv7_statepassing_clampw.cu:191 asserts.
+ *   The layout inside `s` is private to this library (forward and backward must both come
+ *   from it).
+ * ------------------------------------------------------------------------------------- */
+#define RWKV7_CHUNK_LEN 16
+int rwkv7_statepassing_forward(void* stream, int B, int T, int H,
+                               const float* s0, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
+                               const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b,
+                               rwkv_bf16* y, float* sT, float* s, float* sa);
+int rwkv7_statepassing_backward(void* stream, int B, int T, int H,
+                                const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k, const rwkv_bf16* v,
+                                const rwkv_bf16* a, const rwkv_bf16* b, const rwkv_bf16* dy, const float* dsT,
+                                const float* s, const float* sa, float* ds0,
+                                rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv,
+                                rwkv_bf16* da, rwkv_bf16* db);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RWKV_HIP_H */

@@ -1,0 +1,249 @@
+"""CPU oracle: RWKV-5 / RWKV-6 / RWKV-6-with-state WKV (TEST INFRASTRUCTURE, not product code).
+
+Index convention (same as the reference): i = value/output channel, j = key channel,
+state S[b,h,i,j].  `w` below is always the DECAY in (0,1) unless a name says `raw`.
+
+    y_t[i]      = sum_j r_t[j] * (u[j] * k_t[j] * v_t[i] + S_t[i,j])
+    S_{t+1}[i,j] = w_t[j] * S_t[i,j] + k_t[j] * v_t[i]            S_0 = s0 (or 0)
+
+Pinning (tests/test_oracle_wkv56.py): sum form vs recurrent form; constant-per-head
+special case vs a plain matmul; w=1,u=1 vs cumsum (causal linear attention); wkv6 with
+time-constant w equals wkv5; splitting T with a state hand-off equals one call; the
+hand-derived backward vs fp64 autograd of the sum form; gw[T-1]=0 and gw[0]=0 iff s0=0.
+"""
+
+import torch
+
+from . import bf16_round
+
+
+# --------------------------------------------------------------------------------------
+# decay pre-transforms done by the reference wrappers
+# --------------------------------------------------------------------------------------
+
+def wkv5_decays(w_raw):
+    """ew = -exp(w_raw), eew = exp(ew), both fp32.  Follows wkv5_bf16/run.py:63-64."""
+    ew = -torch.exp(w_raw.float())
+    return torch.exp(ew), ew
+
+
+def wkv6_decay(w_raw):
+    """decay = exp(-exp(w_raw)).  Follows wkv6_state/run.py:141 and wkv6/run.py:147-150."""
+    return torch.exp(-torch.exp(w_raw))
+
+
+# --------------------------------------------------------------------------------------
+# definition-level sum forms (tiny shapes only)
+# --------------------------------------------------------------------------------------
+
+def wkv5_sumform(B, T, C, H, r, k, v, w, u):
+    """out[b,t,h,i] = sum_j r[t,j] * sum_{tt<=t} ww * k[tt,j] * v[tt,i],
+    ww = u[h,j] if tt==t else w[h,j]**(t-tt-1).   Follows RUN_FORMULA_1, wkv5/run.py:47-65.
+    `w` is the decay [H,N]."""
+    N = C // H
+    r, k, v = (x.reshape(B, T, H, N) for x in (r, k, v))
+    w = w.reshape(H, N)
+    u = u.reshape(H, N)
+    out = torch.zeros(B, T, H, N, dtype=r.dtype)
+    for t in range(T):
+        for tt in range(t + 1):
+            ww = u if tt == t else w ** (t - tt - 1)                    # [H,N] over j
+            coef = (r[:, t] * ww * k[:, tt]).sum(-1, keepdim=True)      # sum over j -> [B,H,1]
+            out[:, t] += coef * v[:, tt]
+    return out.reshape(B, T, C)
+
+
+def wkv6_sumform(B, T, C, H, r, k, v, w, u, s0=None):
+    """Product-of-decays sum form with the tt=-1 initial-state term.
+    Follows RUN_TORCH, wkv6_state/run.py:137-165 (and wkv6/run.py:193-205 when s0 is None).
+    `w` is the decay [B,T,C]."""
+    N = C // H
+    r, k, v, w = (x.reshape(B, T, H, N) for x in (r, k, v, w))
+    u = u.reshape(H, N)
+    out = torch.zeros(B, T, H, N, dtype=r.dtype)
+    for t in range(T):
+        for tt in range(-1, t + 1):
+            if tt == t:
+                ww = u.expand(B, H, N)
+            else:
+                ww = torch.ones(B, H, N, dtype=r.dtype)
+                for zz in range(tt + 1, t):
+                    ww = ww * w[:, zz]
+            if tt == -1:
+                if s0 is not None:
+                    # out[i] += sum_j r[t,j] * ww[j] * s0[i,j]
+                    out[:, t] += torch.einsum('bhj,bhij->bhi', r[:, t] * ww, s0.reshape(B, H, N, N))
+            else:
+                coef = (r[:, t] * ww * k[:, tt]).sum(-1, keepdim=True)
+                out[:, t] += coef * v[:, tt]
+    return out.reshape(B, T, C)
+
+
+# --------------------------------------------------------------------------------------
+# recurrent form (any size; differentiable; dtype follows the inputs)
+# --------------------------------------------------------------------------------------
+
+def wkv_recurrent(B, T, C, H, r, k, v, w, u, s0=None):
+    """Recurrent form.  Follows RUN_FORMULA_1A, wkv5/run.py:67-87 and wkv6/run.py:207-216
+    (state enters the output before it is updated; bonus u on the current token).
+    `w` is the decay, either [H,N] (wkv5) or [B,T,C] (wkv6).  `u` is [H,N] or, for
+    per-batch gradient partials, [B,H,N].  Returns (y[B,T,C], S_T[B,H,N,N])."""
+    N = C // H
+    r, k, v = (x.reshape(B, T, H, N) for x in (r, k, v))
+    if w.numel() == H * N:
+        w = w.reshape(1, 1, H, N).expand(B, T, H, N)
+    elif w.numel() == B * H * N:
+        w = w.reshape(B, 1, H, N).expand(B, T, H, N)
+    else:
+        w = w.reshape(B, T, H, N)
+    u = u.reshape(-1, H, N)
+    S = torch.zeros(B, H, N, N, dtype=r.dtype) if s0 is None else s0.reshape(B, H, N, N)
+    ys = []
+    for t in range(T):
+        kv = v[:, t, :, :, None] * k[:, t, :, None, :]                      # [B,H,i,j]
+        ys.append(((S + u[:, :, None, :] * kv) * r[:, t, :, None, :]).sum(-1))
+        S = S * w[:, t, :, None, :] + kv
+    return torch.stack(ys, 1).reshape(B, T, C), S
+
+
+def wkv_backward_hand(B, T, C, H, r, k, v, w, u, gy, s0=None):
+    """Hand-derived backward of the recurrent form, two sweeps, no autograd.
+
+    Sweep up (t ascending) rebuilds S_t and gives gr, gu and the bonus-free part dr' of gr;
+    sweep down carries dS and gives gk, gv.  Follows the structure of the reference's
+    recurrent hand backward (RUN_BACKWARD_1A, wkv5/run.py:217-270) and of
+    kernel_backward_111 (wkv6_state/cuda/wkv6state_cuda_v1a.cu:67-188).
+
+    The decay gradient uses P_t[j] = sum_i dS_t[i,j] S_t[i,j]:
+        G_t = w_t * sum_i dS_{t+1}[i,j] S_t[i,j]  =  P_{t+1} - k_t dk'_t  =  P_t - r_t dr'_t,
+    so P is a running scalar per channel (P_T = 0).  This replaces the reference's
+    saaaa/sbbbb/scccc recurrences (wkv6state_cuda_v1a.cu:190-293) by an identity that is
+    pinned against fp64 autograd in tests/test_oracle_wkv56.py.
+
+    `w` is the decay [B,T,C].  Returns gr, gk, gv, G (= w * dL/dw, [B,T,C]), gu[B,H,N]
+    (per-batch partials), gs[B,H,N,N] (= dS_0).
+    """
+    N = C // H
+    r, k, v, w, gy = (x.reshape(B, T, H, N) for x in (r, k, v, w, gy))
+    u = u.reshape(1, H, N)
+    S = torch.zeros(B, H, N, N, dtype=r.dtype) if s0 is None else s0.reshape(B, H, N, N).clone()
+    gr = torch.empty_like(r)
+    gk = torch.empty_like(r)
+    gv = torch.empty_like(r)
+    G = torch.empty_like(r)
+    rdr = torch.empty_like(r)
+    gu = torch.zeros(B, H, N, dtype=r.dtype)
+    for t in range(T):
+        vgy = (v[:, t] * gy[:, t]).sum(-1, keepdim=True)                   # sum_i v_i gy_i
+        drp = torch.einsum('bhi,bhij->bhj', gy[:, t], S)                   # dr'_t[j]
+        gr[:, t] = drp + u * k[:, t] * vgy
+        rdr[:, t] = r[:, t] * drp
+        gu += r[:, t] * k[:, t] * vgy
+        S = S * w[:, t, :, None, :] + v[:, t, :, :, None] * k[:, t, :, None, :]
+    dS = torch.zeros(B, H, N, N, dtype=r.dtype)                            # dS_{t+1}
+    P = torch.zeros(B, H, N, dtype=r.dtype)                                # P_{t+1}
+    for t in range(T - 1, -1, -1):
+        vgy = (v[:, t] * gy[:, t]).sum(-1, keepdim=True)
+        dkp = torch.einsum('bhi,bhij->bhj', v[:, t], dS)                   # dk'_t[j]
+        gk[:, t] = dkp + u * r[:, t] * vgy
+        ruk = (u * r[:, t] * k[:, t]).sum(-1, keepdim=True)
+        gv[:, t] = torch.einsum('bhj,bhij->bhi', k[:, t], dS) + gy[:, t] * ruk
+        G[:, t] = P - k[:, t] * dkp
+        P = G[:, t] + rdr[:, t]
+        dS = dS * w[:, t, :, None, :] + gy[:, t, :, :, None] * r[:, t, :, None, :]
+    return (gr.reshape(B, T, C), gk.reshape(B, T, C), gv.reshape(B, T, C), G.reshape(B, T, C), gu, dS)
+
+
+# --------------------------------------------------------------------------------------
+# special cases that reduce to library routines
+# --------------------------------------------------------------------------------------
+
+def wkv5_matmul_form(B, T, C, H, r, k, v, w_head, u_head):
+    """w and u constant within each head: y = ((R K^T) * A) V with A[t,s] = w^(t-s-1) (s<t), u (s==t).
+    The one-chunk case of RUN_TORCH, wkv5/run.py:295-346.  w_head,u_head: [H]."""
+    N = C // H
+    r, k, v = (x.reshape(B, T, H, N).transpose(1, 2) for x in (r, k, v))       # [B,H,T,N]
+    tt = torch.arange(T)
+    d = (tt[:, None] - tt[None, :] - 1).clamp(min=0).to(r.dtype)
+    A = w_head.reshape(H, 1, 1) ** d                                             # [H,T,T]
+    A = torch.where((tt[:, None] > tt[None, :])[None], A, torch.zeros_like(A))
+    A = A + torch.eye(T, dtype=r.dtype)[None] * u_head.reshape(H, 1, 1)
+    y = ((r @ k.transpose(-1, -2)) * A[None]) @ v
+    return y.transpose(1, 2).reshape(B, T, C)
+
+
+def linear_attention_cumsum(B, T, C, H, r, k, v):
+    """w = 1, u = 1:  y_t[i] = sum_j r_t[j] * cumsum_{s<=t}(k_s[j] v_s[i])."""
+    N = C // H
+    r, k, v = (x.reshape(B, T, H, N) for x in (r, k, v))
+    kv = torch.cumsum(v[..., :, None] * k[..., None, :], dim=1)                  # [B,T,H,i,j]
+    return (kv * r[..., None, :]).sum(-1).reshape(B, T, C)
+
+
+# --------------------------------------------------------------------------------------
+# gradients by autograd, and the bf16 "kernel-faithful" error bar
+# --------------------------------------------------------------------------------------
+
+def _leaf(x, dtype):
+    return x.detach().to(dtype).clone().requires_grad_(True)
+
+
+def wkv5_grads(B, T, C, H, r, k, v, w_raw, u, gy, dtype=torch.float64, per_batch=False):
+    """y and (gr,gk,gv,gw_raw,gu) of wkv5 by autograd through the recurrent form.
+    per_batch=True returns gw,gu as [B,H,N] partials (what the kernels write before the
+    wrapper's torch.sum, wkv5_bf16/run.py:86-87)."""
+    N = C // H
+    r_, k_, v_ = (_leaf(x, dtype) for x in (r, k, v))
+    if per_batch:
+        w_ = _leaf(w_raw.reshape(1, H, N).expand(B, H, N), dtype)
+        u_ = _leaf(u.reshape(1, H, N).expand(B, H, N), dtype)
+    else:
+        w_ = _leaf(w_raw.reshape(H, N), dtype)
+        u_ = _leaf(u.reshape(H, N), dtype)
+    y, _ = wkv_recurrent(B, T, C, H, r_, k_, v_, torch.exp(-torch.exp(w_)), u_)
+    y.backward(gy.to(dtype))
+    return y.detach(), r_.grad, k_.grad, v_.grad, w_.grad, u_.grad
+
+
+def wkv6_grads(B, T, C, H, r, k, v, w_raw, u, gy, s0=None, dtype=torch.float64, per_batch=False):
+    """y and (gr,gk,gv,gw_raw,gu[,gs]) of wkv6 / wkv6_state by autograd."""
+    N = C // H
+    r_, k_, v_, w_ = (_leaf(x, dtype) for x in (r, k, v, w_raw))
+    u_ = _leaf(u.reshape(1, H, N).expand(B, H, N), dtype) if per_batch else _leaf(u.reshape(H, N), dtype)
+    s_ = None if s0 is None else _leaf(s0, dtype)
+    y, _ = wkv_recurrent(B, T, C, H, r_, k_, v_, torch.exp(-torch.exp(w_)), u_, s_)
+    y.backward(gy.to(dtype))
+    out = [y.detach(), r_.grad, k_.grad, v_.grad, w_.grad, u_.grad]
+    if s0 is not None:
+        out.append(s_.grad)
+    return out
+
+
+def emulate_wkv5_bf16(B, T, C, H, r, k, v, w_raw, u, gy):
+    """Error bar for the bf16 wkv5 path: fp32 math on the bf16 inputs with the reference's
+    rounding points -- y, gr, gk, gv stored as bf16 (wkv5_cuda_v1b.cu:59,105,174-175); gw, gu
+    stored per batch as bf16 (:107,136) and summed over B by torch.sum on bf16
+    (wkv5_bf16/run.py:86-87).  The decays are computed in fp32 from the bf16 w (:63-64).
+    fp32 summation order and __expf are not modelled: their effect (~1e-7 relative) is far
+    below the bf16 rounding that sets the bar."""
+    f = torch.float32
+    y, gr, gk, gv, gw, gu = wkv5_grads(B, T, C, H, r, k, v, w_raw, u, gy, dtype=f, per_batch=True)
+    rb = lambda x: x.to(torch.bfloat16)
+    gw = rb(gw).sum(0).reshape(H, C // H)
+    gu = rb(gu).sum(0).reshape(H, C // H)
+    return rb(y), rb(gr), rb(gk), rb(gv), gw, gu
+
+
+def emulate_wkv6_bf16(B, T, C, H, r, k, v, w_raw, u, gy, s0=None):
+    """Error bar for the bf16 wkv6 / wkv6_state paths: fp32 math on bf16 inputs, outputs
+    rounded where the reference kernels round -- y (wkv6state_cuda_v1a.cu:63), gr/gk/gv/gw
+    (:119,143,166,251), per-batch gu as bf16 (:121) then torch.sum over B on bf16
+    (wkv6_state/run.py:123), gs as bf16 (:187)."""
+    f = torch.float32
+    out = wkv6_grads(B, T, C, H, r, k, v, w_raw, u, gy, s0=s0, dtype=f, per_batch=True)
+    rb = lambda x: x.to(torch.bfloat16)
+    y, gr, gk, gv, gw, gu = out[:6]
+    res = [rb(y), rb(gr), rb(gk), rb(gv), rb(gw), rb(gu).sum(0).reshape(H, C // H)]
+    if s0 is not None:
+        res.append(rb(out[6]))
+    return res

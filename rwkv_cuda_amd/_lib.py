@@ -1,0 +1,101 @@
+"""Build and load librwkv_hip.so (the C ABI declared in include/rwkv_hip.h) through ctypes.
+
+`build()` always compiles (hipcc cross-compiles gfx950 without a GPU); `load()` uses the
+library that is already built and only builds when there is none.  There is no CPU or
+PyTorch fallback: if the library cannot be loaded the import of an op fails loudly.
+"""
+
+import ctypes
+import os
+import subprocess
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_ROOT = os.path.dirname(_HERE)
+_CSRC = os.path.join(_HERE, "csrc")
+_INCLUDE = os.path.join(_ROOT, "include")
+LIB_PATH = os.path.join(_HERE, "librwkv_hip.so")
+
+SOURCES = ["abi.hip", "wkv56.hip", "wkv4.hip", "timex.hip", "rwkv7.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    # packed fp32 VALU ops stay off on this target
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+_lib = None
+
+
+def build(verbose=False):
+    """Compile every HIP source into one shared library, in-tree."""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    srcs = [os.path.join(_CSRC, s) for s in SOURCES if os.path.exists(os.path.join(_CSRC, s))]
+    cmd = [hipcc] + HIPCC_FLAGS + ["-I", _INCLUDE, "-I", _CSRC, "-o", LIB_PATH] + srcs
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in res.stdout.splitlines() if "is not a recognized feature" not in l)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + out)
+    if verbose and out.strip():
+        print(out, flush=True)
+    return LIB_PATH
+
+
+_P = ctypes.c_void_p
+_I = ctypes.c_int
+_F = ctypes.c_float
+_Z = ctypes.c_size_t
+
+# name -> (restype, argtypes): one row per symbol in include/rwkv_hip.h
+SIGNATURES = {
+    "rwkv_strerror": (ctypes.c_char_p, [_I]),
+    "rwkv_last_hip_error": (_I, []),
+    "rwkv_abi_version": (_I, []),
+    "rwkv_wkv4_forward": (_I, [_P, _I, _I, _I] + [_P] * 5),
+    "rwkv_wkv4_backward": (_I, [_P, _I, _I, _I] + [_P] * 9),
+    "rwkv_timex_forward": (_I, [_P, _P, _P, _P, _F, _I, _I, _I]),
+    "rwkv_timex_backward": (_I, [_P] * 6 + [_I, _I, _I]),
+    "rwkv_wkv5_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
+    "rwkv_wkv5_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "rwkv_wkv5_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_P, _Z]),
+    "rwkv_wkv6_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
+    "rwkv_wkv6_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "rwkv_wkv6_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z]),
+    "rwkv_wkv6state_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 7),
+    "rwkv_wkv6state_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "rwkv_wkv6state_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, _Z]),
+    "rwkv7_statepassing_forward": (_I, [_P, _I, _I, _I] + [_P] * 11),
+    "rwkv7_statepassing_backward": (_I, [_P, _I, _I, _I] + [_P] * 17),
+}
+
+
+def load():
+    """Return the ctypes handle of the built library (building it once if it is absent)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        build()
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)        # AttributeError here = header and library disagree
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+class RwkvHipError(RuntimeError):
+    pass
+
+
+def check(status):
+    """Raise on a non-zero status from the C ABI."""
+    if status != 0:
+        lib = load()
+        msg = lib.rwkv_strerror(status).decode()
+        if status == -5:
+            msg += f" (hipError {lib.rwkv_last_hip_error()})"
+        raise RwkvHipError(f"librwkv_hip: status {status}: {msg}")

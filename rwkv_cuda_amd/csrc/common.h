@@ -1,0 +1,92 @@
+// Shared device helpers and host-side argument checks for librwkv_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <utility>
+
+#include "rwkv_hip.h"
+
+#define DEVINL __device__ __forceinline__
+
+namespace rwkv {
+
+// ----------------------------------------------------------------------------- bf16 <-> f32
+DEVINL float bf2f(uint16_t x) { return __uint_as_float(static_cast<uint32_t>(x) << 16); }
+DEVINL float bf_lo(uint32_t x) { return __uint_as_float(x << 16); }          // element 0 of a packed pair
+DEVINL float bf_hi(uint32_t x) { return __uint_as_float(x & 0xffff0000u); }  // element 1 of a packed pair
+
+// round-to-nearest-even, NaN stays NaN
+DEVINL uint32_t f2bf_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+DEVINL uint16_t f2bf(float f) { return static_cast<uint16_t>(f2bf_bits(f)); }
+DEVINL uint32_t pack_bf2(float lo, float hi) { return f2bf_bits(lo) | (f2bf_bits(hi) << 16); }
+
+DEVINL void unpack8(const uint4& q, float (&f)[8]) {
+    f[0] = bf_lo(q.x); f[1] = bf_hi(q.x); f[2] = bf_lo(q.y); f[3] = bf_hi(q.y);
+    f[4] = bf_lo(q.z); f[5] = bf_hi(q.z); f[6] = bf_lo(q.w); f[7] = bf_hi(q.w);
+}
+DEVINL uint4 pack8(const float (&f)[8]) {
+    uint4 q;
+    q.x = pack_bf2(f[0], f[1]); q.y = pack_bf2(f[2], f[3]);
+    q.z = pack_bf2(f[4], f[5]); q.w = pack_bf2(f[6], f[7]);
+    return q;
+}
+
+// ----------------------------------------------------------------------------- row broadcast
+// A wave64 is four DPP rows of 16 lanes.  bc<J>(x) is x of lane (row*16 + J): with a vector
+// laid out as x_lane = vec[base + (lane & 15)] this gives vec[base + J] in every lane without
+// an LDS read or an SGPR.  The fused forms below put the broadcast inside the VALU op
+// (v_fmac_f32_dpp / v_mul_f32_dpp row_newbcast), so a broadcast operand costs nothing.
+// The DPP source operand must not have been written by the one or two VALU instructions
+// just before (gfx9 DPP read-after-VALU-write hazard); callers only feed it values that come
+// straight from LDS or that are loop invariant.
+template <int J> DEVINL void fmac_bc(float& acc, float row_vec, float s) {   // acc += row_vec[J] * s
+    asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+        : "+v"(acc) : "v"(row_vec), "v"(s), "n"(J));
+}
+template <int J> DEVINL void mul_bc(float& s, float row_vec) {               // s *= row_vec[J]
+    asm("v_mul_f32_dpp %0, %1, %0 row_newbcast:%2 row_mask:0xf bank_mask:0xf"
+        : "+v"(s) : "v"(row_vec), "n"(J));
+}
+template <int J> DEVINL float bc(float row_vec) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, row_vec),
+                                                                0x150 + J, 0xf, 0xf, true));
+}
+
+template <typename F, int... I> DEVINL void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F> DEVINL void static_for(F&& f) {
+    static_for_impl(static_cast<F&&>(f), std::make_integer_sequence<int, N>{});
+}
+
+// sum over a group of 2^k consecutive lanes (k <= 6); result valid in every lane of the group
+template <int WIDTH> DEVINL float group_sum(float x) {
+#pragma unroll
+    for (int m = WIDTH / 2; m >= 1; m >>= 1) x += __shfl_xor(x, m, 64);
+    return x;
+}
+
+// ----------------------------------------------------------------------------- host checks
+extern thread_local int g_last_hip_error;
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+inline int check_ptrs(std::initializer_list<const void*> ps) {
+    for (const void* p : ps) if (p == nullptr) return RWKV_ERR_NULL;
+    for (const void* p : ps) if (!aligned16(p)) return RWKV_ERR_ALIGN;
+    return RWKV_OK;
+}
+
+inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { g_last_hip_error = static_cast<int>(e); return RWKV_ERR_LAUNCH; }
+    return RWKV_OK;
+}
+
+}  // namespace rwkv

@@ -1,0 +1,424 @@
+// wkv5 / wkv6 / wkv6_state for gfx950: sequential-in-time sweeps with the 64x64 state in VGPRs.
+//
+// One workgroup (4 waves) per (batch, head).  The state S[i][j] (i = value channel, j = key
+// channel) is tiled 16 elements per lane in one of two ways:
+//   shape F  lane = i, wave q holds j in [16q,16q+16)   out[i] = sum_j a[j] S[i][j];  S = S w[j] + b[j] x[i]
+//   shape G  lane = j, wave q holds i in [16q,16q+16)   out[j] = sum_i a[i] S[i][j];  S = S w[j] + x[i] b[j]
+// Vectors indexed by the in-register axis are kept one element per lane, replicated in every
+// 16-lane DPP row, and enter the FMAs through row_newbcast, so a step is 3 VALU ops per state
+// element and four LDS reads per lane.  Inputs are staged through LDS as fp32 in chunks of
+// TC time steps (16-byte global loads, issued one chunk ahead); the four waves' partial sums
+// are combined once per chunk, where the outputs are rounded to bf16 and stored 16 bytes
+// at a time.
+//
+// Passes (what the reference does in wkv5_cuda_v1b.cu / wkv6_cuda_v1.cu / wkv6state_cuda_v1a.cu):
+//   FWD  shape F, t up,   a=r b=k x=v    y_t[i]  = sum_j r(S + u k v)                 S_0 = s0
+//   GR   shape G, t up,   a=gy x=v b=k   gr_t[j] = sum_i gy S + u k (v.gy);  gu;  r*dr' -> workspace
+//   GK   shape G, t down, a=v x=gy b=r   gk_t[j] = sum_i v dS + u r (v.gy);  gw;  gs = dS_0
+//   GV   shape F, t down, a=k b=r x=gy   gv_t[i] = sum_j k dS + gy sum_j(u r k)
+// The decay gradient needs no third recurrence: with P_t[j] = sum_i dS_t[i,j] S_t[i,j],
+//   G_t = w_t * sum_i dS_{t+1} S_t = P_{t+1} - k_t dk'_t,   P_t = G_t + r_t dr'_t,   P_T = 0,
+// where dr', dk' are the bonus-free parts of gr, gk; gw_raw = -exp(w_raw) * G.
+#include "common.h"
+
+namespace rwkv {
+namespace {
+
+constexpr int N = 64;            // head size
+constexpr int TC = 32;           // time steps per staged chunk
+constexpr int NW = 4;            // waves per workgroup
+constexpr int NT = NW * 64;
+constexpr int JW = N / NW;       // state elements per lane
+static_assert(JW == 16, "row broadcast assumes 16 state elements per lane");
+static_assert(TC * N == NT * 8, "staging assumes 8 elements per thread per tensor");
+
+enum { P_FWD = 0, P_GR = 1, P_GK = 2, P_GV = 3 };
+enum { W_HEAD = 0, W_EW = 1, W_RAW = 2 };   // wkv5 (eew[H,N] fp32) / wkv6 (ew fp32 [B,T,C]) / wkv6_state (raw bf16)
+
+struct Args {
+    int T, C, H;
+    const uint16_t *r, *k, *v, *u, *s0, *gy;
+    const void* w;        // W_HEAD: const float* eew[H*N]; W_EW: const float* ew[B*T*C]; W_RAW: const uint16_t* raw
+    const float* ew_head; // W_HEAD, GK only: -exp(w_raw) [H*N]
+    uint16_t *y, *gr, *gk, *gv, *gw, *gu, *gs;
+    float* rdr;           // workspace [B,T,C] fp32: r * dr'
+};
+
+template <int PASS> struct Smem {
+    static constexpr bool kBwd = PASS != P_FWD;
+    static constexpr bool kGK = PASS == P_GK;
+    float r[TC][N];
+    float k[TC][N];
+    float v[(PASS == P_GV) ? 1 : TC][N];
+    float g[kBwd ? TC : 1][N];
+    float w[TC][N];
+    float f[kGK ? TC : 1][N];      // d(log decay)/d(w_raw) * ... : the factor that turns G into gw
+    float rdr[kGK ? TC : 1][N];
+    float part[NW][TC][N];
+    float dot[TC];
+    float u[N];
+};
+
+struct Staged {
+    uint4 r, k, v, g, w0, w1;
+    float4 rdr0, rdr1;
+};
+
+template <int PASS, int WMODE>
+DEVINL void prefetch(Staged& p, const Args& a, size_t base, int c0, int st, int sj) {
+    const int t = c0 + st;
+    const bool ok = t < a.T;
+    const size_t off = base + static_cast<size_t>(t) * a.C + sj;
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    p.r = ok ? *reinterpret_cast<const uint4*>(a.r + off) : z;
+    p.k = ok ? *reinterpret_cast<const uint4*>(a.k + off) : z;
+    if constexpr (PASS != P_GV) p.v = ok ? *reinterpret_cast<const uint4*>(a.v + off) : z;
+    if constexpr (PASS != P_FWD) p.g = ok ? *reinterpret_cast<const uint4*>(a.gy + off) : z;
+    if constexpr (WMODE == W_RAW) {
+        p.w0 = ok ? *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.w) + off) : z;
+    } else if constexpr (WMODE == W_EW) {
+        const float* w = static_cast<const float*>(a.w) + off;
+        p.w0 = ok ? *reinterpret_cast<const uint4*>(w) : z;
+        p.w1 = ok ? *reinterpret_cast<const uint4*>(w + 4) : z;
+    }
+    if constexpr (PASS == P_GK) {
+        const float4 zf = make_float4(0.f, 0.f, 0.f, 0.f);
+        p.rdr0 = ok ? *reinterpret_cast<const float4*>(a.rdr + off) : zf;
+        p.rdr1 = ok ? *reinterpret_cast<const float4*>(a.rdr + off + 4) : zf;
+    }
+}
+
+DEVINL void st8(float* dst, const float (&f)[8]) {
+    *reinterpret_cast<float4*>(dst) = make_float4(f[0], f[1], f[2], f[3]);
+    *reinterpret_cast<float4*>(dst + 4) = make_float4(f[4], f[5], f[6], f[7]);
+}
+DEVINL void ld8f(const float* src, float (&f)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(src);
+    const float4 b = *reinterpret_cast<const float4*>(src + 4);
+    f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+
+// registers -> LDS (fp32), plus the per-step scalar `dot`
+template <int PASS, int WMODE>
+DEVINL void commit(Smem<PASS>& S, const Staged& p, const Args& a, int c0, int st, int sj) {
+    const bool ok = (c0 + st) < a.T;
+    float fr[8], fk[8], fv[8], fg[8];
+    unpack8(p.r, fr);
+    unpack8(p.k, fk);
+    st8(&S.r[st][sj], fr);
+    st8(&S.k[st][sj], fk);
+    if constexpr (PASS != P_GV) { unpack8(p.v, fv); st8(&S.v[st][sj], fv); }
+    if constexpr (PASS != P_FWD) { unpack8(p.g, fg); st8(&S.g[st][sj], fg); }
+    if constexpr (WMODE != W_HEAD) {
+        float fw[8], dec[8];
+        if constexpr (WMODE == W_RAW) {
+            unpack8(p.w0, fw);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) fw[e] = -__expf(fw[e]);       // d(log decay): -exp(w_raw)
+        } else {
+            fw[0] = __uint_as_float(p.w0.x); fw[1] = __uint_as_float(p.w0.y);
+            fw[2] = __uint_as_float(p.w0.z); fw[3] = __uint_as_float(p.w0.w);
+            fw[4] = __uint_as_float(p.w1.x); fw[5] = __uint_as_float(p.w1.y);
+            fw[6] = __uint_as_float(p.w1.z); fw[7] = __uint_as_float(p.w1.w);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dec[e] = ok ? __expf(fw[e]) : 1.0f;  // rows past T leave the state alone
+        st8(&S.w[st][sj], dec);
+        if constexpr (PASS == P_GK) st8(&S.f[st][sj], fw);
+    }
+    if constexpr (PASS == P_GK) {
+        *reinterpret_cast<float4*>(&S.rdr[st][sj]) = p.rdr0;
+        *reinterpret_cast<float4*>(&S.rdr[st][sj + 4]) = p.rdr1;
+    }
+    float d = 0.f;
+    if constexpr (PASS == P_FWD || PASS == P_GV) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d = fmaf(fr[e] * S.u[sj + e], fk[e], d);   // sum_j u r k
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) d = fmaf(fv[e], fg[e], d);                 // sum_i v gy
+    }
+    d = group_sum<8>(d);
+    if ((threadIdx.x & 7) == 0) S.dot[st] = d;
+}
+
+template <int PASS, int WMODE>
+__global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
+    constexpr bool REV = (PASS == P_GK || PASS == P_GV);
+    constexpr bool SHAPE_F = (PASS == P_FWD || PASS == P_GV);
+    __shared__ Smem<PASS> S;
+
+    const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
+    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
+    const int st = tid >> 3, sj = (tid & 7) * 8;            // staging / epilogue coordinates
+    const int rowslot = q * JW + (lane & 15);               // element of a broadcast vector held by this lane
+    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
+    const size_t bh = static_cast<size_t>(b) * a.H + h;
+    const bool stateful = a.s0 != nullptr;
+
+    if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
+
+    // ---- state registers
+    float St[JW];
+#pragma unroll
+    for (int e = 0; e < JW; ++e) St[e] = 0.f;
+    if (stateful) {
+        if constexpr (PASS == P_FWD) {
+            const uint16_t* s = a.s0 + (bh * N + lane) * N + q * JW;        // row i = lane, 16 consecutive j
+            float lo[8], hi[8];
+            unpack8(*reinterpret_cast<const uint4*>(s), lo);
+            unpack8(*reinterpret_cast<const uint4*>(s + 8), hi);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { St[e] = lo[e]; St[8 + e] = hi[e]; }
+        } else if constexpr (PASS == P_GR) {
+#pragma unroll
+            for (int e = 0; e < JW; ++e) St[e] = bf2f(a.s0[(bh * N + q * JW + e) * N + lane]);
+        }
+    }
+    // time-constant decay (wkv5)
+    float w_const = 1.f;
+    if constexpr (WMODE == W_HEAD) {
+        const float* eew = static_cast<const float*>(a.w) + h * N;
+        w_const = SHAPE_F ? eew[rowslot] : eew[lane];
+    }
+
+    float gu_acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) gu_acc[e] = 0.f;
+    float P = 0.f, gw_acc = 0.f;                            // GK scan state (threads < 64)
+
+    const int nchunks = (a.T + TC - 1) / TC;
+    Staged pre;
+    prefetch<PASS, WMODE>(pre, a, base, (REV ? nchunks - 1 : 0) * TC, st, sj);
+    __syncthreads();                                        // S.u visible
+
+    for (int ci = 0; ci < nchunks; ++ci) {
+        const int c0 = (REV ? nchunks - 1 - ci : ci) * TC;
+        __syncthreads();                                    // previous epilogue is done with LDS
+        commit<PASS, WMODE>(S, pre, a, c0, st, sj);
+        __syncthreads();
+        if (ci + 1 < nchunks) prefetch<PASS, WMODE>(pre, a, base, (REV ? nchunks - 2 - ci : ci + 1) * TC, st, sj);
+
+        // ---- TC sequential steps
+#pragma unroll 4
+        for (int tt = 0; tt < TC; ++tt) {
+            const int t = REV ? TC - 1 - tt : tt;
+            float acc = 0.f;
+            if constexpr (SHAPE_F) {
+                const float av = (PASS == P_FWD) ? S.r[t][rowslot] : S.k[t][rowslot];
+                const float bv = (PASS == P_FWD) ? S.k[t][rowslot] : S.r[t][rowslot];
+                const float wv = (WMODE == W_HEAD) ? w_const : S.w[t][rowslot];
+                const float x = (PASS == P_FWD) ? S.v[t][lane] : S.g[t][lane];
+                static_for<JW>([&](auto J) {
+                    fmac_bc<decltype(J)::value>(acc, av, St[decltype(J)::value]);
+                    mul_bc<decltype(J)::value>(St[decltype(J)::value], wv);
+                    fmac_bc<decltype(J)::value>(St[decltype(J)::value], bv, x);
+                });
+            } else {
+                const float av = (PASS == P_GR) ? S.g[t][rowslot] : S.v[t][rowslot];
+                const float xv = (PASS == P_GR) ? S.v[t][rowslot] : S.g[t][rowslot];
+                const float bl = (PASS == P_GR) ? S.k[t][lane] : S.r[t][lane];
+                const float wl = (WMODE == W_HEAD) ? w_const : S.w[t][lane];
+                static_for<JW>([&](auto I) {
+                    fmac_bc<decltype(I)::value>(acc, av, St[decltype(I)::value]);
+                    St[decltype(I)::value] *= wl;
+                    fmac_bc<decltype(I)::value>(St[decltype(I)::value], xv, bl);
+                });
+            }
+            S.part[q][t][lane] = acc;
+        }
+        __syncthreads();
+
+        // ---- chunk epilogue: thread (st, sj..sj+7)
+        const bool ok = (c0 + st) < a.T;
+        const size_t off = base + static_cast<size_t>(c0 + st) * a.C + sj;
+        float sum[8];
+        {
+            float p1[8], p2[8], p3[8];
+            ld8f(&S.part[0][st][sj], sum);
+            ld8f(&S.part[1][st][sj], p1);
+            ld8f(&S.part[2][st][sj], p2);
+            ld8f(&S.part[3][st][sj], p3);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sum[e] = (sum[e] + p1[e]) + (p2[e] + p3[e]);
+        }
+        const float dot = S.dot[st];
+        float out[8];
+        if constexpr (PASS == P_FWD) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) out[e] = fmaf(S.v[st][sj + e], dot, sum[e]);
+            if (ok) *reinterpret_cast<uint4*>(a.y + off) = pack8(out);
+        } else if constexpr (PASS == P_GV) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) out[e] = fmaf(S.g[st][sj + e], dot, sum[e]);
+            if (ok) *reinterpret_cast<uint4*>(a.gv + off) = pack8(out);
+        } else if constexpr (PASS == P_GR) {
+            float rdr[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float rr = S.r[st][sj + e], kk = S.k[st][sj + e];
+                out[e] = fmaf(S.u[sj + e] * kk, dot, sum[e]);
+                rdr[e] = rr * sum[e];
+                gu_acc[e] = fmaf(rr * kk, dot, gu_acc[e]);
+            }
+            if (ok) {
+                *reinterpret_cast<uint4*>(a.gr + off) = pack8(out);
+                *reinterpret_cast<float4*>(a.rdr + off) = make_float4(rdr[0], rdr[1], rdr[2], rdr[3]);
+                *reinterpret_cast<float4*>(a.rdr + off + 4) = make_float4(rdr[4], rdr[5], rdr[6], rdr[7]);
+            }
+        } else {  // P_GK
+            float kdk[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                out[e] = fmaf(S.u[sj + e] * S.r[st][sj + e], dot, sum[e]);
+                kdk[e] = S.k[st][sj + e] * sum[e];
+            }
+            if (ok) *reinterpret_cast<uint4*>(a.gk + off) = pack8(out);
+            st8(&S.k[st][sj], kdk);                          // k is no longer needed: keep k*dk' there
+            __syncthreads();
+            if (tid < N) {                                   // per-channel scan over the chunk, t descending
+                for (int t = TC - 1; t >= 0; --t) {
+                    float G = P - S.k[t][tid];
+                    if (!stateful && (c0 + t) == 0) G = 0.f; // S_0 = 0: exact zero, as the reference leaves it
+                    P = G + S.rdr[t][tid];
+                    if constexpr (WMODE == W_HEAD) gw_acc += G;
+                    else S.part[0][t][tid] = S.f[t][tid] * G;
+                }
+            }
+            if constexpr (WMODE != W_HEAD) {
+                __syncthreads();
+                ld8f(&S.part[0][st][sj], out);
+                if (ok) *reinterpret_cast<uint4*>(a.gw + off) = pack8(out);
+            }
+        }
+    }
+
+    // ---- tails
+    if constexpr (PASS == P_GR) {
+        __syncthreads();
+        st8(&S.part[0][st][sj], gu_acc);
+        __syncthreads();
+        if (tid < N) {
+            float s = 0.f;
+#pragma unroll 8
+            for (int t = 0; t < TC; ++t) s += S.part[0][t][tid];
+            a.gu[static_cast<size_t>(b) * a.C + h * N + tid] = f2bf(s);
+        }
+    }
+    if constexpr (PASS == P_GK) {
+        if constexpr (WMODE == W_HEAD) {
+            if (tid < N) a.gw[static_cast<size_t>(b) * a.C + h * N + tid] = f2bf(a.ew_head[h * N + tid] * gw_acc);
+        }
+        if (a.gs != nullptr) {
+#pragma unroll
+            for (int e = 0; e < JW; ++e) a.gs[(bh * N + q * JW + e) * N + lane] = f2bf(St[e]);
+        }
+    }
+}
+
+template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a) {
+    hipLaunchKernelGGL((wkv_sweep<P_FWD, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
+    return launch_status();
+}
+
+// GR and GV are independent; GK consumes GR's workspace.  All three run on `st` in order.
+template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a) {
+    hipLaunchKernelGGL((wkv_sweep<P_GR, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
+    hipLaunchKernelGGL((wkv_sweep<P_GV, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
+    hipLaunchKernelGGL((wkv_sweep<P_GK, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
+    return launch_status();
+}
+
+int check_dims(int B, int T, int C, int H) {
+    if (B <= 0 || T <= 0 || C <= 0 || H <= 0) return RWKV_ERR_SHAPE;
+    if (C != H * N) return RWKV_ERR_SHAPE;
+    if (static_cast<long long>(B) * H > 0x7fffffffLL) return RWKV_ERR_SHAPE;
+    return RWKV_OK;
+}
+
+size_t ws_bytes(int B, int T, int C, int H) {
+    if (check_dims(B, T, C, H) != RWKV_OK) return 0;
+    return static_cast<size_t>(B) * T * C * sizeof(float);
+}
+
+}  // namespace
+}  // namespace rwkv
+
+using namespace rwkv;
+
+extern "C" {
+
+int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                      const rwkv_bf16* v, const float* eew, const rwkv_bf16* u, rwkv_bf16* y) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, eew, u, y})) return e;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = eew; a.u = u; a.y = y;
+    return launch_fwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a);
+}
+
+size_t rwkv_wkv5_backward_workspace_bytes(int B, int T, int C, int H) { return ws_bytes(B, T, C, H); }
+
+int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                       const rwkv_bf16* v, const float* eew, const float* ew, const rwkv_bf16* u,
+                       const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw,
+                       rwkv_bf16* gu, void* workspace, size_t workspace_bytes) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu})) return e;
+    if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = eew; a.ew_head = ew; a.u = u; a.gy = gy;
+    a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
+    return launch_bwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a);
+}
+
+int rwkv_wkv6_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                      const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, rwkv_bf16* y) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, ew, u, y})) return e;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.y = y;
+    return launch_fwd<W_EW>(static_cast<hipStream_t>(stream), B, a);
+}
+
+size_t rwkv_wkv6_backward_workspace_bytes(int B, int T, int C, int H) { return ws_bytes(B, T, C, H); }
+
+int rwkv_wkv6_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                       const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
+                       rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                       void* workspace, size_t workspace_bytes) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, ew, u, gy, gr, gk, gv, gw, gu})) return e;
+    if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.gy = gy;
+    a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
+    return launch_bwd<W_EW>(static_cast<hipStream_t>(stream), B, a);
+}
+
+int rwkv_wkv6state_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                           const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s,
+                           rwkv_bf16* y) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, w, u, s, y})) return e;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.y = y;
+    return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a);
+}
+
+size_t rwkv_wkv6state_backward_workspace_bytes(int B, int T, int C, int H) { return ws_bytes(B, T, C, H); }
+
+int rwkv_wkv6state_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                            const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s,
+                            const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw,
+                            rwkv_bf16* gu, rwkv_bf16* gs, void* workspace, size_t workspace_bytes) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, w, u, s, gy, gr, gk, gv, gw, gu, gs})) return e;
+    if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.gy = gy;
+    a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.gs = gs; a.rdr = static_cast<float*>(workspace);
+    return launch_bwd<W_RAW>(static_cast<hipStream_t>(stream), B, a);
+}
+
+}  // extern "C"

@@ -1,0 +1,48 @@
+"""RWKV-5 WKV, bf16: drop-in for wkv5_bf16/run.py:44-91 (class WKV_5, RUN_CUDA)."""
+
+import torch
+
+from . import _lib
+from ._call import call, check_tensors, require
+
+HEAD_SIZE = 64
+
+
+class WKV_5(torch.autograd.Function):
+    """Same signature as WKV_5, wkv5_bf16/run.py:44-88: r,k,v[B,T,C], w,u[H,N], all bf16, w raw.
+    ew = -exp(w) and eew = exp(ew) are made in fp32 by the wrapper (:63-64)."""
+
+    @staticmethod
+    def forward(ctx, B, T, C, H, r, k, v, w, u):
+        with torch.no_grad():
+            dev = check_tensors((r, k, v, w, u), torch.bfloat16, "rkvwu")
+            require(HEAD_SIZE == C // H and C == H * HEAD_SIZE, "head size must be 64")
+            require(r.numel() == B * T * C and w.numel() == C, "shape mismatch")
+            ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
+            ew = (-torch.exp(w.float())).contiguous()
+            eew = (torch.exp(ew)).contiguous()
+            ctx.save_for_backward(r, k, v, eew, ew, u)
+            y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
+            call("rwkv_wkv5_forward", dev, B, T, C, H, r, k, v, eew, u, y)
+            return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        with torch.no_grad():
+            B, T, C, H = ctx.B, ctx.T, ctx.C, ctx.H
+            r, k, v, eew, ew, u = ctx.saved_tensors
+            gy = gy.contiguous()
+            dev = check_tensors((gy,), torch.bfloat16, ("gy",))
+            new = lambda *shape: torch.empty(shape, device=dev, dtype=torch.bfloat16)
+            gr, gk, gv = new(B, T, C), new(B, T, C), new(B, T, C)
+            gw, gu = new(B, C), new(B, C)
+            nbytes = _lib.load().rwkv_wkv5_backward_workspace_bytes(B, T, C, H)
+            ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+            call("rwkv_wkv5_backward", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+            gw = torch.sum(gw, 0).view(H, C // H)
+            gu = torch.sum(gu, 0).view(H, C // H)
+            return (None, None, None, None, gr, gk, gv, gw, gu)
+
+
+def RUN_CUDA(B, T, C, H, r, k, v, w, u):
+    return WKV_5.apply(B, T, C, H, r, k, v, w, u)

@@ -1,0 +1,47 @@
+"""RWKV-6 WKV with initial state: drop-in for wkv6_state/run.py:80-127 (class WKV_6STATE, RUN_CUDA)."""
+
+import torch
+
+from . import _lib
+from ._call import call, check_tensors, require
+
+HEAD_SIZE = 64
+
+
+class WKV_6STATE(torch.autograd.Function):
+    """Same signature, dtypes and returned gradients as WKV_6STATE, wkv6_state/run.py:80-124:
+    r,k,v,w[B,T,C], u[H,N], s[B,H,N,N], all bf16; w is the raw decay parameter."""
+
+    @staticmethod
+    def forward(ctx, B, T, C, H, r, k, v, w, u, s):
+        with torch.no_grad():
+            dev = check_tensors((r, k, v, w, u, s), torch.bfloat16, "rkvwus")
+            require(HEAD_SIZE == C // H and C == H * HEAD_SIZE, "head size must be 64")
+            require(r.numel() == B * T * C and s.numel() == B * H * HEAD_SIZE * HEAD_SIZE, "shape mismatch")
+            ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
+            ctx.save_for_backward(r, k, v, w, u, s)
+            y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
+            call("rwkv_wkv6state_forward", dev, B, T, C, H, r, k, v, w, u, s, y)
+            return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        with torch.no_grad():
+            B, T, C, H = ctx.B, ctx.T, ctx.C, ctx.H
+            r, k, v, w, u, s = ctx.saved_tensors
+            gy = gy.contiguous()
+            dev = check_tensors((gy,), torch.bfloat16, ("gy",))
+            new = lambda *shape: torch.empty(shape, device=dev, dtype=torch.bfloat16)
+            gr, gk, gv, gw = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C)
+            gu = new(B, C)
+            gs = new(B, H, C // H, C // H)
+            nbytes = _lib.load().rwkv_wkv6state_backward_workspace_bytes(B, T, C, H)
+            ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+            call("rwkv_wkv6state_backward", dev, B, T, C, H, r, k, v, w, u, s, gy,
+                 gr, gk, gv, gw, gu, gs, ws, nbytes)
+            gu = torch.sum(gu, 0).view(H, C // H)
+            return (None, None, None, None, gr, gk, gv, gw, gu, gs)
+
+
+def RUN_CUDA(B, T, C, H, r, k, v, w, u, s):
+    return WKV_6STATE.apply(B, T, C, H, r, k, v, w, u, s)

@@ -1,0 +1,150 @@
+"""Pins the wkv5 / wkv6 / wkv6_state oracle (CPU only).
+
+Each check is chosen so that a plausible mistake (dropped bonus term, decay applied before
+instead of after the read-out, transposed state, off-by-one in the decay product) fails it.
+"""
+import torch
+
+from oracle import wkv56 as O
+from oracle import err_ratio
+
+D = torch.float64
+
+
+def _inputs(B, T, H, N, seed=0, state=False):
+    g = torch.Generator().manual_seed(seed)
+    C = H * N
+    r, k, v, gy = (torch.randn(B, T, C, generator=g, dtype=D) for _ in range(4))
+    w_raw = torch.randn(B, T, C, generator=g, dtype=D) * 0.7 - 0.6
+    u = torch.randn(H, N, generator=g, dtype=D) * 0.3
+    s0 = torch.randn(B, H, N, N, generator=g, dtype=D) if state else None
+    return C, r, k, v, w_raw, u, gy, s0
+
+
+def test_wkv5_sum_vs_recurrent():
+    B, T, H, N = 2, 7, 2, 4
+    C, r, k, v, w_raw, u, gy, _ = _inputs(B, T, H, N, 1)
+    w = torch.exp(-torch.exp(w_raw[0, 0].reshape(H, N)))
+    y1 = O.wkv5_sumform(B, T, C, H, r, k, v, w, u)
+    y2, _ = O.wkv_recurrent(B, T, C, H, r, k, v, w, u)
+    assert err_ratio(y1, y2) < 1e-13
+
+
+def test_wkv6_sum_vs_recurrent_with_state():
+    B, T, H, N = 3, 7, 2, 4
+    C, r, k, v, w_raw, u, gy, s0 = _inputs(B, T, H, N, 2, state=True)
+    w = O.wkv6_decay(w_raw)
+    y1 = O.wkv6_sumform(B, T, C, H, r, k, v, w, u, s0)
+    y2, _ = O.wkv_recurrent(B, T, C, H, r, k, v, w, u, s0)
+    assert err_ratio(y1, y2) < 1e-13
+    # the state term matters and is not symmetric: transposing s0 must change the result
+    y3, _ = O.wkv_recurrent(B, T, C, H, r, k, v, w, u, s0.transpose(-1, -2))
+    assert err_ratio(y1, y3) > 1e-2
+
+
+def test_constant_per_head_is_plain_matmul():
+    B, T, H, N = 2, 9, 3, 4
+    C, r, k, v, _, _, _, _ = _inputs(B, T, H, N, 3)
+    w_head = torch.tensor([0.9, 0.5, 0.99], dtype=D)
+    u_head = torch.tensor([0.3, -0.2, 1.1], dtype=D)
+    y1 = O.wkv5_matmul_form(B, T, C, H, r, k, v, w_head, u_head)
+    w = w_head[:, None].expand(H, N).contiguous()
+    u = u_head[:, None].expand(H, N).contiguous()
+    y2, _ = O.wkv_recurrent(B, T, C, H, r, k, v, w, u)
+    assert err_ratio(y1, y2) < 1e-13
+
+
+def test_unit_decay_is_cumsum_linear_attention():
+    B, T, H, N = 2, 11, 2, 4
+    C, r, k, v, _, _, _, _ = _inputs(B, T, H, N, 4)
+    one = torch.ones(H, N, dtype=D)
+    y1 = O.linear_attention_cumsum(B, T, C, H, r, k, v)
+    y2, _ = O.wkv_recurrent(B, T, C, H, r, k, v, one, one)
+    assert err_ratio(y1, y2) < 1e-13
+
+
+def test_wkv6_time_constant_decay_equals_wkv5():
+    B, T, H, N = 2, 8, 2, 4
+    C, r, k, v, w_raw, u, gy, _ = _inputs(B, T, H, N, 5)
+    w5 = torch.exp(-torch.exp(w_raw[0, 0].reshape(H, N)))
+    w6 = w5.reshape(1, 1, C).expand(B, T, C).contiguous()
+    y5 = O.wkv5_sumform(B, T, C, H, r, k, v, w5, u)
+    y6 = O.wkv6_sumform(B, T, C, H, r, k, v, w6, u)
+    assert err_ratio(y5, y6) < 1e-13
+
+
+def test_state_handoff_equals_one_call():
+    B, T, H, N = 2, 12, 2, 4
+    C, r, k, v, w_raw, u, gy, s0 = _inputs(B, T, H, N, 6, state=True)
+    w = O.wkv6_decay(w_raw)
+    y, sT = O.wkv_recurrent(B, T, C, H, r, k, v, w, u, s0)
+    h = 5
+    ya, sa = O.wkv_recurrent(B, h, C, H, r[:, :h], k[:, :h], v[:, :h], w[:, :h], u, s0)
+    yb, sb = O.wkv_recurrent(B, T - h, C, H, r[:, h:], k[:, h:], v[:, h:], w[:, h:], u, sa)
+    assert err_ratio(y, torch.cat([ya, yb], 1)) < 1e-13
+    assert err_ratio(sT, sb) < 1e-13
+
+
+def _autograd_of_sumform(B, T, C, H, r, k, v, w_raw, u, gy, s0):
+    leaves = [x.clone().requires_grad_(True) for x in (r, k, v, w_raw, u)]
+    s_ = None if s0 is None else s0.clone().requires_grad_(True)
+    y = O.wkv6_sumform(B, T, C, H, leaves[0], leaves[1], leaves[2], O.wkv6_decay(leaves[3]), leaves[4], s_)
+    y.backward(gy)
+    return [x.grad for x in leaves] + ([] if s0 is None else [s_.grad])
+
+
+def test_hand_backward_vs_autograd_of_sumform():
+    for state in (False, True):
+        B, T, H, N = 2, 7, 2, 4
+        C, r, k, v, w_raw, u, gy, s0 = _inputs(B, T, H, N, 7, state=state)
+        ref = _autograd_of_sumform(B, T, C, H, r, k, v, w_raw, u, gy, s0)
+        w = O.wkv6_decay(w_raw)
+        gr, gk, gv, G, gu, gs = O.wkv_backward_hand(B, T, C, H, r, k, v, w, u, gy, s0)
+        gw = -torch.exp(w_raw) * G
+        for a, b in zip(ref[:5], (gr, gk, gv, gw, gu.sum(0))):
+            assert err_ratio(a, b) < 1e-12
+        if state:
+            assert err_ratio(ref[5], gs) < 1e-12
+        # invariants (w_{T-1} feeds nothing; w_0 multiplies S_0)
+        assert gw.reshape(B, T, C)[:, T - 1].abs().max() < 1e-13
+        g0 = ref[3].reshape(B, T, C)[:, 0].abs().max()
+        assert (g0 > 1e-3) if state else (g0 < 1e-13)
+
+
+def test_recurrent_autograd_vs_sumform_autograd():
+    B, T, H, N = 2, 6, 2, 4
+    C, r, k, v, w_raw, u, gy, s0 = _inputs(B, T, H, N, 8, state=True)
+    ref = _autograd_of_sumform(B, T, C, H, r, k, v, w_raw, u, gy, s0)
+    out = O.wkv6_grads(B, T, C, H, r, k, v, w_raw, u, gy, s0=s0)
+    for a, b in zip(ref, out[1:]):
+        assert err_ratio(a, b) < 1e-12
+    # per-batch partials sum to the parameter gradient
+    outp = O.wkv6_grads(B, T, C, H, r, k, v, w_raw, u, gy, s0=s0, per_batch=True)
+    assert err_ratio(ref[4], outp[5].sum(0)) < 1e-12
+
+
+def test_wkv5_grads_against_sumform_autograd():
+    B, T, H, N = 2, 7, 2, 4
+    C, r, k, v, w_raw, u, gy, _ = _inputs(B, T, H, N, 9)
+    w_raw5 = w_raw[0, 0].reshape(H, N).clone()
+    leaves = [x.clone().requires_grad_(True) for x in (r, k, v, w_raw5, u)]
+    y = O.wkv5_sumform(B, T, C, H, leaves[0], leaves[1], leaves[2], torch.exp(-torch.exp(leaves[3])), leaves[4])
+    y.backward(gy)
+    out = O.wkv5_grads(B, T, C, H, r, k, v, w_raw5, u, gy)
+    assert err_ratio(y.detach(), out[0]) < 1e-13
+    for a, b in zip(leaves, out[1:]):
+        assert err_ratio(a.grad, b) < 1e-12
+    outp = O.wkv5_grads(B, T, C, H, r, k, v, w_raw5, u, gy, per_batch=True)
+    assert err_ratio(leaves[3].grad, outp[4].sum(0)) < 1e-12
+
+
+def test_emulator_is_close_to_fp64_and_bf16_typed():
+    B, T, H, N = 2, 16, 2, 8
+    C, r, k, v, w_raw, u, gy, s0 = _inputs(B, T, H, N, 10, state=True)
+    rb = lambda x: x.to(torch.bfloat16)
+    rq, kq, vq, wq, uq, gq, sq = (rb(x) for x in (r, k, v, w_raw, u, gy, s0))
+    ref = O.wkv6_grads(B, T, C, H, rq, kq, vq, wq, uq, gq, s0=sq)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, rq, kq, vq, wq, uq, gq, s0=sq)
+    for a, b in zip(ref, emu):
+        assert b.dtype == torch.bfloat16
+        assert err_ratio(a, b.double()) < 6e-3
