@@ -54,12 +54,16 @@ int rwkv_abi_version(void);
  *   w[C]  = -exp(w_raw) (the wrapper's pre-transform, wkv/run.py:95), u[C], k,v,y,gy,gk,gv[B,T,C].
  *   gw,gu[B,C] are per-batch partials that the kernel ADDS into (caller zero-fills, as
  *   wkv/run.py:110-111 does); gw already carries the factor w of the w_raw chain rule.
+ *   The backward keeps its per-step intermediates in gk, gv and the workspace (B*T*C floats)
+ *   where the reference uses per-thread arrays of 4096 floats, so T is not limited.
  * ------------------------------------------------------------------------------------- */
 int rwkv_wkv4_forward(void* stream, int B, int T, int C,
                       const float* w, const float* u, const float* k, const float* v, float* y);
+size_t rwkv_wkv4_backward_workspace_bytes(int B, int T, int C);
 int rwkv_wkv4_backward(void* stream, int B, int T, int C,
                        const float* w, const float* u, const float* k, const float* v, const float* gy,
-                       float* gw, float* gu, float* gk, float* gv);
+                       float* gw, float* gu, float* gk, float* gv,
+                       void* workspace, size_t workspace_bytes);
 
 /* ---------------------------------------------------------------------------------------
  * depthwise_conv1d ("TimeX"), fp32.  Replaces cuda_forward / cuda_backward of

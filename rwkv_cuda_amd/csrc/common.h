@@ -72,6 +72,25 @@ template <int WIDTH> DEVINL float group_sum(float x) {
     return x;
 }
 
+// sum over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48); result in all four.
+// Two register-swap steps: permlane16_swap exchanges odd rows of one copy with even rows of
+// the other, permlane32_swap exchanges the wave halves; neither touches LDS.  The s_nop
+// covers the wait states a swap needs after a VALU write of its operands.
+DEVINL float allreduce_rows(float x) {
+#if RWKV_ROWSUM_SHFL
+    x += __shfl_xor(x, 16, 64);
+    x += __shfl_xor(x, 32, 64);
+    return x;
+#else
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    float s = a + b;
+    a = s; b = s;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return a + b;
+#endif
+}
+
 // ----------------------------------------------------------------------------- host checks
 extern thread_local int g_last_hip_error;
 

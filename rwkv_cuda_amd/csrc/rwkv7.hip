@@ -1,0 +1,337 @@
+// RWKV-7 "clamp-w" generalised delta rule with state passing, gfx950.
+//
+//   w_t = exp(-e^{-0.5} sigmoid(w_raw_t));  sa_t = S_t a_t;
+//   S_{t+1} = S_t diag(w_t) + sa_t b_t^T + v_t k_t^T;  y_t = S_{t+1} r_t;  sT = S_T        S[i][j]: i value, j key
+//
+// One workgroup of four waves per (batch, head); each wave owns 16 of the 64 state rows
+// (forward) so that every reduction the recurrence feeds back on stays inside a wave:
+//   layout H   wave q, lane l: row i = 16q + (l&15), columns j = 16(l>>4) + J,  J = 0..15 in VGPRs
+//   layout HT  wave q, lane l: column j = 16q + (l&15), rows i = 16(l>>4) + I,  I = 0..15 in VGPRs
+// A vector indexed by the in-register axis sits one element per lane (lane l holds element l) and
+// enters the FMAs through DPP row_newbcast; sums over the in-register axis are finished across the
+// four 16-lane rows with two register swaps (allreduce_rows).  Forward uses H only and needs no
+// barrier inside a chunk.  Backward keeps S and dS in HT (column sums dr, dw, dk, db, da) and a
+// second copy of dS in H (row sums dv and dSb = dS b); dSb is the only value that crosses waves,
+// once per step through LDS.
+//
+// Like the reference (rwkv7_statepassing_clampw.cu) the forward keeps sa_t and a state checkpoint
+// every 16 steps, and the backward recovers S_t inside a chunk by inverting the step.
+#include "common.h"
+
+namespace rwkv {
+namespace {
+
+constexpr int N = 64;
+constexpr int CL = RWKV7_CHUNK_LEN;   // 16: checkpoint interval = staging chunk
+constexpr int NW = 4;
+constexpr int NT = NW * 64;
+constexpr int JW = 16;
+constexpr float W_SCALE = -0.6065306597f;   // -exp(-0.5)
+
+struct Args7 {
+    int T, H;
+    const uint16_t *r, *w, *k, *v, *a, *b, *dy;
+    const float *s0, *dsT;
+    uint16_t *y, *dr, *dw, *dk, *dv, *da, *db;
+    float *sT, *ds0;
+    float* s;     // checkpoints [B,H,T/CL][j][i]
+    float* sa;    // [B,T,H,N]
+};
+
+DEVINL void unpack4(const uint2& q, float (&f)[4]) {
+    f[0] = bf_lo(q.x); f[1] = bf_hi(q.x); f[2] = bf_lo(q.y); f[3] = bf_hi(q.y);
+}
+DEVINL uint2 pack4(const float (&f)[4]) {
+    uint2 q;
+    q.x = pack_bf2(f[0], f[1]); q.y = pack_bf2(f[2], f[3]);
+    return q;
+}
+DEVINL void st4(float* dst, const float (&f)[4]) { *reinterpret_cast<float4*>(dst) = make_float4(f[0], f[1], f[2], f[3]); }
+DEVINL uint2 ldg4(const uint16_t* p) { return *reinterpret_cast<const uint2*>(p); }
+
+// ------------------------------------------------------------------------------------ forward
+struct SmemF {
+    float r[CL][N], w[CL][N], k[CL][N], v[CL][N], a[CL][N], b[CL][N];
+    float y[CL][N], sa[CL][N];
+};
+
+__global__ __launch_bounds__(NT) void rwkv7_fwd(const Args7 p) {
+    __shared__ SmemF S;
+    const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6, lo = lane & 15, hi = lane >> 4;
+    const int h = blockIdx.x, b = blockIdx.y, H = p.H, T = p.T;
+    const size_t bh = static_cast<size_t>(b) * H + h;
+    const int st = tid >> 4, sj = (tid & 15) * 4;
+    const int row = q * JW + lo;                                  // this lane's state row i
+    auto off = [&](int t) { return ((static_cast<size_t>(b) * T + t) * H + h) * N + sj; };
+
+    float St[JW];
+    {
+        const float* s0 = p.s0 + (bh * N + row) * N + hi * JW;
+#pragma unroll
+        for (int e = 0; e < JW; e += 4) {
+            const float4 x = *reinterpret_cast<const float4*>(s0 + e);
+            St[e] = x.x; St[e + 1] = x.y; St[e + 2] = x.z; St[e + 3] = x.w;
+        }
+    }
+
+    const int nchunks = T / CL;
+    uint2 gr, gw, gk, gv, ga, gb;
+    auto prefetch = [&](int c) {
+        const size_t o = off(c * CL + st);
+        gr = ldg4(p.r + o); gw = ldg4(p.w + o); gk = ldg4(p.k + o);
+        gv = ldg4(p.v + o); ga = ldg4(p.a + o); gb = ldg4(p.b + o);
+    };
+    prefetch(0);
+
+    for (int c = 0; c < nchunks; ++c) {
+        __syncthreads();
+        {
+            float f[4];
+            unpack4(gr, f); st4(&S.r[st][sj], f);
+            unpack4(gk, f); st4(&S.k[st][sj], f);
+            unpack4(gv, f); st4(&S.v[st][sj], f);
+            unpack4(ga, f); st4(&S.a[st][sj], f);
+            unpack4(gb, f); st4(&S.b[st][sj], f);
+            unpack4(gw, f);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f[e] = __expf(W_SCALE / (1.0f + __expf(-f[e])));
+            st4(&S.w[st][sj], f);
+        }
+        __syncthreads();
+        if (c + 1 < nchunks) prefetch(c + 1);
+
+#pragma unroll 2
+        for (int t = 0; t < CL; ++t) {
+            const float av = S.a[t][lane], bv = S.b[t][lane], kv = S.k[t][lane];
+            const float rv = S.r[t][lane], wv = S.w[t][lane], vi = S.v[t][row];
+            float sa = 0.f;
+            static_for<JW>([&](auto J) { fmac_bc<decltype(J)::value>(sa, av, St[decltype(J)::value]); });
+            sa = allreduce_rows(sa);
+            float y = 0.f;
+            static_for<JW>([&](auto J) {
+                constexpr int j = decltype(J)::value;
+                mul_bc<j>(St[j], wv);
+                fmac_bc<j>(St[j], bv, sa);
+                fmac_bc<j>(St[j], kv, vi);
+                fmac_bc<j>(y, rv, St[j]);
+            });
+            y = allreduce_rows(y);
+            if (hi == 0) { S.sa[t][row] = sa; S.y[t][row] = y; }
+        }
+        // checkpoint S_{(c+1) CL}, stored [j][i] so that the backward reads 16 consecutive rows per lane
+        {
+            float* chk = p.s + (bh * nchunks + c) * (N * N);
+#pragma unroll
+            for (int e = 0; e < JW; ++e) chk[(hi * JW + e) * N + row] = St[e];
+        }
+        __syncthreads();
+        {
+            const size_t o = off(c * CL + st);
+            float f[4] = {S.y[st][sj], S.y[st][sj + 1], S.y[st][sj + 2], S.y[st][sj + 3]};
+            *reinterpret_cast<uint2*>(p.y + o) = pack4(f);
+            *reinterpret_cast<float4*>(p.sa + o) = *reinterpret_cast<const float4*>(&S.sa[st][sj]);
+        }
+    }
+    {
+        float* sT = p.sT + (bh * N + row) * N + hi * JW;
+#pragma unroll
+        for (int e = 0; e < JW; e += 4)
+            *reinterpret_cast<float4*>(sT + e) = make_float4(St[e], St[e + 1], St[e + 2], St[e + 3]);
+    }
+}
+
+// ------------------------------------------------------------------------------------ backward
+struct SmemB {
+    float r[CL][N], w[CL][N], k[CL][N], v[CL][N], a[CL][N], b[CL][N], dy[CL][N], sa[CL][N];
+    float wf[CL][N];                       // d w / d w_raw = W_SCALE * w * sig * (1 - sig)
+    float dr[CL][N], dw[CL][N], dk[CL][N], dv[CL][N], da[CL][N], db[CL][N];
+    float dSb[2][N];
+};
+
+__global__ __launch_bounds__(NT) void rwkv7_bwd(const Args7 p) {
+    __shared__ SmemB S;
+    const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6, lo = lane & 15, hi = lane >> 4;
+    const int h = blockIdx.x, b = blockIdx.y, H = p.H, T = p.T;
+    const size_t bh = static_cast<size_t>(b) * H + h;
+    const int st = tid >> 4, sj = (tid & 15) * 4;
+    const int own = q * JW + lo;           // HT: this lane's column j;  H: this lane's row i
+    auto off = [&](int t) { return ((static_cast<size_t>(b) * T + t) * H + h) * N + sj; };
+
+    float ST[JW], dST[JW], dSH[JW];
+    {
+        const float* g = p.dsT + bh * N * N;
+#pragma unroll
+        for (int e = 0; e < JW; ++e) {
+            dST[e] = g[(hi * JW + e) * N + own];          // dS[i = 16hi+e][j = own]
+            ST[e] = 0.f;
+        }
+        const float* gh = g + own * N + hi * JW;           // dS[i = own][j = 16hi+e]
+#pragma unroll
+        for (int e = 0; e < JW; e += 4) {
+            const float4 x = *reinterpret_cast<const float4*>(gh + e);
+            dSH[e] = x.x; dSH[e + 1] = x.y; dSH[e + 2] = x.z; dSH[e + 3] = x.w;
+        }
+    }
+
+    const int nchunks = T / CL;
+    uint2 gr, gw, gk, gv, ga, gb, gdy;
+    float4 gsa;
+    auto prefetch = [&](int c) {
+        const size_t o = off(c * CL + st);
+        gr = ldg4(p.r + o); gw = ldg4(p.w + o); gk = ldg4(p.k + o); gv = ldg4(p.v + o);
+        ga = ldg4(p.a + o); gb = ldg4(p.b + o); gdy = ldg4(p.dy + o);
+        gsa = *reinterpret_cast<const float4*>(p.sa + o);
+    };
+    prefetch(nchunks - 1);
+
+    for (int c = nchunks - 1; c >= 0; --c) {
+        __syncthreads();
+        {
+            float f[4], g[4];
+            unpack4(gr, f); st4(&S.r[st][sj], f);
+            unpack4(gk, f); st4(&S.k[st][sj], f);
+            unpack4(gv, f); st4(&S.v[st][sj], f);
+            unpack4(ga, f); st4(&S.a[st][sj], f);
+            unpack4(gb, f); st4(&S.b[st][sj], f);
+            unpack4(gdy, f); st4(&S.dy[st][sj], f);
+            *reinterpret_cast<float4*>(&S.sa[st][sj]) = gsa;
+            unpack4(gw, f);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float sig = 1.0f / (1.0f + __expf(-f[e]));
+                const float w = __expf(W_SCALE * sig);
+                f[e] = w;
+                g[e] = W_SCALE * w * sig * (1.0f - sig);
+            }
+            st4(&S.w[st][sj], f);
+            st4(&S.wf[st][sj], g);
+        }
+        // S_{(c+1) CL} from the checkpoint, [j][i]: 16 consecutive rows of column `own`
+        {
+            const float* chk = p.s + (bh * nchunks + c) * (N * N) + own * N + hi * JW;
+#pragma unroll
+            for (int e = 0; e < JW; e += 4) {
+                const float4 x = *reinterpret_cast<const float4*>(chk + e);
+                ST[e] = x.x; ST[e + 1] = x.y; ST[e + 2] = x.z; ST[e + 3] = x.w;
+            }
+        }
+        __syncthreads();
+        if (c > 0) prefetch(c - 1);
+
+        for (int t = CL - 1; t >= 0; --t) {
+            const int par = t & 1;
+            // vectors, one element per lane
+            const float dyv = S.dy[t][lane], vv = S.v[t][lane], sav = S.sa[t][lane];
+            const float rv = S.r[t][lane], kv = S.k[t][lane], bv = S.b[t][lane], wv = S.w[t][lane], av = S.a[t][lane];
+            // scalars of this lane's own column (HT) / row (H)
+            const float rj = S.r[t][own], kj = S.k[t][own], bj = S.b[t][own], wj = S.w[t][own], aj = S.a[t][own];
+            const float dyi = S.dy[t][own];
+            const float nk = -kj, nb = -bj, iw = 1.0f / wj;
+
+            float drp = 0.f, dwp = 0.f, dkp = 0.f, dbp = 0.f, dvp = 0.f, dSbp = 0.f;
+            static_for<JW>([&](auto E) {
+                constexpr int e = decltype(E)::value;
+                // HT: column sums over i and the inverse step
+                fmac_bc<e>(drp, dyv, ST[e]);              // dr_j += dy_i S_{t+1}[i][j]
+                fmac_bc<e>(ST[e], vv, nk);                // S_t = (S_{t+1} - v_i k_j - sa_i b_j) / w_j
+                fmac_bc<e>(ST[e], sav, nb);
+                ST[e] *= iw;
+                fmac_bc<e>(dST[e], dyv, rj);              // dS += dy_i r_j
+                dwp = fmaf(dST[e], ST[e], dwp);
+                fmac_bc<e>(dkp, vv, dST[e]);
+                fmac_bc<e>(dbp, sav, dST[e]);
+                // H: row sums over j
+                fmac_bc<e>(dSH[e], rv, dyi);              // dS += dy_i r_j
+                fmac_bc<e>(dvp, kv, dSH[e]);
+                fmac_bc<e>(dSbp, bv, dSH[e]);
+            });
+            const float dSb = allreduce_rows(dSbp);
+            const float dv = allreduce_rows(dvp);
+            static_for<JW>([&](auto E) {
+                constexpr int e = decltype(E)::value;
+                mul_bc<e>(dSH[e], wv);                    // dS <- dS w_j + dSb_i a_j
+                fmac_bc<e>(dSH[e], av, dSb);
+            });
+            const float dr = allreduce_rows(drp), dw = allreduce_rows(dwp);
+            const float dk = allreduce_rows(dkp), db = allreduce_rows(dbp);
+            if (hi == 0) {
+                S.dSb[par][own] = dSb;
+                S.dv[t][own] = dv;
+                S.dr[t][own] = dr;
+                S.dw[t][own] = dw * S.wf[t][own];
+                S.dk[t][own] = dk;
+                S.db[t][own] = db;
+            }
+            __syncthreads();
+            const float dSbv = S.dSb[par][lane];
+            float dap = 0.f;
+            static_for<JW>([&](auto E) {
+                constexpr int e = decltype(E)::value;
+                fmac_bc<e>(dap, dSbv, ST[e]);             // da_j += S_t[i][j] dSb_i
+                dST[e] *= wj;                             // dS <- dS w_j + dSb_i a_j
+                fmac_bc<e>(dST[e], dSbv, aj);
+            });
+            const float da = allreduce_rows(dap);
+            if (hi == 0) S.da[t][own] = da;
+        }
+        __syncthreads();
+        {
+            const size_t o = off(c * CL + st);
+            auto put = [&](uint16_t* dst, const float (*src)[N]) {
+                float f[4] = {src[st][sj], src[st][sj + 1], src[st][sj + 2], src[st][sj + 3]};
+                *reinterpret_cast<uint2*>(dst + o) = pack4(f);
+            };
+            put(p.dr, S.dr); put(p.dw, S.dw); put(p.dk, S.dk);
+            put(p.dv, S.dv); put(p.da, S.da); put(p.db, S.db);
+        }
+    }
+    {
+        float* d = p.ds0 + (bh * N + own) * N + hi * JW;
+#pragma unroll
+        for (int e = 0; e < JW; e += 4)
+            *reinterpret_cast<float4*>(d + e) = make_float4(dSH[e], dSH[e + 1], dSH[e + 2], dSH[e + 3]);
+    }
+}
+
+int check7(int B, int T, int H) {
+    if (B <= 0 || T <= 0 || H <= 0) return RWKV_ERR_SHAPE;
+    if (T % CL != 0) return RWKV_ERR_SHAPE;
+    if (B > 65535) return RWKV_ERR_SHAPE;
+    return RWKV_OK;
+}
+
+}  // namespace
+}  // namespace rwkv
+
+using namespace rwkv;
+
+extern "C" {
+
+int rwkv7_statepassing_forward(void* stream, int B, int T, int H, const float* s0, const rwkv_bf16* r,
+                               const rwkv_bf16* w, const rwkv_bf16* k, const rwkv_bf16* v, const rwkv_bf16* a,
+                               const rwkv_bf16* b, rwkv_bf16* y, float* sT, float* s, float* sa) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({s0, r, w, k, v, a, b, y, sT, s, sa})) return e;
+    Args7 p{};
+    p.T = T; p.H = H; p.s0 = s0; p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b;
+    p.y = y; p.sT = sT; p.s = s; p.sa = sa;
+    hipLaunchKernelGGL(rwkv7_fwd, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status();
+}
+
+int rwkv7_statepassing_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w,
+                                const rwkv_bf16* k, const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b,
+                                const rwkv_bf16* dy, const float* dsT, const float* s, const float* sa,
+                                float* ds0, rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv,
+                                rwkv_bf16* da, rwkv_bf16* db) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db})) return e;
+    Args7 p{};
+    p.T = T; p.H = H; p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b; p.dy = dy; p.dsT = dsT;
+    p.s = const_cast<float*>(s); p.sa = const_cast<float*>(sa);
+    p.ds0 = ds0; p.dr = dr; p.dw = dw; p.dk = dk; p.dv = dv; p.da = da; p.db = db;
+    hipLaunchKernelGGL(rwkv7_bwd, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status();
+}
+
+}  // extern "C"
