@@ -75,7 +75,8 @@ def grads(B, T, C, w_raw, u, k, v, gy, dtype=torch.float64, per_batch=False):
         w_, u_ = (x.detach().to(dtype).clone().requires_grad_(True) for x in (w_raw, u))
     y = streaming(B, T, C, -torch.exp(w_), u_, k_, v_)
     y.backward(gy.to(dtype))
-    return y.detach(), w_.grad, u_.grad, k_.grad, v_.grad
+    zero = lambda x: torch.zeros_like(x) if x.grad is None else x.grad      # T == 1: w never reaches y
+    return y.detach(), zero(w_), zero(u_), zero(k_), zero(v_)
 
 
 def backward_kernel_order(B, T, C, w, u, k, v, gy):

@@ -188,6 +188,11 @@ def _leaf(x, dtype):
     return x.detach().to(dtype).clone().requires_grad_(True)
 
 
+def _grad(x):
+    # T == 1: the decay never reaches y and autograd leaves its grad unset
+    return torch.zeros_like(x) if x.grad is None else x.grad
+
+
 def wkv5_grads(B, T, C, H, r, k, v, w_raw, u, gy, dtype=torch.float64, per_batch=False):
     """y and (gr,gk,gv,gw_raw,gu) of wkv5 by autograd through the recurrent form.
     per_batch=True returns gw,gu as [B,H,N] partials (what the kernels write before the
@@ -202,7 +207,7 @@ def wkv5_grads(B, T, C, H, r, k, v, w_raw, u, gy, dtype=torch.float64, per_batch
         u_ = _leaf(u.reshape(H, N), dtype)
     y, _ = wkv_recurrent(B, T, C, H, r_, k_, v_, torch.exp(-torch.exp(w_)), u_)
     y.backward(gy.to(dtype))
-    return y.detach(), r_.grad, k_.grad, v_.grad, w_.grad, u_.grad
+    return y.detach(), _grad(r_), _grad(k_), _grad(v_), _grad(w_), _grad(u_)
 
 
 def wkv6_grads(B, T, C, H, r, k, v, w_raw, u, gy, s0=None, dtype=torch.float64, per_batch=False):
@@ -213,9 +218,9 @@ def wkv6_grads(B, T, C, H, r, k, v, w_raw, u, gy, s0=None, dtype=torch.float64, 
     s_ = None if s0 is None else _leaf(s0, dtype)
     y, _ = wkv_recurrent(B, T, C, H, r_, k_, v_, torch.exp(-torch.exp(w_)), u_, s_)
     y.backward(gy.to(dtype))
-    out = [y.detach(), r_.grad, k_.grad, v_.grad, w_.grad, u_.grad]
+    out = [y.detach(), _grad(r_), _grad(k_), _grad(v_), _grad(w_), _grad(u_)]
     if s0 is not None:
-        out.append(s_.grad)
+        out.append(_grad(s_))
     return out
 
 

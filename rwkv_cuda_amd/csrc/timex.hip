@@ -29,7 +29,7 @@ __global__ __launch_bounds__(1024) void timex_conv(const float* __restrict__ w, 
     const int c = blockIdx.x, b0 = blockIdx.y * BB, tid = threadIdx.x;
     const int nthr = T >> 2;
 
-    if (tid < 4) wr[tid] = 0.f;
+    for (int i = tid; i < 4; i += nthr) wr[i] = 0.f;
     for (int d = tid; d < T; d += nthr) wr[4 + d] = w[static_cast<size_t>(c) * T + (T - 1 - d)];
 #pragma unroll
     for (int r = 0; r < BB; ++r) {
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(1024) void timex_gw(const float* __restrict__ k, co
     const int tid = threadIdx.x;
     *reinterpret_cast<float4*>(ks + 4 * tid) = *reinterpret_cast<const float4*>(k + row * T + 4 * tid);
     *reinterpret_cast<float4*>(gs + 4 * tid) = *reinterpret_cast<const float4*>(g + row * T + 4 * tid);
-    if (tid < 4) gs[T + tid] = 0.f;
+    for (int i = tid; i < 4; i += (T >> 2)) gs[T + i] = 0.f;
     __syncthreads();
 
     const int d0 = 4 * tid;

@@ -1,0 +1,72 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header declares,
+and rejects bad arguments with status codes before anything reaches the GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from rwkv_cuda_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "rwkv_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rwkv7?_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_bindings_agree(lib):
+    names = _declared_symbols()
+    assert len(names) == 19
+    assert sorted(_lib.SIGNATURES) == names
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in rwkv_hip.h but not exported"
+
+
+def test_status_text(lib):
+    assert lib.rwkv_abi_version() == 1
+    assert lib.rwkv_strerror(0) == b"ok"
+    for code in (-1, -2, -3, -4, -5, -99):
+        assert len(lib.rwkv_strerror(code)) > 0
+
+
+def test_bad_arguments_are_rejected_without_a_launch(lib):
+    p = 0x1000  # never dereferenced: every call below fails validation first
+    # shapes
+    assert lib.rwkv_wkv6_forward(None, 0, 8, 64, 1, p, p, p, p, p, p) == -1
+    assert lib.rwkv_wkv6_forward(None, 1, 8, 96, 1, p, p, p, p, p, p) == -1          # C != H*64
+    assert lib.rwkv_wkv5_forward(None, 1, 8, 128, 1, p, p, p, p, p, p) == -1
+    assert lib.rwkv7_statepassing_forward(None, 1, 24, 1, *([p] * 11)) == -1         # T % 16
+    assert lib.rwkv_timex_forward(None, p, p, p, 0.0, 1, 1, 6) == -1                 # T % 4
+    assert lib.rwkv_wkv4_forward(None, 1, 0, 4, p, p, p, p, p) == -1
+    # null / misaligned pointers
+    assert lib.rwkv_wkv6_forward(None, 1, 8, 64, 1, p, p, None, p, p, p) == -2
+    assert lib.rwkv_wkv6state_forward(None, 1, 8, 64, 1, p, p, p, p, p, p + 2, p) == -3
+    assert lib.rwkv_wkv4_forward(None, 1, 4, 4, p, p, p, p, None) == -2
+    # workspace
+    need = lib.rwkv_wkv6state_backward_workspace_bytes(2, 8, 128, 2)
+    assert need == 2 * 8 * 128 * 4
+    assert lib.rwkv_wkv6state_backward(None, 2, 8, 128, 2, *([p] * 13), None, 0) == -4
+    assert lib.rwkv_wkv6state_backward(None, 2, 8, 128, 2, *([p] * 13), p, need - 1) == -4
+    assert lib.rwkv_wkv6_backward_workspace_bytes(1, 1, 96, 1) == 0
+    assert lib.rwkv_wkv4_backward(None, 1, 4, 4, *([p] * 9), None, 0) == -4
+    with pytest.raises(_lib.RwkvHipError):
+        _lib.check(-1)
+
+
+def test_ops_refuse_cpu_tensors():
+    from rwkv_cuda_amd import wkv6_state, wkv, rwkv7_fast_fused
+    bf = torch.bfloat16
+    B, T, H = 1, 16, 1
+    C = 64
+    x = torch.zeros(B, T, C, dtype=bf)
+    with pytest.raises(AssertionError):
+        wkv6_state.RUN_CUDA(B, T, C, H, x, x, x, x, torch.zeros(H, 64, dtype=bf), torch.zeros(B, H, 64, 64, dtype=bf))
+    with pytest.raises(AssertionError):
+        wkv.WKV.apply(B, T, C, torch.zeros(C), torch.zeros(C), x.float(), x.float())
+    x4 = x.view(B, T, H, 64)
+    with pytest.raises(AssertionError):
+        rwkv7_fast_fused.RWKV7_STATE_PASSING_CLAMPW_CUDA_OP.apply(torch.zeros(B, H, 64, 64), x4, x4, x4, x4, x4, x4)
