@@ -1,0 +1,341 @@
+#!/usr/bin/env python3
+"""Headline benchmark: WKV6 bf16 forward+backward at B=8, T=4096, C=2048 (H=32, N=64) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wkv6|wkv6_state|wkv5|rwkv7|wkv4|timex]
+
+A "step" is one forward + one backward of the operator over one batch of synthetic inputs that are
+already resident in HBM, through the same C-ABI calls and the same wrapper-side torch work
+(decay pre-transform, per-batch gradient sums) as the autograd.Function does.  Prints ONE JSON line.
+
+  value            whole-job throughput in Mtokens/s (tokens = B*T per step)
+  roofline         the slowest kernel of the step, timed alone with HIP events on the stream it is
+                   launched on: achieved = its algorithmic bytes / its mean duration, against 8 TB/s
+  cpu_baseline     the CPU oracle (a port of the reference's PyTorch recurrence, fp32, autograd) timed on
+                   this host's cores on a bounded sample (T_cpu steps of the same B, H, N)
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), keyed
+# by kernel label at the headline shape; None = not measured for the current kernels.
+TRAFFIC_MEASURED = {}
+
+
+def _events(n):
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def time_gpu(fn, iters, warmup):
+    """Mean milliseconds per call of fn, HIP events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    a, b = _events(2)
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
+# --------------------------------------------------------------------------------------------
+# workloads: each returns (step_fn, tokens_per_step, kernels, config, cpu_baseline_fn)
+# kernels: list of (label, fn, algorithmic_bytes) -- every kernel the step launches from the library
+# --------------------------------------------------------------------------------------------
+
+def make_wkv6(dev, state):
+    from rwkv_cuda_amd import _lib, synth
+    from rwkv_cuda_amd._call import call
+    lib = _lib.load()
+    B, T, H, N = 8, 4096, 32, 64
+    C = H * N
+    bf = torch.bfloat16
+    r, k, v, w, u, gy, s0 = (x.to(dev) if x is not None else None for x in synth.wkv6_inputs(B, T, C, H, seed=42, state=state))
+    new = lambda *s: torch.empty(s, device=dev, dtype=bf)
+    y, gr, gk, gv, gw, gu = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C), new(B, C)
+    nbytes = lib.rwkv_wkv6_backward_workspace_bytes(B, T, C, H)
+    ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+    tok = B * T
+    if state:
+        gs = new(B, H, N, N)
+
+        def step():
+            call("rwkv_wkv6state_forward", dev, B, T, C, H, r, k, v, w, u, s0, y)
+            call("rwkv_wkv6state_backward", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes)
+            return torch.sum(gu, 0).view(H, N)
+
+        kernels = [("wkv6state forward", lambda: call("rwkv_wkv6state_forward", dev, B, T, C, H, r, k, v, w, u, s0, y), 10 * C * tok),
+                   ("wkv6state backward (3 kernels)", lambda: call("rwkv_wkv6state_backward", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes), 18 * C * tok)]
+        name = "wkv6_state"
+    else:
+        ew_keep = (-torch.exp(w.float())).contiguous()
+
+        def step():
+            ew = (-torch.exp(w.float())).contiguous()               # wrapper pre-transform, wkv6/run.py:147
+            call("rwkv_wkv6_forward", dev, B, T, C, H, r, k, v, ew, u, y)
+            call("rwkv_wkv6_backward", dev, B, T, C, H, r, k, v, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+            return torch.sum(gu, 0).view(H, N)                      # wrapper reduction, wkv6/run.py:169
+
+        def bwd(mask):
+            return lambda: call("rwkv_wkv6_backward_passes", dev, B, T, C, H, r, k, v, ew_keep, u, gy, gr, gk, gv, gw, gu, ws, nbytes, mask)
+
+        # algorithmic bytes per kernel: tensors it must read once + outputs it must write once (bf16 = 2 B/elt;
+        # the decay counts 2 B/elt as in the 28*C figure even though this entry point receives it as fp32)
+        kernels = [("wkv6 forward  wkv_sweep<FWD>", lambda: call("rwkv_wkv6_forward", dev, B, T, C, H, r, k, v, ew_keep, u, y), 10 * C * tok),
+                   ("wkv6 backward wkv_sweep<GR>", bwd(1), 12 * C * tok),     # r k v w gy -> gr
+                   ("wkv6 backward wkv_sweep<GV>", bwd(2), 10 * C * tok),     # r k w gy -> gv
+                   ("wkv6 backward wkv_sweep<GK>", bwd(4), 14 * C * tok)]     # r k v w gy -> gk gw
+        name = "wkv6"
+
+    def cpu_baseline(t_cpu=256):
+        from oracle import wkv56 as O
+        rr, kk, vv, ww, uu, gg, ss = synth.wkv6_inputs(B, t_cpu, C, H, seed=42, state=state)
+        f = torch.float32
+        t0 = time.perf_counter()
+        O.wkv6_grads(B, t_cpu, C, H, rr.float(), kk.float(), vv.float(), ww.float(), uu.float(), gg.float(),
+                     s0=None if ss is None else ss.float(), dtype=f)
+        dt = time.perf_counter() - t0
+        return B * t_cpu / dt / 1e6, f"{name} fwd+bwd, fp32 autograd of the recurrent form, B{B} H{H} N{N}, T_cpu={t_cpu} ({dt:.1f} s)"
+
+    cfg = {"workload": f"{name} bf16 fwd+bwd B{B} T{T} C{C} H{H} N{N}", "B": B, "T": T, "C": C, "H": H, "N": N,
+           "algorithmic_bytes_per_token": 28 * C}
+    return step, tok, kernels, cfg, cpu_baseline, 28 * C * tok
+
+
+def make_wkv5(dev):
+    from rwkv_cuda_amd import _lib, synth
+    from rwkv_cuda_amd._call import call
+    lib = _lib.load()
+    B, T, H, N = 8, 4096, 32, 64
+    C = H * N
+    bf = torch.bfloat16
+    r, k, v, w, u, gy = (x.to(dev) for x in synth.wkv5_inputs(B, T, C, H, seed=42))
+    new = lambda *s: torch.empty(s, device=dev, dtype=bf)
+    y, gr, gk, gv, gw, gu = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C), new(B, C), new(B, C)
+    nbytes = lib.rwkv_wkv5_backward_workspace_bytes(B, T, C, H)
+    ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+    tok = B * T
+    ew = (-torch.exp(w.float())).contiguous()
+    eew = torch.exp(ew).contiguous()
+
+    def step():
+        ew_ = (-torch.exp(w.float())).contiguous()
+        eew_ = torch.exp(ew_).contiguous()
+        call("rwkv_wkv5_forward", dev, B, T, C, H, r, k, v, eew_, u, y)
+        call("rwkv_wkv5_backward", dev, B, T, C, H, r, k, v, eew_, ew_, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+        return torch.sum(gw, 0), torch.sum(gu, 0)
+
+    kernels = [("wkv5 forward", lambda: call("rwkv_wkv5_forward", dev, B, T, C, H, r, k, v, eew, u, y), 8 * C * tok),
+               ("wkv5 backward (3 kernels)", lambda: call("rwkv_wkv5_backward", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes), 14 * C * tok)]
+
+    def cpu_baseline(t_cpu=256):
+        from oracle import wkv56 as O
+        rr, kk, vv, ww, uu, gg = synth.wkv5_inputs(B, t_cpu, C, H, seed=42)
+        t0 = time.perf_counter()
+        O.wkv5_grads(B, t_cpu, C, H, rr.float(), kk.float(), vv.float(), ww.float(), uu.float(), gg.float(), dtype=torch.float32)
+        dt = time.perf_counter() - t0
+        return B * t_cpu / dt / 1e6, f"wkv5 fwd+bwd, fp32 autograd of the recurrent form, B{B} H{H} N{N}, T_cpu={t_cpu} ({dt:.1f} s)"
+
+    cfg = {"workload": f"wkv5 bf16 fwd+bwd B{B} T{T} C{C} H{H} N{N}", "B": B, "T": T, "C": C, "H": H, "N": N,
+           "algorithmic_bytes_per_token": 22 * C}
+    return step, tok, kernels, cfg, cpu_baseline, 22 * C * tok
+
+
+def make_rwkv7(dev):
+    from rwkv_cuda_amd import synth
+    from rwkv_cuda_amd._call import call
+    B, T, H, N = 8, 4096, 64, 64
+    C = H * N
+    TS = T // 4                                                   # four chained T=1024 calls
+    s0, r, w, k, v, a, b, dy, dsT = (x.to(dev) for x in synth.rwkv7_inputs(B, T, H, N, seed=42))
+    seg = [[x[:, i * TS:(i + 1) * TS].contiguous() for x in (r, w, k, v, a, b, dy)] for i in range(4)]
+    f32 = dict(device=dev, dtype=torch.float32)
+    ys = [torch.empty_like(s[0]) for s in seg]
+    sTs = [torch.empty_like(s0) for _ in range(4)]
+    ss = [torch.empty(B, H, TS // 16, N, N, **f32) for _ in range(4)]
+    sas = [torch.empty(B, TS, H, N, **f32) for _ in range(4)]
+    grads = [[torch.empty_like(s[0]) for _ in range(6)] for s in seg]
+    ds = [torch.empty_like(s0) for _ in range(4)]
+    tok = B * T
+
+    def fwd():
+        st = s0
+        for i in range(4):
+            rr, ww, kk, vv, aa, bb, _ = seg[i]
+            call("rwkv7_statepassing_forward", dev, B, TS, H, st, rr, ww, kk, vv, aa, bb, ys[i], sTs[i], ss[i], sas[i])
+            st = sTs[i]
+
+    def bwd():
+        g = dsT
+        for i in (3, 2, 1, 0):
+            rr, ww, kk, vv, aa, bb, dd = seg[i]
+            call("rwkv7_statepassing_backward", dev, B, TS, H, rr, ww, kk, vv, aa, bb, dd, g, ss[i], sas[i], ds[i], *grads[i])
+            g = ds[i]
+
+    def step():
+        fwd()
+        bwd()
+
+    kernels = [("rwkv7 forward x4 (T=1024 each)", fwd, 14 * C * tok), ("rwkv7 backward x4", bwd, 26 * C * tok)]
+
+    def cpu_baseline(t_cpu=64):
+        from oracle import rwkv7 as O
+        args = synth.rwkv7_inputs(B, t_cpu, H, N, seed=42)
+        t0 = time.perf_counter()
+        O.grads(*[x.float() for x in args], dtype=torch.float32)
+        dt = time.perf_counter() - t0
+        return B * t_cpu / dt / 1e6, f"rwkv7 fwd+bwd, fp32 autograd of the einsum step, B{B} H{H} N{N}, T_cpu={t_cpu} ({dt:.1f} s)"
+
+    cfg = {"workload": f"rwkv7 state-passing bf16 fwd+bwd B{B} T{T} (4 x {TS}) C{C} H{H} N{N}", "B": B, "T": T, "C": C,
+           "H": H, "N": N, "algorithmic_bytes_per_token": 40 * C}
+    return step, tok, kernels, cfg, cpu_baseline, 40 * C * tok
+
+
+def make_wkv4(dev):
+    from rwkv_cuda_amd import _lib, synth
+    from rwkv_cuda_amd._call import call
+    lib = _lib.load()
+    B, T, C = 4, 512, 768
+    w_raw, u, k, v, gy = (x.to(dev) for x in synth.wkv4_inputs(B, T, C, seed=42))
+    y, gk, gv = (torch.empty(B, T, C, device=dev) for _ in range(3))
+    nbytes = lib.rwkv_wkv4_backward_workspace_bytes(B, T, C)
+    ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+    tok = B * T
+    w_keep = -torch.exp(w_raw)
+    gwz, guz = torch.zeros(B, C, device=dev), torch.zeros(B, C, device=dev)
+
+    def step():
+        w = -torch.exp(w_raw)
+        call("rwkv_wkv4_forward", dev, B, T, C, w, u, k, v, y)
+        gw, gu = torch.zeros(B, C, device=dev), torch.zeros(B, C, device=dev)
+        call("rwkv_wkv4_backward", dev, B, T, C, w, u, k, v, gy, gw, gu, gk, gv, ws, nbytes)
+        return gw.sum(0), gu.sum(0)
+
+    kernels = [("wkv4 forward", lambda: call("rwkv_wkv4_forward", dev, B, T, C, w_keep, u, k, v, y), 12 * C * tok),
+               ("wkv4 backward", lambda: call("rwkv_wkv4_backward", dev, B, T, C, w_keep, u, k, v, gy, gwz, guz, gk, gv, ws, nbytes), 20 * C * tok)]
+
+    def cpu_baseline():
+        from oracle import wkv4 as O
+        ww, uu, kk, vv, gg = synth.wkv4_inputs(B, T, C, seed=42)
+        t0 = time.perf_counter()
+        kk_, vv_, ww_, uu_ = (x.clone().requires_grad_(True) for x in (kk, vv, ww, uu))
+        O.conv_form(B, T, C, ww_, uu_, kk_, vv_).backward(gg)
+        dt = time.perf_counter() - t0
+        return B * T / dt / 1e6, f"wkv4 fwd+bwd, grouped F.conv1d formulation, fp32, full B{B} T{T} C{C} ({dt:.1f} s)"
+
+    cfg = {"workload": f"wkv4 fp32 fwd+bwd B{B} T{T} C{C}", "B": B, "T": T, "C": C, "algorithmic_bytes_per_token": 32 * C}
+    return step, tok, kernels, cfg, cpu_baseline, 32 * C * tok
+
+
+def make_timex(dev):
+    from rwkv_cuda_amd import synth
+    from rwkv_cuda_amd._call import call
+    B, C, T = 32, 768, 768
+    w, k, g = (x.to(dev) for x in synth.timex_inputs(B, C, T, seed=42))
+    x, gw, gk = (torch.empty(B, C, T, device=dev) for _ in range(3))
+    tok = B * T
+
+    def step():
+        call("rwkv_timex_forward", dev, w, k, x, 0.0, B, C, T)
+        call("rwkv_timex_backward", dev, w, k, g, gw, gk, B, C, T)
+        return gw.sum(0)
+
+    fwd_bytes = (C * T + 2 * B * C * T) * 4
+    bwd_bytes = (C * T + 4 * B * C * T) * 4
+    kernels = [("timex forward", lambda: call("rwkv_timex_forward", dev, w, k, x, 0.0, B, C, T), fwd_bytes),
+               ("timex backward (2 kernels)", lambda: call("rwkv_timex_backward", dev, w, k, g, gw, gk, B, C, T), bwd_bytes)]
+
+    def cpu_baseline(bs=4):
+        from oracle import timex as O
+        ww, kk, gg = synth.timex_inputs(bs, C, T, seed=42)
+        t0 = time.perf_counter()
+        O.grads(ww, kk, gg, bs, C, T, dtype=torch.float32)
+        dt = time.perf_counter() - t0
+        return bs * T / dt / 1e6, f"depthwise_conv1d fwd+bwd, zero-padded grouped F.conv1d, fp32, B={bs} of 32, C{C} T{T} ({dt:.1f} s)"
+
+    cfg = {"workload": f"depthwise_conv1d fp32 fwd+bwd B{B} C{C} T{T}", "B": B, "C": C, "T": T,
+           "algorithmic_bytes_per_step": fwd_bytes + bwd_bytes}
+    return step, tok, kernels, cfg, cpu_baseline, fwd_bytes + bwd_bytes
+
+
+WORKLOADS = {
+    "wkv6": lambda dev: make_wkv6(dev, False),
+    "wkv6_state": lambda dev: make_wkv6(dev, True),
+    "wkv5": make_wkv5,
+    "rwkv7": make_rwkv7,
+    "wkv4": make_wkv4,
+    "timex": make_timex,
+}
+DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "rwkv7": "bf16", "wkv4": "f32", "timex": "f32"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="wkv6", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; every (batch, head) is an independent unit and no "
+                 "multi-GPU path exists, so --gpus must be 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no HIP device visible; the kernels have no CPU path")
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    step, tok, kernels, cfg, cpu_baseline, step_bytes = WORKLOADS[args.workload](dev)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = 1e3 * dt / args.steps
+    mtok = tok / (dt / args.steps) / 1e6
+
+    # per-kernel timing, HIP events on the launch stream
+    per_kernel = []
+    for label, fn, nbytes in kernels:
+        ms = time_gpu(fn, max(5, args.steps), 2)
+        per_kernel.append({"kernel": label, "ms": round(ms, 4), "algorithmic_bytes": nbytes,
+                           "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)})
+    dom = max(per_kernel, key=lambda d: d["ms"])
+    roofline = {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(dom["GBps"] / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_MEASURED.get(dom["kernel"]),
+                "launch_ms": dom["ms"], "algorithmic_bytes": dom["algorithmic_bytes"],
+                "whole_step_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+    out = {
+        "metric": "WKV6 bf16 fwd+bwd Mtokens/s @B8 T4096 C2048; % HBM peak achieved" if args.workload == "wkv6"
+                  else f"{args.workload} fwd+bwd Mtokens/s; % HBM peak achieved",
+        "value": round(mtok, 3), "unit": "Mtokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": DTYPES[args.workload], "data": "synthetic", "config": cfg,
+        "pct_hbm_peak": round(100 * step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+        "roofline": roofline, "kernels": per_kernel,
+    }
+    if not args.no_cpu_baseline:
+        val, sample = cpu_baseline()
+        out["cpu_baseline"] = {"value": round(val, 5), "unit": "Mtokens/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": sample, "host_cpus": os.cpu_count()}
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -109,6 +109,19 @@ int rwkv_wkv6_backward(void* stream, int B, int T, int C, int H,
                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                        void* workspace, size_t workspace_bytes);
 
+/* The same backward restricted to a subset of its kernels, so that a profiler can time one
+ * kernel per call (no counterpart in the reference).  RWKV_PASS_GK reads what RWKV_PASS_GR
+ * left in the workspace; RWKV_PASS_ALL is rwkv_wkv6_backward. */
+#define RWKV_PASS_GR 1u  /* gr, gu, workspace */
+#define RWKV_PASS_GV 2u  /* gv */
+#define RWKV_PASS_GK 4u  /* gk, gw */
+#define RWKV_PASS_ALL 7u
+int rwkv_wkv6_backward_passes(void* stream, int B, int T, int C, int H,
+                              const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                              const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
+                              rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                              void* workspace, size_t workspace_bytes, unsigned passes);
+
 /* ---------------------------------------------------------------------------------------
  * RWKV-6 wkv with initial state.  Replaces cuda_forward / cuda_backward of
  * wkv6_state/cuda/wkv6state_op.cpp:5-6 (kernels: wkv6state_cuda_v1a.cu:6-308).

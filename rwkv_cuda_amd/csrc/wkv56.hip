@@ -322,10 +322,11 @@ template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a) {
 }
 
 // GR and GV are independent; GK consumes GR's workspace.  All three run on `st` in order.
-template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a) {
-    hipLaunchKernelGGL((wkv_sweep<P_GR, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
-    hipLaunchKernelGGL((wkv_sweep<P_GV, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
-    hipLaunchKernelGGL((wkv_sweep<P_GK, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
+// `passes` is a bit mask (RWKV_PASS_*) so that a profiler can time one kernel at a time.
+template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a, unsigned passes = RWKV_PASS_ALL) {
+    if (passes & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
+    if (passes & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
+    if (passes & RWKV_PASS_GK) hipLaunchKernelGGL((wkv_sweep<P_GK, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
     return launch_status();
 }
 
@@ -387,13 +388,21 @@ int rwkv_wkv6_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16
                        const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                        void* workspace, size_t workspace_bytes) {
+    return rwkv_wkv6_backward_passes(stream, B, T, C, H, r, k, v, ew, u, gy, gr, gk, gv, gw, gu, workspace,
+                                     workspace_bytes, RWKV_PASS_ALL);
+}
+
+int rwkv_wkv6_backward_passes(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                              const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
+                              rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                              void* workspace, size_t workspace_bytes, unsigned passes) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, ew, u, gy, gr, gk, gv, gw, gu})) return e;
     if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
-    return launch_bwd<W_EW>(static_cast<hipStream_t>(stream), B, a);
+    return launch_bwd<W_EW>(static_cast<hipStream_t>(stream), B, a, passes);
 }
 
 int rwkv_wkv6state_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
