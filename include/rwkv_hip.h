@@ -48,6 +48,13 @@ int rwkv_last_hip_error(void);
 /* ABI version of this header (bumped when a signature changes). */
 int rwkv_abi_version(void);
 
+/* Which kernels serve wkv6 / wkv6_state (process-wide; meant for tests and profiling, no counterpart
+ * in the reference).  CHUNKED (default): chunked formulation on the matrix cores.  SWEEPS: the
+ * sequential fp32 recurrence kernels, which also serve wkv5. */
+#define RWKV_ALGO_CHUNKED 0
+#define RWKV_ALGO_SWEEPS 1
+int rwkv_wkv6_set_algorithm(int algo);
+
 /* ---------------------------------------------------------------------------------------
  * RWKV-4 wkv, fp32.  Replaces cuda_forward / cuda_backward of wkv/cuda/wkv_op.cpp:3-4
  * (kernels: wkv/cuda/wkv_cuda_v2.cu:4-130).

@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 _INCLUDE = os.path.join(_ROOT, "include")
 LIB_PATH = os.path.join(_HERE, "librwkv_hip.so")
 
-SOURCES = ["abi.hip", "wkv56.hip", "wkv4.hip", "timex.hip", "rwkv7.hip"]
+SOURCES = ["abi.hip", "wkv56.hip", "wkv6_chunk.hip", "wkv4.hip", "timex.hip", "rwkv7.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -53,6 +53,7 @@ SIGNATURES = {
     "rwkv_strerror": (ctypes.c_char_p, [_I]),
     "rwkv_last_hip_error": (_I, []),
     "rwkv_abi_version": (_I, []),
+    "rwkv_wkv6_set_algorithm": (_I, [_I]),
     "rwkv_wkv4_forward": (_I, [_P, _I, _I, _I] + [_P] * 5),
     "rwkv_wkv4_backward_workspace_bytes": (_Z, [_I, _I, _I]),
     "rwkv_wkv4_backward": (_I, [_P, _I, _I, _I] + [_P] * 9 + [_P, _Z]),

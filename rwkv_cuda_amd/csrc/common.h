@@ -108,4 +108,11 @@ inline int launch_status() {
     return RWKV_OK;
 }
 
+// ----------------------------------------------------------------------------- internal launchers
+// wkv6_chunk.hip: chunked MFMA kernels.  wmode: 1 = fp32 ew [B,T,C], 2 = raw bf16 w.
+int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
+                          const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
+                          const uint16_t* s0, uint16_t* y);
+extern int g_wkv6_algorithm;     // RWKV_ALGO_*
+
 }  // namespace rwkv

@@ -378,6 +378,8 @@ int rwkv_wkv6_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16*
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, ew, u, y})) return e;
     Args a{};
+    if (g_wkv6_algorithm == RWKV_ALGO_CHUNKED)
+        return launch_wkv6_fwd_chunk(static_cast<hipStream_t>(stream), W_EW, B, T, C, H, r, k, v, ew, u, nullptr, y);
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.y = y;
     return launch_fwd<W_EW>(static_cast<hipStream_t>(stream), B, a);
 }
@@ -411,6 +413,8 @@ int rwkv_wkv6state_forward(void* stream, int B, int T, int C, int H, const rwkv_
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, w, u, s, y})) return e;
     Args a{};
+    if (g_wkv6_algorithm == RWKV_ALGO_CHUNKED)
+        return launch_wkv6_fwd_chunk(static_cast<hipStream_t>(stream), W_RAW, B, T, C, H, r, k, v, w, u, s, y);
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.y = y;
     return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a);
 }
