@@ -287,6 +287,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="wkv6", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--algo", default="chunked", choices=["chunked", "sweeps"],
+                    help="wkv6 kernels: chunked MFMA formulation (default) or the sequential fp32 sweeps")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so that a rocprofv3 --pmc run holds a kernel of known traffic")
     args = ap.parse_args()
@@ -298,6 +300,8 @@ def main():
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    from rwkv_cuda_amd import _lib
+    _lib.check(_lib.load().rwkv_wkv6_set_algorithm(0 if args.algo == "chunked" else 1))
     step, tok, kernels, cfg, cpu_baseline, step_bytes = WORKLOADS[args.workload](dev)
 
     if args.calibrate_copy:

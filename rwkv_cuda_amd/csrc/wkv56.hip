@@ -1,9 +1,9 @@
 // wkv5 / wkv6 / wkv6_state for gfx950: sequential-in-time sweeps with the 64x64 state in VGPRs.
 //
-// One workgroup (4 waves) per (batch, head).  The state S[i][j] (i = value channel, j = key
+// One workgroup (8 waves) per (batch, head).  The state S[i][j] (i = value channel, j = key
 // channel) is tiled 16 elements per lane in one of two ways:
-//   shape F  lane = i, wave q holds j in [16q,16q+16)   out[i] = sum_j a[j] S[i][j];  S = S w[j] + b[j] x[i]
-//   shape G  lane = j, wave q holds i in [16q,16q+16)   out[j] = sum_i a[i] S[i][j];  S = S w[j] + x[i] b[j]
+//   shape F  lane = i, wave q holds j in [8q,8q+8)   out[i] = sum_j a[j] S[i][j];  S = S w[j] + b[j] x[i]
+//   shape G  lane = j, wave q holds i in [8q,8q+8)   out[j] = sum_i a[i] S[i][j];  S = S w[j] + x[i] b[j]
 // Vectors indexed by the in-register axis are kept one element per lane, replicated in every
 // 16-lane DPP row, and enter the FMAs through row_newbcast, so a step is 3 VALU ops per state
 // element and four LDS reads per lane.  Inputs are staged through LDS as fp32 in chunks of
@@ -26,11 +26,12 @@ namespace {
 
 constexpr int N = 64;            // head size
 constexpr int TC = 32;           // time steps per staged chunk
-constexpr int NW = 4;            // waves per workgroup
+constexpr int NW = 8;            // waves per workgroup: two per SIMD (one wave per SIMD issues VALU ~3x slower)
 constexpr int NT = NW * 64;
 constexpr int JW = N / NW;       // state elements per lane
-static_assert(JW == 16, "row broadcast assumes 16 state elements per lane");
-static_assert(TC * N == NT * 8, "staging assumes 8 elements per thread per tensor");
+constexpr int NSTAGE = TC * N / 8;   // threads that stage / finish a chunk (8 elements each)
+static_assert(JW <= 16 && (JW & (JW - 1)) == 0, "row broadcast: the state elements of a lane must fit one 16-lane row");
+static_assert(NSTAGE <= NT && NSTAGE % 64 == 0, "staging threads are whole waves");
 
 enum { P_FWD = 0, P_GR = 1, P_GK = 2, P_GV = 3 };
 enum { W_HEAD = 0, W_EW = 1, W_RAW = 2 };   // wkv5 (eew[H,N] fp32) / wkv6 (ew fp32 [B,T,C]) / wkv6_state (raw bf16)
@@ -151,7 +152,7 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
     const int st = tid >> 3, sj = (tid & 7) * 8;            // staging / epilogue coordinates
-    const int rowslot = q * JW + (lane & 15);               // element of a broadcast vector held by this lane
+    const int rowslot = q * JW + (lane & (JW - 1));         // element of a broadcast vector held by this lane
     const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
     const size_t bh = static_cast<size_t>(b) * a.H + h;
     const bool stateful = a.s0 != nullptr;
@@ -164,12 +165,12 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     for (int e = 0; e < JW; ++e) St[e] = 0.f;
     if (stateful) {
         if constexpr (PASS == P_FWD) {
-            const uint16_t* s = a.s0 + (bh * N + lane) * N + q * JW;        // row i = lane, 16 consecutive j
-            float lo[8], hi[8];
+            const uint16_t* s = a.s0 + (bh * N + lane) * N + q * JW;        // row i = lane, JW consecutive j
+            static_assert(JW == 8, "one 16-byte load per lane");
+            float lo[8];
             unpack8(*reinterpret_cast<const uint4*>(s), lo);
-            unpack8(*reinterpret_cast<const uint4*>(s + 8), hi);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { St[e] = lo[e]; St[8 + e] = hi[e]; }
+            for (int e = 0; e < 8; ++e) St[e] = lo[e];
         } else if constexpr (PASS == P_GR) {
 #pragma unroll
             for (int e = 0; e < JW; ++e) St[e] = bf2f(a.s0[(bh * N + q * JW + e) * N + lane]);
@@ -188,16 +189,17 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     float P = 0.f, gw_acc = 0.f;                            // GK scan state (threads < 64)
 
     const int nchunks = (a.T + TC - 1) / TC;
+    const bool stager = tid < NSTAGE;                       // whole waves
     Staged pre;
-    prefetch<PASS, WMODE>(pre, a, base, (REV ? nchunks - 1 : 0) * TC, st, sj);
+    if (stager) prefetch<PASS, WMODE>(pre, a, base, (REV ? nchunks - 1 : 0) * TC, st, sj);
     __syncthreads();                                        // S.u visible
 
     for (int ci = 0; ci < nchunks; ++ci) {
         const int c0 = (REV ? nchunks - 1 - ci : ci) * TC;
         __syncthreads();                                    // previous epilogue is done with LDS
-        commit<PASS, WMODE>(S, pre, a, c0, st, sj);
+        if (stager) commit<PASS, WMODE>(S, pre, a, c0, st, sj);
         __syncthreads();
-        if (ci + 1 < nchunks) prefetch<PASS, WMODE>(pre, a, base, (REV ? nchunks - 2 - ci : ci + 1) * TC, st, sj);
+        if (stager && ci + 1 < nchunks) prefetch<PASS, WMODE>(pre, a, base, (REV ? nchunks - 2 - ci : ci + 1) * TC, st, sj);
 
         // ---- TC sequential steps
 #pragma unroll 4
@@ -229,34 +231,34 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
         }
         __syncthreads();
 
-        // ---- chunk epilogue: thread (st, sj..sj+7)
-        const bool ok = (c0 + st) < a.T;
-        const size_t off = base + static_cast<size_t>(c0 + st) * a.C + sj;
+        // ---- chunk epilogue: thread (st, sj..sj+7) of the staging waves
+        const bool ok = stager && (c0 + st) < a.T;
+        const int es = stager ? st : 0;                       // the other waves only keep the barriers company
+        const size_t off = base + static_cast<size_t>(c0 + es) * a.C + sj;
         float sum[8];
-        {
-            float p1[8], p2[8], p3[8];
-            ld8f(&S.part[0][st][sj], sum);
-            ld8f(&S.part[1][st][sj], p1);
-            ld8f(&S.part[2][st][sj], p2);
-            ld8f(&S.part[3][st][sj], p3);
+        ld8f(&S.part[0][es][sj], sum);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) sum[e] = (sum[e] + p1[e]) + (p2[e] + p3[e]);
+        for (int w = 1; w < NW; ++w) {
+            float p1[8];
+            ld8f(&S.part[w][es][sj], p1);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sum[e] += p1[e];
         }
-        const float dot = S.dot[st];
+        const float dot = S.dot[es];
         float out[8];
         if constexpr (PASS == P_FWD) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) out[e] = fmaf(S.v[st][sj + e], dot, sum[e]);
+            for (int e = 0; e < 8; ++e) out[e] = fmaf(S.v[es][sj + e], dot, sum[e]);
             if (ok) *reinterpret_cast<uint4*>(a.y + off) = pack8(out);
         } else if constexpr (PASS == P_GV) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) out[e] = fmaf(S.g[st][sj + e], dot, sum[e]);
+            for (int e = 0; e < 8; ++e) out[e] = fmaf(S.g[es][sj + e], dot, sum[e]);
             if (ok) *reinterpret_cast<uint4*>(a.gv + off) = pack8(out);
         } else if constexpr (PASS == P_GR) {
             float rdr[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float rr = S.r[st][sj + e], kk = S.k[st][sj + e];
+                const float rr = S.r[es][sj + e], kk = S.k[es][sj + e];
                 out[e] = fmaf(S.u[sj + e] * kk, dot, sum[e]);
                 rdr[e] = rr * sum[e];
                 gu_acc[e] = fmaf(rr * kk, dot, gu_acc[e]);
@@ -270,11 +272,11 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
             float kdk[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                out[e] = fmaf(S.u[sj + e] * S.r[st][sj + e], dot, sum[e]);
-                kdk[e] = S.k[st][sj + e] * sum[e];
+                out[e] = fmaf(S.u[sj + e] * S.r[es][sj + e], dot, sum[e]);
+                kdk[e] = S.k[es][sj + e] * sum[e];
             }
             if (ok) *reinterpret_cast<uint4*>(a.gk + off) = pack8(out);
-            st8(&S.k[st][sj], kdk);                          // k is no longer needed: keep k*dk' there
+            if (stager) st8(&S.k[st][sj], kdk);              // k is no longer needed: keep k*dk' there
             __syncthreads();
             if (tid < N) {                                   // per-channel scan over the chunk, t descending
                 for (int t = TC - 1; t >= 0; --t) {
@@ -287,7 +289,7 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
             }
             if constexpr (WMODE != W_HEAD) {
                 __syncthreads();
-                ld8f(&S.part[0][st][sj], out);
+                ld8f(&S.part[0][es][sj], out);
                 if (ok) *reinterpret_cast<uint4*>(a.gw + off) = pack8(out);
             }
         }
@@ -296,7 +298,7 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     // ---- tails
     if constexpr (PASS == P_GR) {
         __syncthreads();
-        st8(&S.part[0][st][sj], gu_acc);
+        if (stager) st8(&S.part[0][st][sj], gu_acc);
         __syncthreads();
         if (tid < N) {
             float s = 0.f;
@@ -324,7 +326,16 @@ template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a) {
 // GR and GV are independent; GK consumes GR's workspace.  All three run on `st` in order.
 // `passes` is a bit mask (RWKV_PASS_*) so that a profiler can time one kernel at a time.
 template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a, unsigned passes = RWKV_PASS_ALL) {
-    if (passes & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
+    const bool chunked = WMODE != W_HEAD && g_wkv6_algorithm == RWKV_ALGO_CHUNKED;
+    if ((passes & RWKV_PASS_GR) && chunked) {
+        if (int e = launch_wkv6_bwd_a_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, a.w, a.u, a.s0, a.gy, a.gr, a.gu, a.rdr)) return e;
+    } else if (passes & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
+    if (chunked) {
+        // the chunked second sweep produces gk, gv, gw (and gs) together: it runs for GK, and GV alone is a no-op
+        if (passes & RWKV_PASS_GK)
+            if (int e = launch_wkv6_bwd_b_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, a.w, a.u, a.s0, a.gy, a.gk, a.gv, a.gw, a.gs, a.rdr)) return e;
+        return launch_status();
+    }
     if (passes & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
     if (passes & RWKV_PASS_GK) hipLaunchKernelGGL((wkv_sweep<P_GK, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
     return launch_status();
