@@ -25,6 +25,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+ALGO = "chunked"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), keyed
 # by kernel label at the headline shape; None = not measured for the current kernels.
@@ -79,23 +80,30 @@ def make_wkv6(dev, state):
                    ("wkv6state backward (3 kernels)", lambda: call("rwkv_wkv6state_backward", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes), 18 * C * tok)]
         name = "wkv6_state"
     else:
-        ew_keep = (-torch.exp(w.float())).contiguous()
-
         def step():
-            ew = (-torch.exp(w.float())).contiguous()               # wrapper pre-transform, wkv6/run.py:147
-            call("rwkv_wkv6_forward", dev, B, T, C, H, r, k, v, ew, u, y)
-            call("rwkv_wkv6_backward", dev, B, T, C, H, r, k, v, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+            # what WKV_6.forward / backward do: raw bf16 decay straight into the kernels, per-batch gu summed by torch
+            call("rwkv_wkv6raw_forward", dev, B, T, C, H, r, k, v, w, u, y)
+            call("rwkv_wkv6raw_backward", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
             return torch.sum(gu, 0).view(H, N)                      # wrapper reduction, wkv6/run.py:169
 
         def bwd(mask):
-            return lambda: call("rwkv_wkv6_backward_passes", dev, B, T, C, H, r, k, v, ew_keep, u, gy, gr, gk, gv, gw, gu, ws, nbytes, mask)
+            def run():
+                lib.rwkv_wkv6_set_backward_passes(mask)
+                call("rwkv_wkv6raw_backward", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+                lib.rwkv_wkv6_set_backward_passes(7)
+            return run
 
-        # algorithmic bytes per kernel: tensors it must read once + outputs it must write once (bf16 = 2 B/elt;
-        # the decay counts 2 B/elt as in the 28*C figure even though this entry point receives it as fp32)
-        kernels = [("wkv6 forward  wkv_sweep<FWD>", lambda: call("rwkv_wkv6_forward", dev, B, T, C, H, r, k, v, ew_keep, u, y), 10 * C * tok),
-                   ("wkv6 backward wkv_sweep<GR>", bwd(1), 12 * C * tok),     # r k v w gy -> gr
-                   ("wkv6 backward wkv_sweep<GV>", bwd(2), 10 * C * tok),     # r k w gy -> gv
-                   ("wkv6 backward wkv_sweep<GK>", bwd(4), 14 * C * tok)]     # r k v w gy -> gk gw
+        # algorithmic bytes per kernel: tensors it must read once + outputs it must write once, 2 B per element
+        fwd = lambda: call("rwkv_wkv6raw_forward", dev, B, T, C, H, r, k, v, w, u, y)
+        if ALGO == "chunked":
+            kernels = [("wkv6_fwd_chunk", fwd, 10 * C * tok),                 # r k v w -> y
+                       ("wkv6_bwd_a_chunk", bwd(1), 12 * C * tok),            # r k v w gy -> gr (+ fp32 workspace)
+                       ("wkv6_bwd_b_chunk", bwd(4), 16 * C * tok)]            # r k v w gy -> gk gv gw
+        else:
+            kernels = [("wkv_sweep<FWD>", fwd, 10 * C * tok),
+                       ("wkv_sweep<GR>", bwd(1), 12 * C * tok),               # r k v w gy -> gr
+                       ("wkv_sweep<GV>", bwd(2), 10 * C * tok),               # r k w gy -> gv
+                       ("wkv_sweep<GK>", bwd(4), 14 * C * tok)]               # r k v w gy -> gk gw
         name = "wkv6"
 
     def cpu_baseline(t_cpu=256):
@@ -301,6 +309,8 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     from rwkv_cuda_amd import _lib
+    global ALGO
+    ALGO = args.algo
     _lib.check(_lib.load().rwkv_wkv6_set_algorithm(0 if args.algo == "chunked" else 1))
     step, tok, kernels, cfg, cpu_baseline, step_bytes = WORKLOADS[args.workload](dev)
 

@@ -116,18 +116,28 @@ int rwkv_wkv6_backward(void* stream, int B, int T, int C, int H,
                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                        void* workspace, size_t workspace_bytes);
 
-/* The same backward restricted to a subset of its kernels, so that a profiler can time one
- * kernel per call (no counterpart in the reference).  RWKV_PASS_GK reads what RWKV_PASS_GR
- * left in the workspace; RWKV_PASS_ALL is rwkv_wkv6_backward. */
-#define RWKV_PASS_GR 1u  /* gr, gu, workspace */
-#define RWKV_PASS_GV 2u  /* gv */
-#define RWKV_PASS_GK 4u  /* gk, gw */
+/* RWKV-6 wkv without state, taking the RAW bf16 decay parameter w[B,T,C] (the kernels apply exp(-exp(w)) and
+ * return gw w.r.t. w): the wrapper-side pre-transform ew = -exp(w.float()) of wkv6/run.py:147 folded into the
+ * kernels, which removes an fp32 [B,T,C] temporary and three elementwise passes.  No counterpart in the reference's
+ * C++ shim; the Python class WKV_6 keeps its reference signature and calls these. */
+int rwkv_wkv6raw_forward(void* stream, int B, int T, int C, int H,
+                         const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                         const rwkv_bf16* w, const rwkv_bf16* u, rwkv_bf16* y);
+int rwkv_wkv6raw_backward(void* stream, int B, int T, int C, int H,
+                          const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                          const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* gy,
+                          rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                          void* workspace, size_t workspace_bytes);
+
+/* Restrict the wkv6 / wkv6raw / wkv6state backward to a subset of its kernels, so that a profiler can time one
+ * kernel per call (process-wide; no counterpart in the reference; RWKV_PASS_ALL restores normal operation).
+ * Sequential kernels: GR (gr, gu, workspace), GV (gv), GK (gk, gw, gs; reads the workspace GR left).
+ * Chunked kernels: GR selects the first sweep (gr, gu, workspace), GK the second (gk, gv, gw, gs); GV alone is empty. */
+#define RWKV_PASS_GR 1u
+#define RWKV_PASS_GV 2u
+#define RWKV_PASS_GK 4u
 #define RWKV_PASS_ALL 7u
-int rwkv_wkv6_backward_passes(void* stream, int B, int T, int C, int H,
-                              const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
-                              const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
-                              rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
-                              void* workspace, size_t workspace_bytes, unsigned passes);
+int rwkv_wkv6_set_backward_passes(unsigned passes);
 
 /* ---------------------------------------------------------------------------------------
  * RWKV-6 wkv with initial state.  Replaces cuda_forward / cuda_backward of

@@ -65,7 +65,9 @@ SIGNATURES = {
     "rwkv_wkv6_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
     "rwkv_wkv6_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv6_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z]),
-    "rwkv_wkv6_backward_passes": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z, ctypes.c_uint]),
+    "rwkv_wkv6raw_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
+    "rwkv_wkv6raw_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z]),
+    "rwkv_wkv6_set_backward_passes": (_I, [ctypes.c_uint]),
     "rwkv_wkv6state_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 7),
     "rwkv_wkv6state_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv6state_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, _Z]),

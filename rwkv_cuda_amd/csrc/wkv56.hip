@@ -22,6 +22,7 @@
 #include "common.h"
 
 namespace rwkv {
+extern unsigned g_bwd_passes;
 namespace {
 
 constexpr int N = 64;            // head size
@@ -358,7 +359,17 @@ size_t ws_bytes(int B, int T, int C, int H) {
 
 using namespace rwkv;
 
+namespace rwkv {
+unsigned g_bwd_passes = RWKV_PASS_ALL;
+}
+
 extern "C" {
+
+int rwkv_wkv6_set_backward_passes(unsigned passes) {
+    if (passes == 0 || passes > RWKV_PASS_ALL) return RWKV_ERR_SHAPE;
+    g_bwd_passes = passes;
+    return RWKV_OK;
+}
 
 int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                       const rwkv_bf16* v, const float* eew, const rwkv_bf16* u, rwkv_bf16* y) {
@@ -401,14 +412,7 @@ int rwkv_wkv6_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16
                        const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                        void* workspace, size_t workspace_bytes) {
-    return rwkv_wkv6_backward_passes(stream, B, T, C, H, r, k, v, ew, u, gy, gr, gk, gv, gw, gu, workspace,
-                                     workspace_bytes, RWKV_PASS_ALL);
-}
-
-int rwkv_wkv6_backward_passes(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
-                              const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
-                              rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
-                              void* workspace, size_t workspace_bytes, unsigned passes) {
+    const unsigned passes = g_bwd_passes;
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, ew, u, gy, gr, gk, gv, gw, gu})) return e;
     if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
@@ -416,6 +420,30 @@ int rwkv_wkv6_backward_passes(void* stream, int B, int T, int C, int H, const rw
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
     return launch_bwd<W_EW>(static_cast<hipStream_t>(stream), B, a, passes);
+}
+
+int rwkv_wkv6raw_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                         const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, rwkv_bf16* y) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, w, u, y})) return e;
+    if (g_wkv6_algorithm == RWKV_ALGO_CHUNKED)
+        return launch_wkv6_fwd_chunk(static_cast<hipStream_t>(stream), W_RAW, B, T, C, H, r, k, v, w, u, nullptr, y);
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.y = y;
+    return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a);
+}
+
+int rwkv_wkv6raw_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                          const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* gy,
+                          rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                          void* workspace, size_t workspace_bytes) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, w, u, gy, gr, gk, gv, gw, gu})) return e;
+    if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.gy = gy;
+    a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
+    return launch_bwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, g_bwd_passes);
 }
 
 int rwkv_wkv6state_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
@@ -442,7 +470,7 @@ int rwkv_wkv6state_backward(void* stream, int B, int T, int C, int H, const rwkv
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.gs = gs; a.rdr = static_cast<float*>(workspace);
-    return launch_bwd<W_RAW>(static_cast<hipStream_t>(stream), B, a);
+    return launch_bwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, g_bwd_passes);
 }
 
 }  // extern "C"

@@ -669,6 +669,7 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_a_chunk(const ArgsB a) {
 // halves' partial sums, so each wave scans its own part and only the chunk totals cross waves.
 // ======================================================================================================================
 constexpr float LN2 = 0.69314718055994530942f;
+constexpr int STAGES_B = 2;       // the second sweep carries two copies of the state: fewer input stages fit the registers
 
 struct alignas(16) SmemB {
     uint32_t Rp[L][RS];            // r e^{c_t - c_m}      cells along j  [t][j]   A of A^T tiles
@@ -722,7 +723,7 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_b_chunk(const ArgsB a) {
 
     const int nchunks = (T + L - 1) / L;
     struct Raw { uint32_t r[2], k[2], v[2], g[2], w[2][2]; float2 d[2]; };
-    Raw ring[STAGES];
+    Raw ring[STAGES_B];
     auto prefetch = [&](int c, Raw& x) __attribute__((always_inline)) {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
@@ -742,7 +743,7 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_b_chunk(const ArgsB a) {
         }
     };
     // chunks are visited last to first; ci counts visits
-    static_for<STAGES>([&](auto Z) { if (decltype(Z)::value < nchunks) prefetch(nchunks - 1 - decltype(Z)::value, ring[decltype(Z)::value]); });
+    static_for<STAGES_B>([&](auto Z) { if (decltype(Z)::value < nchunks) prefetch(nchunks - 1 - decltype(Z)::value, ring[decltype(Z)::value]); });
 
     auto process = [&](const int ci, Raw& x) __attribute__((always_inline)) {
         const int c = nchunks - 1 - ci, c0 = c * L;
@@ -836,7 +837,7 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_b_chunk(const ArgsB a) {
             *reinterpret_cast<uint32_t*>(gt + (2 * jp + 1) * (2 * VS) + pt0) = (x.g[0] >> 16) | (x.g[1] & 0xffff0000u);
         }
         __syncthreads();
-        if (ci + STAGES < nchunks) prefetch(nchunks - 1 - (ci + STAGES), x);
+        if (ci + STAGES_B < nchunks) prefetch(nchunks - 1 - (ci + STAGES_B), x);
 
         const int jl = 16 * q + l16;                   // D: this lane's key channel;  E: this lane's value channel
         const float d1j = S.d1[jl], d2j = S.d2[jl], decj = S.dec[jl];
@@ -1075,8 +1076,8 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_b_chunk(const ArgsB a) {
         }
     };
 
-    for (int cb = 0; cb < nchunks; cb += STAGES)
-        static_for<STAGES>([&](auto Z) { if (cb + decltype(Z)::value < nchunks) process(cb + decltype(Z)::value, ring[decltype(Z)::value]); });
+    for (int cb = 0; cb < nchunks; cb += STAGES_B)
+        static_for<STAGES_B>([&](auto Z) { if (cb + decltype(Z)::value < nchunks) process(cb + decltype(Z)::value, ring[decltype(Z)::value]); });
 
     if (a.gs != nullptr) {
         uint16_t* s = a.gs + bh * N * N + 16 * q + l16;

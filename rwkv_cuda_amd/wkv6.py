@@ -10,7 +10,9 @@ HEAD_SIZE = 64
 
 class WKV_6(torch.autograd.Function):
     """Same signature as WKV_6, wkv6/run.py:128-170: r,k,v,w[B,T,C], u[H,N] bf16, w raw.
-    The wrapper computes ew = -exp(w) in fp32 (:147) and the kernel applies exp(ew)."""
+    The reference wrapper computes ew = -exp(w.float()) (:147) and its kernel applies exp(ew); here the raw
+    w goes straight to the kernels (rwkv_wkv6raw_*), which evaluate the same two exponentials in fp32.
+    The fp32-ew entry points rwkv_wkv6_forward/backward stay available for callers of the C ABI."""
 
     @staticmethod
     def forward(ctx, B, T, C, H, r, k, v, w, u):
@@ -19,17 +21,16 @@ class WKV_6(torch.autograd.Function):
             require(HEAD_SIZE == C // H and C == H * HEAD_SIZE, "head size must be 64")
             require(r.numel() == B * T * C, "shape mismatch")
             ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
-            ew = (-torch.exp(w.float())).contiguous()
-            ctx.save_for_backward(r, k, v, ew, u)
+            ctx.save_for_backward(r, k, v, w, u)
             y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
-            call("rwkv_wkv6_forward", dev, B, T, C, H, r, k, v, ew, u, y)
+            call("rwkv_wkv6raw_forward", dev, B, T, C, H, r, k, v, w, u, y)
             return y
 
     @staticmethod
     def backward(ctx, gy):
         with torch.no_grad():
             B, T, C, H = ctx.B, ctx.T, ctx.C, ctx.H
-            r, k, v, ew, u = ctx.saved_tensors
+            r, k, v, w, u = ctx.saved_tensors
             gy = gy.contiguous()
             dev = check_tensors((gy,), torch.bfloat16, ("gy",))
             new = lambda *shape: torch.empty(shape, device=dev, dtype=torch.bfloat16)
@@ -37,7 +38,7 @@ class WKV_6(torch.autograd.Function):
             gu = new(B, C)
             nbytes = _lib.load().rwkv_wkv6_backward_workspace_bytes(B, T, C, H)
             ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
-            call("rwkv_wkv6_backward", dev, B, T, C, H, r, k, v, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+            call("rwkv_wkv6raw_backward", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
             gu = torch.sum(gu, 0).view(H, C // H)
             return (None, None, None, None, gr, gk, gv, gw, gu)
 

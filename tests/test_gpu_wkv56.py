@@ -114,3 +114,60 @@ def test_wkv6_full_size_sampled_heads(lib):
             print(f"  {name}: {e:.3e}", flush=True)
             # pure bf16 output rounding is 1.7e-3; gu is a bf16 sum of 8 bf16 partials
             assert e < (4e-3 if name == "gu" else 2.5e-3), (name, e)
+
+
+def test_wkv6_fp32_ew_c_abi(lib):
+    """The reference's own wkv6 boundary: the decay arrives as fp32 ew = -exp(w) (wkv6/run.py:147)."""
+    B, T, H = 2, 70, 2
+    C = H * 64
+    r, k, v, w, u, gy, _ = synth.wkv6_inputs(B, T, C, H, seed=15)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy)
+    d = [x.to(DEV) for x in (r, k, v, w, u, gy)]
+    ew = (-torch.exp(d[3].float())).contiguous()
+    for algo in (0, 1):
+        print(f"\nwkv6 fp32-ew C-ABI algo={algo}", flush=True)
+        lib.rwkv_wkv6_set_algorithm(algo)
+        try:
+            y = garbage((B, T, C), BF)
+            call("rwkv_wkv6_forward", d[0].device, B, T, C, H, d[0], d[1], d[2], ew, d[4], y)
+            gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
+            gu = garbage((B, C), BF)
+            n = lib.rwkv_wkv6_backward_workspace_bytes(B, T, C, H)
+            ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+            call("rwkv_wkv6_backward", d[0].device, B, T, C, H, d[0], d[1], d[2], ew, d[4], d[5], gr, gk, gv, gw, gu, ws, n)
+            torch.cuda.synchronize()
+        finally:
+            lib.rwkv_wkv6_set_algorithm(0)
+        for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y, gr, gk, gv, gw, gu.sum(0).view(H, 64)]):
+            assert_no_worse(name, a, e, g)
+
+
+@pytest.mark.parametrize("algo", [0, 1])
+def test_wkv6_state_both_algorithms_and_extreme_decays(lib, algo):
+    """Chunked (matrix-core) and sequential kernels against the oracle, on ordinary inputs and on decays so strong
+    (w_raw up to 3: one step multiplies the state by e^-20) that the chunked kernels must take their exact path."""
+    B, T, H = 2, 100, 2
+    C = H * 64
+    for extreme in (False, True):
+        r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=16, state=True)
+        if extreme:
+            w = w.float()
+            w[:, 40:60, :64] = 2.5
+            w[1, 70:, 100] = 3.0
+            w[0, 5:9, 70:90] = 2.0
+            w = w.to(BF)
+        ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+        emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+        print(f"\nwkv6_state algo={algo} extreme={extreme}", flush=True)
+        lib.rwkv_wkv6_set_algorithm(algo)
+        try:
+            t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u, s0)]
+            y = wkv6_state.RUN_CUDA(B, T, C, H, *t)
+            y.backward(gy.to(DEV))
+            torch.cuda.synchronize()
+        finally:
+            lib.rwkv_wkv6_set_algorithm(0)
+        for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, emu, [y] + [x.grad for x in t]):
+            assert torch.isfinite(g).all(), name
+            assert_no_worse(name, a, e, g)
