@@ -29,7 +29,12 @@ ALGO = "chunked"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), keyed
 # by kernel label at the headline shape; None = not measured for the current kernels.
-TRAFFIC_MEASURED = {}
+TRAFFIC_MEASURED = {
+    # profiles/wkv6_chunk_kernels_B8_T4096_C2048.md  (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB)
+    "wkv6_fwd_chunk": 537e6 + 134e6,
+    "wkv6_bwd_a_chunk": 671e6 + 403e6,
+    "wkv6_bwd_b_chunk": 941e6 + 404e6,
+}
 
 
 def _events(n):
