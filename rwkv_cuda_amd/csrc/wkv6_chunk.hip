@@ -82,23 +82,51 @@ DEVINL float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 // dword position, inside a stored row, of the (H, L) pair of elements (2p, 2p+1): groups of 4 elements are H01 H23 L01 L23
 DEVINL int hpos(int p) { return 4 * (p >> 1) + (p & 1); }
 
+DEVINL bf16x8 lds_op_sw(const uint32_t* p) {       // the same cell with its halves exchanged: [l0..l3 | h0..h3]
+    const uint2 lo = *reinterpret_cast<const uint2*>(p + 2);
+    const uint2 hi = *reinterpret_cast<const uint2*>(p);
+    return as_op(lo.x, lo.y, hi.x, hi.y);
+}
+// full product of two hi/lo cells read from LDS: A (and A with halves exchanged) against B
+DEVINL f32x4 mfma_full_lds(const uint32_t* pa, bf16x8 b, f32x4 c) { return mfma(lds_op_sw(pa), b, mfma(lds_op(pa), b, c)); }
+
+// In-chunk exponents, in log2 units, for the two tokens (t0, t0+1) of one channel held by a thread.
+// near = sum of lam over the tokens of the same half-chunk that lie between this pair and the middle of the chunk.
+//   first half : Ea_t = 2^{-sum_{z=t..15} lam},  Eb_t = 2^{sum_{z=t+1..15} lam}
+//   second half: Ea_t = 2^{sum_{z=16..t-1} lam}, Eb_t = 2^{-sum_{z=16..t} lam}
+struct Scale { float ea[2], eb[2]; };
+DEVINL Scale chunk_scale(bool second_half, float near, float lam0, float lam1) {
+    Scale s;
+    if (!second_half) {
+        const float s1 = lam1 + near, s0 = lam0 + s1;          // suffix sums from t0+1, t0
+        s.ea[0] = exp2_fast(-s0); s.ea[1] = exp2_fast(-s1);
+        s.eb[0] = exp2_fast(s1);  s.eb[1] = exp2_fast(near);
+    } else {
+        const float p1 = near + lam0, p2 = p1 + lam1;          // prefix sums up to t0+1, t0+2
+        s.ea[0] = exp2_fast(near); s.ea[1] = exp2_fast(p1);
+        s.eb[0] = exp2_fast(-p1);  s.eb[1] = exp2_fast(-p2);
+    }
+    return s;
+}
+
 struct alignas(16) SmemFwd {
-    uint32_t Rs[L][RS];            // r e^{c_t}             [t][j]   A operand of  Rs S0^T
-    uint32_t Rp[L][RS];            // r e^{c_t - c_m}       [t][j]   B operand of  A^T = K' R'^T
-    uint32_t Kp[L][RS];            // k e^{c_m - c_{t+1}}   [s][j]   A operand of  A^T
-    uint32_t Ke[N][TS];            // k e^{c_L - c_{s+1}}   [j][s]   A operand of  S^T += Ke^T V
-    uint32_t Am[L][TS];            // A                     [t][s]   A operand of  A V
-    uint32_t Vt[N][VS];            // v, plain bf16         [i][s]   B operand
+    uint32_t Rp[L][RS];            // r e^{c_t - c_m}       cells along j       [t][j]   B operand of  A^T = K' R'^T, A operand of R' (d1 S0)^T
+    uint32_t Kp[L][RS];            // k e^{c_m - c_{s+1}}   cells along j       [s][j]   A operand of  A^T
+    uint32_t KpT[N][TS];           // the same values       cells along tokens  [j][s]   A operand of  S^T += K'^T V
+    uint32_t Am[L][TS];            // A                     cells along s       [t][s]   A operand of  A V
+    uint32_t Vd[N][TS];            // v, [v0 v1 v2 v3 | v0 v1 v2 v3] per 4 tokens [i][s] B operand
     float X[L][N];                 // r u k [t][j], summed over j into the diagonal of A;  exact path: r
     float raw[2][L][N];            // exact path only: k, decay as fp32 [t][j]
-    float dec[N];                  // e^{c_L}[j]   (exact path: u)
-    float part[8][N];              // sum of lam (in log2 units) over each eighth of the chunk
+    float d1[N], d2[N], dec[N];    // e^{c_m}, e^{c_L - c_m}, e^{c_L}   (exact path: d1 = u)
+    float part[8][N];              // sum of lam (log2 units) over each eighth of the chunk
+    uint32_t flag[8];              // per wave: some channel decays too fast for the mid-point factors
     float Y[2][2][L][RS];          // output staging, double buffered: partial sums of the two key-channel halves
 };
 
 // One workgroup of 8 waves per (batch, head).  Wave (q = wid & 3, jh = wid >> 2) owns value channels [16q, 16q+16) and the
 // key-channel half [32jh, 32jh+32) of the state: S^T[j][i] in two accumulator tiles,  D[m][v] <-> j = 32jh + 16m + 4g + v.
-// The accumulator layout is used as is as the B operand of Rs S0^T (lane group g holds channels 4g..4g+3 of each tile).
+// The accumulator layout is used as is as the B operand of R' (d1 S0)^T (lane group g holds channels 4g..4g+3 of each tile).
+// Three barriers per chunk: [scan parts] B2 [operands] B3 [A tiles | store of the previous chunk | R' S0^T] B4 [A V, state].
 template <int WMODE>
 __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
     __shared__ SmemFwd S;
@@ -113,6 +141,7 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
     const uint16_t* __restrict__ vb_ = a.v + base;
     // prep coordinates: channel pair (2 jp, 2 jp + 1), tokens 4 wid + 2 th + {0, 1}
     const int jp = lane & 31, th = lane >> 5, pt0 = 4 * wid + 2 * th;
+    const bool second = wid >= 4;
     float uj[2];
     {
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + 2 * jp);
@@ -139,93 +168,122 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
     struct Raw { uint32_t r[2], k[2], v[2], w[2][2]; };
     Raw ring[STAGES];
     auto prefetch = [&](int c, Raw& x) __attribute__((always_inline)) {
-        uint32_t (&qr)[2] = x.r; uint32_t (&qk)[2] = x.k; uint32_t (&qv)[2] = x.v; uint32_t (&qw)[2][2] = x.w;
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int t = c * L + pt0 + e;
             const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C + 2 * jp;
-            qr[e] = *reinterpret_cast<const uint32_t*>(rb + o);
-            qk[e] = *reinterpret_cast<const uint32_t*>(kb + o);
-            qv[e] = *reinterpret_cast<const uint32_t*>(vb_ + o);
+            x.r[e] = *reinterpret_cast<const uint32_t*>(rb + o);
+            x.k[e] = *reinterpret_cast<const uint32_t*>(kb + o);
+            x.v[e] = *reinterpret_cast<const uint32_t*>(vb_ + o);
             if constexpr (WMODE == W_RAW) {
-                qw[e][0] = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + base + o);
+                x.w[e][0] = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + base + o);
             } else {
-                const uint2 x = *reinterpret_cast<const uint2*>(static_cast<const float*>(a.w) + base + o);
-                qw[e][0] = x.x; qw[e][1] = x.y;
+                const uint2 y = *reinterpret_cast<const uint2*>(static_cast<const float*>(a.w) + base + o);
+                x.w[e][0] = y.x; x.w[e][1] = y.y;
             }
         }
     };
     static_for<STAGES>([&](auto Z) { if (decltype(Z)::value < nchunks) prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
 
-    auto process = [&](const int c, Raw& x) __attribute__((always_inline)) {
-        uint32_t (&qr)[2] = x.r; uint32_t (&qk)[2] = x.k; uint32_t (&qv)[2] = x.v; uint32_t (&qw)[2][2] = x.w;
-        const int c0 = c * L, buf = c & 1;
-        // ------------------------------------------------------------------ prep
-        // element [e][z]: token pt0 + e, channel 2 jp + z.  lam is kept in log2 units.
-        float pr[2][2], pk[2][2], plam[2][2];
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const bool ok = (c0 + pt0 + e) < T;            // rows past T: no input, no decay
-            if (!ok) { qr[e] = 0; qk[e] = 0; qv[e] = 0; }
-            pr[e][0] = bf_lo(qr[e]); pr[e][1] = bf_hi(qr[e]);
-            pk[e][0] = bf_lo(qk[e]); pk[e][1] = bf_hi(qk[e]);
+    // rows (c0 + t) of staging buffer `buf` -> y, by 256 threads
+    auto store_y = [&](int c0, int buf, int idx) __attribute__((always_inline)) {
+        const int t = idx >> 3, i0 = (idx & 7) * 8;
+        if (c0 + t < T) {
+            float f[8];
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
-                float lam;
-                if constexpr (WMODE == W_RAW) lam = -exp2_fast(LOG2E * (z ? bf_hi(qw[e][0]) : bf_lo(qw[e][0])));
-                else lam = __uint_as_float(qw[e][z]);
-                plam[e][z] = ok ? lam * LOG2E : 0.f;
+                const float4 x0 = *reinterpret_cast<const float4*>(&S.Y[buf][0][t][i0 + 4 * z]);
+                const float4 x1 = *reinterpret_cast<const float4*>(&S.Y[buf][1][t][i0 + 4 * z]);
+                f[4 * z] = x0.x + x1.x; f[4 * z + 1] = x0.y + x1.y; f[4 * z + 2] = x0.z + x1.z; f[4 * z + 3] = x0.w + x1.w;
             }
+            *reinterpret_cast<uint4*>(a.y + base + static_cast<size_t>(c0 + t) * C + i0) = pack8(f);
         }
-        // sums over this wave's 4 tokens: lanes 0..31 hold tokens 0,1, lanes 32..63 tokens 2,3 of the same channels
-        float s2[2], s4[2], other[2];
+    };
+
+    auto process = [&](const int c, Raw& x) __attribute__((always_inline)) {
+        const int c0 = c * L, buf = c & 1;
+        if (c0 + L > T) {                              // last, partial chunk: rows past T carry no input and no decay
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+                if (c0 + pt0 + e >= T) {
+                    x.r[e] = 0; x.k[e] = 0; x.v[e] = 0;
+                    x.w[e][0] = (WMODE == W_RAW) ? 0xff80ff80u : 0u;   // w = -inf  ->  lam = -exp(w) = 0
+                    x.w[e][1] = 0u;
+                }
+        }
+        // ------------------------------------------------------------------ scan.  element [e][z]: token pt0 + e, channel 2 jp + z
+        float plam[2][2];                              // lam in log2 units
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+#pragma unroll
+            for (int z = 0; z < 2; ++z) {
+                if constexpr (WMODE == W_RAW) plam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e][0]) : bf_lo(x.w[e][0])));
+                else plam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+            }
+        float s2[2], other[2];
 #pragma unroll
         for (int z = 0; z < 2; ++z) {
             s2[z] = plam[0][z] + plam[1][z];
-            other[z] = __shfl_xor(s2[z], 32, 64);
-            s4[z] = s2[z] + other[z];
+            other[z] = __shfl_xor(s2[z], 32, 64);      // the other two tokens of this wave's four
         }
-        if (th == 0) *reinterpret_cast<float2*>(&S.part[wid][2 * jp]) = make_float2(s4[0], s4[1]);
-        // a chunk whose decays could overflow the mid-point factors is redone exactly; any half-chunk sum beyond
-        // the limit implies an eighth beyond limit/4, so this local test is sufficient (and conservative)
-        const bool exact = __syncthreads_or((-s4[0] > 0.25f * RANGE_LIMIT * LOG2E) || (-s4[1] > 0.25f * RANGE_LIMIT * LOG2E)) != 0;
-        float pre[2] = {0.f, 0.f}, cm[2] = {0.f, 0.f}, cl[2] = {0.f, 0.f};   // before this wave's tokens / middle / whole
+        const float s4a = s2[0] + other[0], s4b = s2[1] + other[1];
+        if (th == 0) *reinterpret_cast<float2*>(&S.part[wid][2 * jp]) = make_float2(s4a, s4b);
+        // A chunk whose decays could overflow the mid-point factors is redone exactly.  A half-chunk sum beyond the limit
+        // implies an eighth beyond limit/4, so this local test is sufficient (and conservative).
+        const bool fast_decay = (-s4a > 0.25f * RANGE_LIMIT * LOG2E) || (-s4b > 0.25f * RANGE_LIMIT * LOG2E);
+        const unsigned long long any = __ballot(fast_decay);
+        if (lane == 0) S.flag[wid] = any != 0ull;
+        __syncthreads();                               // B2
+        const uint4 f0 = *reinterpret_cast<const uint4*>(&S.flag[0]), f1 = *reinterpret_cast<const uint4*>(&S.flag[4]);
+        const bool exact = (f0.x | f0.y | f0.z | f0.w | f1.x | f1.y | f1.z | f1.w) != 0;
+        // tokens of this half-chunk between this thread's pair and the middle of the chunk
+        float near[2];
+        near[0] = second ? (th ? other[0] : 0.f) : (th ? 0.f : other[0]);
+        near[1] = second ? (th ? other[1] : 0.f) : (th ? 0.f : other[1]);
+        {
+            const int lo = second ? 4 : wid + 1, hi = second ? wid : 4;      // wave-uniform bounds
+            for (int w8 = lo; w8 < hi; ++w8) {
+                const float2 y = *reinterpret_cast<const float2*>(&S.part[w8][2 * jp]);
+                near[0] += y.x; near[1] += y.y;
+            }
+        }
+        if (wid == 0 && th == 0) {                     // per-channel factors of the whole chunk
+            float cm[2] = {0.f, 0.f}, ch[2] = {0.f, 0.f};
 #pragma unroll
-        for (int w8 = 0; w8 < 8; ++w8) {
-            const float2 x = *reinterpret_cast<const float2*>(&S.part[w8][2 * jp]);
-            if (w8 < wid) { pre[0] += x.x; pre[1] += x.y; }
-            if (w8 < 4) { cm[0] += x.x; cm[1] += x.y; }
-            cl[0] += x.x; cl[1] += x.y;
+            for (int w8 = 0; w8 < 4; ++w8) {
+                const float2 y0 = *reinterpret_cast<const float2*>(&S.part[w8][2 * jp]);
+                const float2 y1 = *reinterpret_cast<const float2*>(&S.part[4 + w8][2 * jp]);
+                cm[0] += y0.x; cm[1] += y0.y; ch[0] += y1.x; ch[1] += y1.y;
+            }
+            if (!exact) *reinterpret_cast<float2*>(&S.d1[2 * jp]) = make_float2(exp2_fast(cm[0]), exp2_fast(cm[1]));
+            else *reinterpret_cast<float2*>(&S.d1[2 * jp]) = make_float2(uj[0], uj[1]);
+            *reinterpret_cast<float2*>(&S.d2[2 * jp]) = make_float2(exp2_fast(ch[0]), exp2_fast(ch[1]));
+            *reinterpret_cast<float2*>(&S.dec[2 * jp]) = make_float2(exp2_fast(cm[0] + ch[0]), exp2_fast(cm[1] + ch[1]));
         }
-        if (th) { pre[0] += other[0]; pre[1] += other[1]; }
+        float pr[2][2], pk[2][2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            pr[e][0] = bf_lo(x.r[e]); pr[e][1] = bf_hi(x.r[e]);
+            pk[e][0] = bf_lo(x.k[e]); pk[e][1] = bf_hi(x.k[e]);
+        }
         if (!exact) {
-            float rp[2][2], rs[2][2], kp[2][2], ke[2][2];
+            float rp[2][2], kp[2][2];
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
-                const float d1 = exp2_fast(cm[z]), d2 = exp2_fast(cl[z] - cm[z]);
-                if (wid == 0 && th == 0) S.dec[2 * jp + z] = exp2_fast(cl[z]);
-                const float ct0 = pre[z], ct1 = ct0 + plam[0][z], ct2 = ct1 + plam[1][z];
-                rp[0][z] = pr[0][z] * exp2_fast(ct0 - cm[z]);
-                rp[1][z] = pr[1][z] * exp2_fast(ct1 - cm[z]);
-                kp[0][z] = pk[0][z] * exp2_fast(cm[z] - ct1);
-                kp[1][z] = pk[1][z] * exp2_fast(cm[z] - ct2);
-#pragma unroll
-                for (int e = 0; e < 2; ++e) { rs[e][z] = rp[e][z] * d1; ke[e][z] = kp[e][z] * d2; }
+                const Scale sc = chunk_scale(second, near[z], plam[0][z], plam[1][z]);
+                rp[0][z] = pr[0][z] * sc.ea[0]; rp[1][z] = pr[1][z] * sc.ea[1];
+                kp[0][z] = pk[0][z] * sc.eb[0]; kp[1][z] = pk[1][z] * sc.eb[1];
+                const HL y = hilo2(kp[0][z], kp[1][z]);              // pair along the two tokens
+                S.KpT[2 * jp + z][4 * wid + th] = y.h;
+                S.KpT[2 * jp + z][4 * wid + 2 + th] = y.l;
             }
             const int ph = hpos(jp);
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
                 const int t = pt0 + e;
-                HL x = hilo2(rp[e][0], rp[e][1]); S.Rp[t][ph] = x.h; S.Rp[t][ph + 2] = x.l;
-                x = hilo2(rs[e][0], rs[e][1]);    S.Rs[t][ph] = x.h; S.Rs[t][ph + 2] = x.l;
-                x = hilo2(kp[e][0], kp[e][1]);    S.Kp[t][ph] = x.h; S.Kp[t][ph + 2] = x.l;
+                HL y = hilo2(rp[e][0], rp[e][1]); S.Rp[t][ph] = y.h; S.Rp[t][ph + 2] = y.l;
+                y = hilo2(kp[e][0], kp[e][1]);    S.Kp[t][ph] = y.h; S.Kp[t][ph + 2] = y.l;
                 *reinterpret_cast<float2*>(&S.X[t][2 * jp]) = make_float2(pr[e][0] * uj[0] * pk[e][0], pr[e][1] * uj[1] * pk[e][1]);
-            }
-#pragma unroll
-            for (int z = 0; z < 2; ++z) {                  // Ke^T: pair along the two tokens
-                const HL x = hilo2(ke[0][z], ke[1][z]);
-                S.Ke[2 * jp + z][4 * wid + th] = x.h;
-                S.Ke[2 * jp + z][4 * wid + 2 + th] = x.l;
             }
         } else {
 #pragma unroll
@@ -235,35 +293,33 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
                 *reinterpret_cast<float2*>(&S.raw[0][t][2 * jp]) = make_float2(pk[e][0], pk[e][1]);
                 *reinterpret_cast<float2*>(&S.raw[1][t][2 * jp]) = make_float2(exp2_fast(plam[e][0]), exp2_fast(plam[e][1]));
             }
-            if (wid == 0 && th == 0) *reinterpret_cast<float2*>(&S.dec[2 * jp]) = make_float2(uj[0], uj[1]);
         }
-        // V^T[i][s]: the two tokens of channel 2jp+z are one dword
-        {
-            uint16_t* vt = reinterpret_cast<uint16_t*>(&S.Vt[0][0]);
-            *reinterpret_cast<uint32_t*>(vt + (2 * jp) * (2 * VS) + pt0) = (qv[0] & 0xffffu) | (qv[1] << 16);
-            *reinterpret_cast<uint32_t*>(vt + (2 * jp + 1) * (2 * VS) + pt0) = (qv[0] >> 16) | (qv[1] & 0xffff0000u);
+        {   // v: the two tokens of channel 2jp+z are one dword, stored in both halves of the cell
+            const uint32_t v0 = (x.v[0] & 0xffffu) | (x.v[1] << 16), v1 = (x.v[0] >> 16) | (x.v[1] & 0xffff0000u);
+            S.Vd[2 * jp][4 * wid + th] = v0;     S.Vd[2 * jp][4 * wid + 2 + th] = v0;
+            S.Vd[2 * jp + 1][4 * wid + th] = v1; S.Vd[2 * jp + 1][4 * wid + 2 + th] = v1;
         }
-        __syncthreads();
+        __syncthreads();                               // B3
         if (c + STAGES < nchunks) prefetch(c + STAGES, x);   // this register set is free again
 
+        f32x4 Y[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
         if (!exact) {
-            // -------------------------------------------------------------- A^T tiles: waves 0,1,2 -> A(0,0) A(1,0) A(1,1)
             if (wid < 3) {
+                // ---------------------------------------------------------- A^T tiles: waves 0,1,2 -> A(0,0) A(1,0) A(1,1)
                 const int ta = (wid == 0) ? 0 : 1, tb = (wid == 2) ? 1 : 0;
                 f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int js = 0; js < 4; js += 2) {     // rows of the result: s (from K'), columns: t (from R')
-                    acc0 = mfma_full(lds_op(&S.Kp[16 * tb + l16][16 * js + 4 * g]), lds_op(&S.Rp[16 * ta + l16][16 * js + 4 * g]), acc0);
-                    acc1 = mfma_full(lds_op(&S.Kp[16 * tb + l16][16 * js + 16 + 4 * g]), lds_op(&S.Rp[16 * ta + l16][16 * js + 16 + 4 * g]), acc1);
+                    acc0 = mfma_full_lds(&S.Kp[16 * tb + l16][16 * js + 4 * g], lds_op(&S.Rp[16 * ta + l16][16 * js + 4 * g]), acc0);
+                    acc1 = mfma_full_lds(&S.Kp[16 * tb + l16][16 * js + 16 + 4 * g], lds_op(&S.Rp[16 * ta + l16][16 * js + 16 + 4 * g]), acc1);
                 }
                 f32x4 acc = acc0 + acc1;                // acc[v]: s = 4g + v, t = l16
                 if (ta == tb) {
-                    // diagonal: sum_j r u k of row t = 16 ta + l16 (this lane sums 16 channels, the 4 groups the rest)
-                    float d = 0.f;
+                    float d = 0.f;                      // diagonal: sum_j r u k of row t = 16 ta + l16
 #pragma unroll
                     for (int z = 0; z < 4; ++z) {
-                        const float4 x = *reinterpret_cast<const float4*>(&S.X[16 * ta + l16][16 * g + 4 * z]);
-                        d += (x.x + x.y) + (x.z + x.w);
+                        const float4 y = *reinterpret_cast<const float4*>(&S.X[16 * ta + l16][16 * g + 4 * z]);
+                        d += (y.x + y.y) + (y.z + y.w);
                     }
                     d = allreduce_rows(d);
 #pragma unroll
@@ -274,21 +330,23 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
                 }
                 const HL x0 = hilo2(acc[0], acc[1]), x1 = hilo2(acc[2], acc[3]);
                 *reinterpret_cast<uint4*>(&S.Am[16 * ta + l16][16 * tb + 4 * g]) = make_uint4(x0.h, x1.h, x0.l, x1.l);
+            } else if (wid >= 4 && c > 0) {
+                store_y(c0 - L, buf ^ 1, tid - 256);   // the previous chunk's output leaves while the tiles are computed
             }
-            // -------------------------------------------------------------- Y (this half of j) = Rs S0^T
-            f32x4 Y[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+            // -------------------------------------------------------------- Y (this half of j) = R' (d1 S0)^T
 #pragma unroll
             for (int m = 0; m < 2; ++m) {
-                const HL x0 = hilo2(D[m][0], D[m][1]), x1 = hilo2(D[m][2], D[m][3]);
+                const int j0 = 32 * jh + 16 * m + 4 * g;
+                const float4 dd = *reinterpret_cast<const float4*>(&S.d1[j0]);
+                const HL x0 = hilo2(D[m][0] * dd.x, D[m][1] * dd.y), x1 = hilo2(D[m][2] * dd.z, D[m][3] * dd.w);
                 const bf16x8 sb = as_op(x0.h, x1.h, x0.l, x1.l);
 #pragma unroll
-                for (int mt = 0; mt < 2; ++mt)
-                    Y[mt] = mfma_full(lds_op(&S.Rs[16 * mt + l16][32 * jh + 16 * m + 4 * g]), sb, Y[mt]);
+                for (int mt = 0; mt < 2; ++mt) Y[mt] = mfma_full_lds(&S.Rp[16 * mt + l16][j0], sb, Y[mt]);
             }
-            __syncthreads();                           // A is in LDS
-            // -------------------------------------------------------------- Y += A V (tokens of half jh);  S^T = S^T diag(dec) + Ke^T V
-            const bf16x8 vb0 = lds_dup(&S.Vt[16 * q + l16][2 * g]);        // tokens  4g..4g+3
-            const bf16x8 vb1 = lds_dup(&S.Vt[16 * q + l16][8 + 2 * g]);    // tokens 16+4g..
+            __syncthreads();                           // B4: A is in LDS
+            // -------------------------------------------------------------- Y += A V (tokens of half jh);  S^T = S^T diag(dec) + diag(d2) K'^T V
+            const bf16x8 vb0 = lds_op(&S.Vd[16 * q + l16][4 * g]);        // tokens  4g..4g+3
+            const bf16x8 vb1 = lds_op(&S.Vd[16 * q + l16][16 + 4 * g]);   // tokens 16+4g..
             if (jh == 0) {
                 Y[0] = mfma(lds_op(&S.Am[l16][4 * g]), vb0, Y[0]);
                 Y[1] = mfma(lds_op(&S.Am[16 + l16][4 * g]), vb0, Y[1]);
@@ -298,10 +356,13 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
 #pragma unroll
             for (int m = 0; m < 2; ++m) {
                 const int j0 = 32 * jh + 16 * m;
-                const float4 dj = *reinterpret_cast<const float4*>(&S.dec[j0 + 4 * g]);
-                f32x4 x = {D[m][0] * dj.x, D[m][1] * dj.y, D[m][2] * dj.z, D[m][3] * dj.w};
-                x = mfma(lds_op(&S.Ke[j0 + l16][4 * g]), vb0, x);
-                D[m] = mfma(lds_op(&S.Ke[j0 + l16][16 + 4 * g]), vb1, x);
+                f32x4 U = {0.f, 0.f, 0.f, 0.f};
+                U = mfma(lds_op(&S.KpT[j0 + l16][4 * g]), vb0, U);
+                U = mfma(lds_op(&S.KpT[j0 + l16][16 + 4 * g]), vb1, U);
+                const float4 de = *reinterpret_cast<const float4*>(&S.dec[j0 + 4 * g]);
+                const float4 d2 = *reinterpret_cast<const float4*>(&S.d2[j0 + 4 * g]);
+                D[m][0] = fmaf(D[m][0], de.x, d2.x * U[0]); D[m][1] = fmaf(D[m][1], de.y, d2.y * U[1]);
+                D[m][2] = fmaf(D[m][2], de.z, d2.z * U[2]); D[m][3] = fmaf(D[m][3], de.w, d2.w * U[3]);
             }
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
@@ -310,16 +371,17 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
         } else {
             // -------------------------------------------------------------- exact path: 32 sequential steps
             // lane (i = 16q + l16, group g) holds S[i][j] for j = 32 jh + 16 m + 4 g + v
+            if (wid >= 4 && c > 0) store_y(c0 - L, buf ^ 1, tid - 256);
             __syncthreads();                           // keeps the barrier count equal on both paths
             float uv[2][4];
 #pragma unroll
             for (int m = 0; m < 2; ++m) {
-                const float4 x = *reinterpret_cast<const float4*>(&S.dec[32 * jh + 16 * m + 4 * g]);
-                uv[m][0] = x.x; uv[m][1] = x.y; uv[m][2] = x.z; uv[m][3] = x.w;
+                const float4 y = *reinterpret_cast<const float4*>(&S.d1[32 * jh + 16 * m + 4 * g]);   // u on this path
+                uv[m][0] = y.x; uv[m][1] = y.y; uv[m][2] = y.z; uv[m][3] = y.w;
             }
-            const uint16_t* vt = reinterpret_cast<const uint16_t*>(&S.Vt[16 * q + l16][0]);
+            const uint16_t* vt = reinterpret_cast<const uint16_t*>(&S.Vd[16 * q + l16][0]);
             for (int t = 0; t < L; ++t) {
-                const float vi = bf2f(vt[t]);
+                const float vi = bf2f(vt[8 * (t >> 2) + (t & 3)]);
                 float yp = 0.f;
 #pragma unroll
                 for (int m = 0; m < 2; ++m) {
@@ -339,26 +401,14 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
                 if (g == 0) S.Y[buf][jh][t][16 * q + l16] = y;
             }
         }
-        __syncthreads();
-        if (tid < 256) {
-            const int t = tid >> 3, i0 = (tid & 7) * 8;
-            if (c0 + t < T) {
-                float f[8];
-#pragma unroll
-                for (int z = 0; z < 2; ++z) {
-                    const float4 x0 = *reinterpret_cast<const float4*>(&S.Y[buf][0][t][i0 + 4 * z]);
-                    const float4 x1 = *reinterpret_cast<const float4*>(&S.Y[buf][1][t][i0 + 4 * z]);
-                    f[4 * z] = x0.x + x1.x; f[4 * z + 1] = x0.y + x1.y; f[4 * z + 2] = x0.z + x1.z; f[4 * z + 3] = x0.w + x1.w;
-                }
-                *reinterpret_cast<uint4*>(a.y + base + static_cast<size_t>(c0 + t) * C + i0) = pack8(f);
-            }
-        }
     };
 
     for (int cb = 0; cb < nchunks; cb += STAGES)
         static_for<STAGES>([&](auto Z) { if (cb + decltype(Z)::value < nchunks) process(cb + decltype(Z)::value, ring[decltype(Z)::value]); });
-}
 
+    __syncthreads();
+    if (tid < 256) store_y((nchunks - 1) * L, (nchunks - 1) & 1, tid);
+}
 
 // ======================================================================================================================
 // Backward, first sweep (time ascending): gr, gu and the workspace r * dr' that the decay gradient needs.
