@@ -16,15 +16,13 @@ DEVINL float bf2f(uint16_t x) { return __uint_as_float(static_cast<uint32_t>(x) 
 DEVINL float bf_lo(uint32_t x) { return __uint_as_float(x << 16); }          // element 0 of a packed pair
 DEVINL float bf_hi(uint32_t x) { return __uint_as_float(x & 0xffff0000u); }  // element 1 of a packed pair
 
-// round-to-nearest-even, NaN stays NaN
-DEVINL uint32_t f2bf_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+// fp32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950; NaN stays NaN)
+DEVINL uint16_t f2bf(float f) { return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f)); }
+DEVINL uint32_t pack_bf2(float lo, float hi) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const bf16x2_t p = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+    return __builtin_bit_cast(uint32_t, p);
 }
-DEVINL uint16_t f2bf(float f) { return static_cast<uint16_t>(f2bf_bits(f)); }
-DEVINL uint32_t pack_bf2(float lo, float hi) { return f2bf_bits(lo) | (f2bf_bits(hi) << 16); }
 
 DEVINL void unpack8(const uint4& q, float (&f)[8]) {
     f[0] = bf_lo(q.x); f[1] = bf_hi(q.x); f[2] = bf_lo(q.y); f[3] = bf_hi(q.y);

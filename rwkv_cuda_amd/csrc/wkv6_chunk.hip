@@ -142,6 +142,11 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
     // prep coordinates: channel pair (2 jp, 2 jp + 1), tokens 4 wid + 2 th + {0, 1}
     const int jp = lane & 31, th = lane >> 5, pt0 = 4 * wid + 2 * th;
     const bool second = wid >= 4;
+    // [channel][token] arrays keep the 16-byte cell of tokens 4c..4c+3 of row `ch` at cell index c ^ ((ch >> 1) & 7), which
+    // spreads the one-dword-per-lane writes of the prep over the banks.  Writer: rows 2jp, 2jp+1, cell wid.
+    // Reader: rows (multiple of 16) + l16, cells g and 4 + g.
+    const int wcell = 4 * (wid ^ (jp & 7));
+    const int rc0 = 4 * (g ^ ((l16 >> 1) & 7)), rc1 = 4 * ((4 + g) ^ ((l16 >> 1) & 7));
     float uj[2];
     {
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + 2 * jp);
@@ -274,15 +279,17 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
                 rp[0][z] = pr[0][z] * sc.ea[0]; rp[1][z] = pr[1][z] * sc.ea[1];
                 kp[0][z] = pk[0][z] * sc.eb[0]; kp[1][z] = pk[1][z] * sc.eb[1];
                 const HL y = hilo2(kp[0][z], kp[1][z]);              // pair along the two tokens
-                S.KpT[2 * jp + z][4 * wid + th] = y.h;
-                S.KpT[2 * jp + z][4 * wid + 2 + th] = y.l;
+                S.KpT[2 * jp + z][wcell + th] = y.h;
+                S.KpT[2 * jp + z][wcell + 2 + th] = y.l;
             }
             const int ph = hpos(jp);
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
                 const int t = pt0 + e;
-                HL y = hilo2(rp[e][0], rp[e][1]); S.Rp[t][ph] = y.h; S.Rp[t][ph + 2] = y.l;
-                y = hilo2(kp[e][0], kp[e][1]);    S.Kp[t][ph] = y.h; S.Kp[t][ph + 2] = y.l;
+                // cells of rows written by the upper half-wave are stored with their halves exchanged: every consumer adds
+                // both orders (mfma_full), and the two half-waves then hit disjoint LDS banks
+                HL y = hilo2(rp[e][0], rp[e][1]); S.Rp[t][ph + 2 * th] = y.h; S.Rp[t][ph + 2 - 2 * th] = y.l;
+                y = hilo2(kp[e][0], kp[e][1]);    S.Kp[t][ph + 2 * th] = y.h; S.Kp[t][ph + 2 - 2 * th] = y.l;
                 *reinterpret_cast<float2*>(&S.X[t][2 * jp]) = make_float2(pr[e][0] * uj[0] * pk[e][0], pr[e][1] * uj[1] * pk[e][1]);
             }
         } else {
@@ -296,8 +303,8 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
         }
         {   // v: the two tokens of channel 2jp+z are one dword, stored in both halves of the cell
             const uint32_t v0 = (x.v[0] & 0xffffu) | (x.v[1] << 16), v1 = (x.v[0] >> 16) | (x.v[1] & 0xffff0000u);
-            S.Vd[2 * jp][4 * wid + th] = v0;     S.Vd[2 * jp][4 * wid + 2 + th] = v0;
-            S.Vd[2 * jp + 1][4 * wid + th] = v1; S.Vd[2 * jp + 1][4 * wid + 2 + th] = v1;
+            S.Vd[2 * jp][wcell + th] = v0;     S.Vd[2 * jp][wcell + 2 + th] = v0;
+            S.Vd[2 * jp + 1][wcell + th] = v1; S.Vd[2 * jp + 1][wcell + 2 + th] = v1;
         }
         __syncthreads();                               // B3
         if (c + STAGES < nchunks) prefetch(c + STAGES, x);   // this register set is free again
@@ -345,8 +352,8 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
             }
             __syncthreads();                           // B4: A is in LDS
             // -------------------------------------------------------------- Y += A V (tokens of half jh);  S^T = S^T diag(dec) + diag(d2) K'^T V
-            const bf16x8 vb0 = lds_op(&S.Vd[16 * q + l16][4 * g]);        // tokens  4g..4g+3
-            const bf16x8 vb1 = lds_op(&S.Vd[16 * q + l16][16 + 4 * g]);   // tokens 16+4g..
+            const bf16x8 vb0 = lds_op(&S.Vd[16 * q + l16][rc0]);        // tokens  4g..4g+3
+            const bf16x8 vb1 = lds_op(&S.Vd[16 * q + l16][rc1]);   // tokens 16+4g..
             if (jh == 0) {
                 Y[0] = mfma(lds_op(&S.Am[l16][4 * g]), vb0, Y[0]);
                 Y[1] = mfma(lds_op(&S.Am[16 + l16][4 * g]), vb0, Y[1]);
@@ -357,8 +364,8 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
             for (int m = 0; m < 2; ++m) {
                 const int j0 = 32 * jh + 16 * m;
                 f32x4 U = {0.f, 0.f, 0.f, 0.f};
-                U = mfma(lds_op(&S.KpT[j0 + l16][4 * g]), vb0, U);
-                U = mfma(lds_op(&S.KpT[j0 + l16][16 + 4 * g]), vb1, U);
+                U = mfma(lds_op(&S.KpT[j0 + l16][rc0]), vb0, U);
+                U = mfma(lds_op(&S.KpT[j0 + l16][rc1]), vb1, U);
                 const float4 de = *reinterpret_cast<const float4*>(&S.dec[j0 + 4 * g]);
                 const float4 d2 = *reinterpret_cast<const float4*>(&S.d2[j0 + 4 * g]);
                 D[m][0] = fmaf(D[m][0], de.x, d2.x * U[0]); D[m][1] = fmaf(D[m][1], de.y, d2.y * U[1]);
@@ -381,7 +388,7 @@ __global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
             }
             const uint16_t* vt = reinterpret_cast<const uint16_t*>(&S.Vd[16 * q + l16][0]);
             for (int t = 0; t < L; ++t) {
-                const float vi = bf2f(vt[8 * (t >> 2) + (t & 3)]);
+                const float vi = bf2f(vt[8 * ((t >> 2) ^ ((l16 >> 1) & 7)) + (t & 3)]);
                 float yp = 0.f;
 #pragma unroll
                 for (int m = 0; m < 2; ++m) {
@@ -439,6 +446,7 @@ struct alignas(16) SmemA {
     float u[N];
     float vgy[2][L];               // gy_t . v_t  (two partial sums)
     float part[8][N];
+    uint32_t flag[8];
     float P[2][2][L][RS];          // staging, double buffered: partial dr' of the two value-channel halves
 };
 
@@ -519,7 +527,13 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_a_chunk(const ArgsB a) {
             s4[z] = s2[z] + other[z];
         }
         if (th == 0) *reinterpret_cast<float2*>(&S.part[wid][2 * jp]) = make_float2(s4[0], s4[1]);
-        const bool exact = __syncthreads_or((-s4[0] > 0.25f * RANGE_LIMIT * LOG2E) || (-s4[1] > 0.25f * RANGE_LIMIT * LOG2E)) != 0;
+        {
+            const unsigned long long any = __ballot((-s4[0] > 0.25f * RANGE_LIMIT * LOG2E) || (-s4[1] > 0.25f * RANGE_LIMIT * LOG2E));
+            if (lane == 0) S.flag[wid] = any != 0ull;
+        }
+        __syncthreads();
+        const uint4 fl0 = *reinterpret_cast<const uint4*>(&S.flag[0]), fl1 = *reinterpret_cast<const uint4*>(&S.flag[4]);
+        const bool exact = (fl0.x | fl0.y | fl0.z | fl0.w | fl1.x | fl1.y | fl1.z | fl1.w) != 0;
         float pre[2] = {0.f, 0.f}, cm[2] = {0.f, 0.f}, cl[2] = {0.f, 0.f};
 #pragma unroll
         for (int w8 = 0; w8 < 8; ++w8) {
@@ -739,6 +753,7 @@ struct alignas(16) SmemB {
     float vgy[2][L];
     float ruk[2][L];               // exact path: sum_j r u k (two partial sums)
     float part[8][N];
+    uint32_t flag[8];
     float Ptot[2][N];              // chunk totals of (r dr' - k dk'), two partial sums
     float Pk[2][L][RS], Pv[2][L][RS], Pw[2][L][RS];   // staging: partial dk', gv, G of the two halves
 };
@@ -820,7 +835,13 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_b_chunk(const ArgsB a) {
             s4[z] = s2[z] + other[z];
         }
         if (th == 0) *reinterpret_cast<float2*>(&S.part[wid][2 * jp]) = make_float2(s4[0], s4[1]);
-        const bool exact = __syncthreads_or((-s4[0] > 0.25f * RANGE_LIMIT * LOG2E) || (-s4[1] > 0.25f * RANGE_LIMIT * LOG2E)) != 0;
+        {
+            const unsigned long long any = __ballot((-s4[0] > 0.25f * RANGE_LIMIT * LOG2E) || (-s4[1] > 0.25f * RANGE_LIMIT * LOG2E));
+            if (lane == 0) S.flag[wid] = any != 0ull;
+        }
+        __syncthreads();
+        const uint4 fl0 = *reinterpret_cast<const uint4*>(&S.flag[0]), fl1 = *reinterpret_cast<const uint4*>(&S.flag[4]);
+        const bool exact = (fl0.x | fl0.y | fl0.z | fl0.w | fl1.x | fl1.y | fl1.z | fl1.w) != 0;
         // totals of the chunk processed before this one (later in time) are complete now
         Pend += S.Ptot[0][16 * q + l16] + S.Ptot[1][16 * q + l16];
         float pre[2] = {0.f, 0.f}, cm[2] = {0.f, 0.f}, cl[2] = {0.f, 0.f};
