@@ -499,9 +499,9 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_a_chunk(const ArgsB a) {
     };
     static_for<STAGES>([&](auto Z) { if (decltype(Z)::value < nchunks) prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
 
-    float gu_acc[8];
+    float gu_acc[4];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) gu_acc[e] = 0.f;
+    for (int e = 0; e < 4; ++e) gu_acc[e] = 0.f;
 
     auto process = [&](const int c, Raw& x) __attribute__((always_inline)) {
         const int c0 = c * L, buf = c & 1;
@@ -670,32 +670,30 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_a_chunk(const ArgsB a) {
             }
         }
         __syncthreads();
-        if (tid < 256) {
-            const int t = tid >> 3, j0 = (tid & 7) * 8;
-            float drp[8], rr[8], kk[8];
-#pragma unroll
-            for (int z = 0; z < 2; ++z) {
-                const float4 x0 = *reinterpret_cast<const float4*>(&S.P[buf][0][t][j0 + 4 * z]);
-                const float4 x1 = *reinterpret_cast<const float4*>(&S.P[buf][1][t][j0 + 4 * z]);
-                const float4 ea = *reinterpret_cast<const float4*>(&S.Ea[t][j0 + 4 * z]);
-                drp[4 * z] = (x0.x + x1.x) * ea.x; drp[4 * z + 1] = (x0.y + x1.y) * ea.y;
-                drp[4 * z + 2] = (x0.z + x1.z) * ea.z; drp[4 * z + 3] = (x0.w + x1.w) * ea.w;
-            }
-            unpack8(*reinterpret_cast<const uint4*>(&S.Rr[t][j0 >> 1]), rr);
-            unpack8(*reinterpret_cast<const uint4*>(&S.Kr[t][j0 >> 1]), kk);
+        {
+            const int t = tid >> 4, j0 = (tid & 15) * 4;
+            const float4 x0 = *reinterpret_cast<const float4*>(&S.P[buf][0][t][j0]);
+            const float4 x1 = *reinterpret_cast<const float4*>(&S.P[buf][1][t][j0]);
+            const float4 ea = *reinterpret_cast<const float4*>(&S.Ea[t][j0]);
+            const float drp[4] = {(x0.x + x1.x) * ea.x, (x0.y + x1.y) * ea.y, (x0.z + x1.z) * ea.z, (x0.w + x1.w) * ea.w};
+            const uint2 rq = *reinterpret_cast<const uint2*>(&S.Rr[t][j0 >> 1]);
+            const uint2 kq = *reinterpret_cast<const uint2*>(&S.Kr[t][j0 >> 1]);
+            const float rr[4] = {bf_lo(rq.x), bf_hi(rq.x), bf_lo(rq.y), bf_hi(rq.y)};
+            const float kk[4] = {bf_lo(kq.x), bf_hi(kq.x), bf_lo(kq.y), bf_hi(kq.y)};
+            const float4 uu = *reinterpret_cast<const float4*>(&S.u[j0]);
+            const float ue[4] = {uu.x, uu.y, uu.z, uu.w};
             const float vgy = S.vgy[0][t] + S.vgy[1][t];
-            float out[8], rdr[8];
+            float out[4], rdr[4];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                out[e] = fmaf(S.u[j0 + e] * kk[e], vgy, drp[e]);
+            for (int e = 0; e < 4; ++e) {
+                out[e] = fmaf(ue[e] * kk[e], vgy, drp[e]);
                 rdr[e] = rr[e] * drp[e];
                 gu_acc[e] = fmaf(rr[e] * kk[e], vgy, gu_acc[e]);
             }
             if (c0 + t < T) {
                 const size_t off = base + static_cast<size_t>(c0 + t) * C + j0;
-                *reinterpret_cast<uint4*>(a.gr + off) = pack8(out);
+                *reinterpret_cast<uint2*>(a.gr + off) = make_uint2(pack_bf2(out[0], out[1]), pack_bf2(out[2], out[3]));
                 *reinterpret_cast<float4*>(a.rdr + off) = make_float4(rdr[0], rdr[1], rdr[2], rdr[3]);
-                *reinterpret_cast<float4*>(a.rdr + off + 4) = make_float4(rdr[4], rdr[5], rdr[6], rdr[7]);
             }
         }
     };
@@ -705,10 +703,10 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_a_chunk(const ArgsB a) {
 
     // gu[j] = sum over the 32 staging rows of the per-thread accumulators
     __syncthreads();
-    if (tid < 256) {
+    {
         float* G = &S.P[0][0][0][0];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) G[(tid >> 3) * RS + (tid & 7) * 8 + e] = gu_acc[e];
+        for (int e = 0; e < 4; ++e) G[(tid >> 4) * RS + (tid & 15) * 4 + e] = gu_acc[e];
     }
     __syncthreads();
     if (tid < N) {
@@ -1104,46 +1102,43 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_b_chunk(const ArgsB a) {
             if (g == 0) S.Ptot[hf][jl] = Pp - ((hf == 0) ? Pend : 0.f);
         }
         __syncthreads();
-        if (tid < 256) {
-            const int t = tid >> 3, j0 = (tid & 7) * 8;
-            float dk[8], dv[8], gw[8], rr[8], kk[8], gg[8];
-#pragma unroll
-            for (int z = 0; z < 2; ++z) {
-                const float4 k0 = *reinterpret_cast<const float4*>(&S.Pk[0][t][j0 + 4 * z]);
-                const float4 k1 = *reinterpret_cast<const float4*>(&S.Pk[1][t][j0 + 4 * z]);
-                const float4 eb = *reinterpret_cast<const float4*>(&S.Eb[t][j0 + 4 * z]);
-                dk[4 * z] = (k0.x + k1.x) * eb.x; dk[4 * z + 1] = (k0.y + k1.y) * eb.y;
-                dk[4 * z + 2] = (k0.z + k1.z) * eb.z; dk[4 * z + 3] = (k0.w + k1.w) * eb.w;
-                const float4 v0 = *reinterpret_cast<const float4*>(&S.Pv[0][t][j0 + 4 * z]);
-                const float4 v1 = *reinterpret_cast<const float4*>(&S.Pv[1][t][j0 + 4 * z]);
-                dv[4 * z] = v0.x + v1.x; dv[4 * z + 1] = v0.y + v1.y; dv[4 * z + 2] = v0.z + v1.z; dv[4 * z + 3] = v0.w + v1.w;
-                const float4 w0 = *reinterpret_cast<const float4*>(&S.Pw[0][t][j0 + 4 * z]);
-                const float4 w1 = *reinterpret_cast<const float4*>(&S.Pw[1][t][j0 + 4 * z]);
-                const float4 lm = *reinterpret_cast<const float4*>(&S.lam[t][j0 + 4 * z]);
-                gw[4 * z] = (w0.x + w1.x) * lm.x; gw[4 * z + 1] = (w0.y + w1.y) * lm.y;
-                gw[4 * z + 2] = (w0.z + w1.z) * lm.z; gw[4 * z + 3] = (w0.w + w1.w) * lm.w;
-            }
-            unpack8(*reinterpret_cast<const uint4*>(&S.Rr[t][j0 >> 1]), rr);
+        {
+            const int t = tid >> 4, j0 = (tid & 15) * 4;
+            const float4 k0 = *reinterpret_cast<const float4*>(&S.Pk[0][t][j0]);
+            const float4 k1 = *reinterpret_cast<const float4*>(&S.Pk[1][t][j0]);
+            const float4 eb = *reinterpret_cast<const float4*>(&S.Eb[t][j0]);
+            float dk[4] = {(k0.x + k1.x) * eb.x, (k0.y + k1.y) * eb.y, (k0.z + k1.z) * eb.z, (k0.w + k1.w) * eb.w};
+            const float4 v0 = *reinterpret_cast<const float4*>(&S.Pv[0][t][j0]);
+            const float4 v1 = *reinterpret_cast<const float4*>(&S.Pv[1][t][j0]);
+            float dv[4] = {v0.x + v1.x, v0.y + v1.y, v0.z + v1.z, v0.w + v1.w};
+            const float4 w0 = *reinterpret_cast<const float4*>(&S.Pw[0][t][j0]);
+            const float4 w1 = *reinterpret_cast<const float4*>(&S.Pw[1][t][j0]);
+            const float4 lm = *reinterpret_cast<const float4*>(&S.lam[t][j0]);
+            float gw[4] = {(w0.x + w1.x) * lm.x, (w0.y + w1.y) * lm.y, (w0.z + w1.z) * lm.z, (w0.w + w1.w) * lm.w};
+            const uint2 rq = *reinterpret_cast<const uint2*>(&S.Rr[t][j0 >> 1]);
+            const float rr[4] = {bf_lo(rq.x), bf_hi(rq.x), bf_lo(rq.y), bf_hi(rq.y)};
+            const float4 uu = *reinterpret_cast<const float4*>(&S.u[j0]);
+            const float ue[4] = {uu.x, uu.y, uu.z, uu.w};
             const float vgy = S.vgy[0][t] + S.vgy[1][t];
             if (exact) {                               // the bonus term of gv is not inside a tile here
-                unpack8(*reinterpret_cast<const uint4*>(&S.GY[t][j0 >> 1]), gg);
+                const uint2 gq = *reinterpret_cast<const uint2*>(&S.GY[t][j0 >> 1]);
+                const float gg[4] = {bf_lo(gq.x), bf_hi(gq.x), bf_lo(gq.y), bf_hi(gq.y)};
                 const float ruk = S.ruk[0][t] + S.ruk[1][t];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) dv[e] = fmaf(gg[e], ruk, dv[e]);
+                for (int e = 0; e < 4; ++e) dv[e] = fmaf(gg[e], ruk, dv[e]);
             }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) dk[e] = fmaf(S.u[j0 + e] * rr[e], vgy, dk[e]);
+            for (int e = 0; e < 4; ++e) dk[e] = fmaf(ue[e] * rr[e], vgy, dk[e]);
             if (!stateful && c0 + t == 0) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) gw[e] = 0.f;              // S_0 = 0: exact zero, as the reference leaves it
+                for (int e = 0; e < 4; ++e) gw[e] = 0.f;              // S_0 = 0: exact zero, as the reference leaves it
             }
             if (c0 + t < T) {
                 const size_t off = base + static_cast<size_t>(c0 + t) * C + j0;
-                *reinterpret_cast<uint4*>(a.gk + off) = pack8(dk);
-                *reinterpret_cast<uint4*>(a.gv + off) = pack8(dv);
-                *reinterpret_cast<uint4*>(a.gw + off) = pack8(gw);
+                *reinterpret_cast<uint2*>(a.gk + off) = make_uint2(pack_bf2(dk[0], dk[1]), pack_bf2(dk[2], dk[3]));
+                *reinterpret_cast<uint2*>(a.gv + off) = make_uint2(pack_bf2(dv[0], dv[1]), pack_bf2(dv[2], dv[3]));
+                *reinterpret_cast<uint2*>(a.gw + off) = make_uint2(pack_bf2(gw[0], gw[1]), pack_bf2(gw[2], gw[3]));
             }
-            (void)kk;
         }
     };
 
