@@ -1,0 +1,436 @@
+// wkv6 / wkv6_state forward: chunked formulation, wave-specialised workgroup (gfx950).
+//
+// One workgroup of 12 waves per (batch, head) walks the sequence in chunks of L = 32 tokens (formulas in wkv6_chunk.h).
+//   waves 0..7  ("prep")  load r, k, v, w two chunks ahead, take the in-chunk decay sums, and write the bf16 hi / lo planes of
+//                         R', K' and plain v into LDS in their natural [token][channel] layout; waves 0..2 also form the
+//                         causal tile A from those planes.
+//   waves 8..11 ("state") wave q owns value channels [16q, 16q+16) of the state for ALL key channels: S^T[j][i] in four 16x16
+//                         accumulator tiles.  Nothing it produces is a partial sum, so y goes from registers to memory.
+// The two kinds of wave meet at two barriers per chunk and otherwise run different chunks: while the state waves consume
+// chunk i, the prep waves write the operands of chunk i+1 (other buffer) and scan chunk i+2.
+//
+// Every operand whose contraction runs over tokens (v and K' in the state update, v in A V) is needed "transposed", i.e.
+// with a lane per channel and the tokens along the K slots.  Instead of writing transposed copies to LDS (narrow, bank
+// conflicting stores) the state waves multiply the natural planes by a one-hot selection matrix on the matrix cores:
+// the accumulator of  X[token][channel] * Sel  has a lane per selected channel and tokens down the registers, which after
+// packing to bf16 (exact: the inputs are bf16) IS the operand layout.  K slots may be assigned to channels or tokens in any
+// order as long as both operands agree, so accumulator layouts are used directly everywhere:
+//   state tile m, row 4g+v  <->  key channel 32 (m>>1) + 8g + 4 (m&1) + v     (so lane group g reads 8 consecutive channels)
+//   token slot (g, e)       <->  token 16 (e>>2) + 4g + (e&3);  A is stored with token s at position 8 ((s&15)>>2) + 4 (s>>4) + (s&3).
+#include "wkv6_chunk.h"
+
+namespace rwkv {
+namespace {
+
+constexpr int NPREP = 8;
+constexpr int NSTATE = 4;
+constexpr int NTF = (NPREP + NSTATE) * 64;
+constexpr int OS = 40;            // row stride (dwords) of a bf16 [token][channel] plane: 160 B, conflict-free for 16-byte reads
+
+struct alignas(16) OperandSet {
+    uint32_t RpH[L][OS], RpL[L][OS];   // r e^{c_t - c_m}      hi, lo   (exact path: r as fp32 [t][j] over both planes)
+    uint32_t KpH[L][OS], KpL[L][OS];   // k e^{c_m - c_{s+1}}  hi, lo   (exact path: k as fp32)
+    uint32_t V[L][OS];                 // v
+    float Wx[L][N];                    // exact path: decay of every step
+    float d1[N], d2[N], dec[N];        // e^{c_m}, e^{c_L - c_m}, e^{c_L}
+    float diag[L];                     // sum_j r u k
+    uint32_t exact, pad[3];
+};
+
+struct alignas(16) SmemF {
+    OperandSet set[2];
+    uint32_t AmH[L][OS], AmL[L][OS];   // A[t][position of s], hi and lo
+    float u[N];
+    float part[2][NPREP][N];           // sums of lam over each eighth of a chunk
+    uint32_t flag[2][NPREP];
+};
+
+template <int CTRL, int ROW_MASK> DEVINL float dpp_add(float x) {
+    return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xf, true));
+}
+// sum over lanes 0..31 in lane 31 and over lanes 32..63 in lane 63
+DEVINL float half_wave_sum(float x) {
+    x = dpp_add<0x118, 0xf>(x);       // row_shr:8
+    x = dpp_add<0x114, 0xf>(x);       // row_shr:4
+    x = dpp_add<0x112, 0xf>(x);       // row_shr:2
+    x = dpp_add<0x111, 0xf>(x);       // row_shr:1   -> lane 15 of every row holds the row sum
+    x = dpp_add<0x142, 0xa>(x);       // row_bcast:15 into rows 1 and 3
+    return x;
+}
+
+DEVINL uint4 one_hot(bool on, int e) {                       // 8 bf16 slots, 1.0 in slot e
+    const uint32_t bits = (e & 1) ? 0x3f800000u : 0x00003f80u;
+    const int d = e >> 1;
+    return make_uint4(on && d == 0 ? bits : 0u, on && d == 1 ? bits : 0u, on && d == 2 ? bits : 0u, on && d == 3 ? bits : 0u);
+}
+DEVINL bf16x8 op4(const uint4& x) { return __builtin_bit_cast(bf16x8, x); }
+
+// ---------------------------------------------------------------------------------------------------- prep waves
+template <int WMODE>
+DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base, const int h, const int nchunks) {
+    const int lane = tid & 63, wid = tid >> 6, l16 = lane & 15, g = lane >> 4;
+    const int T = a.T, C = a.C;
+    const uint16_t* __restrict__ rb = a.r + base;
+    const uint16_t* __restrict__ kb = a.k + base;
+    const uint16_t* __restrict__ vb = a.v + base;
+    // channel pair (2 jp, 2 jp + 1), tokens 4 wid + 2 th + {0, 1}
+    const int jp = lane & 31, th = lane >> 5, pt0 = 4 * wid + 2 * th;
+    const bool second = wid >= 4;
+    float uj[2];
+    {
+        const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + 2 * jp);
+        uj[0] = bf_lo(x); uj[1] = bf_hi(x);
+    }
+    struct Raw { uint32_t r[2], k[2], v[2], w[2][2]; float lam[2][2], other[2]; };
+    Raw ring[STAGES];
+    // The loads of a chunk are issued STAGES chunks before they are used.  They are written as asm so that the wait before
+    // the first use can name the number of younger loads that may still be in flight (the compiler would wait for all of
+    // them); every call issues the same eight loads (chunk index clamped), which keeps that number fixed.
+    const uint32_t* __restrict__ wb32 = reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + base);
+    const float* __restrict__ wbf = static_cast<const float*>(a.w) + base;
+    auto prefetch = [&](int c, Raw& x) __attribute__((always_inline)) {
+        c = c < nchunks ? c : nchunks - 1;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int t = c * L + pt0 + e;
+            const uint32_t o = (static_cast<uint32_t>(t < T ? t : T - 1) * C + 2 * jp) * 2;    // byte offset of the channel pair
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.r[e]) : "v"(o), "s"(rb));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.k[e]) : "v"(o), "s"(kb));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.v[e]) : "v"(o), "s"(vb));
+            if constexpr (WMODE == W_RAW) {
+                asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.w[e][0]) : "v"(o), "s"(wb32));
+            } else {
+                uint2 y;
+                asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(y) : "v"(2 * o), "s"(wbf));
+                x.w[e][0] = y.x; x.w[e][1] = y.y;
+            }
+        }
+    };
+    // wait until at most `younger` loads issued after those of x are outstanding
+    auto arrived = [&](Raw& x, auto younger) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(%10)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                     "+v"(x.w[0][0]), "+v"(x.w[0][1]), "+v"(x.w[1][0]), "+v"(x.w[1][1]) : "n"(decltype(younger)::value));
+    };
+    static_for<STAGES>([&](auto Z) { prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
+
+    // ---- scan of chunk c: lam (log2 units) of this thread's four elements, sums over each eighth of the chunk
+    auto scan = [&](const int c, Raw& x) __attribute__((always_inline)) {
+        const int c0 = c * L, pb = c & 1;
+        if (c0 + L > T) {                              // last, partial chunk: rows past T carry no input and no decay
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+                if (c0 + pt0 + e >= T) {
+                    x.r[e] = 0; x.k[e] = 0; x.v[e] = 0;
+                    x.w[e][0] = (WMODE == W_RAW) ? 0xff80ff80u : 0u;   // w = -inf  ->  lam = -exp(w) = 0
+                    x.w[e][1] = 0u;
+                }
+        }
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+#pragma unroll
+            for (int z = 0; z < 2; ++z) {
+                if constexpr (WMODE == W_RAW) x.lam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e][0]) : bf_lo(x.w[e][0])));
+                else x.lam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+            }
+        float s2[2];
+#pragma unroll
+        for (int z = 0; z < 2; ++z) {
+            s2[z] = x.lam[0][z] + x.lam[1][z];
+            x.other[z] = __shfl_xor(s2[z], 32, 64);    // the other two tokens of this wave's four
+        }
+        const float s4a = s2[0] + x.other[0], s4b = s2[1] + x.other[1];
+        if (th == 0) *reinterpret_cast<float2*>(&S.part[pb][wid][2 * jp]) = make_float2(s4a, s4b);
+        // A chunk whose decays could overflow the mid-point factors is redone exactly.  A half-chunk sum beyond the limit
+        // implies an eighth beyond limit/4, so this local test is sufficient (and conservative).
+        const bool fast_decay = (-s4a > 0.25f * RANGE_LIMIT * LOG2E) || (-s4b > 0.25f * RANGE_LIMIT * LOG2E);
+        const unsigned long long any = __ballot(fast_decay);
+        if (lane == 0) S.flag[pb][wid] = any != 0ull;
+    };
+
+    // ---- operands of chunk c into set c & 1; returns whether the chunk takes the exact path
+    auto operands = [&](const int c, Raw& x) __attribute__((always_inline)) -> bool {
+        OperandSet& O = S.set[c & 1];
+        const int pb = c & 1;
+        const uint4 f0 = *reinterpret_cast<const uint4*>(&S.flag[pb][0]), f1 = *reinterpret_cast<const uint4*>(&S.flag[pb][4]);
+        const bool exact = (f0.x | f0.y | f0.z | f0.w | f1.x | f1.y | f1.z | f1.w) != 0;
+        if (tid == 0) O.exact = exact;
+        // tokens of this half-chunk between this thread's pair and the middle of the chunk
+        float near[2];
+        near[0] = second ? (th ? x.other[0] : 0.f) : (th ? 0.f : x.other[0]);
+        near[1] = second ? (th ? x.other[1] : 0.f) : (th ? 0.f : x.other[1]);
+        {
+            const int lo = second ? 4 : wid + 1, hi = second ? wid : 4;      // wave-uniform bounds
+            for (int w8 = lo; w8 < hi; ++w8) {
+                const float2 y = *reinterpret_cast<const float2*>(&S.part[pb][w8][2 * jp]);
+                near[0] += y.x; near[1] += y.y;
+            }
+        }
+        if (wid == 0 && th == 0) {                     // per-channel factors of the whole chunk
+            float cm[2] = {0.f, 0.f}, ch[2] = {0.f, 0.f};
+#pragma unroll
+            for (int w8 = 0; w8 < 4; ++w8) {
+                const float2 y0 = *reinterpret_cast<const float2*>(&S.part[pb][w8][2 * jp]);
+                const float2 y1 = *reinterpret_cast<const float2*>(&S.part[pb][4 + w8][2 * jp]);
+                cm[0] += y0.x; cm[1] += y0.y; ch[0] += y1.x; ch[1] += y1.y;
+            }
+            *reinterpret_cast<float2*>(&O.d1[2 * jp]) = make_float2(exp2_fast(cm[0]), exp2_fast(cm[1]));
+            *reinterpret_cast<float2*>(&O.d2[2 * jp]) = make_float2(exp2_fast(ch[0]), exp2_fast(ch[1]));
+            *reinterpret_cast<float2*>(&O.dec[2 * jp]) = make_float2(exp2_fast(cm[0] + ch[0]), exp2_fast(cm[1] + ch[1]));
+        }
+        float pr[2][2], pk[2][2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            pr[e][0] = bf_lo(x.r[e]); pr[e][1] = bf_hi(x.r[e]);
+            pk[e][0] = bf_lo(x.k[e]); pk[e][1] = bf_hi(x.k[e]);
+        }
+        if (!exact) {
+            float rp[2][2], kp[2][2];
+#pragma unroll
+            for (int z = 0; z < 2; ++z) {
+                const Scale sc = chunk_scale(second, near[z], x.lam[0][z], x.lam[1][z]);
+                rp[0][z] = pr[0][z] * sc.ea[0]; rp[1][z] = pr[1][z] * sc.ea[1];
+                kp[0][z] = pk[0][z] * sc.eb[0]; kp[1][z] = pk[1][z] * sc.eb[1];
+            }
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int t = pt0 + e;
+                HL y = hilo2(rp[e][0], rp[e][1]); O.RpH[t][jp] = y.h; O.RpL[t][jp] = y.l;
+                y = hilo2(kp[e][0], kp[e][1]);    O.KpH[t][jp] = y.h; O.KpL[t][jp] = y.l;
+                const float d = half_wave_sum(fmaf(pr[e][0] * uj[0], pk[e][0], pr[e][1] * uj[1] * pk[e][1]));
+                if (jp == 31) O.diag[t] = d;
+            }
+        } else {
+            float* R = reinterpret_cast<float*>(&O.RpH[0][0]);
+            float* K = reinterpret_cast<float*>(&O.KpH[0][0]);
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const int t = pt0 + e;
+                *reinterpret_cast<float2*>(&R[t * N + 2 * jp]) = make_float2(pr[e][0], pr[e][1]);
+                *reinterpret_cast<float2*>(&K[t * N + 2 * jp]) = make_float2(pk[e][0], pk[e][1]);
+                *reinterpret_cast<float2*>(&O.Wx[t][2 * jp]) = make_float2(exp2_fast(x.lam[e][0]), exp2_fast(x.lam[e][1]));
+            }
+        }
+        O.V[pt0][jp] = x.v[0];
+        O.V[pt0 + 1][jp] = x.v[1];
+        return exact;
+    };
+
+    // ---- causal tile of chunk c (waves 0, 1, 2 -> quadrants (t,s) = (0,0) (1,0) (1,1)); rows of the accumulator are s
+    auto tile = [&](const int c) __attribute__((always_inline)) {
+        const OperandSet& O = S.set[c & 1];
+        const int ta = (wid == 0) ? 0 : 1, tb = (wid == 2) ? 1 : 0;
+        f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const bf16x8 kh = lds_op(&O.KpH[16 * tb + l16][16 * ks + 4 * g]), kl = lds_op(&O.KpL[16 * tb + l16][16 * ks + 4 * g]);
+            const bf16x8 rh = lds_op(&O.RpH[16 * ta + l16][16 * ks + 4 * g]), rl = lds_op(&O.RpL[16 * ta + l16][16 * ks + 4 * g]);
+            acc0 = mfma(kh, rh, acc0);
+            acc1 = mfma(kh, rl, acc1);
+            acc1 = mfma(kl, rh, acc1);
+        }
+        f32x4 acc = acc0 + acc1;                        // acc[v]: s = 16 tb + 4g + v, t = 16 ta + l16
+        if (ta == tb) {
+            const float d = O.diag[16 * ta + l16];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int sl = 4 * g + v;
+                acc[v] = (sl < l16) ? acc[v] : (sl == l16 ? d : 0.f);
+            }
+        }
+        const HL x0 = hilo2(acc[0], acc[1]), x1 = hilo2(acc[2], acc[3]);
+        *reinterpret_cast<uint2*>(&S.AmH[16 * ta + l16][4 * g + 2 * tb]) = make_uint2(x0.h, x1.h);
+        *reinterpret_cast<uint2*>(&S.AmL[16 * ta + l16][4 * g + 2 * tb]) = make_uint2(x0.l, x1.l);
+    };
+
+    static_for<STAGES>([&](auto Z) { arrived(ring[decltype(Z)::value], std::integral_constant<int, 0>{}); });
+    scan(0, ring[0]);
+    if (nchunks > 1) scan(1, ring[1]);
+    __syncthreads();
+    bool exact_cur = operands(0, ring[0]);
+    prefetch(STAGES, ring[0]);
+    __syncthreads();
+    for (int ib = 0; ib < nchunks; ib += STAGES)
+        static_for<STAGES>([&](auto Z) {
+            constexpr int z = decltype(Z)::value;
+            const int i = ib + z;
+            if (i < nchunks) {
+                bool exact_next = false;
+                if (i + 1 < nchunks) {
+                    exact_next = operands(i + 1, ring[(z + 1) % STAGES]);
+                }
+                prefetch(i + 1 + STAGES, ring[(z + 1) % STAGES]);
+                __syncthreads();
+                // younger than the loads of chunk i+2: those of chunks i+3, i+4, i+5
+                arrived(ring[(z + 2) % STAGES], std::integral_constant<int, 8 * (STAGES - 1)>{});
+                if (i + 2 < nchunks) scan(i + 2, ring[(z + 2) % STAGES]);
+                if (wid < 3 && !exact_cur) tile(i);
+                __syncthreads();
+                exact_cur = exact_next;
+            }
+        });
+}
+
+// ---------------------------------------------------------------------------------------------------- state waves
+template <int WMODE>
+DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base, const size_t bh, const int nchunks) {
+    const int lane = tid & 63, q = (tid >> 6) - NPREP, l16 = lane & 15, g = lane >> 4;
+    const int T = a.T, C = a.C;
+    const int i_own = 16 * q + l16;                    // this lane's value channel as a column of the state tiles
+    int j0[4];                                         // first key channel of this lane's four rows in tile m
+#pragma unroll
+    for (int m = 0; m < 4; ++m) j0[m] = 32 * (m >> 1) + 8 * g + 4 * (m & 1);
+
+    f32x4 D[4];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) D[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (a.s0 != nullptr) {
+        const uint16_t* s = a.s0 + (bh * N + i_own) * N;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            const uint2 x = *reinterpret_cast<const uint2*>(s + j0[m]);
+            D[m] = f32x4{bf_lo(x.x), bf_hi(x.x), bf_lo(x.y), bf_hi(x.y)};
+        }
+    }
+    // selection matrices (B operands).  v: column n <-> channel 16q + n of the 32-channel half q>>1;
+    // K', parity p: column n = row r of a state tile <-> channel 8 (r>>2) + 4p + (r&3) of the half.
+    const bf16x8 selV = op4(one_hot(g == 2 * (q & 1) + (l16 >> 3), l16 & 7));
+    const bf16x8 selK0 = op4(one_hot(g == (l16 >> 2), l16 & 3));
+    const bf16x8 selK1 = op4(one_hot(g == (l16 >> 2), 4 + (l16 & 3)));
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+
+    bf16x8 Vop = op4(make_uint4(0, 0, 0, 0));          // v of the current chunk: lane = value channel, slots = tokens
+    f32x4 Y[2] = {zero4, zero4};                        // y^T of the current chunk: lane = token, rows = value channels 16q + 4g + v
+
+    // y of chunk c: add A V and store
+    auto finish = [&](const int c) __attribute__((always_inline)) {
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            Y[tt] = mfma(Vop, lds_op(&S.AmH[16 * tt + l16][4 * g]), Y[tt]);
+            Y[tt] = mfma(Vop, lds_op(&S.AmL[16 * tt + l16][4 * g]), Y[tt]);
+            const int t = c * L + 16 * tt + l16;
+            if (t < T)
+                *reinterpret_cast<uint2*>(a.y + base + static_cast<size_t>(t) * C + 16 * q + 4 * g) =
+                    make_uint2(pack_bf2(Y[tt][0], Y[tt][1]), pack_bf2(Y[tt][2], Y[tt][3]));
+        }
+    };
+
+    __syncthreads();
+    __syncthreads();
+    bool exact_prev = true;
+    for (int i = 0; i < nchunks; ++i) {
+        const OperandSet& O = S.set[i & 1];
+        if (!exact_prev) finish(i - 1);
+        const bool exact = O.exact != 0;
+        if (!exact) {
+            // ------------------------------------------------------------ y^T = (d1 S) R'^T, contraction over key channels
+            Y[0] = zero4; Y[1] = zero4;
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const float4 da = *reinterpret_cast<const float4*>(&O.d1[j0[2 * ks]]);
+                const float4 db = *reinterpret_cast<const float4*>(&O.d1[j0[2 * ks + 1]]);
+                const HL x0 = hilo2(D[2 * ks][0] * da.x, D[2 * ks][1] * da.y), x1 = hilo2(D[2 * ks][2] * da.z, D[2 * ks][3] * da.w);
+                const HL x2 = hilo2(D[2 * ks + 1][0] * db.x, D[2 * ks + 1][1] * db.y), x3 = hilo2(D[2 * ks + 1][2] * db.z, D[2 * ks + 1][3] * db.w);
+                const bf16x8 sh = as_op(x0.h, x1.h, x2.h, x3.h), sl = as_op(x0.l, x1.l, x2.l, x3.l);
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt) {
+                    const bf16x8 rh = lds_op(&O.RpH[16 * tt + l16][16 * ks + 4 * g]), rl = lds_op(&O.RpL[16 * tt + l16][16 * ks + 4 * g]);
+                    Y[tt] = mfma(sh, rh, Y[tt]);
+                    Y[tt] = mfma(sh, rl, Y[tt]);
+                    Y[tt] = mfma(sl, rh, Y[tt]);
+                }
+            }
+            // ------------------------------------------------------------ v with a lane per value channel
+            {
+                const f32x4 z0 = mfma(lds_op(&O.V[l16][16 * (q >> 1) + 4 * g]), selV, zero4);
+                const f32x4 z1 = mfma(lds_op(&O.V[16 + l16][16 * (q >> 1) + 4 * g]), selV, zero4);
+                Vop = as_op(cvt2(z0[0], z0[1]), cvt2(z0[2], z0[3]), cvt2(z1[0], z1[1]), cvt2(z1[2], z1[3]));
+            }
+        } else {
+            // ------------------------------------------------------------ exact path: 32 sequential steps
+            const float* R = reinterpret_cast<const float*>(&O.RpH[0][0]);
+            const float* K = reinterpret_cast<const float*>(&O.KpH[0][0]);
+            float uv[4][4];
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const float4 y = *reinterpret_cast<const float4*>(&S.u[j0[m]]);
+                uv[m][0] = y.x; uv[m][1] = y.y; uv[m][2] = y.z; uv[m][3] = y.w;
+            }
+            for (int t = 0; t < L; ++t) {
+                const uint32_t vv = O.V[t][i_own >> 1];
+                const float vi = (l16 & 1) ? bf_hi(vv) : bf_lo(vv);
+                float yp = 0.f;
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    const float4 r4 = *reinterpret_cast<const float4*>(&R[t * N + j0[m]]);
+                    const float4 k4 = *reinterpret_cast<const float4*>(&K[t * N + j0[m]]);
+                    const float4 w4 = *reinterpret_cast<const float4*>(&O.Wx[t][j0[m]]);
+                    const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, ww[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const float kv = kk[v] * vi;
+                        yp = fmaf(rr[v], fmaf(uv[m][v], kv, D[m][v]), yp);
+                        D[m][v] = fmaf(D[m][v], ww[v], kv);
+                    }
+                }
+                const float y = allreduce_rows(yp);
+                if (g == 0 && i * L + t < T) a.y[base + static_cast<size_t>(i * L + t) * C + i_own] = f2bf(y);
+            }
+        }
+        __syncthreads();
+        if (!exact) {
+            // ------------------------------------------------------------ S^T = diag(dec) S^T + diag(d2) K'^T V
+#pragma unroll
+            for (int mh = 0; mh < 2; ++mh) {
+                const bf16x8 ah0 = lds_op(&O.KpH[l16][16 * mh + 4 * g]), ah1 = lds_op(&O.KpH[16 + l16][16 * mh + 4 * g]);
+                const bf16x8 al0 = lds_op(&O.KpL[l16][16 * mh + 4 * g]), al1 = lds_op(&O.KpL[16 + l16][16 * mh + 4 * g]);
+#pragma unroll
+                for (int par = 0; par < 2; ++par) {
+                    const int m = 2 * mh + par;
+                    const bf16x8 sel = par ? selK1 : selK0;
+                    const f32x4 zh0 = mfma(ah0, sel, zero4), zh1 = mfma(ah1, sel, zero4);
+                    const f32x4 zl0 = mfma(al0, sel, zero4), zl1 = mfma(al1, sel, zero4);
+                    const bf16x8 kh = as_op(cvt2(zh0[0], zh0[1]), cvt2(zh0[2], zh0[3]), cvt2(zh1[0], zh1[1]), cvt2(zh1[2], zh1[3]));
+                    const bf16x8 kl = as_op(cvt2(zl0[0], zl0[1]), cvt2(zl0[2], zl0[3]), cvt2(zl1[0], zl1[1]), cvt2(zl1[2], zl1[3]));
+                    f32x4 U = mfma(kh, Vop, zero4);
+                    U = mfma(kl, Vop, U);
+                    const float4 de = *reinterpret_cast<const float4*>(&O.dec[j0[m]]);
+                    const float4 d2 = *reinterpret_cast<const float4*>(&O.d2[j0[m]]);
+                    D[m][0] = fmaf(D[m][0], de.x, d2.x * U[0]); D[m][1] = fmaf(D[m][1], de.y, d2.y * U[1]);
+                    D[m][2] = fmaf(D[m][2], de.z, d2.z * U[2]); D[m][3] = fmaf(D[m][3], de.w, d2.w * U[3]);
+                }
+            }
+        }
+        __syncthreads();
+        exact_prev = exact;
+    }
+    if (!exact_prev) finish(nchunks - 1);
+}
+
+template <int WMODE>
+__global__ __launch_bounds__(NTF) void wkv6_fwd_ws(const ArgsC a) {
+    __shared__ SmemF S;
+    const int tid = threadIdx.x;
+    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
+    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
+    const size_t bh = static_cast<size_t>(b) * a.H + h;
+    const int nchunks = (a.T + L - 1) / L;
+    // positions of A that no tile ever writes (t < 16 <= s) must read as zero
+    for (int i = tid; i < L * OS; i += NTF) { (&S.AmH[0][0])[i] = 0; (&S.AmL[0][0])[i] = 0; }
+    if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
+    if (tid < NPREP * 64) fwd_prep<WMODE>(S, a, tid, base, h, nchunks);
+    else fwd_state<WMODE>(S, a, tid, base, bh, nchunks);
+}
+
+}  // namespace
+
+int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
+                          const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
+                          const uint16_t* s0, uint16_t* y) {
+    ArgsC a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y;
+    if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_fwd_ws<W_RAW>, dim3(B * H), dim3(NTF), 0, st, a);
+    else hipLaunchKernelGGL(wkv6_fwd_ws<W_EW>, dim3(B * H), dim3(NTF), 0, st, a);
+    return launch_status();
+}
+
+}  // namespace rwkv
