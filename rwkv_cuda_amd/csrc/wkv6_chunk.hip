@@ -24,314 +24,6 @@
 namespace rwkv {
 namespace {
 
-struct alignas(16) SmemFwd {
-    uint32_t Rp[L][RS];            // r e^{c_t - c_m}       cells along j       [t][j]   B operand of  A^T = K' R'^T, A operand of R' (d1 S0)^T
-    uint32_t Kp[L][RS];            // k e^{c_m - c_{s+1}}   cells along j       [s][j]   A operand of  A^T
-    uint32_t KpT[N][TS];           // the same values       cells along tokens  [j][s]   A operand of  S^T += K'^T V
-    uint32_t Am[L][TS];            // A                     cells along s       [t][s]   A operand of  A V
-    uint32_t Vd[N][TS];            // v, [v0 v1 v2 v3 | v0 v1 v2 v3] per 4 tokens [i][s] B operand
-    float X[L][N];                 // r u k [t][j], summed over j into the diagonal of A;  exact path: r
-    float raw[2][L][N];            // exact path only: k, decay as fp32 [t][j]
-    float d1[N], d2[N], dec[N];    // e^{c_m}, e^{c_L - c_m}, e^{c_L}   (exact path: d1 = u)
-    float part[8][N];              // sum of lam (log2 units) over each eighth of the chunk
-    uint32_t flag[8];              // per wave: some channel decays too fast for the mid-point factors
-    float Y[2][2][L][RS];          // output staging, double buffered: partial sums of the two key-channel halves
-};
-
-// One workgroup of 8 waves per (batch, head).  Wave (q = wid & 3, jh = wid >> 2) owns value channels [16q, 16q+16) and the
-// key-channel half [32jh, 32jh+32) of the state: S^T[j][i] in two accumulator tiles,  D[m][v] <-> j = 32jh + 16m + 4g + v.
-// The accumulator layout is used as is as the B operand of R' (d1 S0)^T (lane group g holds channels 4g..4g+3 of each tile).
-// Three barriers per chunk: [scan parts] B2 [operands] B3 [A tiles | store of the previous chunk | R' S0^T] B4 [A V, state].
-template <int WMODE>
-__global__ __launch_bounds__(NT) void wkv6_fwd_chunk(const ArgsC a) {
-    __shared__ SmemFwd S;
-    const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6, l16 = lane & 15, g = lane >> 4;
-    const int q = wid & 3, jh = wid >> 2;
-    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
-    const int T = a.T, C = a.C;
-    const size_t base = static_cast<size_t>(b) * T * C + static_cast<size_t>(h) * N;
-    const size_t bh = static_cast<size_t>(b) * a.H + h;
-    const uint16_t* __restrict__ rb = a.r + base;
-    const uint16_t* __restrict__ kb = a.k + base;
-    const uint16_t* __restrict__ vb_ = a.v + base;
-    // prep coordinates: channel pair (2 jp, 2 jp + 1), tokens 4 wid + 2 th + {0, 1}
-    const int jp = lane & 31, th = lane >> 5, pt0 = 4 * wid + 2 * th;
-    const bool second = wid >= 4;
-    // [channel][token] arrays keep the 16-byte cell of tokens 4c..4c+3 of row `ch` at cell index c ^ ((ch >> 1) & 7), which
-    // spreads the one-dword-per-lane writes of the prep over the banks.  Writer: rows 2jp, 2jp+1, cell wid.
-    // Reader: rows (multiple of 16) + l16, cells g and 4 + g.
-    const int wcell = 4 * (wid ^ (jp & 7));
-    const int rc0 = 4 * (g ^ ((l16 >> 1) & 7)), rc1 = 4 * ((4 + g) ^ ((l16 >> 1) & 7));
-    float uj[2];
-    {
-        const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + 2 * jp);
-        uj[0] = bf_lo(x); uj[1] = bf_hi(x);
-    }
-
-    f32x4 D[2];
-    D[0] = D[1] = f32x4{0.f, 0.f, 0.f, 0.f};
-    if (a.s0 != nullptr) {
-        const uint16_t* s = a.s0 + (bh * N + q * 16 + l16) * N + 32 * jh;
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-            const uint2 x = *reinterpret_cast<const uint2*>(s + 16 * m + 4 * g);
-            D[m] = f32x4{bf_lo(x.x), bf_hi(x.x), bf_lo(x.y), bf_hi(x.y)};
-        }
-    }
-    // the upper-right 16x16 tile of A (t < 16 <= s) is never written: keep it zero
-    for (int i = tid; i < L * TS; i += NT) (&S.Am[0][0])[i] = 0;
-
-    const int nchunks = (T + L - 1) / L;
-    // Raw bits of the chunks to come (two channels per load), converted only when a chunk is prepared.  HBM latency is
-    // a few microseconds and a chunk is ~1 us of work, so STAGES chunks are kept in flight (one register set each; the
-    // chunk loop is unrolled by STAGES to keep the set index static).
-    struct Raw { uint32_t r[2], k[2], v[2], w[2][2]; };
-    Raw ring[STAGES];
-    auto prefetch = [&](int c, Raw& x) __attribute__((always_inline)) {
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const int t = c * L + pt0 + e;
-            const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C + 2 * jp;
-            x.r[e] = *reinterpret_cast<const uint32_t*>(rb + o);
-            x.k[e] = *reinterpret_cast<const uint32_t*>(kb + o);
-            x.v[e] = *reinterpret_cast<const uint32_t*>(vb_ + o);
-            if constexpr (WMODE == W_RAW) {
-                x.w[e][0] = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + base + o);
-            } else {
-                const uint2 y = *reinterpret_cast<const uint2*>(static_cast<const float*>(a.w) + base + o);
-                x.w[e][0] = y.x; x.w[e][1] = y.y;
-            }
-        }
-    };
-    static_for<STAGES>([&](auto Z) { if (decltype(Z)::value < nchunks) prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
-
-    // rows (c0 + t) of staging buffer `buf` -> y, by 256 threads
-    auto store_y = [&](int c0, int buf, int idx) __attribute__((always_inline)) {
-        const int t = idx >> 3, i0 = (idx & 7) * 8;
-        if (c0 + t < T) {
-            float f[8];
-#pragma unroll
-            for (int z = 0; z < 2; ++z) {
-                const float4 x0 = *reinterpret_cast<const float4*>(&S.Y[buf][0][t][i0 + 4 * z]);
-                const float4 x1 = *reinterpret_cast<const float4*>(&S.Y[buf][1][t][i0 + 4 * z]);
-                f[4 * z] = x0.x + x1.x; f[4 * z + 1] = x0.y + x1.y; f[4 * z + 2] = x0.z + x1.z; f[4 * z + 3] = x0.w + x1.w;
-            }
-            *reinterpret_cast<uint4*>(a.y + base + static_cast<size_t>(c0 + t) * C + i0) = pack8(f);
-        }
-    };
-
-    auto process = [&](const int c, Raw& x) __attribute__((always_inline)) {
-        const int c0 = c * L, buf = c & 1;
-        if (c0 + L > T) {                              // last, partial chunk: rows past T carry no input and no decay
-#pragma unroll
-            for (int e = 0; e < 2; ++e)
-                if (c0 + pt0 + e >= T) {
-                    x.r[e] = 0; x.k[e] = 0; x.v[e] = 0;
-                    x.w[e][0] = (WMODE == W_RAW) ? 0xff80ff80u : 0u;   // w = -inf  ->  lam = -exp(w) = 0
-                    x.w[e][1] = 0u;
-                }
-        }
-        // ------------------------------------------------------------------ scan.  element [e][z]: token pt0 + e, channel 2 jp + z
-        float plam[2][2];                              // lam in log2 units
-#pragma unroll
-        for (int e = 0; e < 2; ++e)
-#pragma unroll
-            for (int z = 0; z < 2; ++z) {
-                if constexpr (WMODE == W_RAW) plam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e][0]) : bf_lo(x.w[e][0])));
-                else plam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
-            }
-        float s2[2], other[2];
-#pragma unroll
-        for (int z = 0; z < 2; ++z) {
-            s2[z] = plam[0][z] + plam[1][z];
-            other[z] = __shfl_xor(s2[z], 32, 64);      // the other two tokens of this wave's four
-        }
-        const float s4a = s2[0] + other[0], s4b = s2[1] + other[1];
-        if (th == 0) *reinterpret_cast<float2*>(&S.part[wid][2 * jp]) = make_float2(s4a, s4b);
-        // A chunk whose decays could overflow the mid-point factors is redone exactly.  A half-chunk sum beyond the limit
-        // implies an eighth beyond limit/4, so this local test is sufficient (and conservative).
-        const bool fast_decay = (-s4a > 0.25f * RANGE_LIMIT * LOG2E) || (-s4b > 0.25f * RANGE_LIMIT * LOG2E);
-        const unsigned long long any = __ballot(fast_decay);
-        if (lane == 0) S.flag[wid] = any != 0ull;
-        __syncthreads();                               // B2
-        const uint4 f0 = *reinterpret_cast<const uint4*>(&S.flag[0]), f1 = *reinterpret_cast<const uint4*>(&S.flag[4]);
-        const bool exact = (f0.x | f0.y | f0.z | f0.w | f1.x | f1.y | f1.z | f1.w) != 0;
-        // tokens of this half-chunk between this thread's pair and the middle of the chunk
-        float near[2];
-        near[0] = second ? (th ? other[0] : 0.f) : (th ? 0.f : other[0]);
-        near[1] = second ? (th ? other[1] : 0.f) : (th ? 0.f : other[1]);
-        {
-            const int lo = second ? 4 : wid + 1, hi = second ? wid : 4;      // wave-uniform bounds
-            for (int w8 = lo; w8 < hi; ++w8) {
-                const float2 y = *reinterpret_cast<const float2*>(&S.part[w8][2 * jp]);
-                near[0] += y.x; near[1] += y.y;
-            }
-        }
-        if (wid == 0 && th == 0) {                     // per-channel factors of the whole chunk
-            float cm[2] = {0.f, 0.f}, ch[2] = {0.f, 0.f};
-#pragma unroll
-            for (int w8 = 0; w8 < 4; ++w8) {
-                const float2 y0 = *reinterpret_cast<const float2*>(&S.part[w8][2 * jp]);
-                const float2 y1 = *reinterpret_cast<const float2*>(&S.part[4 + w8][2 * jp]);
-                cm[0] += y0.x; cm[1] += y0.y; ch[0] += y1.x; ch[1] += y1.y;
-            }
-            if (!exact) *reinterpret_cast<float2*>(&S.d1[2 * jp]) = make_float2(exp2_fast(cm[0]), exp2_fast(cm[1]));
-            else *reinterpret_cast<float2*>(&S.d1[2 * jp]) = make_float2(uj[0], uj[1]);
-            *reinterpret_cast<float2*>(&S.d2[2 * jp]) = make_float2(exp2_fast(ch[0]), exp2_fast(ch[1]));
-            *reinterpret_cast<float2*>(&S.dec[2 * jp]) = make_float2(exp2_fast(cm[0] + ch[0]), exp2_fast(cm[1] + ch[1]));
-        }
-        float pr[2][2], pk[2][2];
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            pr[e][0] = bf_lo(x.r[e]); pr[e][1] = bf_hi(x.r[e]);
-            pk[e][0] = bf_lo(x.k[e]); pk[e][1] = bf_hi(x.k[e]);
-        }
-        if (!exact) {
-            float rp[2][2], kp[2][2];
-#pragma unroll
-            for (int z = 0; z < 2; ++z) {
-                const Scale sc = chunk_scale(second, near[z], plam[0][z], plam[1][z]);
-                rp[0][z] = pr[0][z] * sc.ea[0]; rp[1][z] = pr[1][z] * sc.ea[1];
-                kp[0][z] = pk[0][z] * sc.eb[0]; kp[1][z] = pk[1][z] * sc.eb[1];
-                const HL y = hilo2(kp[0][z], kp[1][z]);              // pair along the two tokens
-                S.KpT[2 * jp + z][wcell + th] = y.h;
-                S.KpT[2 * jp + z][wcell + 2 + th] = y.l;
-            }
-            const int ph = hpos(jp);
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const int t = pt0 + e;
-                // cells of rows written by the upper half-wave are stored with their halves exchanged: every consumer adds
-                // both orders (mfma_full), and the two half-waves then hit disjoint LDS banks
-                HL y = hilo2(rp[e][0], rp[e][1]); S.Rp[t][ph + 2 * th] = y.h; S.Rp[t][ph + 2 - 2 * th] = y.l;
-                y = hilo2(kp[e][0], kp[e][1]);    S.Kp[t][ph + 2 * th] = y.h; S.Kp[t][ph + 2 - 2 * th] = y.l;
-                *reinterpret_cast<float2*>(&S.X[t][2 * jp]) = make_float2(pr[e][0] * uj[0] * pk[e][0], pr[e][1] * uj[1] * pk[e][1]);
-            }
-        } else {
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const int t = pt0 + e;
-                *reinterpret_cast<float2*>(&S.X[t][2 * jp]) = make_float2(pr[e][0], pr[e][1]);
-                *reinterpret_cast<float2*>(&S.raw[0][t][2 * jp]) = make_float2(pk[e][0], pk[e][1]);
-                *reinterpret_cast<float2*>(&S.raw[1][t][2 * jp]) = make_float2(exp2_fast(plam[e][0]), exp2_fast(plam[e][1]));
-            }
-        }
-        {   // v: the two tokens of channel 2jp+z are one dword, stored in both halves of the cell
-            const uint32_t v0 = (x.v[0] & 0xffffu) | (x.v[1] << 16), v1 = (x.v[0] >> 16) | (x.v[1] & 0xffff0000u);
-            S.Vd[2 * jp][wcell + th] = v0;     S.Vd[2 * jp][wcell + 2 + th] = v0;
-            S.Vd[2 * jp + 1][wcell + th] = v1; S.Vd[2 * jp + 1][wcell + 2 + th] = v1;
-        }
-        __syncthreads();                               // B3
-        if (c + STAGES < nchunks) prefetch(c + STAGES, x);   // this register set is free again
-
-        f32x4 Y[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
-        if (!exact) {
-            if (wid < 3) {
-                // ---------------------------------------------------------- A^T tiles: waves 0,1,2 -> A(0,0) A(1,0) A(1,1)
-                const int ta = (wid == 0) ? 0 : 1, tb = (wid == 2) ? 1 : 0;
-                f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int js = 0; js < 4; js += 2) {     // rows of the result: s (from K'), columns: t (from R')
-                    acc0 = mfma_full_lds(&S.Kp[16 * tb + l16][16 * js + 4 * g], lds_op(&S.Rp[16 * ta + l16][16 * js + 4 * g]), acc0);
-                    acc1 = mfma_full_lds(&S.Kp[16 * tb + l16][16 * js + 16 + 4 * g], lds_op(&S.Rp[16 * ta + l16][16 * js + 16 + 4 * g]), acc1);
-                }
-                f32x4 acc = acc0 + acc1;                // acc[v]: s = 4g + v, t = l16
-                if (ta == tb) {
-                    float d = 0.f;                      // diagonal: sum_j r u k of row t = 16 ta + l16
-#pragma unroll
-                    for (int z = 0; z < 4; ++z) {
-                        const float4 y = *reinterpret_cast<const float4*>(&S.X[16 * ta + l16][16 * g + 4 * z]);
-                        d += (y.x + y.y) + (y.z + y.w);
-                    }
-                    d = allreduce_rows(d);
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const int sl = 4 * g + v;
-                        acc[v] = (sl < l16) ? acc[v] : (sl == l16 ? d : 0.f);
-                    }
-                }
-                const HL x0 = hilo2(acc[0], acc[1]), x1 = hilo2(acc[2], acc[3]);
-                *reinterpret_cast<uint4*>(&S.Am[16 * ta + l16][16 * tb + 4 * g]) = make_uint4(x0.h, x1.h, x0.l, x1.l);
-            } else if (wid >= 4 && c > 0) {
-                store_y(c0 - L, buf ^ 1, tid - 256);   // the previous chunk's output leaves while the tiles are computed
-            }
-            // -------------------------------------------------------------- Y (this half of j) = R' (d1 S0)^T
-#pragma unroll
-            for (int m = 0; m < 2; ++m) {
-                const int j0 = 32 * jh + 16 * m + 4 * g;
-                const float4 dd = *reinterpret_cast<const float4*>(&S.d1[j0]);
-                const HL x0 = hilo2(D[m][0] * dd.x, D[m][1] * dd.y), x1 = hilo2(D[m][2] * dd.z, D[m][3] * dd.w);
-                const bf16x8 sb = as_op(x0.h, x1.h, x0.l, x1.l);
-#pragma unroll
-                for (int mt = 0; mt < 2; ++mt) Y[mt] = mfma_full_lds(&S.Rp[16 * mt + l16][j0], sb, Y[mt]);
-            }
-            __syncthreads();                           // B4: A is in LDS
-            // -------------------------------------------------------------- Y += A V (tokens of half jh);  S^T = S^T diag(dec) + diag(d2) K'^T V
-            const bf16x8 vb0 = lds_op(&S.Vd[16 * q + l16][rc0]);        // tokens  4g..4g+3
-            const bf16x8 vb1 = lds_op(&S.Vd[16 * q + l16][rc1]);   // tokens 16+4g..
-            if (jh == 0) {
-                Y[0] = mfma(lds_op(&S.Am[l16][4 * g]), vb0, Y[0]);
-                Y[1] = mfma(lds_op(&S.Am[16 + l16][4 * g]), vb0, Y[1]);
-            } else {
-                Y[1] = mfma(lds_op(&S.Am[16 + l16][16 + 4 * g]), vb1, Y[1]);
-            }
-#pragma unroll
-            for (int m = 0; m < 2; ++m) {
-                const int j0 = 32 * jh + 16 * m;
-                f32x4 U = {0.f, 0.f, 0.f, 0.f};
-                U = mfma(lds_op(&S.KpT[j0 + l16][rc0]), vb0, U);
-                U = mfma(lds_op(&S.KpT[j0 + l16][rc1]), vb1, U);
-                const float4 de = *reinterpret_cast<const float4*>(&S.dec[j0 + 4 * g]);
-                const float4 d2 = *reinterpret_cast<const float4*>(&S.d2[j0 + 4 * g]);
-                D[m][0] = fmaf(D[m][0], de.x, d2.x * U[0]); D[m][1] = fmaf(D[m][1], de.y, d2.y * U[1]);
-                D[m][2] = fmaf(D[m][2], de.z, d2.z * U[2]); D[m][3] = fmaf(D[m][3], de.w, d2.w * U[3]);
-            }
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) S.Y[buf][jh][16 * mt + 4 * g + v][16 * q + l16] = Y[mt][v];
-        } else {
-            // -------------------------------------------------------------- exact path: 32 sequential steps
-            // lane (i = 16q + l16, group g) holds S[i][j] for j = 32 jh + 16 m + 4 g + v
-            if (wid >= 4 && c > 0) store_y(c0 - L, buf ^ 1, tid - 256);
-            __syncthreads();                           // keeps the barrier count equal on both paths
-            float uv[2][4];
-#pragma unroll
-            for (int m = 0; m < 2; ++m) {
-                const float4 y = *reinterpret_cast<const float4*>(&S.d1[32 * jh + 16 * m + 4 * g]);   // u on this path
-                uv[m][0] = y.x; uv[m][1] = y.y; uv[m][2] = y.z; uv[m][3] = y.w;
-            }
-            const uint16_t* vt = reinterpret_cast<const uint16_t*>(&S.Vd[16 * q + l16][0]);
-            for (int t = 0; t < L; ++t) {
-                const float vi = bf2f(vt[8 * ((t >> 2) ^ ((l16 >> 1) & 7)) + (t & 3)]);
-                float yp = 0.f;
-#pragma unroll
-                for (int m = 0; m < 2; ++m) {
-                    const int j0 = 32 * jh + 16 * m + 4 * g;
-                    const float4 r4 = *reinterpret_cast<const float4*>(&S.X[t][j0]);
-                    const float4 k4 = *reinterpret_cast<const float4*>(&S.raw[0][t][j0]);
-                    const float4 w4 = *reinterpret_cast<const float4*>(&S.raw[1][t][j0]);
-                    const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, ww[4] = {w4.x, w4.y, w4.z, w4.w};
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const float kv = kk[v] * vi;
-                        yp = fmaf(rr[v], fmaf(uv[m][v], kv, D[m][v]), yp);
-                        D[m][v] = fmaf(D[m][v], ww[v], kv);
-                    }
-                }
-                const float y = allreduce_rows(yp);
-                if (g == 0) S.Y[buf][jh][t][16 * q + l16] = y;
-            }
-        }
-    };
-
-    for (int cb = 0; cb < nchunks; cb += STAGES)
-        static_for<STAGES>([&](auto Z) { if (cb + decltype(Z)::value < nchunks) process(cb + decltype(Z)::value, ring[decltype(Z)::value]); });
-
-    __syncthreads();
-    if (tid < 256) store_y((nchunks - 1) * L, (nchunks - 1) & 1, tid);
-}
-
 // ======================================================================================================================
 // Backward, first sweep (time ascending): gr, gu and the workspace r * dr' that the decay gradient needs.
 //     dr'_t[j] = sum_i gy_t[i] S_t[i][j] = Ea_t[j] ( e^{c_m}[j] (GY S0)[t][j] + (Bm K')[t][j] ),   Ea_t = e^{c_t - c_m},
@@ -368,7 +60,7 @@ struct alignas(16) SmemA {
 template <int WMODE>
 __global__ __launch_bounds__(NT) void wkv6_bwd_a_chunk(const ArgsB a) {
     __shared__ SmemA S;
-    const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6, l16 = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x, lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, g = lane >> 4;
     const int q = wid & 3, ih = wid >> 2;
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
     const int T = a.T, C = a.C;
@@ -395,24 +87,35 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_a_chunk(const ArgsB a) {
     const int nchunks = (T + L - 1) / L;
     struct Raw { uint32_t r[2], k[2], v[2], g[2], w[2][2]; };
     Raw ring[STAGES];
+    // Loads are asm so that the wait before their first use can leave the younger batches in flight (the compiler would
+    // wait for every outstanding load); each call issues the same ten loads (chunk index clamped), so that count is fixed.
+    const uint32_t* __restrict__ wb32 = reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + base);
+    const float* __restrict__ wbf = static_cast<const float*>(a.w) + base;
     auto prefetch = [&](int c, Raw& x) __attribute__((always_inline)) {
+        c = c < nchunks ? c : nchunks - 1;
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int t = c * L + pt0 + e;
-            const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C + 2 * jp;
-            x.r[e] = *reinterpret_cast<const uint32_t*>(rb + o);
-            x.k[e] = *reinterpret_cast<const uint32_t*>(kb + o);
-            x.v[e] = *reinterpret_cast<const uint32_t*>(vb_ + o);
-            x.g[e] = *reinterpret_cast<const uint32_t*>(gb + o);
+            const uint32_t o = (static_cast<uint32_t>(t < T ? t : T - 1) * C + 2 * jp) * 2;    // byte offset
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.r[e]) : "v"(o), "s"(rb));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.k[e]) : "v"(o), "s"(kb));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.v[e]) : "v"(o), "s"(vb_));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.g[e]) : "v"(o), "s"(gb));
             if constexpr (WMODE == W_RAW) {
-                x.w[e][0] = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + base + o);
+                asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.w[e][0]) : "v"(o), "s"(wb32));
             } else {
-                const uint2 y = *reinterpret_cast<const uint2*>(static_cast<const float*>(a.w) + base + o);
+                uint2 y;
+                asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(y) : "v"(2 * o), "s"(wbf));
                 x.w[e][0] = y.x; x.w[e][1] = y.y;
             }
         }
     };
-    static_for<STAGES>([&](auto Z) { if (decltype(Z)::value < nchunks) prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
+    // the batches of the next STAGES - 1 chunks (ten loads each) may stay in flight
+    auto arrived = [&](Raw& x) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(%12)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                     "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[0][1]), "+v"(x.w[1][0]), "+v"(x.w[1][1]) : "n"(10 * (STAGES - 1)));
+    };
+    static_for<STAGES>([&](auto Z) { prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
 
     float gu_acc[4];
 #pragma unroll
@@ -420,6 +123,7 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_a_chunk(const ArgsB a) {
 
     auto process = [&](const int c, Raw& x) __attribute__((always_inline)) {
         const int c0 = c * L, buf = c & 1;
+        arrived(x);
         float pk[2][2], plam[2][2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
@@ -500,7 +204,7 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_a_chunk(const ArgsB a) {
             *reinterpret_cast<uint32_t*>(vt + (2 * jp + 1) * (2 * VS) + pt0) = (x.v[0] >> 16) | (x.v[1] & 0xffff0000u);
         }
         __syncthreads();
-        if (c + STAGES < nchunks) prefetch(c + STAGES, x);
+        prefetch(c + STAGES, x);
 
         const float d1j = S.d1[16 * q + l16], d2j = S.d2[16 * q + l16], decj = S.dec[16 * q + l16];
         if (!exact) {
@@ -702,29 +406,40 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_b_chunk(const ArgsB a) {
     const int nchunks = (T + L - 1) / L;
     struct Raw { uint32_t r[2], k[2], v[2], g[2], w[2][2]; float2 d[2]; };
     Raw ring[STAGES_B];
+    // asm loads with an explicit wait, as in the first sweep; twelve loads per call
+    const uint32_t* __restrict__ wb32 = reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + base);
+    const float* __restrict__ wbf = static_cast<const float*>(a.w) + base;
     auto prefetch = [&](int c, Raw& x) __attribute__((always_inline)) {
+        c = c > 0 ? c : 0;
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int t = c * L + pt0 + e;
-            const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C + 2 * jp;
-            x.r[e] = *reinterpret_cast<const uint32_t*>(rb + o);
-            x.k[e] = *reinterpret_cast<const uint32_t*>(kb + o);
-            x.v[e] = *reinterpret_cast<const uint32_t*>(vb_ + o);
-            x.g[e] = *reinterpret_cast<const uint32_t*>(gb + o);
-            x.d[e] = *reinterpret_cast<const float2*>(db + o);
+            const uint32_t o = (static_cast<uint32_t>(t < T ? t : T - 1) * C + 2 * jp) * 2;    // byte offset
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.r[e]) : "v"(o), "s"(rb));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.k[e]) : "v"(o), "s"(kb));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.v[e]) : "v"(o), "s"(vb_));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.g[e]) : "v"(o), "s"(gb));
+            asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(x.d[e]) : "v"(2 * o), "s"(db));
             if constexpr (WMODE == W_RAW) {
-                x.w[e][0] = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + base + o);
+                asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.w[e][0]) : "v"(o), "s"(wb32));
             } else {
-                const uint2 y = *reinterpret_cast<const uint2*>(static_cast<const float*>(a.w) + base + o);
+                uint2 y;
+                asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(y) : "v"(2 * o), "s"(wbf));
                 x.w[e][0] = y.x; x.w[e][1] = y.y;
             }
         }
     };
+    auto arrived = [&](Raw& x) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(%14)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                     "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[0][1]), "+v"(x.w[1][0]), "+v"(x.w[1][1]),
+                     "+v"(x.d[0]), "+v"(x.d[1]) : "n"(12 * (STAGES_B - 1)));
+    };
     // chunks are visited last to first; ci counts visits
-    static_for<STAGES_B>([&](auto Z) { if (decltype(Z)::value < nchunks) prefetch(nchunks - 1 - decltype(Z)::value, ring[decltype(Z)::value]); });
+    static_for<STAGES_B>([&](auto Z) { prefetch(nchunks - 1 - decltype(Z)::value, ring[decltype(Z)::value]); });
 
     auto process = [&](const int ci, Raw& x) __attribute__((always_inline)) {
         const int c = nchunks - 1 - ci, c0 = c * L;
+        arrived(x);
         float pr[2][2], pk[2][2], plam[2][2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
@@ -821,7 +536,7 @@ __global__ __launch_bounds__(NT) void wkv6_bwd_b_chunk(const ArgsB a) {
             *reinterpret_cast<uint32_t*>(gt + (2 * jp + 1) * (2 * VS) + pt0) = (x.g[0] >> 16) | (x.g[1] & 0xffff0000u);
         }
         __syncthreads();
-        if (ci + STAGES_B < nchunks) prefetch(nchunks - 1 - (ci + STAGES_B), x);
+        prefetch(nchunks - 1 - (ci + STAGES_B), x);
 
         const int jl = 16 * q + l16;                   // D: this lane's key channel;  E: this lane's value channel
         const float d1j = S.d1[jl], d2j = S.d2[jl], decj = S.dec[jl];

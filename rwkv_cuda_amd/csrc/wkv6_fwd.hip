@@ -1,11 +1,12 @@
 // wkv6 / wkv6_state forward: chunked formulation, wave-specialised workgroup (gfx950).
 //
-// One workgroup of 12 waves per (batch, head) walks the sequence in chunks of L = 32 tokens (formulas in wkv6_chunk.h).
-//   waves 0..7  ("prep")  load r, k, v, w two chunks ahead, take the in-chunk decay sums, and write the bf16 hi / lo planes of
+// One workgroup of 16 waves per (batch, head) walks the sequence in chunks of L = 32 tokens (formulas in wkv6_chunk.h).
+//   waves 0..7  ("prep")  load r, k, v, w ahead of time, take the in-chunk decay sums, and write the bf16 hi / lo planes of
 //                         R', K' and plain v into LDS in their natural [token][channel] layout; waves 0..2 also form the
 //                         causal tile A from those planes.
-//   waves 8..11 ("state") wave q owns value channels [16q, 16q+16) of the state for ALL key channels: S^T[j][i] in four 16x16
-//                         accumulator tiles.  Nothing it produces is a partial sum, so y goes from registers to memory.
+//   waves 8..15 ("state") wave (q, jh) owns value channels [16q, 16q+16) x key channels [32jh, 32jh+32) of the state:
+//                         S^T[j][i] in two 16x16 accumulator tiles.  The two waves of a q exchange one partial y tile
+//                         (a 16-byte LDS write and read per lane) and each stores 16 tokens of y straight from registers.
 // The two kinds of wave meet at two barriers per chunk and otherwise run different chunks: while the state waves consume
 // chunk i, the prep waves write the operands of chunk i+1 (other buffer) and scan chunk i+2.
 //
@@ -23,7 +24,7 @@ namespace rwkv {
 namespace {
 
 constexpr int NPREP = 8;
-constexpr int NSTATE = 4;
+constexpr int NSTATE = 8;
 constexpr int NTF = (NPREP + NSTATE) * 64;
 constexpr int OS = 40;            // row stride (dwords) of a bf16 [token][channel] plane: 160 B, conflict-free for 16-byte reads
 
@@ -39,7 +40,9 @@ struct alignas(16) OperandSet {
 
 struct alignas(16) SmemF {
     OperandSet set[2];
-    uint32_t AmH[L][OS], AmL[L][OS];   // A[t][position of s], hi and lo
+    uint32_t AmH[2][L][OS], AmL[2][L][OS];   // A[t][position of s], hi and lo, double buffered
+    float4 Xch[2][NSTATE][64];         // partial y tile handed to the partner wave, double buffered
+    float Yx[2][2][L][N];              // exact path: partial y of the two key-channel halves, double buffered
     float u[N];
     float part[2][NPREP][N];           // sums of lam over each eighth of a chunk
     uint32_t flag[2][NPREP];
@@ -68,7 +71,7 @@ DEVINL bf16x8 op4(const uint4& x) { return __builtin_bit_cast(bf16x8, x); }
 // ---------------------------------------------------------------------------------------------------- prep waves
 template <int WMODE>
 DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base, const int h, const int nchunks) {
-    const int lane = tid & 63, wid = tid >> 6, l16 = lane & 15, g = lane >> 4;
+    const int lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
     const uint16_t* __restrict__ rb = a.r + base;
     const uint16_t* __restrict__ kb = a.k + base;
@@ -81,7 +84,7 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + 2 * jp);
         uj[0] = bf_lo(x); uj[1] = bf_hi(x);
     }
-    struct Raw { uint32_t r[2], k[2], v[2], w[2][2]; float lam[2][2], other[2]; };
+    struct Raw { uint32_t r[2], k[2], v[2], w[2][2]; float lam[2][2], other[2], kp[2][2]; };
     Raw ring[STAGES];
     // The loads of a chunk are issued STAGES chunks before they are used.  They are written as asm so that the wait before
     // the first use can name the number of younger loads that may still be in flight (the compiler would wait for all of
@@ -147,25 +150,78 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         if (lane == 0) S.flag[pb][wid] = any != 0ull;
     };
 
-    // ---- operands of chunk c into set c & 1; returns whether the chunk takes the exact path
-    auto operands = [&](const int c, Raw& x) __attribute__((always_inline)) -> bool {
+    // ---- operands of chunk c into set c & 1, first part: R' planes (and the K' values kept in registers for the second
+    //      part); returns whether the chunk takes the exact path
+    auto operands_a = [&](const int c, Raw& x) __attribute__((always_inline)) -> bool {
         OperandSet& O = S.set[c & 1];
         const int pb = c & 1;
         const uint4 f0 = *reinterpret_cast<const uint4*>(&S.flag[pb][0]), f1 = *reinterpret_cast<const uint4*>(&S.flag[pb][4]);
+        // sums of lam over the eighths of this thread's half-chunk; those between this wave's eighth and the middle count
+        float2 pe[4];
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4) pe[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * second + w4][2 * jp]);
         const bool exact = (f0.x | f0.y | f0.z | f0.w | f1.x | f1.y | f1.z | f1.w) != 0;
         if (tid == 0) O.exact = exact;
-        // tokens of this half-chunk between this thread's pair and the middle of the chunk
         float near[2];
         near[0] = second ? (th ? x.other[0] : 0.f) : (th ? 0.f : x.other[0]);
         near[1] = second ? (th ? x.other[1] : 0.f) : (th ? 0.f : x.other[1]);
-        {
-            const int lo = second ? 4 : wid + 1, hi = second ? wid : 4;      // wave-uniform bounds
-            for (int w8 = lo; w8 < hi; ++w8) {
-                const float2 y = *reinterpret_cast<const float2*>(&S.part[pb][w8][2 * jp]);
-                near[0] += y.x; near[1] += y.y;
+        const int w_own = wid & 3;
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4) {
+            const bool between = second ? (w4 < w_own) : (w4 > w_own);      // wave-uniform
+            near[0] += between ? pe[w4].x : 0.f;
+            near[1] += between ? pe[w4].y : 0.f;
+        }
+        float pr[2][2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) { pr[e][0] = bf_lo(x.r[e]); pr[e][1] = bf_hi(x.r[e]); }
+        if (!exact) {
+            float rp[2][2];
+#pragma unroll
+            for (int z = 0; z < 2; ++z) {
+                const Scale sc = chunk_scale(second, near[z], x.lam[0][z], x.lam[1][z]);
+                rp[0][z] = pr[0][z] * sc.ea[0]; rp[1][z] = pr[1][z] * sc.ea[1];
+                x.kp[0][z] = (z ? bf_hi(x.k[0]) : bf_lo(x.k[0])) * sc.eb[0];
+                x.kp[1][z] = (z ? bf_hi(x.k[1]) : bf_lo(x.k[1])) * sc.eb[1];
+            }
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const HL y = hilo2(rp[e][0], rp[e][1]);
+                O.RpH[pt0 + e][jp] = y.h; O.RpL[pt0 + e][jp] = y.l;
+            }
+        } else {
+            float* R = reinterpret_cast<float*>(&O.RpH[0][0]);
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                *reinterpret_cast<float2*>(&R[(pt0 + e) * N + 2 * jp]) = make_float2(pr[e][0], pr[e][1]);
+                *reinterpret_cast<float2*>(&O.Wx[pt0 + e][2 * jp]) = make_float2(exp2_fast(x.lam[e][0]), exp2_fast(x.lam[e][1]));
             }
         }
-        if (wid == 0 && th == 0) {                     // per-channel factors of the whole chunk
+        return exact;
+    };
+    // ---- second part: K' planes, v, the diagonal of A; wave 3 adds the per-channel factors of the whole chunk
+    auto operands_b = [&](const int c, Raw& x, const bool exact) __attribute__((always_inline)) {
+        OperandSet& O = S.set[c & 1];
+        const int pb = c & 1;
+        float pk[2][2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) { pk[e][0] = bf_lo(x.k[e]); pk[e][1] = bf_hi(x.k[e]); }
+        if (!exact) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const HL y = hilo2(x.kp[e][0], x.kp[e][1]);
+                O.KpH[pt0 + e][jp] = y.h; O.KpL[pt0 + e][jp] = y.l;
+                const float d = half_wave_sum(fmaf(bf_lo(x.r[e]) * uj[0], pk[e][0], bf_hi(x.r[e]) * uj[1] * pk[e][1]));
+                if (jp == 31) O.diag[pt0 + e] = d;
+            }
+        } else {
+            float* K = reinterpret_cast<float*>(&O.KpH[0][0]);
+#pragma unroll
+            for (int e = 0; e < 2; ++e) *reinterpret_cast<float2*>(&K[(pt0 + e) * N + 2 * jp]) = make_float2(pk[e][0], pk[e][1]);
+        }
+        O.V[pt0][jp] = x.v[0];
+        O.V[pt0 + 1][jp] = x.v[1];
+        if (wid == 3 && th == 0) {
             float cm[2] = {0.f, 0.f}, ch[2] = {0.f, 0.f};
 #pragma unroll
             for (int w8 = 0; w8 < 4; ++w8) {
@@ -177,42 +233,6 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
             *reinterpret_cast<float2*>(&O.d2[2 * jp]) = make_float2(exp2_fast(ch[0]), exp2_fast(ch[1]));
             *reinterpret_cast<float2*>(&O.dec[2 * jp]) = make_float2(exp2_fast(cm[0] + ch[0]), exp2_fast(cm[1] + ch[1]));
         }
-        float pr[2][2], pk[2][2];
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            pr[e][0] = bf_lo(x.r[e]); pr[e][1] = bf_hi(x.r[e]);
-            pk[e][0] = bf_lo(x.k[e]); pk[e][1] = bf_hi(x.k[e]);
-        }
-        if (!exact) {
-            float rp[2][2], kp[2][2];
-#pragma unroll
-            for (int z = 0; z < 2; ++z) {
-                const Scale sc = chunk_scale(second, near[z], x.lam[0][z], x.lam[1][z]);
-                rp[0][z] = pr[0][z] * sc.ea[0]; rp[1][z] = pr[1][z] * sc.ea[1];
-                kp[0][z] = pk[0][z] * sc.eb[0]; kp[1][z] = pk[1][z] * sc.eb[1];
-            }
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const int t = pt0 + e;
-                HL y = hilo2(rp[e][0], rp[e][1]); O.RpH[t][jp] = y.h; O.RpL[t][jp] = y.l;
-                y = hilo2(kp[e][0], kp[e][1]);    O.KpH[t][jp] = y.h; O.KpL[t][jp] = y.l;
-                const float d = half_wave_sum(fmaf(pr[e][0] * uj[0], pk[e][0], pr[e][1] * uj[1] * pk[e][1]));
-                if (jp == 31) O.diag[t] = d;
-            }
-        } else {
-            float* R = reinterpret_cast<float*>(&O.RpH[0][0]);
-            float* K = reinterpret_cast<float*>(&O.KpH[0][0]);
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const int t = pt0 + e;
-                *reinterpret_cast<float2*>(&R[t * N + 2 * jp]) = make_float2(pr[e][0], pr[e][1]);
-                *reinterpret_cast<float2*>(&K[t * N + 2 * jp]) = make_float2(pk[e][0], pk[e][1]);
-                *reinterpret_cast<float2*>(&O.Wx[t][2 * jp]) = make_float2(exp2_fast(x.lam[e][0]), exp2_fast(x.lam[e][1]));
-            }
-        }
-        O.V[pt0][jp] = x.v[0];
-        O.V[pt0 + 1][jp] = x.v[1];
-        return exact;
     };
 
     // ---- causal tile of chunk c (waves 0, 1, 2 -> quadrants (t,s) = (0,0) (1,0) (1,1)); rows of the accumulator are s
@@ -238,120 +258,137 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
             }
         }
         const HL x0 = hilo2(acc[0], acc[1]), x1 = hilo2(acc[2], acc[3]);
-        *reinterpret_cast<uint2*>(&S.AmH[16 * ta + l16][4 * g + 2 * tb]) = make_uint2(x0.h, x1.h);
-        *reinterpret_cast<uint2*>(&S.AmL[16 * ta + l16][4 * g + 2 * tb]) = make_uint2(x0.l, x1.l);
+        *reinterpret_cast<uint2*>(&S.AmH[c & 1][16 * ta + l16][4 * g + 2 * tb]) = make_uint2(x0.h, x1.h);
+        *reinterpret_cast<uint2*>(&S.AmL[c & 1][16 * ta + l16][4 * g + 2 * tb]) = make_uint2(x0.l, x1.l);
     };
 
     static_for<STAGES>([&](auto Z) { arrived(ring[decltype(Z)::value], std::integral_constant<int, 0>{}); });
     scan(0, ring[0]);
     if (nchunks > 1) scan(1, ring[1]);
     __syncthreads();
-    bool exact_cur = operands(0, ring[0]);
+    bool exact_cur = operands_a(0, ring[0]);
+    operands_b(0, ring[0], exact_cur);
     prefetch(STAGES, ring[0]);
     __syncthreads();
+    // iteration i: scan(i+2), tile(i), operands(i+1); one barrier
     for (int ib = 0; ib < nchunks; ib += STAGES)
         static_for<STAGES>([&](auto Z) {
             constexpr int z = decltype(Z)::value;
             const int i = ib + z;
             if (i < nchunks) {
-                bool exact_next = false;
-                if (i + 1 < nchunks) {
-                    exact_next = operands(i + 1, ring[(z + 1) % STAGES]);
-                }
-                prefetch(i + 1 + STAGES, ring[(z + 1) % STAGES]);
-                __syncthreads();
-                // younger than the loads of chunk i+2: those of chunks i+3, i+4, i+5
-                arrived(ring[(z + 2) % STAGES], std::integral_constant<int, 8 * (STAGES - 1)>{});
+                // younger than the loads of chunk i+2: those of chunks i+3 and i+4
+                arrived(ring[(z + 2) % STAGES], std::integral_constant<int, 8 * (STAGES - 2)>{});
                 if (i + 2 < nchunks) scan(i + 2, ring[(z + 2) % STAGES]);
                 if (wid < 3 && !exact_cur) tile(i);
+                bool exact_next = false;
+                if (i + 1 < nchunks) {
+                    exact_next = operands_a(i + 1, ring[(z + 1) % STAGES]);
+                    operands_b(i + 1, ring[(z + 1) % STAGES], exact_next);
+                }
+                prefetch(i + 1 + STAGES, ring[(z + 1) % STAGES]);
                 __syncthreads();
                 exact_cur = exact_next;
             }
         });
+    __syncthreads();
 }
 
 // ---------------------------------------------------------------------------------------------------- state waves
 template <int WMODE>
 DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base, const size_t bh, const int nchunks) {
-    const int lane = tid & 63, q = (tid >> 6) - NPREP, l16 = lane & 15, g = lane >> 4;
+    const int lane = tid & 63, sw = __builtin_amdgcn_readfirstlane(tid >> 6) - NPREP, q = sw & 3, jh = sw >> 2, l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
     const int i_own = 16 * q + l16;                    // this lane's value channel as a column of the state tiles
-    int j0[4];                                         // first key channel of this lane's four rows in tile m
-#pragma unroll
-    for (int m = 0; m < 4; ++m) j0[m] = 32 * (m >> 1) + 8 * g + 4 * (m & 1);
+    const int j0[2] = {32 * jh + 8 * g, 32 * jh + 8 * g + 4};   // first key channel of this lane's four rows in tile mm
 
-    f32x4 D[4];
-#pragma unroll
-    for (int m = 0; m < 4; ++m) D[m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    f32x4 D[2];
+    D[0] = D[1] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (a.s0 != nullptr) {
-        const uint16_t* s = a.s0 + (bh * N + i_own) * N;
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-            const uint2 x = *reinterpret_cast<const uint2*>(s + j0[m]);
-            D[m] = f32x4{bf_lo(x.x), bf_hi(x.x), bf_lo(x.y), bf_hi(x.y)};
-        }
+        const uint4 x = *reinterpret_cast<const uint4*>(a.s0 + (bh * N + i_own) * N + j0[0]);
+        D[0] = f32x4{bf_lo(x.x), bf_hi(x.x), bf_lo(x.y), bf_hi(x.y)};
+        D[1] = f32x4{bf_lo(x.z), bf_hi(x.z), bf_lo(x.w), bf_hi(x.w)};
     }
     // selection matrices (B operands).  v: column n <-> channel 16q + n of the 32-channel half q>>1;
-    // K', parity p: column n = row r of a state tile <-> channel 8 (r>>2) + 4p + (r&3) of the half.
+    // K', parity p: column n = row r of a state tile <-> channel 8 (r>>2) + 4p + (r&3) of the half jh.
     const bf16x8 selV = op4(one_hot(g == 2 * (q & 1) + (l16 >> 3), l16 & 7));
     const bf16x8 selK0 = op4(one_hot(g == (l16 >> 2), l16 & 3));
     const bf16x8 selK1 = op4(one_hot(g == (l16 >> 2), 4 + (l16 & 3)));
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
 
-    bf16x8 Vop = op4(make_uint4(0, 0, 0, 0));          // v of the current chunk: lane = value channel, slots = tokens
-    f32x4 Y[2] = {zero4, zero4};                        // y^T of the current chunk: lane = token, rows = value channels 16q + 4g + v
+    bf16x8 Vop = op4(make_uint4(0, 0, 0, 0));          // v of the chunk in flight: lane = value channel, K slots = tokens
+    f32x4 Yk = zero4;                                  // y^T rows 16q + 4g + v, tokens 16 jh + l16: this half of the key channels
 
-    // y of chunk c: add A V and store
-    auto finish = [&](const int c) __attribute__((always_inline)) {
-#pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-            Y[tt] = mfma(Vop, lds_op(&S.AmH[16 * tt + l16][4 * g]), Y[tt]);
-            Y[tt] = mfma(Vop, lds_op(&S.AmL[16 * tt + l16][4 * g]), Y[tt]);
-            const int t = c * L + 16 * tt + l16;
+    // y of chunk c (tokens 16 jh + l16): own half + partner's half + A V
+    auto finish = [&](const int c, const bool was_exact) __attribute__((always_inline)) {
+        if (!was_exact) {
+            const float4 p = S.Xch[c & 1][sw ^ 4][lane];
+            f32x4 Y = Yk + f32x4{p.x, p.y, p.z, p.w};
+            Y = mfma(Vop, lds_op(&S.AmH[c & 1][16 * jh + l16][4 * g]), Y);
+            Y = mfma(Vop, lds_op(&S.AmL[c & 1][16 * jh + l16][4 * g]), Y);
+            const int t = c * L + 16 * jh + l16;
             if (t < T)
                 *reinterpret_cast<uint2*>(a.y + base + static_cast<size_t>(t) * C + 16 * q + 4 * g) =
-                    make_uint2(pack_bf2(Y[tt][0], Y[tt][1]), pack_bf2(Y[tt][2], Y[tt][3]));
+                    make_uint2(pack_bf2(Y[0], Y[1]), pack_bf2(Y[2], Y[3]));
+        } else {                                       // exact path: add the two halves and store
+            const int idx = tid - NPREP * 64, t = idx >> 4, i4 = (idx & 15) * 4;
+            const float4 p0 = *reinterpret_cast<const float4*>(&S.Yx[c & 1][0][t][i4]);
+            const float4 p1 = *reinterpret_cast<const float4*>(&S.Yx[c & 1][1][t][i4]);
+            if (c * L + t < T)
+                *reinterpret_cast<uint2*>(a.y + base + static_cast<size_t>(c * L + t) * C + i4) =
+                    make_uint2(pack_bf2(p0.x + p1.x, p0.y + p1.y), pack_bf2(p0.z + p1.z, p0.w + p1.w));
         }
     };
 
     __syncthreads();
     __syncthreads();
-    bool exact_prev = true;
+    bool exact_prev = false;
     for (int i = 0; i < nchunks; ++i) {
         const OperandSet& O = S.set[i & 1];
-        if (!exact_prev) finish(i - 1);
         const bool exact = O.exact != 0;
+        if (i > 0) finish(i - 1, exact_prev);
         if (!exact) {
-            // ------------------------------------------------------------ y^T = (d1 S) R'^T, contraction over key channels
-            Y[0] = zero4; Y[1] = zero4;
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                const float4 da = *reinterpret_cast<const float4*>(&O.d1[j0[2 * ks]]);
-                const float4 db = *reinterpret_cast<const float4*>(&O.d1[j0[2 * ks + 1]]);
-                const HL x0 = hilo2(D[2 * ks][0] * da.x, D[2 * ks][1] * da.y), x1 = hilo2(D[2 * ks][2] * da.z, D[2 * ks][3] * da.w);
-                const HL x2 = hilo2(D[2 * ks + 1][0] * db.x, D[2 * ks + 1][1] * db.y), x3 = hilo2(D[2 * ks + 1][2] * db.z, D[2 * ks + 1][3] * db.w);
-                const bf16x8 sh = as_op(x0.h, x1.h, x2.h, x3.h), sl = as_op(x0.l, x1.l, x2.l, x3.l);
-#pragma unroll
-                for (int tt = 0; tt < 2; ++tt) {
-                    const bf16x8 rh = lds_op(&O.RpH[16 * tt + l16][16 * ks + 4 * g]), rl = lds_op(&O.RpL[16 * tt + l16][16 * ks + 4 * g]);
-                    Y[tt] = mfma(sh, rh, Y[tt]);
-                    Y[tt] = mfma(sh, rl, Y[tt]);
-                    Y[tt] = mfma(sl, rh, Y[tt]);
-                }
-            }
+            // ------------------------------------------------------------ y^T = (d1 S) R'^T over this wave's key channels
+            const float4 da = *reinterpret_cast<const float4*>(&O.d1[j0[0]]);
+            const float4 db = *reinterpret_cast<const float4*>(&O.d1[j0[1]]);
+            const bf16x8 rh0 = lds_op(&O.RpH[l16][16 * jh + 4 * g]), rl0 = lds_op(&O.RpL[l16][16 * jh + 4 * g]);
+            const bf16x8 rh1 = lds_op(&O.RpH[16 + l16][16 * jh + 4 * g]), rl1 = lds_op(&O.RpL[16 + l16][16 * jh + 4 * g]);
+            const bf16x8 va0 = lds_op(&O.V[l16][16 * (q >> 1) + 4 * g]), va1 = lds_op(&O.V[16 + l16][16 * (q >> 1) + 4 * g]);
+            const HL x0 = hilo2(D[0][0] * da.x, D[0][1] * da.y), x1 = hilo2(D[0][2] * da.z, D[0][3] * da.w);
+            const HL x2 = hilo2(D[1][0] * db.x, D[1][1] * db.y), x3 = hilo2(D[1][2] * db.z, D[1][3] * db.w);
+            const bf16x8 sh = as_op(x0.h, x1.h, x2.h, x3.h), sl = as_op(x0.l, x1.l, x2.l, x3.l);
+            f32x4 Y0 = mfma(sh, rh0, zero4), Y1 = mfma(sh, rh1, zero4);
+            Y0 = mfma(sh, rl0, Y0); Y1 = mfma(sh, rl1, Y1);
+            Y0 = mfma(sl, rh0, Y0); Y1 = mfma(sl, rh1, Y1);
+            // the partner wave (other key-channel half) finishes the other 16 tokens
+            S.Xch[i & 1][sw][lane] = jh ? make_float4(Y0[0], Y0[1], Y0[2], Y0[3]) : make_float4(Y1[0], Y1[1], Y1[2], Y1[3]);
+            Yk = jh ? Y1 : Y0;
             // ------------------------------------------------------------ v with a lane per value channel
-            {
-                const f32x4 z0 = mfma(lds_op(&O.V[l16][16 * (q >> 1) + 4 * g]), selV, zero4);
-                const f32x4 z1 = mfma(lds_op(&O.V[16 + l16][16 * (q >> 1) + 4 * g]), selV, zero4);
-                Vop = as_op(cvt2(z0[0], z0[1]), cvt2(z0[2], z0[3]), cvt2(z1[0], z1[1]), cvt2(z1[2], z1[3]));
+            const f32x4 z0 = mfma(va0, selV, zero4), z1 = mfma(va1, selV, zero4);
+            Vop = as_op(cvt2(z0[0], z0[1]), cvt2(z0[2], z0[3]), cvt2(z1[0], z1[1]), cvt2(z1[2], z1[3]));
+            // ------------------------------------------------------------ S^T = diag(dec) S^T + diag(d2) K'^T V
+            const bf16x8 ah0 = lds_op(&O.KpH[l16][16 * jh + 4 * g]), ah1 = lds_op(&O.KpH[16 + l16][16 * jh + 4 * g]);
+            const bf16x8 al0 = lds_op(&O.KpL[l16][16 * jh + 4 * g]), al1 = lds_op(&O.KpL[16 + l16][16 * jh + 4 * g]);
+#pragma unroll
+            for (int par = 0; par < 2; ++par) {
+                const bf16x8 sel = par ? selK1 : selK0;
+                const f32x4 zh0 = mfma(ah0, sel, zero4), zh1 = mfma(ah1, sel, zero4);
+                const f32x4 zl0 = mfma(al0, sel, zero4), zl1 = mfma(al1, sel, zero4);
+                const bf16x8 kh = as_op(cvt2(zh0[0], zh0[1]), cvt2(zh0[2], zh0[3]), cvt2(zh1[0], zh1[1]), cvt2(zh1[2], zh1[3]));
+                const bf16x8 kl = as_op(cvt2(zl0[0], zl0[1]), cvt2(zl0[2], zl0[3]), cvt2(zl1[0], zl1[1]), cvt2(zl1[2], zl1[3]));
+                f32x4 U = mfma(kh, Vop, zero4);
+                U = mfma(kl, Vop, U);
+                const float4 de = *reinterpret_cast<const float4*>(&O.dec[j0[par]]);
+                const float4 d2 = *reinterpret_cast<const float4*>(&O.d2[j0[par]]);
+                D[par][0] = fmaf(D[par][0], de.x, d2.x * U[0]); D[par][1] = fmaf(D[par][1], de.y, d2.y * U[1]);
+                D[par][2] = fmaf(D[par][2], de.z, d2.z * U[2]); D[par][3] = fmaf(D[par][3], de.w, d2.w * U[3]);
             }
         } else {
             // ------------------------------------------------------------ exact path: 32 sequential steps
             const float* R = reinterpret_cast<const float*>(&O.RpH[0][0]);
             const float* K = reinterpret_cast<const float*>(&O.KpH[0][0]);
-            float uv[4][4];
+            float uv[2][4];
 #pragma unroll
-            for (int m = 0; m < 4; ++m) {
+            for (int m = 0; m < 2; ++m) {
                 const float4 y = *reinterpret_cast<const float4*>(&S.u[j0[m]]);
                 uv[m][0] = y.x; uv[m][1] = y.y; uv[m][2] = y.z; uv[m][3] = y.w;
             }
@@ -360,7 +397,7 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
                 const float vi = (l16 & 1) ? bf_hi(vv) : bf_lo(vv);
                 float yp = 0.f;
 #pragma unroll
-                for (int m = 0; m < 4; ++m) {
+                for (int m = 0; m < 2; ++m) {
                     const float4 r4 = *reinterpret_cast<const float4*>(&R[t * N + j0[m]]);
                     const float4 k4 = *reinterpret_cast<const float4*>(&K[t * N + j0[m]]);
                     const float4 w4 = *reinterpret_cast<const float4*>(&O.Wx[t][j0[m]]);
@@ -373,37 +410,14 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
                     }
                 }
                 const float y = allreduce_rows(yp);
-                if (g == 0 && i * L + t < T) a.y[base + static_cast<size_t>(i * L + t) * C + i_own] = f2bf(y);
-            }
-        }
-        __syncthreads();
-        if (!exact) {
-            // ------------------------------------------------------------ S^T = diag(dec) S^T + diag(d2) K'^T V
-#pragma unroll
-            for (int mh = 0; mh < 2; ++mh) {
-                const bf16x8 ah0 = lds_op(&O.KpH[l16][16 * mh + 4 * g]), ah1 = lds_op(&O.KpH[16 + l16][16 * mh + 4 * g]);
-                const bf16x8 al0 = lds_op(&O.KpL[l16][16 * mh + 4 * g]), al1 = lds_op(&O.KpL[16 + l16][16 * mh + 4 * g]);
-#pragma unroll
-                for (int par = 0; par < 2; ++par) {
-                    const int m = 2 * mh + par;
-                    const bf16x8 sel = par ? selK1 : selK0;
-                    const f32x4 zh0 = mfma(ah0, sel, zero4), zh1 = mfma(ah1, sel, zero4);
-                    const f32x4 zl0 = mfma(al0, sel, zero4), zl1 = mfma(al1, sel, zero4);
-                    const bf16x8 kh = as_op(cvt2(zh0[0], zh0[1]), cvt2(zh0[2], zh0[3]), cvt2(zh1[0], zh1[1]), cvt2(zh1[2], zh1[3]));
-                    const bf16x8 kl = as_op(cvt2(zl0[0], zl0[1]), cvt2(zl0[2], zl0[3]), cvt2(zl1[0], zl1[1]), cvt2(zl1[2], zl1[3]));
-                    f32x4 U = mfma(kh, Vop, zero4);
-                    U = mfma(kl, Vop, U);
-                    const float4 de = *reinterpret_cast<const float4*>(&O.dec[j0[m]]);
-                    const float4 d2 = *reinterpret_cast<const float4*>(&O.d2[j0[m]]);
-                    D[m][0] = fmaf(D[m][0], de.x, d2.x * U[0]); D[m][1] = fmaf(D[m][1], de.y, d2.y * U[1]);
-                    D[m][2] = fmaf(D[m][2], de.z, d2.z * U[2]); D[m][3] = fmaf(D[m][3], de.w, d2.w * U[3]);
-                }
+                if (g == 0) S.Yx[i & 1][jh][t][i_own] = y;
             }
         }
         __syncthreads();
         exact_prev = exact;
     }
-    if (!exact_prev) finish(nchunks - 1);
+    __syncthreads();
+    finish(nchunks - 1, exact_prev);
 }
 
 template <int WMODE>
@@ -415,9 +429,9 @@ __global__ __launch_bounds__(NTF) void wkv6_fwd_ws(const ArgsC a) {
     const size_t bh = static_cast<size_t>(b) * a.H + h;
     const int nchunks = (a.T + L - 1) / L;
     // positions of A that no tile ever writes (t < 16 <= s) must read as zero
-    for (int i = tid; i < L * OS; i += NTF) { (&S.AmH[0][0])[i] = 0; (&S.AmL[0][0])[i] = 0; }
+    for (int i = tid; i < 2 * L * OS; i += NTF) { (&S.AmH[0][0][0])[i] = 0; (&S.AmL[0][0][0])[i] = 0; }
     if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
-    if (tid < NPREP * 64) fwd_prep<WMODE>(S, a, tid, base, h, nchunks);
+    if (__builtin_amdgcn_readfirstlane(tid >> 6) < NPREP) fwd_prep<WMODE>(S, a, tid, base, h, nchunks);
     else fwd_state<WMODE>(S, a, tid, base, bh, nchunks);
 }
 
