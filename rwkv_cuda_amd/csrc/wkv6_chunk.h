@@ -28,6 +28,14 @@ struct ArgsC {
     uint16_t* y;
 };
 
+struct ArgsB {
+    int T, C, H;
+    const uint16_t *r, *k, *v, *u, *s0, *gy;
+    const void* w;
+    uint16_t *gr, *gk, *gv, *gw, *gu, *gs;
+    float* rdr;                   // workspace [B,T,C] fp32
+};
+
 // Operand format.  An fp32 value x is used as hi = bf16(x), lo = bf16(x - hi).  Along the K axis of an MFMA a lane holds
 // 8 slots = 4 consecutive elements e0..e3 as  P = [h0 h1 h2 h3 | l0 l1 l2 l3]  (dwords H01, H23, L01, L23).  With the
 // halves exchanged, P~ = [l0 l1 l2 l3 | h0 h1 h2 h3] (a register renaming, no instruction), and Q in the same format,

@@ -33,14 +33,6 @@ namespace {
 // ======================================================================================================================
 constexpr int PS = 36;            // row stride (dwords) of plain bf16 [token][channel] arrays: 144 B
 
-struct ArgsB {
-    int T, C, H;
-    const uint16_t *r, *k, *v, *u, *s0, *gy;
-    const void* w;
-    uint16_t *gr, *gk, *gv, *gw, *gu, *gs;
-    float* rdr;                   // workspace [B,T,C] fp32
-};
-
 struct alignas(16) SmemA {
     uint32_t KpT[N][TS];           // k e^{c_m - c_{s+1}}  hi/lo cells along tokens [j][s]   (exact path: decay as float [t][j])
     uint32_t Bm[L][TS];            // gy_t . v_s (s < t)   hi/lo cells along s      [t][s]
@@ -795,18 +787,6 @@ int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
     a.gr = gr; a.gu = gu; a.rdr = rdr;
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_bwd_a_chunk<W_RAW>, dim3(B * H), dim3(NT), 0, st, a);
     else hipLaunchKernelGGL(wkv6_bwd_a_chunk<W_EW>, dim3(B * H), dim3(NT), 0, st, a);
-    return launch_status();
-}
-
-int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
-                            const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
-                            const uint16_t* s0, const uint16_t* gy, uint16_t* gk, uint16_t* gv, uint16_t* gw,
-                            uint16_t* gs, const float* rdr) {
-    ArgsB a{};
-    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.gy = gy;
-    a.gk = gk; a.gv = gv; a.gw = gw; a.gs = gs; a.rdr = const_cast<float*>(rdr);
-    if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_bwd_b_chunk<W_RAW>, dim3(B * H), dim3(NT), 0, st, a);
-    else hipLaunchKernelGGL(wkv6_bwd_b_chunk<W_EW>, dim3(B * H), dim3(NT), 0, st, a);
     return launch_status();
 }
 
