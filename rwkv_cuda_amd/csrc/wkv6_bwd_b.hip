@@ -47,6 +47,7 @@ struct alignas(16) SmemB2 {
     SetB set[2];
     uint32_t AmH[L][OS], AmL[L][OS];   // A[tau][s]  as [s][position of tau], hi and lo
     uint32_t BmH[L][OS], BmL[L][OS];   // Bm[tau][s] (s < tau) likewise
+    uint4 sel[4][64];                  // selection operands per lane: tile parity 0, 1; own slice of an even, odd wave
     float vgy[L];                      // gy_s . v_s
     float u[N];
     float pc[N];                       // P per channel, when it changes layout around an exact chunk
@@ -84,6 +85,10 @@ DEVINL bf16x8 op4(const uint4& x) { return __builtin_bit_cast(bf16x8, x); }
 // two accumulator tiles (tokens 0..15 and 16..31 down the rows) -> one operand with the tokens along the K slots
 DEVINL bf16x8 pack_tokens(const f32x4& z0, const f32x4& z1) {
     return as_op(cvt2(z0[0], z0[1]), cvt2(z0[2], z0[3]), cvt2(z1[0], z1[1]), cvt2(z1[2], z1[3]));
+}
+// 8-byte store at a wave-uniform base plus a 32-bit per-lane byte offset (keeps the address out of the vector registers)
+DEVINL void store8(const void* sbase, uint32_t byte_off, const uint2& x) {
+    asm volatile("global_store_dwordx2 %0, %1, %2" : : "v"(byte_off), "v"(x), "s"(sbase) : "memory");
 }
 DEVINL void unpack4(const uint2& x, float (&f)[4]) { f[0] = bf_lo(x.x); f[1] = bf_hi(x.x); f[2] = bf_lo(x.y); f[3] = bf_hi(x.y); }
 
@@ -358,9 +363,6 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
     f32x4 D[4];
 #pragma unroll
     for (int m = 0; m < 4; ++m) D[m] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const bf16x8 selOwn = op4(one_hot(g == 2 * (q & 1) + (l16 >> 3), l16 & 7));   // column n <-> channel 16q + n of the half q>>1
-    const bf16x8 selT0 = op4(one_hot(g == (l16 >> 2), l16 & 3));                  // column r <-> channel 8 (r>>2) + (r&3) of a half
-    const bf16x8 selT1 = op4(one_hot(g == (l16 >> 2), 4 + (l16 & 3)));            //              ...     8 (r>>2) + 4 + (r&3)
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     float Pend[4] = {0.f, 0.f, 0.f, 0.f};              // P at the end of the current chunk for channels j4 + v (same in all 16 lanes of a row)
 
@@ -390,6 +392,7 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
             __builtin_amdgcn_sched_barrier(0);
             // ------------------------------------------------------------ R'^T of the own key channels
             {
+                const bf16x8 selOwn = op4(S.sel[2 + (q & 1)][lane]);
                 const f32x4 zh0 = mfma(lds_op(&O.RpH[l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
                 const f32x4 zh1 = mfma(lds_op(&O.RpH[16 + l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
                 const f32x4 zl0 = mfma(lds_op(&O.RpL[l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
@@ -404,7 +407,7 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 const bf16x8 a0 = lds_op(&O.GY[l16][16 * mh + 4 * g]), a1 = lds_op(&O.GY[16 + l16][16 * mh + 4 * g]);
 #pragma unroll
                 for (int par = 0; par < 2; ++par) {
-                    const bf16x8 sel = par ? selT1 : selT0;
+                    const bf16x8 sel = op4(S.sel[par][lane]);
                     const bf16x8 gt = pack_tokens(mfma(a0, sel, zero4), mfma(a1, sel, zero4));   // lane = value-channel row, slots = tokens
                     f32x4 U = mfma(gt, rtH, zero4);
                     U = mfma(gt, rtL, U);
@@ -463,6 +466,8 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 u4[0] = z.x; u4[1] = z.y; u4[2] = z.z; u4[3] = z.w;
             }
             float tot1[4] = {0.f, 0.f, 0.f, 0.f};
+            uint2 out_k[2], out_w[2];                   // stored after both tiles: a store in between would make every later
+                                                        // register reload from scratch wait for its acknowledgement
 #pragma unroll
             for (int st = 1; st >= 0; --st) {           // later tokens first: their total enters the earlier tile's suffix
                 const int s = 16 * st + l16, tg = c0 + s;
@@ -492,12 +497,18 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                     gw[v] = (!stateful && tg == 0) ? 0.f : lm[v] * Gt;
                     if (st == 1) tot1[v] = tot; else Pend[v] += tot + tot1[v];
                 }
-                if (tg < T) {
-                    const size_t off = base + static_cast<size_t>(tg) * C + j4;
-                    *reinterpret_cast<uint2*>(a.gk + off) = make_uint2(pack_bf2(gk[0], gk[1]), pack_bf2(gk[2], gk[3]));
-                    *reinterpret_cast<uint2*>(a.gw + off) = make_uint2(pack_bf2(gw[0], gw[1]), pack_bf2(gw[2], gw[3]));
-                }
+                out_k[st] = make_uint2(pack_bf2(gk[0], gk[1]), pack_bf2(gk[2], gk[3]));
+                out_w[st] = make_uint2(pack_bf2(gw[0], gw[1]), pack_bf2(gw[2], gw[3]));
                 __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                const int tg = c0 + 16 * st + l16;
+                if (tg < T) {
+                    const uint32_t off = (static_cast<uint32_t>(tg) * C + j4) * 2;
+                    store8(a.gk + base, off, out_k[st]);
+                    store8(a.gw + base, off, out_w[st]);
+                }
             }
         }
         __syncthreads();
@@ -525,9 +536,6 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
     f32x4 E[4];
 #pragma unroll
     for (int m = 0; m < 4; ++m) E[m] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const bf16x8 selOwn = op4(one_hot(g == 2 * (q & 1) + (l16 >> 3), l16 & 7));
-    const bf16x8 selT0 = op4(one_hot(g == (l16 >> 2), l16 & 3));
-    const bf16x8 selT1 = op4(one_hot(g == (l16 >> 2), 4 + (l16 & 3)));
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
 
     __syncthreads();
@@ -556,8 +564,11 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
-            gto = pack_tokens(mfma(lds_op(&O.GY[l16][16 * (q >> 1) + 4 * g]), selOwn, zero4),
-                              mfma(lds_op(&O.GY[16 + l16][16 * (q >> 1) + 4 * g]), selOwn, zero4));
+            {
+                const bf16x8 selOwn = op4(S.sel[2 + (q & 1)][lane]);
+                gto = pack_tokens(mfma(lds_op(&O.GY[l16][16 * (q >> 1) + 4 * g]), selOwn, zero4),
+                                  mfma(lds_op(&O.GY[16 + l16][16 * (q >> 1) + 4 * g]), selOwn, zero4));
+            }
             // ------------------------------------------------------------ dS^T = diag(dec) dS^T + diag(d1) R'^T GY
 #pragma unroll
             for (int mh = 0; mh < 2; ++mh) {
@@ -565,7 +576,7 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 const bf16x8 al0 = lds_op(&O.RpL[l16][16 * mh + 4 * g]), al1 = lds_op(&O.RpL[16 + l16][16 * mh + 4 * g]);
 #pragma unroll
                 for (int par = 0; par < 2; ++par) {
-                    const bf16x8 sel = par ? selT1 : selT0;
+                    const bf16x8 sel = op4(S.sel[par][lane]);
                     const bf16x8 rh = pack_tokens(mfma(ah0, sel, zero4), mfma(ah1, sel, zero4));
                     const bf16x8 rl = pack_tokens(mfma(al0, sel, zero4), mfma(al1, sel, zero4));
                     f32x4 U = mfma(rh, gto, zero4);
@@ -617,9 +628,7 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 const int s = 16 * st + l16, tg = c0 + s;
                 f32x4 y = mfma(gto, lds_op(&S.AmH[s][4 * g]), dvin[st]);
                 y = mfma(gto, lds_op(&S.AmL[s][4 * g]), y);
-                if (tg < T)
-                    *reinterpret_cast<uint2*>(a.gv + base + static_cast<size_t>(tg) * C + i4) =
-                        make_uint2(pack_bf2(y[0], y[1]), pack_bf2(y[2], y[3]));
+                if (tg < T) store8(a.gv + base, (static_cast<uint32_t>(tg) * C + i4) * 2, make_uint2(pack_bf2(y[0], y[1]), pack_bf2(y[2], y[3])));
             }
         }
         __syncthreads();
@@ -637,6 +646,13 @@ __global__ __launch_bounds__(NTB) void wkv6_bwd_b_ws(const ArgsB a) {
     // positions of the tiles that are never written (s >= 16 > tau) must read as zero
     for (int i = tid; i < 4 * L * OS; i += NTB) (&S.AmH[0][0])[i] = 0;
     if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
+    if (tid < 256) {
+        // One-hot B operands of the transposing products, per lane (column n = l16, K-slot group g).
+        //   0, 1: column r <-> channel 8 (r>>2) + 4 p + (r&3) of a 32-channel half (rows of state tile parity p)
+        //   2, 3: column n <-> channel 16 (q&1) + n of the half q>>1 (the 16 channels a wave owns)
+        const int k = tid >> 6, ln = tid & 63, c16 = ln & 15, gg = ln >> 4;
+        S.sel[k][ln] = (k < 2) ? one_hot(gg == (c16 >> 2), 4 * k + (c16 & 3)) : one_hot(gg == 2 * (k & 1) + (c16 >> 3), c16 & 7);
+    }
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
     if (wid < NPREP) bwd_prep<WMODE>(S, a, tid, base, h, nchunks);
     else if (wid < NPREP + 4) bwd_state_d<WMODE>(S, a, tid, base, bh, nchunks);
