@@ -27,6 +27,7 @@ constexpr int NPREP = 8;
 constexpr int NTB = 1024;
 constexpr int OS = 40;            // row stride (dwords) of a bf16 [token][channel] plane: 160 B, conflict-free for 16-byte reads
 constexpr int FS = 72;            // row stride (dwords) of an fp32 [token][channel] array
+constexpr int AS = 24;            // row stride (dwords) of a tile plane [s][32 positions of tau]
 constexpr float LN2 = 0.69314718055994530942f;
 constexpr int STB = 3;            // visits of input kept in flight
 
@@ -45,9 +46,11 @@ struct alignas(16) SetB {
 
 struct alignas(16) SmemB2 {
     SetB set[2];
-    uint32_t AmH[L][OS], AmL[L][OS];   // A[tau][s]  as [s][position of tau], hi and lo
-    uint32_t BmH[L][OS], BmL[L][OS];   // Bm[tau][s] (s < tau) likewise
-    uint4 sel[4][64];                  // selection operands per lane: tile parity 0, 1; own slice of an even, odd wave
+    uint32_t AmH[L][AS], AmL[L][AS];   // A[tau][s]  as [s][position of tau], hi and lo
+    uint32_t BmH[L][AS], BmL[L][AS];   // Bm[tau][s] (s < tau) likewise
+    uint4 sel[2][64];                  // selection operands per lane, tile parity 0 and 1
+    uint4 TR[4][2][64];                // R'^T tile m (hi, lo): lane = row r of the tile, K slots = tokens; written by D wave m
+    uint4 TG[4][64];                   // gy^T tile m likewise; written by E wave m
     float vgy[L];                      // gy_s . v_s
     float u[N];
     float pc[N];                       // P per channel, when it changes layout around an exact chunk
@@ -316,8 +319,8 @@ DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base
         const HL x0 = hilo2(acc[0], acc[1]), x1 = hilo2(acc[2], acc[3]);
         uint32_t* H = wid < 3 ? &S.AmH[0][0] : &S.BmH[0][0];
         uint32_t* Lo = wid < 3 ? &S.AmL[0][0] : &S.BmL[0][0];
-        *reinterpret_cast<uint2*>(&H[(16 * tb + l16) * OS + 4 * g + 2 * ta]) = make_uint2(x0.h, x1.h);
-        *reinterpret_cast<uint2*>(&Lo[(16 * tb + l16) * OS + 4 * g + 2 * ta]) = make_uint2(x0.l, x1.l);
+        *reinterpret_cast<uint2*>(&H[(16 * tb + l16) * AS + 4 * g + 2 * ta]) = make_uint2(x0.h, x1.h);
+        *reinterpret_cast<uint2*>(&Lo[(16 * tb + l16) * AS + 4 * g + 2 * ta]) = make_uint2(x0.l, x1.l);
     };
 
     static_for<STB>([&](auto Z) { arrived(ring[decltype(Z)::value], std::integral_constant<int, 0>{}); });
@@ -354,8 +357,9 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
     const int lane = tid & 63, q = (__builtin_amdgcn_readfirstlane(tid >> 6) - NPREP) & 3, l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
     const bool stateful = a.s0 != nullptr;
-    const int j_own = 16 * q + l16;                    // state column / operand row of this lane
-    const int j4 = 16 * q + 4 * g;                     // output rows of this lane: key channels j4 .. j4+3
+    // this wave owns the key channels of state tile q:  column / operand row r = l16  <->  j_own
+    const int j_own = 32 * (q >> 1) + 8 * (l16 >> 2) + 4 * (q & 1) + (l16 & 3);
+    const int j4 = 32 * (q >> 1) + 8 * g + 4 * (q & 1);      // output rows 4g + v of this lane: key channels j4 .. j4+3
     int i0[4];                                         // first value channel of this lane's four rows in state tile m
 #pragma unroll
     for (int m = 0; m < 4; ++m) i0[m] = 32 * (m >> 1) + 8 * g + 4 * (m & 1);
@@ -392,30 +396,14 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
             __builtin_amdgcn_sched_barrier(0);
             // ------------------------------------------------------------ R'^T of the own key channels
             {
-                const bf16x8 selOwn = op4(S.sel[2 + (q & 1)][lane]);
+                const bf16x8 selOwn = op4(S.sel[q & 1][lane]);
                 const f32x4 zh0 = mfma(lds_op(&O.RpH[l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
                 const f32x4 zh1 = mfma(lds_op(&O.RpH[16 + l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
                 const f32x4 zl0 = mfma(lds_op(&O.RpL[l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
                 const f32x4 zl1 = mfma(lds_op(&O.RpL[16 + l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
                 rtH = pack_tokens(zh0, zh1); rtL = pack_tokens(zl0, zl1);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            // ------------------------------------------------------------ dS = dS diag(dec) + diag(d1) GY^T R'
-            const float decj = O.dec[j_own], d1j = O.d1[j_own];
-#pragma unroll
-            for (int mh = 0; mh < 2; ++mh) {
-                const bf16x8 a0 = lds_op(&O.GY[l16][16 * mh + 4 * g]), a1 = lds_op(&O.GY[16 + l16][16 * mh + 4 * g]);
-#pragma unroll
-                for (int par = 0; par < 2; ++par) {
-                    const bf16x8 sel = op4(S.sel[par][lane]);
-                    const bf16x8 gt = pack_tokens(mfma(a0, sel, zero4), mfma(a1, sel, zero4));   // lane = value-channel row, slots = tokens
-                    f32x4 U = mfma(gt, rtH, zero4);
-                    U = mfma(gt, rtL, U);
-                    const int m = 2 * mh + par;
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) D[m][v] = fmaf(D[m][v], decj, d1j * U[v]);
-                }
-                __builtin_amdgcn_sched_barrier(0);
+                S.TR[q][0][lane] = __builtin_bit_cast(uint4, rtH);          // the E waves use it as a row operand of their update
+                S.TR[q][1][lane] = __builtin_bit_cast(uint4, rtL);
             }
         } else {
             // ------------------------------------------------------------ exact path: 32 sequential steps, time descending
@@ -472,9 +460,10 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
             for (int st = 1; st >= 0; --st) {           // later tokens first: their total enters the earlier tile's suffix
                 const int s = 16 * st + l16, tg = c0 + s;
                 // ---------------------------------------------------- sum_{tau > s} Bm[tau][s] R'_tau[j]
-                f32x4 dq = mfma(rtH, lds_op(&S.BmH[s][4 * g]), zero4);
+                const bf16x8 bh_ = lds_op(&S.BmH[s][4 * g]);
+                f32x4 dq = mfma(rtH, bh_, zero4);
                 dq = mfma(rtH, lds_op(&S.BmL[s][4 * g]), dq);
-                dq = mfma(rtL, lds_op(&S.BmH[s][4 * g]), dq);
+                dq = mfma(rtL, bh_, dq);
                 const float4 eb4 = *reinterpret_cast<const float4*>(&O.Eb[s][j4]);
                 const float4 lm4 = *reinterpret_cast<const float4*>(&O.lam[s][j4]);
                 const float4 rd4 = *reinterpret_cast<const float4*>(&O.rdr[s][j4]);
@@ -510,6 +499,17 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                     store8(a.gw + base, off, out_w[st]);
                 }
             }
+            __builtin_amdgcn_sched_barrier(0);
+            // ------------------------------------------------------------ dS = dS diag(dec) + diag(d1) GY^T R'
+            const float decj = O.dec[j_own], d1j = O.d1[j_own];
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const bf16x8 gt = op4(S.TG[m][lane]);   // gy^T of state tile m: lane = value-channel row, slots = tokens
+                f32x4 U = mfma(gt, rtH, zero4);
+                U = mfma(gt, rtL, U);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) D[m][v] = fmaf(D[m][v], decj, d1j * U[v]);
+            }
         }
         __syncthreads();
     }
@@ -527,8 +527,9 @@ template <int WMODE>
 DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t base, const int nchunks) {
     const int lane = tid & 63, q = (__builtin_amdgcn_readfirstlane(tid >> 6) - NPREP) & 3, l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
-    const int i_own = 16 * q + l16;                    // state column / operand row of this lane
-    const int i4 = 16 * q + 4 * g;                     // output rows: value channels i4 .. i4+3
+    // this wave owns the value channels of state tile q:  column / operand row r = l16  <->  i_own
+    const int i_own = 32 * (q >> 1) + 8 * (l16 >> 2) + 4 * (q & 1) + (l16 & 3);
+    const int i4 = 32 * (q >> 1) + 8 * g + 4 * (q & 1);      // output rows 4g + v: value channels i4 .. i4+3
     int j0[4];                                         // first key channel of this lane's four rows in state tile m
 #pragma unroll
     for (int m = 0; m < 4; ++m) j0[m] = 32 * (m >> 1) + 8 * g + 4 * (m & 1);
@@ -565,29 +566,10 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
             }
             __builtin_amdgcn_sched_barrier(0);
             {
-                const bf16x8 selOwn = op4(S.sel[2 + (q & 1)][lane]);
+                const bf16x8 selOwn = op4(S.sel[q & 1][lane]);
                 gto = pack_tokens(mfma(lds_op(&O.GY[l16][16 * (q >> 1) + 4 * g]), selOwn, zero4),
                                   mfma(lds_op(&O.GY[16 + l16][16 * (q >> 1) + 4 * g]), selOwn, zero4));
-            }
-            // ------------------------------------------------------------ dS^T = diag(dec) dS^T + diag(d1) R'^T GY
-#pragma unroll
-            for (int mh = 0; mh < 2; ++mh) {
-                const bf16x8 ah0 = lds_op(&O.RpH[l16][16 * mh + 4 * g]), ah1 = lds_op(&O.RpH[16 + l16][16 * mh + 4 * g]);
-                const bf16x8 al0 = lds_op(&O.RpL[l16][16 * mh + 4 * g]), al1 = lds_op(&O.RpL[16 + l16][16 * mh + 4 * g]);
-#pragma unroll
-                for (int par = 0; par < 2; ++par) {
-                    const bf16x8 sel = op4(S.sel[par][lane]);
-                    const bf16x8 rh = pack_tokens(mfma(ah0, sel, zero4), mfma(ah1, sel, zero4));
-                    const bf16x8 rl = pack_tokens(mfma(al0, sel, zero4), mfma(al1, sel, zero4));
-                    f32x4 U = mfma(rh, gto, zero4);
-                    U = mfma(rl, gto, U);
-                    const int m = 2 * mh + par;
-                    const float4 de = *reinterpret_cast<const float4*>(&O.dec[j0[m]]);
-                    const float4 d1 = *reinterpret_cast<const float4*>(&O.d1[j0[m]]);
-                    E[m][0] = fmaf(E[m][0], de.x, d1.x * U[0]); E[m][1] = fmaf(E[m][1], de.y, d1.y * U[1]);
-                    E[m][2] = fmaf(E[m][2], de.z, d1.z * U[2]); E[m][3] = fmaf(E[m][3], de.w, d1.w * U[3]);
-                }
-                __builtin_amdgcn_sched_barrier(0);
+                S.TG[q][lane] = __builtin_bit_cast(uint4, gto);             // the D waves use it as a row operand of their update
             }
         } else {
             // ------------------------------------------------------------ exact path: 32 sequential steps, time descending
@@ -630,6 +612,17 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 y = mfma(gto, lds_op(&S.AmL[s][4 * g]), y);
                 if (tg < T) store8(a.gv + base, (static_cast<uint32_t>(tg) * C + i4) * 2, make_uint2(pack_bf2(y[0], y[1]), pack_bf2(y[2], y[3])));
             }
+            __builtin_amdgcn_sched_barrier(0);
+            // ------------------------------------------------------------ dS^T = diag(dec) dS^T + diag(d1) R'^T GY
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                f32x4 U = mfma(op4(S.TR[m][0][lane]), gto, zero4);   // R'^T of state tile m: lane = key-channel row, slots = tokens
+                U = mfma(op4(S.TR[m][1][lane]), gto, U);
+                const float4 de = *reinterpret_cast<const float4*>(&O.dec[j0[m]]);
+                const float4 d1 = *reinterpret_cast<const float4*>(&O.d1[j0[m]]);
+                E[m][0] = fmaf(E[m][0], de.x, d1.x * U[0]); E[m][1] = fmaf(E[m][1], de.y, d1.y * U[1]);
+                E[m][2] = fmaf(E[m][2], de.z, d1.z * U[2]); E[m][3] = fmaf(E[m][3], de.w, d1.w * U[3]);
+            }
         }
         __syncthreads();
     }
@@ -644,14 +637,13 @@ __global__ __launch_bounds__(NTB) void wkv6_bwd_b_ws(const ArgsB a) {
     const size_t bh = static_cast<size_t>(b) * a.H + h;
     const int nchunks = (a.T + L - 1) / L;
     // positions of the tiles that are never written (s >= 16 > tau) must read as zero
-    for (int i = tid; i < 4 * L * OS; i += NTB) (&S.AmH[0][0])[i] = 0;
+    for (int i = tid; i < 4 * L * AS; i += NTB) (&S.AmH[0][0])[i] = 0;
     if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
-    if (tid < 256) {
-        // One-hot B operands of the transposing products, per lane (column n = l16, K-slot group g).
-        //   0, 1: column r <-> channel 8 (r>>2) + 4 p + (r&3) of a 32-channel half (rows of state tile parity p)
-        //   2, 3: column n <-> channel 16 (q&1) + n of the half q>>1 (the 16 channels a wave owns)
-        const int k = tid >> 6, ln = tid & 63, c16 = ln & 15, gg = ln >> 4;
-        S.sel[k][ln] = (k < 2) ? one_hot(gg == (c16 >> 2), 4 * k + (c16 & 3)) : one_hot(gg == 2 * (k & 1) + (c16 >> 3), c16 & 7);
+    if (tid < 128) {
+        // One-hot B operand of the transposing products, per lane (column r = l16, K-slot group g), for tile parity p:
+        // column r <-> channel 8 (r>>2) + 4 p + (r&3) of a 32-channel half.
+        const int p = tid >> 6, ln = tid & 63, c16 = ln & 15, gg = ln >> 4;
+        S.sel[p][ln] = one_hot(gg == (c16 >> 2), 4 * p + (c16 & 3));
     }
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
     if (wid < NPREP) bwd_prep<WMODE>(S, a, tid, base, h, nchunks);
