@@ -15,7 +15,7 @@ _CSRC = os.path.join(_HERE, "csrc")
 _INCLUDE = os.path.join(_ROOT, "include")
 LIB_PATH = os.path.join(_HERE, "librwkv_hip.so")
 
-SOURCES = ["abi.hip", "wkv56.hip", "wkv6_chunk.hip", "wkv6_fwd.hip", "wkv6_bwd_b.hip", "wkv4.hip", "timex.hip", "rwkv7.hip"]
+SOURCES = ["abi.hip", "wkv56.hip", "wkv6_fwd.hip", "wkv6_bwd_a.hip", "wkv6_bwd_b.hip", "wkv4.hip", "timex.hip", "rwkv7.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

@@ -1,0 +1,445 @@
+// wkv6 / wkv6_state backward, first sweep (time ascending): gr, gu and the workspace r * dr' that the decay gradient needs.
+// Wave-specialised workgroup (gfx950); formulas and symbols as in wkv6_chunk.h, S the state at the START of a chunk:
+//     dr'_t[j] = Ea_t[j] ( d1[j] (GY S)[t][j] + sum_{s<t} Bm[t][s] K'_s[j] ),    Bm[t][s] = gy_t . v_s,   Ea_t = e^{c_t - c_m}
+//     gr = dr' + u k_t (gy_t . v_t),     gu[j] = sum_t r_t[j] k_t[j] (gy_t . v_t),     S_L = S diag(dec) + diag(d2) V^T K'
+// One workgroup of 16 waves per (batch, head):
+//   waves 0..7  ("prep")   load r, k, v, w, gy ahead of time, take the decay sums, write K' (hi / lo bf16 planes), r, k, v, gy and
+//                          Ea into LDS in natural [token][channel] layout; waves 0..2 form the causal tile Bm.
+//   waves 8..15 ("state")  wave (q, ih) keeps S[i][j] for the key channels of state tile q and the value-channel half ih
+//                          (lane = j, registers = 32 values of i).  dr' comes out with a lane per TOKEN and four consecutive key
+//                          channels per lane; the two waves of a q exchange one partial tile and each finishes 16 tokens:
+//                          gr and r dr' are stored from registers.
+// K-slot conventions, selection-matrix transposes and tile storage are those of the forward kernel (wkv6_fwd.hip).
+// Two barriers per chunk:  [tile(i) | first half of operands(i+1) | GY S, K'^T, V^T, state update]  B
+//                          [scan(i+2), second half of operands(i+1) | Bm K', epilogue, stores]  B.
+#include "wkv6_chunk.h"
+
+namespace rwkv {
+namespace {
+
+constexpr int NPREP = 8;
+constexpr int NSTATE = 8;
+constexpr int NTA = (NPREP + NSTATE) * 64;
+constexpr int STA = 3;            // chunks of input kept in flight
+
+struct alignas(16) SetA {
+    uint32_t KpH[L][OS], KpL[L][OS];   // k e^{c_m - c_{s+1}}  hi, lo
+    uint32_t Rr[L][OS], Kr[L][OS];     // r, k
+    uint32_t V[L][OS], GY[L][OS];      // v, gy
+    float Ea[L][FS];                   // e^{c_t - c_m}                 (exact path: decay of each step)
+    float d1[N], d2[N], dec[N];        // e^{c_m}, e^{c_L - c_m}, e^{c_L}
+    uint32_t exact, pad[3];
+};
+
+struct alignas(16) SmemA2 {
+    SetA set[2];
+    uint32_t BmH[L][AS], BmL[L][AS];   // Bm[t][s] (s < t) as [t][position of s], hi and lo
+    uint4 sel[2][64];                  // selection operands per lane, tile parity 0 and 1
+    float4 Xch[NSTATE][64];            // partial (GY S)^T tile handed to the partner wave
+    float Yx[2][L][N];                 // exact path: partial dr' of the two value-channel halves;  at the end: gu partial sums
+    float Vx[2][L];                    // exact path: partial gy . v
+    float vgy[L];                      // gy_t . v_t
+    float gfast[2][N];                 // gu of the chunked path, two token halves
+    float u[N];
+    float part[2][NPREP][N];
+    uint32_t flag[2][NPREP];
+};
+
+// ---------------------------------------------------------------------------------------------------- prep waves
+template <int WMODE>
+DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base, const int nchunks) {
+    const int lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, g = lane >> 4;
+    const int T = a.T, C = a.C;
+    const uint16_t* __restrict__ rb = a.r + base;
+    const uint16_t* __restrict__ kb = a.k + base;
+    const uint16_t* __restrict__ vb = a.v + base;
+    const uint16_t* __restrict__ gb = a.gy + base;
+    // channel pair (2 jp, 2 jp + 1), tokens 4 wid + 2 th + {0, 1}
+    const int jp = lane & 31, th = lane >> 5, pt0 = 4 * wid + 2 * th;
+    const bool second = wid >= 4;
+    struct Raw { uint32_t r[2], k[2], v[2], g[2], w[2][WMODE == W_RAW ? 1 : 2]; float lam[2][2], other[2], kp[2][2]; };
+    Raw ring[STA];
+    // Loads are asm so that the wait before their first use can leave the younger batches in flight; every call issues the
+    // same ten loads (chunk index clamped), which keeps the count fixed.
+    const uint32_t* __restrict__ wb32 = reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + base);
+    const float* __restrict__ wbf = static_cast<const float*>(a.w) + base;
+    auto prefetch = [&](int c, Raw& x) __attribute__((always_inline)) {
+        c = c < nchunks ? c : nchunks - 1;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int t = c * L + pt0 + e;
+            const uint32_t o = (static_cast<uint32_t>(t < T ? t : T - 1) * C + 2 * jp) * 2;    // byte offset of the channel pair
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.r[e]) : "v"(o), "s"(rb));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.k[e]) : "v"(o), "s"(kb));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.v[e]) : "v"(o), "s"(vb));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.g[e]) : "v"(o), "s"(gb));
+            if constexpr (WMODE == W_RAW) {
+                asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.w[e][0]) : "v"(o), "s"(wb32));
+            } else {
+                uint2 y;
+                asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(y) : "v"(2 * o), "s"(wbf));
+                x.w[e][0] = y.x; x.w[e][1] = y.y;
+            }
+        }
+    };
+    auto arrived = [&](Raw& x, auto younger) __attribute__((always_inline)) {
+        if constexpr (WMODE == W_RAW)
+            asm volatile("s_waitcnt vmcnt(%10)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[1][0]) : "n"(decltype(younger)::value));
+        else
+            asm volatile("s_waitcnt vmcnt(%12)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[0][1]), "+v"(x.w[1][0]), "+v"(x.w[1][1])
+                         : "n"(decltype(younger)::value));
+    };
+    static_for<STA>([&](auto Z) { prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
+
+    // ---- scan of chunk c: lam (log2 units) of this thread's four elements, sums over each eighth of the chunk
+    auto scan = [&](const int c, Raw& x) __attribute__((always_inline)) {
+        const int c0 = c * L, pb = c & 1;
+        if (c0 + L > T) {                              // last, partial chunk: rows past T carry no input and no decay
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+                if (c0 + pt0 + e >= T) {
+                    x.r[e] = 0; x.k[e] = 0; x.v[e] = 0; x.g[e] = 0;
+                    if constexpr (WMODE == W_RAW) x.w[e][0] = 0xff80ff80u;   // w = -inf  ->  lam = -exp(w) = 0
+                    else { x.w[e][0] = 0u; x.w[e][1] = 0u; }
+                }
+        }
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+#pragma unroll
+            for (int z = 0; z < 2; ++z) {
+                if constexpr (WMODE == W_RAW) x.lam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e][0]) : bf_lo(x.w[e][0])));
+                else x.lam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+            }
+        float s2[2];
+#pragma unroll
+        for (int z = 0; z < 2; ++z) {
+            s2[z] = x.lam[0][z] + x.lam[1][z];
+            x.other[z] = __shfl_xor(s2[z], 32, 64);    // the other two tokens of this wave's four
+        }
+        const float s4a = s2[0] + x.other[0], s4b = s2[1] + x.other[1];
+        if (th == 0) *reinterpret_cast<float2*>(&S.part[pb][wid][2 * jp]) = make_float2(s4a, s4b);
+        // A chunk whose decays could overflow the mid-point factors is redone exactly (see wkv6_chunk.h).
+        const bool fast_decay = (-s4a > 0.25f * RANGE_LIMIT * LOG2E) || (-s4b > 0.25f * RANGE_LIMIT * LOG2E);
+        const unsigned long long any = __ballot(fast_decay);
+        if (lane == 0) S.flag[pb][wid] = any != 0ull;
+    };
+
+    // ---- operands of chunk c into set c & 1, first part: Ea, plain r (K' values stay in registers)
+    auto operands_a = [&](const int c, Raw& x) __attribute__((always_inline)) -> bool {
+        SetA& O = S.set[c & 1];
+        const int pb = c & 1;
+        const uint4 f0 = *reinterpret_cast<const uint4*>(&S.flag[pb][0]), f1 = *reinterpret_cast<const uint4*>(&S.flag[pb][4]);
+        float2 pe[4];
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4) pe[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * second + w4][2 * jp]);
+        const bool exact = (f0.x | f0.y | f0.z | f0.w | f1.x | f1.y | f1.z | f1.w) != 0;
+        if (tid == 0) O.exact = exact;
+        float near[2];
+        near[0] = second ? (th ? x.other[0] : 0.f) : (th ? 0.f : x.other[0]);
+        near[1] = second ? (th ? x.other[1] : 0.f) : (th ? 0.f : x.other[1]);
+        const int w_own = wid & 3;
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4) {
+            const bool between = second ? (w4 < w_own) : (w4 > w_own);      // wave-uniform
+            near[0] += between ? pe[w4].x : 0.f;
+            near[1] += between ? pe[w4].y : 0.f;
+        }
+        if (!exact) {
+            float ea[2][2];
+#pragma unroll
+            for (int z = 0; z < 2; ++z) {
+                const Scale sc = chunk_scale(second, near[z], x.lam[0][z], x.lam[1][z]);
+                ea[0][z] = sc.ea[0]; ea[1][z] = sc.ea[1];
+                x.kp[0][z] = (z ? bf_hi(x.k[0]) : bf_lo(x.k[0])) * sc.eb[0];
+                x.kp[1][z] = (z ? bf_hi(x.k[1]) : bf_lo(x.k[1])) * sc.eb[1];
+            }
+#pragma unroll
+            for (int e = 0; e < 2; ++e) *reinterpret_cast<float2*>(&O.Ea[pt0 + e][2 * jp]) = make_float2(ea[e][0], ea[e][1]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+                *reinterpret_cast<float2*>(&O.Ea[pt0 + e][2 * jp]) = make_float2(exp2_fast(x.lam[e][0]), exp2_fast(x.lam[e][1]));
+        }
+        O.Rr[pt0][jp] = x.r[0];
+        O.Rr[pt0 + 1][jp] = x.r[1];
+        return exact;
+    };
+    // ---- second part: K' planes, k, v, gy; wave 3 adds the per-channel factors of the chunk
+    auto operands_b = [&](const int c, Raw& x, const bool exact) __attribute__((always_inline)) {
+        SetA& O = S.set[c & 1];
+        const int pb = c & 1;
+        if (!exact) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const HL y = hilo2(x.kp[e][0], x.kp[e][1]);
+                O.KpH[pt0 + e][jp] = y.h; O.KpL[pt0 + e][jp] = y.l;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            O.Kr[pt0 + e][jp] = x.k[e];
+            O.V[pt0 + e][jp] = x.v[e];
+            O.GY[pt0 + e][jp] = x.g[e];
+        }
+        if (wid == 3 && th == 0) {
+            float cm[2] = {0.f, 0.f}, ch[2] = {0.f, 0.f};
+#pragma unroll
+            for (int w8 = 0; w8 < 4; ++w8) {
+                const float2 y0 = *reinterpret_cast<const float2*>(&S.part[pb][w8][2 * jp]);
+                const float2 y1 = *reinterpret_cast<const float2*>(&S.part[pb][4 + w8][2 * jp]);
+                cm[0] += y0.x; cm[1] += y0.y; ch[0] += y1.x; ch[1] += y1.y;
+            }
+            *reinterpret_cast<float2*>(&O.d1[2 * jp]) = make_float2(exp2_fast(cm[0]), exp2_fast(cm[1]));
+            *reinterpret_cast<float2*>(&O.d2[2 * jp]) = make_float2(exp2_fast(ch[0]), exp2_fast(ch[1]));
+            *reinterpret_cast<float2*>(&O.dec[2 * jp]) = make_float2(exp2_fast(cm[0] + ch[0]), exp2_fast(cm[1] + ch[1]));
+        }
+    };
+
+    // ---- causal tile of chunk c: waves 0..2, quadrants (t tile, s tile) = (0,0) (1,0) (1,1).  Accumulator rows are s,
+    //      lanes are t; stored as [t][position of s].  The diagonal gy_t . v_t goes to vgy.
+    auto tile = [&](const int c) __attribute__((always_inline)) {
+        const SetA& O = S.set[c & 1];
+        const int ta = (wid == 0) ? 0 : 1, tb = (wid == 2) ? 1 : 0;          // t tile, s tile
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+            acc = mfma(lds_op(&O.V[16 * tb + l16][16 * ks + 4 * g]), lds_op(&O.GY[16 * ta + l16][16 * ks + 4 * g]), acc);
+        if (ta == tb) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int sl = 4 * g + v;
+                if (sl == l16) S.vgy[16 * ta + l16] = acc[v];
+                acc[v] = (sl < l16) ? acc[v] : 0.f;
+            }
+        }
+        const HL x0 = hilo2(acc[0], acc[1]), x1 = hilo2(acc[2], acc[3]);
+        *reinterpret_cast<uint2*>(&S.BmH[16 * ta + l16][4 * g + 2 * tb]) = make_uint2(x0.h, x1.h);
+        *reinterpret_cast<uint2*>(&S.BmL[16 * ta + l16][4 * g + 2 * tb]) = make_uint2(x0.l, x1.l);
+    };
+
+    static_for<STA>([&](auto Z) { arrived(ring[decltype(Z)::value], std::integral_constant<int, 0>{}); });
+    scan(0, ring[0]);
+    if (nchunks > 1) scan(1, ring[1]);
+    __syncthreads();
+    bool exact_cur = operands_a(0, ring[0]);
+    operands_b(0, ring[0], exact_cur);
+    prefetch(STA, ring[0]);
+    __syncthreads();
+    for (int ib = 0; ib < nchunks; ib += STA)
+        static_for<STA>([&](auto Z) {
+            constexpr int z = decltype(Z)::value;
+            const int i = ib + z;
+            if (i < nchunks) {
+                if (wid < 3 && !exact_cur) tile(i);
+                bool exact_next = false;
+                if (i + 1 < nchunks) exact_next = operands_a(i + 1, ring[(z + 1) % STA]);
+                __syncthreads();
+                // younger than the loads of chunk i+2: those of chunk i+3
+                arrived(ring[(z + 2) % STA], std::integral_constant<int, 10 * (STA - 2)>{});
+                if (i + 2 < nchunks) scan(i + 2, ring[(z + 2) % STA]);
+                if (i + 1 < nchunks) operands_b(i + 1, ring[(z + 1) % STA], exact_next);
+                prefetch(i + 1 + STA, ring[(z + 1) % STA]);
+                __syncthreads();
+                exact_cur = exact_next;
+            }
+        });
+    __syncthreads();                                   // the state waves publish their gu sums
+    if (tid < N) {
+        float s = S.gfast[0][tid] + S.gfast[1][tid];
+        for (int t = 0; t < L; ++t) s += S.Yx[0][t][tid];
+        a.gu[static_cast<size_t>(blockIdx.x / a.H) * C + (blockIdx.x % a.H) * N + tid] = f2bf(s);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------- state waves
+template <int WMODE>
+DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t base, const size_t bh, const int nchunks) {
+    const int lane = tid & 63, sw = __builtin_amdgcn_readfirstlane(tid >> 6) - NPREP, q = sw & 3, ih = sw >> 2, l16 = lane & 15, g = lane >> 4;
+    const int T = a.T, C = a.C;
+    // this wave owns the key channels of state tile q:  column / operand row r = l16  <->  j_own
+    const int j_own = 32 * (q >> 1) + 8 * (l16 >> 2) + 4 * (q & 1) + (l16 & 3);
+    const int j4 = 32 * (q >> 1) + 8 * g + 4 * (q & 1);      // output rows 4g + v of this lane: key channels j4 .. j4+3
+    const int i0[2] = {32 * ih + 8 * g, 32 * ih + 8 * g + 4};   // first value channel of this lane's four rows in tile mm
+    const int idx = tid - NPREP * 64, xt = idx >> 4, xj = (idx & 15) * 4;   // exact path: (token, channels) this thread finishes
+
+    f32x4 D[2];
+    D[0] = D[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (a.s0 != nullptr) {
+        const uint16_t* s = a.s0 + bh * N * N + j_own;
+#pragma unroll
+        for (int mm = 0; mm < 2; ++mm)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) D[mm][v] = bf2f(s[(i0[mm] + v) * N]);
+    }
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    float gu_acc[4] = {0.f, 0.f, 0.f, 0.f};            // chunked path: lane = token of tile ih, rows j4 + v
+    float gu_x[4] = {0.f, 0.f, 0.f, 0.f};              // exact path: token xt, channels xj + e
+
+    __syncthreads();
+    __syncthreads();
+    for (int i = 0; i < nchunks; ++i) {
+        const int c0 = i * L;
+        const SetA& O = S.set[i & 1];
+        const bool exact = O.exact != 0;
+        f32x4 own;                                     // (GY S)^T of this half of i: rows j4 + v, token 16 ih + l16
+        bf16x8 ktH, ktL;                               // K'^T of the own key channels: lane = j_own, K slots = tokens
+        if (!exact) {
+            const float d1j = O.d1[j_own];
+            const HL x0 = hilo2(D[0][0] * d1j, D[0][1] * d1j), x1 = hilo2(D[0][2] * d1j, D[0][3] * d1j);
+            const HL x2 = hilo2(D[1][0] * d1j, D[1][1] * d1j), x3 = hilo2(D[1][2] * d1j, D[1][3] * d1j);
+            const bf16x8 sh = as_op(x0.h, x1.h, x2.h, x3.h), sl = as_op(x0.l, x1.l, x2.l, x3.l);
+            const bf16x8 g0 = lds_op(&O.GY[l16][16 * ih + 4 * g]), g1 = lds_op(&O.GY[16 + l16][16 * ih + 4 * g]);
+            f32x4 Y0 = mfma(sh, g0, zero4), Y1 = mfma(sh, g1, zero4);
+            Y0 = mfma(sl, g0, Y0); Y1 = mfma(sl, g1, Y1);
+            S.Xch[sw][lane] = ih ? make_float4(Y0[0], Y0[1], Y0[2], Y0[3]) : make_float4(Y1[0], Y1[1], Y1[2], Y1[3]);
+            own = ih ? Y1 : Y0;
+            __builtin_amdgcn_sched_barrier(0);
+            // ------------------------------------------------------------ K'^T of the own key channels
+            {
+                const bf16x8 selOwn = op4(S.sel[q & 1][lane]);
+                const f32x4 zh0 = mfma(lds_op(&O.KpH[l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
+                const f32x4 zh1 = mfma(lds_op(&O.KpH[16 + l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
+                const f32x4 zl0 = mfma(lds_op(&O.KpL[l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
+                const f32x4 zl1 = mfma(lds_op(&O.KpL[16 + l16][16 * (q >> 1) + 4 * g]), selOwn, zero4);
+                ktH = pack_tokens(zh0, zh1); ktL = pack_tokens(zl0, zl1);
+            }
+            // ------------------------------------------------------------ S = S diag(dec) + diag(d2) V^T K'
+            const float decj = O.dec[j_own], d2j = O.d2[j_own];
+            const bf16x8 v0 = lds_op(&O.V[l16][16 * ih + 4 * g]), v1 = lds_op(&O.V[16 + l16][16 * ih + 4 * g]);
+#pragma unroll
+            for (int mm = 0; mm < 2; ++mm) {
+                const bf16x8 sel = op4(S.sel[mm][lane]);
+                const bf16x8 vt = pack_tokens(mfma(v0, sel, zero4), mfma(v1, sel, zero4));   // lane = value-channel row, slots = tokens
+                f32x4 U = mfma(vt, ktH, zero4);
+                U = mfma(vt, ktL, U);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) D[mm][v] = fmaf(D[mm][v], decj, d2j * U[v]);
+            }
+        } else {
+            // ------------------------------------------------------------ exact path: 32 sequential steps
+            for (int t = 0; t < L; ++t) {
+                float vv[2][4], gg[2][4];
+#pragma unroll
+                for (int mm = 0; mm < 2; ++mm) {
+                    unpack4(*reinterpret_cast<const uint2*>(&O.V[t][i0[mm] >> 1]), vv[mm]);
+                    unpack4(*reinterpret_cast<const uint2*>(&O.GY[t][i0[mm] >> 1]), gg[mm]);
+                }
+                const uint32_t kq = O.Kr[t][j_own >> 1];
+                const float kj = (j_own & 1) ? bf_hi(kq) : bf_lo(kq), wj = O.Ea[t][j_own];
+                float dr = 0.f, vg = 0.f;
+#pragma unroll
+                for (int mm = 0; mm < 2; ++mm)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        dr = fmaf(gg[mm][v], D[mm][v], dr);
+                        vg = fmaf(gg[mm][v], vv[mm][v], vg);
+                        D[mm][v] = fmaf(D[mm][v], wj, vv[mm][v] * kj);
+                    }
+                dr = allreduce_rows(dr); vg = allreduce_rows(vg);
+                if (g == 0) S.Yx[ih][t][j_own] = dr;
+                if (q == 0 && lane == 0) S.Vx[ih][t] = vg;
+            }
+        }
+        __syncthreads();
+        if (!exact) {
+            const int t = 16 * ih + l16, tg = c0 + t;
+            const float4 p = S.Xch[sw ^ 4][lane];
+            const bf16x8 bh_ = lds_op(&S.BmH[t][4 * g]);
+            f32x4 dr = own + f32x4{p.x, p.y, p.z, p.w};
+            dr = mfma(ktH, bh_, dr);
+            dr = mfma(ktH, lds_op(&S.BmL[t][4 * g]), dr);
+            dr = mfma(ktL, bh_, dr);
+            const float4 ea4 = *reinterpret_cast<const float4*>(&O.Ea[t][j4]);
+            const float4 u4 = *reinterpret_cast<const float4*>(&S.u[j4]);
+            float rr[4], kk[4];
+            unpack4(*reinterpret_cast<const uint2*>(&O.Rr[t][j4 >> 1]), rr);
+            unpack4(*reinterpret_cast<const uint2*>(&O.Kr[t][j4 >> 1]), kk);
+            const float vgy = S.vgy[t];
+            const float ea[4] = {ea4.x, ea4.y, ea4.z, ea4.w}, uu[4] = {u4.x, u4.y, u4.z, u4.w};
+            float gr[4], rd[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float drp = dr[v] * ea[v];
+                const float kv = kk[v] * vgy;
+                gr[v] = fmaf(uu[v], kv, drp);
+                rd[v] = rr[v] * drp;
+                gu_acc[v] = fmaf(rr[v], kv, gu_acc[v]);
+            }
+            if (tg < T) {
+                const uint32_t o = static_cast<uint32_t>(tg) * C + j4;
+                store8(a.gr + base, o * 2, make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3])));
+                store16(a.rdr + base, o * 4, f32x4{rd[0], rd[1], rd[2], rd[3]});
+            }
+        } else {
+            // exact path: add the two halves; token xt, key channels xj .. xj+3
+            const float4 p0 = *reinterpret_cast<const float4*>(&S.Yx[0][xt][xj]);
+            const float4 p1 = *reinterpret_cast<const float4*>(&S.Yx[1][xt][xj]);
+            const float4 u4 = *reinterpret_cast<const float4*>(&S.u[xj]);
+            const float vg = S.Vx[0][xt] + S.Vx[1][xt];
+            float rr[4], kk[4];
+            unpack4(*reinterpret_cast<const uint2*>(&O.Rr[xt][xj >> 1]), rr);
+            unpack4(*reinterpret_cast<const uint2*>(&O.Kr[xt][xj >> 1]), kk);
+            const float dr[4] = {p0.x + p1.x, p0.y + p1.y, p0.z + p1.z, p0.w + p1.w}, uu[4] = {u4.x, u4.y, u4.z, u4.w};
+            float gr[4], rd[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float kv = kk[e] * vg;
+                gr[e] = fmaf(uu[e], kv, dr[e]);
+                rd[e] = rr[e] * dr[e];
+                gu_x[e] = fmaf(rr[e], kv, gu_x[e]);
+            }
+            if (c0 + xt < T) {
+                const uint32_t o = static_cast<uint32_t>(c0 + xt) * C + xj;
+                store8(a.gr + base, o * 2, make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3])));
+                store16(a.rdr + base, o * 4, f32x4{rd[0], rd[1], rd[2], rd[3]});
+            }
+        }
+        __syncthreads();
+    }
+    // gu: the chunked path sums over the 16 tokens of a row of lanes; the exact path's sums go by (token, channel) rows
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const float s = row_sum_to_last(gu_acc[v]);
+        if (l16 == 15) S.gfast[ih][j4 + v] = s;
+    }
+    *reinterpret_cast<float4*>(&S.Yx[0][xt][xj]) = make_float4(gu_x[0], gu_x[1], gu_x[2], gu_x[3]);
+    __syncthreads();
+}
+
+template <int WMODE>
+__global__ __launch_bounds__(NTA) void wkv6_bwd_a_ws(const ArgsB a) {
+    __shared__ SmemA2 S;
+    const int tid = threadIdx.x;
+    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
+    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
+    const size_t bh = static_cast<size_t>(b) * a.H + h;
+    const int nchunks = (a.T + L - 1) / L;
+    // positions of the tile that are never written (t < 16 <= s) must read as zero
+    for (int i = tid; i < 2 * L * AS; i += NTA) (&S.BmH[0][0])[i] = 0;
+    if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
+    if (tid < 128) {
+        // One-hot B operand of the transposing products, per lane (column r = l16, K-slot group g), for tile parity p:
+        // column r <-> channel 8 (r>>2) + 4 p + (r&3) of a 32-channel half.
+        const int p = tid >> 6, ln = tid & 63, c16 = ln & 15, gg = ln >> 4;
+        S.sel[p][ln] = one_hot(gg == (c16 >> 2), 4 * p + (c16 & 3));
+    }
+    if (__builtin_amdgcn_readfirstlane(tid >> 6) < NPREP) bwa_prep<WMODE>(S, a, tid, base, nchunks);
+    else bwa_state<WMODE>(S, a, tid, base, bh, nchunks);
+}
+
+}  // namespace
+
+int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
+                            const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
+                            const uint16_t* s0, const uint16_t* gy, uint16_t* gr, uint16_t* gu, float* rdr) {
+    ArgsB a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.gy = gy;
+    a.gr = gr; a.gu = gu; a.rdr = rdr;
+    if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_bwd_a_ws<W_RAW>, dim3(B * H), dim3(NTA), 0, st, a);
+    else hipLaunchKernelGGL(wkv6_bwd_a_ws<W_EW>, dim3(B * H), dim3(NTA), 0, st, a);
+    return launch_status();
+}
+
+}  // namespace rwkv

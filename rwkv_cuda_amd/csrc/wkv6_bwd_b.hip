@@ -25,10 +25,6 @@ namespace {
 
 constexpr int NPREP = 8;
 constexpr int NTB = 1024;
-constexpr int OS = 40;            // row stride (dwords) of a bf16 [token][channel] plane: 160 B, conflict-free for 16-byte reads
-constexpr int FS = 72;            // row stride (dwords) of an fp32 [token][channel] array
-constexpr int AS = 24;            // row stride (dwords) of a tile plane [s][32 positions of tau]
-constexpr float LN2 = 0.69314718055994530942f;
 constexpr int STB = 3;            // visits of input kept in flight
 
 struct alignas(16) SetB {
@@ -57,43 +53,6 @@ struct alignas(16) SmemB2 {
     float part[2][NPREP][N];
     uint32_t flag[2][NPREP];
 };
-
-template <int CTRL, int ROW_MASK> DEVINL float dpp_add(float x) {
-    return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xf, true));
-}
-// sum over lanes 0..31 in lane 31 and over lanes 32..63 in lane 63
-DEVINL float half_wave_sum(float x) {
-    x = dpp_add<0x118, 0xf>(x);       // row_shr:8
-    x = dpp_add<0x114, 0xf>(x);       // row_shr:4
-    x = dpp_add<0x112, 0xf>(x);       // row_shr:2
-    x = dpp_add<0x111, 0xf>(x);       // row_shr:1   -> lane 15 of every row holds the row sum
-    x = dpp_add<0x142, 0xa>(x);       // row_bcast:15 into rows 1 and 3
-    return x;
-}
-// inclusive suffix sum over the 16 lanes of a row: lane l gets sum of lanes l..15
-DEVINL float row_suffix_sum(float x) {
-    x = dpp_add<0x101, 0xf>(x);       // row_shl:1
-    x = dpp_add<0x102, 0xf>(x);       // row_shl:2
-    x = dpp_add<0x104, 0xf>(x);       // row_shl:4
-    x = dpp_add<0x108, 0xf>(x);       // row_shl:8
-    return x;
-}
-
-DEVINL uint4 one_hot(bool on, int e) {                       // 8 bf16 slots, 1.0 in slot e
-    const uint32_t bits = (e & 1) ? 0x3f800000u : 0x00003f80u;
-    const int d = e >> 1;
-    return make_uint4(on && d == 0 ? bits : 0u, on && d == 1 ? bits : 0u, on && d == 2 ? bits : 0u, on && d == 3 ? bits : 0u);
-}
-DEVINL bf16x8 op4(const uint4& x) { return __builtin_bit_cast(bf16x8, x); }
-// two accumulator tiles (tokens 0..15 and 16..31 down the rows) -> one operand with the tokens along the K slots
-DEVINL bf16x8 pack_tokens(const f32x4& z0, const f32x4& z1) {
-    return as_op(cvt2(z0[0], z0[1]), cvt2(z0[2], z0[3]), cvt2(z1[0], z1[1]), cvt2(z1[2], z1[3]));
-}
-// 8-byte store at a wave-uniform base plus a 32-bit per-lane byte offset (keeps the address out of the vector registers)
-DEVINL void store8(const void* sbase, uint32_t byte_off, const uint2& x) {
-    asm volatile("global_store_dwordx2 %0, %1, %2" : : "v"(byte_off), "v"(x), "s"(sbase) : "memory");
-}
-DEVINL void unpack4(const uint2& x, float (&f)[4]) { f[0] = bf_lo(x.x); f[1] = bf_hi(x.x); f[2] = bf_lo(x.y); f[3] = bf_hi(x.y); }
 
 // ---------------------------------------------------------------------------------------------------- prep waves
 template <int WMODE>

@@ -1,4 +1,26 @@
-// Shared pieces of the chunked wkv6 kernels (gfx950): constants, the hi/lo bf16 operand format, in-chunk decay factors.
+// wkv6 / wkv6_state, chunked formulation on the matrix cores (gfx950, v_mfma_f32_16x16x32_bf16).
+//
+// Time is cut into chunks of L = 32 steps.  With lam_t[j] = log w_t[j] <= 0 and the in-chunk
+// cumulative sums c_t = sum_{z<t} lam_z (c_0 = 0), everything is referred to the chunk's MIDDLE
+// (m = 16) so that neither factor of a product can run away unless 16 consecutive decays shrink a
+// channel by more than e^-60 (then the chunk is redone step by step, see `exact`):
+//     R'_t = r_t e^{c_t - c_m}        K'_s = k_s e^{c_m - c_{s+1}}
+//     Rs_t = r_t e^{c_t}     = R'_t e^{c_m}            (reads the state that entered the chunk)
+//     Ke_s = k_s e^{c_L - c_{s+1}} = K'_s e^{c_L - c_m} (carries token s to the end of the chunk)
+//     A[t,s] = sum_j R'_t[j] K'_s[j]  (s < t),   A[t,t] = sum_j r_t[j] u[j] k_t[j]
+//     Y   = Rs S0^T + A V                               S[i][j]: i value channel, j key channel
+//     S_L = S0 diag(e^{c_L}) + V^T Ke
+// Every product runs on bf16 MFMA with fp32 accumulation; an fp32 operand x is split into
+// hi = bf16(x), lo = bf16(x - hi) (v, gy are exact in bf16 and need no split), which keeps ~16
+// mantissa bits per operand -- far below the bf16 rounding of the outputs, which is the error
+// the original fp32 kernels have.
+//
+// The state never leaves the accumulator registers: the accumulator layout of a 16x16 tile
+// (lane = column, lane group g and register v = row 4g+v) is used AS IS as the B operand of the
+// next chunk's Rs S0^T product, because the K slots of an MFMA may be assigned to channels in any
+// order as long as the A operand uses the same order; no transpose is ever needed.
+//
+// This header: constants, the hi/lo bf16 operand format, in-chunk decay factors, helpers of the wave-specialised kernels.
 #pragma once
 #include "common.h"
 
@@ -97,6 +119,61 @@ DEVINL Scale chunk_scale(bool second_half, float near, float lam0, float lam1) {
     }
     return s;
 }
+
+
+// ----------------------------------------------------------------------------------------------------------------------
+// Pieces shared by the wave-specialised kernels (forward, both backward sweeps).
+constexpr int OS = 40;            // row stride (dwords) of a bf16 [token][channel] plane: 160 B, conflict-free for 16-byte reads
+constexpr int FS = 72;            // row stride (dwords) of an fp32 [token][channel] array
+constexpr int AS = 24;            // row stride (dwords) of a tile plane [row][32 permuted positions]
+constexpr float LN2 = 0.69314718055994530942f;
+
+template <int CTRL, int ROW_MASK> DEVINL float dpp_add(float x) {
+    return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xf, true));
+}
+// sum over lanes 0..31 in lane 31 and over lanes 32..63 in lane 63
+DEVINL float half_wave_sum(float x) {
+    x = dpp_add<0x118, 0xf>(x);       // row_shr:8
+    x = dpp_add<0x114, 0xf>(x);       // row_shr:4
+    x = dpp_add<0x112, 0xf>(x);       // row_shr:2
+    x = dpp_add<0x111, 0xf>(x);       // row_shr:1   -> lane 15 of every row holds the row sum
+    x = dpp_add<0x142, 0xa>(x);       // row_bcast:15 into rows 1 and 3
+    return x;
+}
+// sum over the 16 lanes of a row, valid in lane 15 of the row
+DEVINL float row_sum_to_last(float x) {
+    x = dpp_add<0x118, 0xf>(x);
+    x = dpp_add<0x114, 0xf>(x);
+    x = dpp_add<0x112, 0xf>(x);
+    x = dpp_add<0x111, 0xf>(x);
+    return x;
+}
+// inclusive suffix sum over the 16 lanes of a row: lane l gets the sum of lanes l..15
+DEVINL float row_suffix_sum(float x) {
+    x = dpp_add<0x101, 0xf>(x);       // row_shl:1
+    x = dpp_add<0x102, 0xf>(x);       // row_shl:2
+    x = dpp_add<0x104, 0xf>(x);       // row_shl:4
+    x = dpp_add<0x108, 0xf>(x);       // row_shl:8
+    return x;
+}
+DEVINL uint4 one_hot(bool on, int e) {                       // 8 bf16 slots, 1.0 in slot e
+    const uint32_t bits = (e & 1) ? 0x3f800000u : 0x00003f80u;
+    const int d = e >> 1;
+    return make_uint4(on && d == 0 ? bits : 0u, on && d == 1 ? bits : 0u, on && d == 2 ? bits : 0u, on && d == 3 ? bits : 0u);
+}
+DEVINL bf16x8 op4(const uint4& x) { return __builtin_bit_cast(bf16x8, x); }
+// two accumulator tiles (tokens 0..15 and 16..31 down the rows) -> one operand with the tokens along the K slots
+DEVINL bf16x8 pack_tokens(const f32x4& z0, const f32x4& z1) {
+    return as_op(cvt2(z0[0], z0[1]), cvt2(z0[2], z0[3]), cvt2(z1[0], z1[1]), cvt2(z1[2], z1[3]));
+}
+// stores at a wave-uniform base plus a 32-bit per-lane byte offset (keeps the address out of the vector registers)
+DEVINL void store8(const void* sbase, uint32_t byte_off, const uint2& x) {
+    asm volatile("global_store_dwordx2 %0, %1, %2" : : "v"(byte_off), "v"(x), "s"(sbase) : "memory");
+}
+DEVINL void store16(const void* sbase, uint32_t byte_off, const f32x4& x) {
+    asm volatile("global_store_dwordx4 %0, %1, %2" : : "v"(byte_off), "v"(x), "s"(sbase) : "memory");
+}
+DEVINL void unpack4(const uint2& x, float (&f)[4]) { f[0] = bf_lo(x.x); f[1] = bf_hi(x.x); f[2] = bf_lo(x.y); f[3] = bf_hi(x.y); }
 
 }  // namespace
 }  // namespace rwkv

@@ -26,7 +26,6 @@ namespace {
 constexpr int NPREP = 8;
 constexpr int NSTATE = 8;
 constexpr int NTF = (NPREP + NSTATE) * 64;
-constexpr int OS = 40;            // row stride (dwords) of a bf16 [token][channel] plane: 160 B, conflict-free for 16-byte reads
 
 struct alignas(16) OperandSet {
     uint32_t RpH[L][OS], RpL[L][OS];   // r e^{c_t - c_m}      hi, lo   (exact path: r as fp32 [t][j] over both planes)
@@ -47,26 +46,6 @@ struct alignas(16) SmemF {
     float part[2][NPREP][N];           // sums of lam over each eighth of a chunk
     uint32_t flag[2][NPREP];
 };
-
-template <int CTRL, int ROW_MASK> DEVINL float dpp_add(float x) {
-    return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xf, true));
-}
-// sum over lanes 0..31 in lane 31 and over lanes 32..63 in lane 63
-DEVINL float half_wave_sum(float x) {
-    x = dpp_add<0x118, 0xf>(x);       // row_shr:8
-    x = dpp_add<0x114, 0xf>(x);       // row_shr:4
-    x = dpp_add<0x112, 0xf>(x);       // row_shr:2
-    x = dpp_add<0x111, 0xf>(x);       // row_shr:1   -> lane 15 of every row holds the row sum
-    x = dpp_add<0x142, 0xa>(x);       // row_bcast:15 into rows 1 and 3
-    return x;
-}
-
-DEVINL uint4 one_hot(bool on, int e) {                       // 8 bf16 slots, 1.0 in slot e
-    const uint32_t bits = (e & 1) ? 0x3f800000u : 0x00003f80u;
-    const int d = e >> 1;
-    return make_uint4(on && d == 0 ? bits : 0u, on && d == 1 ? bits : 0u, on && d == 2 ? bits : 0u, on && d == 3 ? bits : 0u);
-}
-DEVINL bf16x8 op4(const uint4& x) { return __builtin_bit_cast(bf16x8, x); }
 
 // ---------------------------------------------------------------------------------------------------- prep waves
 template <int WMODE>
