@@ -319,7 +319,10 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     }
 }
 
+// The chunked matrix-core kernels serve all three decay conventions; the sequential sweeps remain as the second algorithm.
 template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a) {
+    if (g_wkv6_algorithm == RWKV_ALGO_CHUNKED)
+        return launch_wkv6_fwd_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, a.w, a.u, a.s0, a.y);
     hipLaunchKernelGGL((wkv_sweep<P_FWD, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
     return launch_status();
 }
@@ -327,14 +330,15 @@ template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a) {
 // GR and GV are independent; GK consumes GR's workspace.  All three run on `st` in order.
 // `passes` is a bit mask (RWKV_PASS_*) so that a profiler can time one kernel at a time.
 template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a, unsigned passes = RWKV_PASS_ALL) {
-    const bool chunked = WMODE != W_HEAD && g_wkv6_algorithm == RWKV_ALGO_CHUNKED;
+    const bool chunked = g_wkv6_algorithm == RWKV_ALGO_CHUNKED;
+    const void* w = (WMODE == W_HEAD) ? static_cast<const void*>(a.ew_head) : a.w;   // wkv5: the log decay
     if ((passes & RWKV_PASS_GR) && chunked) {
-        if (int e = launch_wkv6_bwd_a_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, a.w, a.u, a.s0, a.gy, a.gr, a.gu, a.rdr)) return e;
+        if (int e = launch_wkv6_bwd_a_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, w, a.u, a.s0, a.gy, a.gr, a.gu, a.rdr)) return e;
     } else if (passes & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
     if (chunked) {
         // the chunked second sweep produces gk, gv, gw (and gs) together: it runs for GK, and GV alone is a no-op
         if (passes & RWKV_PASS_GK)
-            if (int e = launch_wkv6_bwd_b_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, a.w, a.u, a.s0, a.gy, a.gk, a.gv, a.gw, a.gs, a.rdr)) return e;
+            if (int e = launch_wkv6_bwd_b_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, w, a.u, a.s0, a.gy, a.gk, a.gv, a.gw, a.gs, a.rdr)) return e;
         return launch_status();
     }
     if (passes & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
@@ -400,8 +404,6 @@ int rwkv_wkv6_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16*
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, ew, u, y})) return e;
     Args a{};
-    if (g_wkv6_algorithm == RWKV_ALGO_CHUNKED)
-        return launch_wkv6_fwd_chunk(static_cast<hipStream_t>(stream), W_EW, B, T, C, H, r, k, v, ew, u, nullptr, y);
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.y = y;
     return launch_fwd<W_EW>(static_cast<hipStream_t>(stream), B, a);
 }
@@ -426,8 +428,6 @@ int rwkv_wkv6raw_forward(void* stream, int B, int T, int C, int H, const rwkv_bf
                          const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, rwkv_bf16* y) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, w, u, y})) return e;
-    if (g_wkv6_algorithm == RWKV_ALGO_CHUNKED)
-        return launch_wkv6_fwd_chunk(static_cast<hipStream_t>(stream), W_RAW, B, T, C, H, r, k, v, w, u, nullptr, y);
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.y = y;
     return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a);
@@ -452,8 +452,6 @@ int rwkv_wkv6state_forward(void* stream, int B, int T, int C, int H, const rwkv_
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, w, u, s, y})) return e;
     Args a{};
-    if (g_wkv6_algorithm == RWKV_ALGO_CHUNKED)
-        return launch_wkv6_fwd_chunk(static_cast<hipStream_t>(stream), W_RAW, B, T, C, H, r, k, v, w, u, s, y);
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.y = y;
     return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a);
 }

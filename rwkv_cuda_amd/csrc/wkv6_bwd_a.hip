@@ -57,7 +57,7 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
     // channel pair (2 jp, 2 jp + 1), tokens 4 wid + 2 th + {0, 1}
     const int jp = lane & 31, th = lane >> 5, pt0 = 4 * wid + 2 * th;
     const bool second = wid >= 4;
-    struct Raw { uint32_t r[2], k[2], v[2], g[2], w[2][WMODE == W_RAW ? 1 : 2]; float lam[2][2], other[2], kp[2][2]; };
+    struct Raw { uint32_t r[2], k[2], v[2], g[2], w[2][WMODE == W_EW ? 2 : 1]; float lam[2][2], other[2], kp[2][2]; };
     Raw ring[STA];
     // Loads are asm so that the wait before their first use can leave the younger batches in flight; every call issues the
     // same ten loads (chunk index clamped), which keeps the count fixed.
@@ -75,22 +75,32 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
             asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.g[e]) : "v"(o), "s"(gb));
             if constexpr (WMODE == W_RAW) {
                 asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.w[e][0]) : "v"(o), "s"(wb32));
-            } else {
+            } else if constexpr (WMODE == W_EW) {
                 uint2 y;
                 asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(y) : "v"(2 * o), "s"(wbf));
                 x.w[e][0] = y.x; x.w[e][1] = y.y;
             }
         }
     };
+    constexpr int NLOADS = WMODE == W_HEAD ? 8 : 10;   // loads per prefetch call
     auto arrived = [&](Raw& x, auto younger) __attribute__((always_inline)) {
         if constexpr (WMODE == W_RAW)
             asm volatile("s_waitcnt vmcnt(%10)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
-                         "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[1][0]) : "n"(decltype(younger)::value));
-        else
+                         "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[1][0]) : "n"(decltype(younger)::value * NLOADS));
+        else if constexpr (WMODE == W_EW)
             asm volatile("s_waitcnt vmcnt(%12)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
                          "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[0][1]), "+v"(x.w[1][0]), "+v"(x.w[1][1])
-                         : "n"(decltype(younger)::value));
+                         : "n"(decltype(younger)::value * NLOADS));
+        else
+            asm volatile("s_waitcnt vmcnt(%8)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.g[0]), "+v"(x.g[1]) : "n"(decltype(younger)::value * NLOADS));
     };
+    // wkv5: one decay per channel for the whole sequence, given as ew = -exp(w_raw) = log of the decay
+    float lamc[2] = {0.f, 0.f};
+    if constexpr (WMODE == W_HEAD) {
+        const float2 e2 = *reinterpret_cast<const float2*>(static_cast<const float*>(a.w) + (blockIdx.x % a.H) * N + 2 * jp);
+        lamc[0] = LOG2E * e2.x; lamc[1] = LOG2E * e2.y;
+    }
     static_for<STA>([&](auto Z) { prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
 
     // ---- scan of chunk c: lam (log2 units) of this thread's four elements, sums over each eighth of the chunk
@@ -102,7 +112,7 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
                 if (c0 + pt0 + e >= T) {
                     x.r[e] = 0; x.k[e] = 0; x.v[e] = 0; x.g[e] = 0;
                     if constexpr (WMODE == W_RAW) x.w[e][0] = 0xff80ff80u;   // w = -inf  ->  lam = -exp(w) = 0
-                    else { x.w[e][0] = 0u; x.w[e][1] = 0u; }
+                    if constexpr (WMODE == W_EW) { x.w[e][0] = 0u; x.w[e][1] = 0u; }
                 }
         }
 #pragma unroll
@@ -110,7 +120,8 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
                 if constexpr (WMODE == W_RAW) x.lam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e][0]) : bf_lo(x.w[e][0])));
-                else x.lam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+                else if constexpr (WMODE == W_EW) x.lam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+                else x.lam[e][z] = (c0 + pt0 + e < T) ? lamc[z] : 0.f;
             }
         float s2[2];
 #pragma unroll
@@ -237,7 +248,7 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
                 if (i + 1 < nchunks) exact_next = operands_a(i + 1, ring[(z + 1) % STA]);
                 __syncthreads();
                 // younger than the loads of chunk i+2: those of chunk i+3
-                arrived(ring[(z + 2) % STA], std::integral_constant<int, 10 * (STA - 2)>{});
+                arrived(ring[(z + 2) % STA], std::integral_constant<int, STA - 2>{});
                 if (i + 2 < nchunks) scan(i + 2, ring[(z + 2) % STA]);
                 if (i + 1 < nchunks) operands_b(i + 1, ring[(z + 1) % STA], exact_next);
                 prefetch(i + 1 + STA, ring[(z + 1) % STA]);
@@ -438,7 +449,8 @@ int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.gy = gy;
     a.gr = gr; a.gu = gu; a.rdr = rdr;
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_bwd_a_ws<W_RAW>, dim3(B * H), dim3(NTA), 0, st, a);
-    else hipLaunchKernelGGL(wkv6_bwd_a_ws<W_EW>, dim3(B * H), dim3(NTA), 0, st, a);
+    else if (wmode == W_EW) hipLaunchKernelGGL(wkv6_bwd_a_ws<W_EW>, dim3(B * H), dim3(NTA), 0, st, a);
+    else hipLaunchKernelGGL(wkv6_bwd_a_ws<W_HEAD>, dim3(B * H), dim3(NTA), 0, st, a);
     return launch_status();
 }
 

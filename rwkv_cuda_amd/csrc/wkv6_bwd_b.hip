@@ -71,7 +71,7 @@ DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + 2 * jp);
         uj[0] = bf_lo(x); uj[1] = bf_hi(x);
     }
-    struct Raw { uint32_t r[2], k[2], v[2], g[2], w[2][WMODE == W_RAW ? 1 : 2]; float2 d[2]; float lam[2][2], other[2], kp[2][2]; };
+    struct Raw { uint32_t r[2], k[2], v[2], g[2], w[2][WMODE == W_EW ? 2 : 1]; float2 d[2]; float lam[2][2], other[2], kp[2][2]; };
     Raw ring[STB];
     // Loads are asm so that the wait before their first use can leave the younger batches in flight; every call issues the
     // same twelve loads (visit index clamped), which keeps the count fixed.  Visit ci reads chunk nchunks - 1 - ci.
@@ -91,23 +91,33 @@ DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base
             asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(x.d[e]) : "v"(2 * o), "s"(db));
             if constexpr (WMODE == W_RAW) {
                 asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.w[e][0]) : "v"(o), "s"(wb32));
-            } else {
+            } else if constexpr (WMODE == W_EW) {
                 uint2 y;
                 asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(y) : "v"(2 * o), "s"(wbf));
                 x.w[e][0] = y.x; x.w[e][1] = y.y;
             }
         }
     };
+    constexpr int NLOADS = WMODE == W_HEAD ? 10 : 12;  // loads per prefetch call
     auto arrived = [&](Raw& x, auto younger) __attribute__((always_inline)) {
         if constexpr (WMODE == W_RAW)
             asm volatile("s_waitcnt vmcnt(%12)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
                          "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[1][0]), "+v"(x.d[0]), "+v"(x.d[1])
-                         : "n"(decltype(younger)::value));
-        else
+                         : "n"(decltype(younger)::value * NLOADS));
+        else if constexpr (WMODE == W_EW)
             asm volatile("s_waitcnt vmcnt(%14)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
                          "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[0][1]), "+v"(x.w[1][0]), "+v"(x.w[1][1]), "+v"(x.d[0]), "+v"(x.d[1])
-                         : "n"(decltype(younger)::value));
+                         : "n"(decltype(younger)::value * NLOADS));
+        else
+            asm volatile("s_waitcnt vmcnt(%10)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.d[0]), "+v"(x.d[1]) : "n"(decltype(younger)::value * NLOADS));
     };
+    // wkv5: one decay per channel for the whole sequence, given as ew = -exp(w_raw) = log of the decay
+    float lamc[2] = {0.f, 0.f};
+    if constexpr (WMODE == W_HEAD) {
+        const float2 e2 = *reinterpret_cast<const float2*>(static_cast<const float*>(a.w) + h * N + 2 * jp);
+        lamc[0] = LOG2E * e2.x; lamc[1] = LOG2E * e2.y;
+    }
     static_for<STB>([&](auto Z) { prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
 
     // ---- scan of visit ci: lam (log2 units) of this thread's four elements, sums over each eighth of the chunk
@@ -119,7 +129,7 @@ DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base
                 if (c0 + pt0 + e >= T) {
                     x.r[e] = 0; x.k[e] = 0; x.v[e] = 0; x.g[e] = 0; x.d[e] = make_float2(0.f, 0.f);
                     if constexpr (WMODE == W_RAW) x.w[e][0] = 0xff80ff80u;   // w = -inf  ->  lam = -exp(w) = 0
-                    else { x.w[e][0] = 0u; x.w[e][1] = 0u; }
+                    if constexpr (WMODE == W_EW) { x.w[e][0] = 0u; x.w[e][1] = 0u; }
                 }
         }
 #pragma unroll
@@ -127,7 +137,8 @@ DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
                 if constexpr (WMODE == W_RAW) x.lam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e][0]) : bf_lo(x.w[e][0])));
-                else x.lam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+                else if constexpr (WMODE == W_EW) x.lam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+                else x.lam[e][z] = (c0 + pt0 + e < T) ? lamc[z] : 0.f;
             }
         float s2[2];
 #pragma unroll
@@ -300,7 +311,7 @@ DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base
                 if (i + 1 < nchunks) exact_next = operands_a(i + 1, ring[(z + 1) % STB]);
                 __syncthreads();
                 // younger than the loads of visit i+2: those of visit i+3
-                arrived(ring[(z + 2) % STB], std::integral_constant<int, 12 * (STB - 2)>{});
+                arrived(ring[(z + 2) % STB], std::integral_constant<int, STB - 2>{});
                 if (i + 2 < nchunks) scan(i + 2, ring[(z + 2) % STB]);
                 if (i + 1 < nchunks) operands_b(i + 1, ring[(z + 1) % STB], exact_next);
                 prefetch(i + 1 + STB, ring[(z + 1) % STB]);
@@ -327,6 +338,8 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
 #pragma unroll
     for (int m = 0; m < 4; ++m) D[m] = f32x4{0.f, 0.f, 0.f, 0.f};
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    float gw_acc[4] = {0.f, 0.f, 0.f, 0.f};            // wkv5: sum over tokens of G (chunked path: this lane's tokens)
+    float gw_lane = 0.f;                               //       exact path: channel j_own
     float Pend[4] = {0.f, 0.f, 0.f, 0.f};              // P at the end of the current chunk for channels j4 + v (same in all 16 lanes of a row)
 
     __syncthreads();
@@ -396,8 +409,9 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 P = Gt + rdrj;
                 if (g == 0 && tg < T) {
                     a.gk[base + static_cast<size_t>(tg) * C + j_own] = f2bf(fmaf(uj * rj, vg, dkp));
-                    a.gw[base + static_cast<size_t>(tg) * C + j_own] = f2bf((!stateful && tg == 0) ? 0.f : lmj * Gt);
+                    if constexpr (WMODE != W_HEAD) a.gw[base + static_cast<size_t>(tg) * C + j_own] = f2bf((!stateful && tg == 0) ? 0.f : lmj * Gt);
                 }
+                if constexpr (WMODE == W_HEAD) gw_lane += (tg == 0 || tg >= T) ? 0.f : Gt;
             }
             if (g == 0) S.pc[j_own] = P;
             const float4 p4 = *reinterpret_cast<const float4*>(&S.pc[j4]);
@@ -443,6 +457,7 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                     const float tot = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, suf), 0x150, 0xf, 0xf, true));
                     const float Gt = (suf - dl) + (st == 0 ? tot1[v] : 0.f) + Pend[v] - kd;
                     gw[v] = (!stateful && tg == 0) ? 0.f : lm[v] * Gt;
+                    if constexpr (WMODE == W_HEAD) gw_acc[v] += (tg == 0 || tg >= T) ? 0.f : Gt;
                     if (st == 1) tot1[v] = tot; else Pend[v] += tot + tot1[v];
                 }
                 out_k[st] = make_uint2(pack_bf2(gk[0], gk[1]), pack_bf2(gk[2], gk[3]));
@@ -455,7 +470,7 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 if (tg < T) {
                     const uint32_t off = (static_cast<uint32_t>(tg) * C + j4) * 2;
                     store8(a.gk + base, off, out_k[st]);
-                    store8(a.gw + base, off, out_w[st]);
+                    if constexpr (WMODE != W_HEAD) store8(a.gw + base, off, out_w[st]);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -471,6 +486,17 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
             }
         }
         __syncthreads();
+    }
+    if constexpr (WMODE == W_HEAD) {                   // gw[b][h][j] = ew_j sum_t G_t[j]
+        if (g == 0) S.pc[j_own] = gw_lane;
+        const float4 px = *reinterpret_cast<const float4*>(&S.pc[j4]);
+        const float4 e4 = *reinterpret_cast<const float4*>(static_cast<const float*>(a.w) + (bh % a.H) * N + j4);
+        const float pxv[4] = {px.x, px.y, px.z, px.w}, ev[4] = {e4.x, e4.y, e4.z, e4.w};
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const float s = row_sum_to_last(gw_acc[v]) + pxv[v];
+            if (l16 == 15) a.gw[bh * N + j4 + v] = f2bf(ev[v] * s);
+        }
     }
     if (a.gs != nullptr) {
         uint16_t* s = a.gs + bh * N * N + j_own;
@@ -620,7 +646,8 @@ int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.gy = gy;
     a.gk = gk; a.gv = gv; a.gw = gw; a.gs = gs; a.rdr = const_cast<float*>(rdr);
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_bwd_b_ws<W_RAW>, dim3(B * H), dim3(NTB), 0, st, a);
-    else hipLaunchKernelGGL(wkv6_bwd_b_ws<W_EW>, dim3(B * H), dim3(NTB), 0, st, a);
+    else if (wmode == W_EW) hipLaunchKernelGGL(wkv6_bwd_b_ws<W_EW>, dim3(B * H), dim3(NTB), 0, st, a);
+    else hipLaunchKernelGGL(wkv6_bwd_b_ws<W_HEAD>, dim3(B * H), dim3(NTB), 0, st, a);
     return launch_status();
 }
 

@@ -41,7 +41,8 @@ constexpr float LOG2E = 1.44269504088896340736f;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-enum { W_EW = 1, W_RAW = 2 };     // wkv6: fp32 ew = -exp(w_raw) [B,T,C];  wkv6_state: raw bf16 w
+enum { W_HEAD = 0, W_EW = 1, W_RAW = 2 };   // wkv5: fp32 [H,N] (forward: decay eew, backward: ew = log decay);
+                                             // wkv6: fp32 ew = -exp(w_raw) [B,T,C];  wkv6_state: raw bf16 w [B,T,C]
 
 struct ArgsC {
     int T, C, H;

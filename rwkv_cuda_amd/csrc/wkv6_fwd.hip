@@ -63,7 +63,7 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + 2 * jp);
         uj[0] = bf_lo(x); uj[1] = bf_hi(x);
     }
-    struct Raw { uint32_t r[2], k[2], v[2], w[2][2]; float lam[2][2], other[2], kp[2][2]; };
+    struct Raw { uint32_t r[2], k[2], v[2], w[2][WMODE == W_EW ? 2 : 1]; float lam[2][2], other[2], kp[2][2]; };
     Raw ring[STAGES];
     // The loads of a chunk are issued STAGES chunks before they are used.  They are written as asm so that the wait before
     // the first use can name the number of younger loads that may still be in flight (the compiler would wait for all of
@@ -81,7 +81,7 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
             asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.v[e]) : "v"(o), "s"(vb));
             if constexpr (WMODE == W_RAW) {
                 asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.w[e][0]) : "v"(o), "s"(wb32));
-            } else {
+            } else if constexpr (WMODE == W_EW) {
                 uint2 y;
                 asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(y) : "v"(2 * o), "s"(wbf));
                 x.w[e][0] = y.x; x.w[e][1] = y.y;
@@ -89,10 +89,24 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         }
     };
     // wait until at most `younger` loads issued after those of x are outstanding
+    constexpr int NLOADS = WMODE == W_HEAD ? 6 : 8;    // loads per prefetch call
     auto arrived = [&](Raw& x, auto younger) __attribute__((always_inline)) {
-        asm volatile("s_waitcnt vmcnt(%10)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
-                     "+v"(x.w[0][0]), "+v"(x.w[0][1]), "+v"(x.w[1][0]), "+v"(x.w[1][1]) : "n"(decltype(younger)::value));
+        if constexpr (WMODE == W_EW)
+            asm volatile("s_waitcnt vmcnt(%10)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.w[0][0]), "+v"(x.w[0][1]), "+v"(x.w[1][0]), "+v"(x.w[1][1]) : "n"(decltype(younger)::value * NLOADS));
+        else if constexpr (WMODE == W_RAW)
+            asm volatile("s_waitcnt vmcnt(%8)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.w[0][0]), "+v"(x.w[1][0]) : "n"(decltype(younger)::value * NLOADS));
+        else
+            asm volatile("s_waitcnt vmcnt(%6)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1])
+                         : "n"(decltype(younger)::value * NLOADS));
     };
+    // wkv5: one decay per channel for the whole sequence, given as eew = exp(-exp(w_raw)); lam = log2(eew)
+    float lamc[2] = {0.f, 0.f};
+    if constexpr (WMODE == W_HEAD) {
+        const float2 e2 = *reinterpret_cast<const float2*>(static_cast<const float*>(a.w) + h * N + 2 * jp);
+        lamc[0] = __builtin_amdgcn_logf(e2.x); lamc[1] = __builtin_amdgcn_logf(e2.y);
+    }
     static_for<STAGES>([&](auto Z) { prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
 
     // ---- scan of chunk c: lam (log2 units) of this thread's four elements, sums over each eighth of the chunk
@@ -103,8 +117,8 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
             for (int e = 0; e < 2; ++e)
                 if (c0 + pt0 + e >= T) {
                     x.r[e] = 0; x.k[e] = 0; x.v[e] = 0;
-                    x.w[e][0] = (WMODE == W_RAW) ? 0xff80ff80u : 0u;   // w = -inf  ->  lam = -exp(w) = 0
-                    x.w[e][1] = 0u;
+                    if constexpr (WMODE == W_RAW) x.w[e][0] = 0xff80ff80u;   // w = -inf  ->  lam = -exp(w) = 0
+                    if constexpr (WMODE == W_EW) { x.w[e][0] = 0u; x.w[e][1] = 0u; }
                 }
         }
 #pragma unroll
@@ -112,7 +126,8 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
                 if constexpr (WMODE == W_RAW) x.lam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e][0]) : bf_lo(x.w[e][0])));
-                else x.lam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+                else if constexpr (WMODE == W_EW) x.lam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+                else x.lam[e][z] = (c0 + pt0 + e < T) ? lamc[z] : 0.f;
             }
         float s2[2];
 #pragma unroll
@@ -256,7 +271,7 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
             const int i = ib + z;
             if (i < nchunks) {
                 // younger than the loads of chunk i+2: those of chunks i+3 and i+4
-                arrived(ring[(z + 2) % STAGES], std::integral_constant<int, 8 * (STAGES - 2)>{});
+                arrived(ring[(z + 2) % STAGES], std::integral_constant<int, STAGES - 2>{});
                 if (i + 2 < nchunks) scan(i + 2, ring[(z + 2) % STAGES]);
                 if (wid < 3 && !exact_cur) tile(i);
                 bool exact_next = false;
@@ -422,7 +437,8 @@ int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H,
     ArgsC a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y;
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_fwd_ws<W_RAW>, dim3(B * H), dim3(NTF), 0, st, a);
-    else hipLaunchKernelGGL(wkv6_fwd_ws<W_EW>, dim3(B * H), dim3(NTF), 0, st, a);
+    else if (wmode == W_EW) hipLaunchKernelGGL(wkv6_fwd_ws<W_EW>, dim3(B * H), dim3(NTF), 0, st, a);
+    else hipLaunchKernelGGL(wkv6_fwd_ws<W_HEAD>, dim3(B * H), dim3(NTF), 0, st, a);
     return launch_status();
 }
 
