@@ -30,10 +30,10 @@ ALGO = "chunked"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), keyed
 # by kernel label at the headline shape; None = not measured for the current kernels.
 TRAFFIC_MEASURED = {
-    # profiles/wkv6_chunk_kernels_B8_T4096_C2048.md  (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB)
-    "wkv6_fwd_chunk": 537e6 + 134e6,
-    "wkv6_bwd_a_chunk": 671e6 + 403e6,
-    "wkv6_bwd_b_chunk": 941e6 + 404e6,
+    # profiles/wkv6_ws_kernels_B8_T4096_C2048.md  (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB)
+    "wkv6_fwd_ws": 537e6 + 134e6,
+    "wkv6_bwd_a_ws": 671e6 + 403e6,
+    "wkv6_bwd_b_ws": 941e6 + 404e6,
 }
 
 
@@ -101,9 +101,9 @@ def make_wkv6(dev, state):
         # algorithmic bytes per kernel: tensors it must read once + outputs it must write once, 2 B per element
         fwd = lambda: call("rwkv_wkv6raw_forward", dev, B, T, C, H, r, k, v, w, u, y)
         if ALGO == "chunked":
-            kernels = [("wkv6_fwd_chunk", fwd, 10 * C * tok),                 # r k v w -> y
-                       ("wkv6_bwd_a_chunk", bwd(1), 12 * C * tok),            # r k v w gy -> gr (+ fp32 workspace)
-                       ("wkv6_bwd_b_chunk", bwd(4), 16 * C * tok)]            # r k v w gy -> gk gv gw
+            kernels = [("wkv6_fwd_ws", fwd, 10 * C * tok),                    # r k v w -> y
+                       ("wkv6_bwd_a_ws", bwd(1), 12 * C * tok),               # r k v w gy -> gr (+ fp32 workspace)
+                       ("wkv6_bwd_b_ws", bwd(4), 16 * C * tok)]               # r k v w gy -> gk gv gw
         else:
             kernels = [("wkv_sweep<FWD>", fwd, 10 * C * tok),
                        ("wkv_sweep<GR>", bwd(1), 12 * C * tok),               # r k v w gy -> gr
@@ -149,8 +149,16 @@ def make_wkv5(dev):
         call("rwkv_wkv5_backward", dev, B, T, C, H, r, k, v, eew_, ew_, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
         return torch.sum(gw, 0), torch.sum(gu, 0)
 
-    kernels = [("wkv5 forward", lambda: call("rwkv_wkv5_forward", dev, B, T, C, H, r, k, v, eew, u, y), 8 * C * tok),
-               ("wkv5 backward (3 kernels)", lambda: call("rwkv_wkv5_backward", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes), 14 * C * tok)]
+    def bwd(mask):
+        def run():
+            lib.rwkv_wkv6_set_backward_passes(mask)
+            call("rwkv_wkv5_backward", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+            lib.rwkv_wkv6_set_backward_passes(7)
+        return run
+
+    kernels = [("wkv6_fwd_ws<head decay>", lambda: call("rwkv_wkv5_forward", dev, B, T, C, H, r, k, v, eew, u, y), 8 * C * tok),
+               ("wkv6_bwd_a_ws<head decay>", bwd(1), 10 * C * tok),           # r k v gy -> gr (+ fp32 workspace)
+               ("wkv6_bwd_b_ws<head decay>", bwd(4), 12 * C * tok)]           # r k v gy -> gk gv
 
     def cpu_baseline(t_cpu=256):
         from oracle import wkv56 as O

@@ -396,7 +396,7 @@ int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = eew; a.ew_head = ew; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
-    return launch_bwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a);
+    return launch_bwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a, g_bwd_passes);
 }
 
 int rwkv_wkv6_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
