@@ -171,3 +171,32 @@ def test_wkv6_state_both_algorithms_and_extreme_decays(lib, algo):
         for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, emu, [y] + [x.grad for x in t]):
             assert torch.isfinite(g).all(), name
             assert_no_worse(name, a, e, g)
+
+
+@pytest.mark.parametrize("algo", [0, 1])
+def test_wkv5_both_algorithms_and_strong_decays(lib, algo):
+    """wkv5 (one decay per head channel) on the chunked and on the sequential kernels; with w_raw up to 2.5 some
+    channels lose e^-12 per step, which sends every chunk of that head down the chunked kernels' exact path."""
+    B, T, H = 2, 83, 2
+    C = H * 64
+    for strong in (False, True):
+        r, k, v, w, u, gy = synth.wkv5_inputs(B, T, C, H, seed=21)
+        if strong:
+            w = w.float()
+            w[1, 10:20] = 2.5
+            w[1, 40] = 1.5
+            w = w.to(BF)
+        ref = O.wkv5_grads(B, T, C, H, r, k, v, w, u, gy)
+        emu = O.emulate_wkv5_bf16(B, T, C, H, r, k, v, w, u, gy)
+        print(f"\nwkv5 algo={algo} strong={strong}", flush=True)
+        lib.rwkv_wkv6_set_algorithm(algo)
+        try:
+            t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u)]
+            y = wkv5_bf16.RUN_CUDA(B, T, C, H, *t)
+            y.backward(gy.to(DEV))
+            torch.cuda.synchronize()
+        finally:
+            lib.rwkv_wkv6_set_algorithm(0)
+        for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y] + [x.grad for x in t]):
+            assert torch.isfinite(g).all(), name
+            assert_no_worse(name, a, e, g)
