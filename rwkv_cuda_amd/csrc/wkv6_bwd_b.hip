@@ -51,7 +51,7 @@ struct alignas(16) SmemB2 {
     float u[N];
     float pc[N];                       // P per channel, when it changes layout around an exact chunk
     float part[2][NPREP][N];
-    uint32_t flag[2][NPREP];
+    alignas(8) uint8_t flag[2][NPREP]; // per prep wave: some channel decays too fast for the mid-point factors
 };
 
 // ---------------------------------------------------------------------------------------------------- prep waves
@@ -147,32 +147,33 @@ DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base
             x.other[z] = __shfl_xor(s2[z], 32, 64);    // the other two tokens of this wave's four
         }
         const float s4a = s2[0] + x.other[0], s4b = s2[1] + x.other[1];
-        if (th == 0) *reinterpret_cast<float2*>(&S.part[pb][wid][2 * jp]) = make_float2(s4a, s4b);
+        *reinterpret_cast<float2*>(&S.part[pb][wid][2 * jp]) = make_float2(s4a, s4b);   // both half-waves hold the same sums
         // A chunk whose decays could overflow the mid-point factors is redone exactly (see wkv6_chunk.h).
         const bool fast_decay = (-s4a > 0.25f * RANGE_LIMIT * LOG2E) || (-s4b > 0.25f * RANGE_LIMIT * LOG2E);
         const unsigned long long any = __ballot(fast_decay);
-        if (lane == 0) S.flag[pb][wid] = any != 0ull;
+        if (lane == 0) S.flag[pb][wid] = any != 0ull ? 1 : 0;
     };
 
     // ---- operands of visit ci into set ci & 1, first part: R' planes, Eb, plain r (K' values stay in registers)
     auto operands_a = [&](const int ci, Raw& x) __attribute__((always_inline)) -> bool {
         SetB& O = S.set[ci & 1];
         const int pb = ci & 1;
-        const uint4 f0 = *reinterpret_cast<const uint4*>(&S.flag[pb][0]), f1 = *reinterpret_cast<const uint4*>(&S.flag[pb][4]);
+        const uint2 f8 = *reinterpret_cast<const uint2*>(&S.flag[pb][0]);
         float2 pe[4];
 #pragma unroll
         for (int w4 = 0; w4 < 4; ++w4) pe[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * second + w4][2 * jp]);
-        const bool exact = (f0.x | f0.y | f0.z | f0.w | f1.x | f1.y | f1.z | f1.w) != 0;
+        const bool exact = __builtin_amdgcn_readfirstlane(f8.x | f8.y) != 0;     // the same in every wave: a scalar
         if (tid == 0) O.exact = exact;
         float near[2];
         near[0] = second ? (th ? x.other[0] : 0.f) : (th ? 0.f : x.other[0]);
         near[1] = second ? (th ? x.other[1] : 0.f) : (th ? 0.f : x.other[1]);
-        const int w_own = wid & 3;
-#pragma unroll
-        for (int w4 = 0; w4 < 4; ++w4) {
-            const bool between = second ? (w4 < w_own) : (w4 > w_own);      // wave-uniform
-            near[0] += between ? pe[w4].x : 0.f;
-            near[1] += between ? pe[w4].y : 0.f;
+        {   // eighths between this wave's and the middle: first half w_own+1..3, second half 0..w_own-1 (scalar branches)
+            const int w_own = wid & 3;
+            const int lo = second ? 0 : w_own + 1, hi = second ? w_own : 4;
+            if (lo <= 0 && 0 < hi) { near[0] += pe[0].x; near[1] += pe[0].y; }
+            if (lo <= 1 && 1 < hi) { near[0] += pe[1].x; near[1] += pe[1].y; }
+            if (lo <= 2 && 2 < hi) { near[0] += pe[2].x; near[1] += pe[2].y; }
+            if (lo <= 3 && 3 < hi) { near[0] += pe[3].x; near[1] += pe[3].y; }
         }
         float pr[2][2];
 #pragma unroll
@@ -347,7 +348,7 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
     for (int i = 0; i < nchunks; ++i) {
         const int c0 = (nchunks - 1 - i) * L;
         const SetB& O = S.set[i & 1];
-        const bool exact = O.exact != 0;
+        const bool exact = __builtin_amdgcn_readfirstlane(O.exact) != 0;
         f32x4 dkin[2];                                 // (V dS)^T: rows j4 + v, lane = token 16 st + l16
         bf16x8 rtH, rtL;                               // R'^T of this wave's key channels: lane = j_own, K slots = tokens
         if (!exact) {
@@ -529,7 +530,7 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
     for (int i = 0; i < nchunks; ++i) {
         const int c0 = (nchunks - 1 - i) * L;
         const SetB& O = S.set[i & 1];
-        const bool exact = O.exact != 0;
+        const bool exact = __builtin_amdgcn_readfirstlane(O.exact) != 0;
         f32x4 dvin[2];                                 // (K' diag(d2) dS^T)^T: rows i4 + v, lane = token 16 st + l16
         bf16x8 gto;                                    // gy^T of this wave's value channels: lane = i_own, K slots = tokens
         if (!exact) {
