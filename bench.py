@@ -25,6 +25,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 ALGO = "chunked"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), keyed
@@ -264,18 +265,23 @@ def make_timex(dev):
     from rwkv_cuda_amd._call import call
     B, C, T = 32, 768, 768
     w, k, g = (x.to(dev) for x in synth.timex_inputs(B, C, T, seed=42))
-    x, gw, gk = (torch.empty(B, C, T, device=dev) for _ in range(3))
+    x, gk = (torch.empty(B, C, T, device=dev) for _ in range(2))
+    gw = torch.empty(C, T, device=dev)
     tok = B * T
 
+    # what TimeX.apply(...).backward() launches at this shape: gw comes out summed over the batch
     def step():
         call("rwkv_timex_forward", dev, w, k, x, 0.0, B, C, T)
-        call("rwkv_timex_backward", dev, w, k, g, gw, gk, B, C, T)
-        return gw.sum(0)
+        call("rwkv_timex_backward_sum", dev, w, k, g, gw, gk, B, C, T)
 
     fwd_bytes = (C * T + 2 * B * C * T) * 4
-    bwd_bytes = (C * T + 4 * B * C * T) * 4
-    kernels = [("timex forward", lambda: call("rwkv_timex_forward", dev, w, k, x, 0.0, B, C, T), fwd_bytes),
-               ("timex backward (2 kernels)", lambda: call("rwkv_timex_backward", dev, w, k, g, gw, gk, B, C, T), bwd_bytes)]
+    bwd_bytes = (2 * C * T + 3 * B * C * T) * 4
+    # The direct convolution does T (T + 1) / 2 multiply-adds per row and output array, in fp32: 64 flop per byte at
+    # T = 768, three times the ratio of the fp32 matrix peak to the HBM peak, so these kernels are bound by the former.
+    conv_flops = B * C * T * (T + 1)
+    kernels = [("timex_conv_mfma (forward)", lambda: call("rwkv_timex_forward", dev, w, k, x, 0.0, B, C, T), fwd_bytes, conv_flops),
+               ("timex backward (timex_conv_mfma + timex_gw_sum_mfma)",
+                lambda: call("rwkv_timex_backward_sum", dev, w, k, g, gw, gk, B, C, T), bwd_bytes, 2 * conv_flops)]
 
     def cpu_baseline(bs=4):
         from oracle import timex as O
@@ -286,7 +292,7 @@ def make_timex(dev):
         return bs * T / dt / 1e6, f"depthwise_conv1d fwd+bwd, zero-padded grouped F.conv1d, fp32, B={bs} of 32, C{C} T{T} ({dt:.1f} s)"
 
     cfg = {"workload": f"depthwise_conv1d fp32 fwd+bwd B{B} C{C} T{T}", "B": B, "C": C, "T": T,
-           "algorithmic_bytes_per_step": fwd_bytes + bwd_bytes}
+           "algorithmic_bytes_per_step": fwd_bytes + bwd_bytes, "algorithmic_flops_per_step": 3 * conv_flops}
     return step, tok, kernels, cfg, cpu_baseline, fwd_bytes + bwd_bytes
 
 
@@ -348,15 +354,22 @@ def main():
 
     # per-kernel timing, HIP events on the launch stream
     per_kernel = []
-    for label, fn, nbytes in kernels:
+    for label, fn, nbytes, *flops in kernels:
         ms = time_gpu(fn, max(5, args.steps), 2)
         per_kernel.append({"kernel": label, "ms": round(ms, 4), "algorithmic_bytes": nbytes,
                            "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)})
+        if flops:                                # a kernel bound by the fp32 matrix cores, not by HBM
+            per_kernel[-1].update(algorithmic_flops=flops[0], TFLOPs=round(flops[0] / (ms * 1e-3) / 1e12, 2))
     dom = max(per_kernel, key=lambda d: d["ms"])
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(dom["GBps"] / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_MEASURED.get(dom["kernel"]),
                 "launch_ms": dom["ms"], "algorithmic_bytes": dom["algorithmic_bytes"],
                 "whole_step_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    if "TFLOPs" in dom:
+        roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["TFLOPs"], "peak": FP32_MFMA_PEAK_TFLOPS,
+                    "unit": "TFLOP/s", "frac": round(dom["TFLOPs"] / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                    "launch_ms": dom["ms"], "algorithmic_flops": dom["algorithmic_flops"],
+                    "hbm_frac": round(dom["GBps"] / HBM_PEAK_GBS, 4)}
 
     out = {
         "metric": "WKV6 bf16 fwd+bwd Mtokens/s @B8 T4096 C2048; % HBM peak achieved" if args.workload == "wkv6"

@@ -82,6 +82,11 @@ int rwkv_wkv4_backward(void* stream, int B, int T, int C,
 int rwkv_timex_forward(void* stream, const float* w, const float* k, float* x, float eps, int B, int C, int T);
 int rwkv_timex_backward(void* stream, const float* w, const float* k, const float* gwk,
                         float* gw, float* gk, int B, int C, int T);
+/* The same backward with the wrapper's sum over the batch (depthwise_conv1d/run.py:102) done inside:
+ * gw_sum[C,T] = sum_b gw[b], gk as above.  Needs T % 32 == 0 and T <= 1024 (RWKV_ERR_SHAPE otherwise:
+ * call rwkv_timex_backward and sum).  The order of every fp32 sum is fixed, so results repeat bit for bit. */
+int rwkv_timex_backward_sum(void* stream, const float* w, const float* k, const float* gwk,
+                            float* gw_sum, float* gk, int B, int C, int T);
 
 /* ---------------------------------------------------------------------------------------
  * RWKV-5 wkv, bf16 I/O.  Replaces cuda_forward / cuda_backward of

@@ -59,6 +59,7 @@ SIGNATURES = {
     "rwkv_wkv4_backward": (_I, [_P, _I, _I, _I] + [_P] * 9 + [_P, _Z]),
     "rwkv_timex_forward": (_I, [_P, _P, _P, _P, _F, _I, _I, _I]),
     "rwkv_timex_backward": (_I, [_P] * 6 + [_I, _I, _I]),
+    "rwkv_timex_backward_sum": (_I, [_P] * 6 + [_I, _I, _I]),
     "rwkv_wkv5_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
     "rwkv_wkv5_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv5_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_P, _Z]),

@@ -104,6 +104,205 @@ __global__ __launch_bounds__(1024) void timex_gw(const float* __restrict__ k, co
     *reinterpret_cast<float4*>(gw + row * T + (T - 4 - d0)) = make_float4(acc[3], acc[2], acc[1], acc[0]);
 }
 
+// ---------------------------------------------------------------------------------------------------- matrix-core path
+// For T a multiple of 32 (and short enough for 32 rows to sit in LDS) the convolution of 32 batch rows of one channel is a
+// product of the lower-triangular Toeplitz matrix W[t][u] = wr[t-u] with the [T x 32] block of inputs, done in fp32 on
+// v_mfma_f32_32x32x2_f32 (lane = (row or column l & 31, K slot half l >> 5); accumulator register v: row 8 (v/4) + 4 (l>>5)
+// + (v&3), column l & 31).  The kernel row is stored in tap order followed by 32 zeros, so a tap of negative lag reads 0
+// and the diagonal block needs no mask.  Output tile o of 32 time steps sums over input tiles 0..o (mirror: o..T/32-1);
+// a wave takes tiles p and T/32-1-p, which balances the triangle.  K slot (half, kk) is input step 16 half + kk of the
+// tile, so a lane reads its 16 B operands as four 16-byte LDS reads.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int MROWS = 32;              // batch rows per workgroup = columns of the product
+constexpr int T_MFMA_MAX = 1024;
+constexpr int TXW = 8;                 // waves per workgroup: two per SIMD, one reads LDS while the other runs MFMAs
+constexpr int TXT = 64 * TXW;
+constexpr int STG = 4;                 // 16-byte global loads in flight per thread while staging
+
+template <bool MIRROR>
+__global__ __launch_bounds__(TXT) void timex_conv_mfma(const float* __restrict__ w, const float* __restrict__ in,
+                                                       float* __restrict__ out, float eps, int B, int C, int T) {
+    extern __shared__ float lds[];
+    float* wp = lds;                   // [T + 32]: wp[x] = w[c][x] (tap order), 0 for x >= T
+    float* rows = lds + T + 32;        // [32][T + 4]
+    const int rs = T + 4;
+    const int c = blockIdx.x, b0 = blockIdx.y * MROWS, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int ln = lane & 31, kh = lane >> 5;
+
+    for (int i = tid; i < T + 32; i += TXT) wp[i] = i < T ? w[static_cast<size_t>(c) * T + i] : 0.f;
+    // rows come in with STG 16-byte loads in flight per thread: one block per CU has nothing else to hide HBM latency with
+    const int q4n = T >> 2, total = MROWS * q4n;
+    for (int base = 0; base < total; base += STG * TXT) {
+        float4 x[STG];
+#pragma unroll
+        for (int s = 0; s < STG; ++s) {
+            const int idx = base + s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
+            // the load itself is unconditional (from a clamped address) so that all STG are issued before the first wait
+            const bool live = idx < total && b0 + r < B;
+            x[s] = *reinterpret_cast<const float4*>(in + (static_cast<size_t>(live ? b0 + r : b0) * C + c) * T + (live ? 4 * q4 : 0));
+        }
+#pragma unroll
+        for (int s = 0; s < STG; ++s) {
+            const int idx = base + s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
+            if (idx < total) *reinterpret_cast<float4*>(rows + r * rs + 4 * q4) = b0 + r < B ? x[s] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    __syncthreads();
+
+    const int nt = T >> 5;
+    const float* brow = rows + ln * rs + 16 * kh;
+    for (int p = wv; 2 * p < nt; p += TXW) {
+#pragma unroll 1
+        for (int side = 0; side < 2; ++side) {
+            const int ot = side == 0 ? p : nt - 1 - p;
+            if (side == 1 && ot == p) break;
+            f32x16 acc, acc1;                              // even / odd K steps: consecutive MFMAs are independent
+#pragma unroll
+            for (int v = 0; v < 16; ++v) { acc[v] = MIRROR ? 0.f : eps; acc1[v] = 0.f; }
+            const int n_in = MIRROR ? nt - ot : ot + 1;
+            // operands of step j + 1 are read while the MFMAs of step j run
+            float a[16], b[16];
+            auto fetch = [&](int j, float (&fa)[16], float (&fb)[16]) {
+                const int it = MIRROR ? ot + j : j;            // input tile
+                const int d = MIRROR ? j : ot - j;             // lag in tiles, >= 0
+                // A[row][K slot]: forward row = t, slot = u: tap T-1-(t-u);  mirror row = u, slot = t: tap T-1-(t-u)
+                const float* ap = wp + (MIRROR ? T - 1 - 32 * d - 16 * kh + ln : T - 1 - 32 * d - ln + 16 * kh);
+#pragma unroll
+                for (int kk = 0; kk < 16; ++kk) fa[kk] = MIRROR ? ap[-kk] : ap[kk];
+#pragma unroll
+                for (int z = 0; z < 4; ++z) {
+                    const float4 x = *reinterpret_cast<const float4*>(brow + 32 * it + 4 * z);
+                    fb[4 * z] = x.x; fb[4 * z + 1] = x.y; fb[4 * z + 2] = x.z; fb[4 * z + 3] = x.w;
+                }
+            };
+            fetch(0, a, b);
+            for (int j = 0; j < n_in; ++j) {
+                float an[16], bn[16];
+                fetch(j + 1 < n_in ? j + 1 : j, an, bn);
+#pragma unroll
+                for (int kk = 0; kk < 16; kk += 2) {
+                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk], b[kk], acc, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk + 1], b[kk + 1], acc1, 0, 0, 0);
+                }
+#pragma unroll
+                for (int kk = 0; kk < 16; ++kk) { a[kk] = an[kk]; b[kk] = bn[kk]; }
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] += acc1[v];
+            if (b0 + ln < B) {
+                float* o = out + (static_cast<size_t>(b0 + ln) * C + c) * T + 32 * ot + 4 * kh;
+#pragma unroll
+                for (int v4 = 0; v4 < 4; ++v4)
+                    *reinterpret_cast<float4*>(o + 8 * v4) = make_float4(acc[4 * v4], acc[4 * v4 + 1], acc[4 * v4 + 2], acc[4 * v4 + 3]);
+            }
+        }
+    }
+}
+
+// Kernel gradient summed over the batch: gws[c][T-1-lag] = sum_b sum_t g[b,c,t] k[b,c,t-lag], i.e. the sum of the lag-th
+// sub-diagonal of M = G^T K (contraction over the batch).  Batch rows are staged ROWS at a time; MFMA number kk contracts
+// rows 2kk and 2kk+1 (K slot = l >> 5), even and odd kk into separate accumulators so that consecutive MFMAs are
+// independent.  A wave owns whole lag tiles d (all tile pairs (tt, tt-d) accumulate into the same registers; d and
+// T/32-1-d together balance the triangle).  A finished tile goes through a per-wave LDS tile, from which lane l sums
+// diagonal l - 31 in row order and adds it to entry l of lag tile d, which no other wave touches: no atomics, every fp32
+// sum in a fixed order.
+constexpr int DIAG_STRIDE = 33;
+__host__ __device__ inline int gw_row_stride(int T) { return T + 32 - (T & 63); }      // = 32 mod 64: the two K halves of a read use different banks
+__host__ __device__ inline size_t gw_lds_floats(int T, int rows) {
+    return 2 * static_cast<size_t>(rows) * gw_row_stride(T) + 2 * static_cast<size_t>(T) + TXW * 32 * DIAG_STRIDE;
+}
+
+template <int ROWS>
+__global__ __launch_bounds__(TXT) void timex_gw_sum_mfma(const float* __restrict__ k, const float* __restrict__ g,
+                                                         float* __restrict__ gws, int B, int C, int T) {
+    extern __shared__ float lds[];
+    const int rs = gw_row_stride(T);
+    float* gr = lds;                           // [ROWS][rs]
+    float* kr = gr + ROWS * rs;                // [ROWS][rs]
+    float* diag = kr + ROWS * rs;              // [T/32 lag tiles][64]: entry l of tile d is the sum for lag 32 d + l - 31
+    const int c = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int ln = lane & 31, kh = lane >> 5;
+    const int nt = T >> 5, q4n = T >> 2;
+    for (int i = tid; i < 2 * T; i += TXT) diag[i] = 0.f;
+    float* tile = diag + 2 * T + wv * (32 * DIAG_STRIDE);         // [32 t][33]: one finished product tile
+
+    for (int b0 = 0; b0 < B; b0 += ROWS) {
+        __syncthreads();
+        const int total = ROWS * q4n;
+        for (int base = 0; base < total; base += (STG / 2) * TXT) {
+            float4 xg[STG / 2], xk[STG / 2];
+#pragma unroll
+            for (int s = 0; s < STG / 2; ++s) {
+                const int idx = base + s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
+                const bool live = idx < total && b0 + r < B;
+                const size_t off = (static_cast<size_t>(live ? b0 + r : b0) * C + c) * T + (live ? 4 * q4 : 0);
+                xg[s] = *reinterpret_cast<const float4*>(g + off);
+                xk[s] = *reinterpret_cast<const float4*>(k + off);
+            }
+#pragma unroll
+            for (int s = 0; s < STG / 2; ++s) {
+                const int idx = base + s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
+                if (idx < total) {
+                    const bool real = b0 + r < B;
+                    *reinterpret_cast<float4*>(gr + r * rs + 4 * q4) = real ? xg[s] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    *reinterpret_cast<float4*>(kr + r * rs + 4 * q4) = real ? xk[s] : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+        }
+        __syncthreads();
+        const float* ga = gr + kh * rs + ln;
+        const float* kb = kr + kh * rs + ln;
+        for (int p = wv; 2 * p < nt; p += TXW) {
+#pragma unroll 1
+            for (int side = 0; side < 2; ++side) {
+                const int d = side == 0 ? p : nt - 1 - p;
+                if (side == 1 && d == p) break;
+                f32x16 acc0, acc1;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.f;
+                constexpr int NK = ROWS / 2;
+                float a[NK], b[NK];
+                auto fetch = [&](int tt, float (&fa)[NK], float (&fb)[NK]) {
+#pragma unroll
+                    for (int kk = 0; kk < NK; ++kk) {
+                        fa[kk] = ga[2 * kk * rs + 32 * tt];
+                        fb[kk] = kb[2 * kk * rs + 32 * (tt - d)];
+                    }
+                };
+                fetch(d, a, b);
+                for (int tt = d; tt < nt; ++tt) {
+                    float an[NK], bn[NK];
+                    fetch(tt + 1 < nt ? tt + 1 : tt, an, bn);
+#pragma unroll
+                    for (int kk = 0; kk < NK; kk += 2) {
+                        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk], b[kk], acc0, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk + 1], b[kk + 1], acc1, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int kk = 0; kk < NK; ++kk) { a[kk] = an[kk]; b[kk] = bn[kk]; }
+                }
+                // accumulator v: t = 8 (v/4) + 4 kh + (v&3), u = ln, of tiles d apart
+#pragma unroll
+                for (int v = 0; v < 16; ++v) tile[(8 * (v >> 2) + 4 * kh + (v & 3)) * DIAG_STRIDE + ln] = acc0[v] + acc1[v];
+                const int dl = lane - 31;                   // diagonal t - u of this lane
+                float sum = 0.f;
+#pragma unroll
+                for (int t = 0; t < 32; ++t) {
+                    const int u = t - dl;
+                    const float x = tile[t * DIAG_STRIDE + (u & 31)];
+                    sum += (u >= 0 && u < 32) ? x : 0.f;
+                }
+                diag[64 * d + lane] += sum;                 // lag tile d belongs to this wave alone
+            }
+        }
+    }
+    __syncthreads();
+    for (int x = tid; x < T; x += TXT) {            // lag = 32 d + e comes from tile d (diagonal e) and tile d + 1 (diagonal e - 32)
+        const int lag = T - 1 - x, d = lag >> 5, e = lag & 31;
+        gws[static_cast<size_t>(c) * T + x] = diag[64 * d + 31 + e] + (d + 1 < nt ? diag[64 * (d + 1) + e - 1] : 0.f);
+    }
+}
+
 constexpr int T_MAX = 4096;
 
 int check_tx(int B, int C, int T) {
@@ -112,6 +311,10 @@ int check_tx(int B, int C, int T) {
     if ((B + BB - 1) / BB > 65535) return RWKV_ERR_SHAPE;
     return RWKV_OK;
 }
+
+// The matrix-core path pays off once the 32 columns of a product are mostly real batch rows.
+bool use_mfma(int B, int T) { return T % 32 == 0 && T <= T_MFMA_MAX && B >= 8; }
+size_t mfma_lds_bytes(int T) { return (static_cast<size_t>(T) + 32 + static_cast<size_t>(MROWS) * (T + 4)) * sizeof(float); }
 
 template <typename K> int raise_lds_limit(K kernel, size_t bytes) {
     if (bytes <= 48 * 1024) return RWKV_OK;
@@ -126,11 +329,34 @@ template <typename K> int raise_lds_limit(K kernel, size_t bytes) {
 
 using namespace rwkv;
 
+// gk = the mirrored convolution of gwk with w.
+int launch_gk(void* stream, const float* w, const float* gwk, float* gk, int B, int C, int T) {
+    if (use_mfma(B, T)) {
+        const size_t lds = mfma_lds_bytes(T);
+        if (int e = raise_lds_limit(timex_conv_mfma<true>, lds)) return e;
+        hipLaunchKernelGGL(timex_conv_mfma<true>, dim3(C, (B + MROWS - 1) / MROWS), dim3(TXT), lds,
+                           static_cast<hipStream_t>(stream), w, gwk, gk, 0.0f, B, C, T);
+    } else {
+        const size_t lds = (static_cast<size_t>(BB + 1) * T + 4) * sizeof(float);
+        if (int e = raise_lds_limit(timex_conv<true>, lds)) return e;
+        hipLaunchKernelGGL(timex_conv<true>, dim3(C, (B + BB - 1) / BB), dim3(T / 4), lds,
+                           static_cast<hipStream_t>(stream), w, gwk, gk, 0.0f, B, C, T);
+    }
+    return RWKV_OK;
+}
+
 extern "C" {
 
 int rwkv_timex_forward(void* stream, const float* w, const float* k, float* x, float eps, int B, int C, int T) {
     if (int e = check_tx(B, C, T)) return e;
     if (int e = check_ptrs({w, k, x})) return e;
+    if (use_mfma(B, T)) {
+        const size_t lds = mfma_lds_bytes(T);
+        if (int e = raise_lds_limit(timex_conv_mfma<false>, lds)) return e;
+        hipLaunchKernelGGL(timex_conv_mfma<false>, dim3(C, (B + MROWS - 1) / MROWS), dim3(TXT), lds,
+                           static_cast<hipStream_t>(stream), w, k, x, eps, B, C, T);
+        return launch_status();
+    }
     const size_t lds = (static_cast<size_t>(BB + 1) * T + 4) * sizeof(float);
     if (int e = raise_lds_limit(timex_conv<false>, lds)) return e;
     hipLaunchKernelGGL(timex_conv<false>, dim3(C, (B + BB - 1) / BB), dim3(T / 4), lds,
@@ -143,12 +369,23 @@ int rwkv_timex_backward(void* stream, const float* w, const float* k, const floa
     if (int e = check_tx(B, C, T)) return e;
     if (int e = check_ptrs({w, k, gwk, gw, gk})) return e;
     if (static_cast<long long>(B) * C > 0x7fffffffLL) return RWKV_ERR_SHAPE;
-    const size_t lds = (static_cast<size_t>(BB + 1) * T + 4) * sizeof(float);
-    if (int e = raise_lds_limit(timex_conv<true>, lds)) return e;
-    hipLaunchKernelGGL(timex_conv<true>, dim3(C, (B + BB - 1) / BB), dim3(T / 4), lds,
-                       static_cast<hipStream_t>(stream), w, gwk, gk, 0.0f, B, C, T);
+    if (int e = launch_gk(stream, w, gwk, gk, B, C, T)) return e;
     hipLaunchKernelGGL(timex_gw, dim3(B * C), dim3(T / 4), (2 * static_cast<size_t>(T) + 4) * sizeof(float),
                        static_cast<hipStream_t>(stream), k, gwk, gw, T);
+    return launch_status();
+}
+
+int rwkv_timex_backward_sum(void* stream, const float* w, const float* k, const float* gwk, float* gw_sum, float* gk,
+                            int B, int C, int T) {
+    if (int e = check_tx(B, C, T)) return e;
+    if (T % 32 != 0 || T > T_MFMA_MAX) return RWKV_ERR_SHAPE;
+    if (int e = check_ptrs({w, k, gwk, gw_sum, gk})) return e;
+    const bool wide = T <= 768;                 // 16 batch rows per pass while they fit in LDS, else 8
+    const size_t lds_gw = gw_lds_floats(T, wide ? 16 : 8) * sizeof(float);
+    auto kernel = wide ? timex_gw_sum_mfma<16> : timex_gw_sum_mfma<8>;
+    if (int e = raise_lds_limit(kernel, lds_gw)) return e;
+    if (int e = launch_gk(stream, w, gwk, gk, B, C, T)) return e;
+    hipLaunchKernelGGL(kernel, dim3(C), dim3(TXT), lds_gw, static_cast<hipStream_t>(stream), k, gwk, gw_sum, B, C, T);
     return launch_status();
 }
 

@@ -5,6 +5,7 @@ import torch
 from ._call import call, check_tensors, require
 
 T_MAX = 4096
+T_SUM_MAX = 1024      # rwkv_timex_backward_sum: T % 32 == 0 and T <= 1024
 
 
 class TimeX(torch.autograd.Function):
@@ -28,8 +29,12 @@ class TimeX(torch.autograd.Function):
         w, k = ctx.saved_tensors
         gwk = gwk.contiguous()
         dev = check_tensors((gwk,), torch.float32, ("gwk",))
-        gw = torch.empty((ctx.B, ctx.C, ctx.T), device=dev, dtype=torch.float32)
         gk = torch.empty((ctx.B, ctx.C, ctx.T), device=dev, dtype=torch.float32)
+        if ctx.T % 32 == 0 and ctx.T <= T_SUM_MAX:       # the sum over the batch of run.py:102 happens in the kernel
+            gw = torch.empty((ctx.C, ctx.T), device=dev, dtype=torch.float32)
+            call("rwkv_timex_backward_sum", dev, w, k, gwk, gw, gk, ctx.B, ctx.C, ctx.T)
+            return (gw, gk, None, None, None, None)
+        gw = torch.empty((ctx.B, ctx.C, ctx.T), device=dev, dtype=torch.float32)
         call("rwkv_timex_backward", dev, w, k, gwk, gw, gk, ctx.B, ctx.C, ctx.T)
         return (gw.sum(dim=0), gk, None, None, None, None)
 

@@ -20,7 +20,7 @@ def _declared_symbols():
 
 def test_header_and_bindings_agree(lib):
     names = _declared_symbols()
-    assert len(names) == 23
+    assert len(names) == 24
     assert sorted(_lib.SIGNATURES) == names
     for n in names:
         assert hasattr(lib, n), f"{n} declared in rwkv_hip.h but not exported"

@@ -51,7 +51,7 @@ def test_wkv4_extreme_k_stays_finite(lib):
     assert e < 1e-3
 
 
-@pytest.mark.parametrize("B,C,T", [(3, 5, 64), (9, 2, 4), (32, 768, 768)])
+@pytest.mark.parametrize("B,C,T", [(3, 5, 64), (9, 2, 4), (40, 3, 96), (17, 2, 1024), (32, 768, 768)])
 def test_timex(lib, B, C, T):
     print(f"\ntimex B={B} C={C} T={T}", flush=True)
     w, k, g = synth.timex_inputs(B, C, T, seed=23)
@@ -68,6 +68,15 @@ def test_timex(lib, B, C, T):
     _check("x", ref[0] + eps, x[:, cs])
     _check("gw", ref[1], gw.sum(0)[cs])
     _check("gk", ref[2], gk[:, cs])
+    if T % 32 == 0 and T <= 1024:             # the entry point that sums gw over the batch itself
+        gws = garbage((C, T), torch.float32)
+        gk2 = garbage((B, C, T), torch.float32)
+        call("rwkv_timex_backward_sum", d[0].device, d[0], d[1], d[2], gws, gk2, B, C, T)
+        again = garbage((C, T), torch.float32)
+        call("rwkv_timex_backward_sum", d[0].device, d[0], d[1], d[2], again, gk2, B, C, T)
+        torch.cuda.synchronize()
+        _check("gw summed in the kernel", ref[1], gws[cs])
+        assert torch.equal(gk2, gk) and torch.equal(gws, again)
     if T <= 64:                               # per-batch gw against the closed form
         gwb, _ = OT.grads_closed_form(w.double(), k.double(), g.double(), B, C, T)
         _check("gw per batch", gwb, gw)
