@@ -7,6 +7,7 @@ PyTorch fallback: if the library cannot be loaded the import of an op fails loud
 
 import ctypes
 import os
+import re
 import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -22,7 +23,15 @@ HIPCC_FLAGS = [
     # packed fp32 VALU ops stay off on this target
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # per-kernel register / scratch report on stderr, parsed by build()
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+
+# The prep waves of these kernels load through inline asm and wait with a hand-counted vmcnt, so the compiler does not
+# know when such a register is valid: a spill of one of them (they have the longest live ranges) would save garbage.
+# The backward sweep B keeps one index of its state waves' epilogue in scratch, outside the loops; anything beyond
+# these counts fails the build.
+SPILL_LIMIT = {"wkv6_fwd_ws": 0, "wkv6_bwd_a_ws": 0, "wkv6_bwd_b_ws": 1}
 
 _lib = None
 
@@ -35,9 +44,21 @@ def build(verbose=False):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in res.stdout.splitlines() if "is not a recognized feature" not in l)
+    lines = res.stdout.splitlines()
+    out = "\n".join(l for l in lines if "is not a recognized feature" not in l and "kernel-resource-usage" not in l)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + out)
+    kernel = None
+    for l in lines:
+        m = re.search(r"remark: Function Name: (\S+)", l)
+        if m:
+            kernel = m.group(1)
+        m = re.search(r"remark:\s+VGPRs Spill: (\d+)", l)
+        if m and kernel:
+            for name, limit in SPILL_LIMIT.items():
+                if name in kernel and int(m.group(1)) > limit:
+                    os.remove(LIB_PATH)
+                    raise RuntimeError(f"{kernel}: {m.group(1)} spilled VGPRs (limit {limit}); its asm-loaded registers must stay in registers")
     if verbose and out.strip():
         print(out, flush=True)
     return LIB_PATH

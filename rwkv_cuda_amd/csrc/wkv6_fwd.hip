@@ -64,8 +64,10 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         uj[0] = bf_lo(x); uj[1] = bf_hi(x);
     }
     struct Raw { uint32_t r[2], k[2], v[2], w[2][WMODE == W_EW ? 2 : 1]; float lam[2][2], other[2], kp[2][2]; };
-    Raw ring[STAGES];
-    // The loads of a chunk are issued STAGES chunks before they are used.  They are written as asm so that the wait before
+    // fp32 decays take two more registers per token: one stage less keeps the ring in registers
+    constexpr int NST = WMODE == W_EW ? STAGES - 1 : STAGES;
+    Raw ring[NST];
+    // The loads of a chunk are issued NST chunks before they are used.  They are written as asm so that the wait before
     // the first use can name the number of younger loads that may still be in flight (the compiler would wait for all of
     // them); every call issues the same eight loads (chunk index clamped), which keeps that number fixed.
     const uint32_t* __restrict__ wb32 = reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + base);
@@ -107,11 +109,35 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         const float2 e2 = *reinterpret_cast<const float2*>(static_cast<const float*>(a.w) + h * N + 2 * jp);
         lamc[0] = __builtin_amdgcn_logf(e2.x); lamc[1] = __builtin_amdgcn_logf(e2.y);
     }
-    static_for<STAGES>([&](auto Z) { prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
+    // wkv5: every full chunk has the same factors, computed here once; a last, partial chunk takes the general route.
+    // Tokens between this thread's pair and the middle of the chunk: 14 - pt0 in the first half, pt0 - 16 in the second.
+    Scale sc_head[2] = {};
+    bool exact_head = false;
+    if constexpr (WMODE == W_HEAD) {
+        const float between = static_cast<float>(second ? pt0 - 16 : 14 - pt0);
+        sc_head[0] = chunk_scale(second, between * lamc[0], lamc[0], lamc[0]);
+        sc_head[1] = chunk_scale(second, between * lamc[1], lamc[1], lamc[1]);
+        const bool fast_decay = (-4.f * lamc[0] > 0.25f * RANGE_LIMIT * LOG2E) || (-4.f * lamc[1] > 0.25f * RANGE_LIMIT * LOG2E);
+        exact_head = __ballot(fast_decay) != 0ull;
+        if (wid == 3 && th == 0)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) {
+                *reinterpret_cast<float2*>(&S.set[pb].d1[2 * jp]) = make_float2(exp2_fast(16.f * lamc[0]), exp2_fast(16.f * lamc[1]));
+                *reinterpret_cast<float2*>(&S.set[pb].d2[2 * jp]) = make_float2(exp2_fast(16.f * lamc[0]), exp2_fast(16.f * lamc[1]));
+                *reinterpret_cast<float2*>(&S.set[pb].dec[2 * jp]) = make_float2(exp2_fast(32.f * lamc[0]), exp2_fast(32.f * lamc[1]));
+            }
+    }
+    auto head_full = [&](const int c) __attribute__((always_inline)) { return WMODE == W_HEAD && c * L + L <= T; };
+    static_for<NST>([&](auto Z) { prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
 
     // ---- scan of chunk c: lam (log2 units) of this thread's four elements, sums over each eighth of the chunk
     auto scan = [&](const int c, Raw& x) __attribute__((always_inline)) {
         const int c0 = c * L, pb = c & 1;
+        if (head_full(c)) {
+#pragma unroll
+            for (int e = 0; e < 2; ++e) { x.lam[e][0] = lamc[0]; x.lam[e][1] = lamc[1]; }
+            return;
+        }
         if (c0 + L > T) {                              // last, partial chunk: rows past T carry no input and no decay
 #pragma unroll
             for (int e = 0; e < 2; ++e)
@@ -149,17 +175,19 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
     auto operands_a = [&](const int c, Raw& x) __attribute__((always_inline)) -> bool {
         OperandSet& O = S.set[c & 1];
         const int pb = c & 1;
-        const uint2 f8 = *reinterpret_cast<const uint2*>(&S.flag[pb][0]);
-        // sums of lam over the eighths of this thread's half-chunk; those between this wave's eighth and the middle count
-        float2 pe[4];
+        const bool hf = head_full(c);
+        bool exact = exact_head;
+        float near[2] = {0.f, 0.f};
+        if (!hf) {
+            const uint2 f8 = *reinterpret_cast<const uint2*>(&S.flag[pb][0]);
+            // sums of lam over the eighths of this thread's half-chunk; those between this wave's eighth and the middle count
+            float2 pe[4];
 #pragma unroll
-        for (int w4 = 0; w4 < 4; ++w4) pe[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * second + w4][2 * jp]);
-        const bool exact = __builtin_amdgcn_readfirstlane(f8.x | f8.y) != 0;     // the same in every wave: a scalar
-        if (tid == 0) O.exact = exact;
-        float near[2];
-        near[0] = second ? (th ? x.other[0] : 0.f) : (th ? 0.f : x.other[0]);
-        near[1] = second ? (th ? x.other[1] : 0.f) : (th ? 0.f : x.other[1]);
-        {   // eighths between this wave's and the middle: first half w_own+1..3, second half 0..w_own-1 (scalar branches)
+            for (int w4 = 0; w4 < 4; ++w4) pe[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * second + w4][2 * jp]);
+            exact = __builtin_amdgcn_readfirstlane(f8.x | f8.y) != 0;            // the same in every wave: a scalar
+            near[0] = second ? (th ? x.other[0] : 0.f) : (th ? 0.f : x.other[0]);
+            near[1] = second ? (th ? x.other[1] : 0.f) : (th ? 0.f : x.other[1]);
+            // eighths between this wave's and the middle: first half w_own+1..3, second half 0..w_own-1 (scalar branches)
             const int w_own = wid & 3;
             const int lo = second ? 0 : w_own + 1, hi = second ? w_own : 4;
             if (lo <= 0 && 0 < hi) { near[0] += pe[0].x; near[1] += pe[0].y; }
@@ -167,6 +195,7 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
             if (lo <= 2 && 2 < hi) { near[0] += pe[2].x; near[1] += pe[2].y; }
             if (lo <= 3 && 3 < hi) { near[0] += pe[3].x; near[1] += pe[3].y; }
         }
+        if (tid == 0) O.exact = exact;
         float pr[2][2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) { pr[e][0] = bf_lo(x.r[e]); pr[e][1] = bf_hi(x.r[e]); }
@@ -174,7 +203,7 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
             float rp[2][2];
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
-                const Scale sc = chunk_scale(second, near[z], x.lam[0][z], x.lam[1][z]);
+                const Scale sc = hf ? sc_head[z] : chunk_scale(second, near[z], x.lam[0][z], x.lam[1][z]);
                 rp[0][z] = pr[0][z] * sc.ea[0]; rp[1][z] = pr[1][z] * sc.ea[1];
                 x.kp[0][z] = (z ? bf_hi(x.k[0]) : bf_lo(x.k[0])) * sc.eb[0];
                 x.kp[1][z] = (z ? bf_hi(x.k[1]) : bf_lo(x.k[1])) * sc.eb[1];
@@ -216,7 +245,7 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         }
         O.V[pt0][jp] = x.v[0];
         O.V[pt0 + 1][jp] = x.v[1];
-        if (wid == 3 && th == 0) {
+        if (wid == 3 && th == 0 && !head_full(c)) {
             float cm[2] = {0.f, 0.f}, ch[2] = {0.f, 0.f};
 #pragma unroll
             for (int w8 = 0; w8 < 4; ++w8) {
@@ -257,30 +286,30 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         *reinterpret_cast<uint2*>(&S.AmL[c & 1][16 * ta + l16][4 * g + 2 * tb]) = make_uint2(x0.l, x1.l);
     };
 
-    static_for<STAGES>([&](auto Z) { arrived(ring[decltype(Z)::value], std::integral_constant<int, 0>{}); });
+    static_for<NST>([&](auto Z) { arrived(ring[decltype(Z)::value], std::integral_constant<int, 0>{}); });
     scan(0, ring[0]);
     if (nchunks > 1) scan(1, ring[1]);
     __syncthreads();
     bool exact_cur = operands_a(0, ring[0]);
     operands_b(0, ring[0], exact_cur);
-    prefetch(STAGES, ring[0]);
+    prefetch(NST, ring[0]);
     __syncthreads();
     // iteration i: scan(i+2), tile(i), operands(i+1); one barrier
-    for (int ib = 0; ib < nchunks; ib += STAGES)
-        static_for<STAGES>([&](auto Z) {
+    for (int ib = 0; ib < nchunks; ib += NST)
+        static_for<NST>([&](auto Z) {
             constexpr int z = decltype(Z)::value;
             const int i = ib + z;
             if (i < nchunks) {
                 // younger than the loads of chunk i+2: those of chunks i+3 and i+4
-                arrived(ring[(z + 2) % STAGES], std::integral_constant<int, STAGES - 2>{});
-                if (i + 2 < nchunks) scan(i + 2, ring[(z + 2) % STAGES]);
+                arrived(ring[(z + 2) % NST], std::integral_constant<int, NST - 2>{});
+                if (i + 2 < nchunks) scan(i + 2, ring[(z + 2) % NST]);
                 if (wid < 3 && !exact_cur) tile(i);
                 bool exact_next = false;
                 if (i + 1 < nchunks) {
-                    exact_next = operands_a(i + 1, ring[(z + 1) % STAGES]);
-                    operands_b(i + 1, ring[(z + 1) % STAGES], exact_next);
+                    exact_next = operands_a(i + 1, ring[(z + 1) % NST]);
+                    operands_b(i + 1, ring[(z + 1) % NST], exact_next);
                 }
-                prefetch(i + 1 + STAGES, ring[(z + 1) % STAGES]);
+                prefetch(i + 1 + NST, ring[(z + 1) % NST]);
                 __syncthreads();
                 exact_cur = exact_next;
             }
