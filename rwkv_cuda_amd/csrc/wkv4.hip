@@ -45,6 +45,85 @@ __global__ __launch_bounds__(NT) void wkv4_fwd(int BC, int T, int C, const float
     }
 }
 
+// ---------------------------------------------------------------------------------------------------- time-parallel form
+// B*C scans of T dependent steps leave most of the chip idle (3072 lanes at B4 C768), so the time axis is cut into NSEG
+// segments that run side by side: a workgroup takes CH channels of one batch row, thread (channel, segment).
+//   1. every segment scans its own steps from the empty state: (p, q, o) of the segment alone;
+//   2. a Kogge-Stone scan over the segments combines them: a state that is n steps older enters with its exponent
+//      lowered by n w (the decay is the same at every step), so after log2(NSEG) rounds segment s knows the state in
+//      front of its first step;
+//   3. every segment repeats its steps from that state and writes the outputs.
+// The formulas of a step are those of the sequential kernel; only the order in which partial sums meet differs.
+constexpr int CH = 16, NSEG = 64, NTS = CH * NSEG;
+struct State3 { float p, q, o; };
+
+// a: the older state, exponent already lowered by the decay over the steps of b
+DEVINL State3 combine(const State3 a, const State3 b) {
+    const float no = fmaxf(a.o, b.o);
+    const float ea = expf(a.o - no), eb = expf(b.o - no);
+    return {ea * a.p + eb * b.p, ea * a.q + eb * b.q, no};
+}
+
+__global__ __launch_bounds__(NTS) void wkv4_fwd_seg(int T, int C, int S, const float* __restrict__ w_,
+                                                   const float* __restrict__ u_, const float* __restrict__ k_,
+                                                   const float* __restrict__ v_, float* __restrict__ y_) {
+    __shared__ State3 X[2][NSEG][CH];
+    const int cl = threadIdx.x % CH, s = threadIdx.x / CH;
+    const int c = blockIdx.x * CH + cl, b = blockIdx.y;
+    const bool live = c < C;
+    const int cc = live ? c : C - 1;
+    const size_t off = static_cast<size_t>(b) * T * C + cc;
+    const float u = u_[cc], w = w_[cc];
+    const float* __restrict__ k = k_ + off;
+    const float* __restrict__ v = v_ + off;
+    float* __restrict__ y = y_ + off;
+    const int t0 = min(s * S, T), t1 = min(t0 + S, T);
+
+    State3 x = {0.f, 0.f, O_INIT};
+    for (int t = t0; t < t1; ++t) {
+        const size_t ii = static_cast<size_t>(t) * C;
+        const float kt = k[ii], vt = v[ii];
+        const float no = fmaxf(w + x.o, kt);
+        const float A = expf(w + x.o - no), Bq = expf(kt - no);
+        x.p = A * x.p + Bq * vt;
+        x.q = A * x.q + Bq;
+        x.o = no;
+    }
+    // Inclusive scan.  Every span is taken as full segments of S steps: only the last live segment can be shorter, and
+    // the prefixes that contain it are needed by nobody.
+    X[0][s][cl] = x;
+    __syncthreads();
+    int cur = 0;
+#pragma unroll
+    for (int d = 1; d < NSEG; d *= 2) {
+        State3 mine = X[cur][s][cl];
+        if (s >= d) {
+            State3 older = X[cur][s - d][cl];
+            older.o += static_cast<float>(d * S) * w;
+            mine = combine(older, mine);
+        }
+        X[cur ^ 1][s][cl] = mine;
+        cur ^= 1;
+        __syncthreads();
+    }
+    x = State3{0.f, 0.f, O_INIT};
+    if (s > 0) x = X[cur][s - 1][cl];
+
+    for (int t = t0; t < t1; ++t) {
+        const size_t ii = static_cast<size_t>(t) * C;
+        const float kt = k[ii], vt = v[ii];
+        float no = fmaxf(x.o, u + kt);
+        float A = expf(x.o - no), Bq = expf(u + kt - no);
+        if (live) y[ii] = (A * x.p + Bq * vt) / (A * x.q + Bq);
+        no = fmaxf(w + x.o, kt);
+        A = expf(w + x.o - no);
+        Bq = expf(kt - no);
+        x.p = A * x.p + Bq * vt;
+        x.q = A * x.q + Bq;
+        x.o = no;
+    }
+}
+
 __global__ __launch_bounds__(NT) void wkv4_bwd(int BC, int T, int C, const float* __restrict__ w_,
                                               const float* __restrict__ u_, const float* __restrict__ k_,
                                               const float* __restrict__ v_, const float* __restrict__ gy_,
@@ -110,6 +189,164 @@ __global__ __launch_bounds__(NT) void wkv4_bwd(int BC, int T, int C, const float
     gu_[static_cast<size_t>(b) * C + c] += gu;
 }
 
+// Backward in the same time-parallel form.  The ascending sweep also carries dp/dw and dq/dw; a state that is n steps
+// older enters with (dp, dq) <- (n p + dp, n q + dq) besides the lowered exponent, since P_{t+n} = e^{n w} P_t + ...
+// gives dP_{t+n}/dw = e^{n w} (n P_t + dP_t/dw) + ...  The descending sweep is a scan of the same kind run from the last
+// segment to the first (only the last live segment can be shorter than S, and there it is always the older operand).
+struct State5 { float p, q, dp, dq, o; };
+
+DEVINL State5 combine(const State5 a, const State5 b) {
+    const float no = fmaxf(a.o, b.o);
+    const float ea = expf(a.o - no), eb = expf(b.o - no);
+    return {ea * a.p + eb * b.p, ea * a.q + eb * b.q, ea * a.dp + eb * b.dp, ea * a.dq + eb * b.dq, no};
+}
+
+__global__ __launch_bounds__(NTS) void wkv4_bwd_seg(int T, int C, int S, const float* __restrict__ w_,
+                                                   const float* __restrict__ u_, const float* __restrict__ k_,
+                                                   const float* __restrict__ v_, const float* __restrict__ gy_,
+                                                   float* __restrict__ gw_, float* __restrict__ gu_,
+                                                   float* __restrict__ gk_, float* __restrict__ gv_,
+                                                   float* __restrict__ ws_) {
+    __shared__ State5 X[2][NSEG][CH];
+    const int cl = threadIdx.x % CH, s = threadIdx.x / CH;
+    const int c = blockIdx.x * CH + cl, b = blockIdx.y;
+    const bool live = c < C;
+    const int cc = live ? c : C - 1;
+    const size_t off = static_cast<size_t>(b) * T * C + cc;
+    const float u = u_[cc], w = w_[cc];
+    const float* __restrict__ k = k_ + off;
+    const float* __restrict__ v = v_ + off;
+    const float* __restrict__ gy = gy_ + off;
+    float* __restrict__ gk = gk_ + off;      // holds z_t until the descending sweep overwrites it
+    float* __restrict__ gv = gv_ + off;      // holds y_t
+    float* __restrict__ ze = ws_ + off;      // zexp_t
+    // lanes past C have no steps: they only keep the barriers company
+    const int t0 = live ? min(s * S, T) : T, t1 = min(t0 + S, T);
+    const float span = static_cast<float>(S);
+
+    // ---- ascending: the segment alone
+    State5 x = {0.f, 0.f, 0.f, 0.f, O_INIT};
+    for (int t = t0; t < t1; ++t) {
+        const size_t ii = static_cast<size_t>(t) * C;
+        const float kt = k[ii], vt = v[ii];
+        const float no = fmaxf(w + x.o, kt);
+        const float A = expf(w + x.o - no), Bq = expf(kt - no);
+        x.dp = A * (x.p + x.dp);
+        x.dq = A * (x.q + x.dq);
+        x.p = A * x.p + Bq * vt;
+        x.q = A * x.q + Bq;
+        x.o = no;
+    }
+    X[0][s][cl] = x;
+    __syncthreads();
+    int cur = 0;
+#pragma unroll
+    for (int d = 1; d < NSEG; d *= 2) {
+        State5 mine = X[cur][s][cl];
+        if (s >= d) {
+            State5 older = X[cur][s - d][cl];
+            const float n = static_cast<float>(d) * span;
+            older.dp += n * older.p;
+            older.dq += n * older.q;
+            older.o += n * w;
+            mine = combine(older, mine);
+        }
+        X[cur ^ 1][s][cl] = mine;
+        cur ^= 1;
+        __syncthreads();
+    }
+    x = State5{0.f, 0.f, 0.f, 0.f, O_INIT};
+    if (s > 0) x = X[cur][s - 1][cl];
+    __syncthreads();                               // X is reused below
+
+    // ---- ascending, from the true state: y, 1/den and zexp are parked for the descending sweep
+    float gw = 0.f, gu = 0.f;
+    for (int t = t0; t < t1; ++t) {
+        const size_t ii = static_cast<size_t>(t) * C;
+        const float kt = k[ii], vt = v[ii], gt = gy[ii];
+        float no = fmaxf(x.o, kt + u);
+        float A = expf(x.o - no), Bq = expf(kt + u - no);
+        const float num = A * x.p + Bq * vt;
+        const float iden = 1.0f / (A * x.q + Bq);
+        const float y = num * iden;
+        gv[ii] = y;
+        gk[ii] = iden;
+        ze[ii] = kt + u - no;
+        gw += gt * (x.dp - x.dq * y) * iden * A;
+        gu += gt * (vt - y) * Bq * iden;
+        no = fmaxf(w + x.o, kt);
+        A = expf(w + x.o - no);
+        Bq = expf(kt - no);
+        x.dp = A * (x.p + x.dp);
+        x.dq = A * (x.q + x.dq);
+        x.p = A * x.p + Bq * vt;
+        x.q = A * x.q + Bq;
+        x.o = no;
+    }
+
+    // ---- descending: the segment alone (p, q stand for gp, gq)
+    State3 g = {0.f, 0.f, O_INIT};
+    for (int t = t1 - 1; t >= t0; --t) {
+        const size_t ii = static_cast<size_t>(t) * C;
+        const float kt = k[ii], gt = gy[ii];
+        const float y = gv[ii], z = gk[ii], zexp = ze[ii];
+        const float no = fmaxf(w + g.o, zexp - kt - u);
+        const float A = expf(w + g.o - no), Bq = gt * z * expf(zexp - kt - u - no);
+        g.p = A * g.p + Bq;
+        g.q = A * g.q - Bq * y;
+        g.o = no;
+    }
+    State3 (*G)[NSEG][CH] = reinterpret_cast<State3 (*)[NSEG][CH]>(&X[0][0][0]);    // [2][NSEG][CH], inside X
+    const int rs = NSEG - 1 - s;                   // position in the descending order
+    G[0][rs][cl] = g;
+    __syncthreads();
+    cur = 0;
+#pragma unroll
+    for (int d = 1; d < NSEG; d *= 2) {
+        State3 mine = G[cur][rs][cl];
+        if (rs >= d) {
+            State3 older = G[cur][rs - d][cl];
+            older.o += static_cast<float>(d) * span * w;
+            mine = combine(older, mine);
+        }
+        G[cur ^ 1][rs][cl] = mine;
+        cur ^= 1;
+        __syncthreads();
+    }
+    g = State3{0.f, 0.f, O_INIT};
+    if (rs > 0) g = G[cur][rs - 1][cl];
+    __syncthreads();
+
+    // ---- descending, from the true state
+    for (int t = t1 - 1; t >= t0; --t) {
+        const size_t ii = static_cast<size_t>(t) * C;
+        const float kt = k[ii], vt = v[ii], gt = gy[ii];
+        const float y = gv[ii], z = gk[ii], zexp = ze[ii];
+        float A = gt * z * expf(zexp);
+        float Bq = expf(kt + g.o);
+        gk[ii] = A * (vt - y) + Bq * (g.p * vt + g.q);
+        gv[ii] = A + Bq * g.p;
+        const float no = fmaxf(w + g.o, zexp - kt - u);
+        A = expf(w + g.o - no);
+        Bq = gt * z * expf(zexp - kt - u - no);
+        g.p = A * g.p + Bq;
+        g.q = A * g.q - Bq * y;
+        g.o = no;
+    }
+
+    // ---- gw, gu: the segments' sums, added in time order
+    float2* part = reinterpret_cast<float2*>(&X[0][0][0]);                         // [NSEG][CH]
+    part[s * CH + cl] = make_float2(gw, gu);
+    __syncthreads();
+    if (s == 0 && live) {
+        float a = 0.f, bsum = 0.f;
+        for (int z = 0; z < NSEG; ++z) { a += part[z * CH + cl].x; bsum += part[z * CH + cl].y; }
+        // the caller's buffers are accumulated into, as the reference does (wkv_cuda_v2.cu:112-113)
+        gw_[static_cast<size_t>(b) * C + c] += a * w;
+        gu_[static_cast<size_t>(b) * C + c] += bsum;
+    }
+}
+
 int check4(int B, int T, int C) {
     if (B <= 0 || T <= 0 || C <= 0) return RWKV_ERR_SHAPE;
     if (static_cast<long long>(B) * C > 0x7fffffffLL) return RWKV_ERR_SHAPE;
@@ -127,9 +364,14 @@ int rwkv_wkv4_forward(void* stream, int B, int T, int C, const float* w, const f
                       const float* v, float* y) {
     if (int e = check4(B, T, C)) return e;
     if (int e = check_ptrs({w, u, k, v, y})) return e;
-    const int BC = B * C;
-    hipLaunchKernelGGL(wkv4_fwd, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
-                       BC, T, C, w, u, k, v, y);
+    if (B > 65535) {                            // beyond the grid's y range: the one-lane-per-scan kernel
+        const int BC = B * C;
+        hipLaunchKernelGGL(wkv4_fwd, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
+                           BC, T, C, w, u, k, v, y);
+        return launch_status();
+    }
+    hipLaunchKernelGGL(wkv4_fwd_seg, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
+                       T, C, (T + NSEG - 1) / NSEG, w, u, k, v, y);
     return launch_status();
 }
 
@@ -145,9 +387,14 @@ int rwkv_wkv4_backward(void* stream, int B, int T, int C, const float* w, const 
     if (int e = check_ptrs({w, u, k, v, gy, gw, gu, gk, gv})) return e;
     if (workspace == nullptr || !aligned16(workspace) || workspace_bytes < rwkv_wkv4_backward_workspace_bytes(B, T, C))
         return RWKV_ERR_WORKSPACE;
-    const int BC = B * C;
-    hipLaunchKernelGGL(wkv4_bwd, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
-                       BC, T, C, w, u, k, v, gy, gw, gu, gk, gv, static_cast<float*>(workspace));
+    if (B > 65535) {                            // beyond the grid's y range: the one-lane-per-scan kernel
+        const int BC = B * C;
+        hipLaunchKernelGGL(wkv4_bwd, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
+                           BC, T, C, w, u, k, v, gy, gw, gu, gk, gv, static_cast<float*>(workspace));
+        return launch_status();
+    }
+    hipLaunchKernelGGL(wkv4_bwd_seg, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
+                       T, C, (T + NSEG - 1) / NSEG, w, u, k, v, gy, gw, gu, gk, gv, static_cast<float*>(workspace));
     return launch_status();
 }
 
