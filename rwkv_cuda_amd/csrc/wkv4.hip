@@ -1,5 +1,4 @@
-// RWKV-4 wkv, fp32, gfx950.  One lane per (batch, channel); lanes of a wave are 64 consecutive
-// channels so every step reads and writes 256 contiguous bytes per tensor.
+// RWKV-4 wkv, fp32, gfx950.
 //
 //   y_t = (e^{o-no} p + e^{u+k_t-no} v_t) / (e^{o-no} q + e^{u+k_t-no}),  no = max(o, u+k_t)
 //   (p,q,o) <- decay by w and add e^{k_t}(v_t, 1), renormalised to the new running maximum o.
@@ -7,6 +6,9 @@
 // sweep must hand to the descending one (y_t, z_t = 1/den_t, zexp_t) is parked in the gv and gk
 // output buffers and in a caller-provided workspace instead of per-thread local arrays, so T is
 // not limited.
+// Two forms of each kernel: the time-parallel one used by the entry points (segments of the time axis
+// side by side, joined by a scan of their states) and the plain one lane per (batch, channel) form,
+// whose lanes of a wave are 64 consecutive channels (256 contiguous bytes per tensor and step).
 #include <math.h>
 
 #include "common.h"
