@@ -110,14 +110,16 @@ __global__ __launch_bounds__(1024) void timex_gw(const float* __restrict__ k, co
 // v_mfma_f32_32x32x2_f32 (lane = (row or column l & 31, K slot half l >> 5); accumulator register v: row 8 (v/4) + 4 (l>>5)
 // + (v&3), column l & 31).  The kernel row is stored in tap order followed by 32 zeros, so a tap of negative lag reads 0
 // and the diagonal block needs no mask.  Output tile o of 32 time steps sums over input tiles 0..o (mirror: o..T/32-1);
-// a wave takes tiles p and T/32-1-p, which balances the triangle.  K slot (half, kk) is input step 16 half + kk of the
+// wave p takes tiles p and T/32-1-p (and p + 8, ...), which balances the triangle.  K slot (half, kk) is input step 16 half + kk of the
 // tile, so a lane reads its 16 B operands as four 16-byte LDS reads.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr int MROWS = 32;              // batch rows per workgroup = columns of the product
 constexpr int T_MFMA_MAX = 1024;
 constexpr int TXW = 8;                 // waves per workgroup: two per SIMD, one reads LDS while the other runs MFMAs
 constexpr int TXT = 64 * TXW;
-constexpr int STG = 4;                 // 16-byte global loads in flight per thread while staging
+constexpr int STG = 4;
+constexpr int PFQ = MROWS * (T_MFMA_MAX / 4) / TXT;     // 16-byte pieces of a unit's rows per thread, at the longest T
+constexpr int NCU = 256;               // workgroups of the persistent kernels: one per CU                 // 16-byte global loads in flight per thread while staging
 
 template <bool MIRROR>
 __global__ __launch_bounds__(TXT) void timex_conv_mfma(const float* __restrict__ w, const float* __restrict__ in,
@@ -126,76 +128,96 @@ __global__ __launch_bounds__(TXT) void timex_conv_mfma(const float* __restrict__
     float* wp = lds;                   // [T + 32]: wp[x] = w[c][x] (tap order), 0 for x >= T
     float* rows = lds + T + 32;        // [32][T + 4]
     const int rs = T + 4;
-    const int c = blockIdx.x, b0 = blockIdx.y * MROWS, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int ln = lane & 31, kh = lane >> 5;
-
-    for (int i = tid; i < T + 32; i += TXT) wp[i] = i < T ? w[static_cast<size_t>(c) * T + i] : 0.f;
-    // rows come in with STG 16-byte loads in flight per thread: one block per CU has nothing else to hide HBM latency with
-    const int q4n = T >> 2, total = MROWS * q4n;
-    for (int base = 0; base < total; base += STG * TXT) {
-        float4 x[STG];
+    const int q4n = T >> 2, total = MROWS * q4n, nt = T >> 5;
+    // A workgroup walks over units (channel, group of 32 batch rows).  One workgroup fills a CU, so nothing else hides the
+    // HBM latency of staging: the rows of the next unit are fetched into registers before the MFMA loop of the current
+    // one and written to LDS after it.  Loads are unconditional (clamped addresses), rows past B are zeroed on the way in.
+    const int nbg = (B + MROWS - 1) / MROWS, nunits = C * nbg;
+    float4 x[PFQ];
+    float wr[2];
+    auto fetch_unit = [&](const int unit) __attribute__((always_inline)) {
+        const int c = unit / nbg, b0 = (unit - c * nbg) * MROWS;
 #pragma unroll
-        for (int s = 0; s < STG; ++s) {
-            const int idx = base + s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
-            // the load itself is unconditional (from a clamped address) so that all STG are issued before the first wait
+        for (int s = 0; s < PFQ; ++s) {
+            const int idx = s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
             const bool live = idx < total && b0 + r < B;
             x[s] = *reinterpret_cast<const float4*>(in + (static_cast<size_t>(live ? b0 + r : b0) * C + c) * T + (live ? 4 * q4 : 0));
         }
 #pragma unroll
-        for (int s = 0; s < STG; ++s) {
-            const int idx = base + s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
+        for (int s = 0; s < 2; ++s) wr[s] = w[static_cast<size_t>(c) * T + min(s * TXT + tid, T - 1)];
+    };
+    auto store_unit = [&](const int unit) __attribute__((always_inline)) {
+        const int c = unit / nbg, b0 = (unit - c * nbg) * MROWS;
+#pragma unroll
+        for (int s = 0; s < PFQ; ++s) {
+            const int idx = s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
             if (idx < total) *reinterpret_cast<float4*>(rows + r * rs + 4 * q4) = b0 + r < B ? x[s] : make_float4(0.f, 0.f, 0.f, 0.f);
         }
-    }
-    __syncthreads();
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+            if (s * TXT + tid < T) wp[s * TXT + tid] = wr[s];
+    };
+    if (tid < 32) wp[T + tid] = 0.f;
+    int unit = blockIdx.x;
+    if (unit < nunits) fetch_unit(unit);
 
-    const int nt = T >> 5;
     const float* brow = rows + ln * rs + 16 * kh;
-    for (int p = wv; 2 * p < nt; p += TXW) {
+    for (; unit < nunits; unit += gridDim.x) {
+        const int c = unit / nbg, b0 = (unit - c * nbg) * MROWS;
+        store_unit(unit);
+        __syncthreads();
+        if (unit + static_cast<int>(gridDim.x) < nunits) fetch_unit(unit + gridDim.x);
+        // (handing tiles out longest-first from an LDS counter was slower: the older wave of a SIMD wins the matrix core,
+        // drains the queue, and the younger one is left alone with a long tile)
+        for (int p = wv; 2 * p < nt; p += TXW) {
 #pragma unroll 1
-        for (int side = 0; side < 2; ++side) {
-            const int ot = side == 0 ? p : nt - 1 - p;
-            if (side == 1 && ot == p) break;
-            f32x16 acc, acc1;                              // even / odd K steps: consecutive MFMAs are independent
+            for (int side = 0; side < 2; ++side) {
+                const int ot = side == 0 ? p : nt - 1 - p;
+                if (side == 1 && ot == p) break;
+                f32x16 acc, acc1;                              // even / odd K steps: consecutive MFMAs are independent
 #pragma unroll
-            for (int v = 0; v < 16; ++v) { acc[v] = MIRROR ? 0.f : eps; acc1[v] = 0.f; }
-            const int n_in = MIRROR ? nt - ot : ot + 1;
-            // operands of step j + 1 are read while the MFMAs of step j run
-            float a[16], b[16];
-            auto fetch = [&](int j, float (&fa)[16], float (&fb)[16]) {
-                const int it = MIRROR ? ot + j : j;            // input tile
-                const int d = MIRROR ? j : ot - j;             // lag in tiles, >= 0
-                // A[row][K slot]: forward row = t, slot = u: tap T-1-(t-u);  mirror row = u, slot = t: tap T-1-(t-u)
-                const float* ap = wp + (MIRROR ? T - 1 - 32 * d - 16 * kh + ln : T - 1 - 32 * d - ln + 16 * kh);
+                for (int v = 0; v < 16; ++v) { acc[v] = MIRROR ? 0.f : eps; acc1[v] = 0.f; }
+                const int n_in = MIRROR ? nt - ot : ot + 1;
+                // operands of step j + 1 are read while the MFMAs of step j run
+                float a[16], b[16];
+                auto fetch = [&](int j, float (&fa)[16], float (&fb)[16]) {
+                    const int it = MIRROR ? ot + j : j;            // input tile
+                    const int d = MIRROR ? j : ot - j;             // lag in tiles, >= 0
+                    // A[row][K slot]: forward row = t, slot = u: tap T-1-(t-u);  mirror row = u, slot = t: tap T-1-(t-u)
+                    const float* ap = wp + (MIRROR ? T - 1 - 32 * d - 16 * kh + ln : T - 1 - 32 * d - ln + 16 * kh);
 #pragma unroll
-                for (int kk = 0; kk < 16; ++kk) fa[kk] = MIRROR ? ap[-kk] : ap[kk];
+                    for (int kk = 0; kk < 16; ++kk) fa[kk] = MIRROR ? ap[-kk] : ap[kk];
 #pragma unroll
-                for (int z = 0; z < 4; ++z) {
-                    const float4 x = *reinterpret_cast<const float4*>(brow + 32 * it + 4 * z);
-                    fb[4 * z] = x.x; fb[4 * z + 1] = x.y; fb[4 * z + 2] = x.z; fb[4 * z + 3] = x.w;
+                    for (int z = 0; z < 4; ++z) {
+                        const float4 y = *reinterpret_cast<const float4*>(brow + 32 * it + 4 * z);
+                        fb[4 * z] = y.x; fb[4 * z + 1] = y.y; fb[4 * z + 2] = y.z; fb[4 * z + 3] = y.w;
+                    }
+                };
+                fetch(0, a, b);
+                for (int j = 0; j < n_in; ++j) {
+                    float an[16], bn[16];
+                    fetch(j + 1 < n_in ? j + 1 : j, an, bn);
+#pragma unroll
+                    for (int kk = 0; kk < 16; kk += 2) {
+                        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk], b[kk], acc, 0, 0, 0);
+                        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk + 1], b[kk + 1], acc1, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int kk = 0; kk < 16; ++kk) { a[kk] = an[kk]; b[kk] = bn[kk]; }
                 }
-            };
-            fetch(0, a, b);
-            for (int j = 0; j < n_in; ++j) {
-                float an[16], bn[16];
-                fetch(j + 1 < n_in ? j + 1 : j, an, bn);
 #pragma unroll
-                for (int kk = 0; kk < 16; kk += 2) {
-                    acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk], b[kk], acc, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[kk + 1], b[kk + 1], acc1, 0, 0, 0);
+                for (int v = 0; v < 16; ++v) acc[v] += acc1[v];
+                if (b0 + ln < B) {
+                    float* o = out + (static_cast<size_t>(b0 + ln) * C + c) * T + 32 * ot + 4 * kh;
+#pragma unroll
+                    for (int v4 = 0; v4 < 4; ++v4)
+                        *reinterpret_cast<float4*>(o + 8 * v4) = make_float4(acc[4 * v4], acc[4 * v4 + 1], acc[4 * v4 + 2], acc[4 * v4 + 3]);
                 }
-#pragma unroll
-                for (int kk = 0; kk < 16; ++kk) { a[kk] = an[kk]; b[kk] = bn[kk]; }
-            }
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[v] += acc1[v];
-            if (b0 + ln < B) {
-                float* o = out + (static_cast<size_t>(b0 + ln) * C + c) * T + 32 * ot + 4 * kh;
-#pragma unroll
-                for (int v4 = 0; v4 < 4; ++v4)
-                    *reinterpret_cast<float4*>(o + 8 * v4) = make_float4(acc[4 * v4], acc[4 * v4 + 1], acc[4 * v4 + 2], acc[4 * v4 + 3]);
             }
         }
+        __syncthreads();               // every wave is done with this unit's rows
     }
 }
 
@@ -207,6 +229,7 @@ __global__ __launch_bounds__(TXT) void timex_conv_mfma(const float* __restrict__
 // diagonal l - 31 in row order and adds it to entry l of lag tile d, which no other wave touches: no atomics, every fp32
 // sum in a fixed order.
 constexpr int DIAG_STRIDE = 33;
+constexpr int T_GW_WIDE = 768;         // up to here 16 batch rows per pass fit in LDS, beyond 8
 __host__ __device__ inline int gw_row_stride(int T) { return T + 32 - (T & 63); }      // = 32 mod 64: the two K halves of a read use different banks
 __host__ __device__ inline size_t gw_lds_floats(int T, int rows) {
     return 2 * static_cast<size_t>(rows) * gw_row_stride(T) + 2 * static_cast<size_t>(T) + TXW * 32 * DIAG_STRIDE;
@@ -220,38 +243,51 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_mfma(const float* __restrict
     float* gr = lds;                           // [ROWS][rs]
     float* kr = gr + ROWS * rs;                // [ROWS][rs]
     float* diag = kr + ROWS * rs;              // [T/32 lag tiles][64]: entry l of tile d is the sum for lag 32 d + l - 31
-    const int c = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int ln = lane & 31, kh = lane >> 5;
-    const int nt = T >> 5, q4n = T >> 2;
-    for (int i = tid; i < 2 * T; i += TXT) diag[i] = 0.f;
+    const int nt = T >> 5, q4n = T >> 2, total = ROWS * q4n;
     float* tile = diag + 2 * T + wv * (32 * DIAG_STRIDE);         // [32 t][33]: one finished product tile
 
-    for (int b0 = 0; b0 < B; b0 += ROWS) {
-        __syncthreads();
-        const int total = ROWS * q4n;
-        for (int base = 0; base < total; base += (STG / 2) * TXT) {
-            float4 xg[STG / 2], xk[STG / 2];
+    // A workgroup walks over its channels (blockIdx.x, + gridDim.x, ...) and, per channel, over passes of ROWS batch rows;
+    // the rows of the next pass are fetched into registers before the MFMA loop of the current one (see timex_conv_mfma).
+    constexpr int PF = ROWS * ((ROWS == 16 ? T_GW_WIDE : T_MFMA_MAX) / 4) / TXT;
+    const int npass = (B + ROWS - 1) / ROWS;
+    const int nmine = (C > static_cast<int>(blockIdx.x) ? (C - 1 - static_cast<int>(blockIdx.x)) / static_cast<int>(gridDim.x) + 1 : 0) * npass;
+    float4 xg[PF], xk[PF];
+    auto fetch_unit = [&](const int u) __attribute__((always_inline)) {
+        const int c = blockIdx.x + (u / npass) * gridDim.x, b0 = (u % npass) * ROWS;
 #pragma unroll
-            for (int s = 0; s < STG / 2; ++s) {
-                const int idx = base + s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
-                const bool live = idx < total && b0 + r < B;
-                const size_t off = (static_cast<size_t>(live ? b0 + r : b0) * C + c) * T + (live ? 4 * q4 : 0);
-                xg[s] = *reinterpret_cast<const float4*>(g + off);
-                xk[s] = *reinterpret_cast<const float4*>(k + off);
-            }
+        for (int s = 0; s < PF; ++s) {
+            const int idx = s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
+            const bool live = idx < total && b0 + r < B;
+            const size_t off = (static_cast<size_t>(live ? b0 + r : b0) * C + c) * T + (live ? 4 * q4 : 0);
+            xg[s] = *reinterpret_cast<const float4*>(g + off);
+            xk[s] = *reinterpret_cast<const float4*>(k + off);
+        }
+    };
+    auto store_unit = [&](const int u) __attribute__((always_inline)) {
+        const int b0 = (u % npass) * ROWS;
 #pragma unroll
-            for (int s = 0; s < STG / 2; ++s) {
-                const int idx = base + s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
-                if (idx < total) {
-                    const bool real = b0 + r < B;
-                    *reinterpret_cast<float4*>(gr + r * rs + 4 * q4) = real ? xg[s] : make_float4(0.f, 0.f, 0.f, 0.f);
-                    *reinterpret_cast<float4*>(kr + r * rs + 4 * q4) = real ? xk[s] : make_float4(0.f, 0.f, 0.f, 0.f);
-                }
+        for (int s = 0; s < PF; ++s) {
+            const int idx = s * TXT + tid, r = idx / q4n, q4 = idx - r * q4n;
+            if (idx < total) {
+                const bool real = b0 + r < B;
+                *reinterpret_cast<float4*>(gr + r * rs + 4 * q4) = real ? xg[s] : make_float4(0.f, 0.f, 0.f, 0.f);
+                *reinterpret_cast<float4*>(kr + r * rs + 4 * q4) = real ? xk[s] : make_float4(0.f, 0.f, 0.f, 0.f);
             }
         }
+    };
+    if (nmine > 0) fetch_unit(0);
+
+    const float* ga = gr + kh * rs + ln;
+    const float* kb = kr + kh * rs + ln;
+    for (int u = 0; u < nmine; ++u) {
+        const int pass = u % npass;
+        if (pass == 0)
+            for (int i = tid; i < 2 * T; i += TXT) diag[i] = 0.f;
+        store_unit(u);
         __syncthreads();
-        const float* ga = gr + kh * rs + ln;
-        const float* kb = kr + kh * rs + ln;
+        if (u + 1 < nmine) fetch_unit(u + 1);
         for (int p = wv; 2 * p < nt; p += TXW) {
 #pragma unroll 1
             for (int side = 0; side < 2; ++side) {
@@ -288,18 +324,22 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_mfma(const float* __restrict
                 float sum = 0.f;
 #pragma unroll
                 for (int t = 0; t < 32; ++t) {
-                    const int u = t - dl;
-                    const float x = tile[t * DIAG_STRIDE + (u & 31)];
-                    sum += (u >= 0 && u < 32) ? x : 0.f;
+                    const int uu = t - dl;
+                    const float y = tile[t * DIAG_STRIDE + (uu & 31)];
+                    sum += (uu >= 0 && uu < 32) ? y : 0.f;
                 }
                 diag[64 * d + lane] += sum;                 // lag tile d belongs to this wave alone
             }
         }
-    }
-    __syncthreads();
-    for (int x = tid; x < T; x += TXT) {            // lag = 32 d + e comes from tile d (diagonal e) and tile d + 1 (diagonal e - 32)
-        const int lag = T - 1 - x, d = lag >> 5, e = lag & 31;
-        gws[static_cast<size_t>(c) * T + x] = diag[64 * d + 31 + e] + (d + 1 < nt ? diag[64 * (d + 1) + e - 1] : 0.f);
+        __syncthreads();
+        if (pass == npass - 1) {
+            const int c = blockIdx.x + (u / npass) * gridDim.x;
+            for (int x = tid; x < T; x += TXT) {        // lag = 32 d + e comes from tile d (diagonal e) and tile d + 1 (diagonal e - 32)
+                const int lag = T - 1 - x, d = lag >> 5, e = lag & 31;
+                gws[static_cast<size_t>(c) * T + x] = diag[64 * d + 31 + e] + (d + 1 < nt ? diag[64 * (d + 1) + e - 1] : 0.f);
+            }
+            __syncthreads();           // diag is cleared for the next channel only after it has been read
+        }
     }
 }
 
@@ -314,6 +354,10 @@ int check_tx(int B, int C, int T) {
 
 // The matrix-core path pays off once the 32 columns of a product are mostly real batch rows.
 bool use_mfma(int B, int T) { return T % 32 == 0 && T <= T_MFMA_MAX && B >= 8; }
+int conv_grid(int B, int C) {
+    const long long units = static_cast<long long>(C) * ((B + MROWS - 1) / MROWS);
+    return static_cast<int>(units < NCU ? units : NCU);
+}
 size_t mfma_lds_bytes(int T) { return (static_cast<size_t>(T) + 32 + static_cast<size_t>(MROWS) * (T + 4)) * sizeof(float); }
 
 template <typename K> int raise_lds_limit(K kernel, size_t bytes) {
@@ -334,7 +378,7 @@ int launch_gk(void* stream, const float* w, const float* gwk, float* gk, int B, 
     if (use_mfma(B, T)) {
         const size_t lds = mfma_lds_bytes(T);
         if (int e = raise_lds_limit(timex_conv_mfma<true>, lds)) return e;
-        hipLaunchKernelGGL(timex_conv_mfma<true>, dim3(C, (B + MROWS - 1) / MROWS), dim3(TXT), lds,
+        hipLaunchKernelGGL(timex_conv_mfma<true>, dim3(conv_grid(B, C)), dim3(TXT), lds,
                            static_cast<hipStream_t>(stream), w, gwk, gk, 0.0f, B, C, T);
     } else {
         const size_t lds = (static_cast<size_t>(BB + 1) * T + 4) * sizeof(float);
@@ -353,7 +397,7 @@ int rwkv_timex_forward(void* stream, const float* w, const float* k, float* x, f
     if (use_mfma(B, T)) {
         const size_t lds = mfma_lds_bytes(T);
         if (int e = raise_lds_limit(timex_conv_mfma<false>, lds)) return e;
-        hipLaunchKernelGGL(timex_conv_mfma<false>, dim3(C, (B + MROWS - 1) / MROWS), dim3(TXT), lds,
+        hipLaunchKernelGGL(timex_conv_mfma<false>, dim3(conv_grid(B, C)), dim3(TXT), lds,
                            static_cast<hipStream_t>(stream), w, k, x, eps, B, C, T);
         return launch_status();
     }
@@ -380,12 +424,12 @@ int rwkv_timex_backward_sum(void* stream, const float* w, const float* k, const 
     if (int e = check_tx(B, C, T)) return e;
     if (T % 32 != 0 || T > T_MFMA_MAX) return RWKV_ERR_SHAPE;
     if (int e = check_ptrs({w, k, gwk, gw_sum, gk})) return e;
-    const bool wide = T <= 768;                 // 16 batch rows per pass while they fit in LDS, else 8
+    const bool wide = T <= T_GW_WIDE;
     const size_t lds_gw = gw_lds_floats(T, wide ? 16 : 8) * sizeof(float);
     auto kernel = wide ? timex_gw_sum_mfma<16> : timex_gw_sum_mfma<8>;
     if (int e = raise_lds_limit(kernel, lds_gw)) return e;
     if (int e = launch_gk(stream, w, gwk, gk, B, C, T)) return e;
-    hipLaunchKernelGGL(kernel, dim3(C), dim3(TXT), lds_gw, static_cast<hipStream_t>(stream), k, gwk, gw_sum, B, C, T);
+    hipLaunchKernelGGL(kernel, dim3(C < NCU ? C : NCU), dim3(TXT), lds_gw, static_cast<hipStream_t>(stream), k, gwk, gw_sum, B, C, T);
     return launch_status();
 }
 
