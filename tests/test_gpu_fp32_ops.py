@@ -23,7 +23,7 @@ def _check(name, ref, got):
     assert a <= TOL and b <= TOL, (name, a, b)
 
 
-@pytest.mark.parametrize("B,T,C", [(2, 37, 70), (1, 1, 3), (4, 512, 768)])
+@pytest.mark.parametrize("B,T,C", [(2, 37, 70), (1, 1, 3), (3, 333, 50), (1, 4100, 20), (4, 512, 768)])
 def test_wkv4(lib, B, T, C):
     print(f"\nwkv4 B={B} T={T} C={C}", flush=True)
     w_raw, u, k, v, gy = synth.wkv4_inputs(B, T, C, seed=21)
