@@ -41,6 +41,9 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.rwkv_wkv5_forward(None, 1, 8, 128, 1, p, p, p, p, p, p) == -1
     assert lib.rwkv7_statepassing_forward(None, 1, 24, 1, *([p] * 11)) == -1         # T % 16
     assert lib.rwkv_timex_forward(None, p, p, p, 0.0, 1, 1, 6) == -1                 # T % 4
+    assert lib.rwkv_timex_backward_sum(None, p, p, p, p, p, 2, 1, 48) == -1           # T % 32
+    assert lib.rwkv_timex_backward_sum(None, p, p, p, p, p, 2, 1, 2048) == -1         # T > 1024
+    assert lib.rwkv_timex_backward_sum(None, p, p, p, None, p, 2, 1, 64) == -2
     assert lib.rwkv_wkv4_forward(None, 1, 0, 4, p, p, p, p, p) == -1
     # null / misaligned pointers
     assert lib.rwkv_wkv6_forward(None, 1, 8, 64, 1, p, p, None, p, p, p) == -2

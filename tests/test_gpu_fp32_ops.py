@@ -36,6 +36,19 @@ def test_wkv4(lib, B, T, C):
         _check(name, a, g)
 
 
+def test_wkv4_more_batch_rows_than_a_grid_dimension(lib):
+    """B > 65535 takes the one-lane-per-scan kernels (the time-parallel ones put B on the grid's y axis)."""
+    B, T, C = 65536, 3, 1
+    w_raw, u, k, v, gy = synth.wkv4_inputs(B, T, C, seed=25)
+    ref = O4.grads(B, T, C, w_raw, u, k, v, gy)
+    t = [x.to(DEV).requires_grad_(True) for x in (w_raw, u, k, v)]
+    y = wkv.WKV.apply(B, T, C, *t)
+    y.backward(gy.to(DEV))
+    torch.cuda.synchronize()
+    for name, a, g in zip(["y", "gw", "gu", "gk", "gv"], ref, [y] + [x.grad for x in t]):
+        _check(name, a, g)
+
+
 def test_wkv4_extreme_k_stays_finite(lib):
     """k ~ U(-1000,1000): the stabilised kernel must not overflow (wkv/run.py:159-169)."""
     B, T, C = 2, 64, 128
