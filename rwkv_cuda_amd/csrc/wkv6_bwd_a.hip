@@ -438,7 +438,9 @@ __global__ __launch_bounds__(NTA) void wkv6_bwd_a_ws(const ArgsB a) {
         S.sel[p][ln] = one_hot(gg == (c16 >> 2), 4 * p + (c16 & 3));
     }
     if (__builtin_amdgcn_readfirstlane(tid >> 6) < NPREP) bwa_prep<WMODE>(S, a, tid, base, nchunks);
-    else bwa_state<WMODE>(S, a, tid, base, bh, nchunks);
+    // The state waves carry the chunk-to-chunk dependence; the prep waves work ahead and have slack.  Issue priority goes
+    // to the state waves (the hardware otherwise favours the oldest waves of a SIMD, which are the prep waves).
+    else { __builtin_amdgcn_s_setprio(2); bwa_state<WMODE>(S, a, tid, base, bh, nchunks); }
 }
 
 }  // namespace
