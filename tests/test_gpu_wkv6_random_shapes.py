@@ -1,0 +1,59 @@
+"""GPU: the chunked matrix-core kernels against the sequential fp32 sweeps on random shapes and decay strengths.
+
+Both algorithms round the same quantities to bf16, so they may differ by one bf16 unit of the value (2^-8 relative);
+a slip in the chunk logic (a partial last chunk, the exact-path switch, state passing) shows up as an error of order one.
+Every result is also checked against the fp64 oracle with the usual bar."""
+import random
+
+import pytest
+import torch
+
+from oracle import wkv56 as O
+from rwkv_cuda_amd import _lib, synth
+from rwkv_cuda_amd._call import call
+from _gpu_util import DEV, assert_no_worse, garbage
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+
+
+def _run(lib, algo, B, T, C, H, d):
+    _lib.check(lib.rwkv_wkv6_set_algorithm(algo))
+    try:
+        y = garbage((B, T, C), BF)
+        call("rwkv_wkv6state_forward", d[0].device, B, T, C, H, *d[:6], y)
+        gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
+        gu = garbage((B, C), BF)
+        gs = garbage((B, H, 64, 64), BF)
+        n = lib.rwkv_wkv6state_backward_workspace_bytes(B, T, C, H)
+        ws = torch.empty(max(n, 16), device=DEV, dtype=torch.uint8)
+        call("rwkv_wkv6state_backward", d[0].device, B, T, C, H, *d[:6], d[6], gr, gk, gv, gw, gu, gs, ws, n)
+        torch.cuda.synchronize()
+    finally:
+        _lib.check(lib.rwkv_wkv6_set_algorithm(0))
+    return [y, gr, gk, gv, gw, gu.sum(0).view(H, 64), gs]
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_wkv6_state_chunked_equals_sweeps(lib, seed):
+    rng = random.Random(seed)
+    B, H, T = rng.randint(1, 3), rng.randint(1, 3), rng.choice([rng.randint(1, 31), rng.randint(32, 200), 32 * rng.randint(1, 5)])
+    C = H * 64
+    print(f"\nseed {seed}: B={B} T={T} H={H}", flush=True)
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=100 + seed, state=True)
+    if seed % 2:                                   # some tokens and channels decay fast enough for the exact path
+        g = torch.Generator().manual_seed(seed)
+        mask = torch.rand(B, T, C, generator=g) < 0.0004    # about one hit per chunk and head: exact and chunked chunks alternate
+        w = torch.where(mask, torch.full_like(w, 2.5), w)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    d = [x.to(DEV) for x in (r, k, v, w, u, s0, gy)]
+    chunked = _run(lib, 0, B, T, C, H, d)
+    sweeps = _run(lib, 1, B, T, C, H, d)
+    for name, a, e, c, s in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, emu, chunked, sweeps):
+        assert_no_worse(name + " (chunked)", a, e, c)
+        peak = float(a.abs().max())
+        if peak > 0.0:
+            diff = float((c.float() - s.float()).abs().max()) / peak
+            print(f"  {name}: chunked vs sweeps, max difference / peak {diff:.3e}", flush=True)
+            assert diff < 2.0 ** -6, (name, diff)
