@@ -320,8 +320,12 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
 }
 
 // The chunked matrix-core kernels serve all three decay conventions; the sequential sweeps remain as the second algorithm.
+// They address one batch row with 32-bit byte offsets (up to 4 bytes per element), so rows of 2^30 elements or more
+// take the sweeps.
+bool use_chunked(const Args& a) { return g_wkv6_algorithm == RWKV_ALGO_CHUNKED && static_cast<long long>(a.T) * a.C < (1LL << 30); }
+
 template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a) {
-    if (g_wkv6_algorithm == RWKV_ALGO_CHUNKED)
+    if (use_chunked(a))
         return launch_wkv6_fwd_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, a.w, a.u, a.s0, a.y);
     hipLaunchKernelGGL((wkv_sweep<P_FWD, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
     return launch_status();
@@ -330,7 +334,7 @@ template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a) {
 // GR and GV are independent; GK consumes GR's workspace.  All three run on `st` in order.
 // `passes` is a bit mask (RWKV_PASS_*) so that a profiler can time one kernel at a time.
 template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a, unsigned passes = RWKV_PASS_ALL) {
-    const bool chunked = g_wkv6_algorithm == RWKV_ALGO_CHUNKED;
+    const bool chunked = use_chunked(a);
     const void* w = (WMODE == W_HEAD) ? static_cast<const void*>(a.ew_head) : a.w;   // wkv5: the log decay
     if ((passes & RWKV_PASS_GR) && chunked) {
         if (int e = launch_wkv6_bwd_a_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, w, a.u, a.s0, a.gy, a.gr, a.gu, a.rdr)) return e;
