@@ -184,6 +184,33 @@ int rwkv7_statepassing_backward(void* stream, int B, int T, int H,
                                 rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv,
                                 rwkv_bf16* da, rwkv_bf16* db);
 
+/* The two siblings of the state-passing op, served by the same kernels:
+ *   rwkv7_state_*  : initial state s0 and its gradient ds0, no final state.  Replaces cuda_forward /
+ *                    cuda_backward of rwkv7_fast_fused/cuda/rwkv7_state_clampw.cpp:10,17.
+ *   rwkv7_forward / rwkv7_backward : zero initial state, no state outputs.  Replaces cuda_forward /
+ *                    cuda_backward of rwkv7_fast_fused/cuda/rwkv7_clampw.cpp:10,17.
+ * Argument order is the reference's after the leading stream; bf16 mode only (the reference's -D_FP32_ build of the
+ * same files is not provided). */
+int rwkv7_state_forward(void* stream, int B, int T, int H,
+                        const float* s0, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
+                        const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b,
+                        rwkv_bf16* y, float* s, float* sa);
+int rwkv7_state_backward(void* stream, int B, int T, int H,
+                         const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k, const rwkv_bf16* v,
+                         const rwkv_bf16* a, const rwkv_bf16* b, const rwkv_bf16* dy,
+                         const float* s, const float* sa, float* ds0,
+                         rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv,
+                         rwkv_bf16* da, rwkv_bf16* db);
+int rwkv7_forward(void* stream, int B, int T, int H,
+                  const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k, const rwkv_bf16* v,
+                  const rwkv_bf16* a, const rwkv_bf16* b, rwkv_bf16* y, float* s, float* sa);
+int rwkv7_backward(void* stream, int B, int T, int H,
+                   const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k, const rwkv_bf16* v,
+                   const rwkv_bf16* a, const rwkv_bf16* b, const rwkv_bf16* dy,
+                   const float* s, const float* sa,
+                   rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv,
+                   rwkv_bf16* da, rwkv_bf16* db);
+
 #ifdef __cplusplus
 }
 #endif

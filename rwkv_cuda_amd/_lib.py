@@ -95,6 +95,10 @@ SIGNATURES = {
     "rwkv_wkv6state_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, _Z]),
     "rwkv7_statepassing_forward": (_I, [_P, _I, _I, _I] + [_P] * 11),
     "rwkv7_statepassing_backward": (_I, [_P, _I, _I, _I] + [_P] * 17),
+    "rwkv7_state_forward": (_I, [_P, _I, _I, _I] + [_P] * 10),
+    "rwkv7_state_backward": (_I, [_P, _I, _I, _I] + [_P] * 16),
+    "rwkv7_forward": (_I, [_P, _I, _I, _I] + [_P] * 9),
+    "rwkv7_backward": (_I, [_P, _I, _I, _I] + [_P] * 15),
 }
 
 

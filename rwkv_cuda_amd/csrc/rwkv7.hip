@@ -72,7 +72,9 @@ __global__ __launch_bounds__(NT) void rwkv7_fwd(const Args7 p) {
     auto off = [&](int t) { return ((static_cast<size_t>(b) * T + t) * H + h) * N + sj; };
 
     float St[JW];
-    {
+#pragma unroll
+    for (int e = 0; e < JW; ++e) St[e] = 0.f;
+    if (p.s0 != nullptr) {                         // the entry points without an initial state start from zero
         const float* s0 = p.s0 + (bh * N + row) * N + hi * JW;
 #pragma unroll
         for (int e = 0; e < JW; e += 4) {
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(NT) void rwkv7_fwd(const Args7 p) {
             *reinterpret_cast<float4*>(p.sa + o) = *reinterpret_cast<const float4*>(&S.sa[st][sj]);
         }
     }
-    {
+    if (p.sT != nullptr) {
         float* sT = p.sT + (bh * N + row) * N + hi * JW;
 #pragma unroll
         for (int e = 0; e < JW; e += 4)
@@ -169,7 +171,9 @@ __global__ __launch_bounds__(NT) void rwkv7_bwd(const Args7 p) {
     auto off = [&](int t) { return ((static_cast<size_t>(b) * T + t) * H + h) * N + sj; };
 
     float ST[JW], dST[JW], dSH[JW];
-    {
+#pragma unroll
+    for (int e = 0; e < JW; ++e) { ST[e] = 0.f; dST[e] = 0.f; dSH[e] = 0.f; }
+    if (p.dsT != nullptr) {                        // no gradient arrives through a final state that is not an output
         const float* g = p.dsT + bh * N * N;
 #pragma unroll
         for (int e = 0; e < JW; ++e) {
@@ -296,7 +300,7 @@ __global__ __launch_bounds__(NT) void rwkv7_bwd(const Args7 p) {
             put(p.dv, S.dv); put(p.da, S.da); put(p.db, S.db);
         }
     }
-    {
+    if (p.ds0 != nullptr) {
         float* d = p.ds0 + (bh * N + own) * N + hi * JW;
 #pragma unroll
         for (int e = 0; e < JW; e += 4)
@@ -311,6 +315,28 @@ int check7(int B, int T, int H) {
     return RWKV_OK;
 }
 
+int launch7_fwd(void* stream, int B, int T, int H, const float* s0, const rwkv_bf16* r, const rwkv_bf16* w,
+                const rwkv_bf16* k, const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b, rwkv_bf16* y,
+                float* sT, float* s, float* sa) {
+    Args7 p{};
+    p.T = T; p.H = H; p.s0 = s0; p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b;
+    p.y = y; p.sT = sT; p.s = s; p.sa = sa;
+    hipLaunchKernelGGL(rwkv7_fwd, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status();
+}
+
+int launch7_bwd(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
+                const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b, const rwkv_bf16* dy, const float* dsT,
+                const float* s, const float* sa, float* ds0, rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk,
+                rwkv_bf16* dv, rwkv_bf16* da, rwkv_bf16* db) {
+    Args7 p{};
+    p.T = T; p.H = H; p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b; p.dy = dy; p.dsT = dsT;
+    p.s = const_cast<float*>(s); p.sa = const_cast<float*>(sa);
+    p.ds0 = ds0; p.dr = dr; p.dw = dw; p.dk = dk; p.dv = dv; p.da = da; p.db = db;
+    hipLaunchKernelGGL(rwkv7_bwd, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status();
+}
+
 }  // namespace
 }  // namespace rwkv
 
@@ -323,11 +349,7 @@ int rwkv7_statepassing_forward(void* stream, int B, int T, int H, const float* s
                                const rwkv_bf16* b, rwkv_bf16* y, float* sT, float* s, float* sa) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({s0, r, w, k, v, a, b, y, sT, s, sa})) return e;
-    Args7 p{};
-    p.T = T; p.H = H; p.s0 = s0; p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b;
-    p.y = y; p.sT = sT; p.s = s; p.sa = sa;
-    hipLaunchKernelGGL(rwkv7_fwd, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
-    return launch_status();
+    return launch7_fwd(stream, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa);
 }
 
 int rwkv7_statepassing_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w,
@@ -337,12 +359,42 @@ int rwkv7_statepassing_backward(void* stream, int B, int T, int H, const rwkv_bf
                                 rwkv_bf16* da, rwkv_bf16* db) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db})) return e;
-    Args7 p{};
-    p.T = T; p.H = H; p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b; p.dy = dy; p.dsT = dsT;
-    p.s = const_cast<float*>(s); p.sa = const_cast<float*>(sa);
-    p.ds0 = ds0; p.dr = dr; p.dw = dw; p.dk = dk; p.dv = dv; p.da = da; p.db = db;
-    hipLaunchKernelGGL(rwkv7_bwd, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
-    return launch_status();
+    return launch7_bwd(stream, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db);
+}
+
+// Initial state with its gradient, no final state: the same kernels without the sT store and with dsT = 0.
+int rwkv7_state_forward(void* stream, int B, int T, int H, const float* s0, const rwkv_bf16* r, const rwkv_bf16* w,
+                        const rwkv_bf16* k, const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b,
+                        rwkv_bf16* y, float* s, float* sa) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({s0, r, w, k, v, a, b, y, s, sa})) return e;
+    return launch7_fwd(stream, B, T, H, s0, r, w, k, v, a, b, y, nullptr, s, sa);
+}
+
+int rwkv7_state_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w,
+                         const rwkv_bf16* k, const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b,
+                         const rwkv_bf16* dy, const float* s, const float* sa, float* ds0, rwkv_bf16* dr,
+                         rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv, rwkv_bf16* da, rwkv_bf16* db) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({r, w, k, v, a, b, dy, s, sa, ds0, dr, dw, dk, dv, da, db})) return e;
+    return launch7_bwd(stream, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, ds0, dr, dw, dk, dv, da, db);
+}
+
+// No state on either side: zero initial state, no final state, no state gradients.
+int rwkv7_forward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
+                  const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b, rwkv_bf16* y, float* s, float* sa) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({r, w, k, v, a, b, y, s, sa})) return e;
+    return launch7_fwd(stream, B, T, H, nullptr, r, w, k, v, a, b, y, nullptr, s, sa);
+}
+
+int rwkv7_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
+                   const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b, const rwkv_bf16* dy, const float* s,
+                   const float* sa, rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv, rwkv_bf16* da,
+                   rwkv_bf16* db) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({r, w, k, v, a, b, dy, s, sa, dr, dw, dk, dv, da, db})) return e;
+    return launch7_bwd(stream, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, nullptr, dr, dw, dk, dv, da, db);
 }
 
 }  // extern "C"

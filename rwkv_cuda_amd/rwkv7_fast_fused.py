@@ -1,6 +1,7 @@
-"""RWKV-7 clamp-w with state passing: drop-in for
-rwkv7_fast_fused/rwkv7_cuda_benchmark_state_passing.py:75-103
-(RWKV7_STATE_PASSING_CLAMPW_CUDA_OP, RWKV7_STATE_PASSING_CLAMPW_CUDA)."""
+"""RWKV-7 clamp-w, bf16: drop-ins for
+rwkv7_fast_fused/rwkv7_cuda_benchmark_state_passing.py:75-103 (RWKV7_STATE_PASSING_CLAMPW_CUDA_OP, ..._CUDA),
+rwkv7_fast_fused/rwkv7_cuda_benchmark_state.py:75-102 (RWKV7_STATE_CLAMPW_CUDA_OP, ..._CUDA: initial state only) and
+rwkv7_fast_fused/rwkv7_cuda_benchmark.py:76-100 (RWKV7_CLAMPW_CUDA_OP, ..._CUDA: no state)."""
 
 import torch
 
@@ -49,3 +50,79 @@ def RWKV7_STATE_PASSING_CLAMPW_CUDA(s0, r, w, k, v, a, b):
     B, T, HC = r.shape
     r, w, k, v, a, b = [i.view(B, T, HC // HEAD_SIZE, HEAD_SIZE) for i in [r, w, k, v, a, b]]
     return RWKV7_STATE_PASSING_CLAMPW_CUDA_OP.apply(s0, r, w, k, v, a, b)
+
+
+def _scratch(r):
+    B, T, H, N = r.shape
+    s = torch.empty(B, H, T // CHUNK_LEN, N, N, dtype=torch.float32, device=r.device)
+    sa = torch.empty(B, T, H, N, dtype=torch.float32, device=r.device)
+    return s, sa
+
+
+class RWKV7_STATE_CLAMPW_CUDA_OP(torch.autograd.Function):
+    """forward(s0, r, w, k, v, a, b) -> y[B,T,H,N]; backward returns (ds0, dr, dw, dk, dv, da, db)
+    (rwkv7_cuda_benchmark_state.py:77-98)."""
+
+    @staticmethod
+    def forward(ctx, s0, r, w, k, v, a, b):
+        B, T, H, N = r.shape
+        require(N == HEAD_SIZE, "head size must be 64")
+        require(T % CHUNK_LEN == 0, "T must be a multiple of CHUNK_LEN")
+        dev = check_tensors((r, w, k, v, a, b), torch.bfloat16, "rwkvab")
+        check_tensors((s0,), torch.float32, ("s0",))
+        require(s0.device == dev and tuple(s0.shape) == (B, H, N, N), "s0 must be [B,H,N,N] on the same device")
+        y = torch.empty_like(v)
+        s, sa = _scratch(r)
+        call("rwkv7_state_forward", dev, B, T, H, s0, r, w, k, v, a, b, y, s, sa)
+        ctx.save_for_backward(r, w, k, v, a, b, s, sa)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        r, w, k, v, a, b, s, sa = ctx.saved_tensors
+        B, T, H, N = r.shape
+        dy = dy.contiguous()
+        dev = check_tensors((dy,), torch.bfloat16, ("dy",))
+        ds0 = torch.empty(B, H, N, N, dtype=torch.float32, device=dev)
+        dr, dw, dk, dv, da, db = [torch.empty_like(x) for x in [r, w, k, v, a, b]]
+        call("rwkv7_state_backward", dev, B, T, H, r, w, k, v, a, b, dy, s, sa, ds0, dr, dw, dk, dv, da, db)
+        return ds0, dr, dw, dk, dv, da, db
+
+
+def RWKV7_STATE_CLAMPW_CUDA(s0, r, w, k, v, a, b):
+    B, T, HC = r.shape
+    r, w, k, v, a, b = [i.view(B, T, HC // HEAD_SIZE, HEAD_SIZE) for i in [r, w, k, v, a, b]]
+    return RWKV7_STATE_CLAMPW_CUDA_OP.apply(s0, r, w, k, v, a, b).view(B, T, HC)
+
+
+class RWKV7_CLAMPW_CUDA_OP(torch.autograd.Function):
+    """forward(r, w, k, v, a, b) -> y[B,T,H,N] from a zero state; backward returns (dr, dw, dk, dv, da, db)
+    (rwkv7_cuda_benchmark.py:78-96)."""
+
+    @staticmethod
+    def forward(ctx, r, w, k, v, a, b):
+        B, T, H, N = r.shape
+        require(N == HEAD_SIZE, "head size must be 64")
+        require(T % CHUNK_LEN == 0, "T must be a multiple of CHUNK_LEN")
+        dev = check_tensors((r, w, k, v, a, b), torch.bfloat16, "rwkvab")
+        y = torch.empty_like(v)
+        s, sa = _scratch(r)
+        call("rwkv7_forward", dev, B, T, H, r, w, k, v, a, b, y, s, sa)
+        ctx.save_for_backward(r, w, k, v, a, b, s, sa)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        r, w, k, v, a, b, s, sa = ctx.saved_tensors
+        B, T, H, N = r.shape
+        dy = dy.contiguous()
+        dev = check_tensors((dy,), torch.bfloat16, ("dy",))
+        dr, dw, dk, dv, da, db = [torch.empty_like(x) for x in [r, w, k, v, a, b]]
+        call("rwkv7_backward", dev, B, T, H, r, w, k, v, a, b, dy, s, sa, dr, dw, dk, dv, da, db)
+        return dr, dw, dk, dv, da, db
+
+
+def RWKV7_CLAMPW_CUDA(r, w, k, v, a, b):
+    B, T, HC = r.shape
+    r, w, k, v, a, b = [i.view(B, T, HC // HEAD_SIZE, HEAD_SIZE) for i in [r, w, k, v, a, b]]
+    return RWKV7_CLAMPW_CUDA_OP.apply(r, w, k, v, a, b).view(B, T, HC)

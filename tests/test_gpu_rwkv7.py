@@ -73,3 +73,37 @@ def test_rwkv7_full_size_chain_equals_one_call(lib):
         e = err_ratio(a, g.double().cpu())
         print(f"  head {h} {name}: {e:.3e}", flush=True)
         assert e < 3e-3, (name, e)
+
+
+@pytest.mark.parametrize("B,T,H", [(2, 32, 2), (1, 48, 1)])
+def test_rwkv7_state_only_and_stateless_ops(lib, B, T, H):
+    """The siblings of the state-passing op (rwkv7_state_clampw: s0 and ds0, no final state; rwkv7_clampw: no state
+    at all) are the state-passing formula with dsT = 0, respectively s0 = 0 and dsT = 0."""
+    print(f"\nrwkv7 siblings B={B} T={T} H={H}", flush=True)
+    s0, r, w, k, v, a, b, dy, dsT = synth.rwkv7_inputs(B, T, H, 64, seed=33)
+    N = 64
+    flat = lambda x: x.contiguous().view(B, T, H * N)
+
+    # initial state only
+    args = (s0, r, w, k, v, a, b, dy, torch.zeros_like(dsT))
+    ref, emu = O.grads(*args), O.emulate_bf16(*args)
+    t = [x.to(DEV).requires_grad_(True) for x in (s0, r, w, k, v, a, b)]
+    y = R.RWKV7_STATE_CLAMPW_CUDA(t[0], *(flat(x) for x in t[1:]))
+    y.backward(flat(dy.to(DEV)))
+    torch.cuda.synchronize()
+    got = [y.detach().view(B, T, H, N), None] + [x.grad for x in t]
+    for name, a_, e, g in zip(NAMES, ref, emu, got):
+        if g is not None:
+            assert_no_worse("state op " + name, a_, e, g)
+
+    # no state
+    args = (torch.zeros_like(s0), r, w, k, v, a, b, dy, torch.zeros_like(dsT))
+    ref, emu = O.grads(*args), O.emulate_bf16(*args)
+    t = [x.to(DEV).requires_grad_(True) for x in (r, w, k, v, a, b)]
+    y = R.RWKV7_CLAMPW_CUDA(*(flat(x) for x in t))
+    y.backward(flat(dy.to(DEV)))
+    torch.cuda.synchronize()
+    got = [y.detach().view(B, T, H, N), None, None] + [x.grad for x in t]
+    for name, a_, e, g in zip(NAMES, ref, emu, got):
+        if g is not None:
+            assert_no_worse("stateless op " + name, a_, e, g)
