@@ -349,6 +349,37 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
         const int c0 = (nchunks - 1 - i) * L;
         const SetB& O = S.set[i & 1];
         const bool exact = __builtin_amdgcn_readfirstlane(O.exact) != 0;
+        if constexpr (WMODE == W_HEAD) {
+            const int cn = nchunks - i;                // the chunk after this one; D is dS at its first token
+            if (cn < nchunks && cn % PCK == 0) {       // P at that boundary from the stored S (see PCK), replacing the carried value
+                const int npck = (nchunks + PCK - 1) / PCK;
+                const float* slot = a.rdr + static_cast<size_t>(gridDim.x / a.H) * T * C + (bh * npck + cn / PCK) * PCK_FLOATS;
+                // D[m][v] <-> sweep A's state wave (q, ih = m >> 1), register 4 (m & 1) + v.  Loaded with a scalar base and one
+                // 32-bit lane offset (per-lane 64-bit addresses kept across the loop cost this wave registers it does not have).
+                uint32_t voff = lane;
+                asm volatile("" : "+v"(voff));         // keeps the shift below inside this block instead of a register held across the loop
+                voff <<= 5;
+                slot += q * 64 * 8;
+                const float* slot1 = slot + 4 * 64 * 8;
+                f32x4 s0, s1, s2, s3;
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(s0) : "v"(voff), "s"(slot));
+                asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=&v"(s1) : "v"(voff), "s"(slot));
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(s2) : "v"(voff), "s"(slot1));
+                asm volatile("global_load_dwordx4 %0, %1, %2 offset:16" : "=&v"(s3) : "v"(voff), "s"(slot1));
+                asm volatile("s_waitcnt vmcnt(0)" : "+v"(s0), "+v"(s1), "+v"(s2), "+v"(s3));
+                float p = 0.f;
+                const f32x4 sv[4] = {s0, s1, s2, s3};
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    p = fmaf(D[m][0], sv[m][0], p); p = fmaf(D[m][1], sv[m][1], p);
+                    p = fmaf(D[m][2], sv[m][2], p); p = fmaf(D[m][3], sv[m][3], p);
+                }
+                p = allreduce_rows(p);                 // over the four lanes that share key channel j_own
+                if (g == 0) S.pc[j_own] = p;
+                const float4 p4 = *reinterpret_cast<const float4*>(&S.pc[j4]);
+                Pend[0] = p4.x; Pend[1] = p4.y; Pend[2] = p4.z; Pend[3] = p4.w;
+            }
+        }
         f32x4 dkin[2];                                 // (V dS)^T: rows j4 + v, lane = token 16 st + l16
         bf16x8 rtH, rtL;                               // R'^T of this wave's key channels: lane = j_own, K slots = tokens
         if (!exact) {
