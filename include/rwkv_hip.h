@@ -93,6 +93,8 @@ int rwkv_timex_backward_sum(void* stream, const float* w, const float* k, const 
  * wkv5_bf16/cuda/wkv5_op.cpp:5-6 (kernels: wkv5_cuda_v1b.cu:6-191).
  *   r,k,v,y,gy,gr,gk,gv[B,T,C] bf16; eew = exp(-exp(w_raw)) and ew = -exp(w_raw), fp32 [H,N]
  *   (wkv5_bf16/run.py:63-64); u[H,N] bf16; gw,gu[B,C] bf16 per-batch partials (fully written).
+ *   Backward workspace (wkv5, wkv6, wkv6_state alike): B*T*C floats (r * dr' between the two sweeps) followed by one
+ *   64x64 fp32 forward state per (b,h) and 128 tokens; private to the library, no initialisation needed.
  * ------------------------------------------------------------------------------------- */
 int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H,
                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,

@@ -357,9 +357,12 @@ int check_dims(int B, int T, int C, int H) {
     return RWKV_OK;
 }
 
+// r * dr' in fp32 [B,T,C], then the forward states that the first chunked sweep hands to the second every PCK chunks
+// (wkv6_chunk.h): [B*H][ceil(chunks / 4)][64*64] fp32
 size_t ws_bytes(int B, int T, int C, int H) {
     if (check_dims(B, T, C, H) != RWKV_OK) return 0;
-    return static_cast<size_t>(B) * T * C * sizeof(float);
+    const size_t nchunks = (static_cast<size_t>(T) + 31) / 32, npck = (nchunks + 3) / 4;
+    return static_cast<size_t>(B) * T * C * sizeof(float) + static_cast<size_t>(B) * H * npck * 64 * 64 * sizeof(float);
 }
 
 }  // namespace
@@ -388,14 +391,7 @@ int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16*
     return launch_fwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a);
 }
 
-// wkv5 adds the states that the first chunked sweep hands to the second every PCK chunks (wkv6_chunk.h)
-static size_t ws5_bytes(int B, int T, int C, int H) {
-    const size_t base = ws_bytes(B, T, C, H);
-    if (base == 0) return 0;
-    const size_t nchunks = (static_cast<size_t>(T) + 31) / 32, npck = (nchunks + 3) / 4;
-    return base + static_cast<size_t>(B) * H * npck * 64 * 64 * sizeof(float);
-}
-size_t rwkv_wkv5_backward_workspace_bytes(int B, int T, int C, int H) { return ws5_bytes(B, T, C, H); }
+size_t rwkv_wkv5_backward_workspace_bytes(int B, int T, int C, int H) { return ws_bytes(B, T, C, H); }
 
 int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                        const rwkv_bf16* v, const float* eew, const float* ew, const rwkv_bf16* u,
@@ -403,7 +399,7 @@ int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16
                        rwkv_bf16* gu, void* workspace, size_t workspace_bytes) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu})) return e;
-    if (workspace == nullptr || workspace_bytes < ws5_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
+    if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = eew; a.ew_head = ew; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);

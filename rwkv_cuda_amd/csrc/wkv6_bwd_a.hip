@@ -295,8 +295,9 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
         const int c0 = i * L;
         const SetA& O = S.set[i & 1];
         const bool exact = __builtin_amdgcn_readfirstlane(O.exact) != 0;
-        if constexpr (WMODE == W_HEAD) {
-            if (i > 0 && i % PCK == 0) {               // S at the start of chunk i, for the second sweep's P (see PCK)
+        {
+            constexpr int pck = WMODE == W_HEAD ? PCK : 4 * PCK;      // wkv5 sums G over time and needs the shorter walk
+            if (i > 0 && i % pck == 0) {               // S at the start of chunk i, for the second sweep's P (see PCK)
                 const int npck = (nchunks + PCK - 1) / PCK;
                 const float* slot = a.rdr + static_cast<size_t>(gridDim.x / a.H) * T * C + (bh * npck + i / PCK) * PCK_FLOATS;
                 store16(slot, (sw * 64 + lane) * 32, D[0]);

@@ -349,9 +349,10 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
         const int c0 = (nchunks - 1 - i) * L;
         const SetB& O = S.set[i & 1];
         const bool exact = __builtin_amdgcn_readfirstlane(O.exact) != 0;
-        if constexpr (WMODE == W_HEAD) {
+        {
+            constexpr int pck = WMODE == W_HEAD ? PCK : 4 * PCK;      // as in the first sweep
             const int cn = nchunks - i;                // the chunk after this one; D is dS at its first token
-            if (cn < nchunks && cn % PCK == 0) {       // P at that boundary from the stored S (see PCK), replacing the carried value
+            if (cn < nchunks && cn % pck == 0) {       // P at that boundary from the stored S (see PCK), replacing the carried value
                 const int npck = (nchunks + PCK - 1) / PCK;
                 const float* slot = a.rdr + static_cast<size_t>(gridDim.x / a.H) * T * C + (bh * npck + cn / PCK) * PCK_FLOATS;
                 // D[m][v] <-> sweep A's state wave (q, ih = m >> 1), register 4 (m & 1) + v.  Loaded with a scalar base and one

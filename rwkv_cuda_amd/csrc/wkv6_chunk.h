@@ -35,11 +35,13 @@ constexpr int RS = 68;            // row stride (dwords) of [token][channel] ope
 constexpr int TS = 36;            // row stride (dwords) of [channel][token] hi/lo operand arrays: 144 B
 constexpr int VS = 20;            // row stride (dwords) of the bf16 [channel][token] array: 80 B
 constexpr int STAGES = 4;         // chunks of input kept in flight
-// wkv5 sums G_t over the whole sequence, and G_t comes from P_t = sum_i dS_t[i,j] S_t[i,j], which the second sweep carries
-// backwards as P_t = P_{t+1} + r_t dr'_t - k_t dk'_t.  The two terms come from different kernels, each good to ~4e-6
-// (hi/lo bf16 products), so P random-walks and the error of sum_t G_t grows like T^1.5 (1.5 % at T = 4096, against
-// the reference's 0.2 %).  Every PCK chunks the first sweep therefore stores its state S, and the second sweep
-// recomputes P from S and its own dS at that boundary, which bounds the walk to PCK * 32 steps.
+// The decay gradient comes from P_t = sum_i dS_t[i,j] S_t[i,j], which the second sweep carries backwards as
+// P_t = P_{t+1} + r_t dr'_t - k_t dk'_t.  The two terms come from different kernels, each good to ~4e-6 (hi/lo bf16
+// products), so P random-walks: wkv6's per-token gw is 5 % worse than the reference's at T = 4096 and keeps growing, and
+// wkv5, which sums G_t over the whole sequence, collects an error ~T^1.5 (1.5 % at T = 4096 against the reference's
+// 0.2 %).  Every PCK chunks (wkv5) or 4 PCK chunks (wkv6) the first sweep therefore stores its state S, and the second
+// sweep recomputes P from S and its own dS at that boundary, which bounds the walk to 128 / 512 steps: wkv5's gw error is
+// then the reference's at any T, wkv6's within 1 % of it.  The workspace holds a slot for every PCK-th chunk in both cases.
 constexpr int PCK = 4;
 constexpr int PCK_FLOATS = 64 * 64;      // one stored state: [8 state waves of sweep A][64 lanes][8 values]
 constexpr float RANGE_LIMIT = 60.0f;
