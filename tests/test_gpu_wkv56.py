@@ -146,6 +146,32 @@ def test_wkv5_full_size_sampled_heads(lib):
             assert e < (4e-3 if name in ("gu", "gw") else 2.5e-3), (name, e)
 
 
+def test_long_sequence_is_no_worse_than_the_reference_kernel(lib):
+    """T = 4096 on one head: errors that grow with the sequence length (the running P of the decay gradient did, until
+    it was re-derived from the states every few chunks) are invisible at the small shapes above."""
+    B, T, H = 1, 4096, 1
+    C = H * 64
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=46, state=True)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u, s0)]
+    y = wkv6_state.RUN_CUDA(B, T, C, H, *t)
+    y.backward(gy.to(DEV))
+    torch.cuda.synchronize()
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, emu, [y] + [x.grad for x in t]):
+        assert_no_worse("wkv6_state T4096 " + name, a, e, g)
+
+    r, k, v, w5, u, gy = synth.wkv5_inputs(2, T, C, H, seed=47)
+    ref = O.wkv5_grads(2, T, C, H, r, k, v, w5, u, gy)
+    emu = O.emulate_wkv5_bf16(2, T, C, H, r, k, v, w5, u, gy)
+    t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w5, u)]
+    y = wkv5_bf16.RUN_CUDA(2, T, C, H, *t)
+    y.backward(gy.to(DEV))
+    torch.cuda.synchronize()
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y] + [x.grad for x in t]):
+        assert_no_worse("wkv5 T4096 " + name, a, e, g)
+
+
 def test_wkv6_fp32_ew_c_abi(lib):
     """The reference's own wkv6 boundary: the decay arrives as fp32 ew = -exp(w) (wkv6/run.py:147)."""
     B, T, H = 2, 70, 2
