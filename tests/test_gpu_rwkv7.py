@@ -107,3 +107,14 @@ def test_rwkv7_state_only_and_stateless_ops(lib, B, T, H):
     for name, a_, e, g in zip(NAMES, ref, emu, got):
         if g is not None:
             assert_no_worse("stateless op " + name, a_, e, g)
+
+
+def test_rwkv7_long_sequence_is_no_worse_than_the_reference_kernel(lib):
+    """T = 2048 on one head: the in-chunk inversion of the backward and the fp32 state must not lose accuracy with length."""
+    B, T, H = 1, 2048, 1
+    args = synth.rwkv7_inputs(B, T, H, 64, seed=34)
+    ref = O.grads(*args)
+    emu = O.emulate_bf16(*args)
+    got = _run(args)
+    for name, a, e, g in zip(NAMES, ref, emu, got):
+        assert_no_worse("rwkv7 T2048 " + name, a, e, g)
