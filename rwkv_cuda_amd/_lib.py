@@ -32,7 +32,7 @@ HIPCC_FLAGS = [
 # The backward sweep B keeps one index of its state waves' epilogue in scratch, outside the loops (three values in the
 # wkv5 instantiation, ILi0E, one of them reloaded once per chunk by a state wave); anything beyond these counts fails the
 # build.
-SPILL_LIMIT = {"wkv6_fwd_ws": 0, "wkv6_bwd_a_ws": 0, "wkv6_bwd_b_wsILi0E": 3, "wkv6_bwd_b_wsILi1E": 9, "wkv6_bwd_b_wsILi2E": 9}
+SPILL_LIMIT = {"wkv6_fwd_ws": 0, "wkv6_bwd_a_ws": 0, "wkv6_bwd_b_wsILi0E": 3, "wkv6_bwd_b_wsILi1E": 1, "wkv6_bwd_b_wsILi2E": 1}
 
 _lib = None
 
