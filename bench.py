@@ -175,6 +175,57 @@ def make_wkv5(dev):
     return step, tok, kernels, cfg, cpu_baseline, 22 * C * tok
 
 
+def make_wkv5_fp32(dev):
+    """The fp32 wkv5 op at the reference's own benchmark shape (wkv5/run.py:395-399)."""
+    from rwkv_cuda_amd import _lib
+    from rwkv_cuda_amd._call import call
+    lib = _lib.load()
+    B, T, H, N = 8, 4096, 64, 64
+    C = H * N
+    g = torch.Generator().manual_seed(42)
+    rnd = lambda *s: (torch.rand(*s, generator=g) * 2 - 1).to(dev)      # uniform(-1,1) as in wkv5/run.py:516-520
+    r, k, v, gy = rnd(B, T, C), rnd(B, T, C), rnd(B, T, C), rnd(B, T, C)
+    w, u = rnd(C), rnd(C)
+    new = lambda *s: torch.empty(s, device=dev, dtype=torch.float32)
+    y, gr, gk, gv, gw, gu = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C), new(B, C), new(B, C)
+    tok = B * T
+    ew = (-torch.exp(w)).contiguous()
+    eew = torch.exp(ew).contiguous()
+
+    def step():
+        ew_ = (-torch.exp(w)).contiguous()
+        eew_ = torch.exp(ew_).contiguous()
+        call("rwkv_wkv5f32_forward", dev, B, T, C, H, r, k, v, eew_, u, y)
+        call("rwkv_wkv5f32_backward", dev, B, T, C, H, r, k, v, eew_, ew_, u, gy, gr, gk, gv, gw, gu)
+        return torch.sum(gw, 0), torch.sum(gu, 0)
+
+    def bwd(mask):
+        def run():
+            lib.rwkv_wkv6_set_backward_passes(mask)
+            call("rwkv_wkv5f32_backward", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu)
+            lib.rwkv_wkv6_set_backward_passes(7)
+        return run
+
+    kernels = [("wkv_sweep<fwd, fp32 I/O>", lambda: call("rwkv_wkv5f32_forward", dev, B, T, C, H, r, k, v, eew, u, y), 16 * C * tok),
+               ("wkv_sweep<gr+gu+gw, fp32 I/O>", bwd(1), 20 * C * tok),       # r k v gy -> gr
+               ("wkv_sweep<gv, fp32 I/O>", bwd(2), 16 * C * tok),             # r k gy -> gv
+               ("wkv_sweep<gk, fp32 I/O>", bwd(4), 20 * C * tok)]             # r k v gy -> gk
+
+    def cpu_baseline(t_cpu=128):
+        from oracle import wkv56 as O
+        gg = torch.Generator().manual_seed(42)
+        rn = lambda *s: torch.rand(*s, generator=gg) * 2 - 1
+        a = [rn(B, t_cpu, C), rn(B, t_cpu, C), rn(B, t_cpu, C), rn(C), rn(C), rn(B, t_cpu, C)]
+        t0 = time.perf_counter()
+        O.wkv5_grads(B, t_cpu, C, H, *a, dtype=torch.float32)
+        dt = time.perf_counter() - t0
+        return B * t_cpu / dt / 1e6, f"wkv5 fwd+bwd, fp32 autograd of the recurrent form, B{B} H{H} N{N}, T_cpu={t_cpu} ({dt:.1f} s)"
+
+    cfg = {"workload": f"wkv5 fp32 fwd+bwd B{B} T{T} C{C} H{H} N{N}", "B": B, "T": T, "C": C, "H": H, "N": N,
+           "algorithmic_bytes_per_token": 44 * C}
+    return step, tok, kernels, cfg, cpu_baseline, 44 * C * tok
+
+
 def make_rwkv7(dev):
     from rwkv_cuda_amd import synth
     from rwkv_cuda_amd._call import call
@@ -301,11 +352,12 @@ WORKLOADS = {
     "wkv6": lambda dev: make_wkv6(dev, False),
     "wkv6_state": lambda dev: make_wkv6(dev, True),
     "wkv5": make_wkv5,
+    "wkv5_fp32": make_wkv5_fp32,
     "rwkv7": make_rwkv7,
     "wkv4": make_wkv4,
     "timex": make_timex,
 }
-DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "rwkv7": "bf16", "wkv4": "f32", "timex": "f32"}
+DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_fp32": "f32", "rwkv7": "bf16", "wkv4": "f32", "timex": "f32"}
 
 
 def main():

@@ -107,6 +107,23 @@ int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H,
                        void* workspace, size_t workspace_bytes);
 
 /* ---------------------------------------------------------------------------------------
+ * RWKV-5 wkv, fp32 I/O.  Replaces cuda_forward / cuda_backward of wkv5/cuda/wkv5_op.cpp:3-4
+ * (kernels: wkv5_cuda_v1e.cu and its siblings, selected by CUDA_KERNEL_VERSION in wkv5/run.py:15).
+ *   Same arguments as the bf16 op with every tensor fp32; gw,gu[B,C] fp32 per-batch partials
+ *   (wkv5/run.py:497-501 sums them over the batch).  Head size 64 only: the reference compiles N
+ *   in (wkv5/run.py:467) and benchmarks N = 64.
+ *   Runs the sequential fp32 sweeps; the decay gradient comes from the reference's own second
+ *   recurrence (dS/dw carried forward in time), so the backward needs no workspace.
+ * ------------------------------------------------------------------------------------- */
+int rwkv_wkv5f32_forward(void* stream, int B, int T, int C, int H,
+                         const float* r, const float* k, const float* v,
+                         const float* eew, const float* u, float* y);
+int rwkv_wkv5f32_backward(void* stream, int B, int T, int C, int H,
+                          const float* r, const float* k, const float* v,
+                          const float* eew, const float* ew, const float* u, const float* gy,
+                          float* gr, float* gk, float* gv, float* gw, float* gu);
+
+/* ---------------------------------------------------------------------------------------
  * RWKV-6 wkv, bf16 I/O, per-token decay.  Replaces cuda_forward / cuda_backward of
  * wkv6/cuda/wkv6_op.cpp:5-6 (kernels: wkv6_cuda_v1.cu:6-223).
  *   w = ew = -exp(w_raw), fp32 [B,T,C] (wkv6/run.py:147); the kernel applies exp(ew).

@@ -37,6 +37,8 @@ static_assert(NSTAGE <= NT && NSTAGE % 64 == 0, "staging threads are whole waves
 enum { P_FWD = 0, P_GR = 1, P_GK = 2, P_GV = 3 };
 enum { W_HEAD = 0, W_EW = 1, W_RAW = 2 };   // wkv5 (eew[H,N] fp32) / wkv6 (ew fp32 [B,T,C]) / wkv6_state (raw bf16)
 
+// Element pointers are typed for the bf16 ops; the fp32 wkv5 op stores float pointers in the same fields and its
+// kernels (F32 = true) read them back as such through load8 / store8 / load1 / store1 below.
 struct Args {
     int T, C, H;
     const uint16_t *r, *k, *v, *u, *s0, *gy;
@@ -61,21 +63,64 @@ template <int PASS> struct Smem {
     float u[N];
 };
 
-struct Staged {
-    uint4 r, k, v, g, w0, w1;
+// eight consecutive elements as they come from memory: bf16 in one 16-byte load, fp32 in two
+template <bool F32> struct Raw8;
+template <> struct Raw8<false> { uint4 q; };
+template <> struct Raw8<true> { float4 a, b; };
+
+template <bool F32> DEVINL Raw8<F32> load8(const uint16_t* p, size_t off, bool ok) {
+    Raw8<F32> x;
+    if constexpr (F32) {
+        const float* f = reinterpret_cast<const float*>(p) + off;
+        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+        x.a = ok ? *reinterpret_cast<const float4*>(f) : z;
+        x.b = ok ? *reinterpret_cast<const float4*>(f + 4) : z;
+    } else {
+        x.q = ok ? *reinterpret_cast<const uint4*>(p + off) : make_uint4(0, 0, 0, 0);
+    }
+    return x;
+}
+template <bool F32> DEVINL void widen8(const Raw8<F32>& x, float (&f)[8]) {
+    if constexpr (F32) {
+        f[0] = x.a.x; f[1] = x.a.y; f[2] = x.a.z; f[3] = x.a.w; f[4] = x.b.x; f[5] = x.b.y; f[6] = x.b.z; f[7] = x.b.w;
+    } else {
+        unpack8(x.q, f);
+    }
+}
+template <bool F32> DEVINL void store8(uint16_t* p, size_t off, const float (&f)[8]) {
+    if constexpr (F32) {
+        float* d = reinterpret_cast<float*>(p) + off;
+        *reinterpret_cast<float4*>(d) = make_float4(f[0], f[1], f[2], f[3]);
+        *reinterpret_cast<float4*>(d + 4) = make_float4(f[4], f[5], f[6], f[7]);
+    } else {
+        *reinterpret_cast<uint4*>(p + off) = pack8(f);
+    }
+}
+template <bool F32> DEVINL float load1(const uint16_t* p, size_t i) {
+    if constexpr (F32) return reinterpret_cast<const float*>(p)[i];
+    else return bf2f(p[i]);
+}
+template <bool F32> DEVINL void store1(uint16_t* p, size_t i, float x) {
+    if constexpr (F32) reinterpret_cast<float*>(p)[i] = x;
+    else p[i] = f2bf(x);
+}
+
+template <bool F32> struct Staged {
+    Raw8<F32> r, k, v, g;
+    uint4 w0, w1;
     float4 rdr0, rdr1;
 };
 
-template <int PASS, int WMODE>
-DEVINL void prefetch(Staged& p, const Args& a, size_t base, int c0, int st, int sj) {
+template <int PASS, int WMODE, bool F32>
+DEVINL void prefetch(Staged<F32>& p, const Args& a, size_t base, int c0, int st, int sj) {
     const int t = c0 + st;
     const bool ok = t < a.T;
     const size_t off = base + static_cast<size_t>(t) * a.C + sj;
     const uint4 z = make_uint4(0, 0, 0, 0);
-    p.r = ok ? *reinterpret_cast<const uint4*>(a.r + off) : z;
-    p.k = ok ? *reinterpret_cast<const uint4*>(a.k + off) : z;
-    if constexpr (PASS != P_GV) p.v = ok ? *reinterpret_cast<const uint4*>(a.v + off) : z;
-    if constexpr (PASS != P_FWD) p.g = ok ? *reinterpret_cast<const uint4*>(a.gy + off) : z;
+    p.r = load8<F32>(a.r, off, ok);
+    p.k = load8<F32>(a.k, off, ok);
+    if constexpr (PASS != P_GV) p.v = load8<F32>(a.v, off, ok);
+    if constexpr (PASS != P_FWD) p.g = load8<F32>(a.gy, off, ok);
     if constexpr (WMODE == W_RAW) {
         p.w0 = ok ? *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(a.w) + off) : z;
     } else if constexpr (WMODE == W_EW) {
@@ -83,7 +128,7 @@ DEVINL void prefetch(Staged& p, const Args& a, size_t base, int c0, int st, int 
         p.w0 = ok ? *reinterpret_cast<const uint4*>(w) : z;
         p.w1 = ok ? *reinterpret_cast<const uint4*>(w + 4) : z;
     }
-    if constexpr (PASS == P_GK) {
+    if constexpr (PASS == P_GK && !F32) {
         const float4 zf = make_float4(0.f, 0.f, 0.f, 0.f);
         p.rdr0 = ok ? *reinterpret_cast<const float4*>(a.rdr + off) : zf;
         p.rdr1 = ok ? *reinterpret_cast<const float4*>(a.rdr + off + 4) : zf;
@@ -101,16 +146,16 @@ DEVINL void ld8f(const float* src, float (&f)[8]) {
 }
 
 // registers -> LDS (fp32), plus the per-step scalar `dot`
-template <int PASS, int WMODE>
-DEVINL void commit(Smem<PASS>& S, const Staged& p, const Args& a, int c0, int st, int sj) {
+template <int PASS, int WMODE, bool F32>
+DEVINL void commit(Smem<PASS>& S, const Staged<F32>& p, const Args& a, int c0, int st, int sj) {
     const bool ok = (c0 + st) < a.T;
     float fr[8], fk[8], fv[8], fg[8];
-    unpack8(p.r, fr);
-    unpack8(p.k, fk);
+    widen8<F32>(p.r, fr);
+    widen8<F32>(p.k, fk);
     st8(&S.r[st][sj], fr);
     st8(&S.k[st][sj], fk);
-    if constexpr (PASS != P_GV) { unpack8(p.v, fv); st8(&S.v[st][sj], fv); }
-    if constexpr (PASS != P_FWD) { unpack8(p.g, fg); st8(&S.g[st][sj], fg); }
+    if constexpr (PASS != P_GV) { widen8<F32>(p.v, fv); st8(&S.v[st][sj], fv); }
+    if constexpr (PASS != P_FWD) { widen8<F32>(p.g, fg); st8(&S.g[st][sj], fg); }
     if constexpr (WMODE != W_HEAD) {
         float fw[8], dec[8];
         if constexpr (WMODE == W_RAW) {
@@ -128,7 +173,7 @@ DEVINL void commit(Smem<PASS>& S, const Staged& p, const Args& a, int c0, int st
         st8(&S.w[st][sj], dec);
         if constexpr (PASS == P_GK) st8(&S.f[st][sj], fw);
     }
-    if constexpr (PASS == P_GK) {
+    if constexpr (PASS == P_GK && !F32) {
         *reinterpret_cast<float4*>(&S.rdr[st][sj]) = p.rdr0;
         *reinterpret_cast<float4*>(&S.rdr[st][sj + 4]) = p.rdr1;
     }
@@ -144,8 +189,9 @@ DEVINL void commit(Smem<PASS>& S, const Staged& p, const Args& a, int c0, int st
     if ((threadIdx.x & 7) == 0) S.dot[st] = d;
 }
 
-template <int PASS, int WMODE>
+template <int PASS, int WMODE, bool F32 = false>
 __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
+    static_assert(!F32 || WMODE == W_HEAD, "fp32 I/O exists for wkv5 only");
     constexpr bool REV = (PASS == P_GK || PASS == P_GV);
     constexpr bool SHAPE_F = (PASS == P_FWD || PASS == P_GV);
     __shared__ Smem<PASS> S;
@@ -158,7 +204,7 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     const size_t bh = static_cast<size_t>(b) * a.H + h;
     const bool stateful = a.s0 != nullptr;
 
-    if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
+    if (tid < N) S.u[tid] = load1<F32>(a.u, h * N + tid);
 
     // ---- state registers
     float St[JW];
@@ -188,19 +234,27 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
 #pragma unroll
     for (int e = 0; e < 8; ++e) gu_acc[e] = 0.f;
     float P = 0.f, gw_acc = 0.f;                            // GK scan state (threads < 64)
+    // fp32 I/O: the P recurrence above loses a digit per decade of T to cancellation, which bf16 outputs hide and
+    // fp32 outputs do not.  GR carries Q = dS/dw instead (Q_{t+1} = S_t + w Q_t, the reference's second recurrence,
+    // wkv5/run.py:249-252) and sums gw[j] = sum_t r_t[j] sum_i gy_t[i] Q_t[i,j] per lane; GK then makes gk only.
+    constexpr bool DIRECT_GW = F32 && PASS == P_GR;
+    constexpr bool SCAN_GW = !F32 && PASS == P_GK;
+    float Q[DIRECT_GW ? JW : 1];
+#pragma unroll
+    for (int e = 0; e < (DIRECT_GW ? JW : 1); ++e) Q[e] = 0.f;
 
     const int nchunks = (a.T + TC - 1) / TC;
     const bool stager = tid < NSTAGE;                       // whole waves
-    Staged pre;
-    if (stager) prefetch<PASS, WMODE>(pre, a, base, (REV ? nchunks - 1 : 0) * TC, st, sj);
+    Staged<F32> pre;
+    if (stager) prefetch<PASS, WMODE, F32>(pre, a, base, (REV ? nchunks - 1 : 0) * TC, st, sj);
     __syncthreads();                                        // S.u visible
 
     for (int ci = 0; ci < nchunks; ++ci) {
         const int c0 = (REV ? nchunks - 1 - ci : ci) * TC;
         __syncthreads();                                    // previous epilogue is done with LDS
-        if (stager) commit<PASS, WMODE>(S, pre, a, c0, st, sj);
+        if (stager) commit<PASS, WMODE, F32>(S, pre, a, c0, st, sj);
         __syncthreads();
-        if (stager && ci + 1 < nchunks) prefetch<PASS, WMODE>(pre, a, base, (REV ? nchunks - 2 - ci : ci + 1) * TC, st, sj);
+        if (stager && ci + 1 < nchunks) prefetch<PASS, WMODE, F32>(pre, a, base, (REV ? nchunks - 2 - ci : ci + 1) * TC, st, sj);
 
         // ---- TC sequential steps
 #pragma unroll 4
@@ -222,11 +276,18 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
                 const float xv = (PASS == P_GR) ? S.v[t][rowslot] : S.g[t][rowslot];
                 const float bl = (PASS == P_GR) ? S.k[t][lane] : S.r[t][lane];
                 const float wl = (WMODE == W_HEAD) ? w_const : S.w[t][lane];
+                float acc2 = 0.f;
                 static_for<JW>([&](auto I) {
-                    fmac_bc<decltype(I)::value>(acc, av, St[decltype(I)::value]);
-                    St[decltype(I)::value] *= wl;
-                    fmac_bc<decltype(I)::value>(St[decltype(I)::value], xv, bl);
+                    constexpr int i = decltype(I)::value;
+                    fmac_bc<i>(acc, av, St[i]);
+                    if constexpr (DIRECT_GW) {
+                        fmac_bc<i>(acc2, av, Q[i]);
+                        Q[i] = fmaf(Q[i], wl, St[i]);
+                    }
+                    St[i] *= wl;
+                    fmac_bc<i>(St[i], xv, bl);
                 });
+                if constexpr (DIRECT_GW) gw_acc = fmaf(S.r[t][lane], acc2, gw_acc);
             }
             S.part[q][t][lane] = acc;
         }
@@ -250,11 +311,11 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
         if constexpr (PASS == P_FWD) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) out[e] = fmaf(S.v[es][sj + e], dot, sum[e]);
-            if (ok) *reinterpret_cast<uint4*>(a.y + off) = pack8(out);
+            if (ok) store8<F32>(a.y, off, out);
         } else if constexpr (PASS == P_GV) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) out[e] = fmaf(S.g[es][sj + e], dot, sum[e]);
-            if (ok) *reinterpret_cast<uint4*>(a.gv + off) = pack8(out);
+            if (ok) store8<F32>(a.gv, off, out);
         } else if constexpr (PASS == P_GR) {
             float rdr[8];
 #pragma unroll
@@ -265,9 +326,11 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
                 gu_acc[e] = fmaf(rr * kk, dot, gu_acc[e]);
             }
             if (ok) {
-                *reinterpret_cast<uint4*>(a.gr + off) = pack8(out);
-                *reinterpret_cast<float4*>(a.rdr + off) = make_float4(rdr[0], rdr[1], rdr[2], rdr[3]);
-                *reinterpret_cast<float4*>(a.rdr + off + 4) = make_float4(rdr[4], rdr[5], rdr[6], rdr[7]);
+                store8<F32>(a.gr, off, out);
+                if constexpr (!F32) {
+                    *reinterpret_cast<float4*>(a.rdr + off) = make_float4(rdr[0], rdr[1], rdr[2], rdr[3]);
+                    *reinterpret_cast<float4*>(a.rdr + off + 4) = make_float4(rdr[4], rdr[5], rdr[6], rdr[7]);
+                }
             }
         } else {  // P_GK
             float kdk[8];
@@ -276,7 +339,8 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
                 out[e] = fmaf(S.u[sj + e] * S.r[es][sj + e], dot, sum[e]);
                 kdk[e] = S.k[es][sj + e] * sum[e];
             }
-            if (ok) *reinterpret_cast<uint4*>(a.gk + off) = pack8(out);
+            if (ok) store8<F32>(a.gk, off, out);
+            if constexpr (SCAN_GW) {
             if (stager) st8(&S.k[st][sj], kdk);              // k is no longer needed: keep k*dk' there
             __syncthreads();
             if (tid < N) {                                   // per-channel scan over the chunk, t descending
@@ -291,7 +355,8 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
             if constexpr (WMODE != W_HEAD) {
                 __syncthreads();
                 ld8f(&S.part[0][es][sj], out);
-                if (ok) *reinterpret_cast<uint4*>(a.gw + off) = pack8(out);
+                if (ok) store8<F32>(a.gw, off, out);
+            }
             }
         }
     }
@@ -305,12 +370,24 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
             float s = 0.f;
 #pragma unroll 8
             for (int t = 0; t < TC; ++t) s += S.part[0][t][tid];
-            a.gu[static_cast<size_t>(b) * a.C + h * N + tid] = f2bf(s);
+            store1<F32>(a.gu, static_cast<size_t>(b) * a.C + h * N + tid, s);
+        }
+        if constexpr (DIRECT_GW) {
+            __syncthreads();
+            S.part[q][0][lane] = gw_acc;
+            __syncthreads();
+            if (tid < N) {
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) s += S.part[w][0][tid];
+                const float eew = static_cast<const float*>(a.w)[h * N + tid];   // d eew / d w_raw = eew * ew
+                store1<F32>(a.gw, static_cast<size_t>(b) * a.C + h * N + tid, a.ew_head[h * N + tid] * eew * s);
+            }
         }
     }
     if constexpr (PASS == P_GK) {
-        if constexpr (WMODE == W_HEAD) {
-            if (tid < N) a.gw[static_cast<size_t>(b) * a.C + h * N + tid] = f2bf(a.ew_head[h * N + tid] * gw_acc);
+        if constexpr (WMODE == W_HEAD && SCAN_GW) {
+            if (tid < N) store1<F32>(a.gw, static_cast<size_t>(b) * a.C + h * N + tid, a.ew_head[h * N + tid] * gw_acc);
         }
         if (a.gs != nullptr) {
 #pragma unroll
@@ -404,6 +481,40 @@ int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = eew; a.ew_head = ew; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
     return launch_bwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a, g_bwd_passes);
+}
+
+// ---- wkv5, fp32 I/O: the sequential fp32 sweeps only (the chunked kernels work to bf16-I/O accuracy)
+namespace {
+const uint16_t* as_elems(const float* p) { return reinterpret_cast<const uint16_t*>(p); }
+uint16_t* out_elems(float* p) { return reinterpret_cast<uint16_t*>(p); }
+}  // namespace
+
+int rwkv_wkv5f32_forward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
+                         const float* eew, const float* u, float* y) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, eew, u, y})) return e;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew; a.u = as_elems(u);
+    a.y = out_elems(y);
+    hipLaunchKernelGGL((wkv_sweep<P_FWD, W_HEAD, true>), dim3(B * H), dim3(NT), 0, static_cast<hipStream_t>(stream), a);
+    return launch_status();
+}
+
+int rwkv_wkv5f32_backward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
+                          const float* eew, const float* ew, const float* u, const float* gy, float* gr, float* gk,
+                          float* gv, float* gw, float* gu) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu})) return e;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew; a.ew_head = ew;
+    a.u = as_elems(u); a.gy = as_elems(gy); a.gr = out_elems(gr); a.gk = out_elems(gk); a.gv = out_elems(gv);
+    a.gw = out_elems(gw); a.gu = out_elems(gu);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // three independent sweeps: gr + gu + gw, gv, gk
+    if (g_bwd_passes & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
+    if (g_bwd_passes & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
+    if (g_bwd_passes & RWKV_PASS_GK) hipLaunchKernelGGL((wkv_sweep<P_GK, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
+    return launch_status();
 }
 
 int rwkv_wkv6_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
