@@ -226,6 +226,57 @@ def make_wkv5_fp32(dev):
     return step, tok, kernels, cfg, cpu_baseline, 44 * C * tok
 
 
+def make_wkv5a(dev):
+    """wkv5a (two-sided decay and bonus, fp32) at the reference's timing shape (wkv5a/run.py:62-66)."""
+    from rwkv_cuda_amd import _lib
+    from rwkv_cuda_amd._call import call
+    lib = _lib.load()
+    B, T, H, N = 8, 4096, 64, 64
+    C = H * N
+    g = torch.Generator().manual_seed(42)
+    rnd = lambda *s, lo=-1.0: (torch.rand(*s, generator=g) * (1.0 - lo) + lo).to(dev)   # wkv5a/run.py:389-398
+    r, k, v, gy = rnd(B, T, C), rnd(B, T, C), rnd(B, T, C), rnd(B, T, C)
+    w1, u1, w2, u2 = rnd(H, N, lo=-8.0), rnd(H, N), rnd(H, N, lo=-8.0), rnd(H, N)
+    new = lambda *s: torch.empty(s, device=dev, dtype=torch.float32)
+    y, gr, gk, gv = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C)
+    gw1, gu1, gw2, gu2 = new(B, C), new(B, C), new(B, C), new(B, C)
+    tok = B * T
+    dec = lambda w: ((-torch.exp(w)).contiguous(), torch.exp(-torch.exp(w)).contiguous())
+    (ew1, eew1), (ew2, eew2) = dec(w1), dec(w2)
+
+    def step():
+        (a1, b1), (a2, b2) = dec(w1), dec(w2)
+        call("rwkv_wkv5a_forward", dev, B, T, C, H, r, k, v, b1, u1, b2, u2, y)
+        call("rwkv_wkv5a_backward", dev, B, T, C, H, r, k, v, b1, a1, u1, b2, a2, u2, gy, gr, gk, gv, gw1, gu1, gw2, gu2)
+        return torch.sum(gw1, 0), torch.sum(gu1, 0), torch.sum(gw2, 0), torch.sum(gu2, 0)
+
+    def bwd(mask):
+        def run():
+            lib.rwkv_wkv6_set_backward_passes(mask)
+            call("rwkv_wkv5a_backward", dev, B, T, C, H, r, k, v, eew1, ew1, u1, eew2, ew2, u2, gy, gr, gk, gv, gw1, gu1, gw2, gu2)
+            lib.rwkv_wkv6_set_backward_passes(7)
+        return run
+
+    kernels = [("wkv_sweep<fwd, two-sided>", lambda: call("rwkv_wkv5a_forward", dev, B, T, C, H, r, k, v, eew1, u1, eew2, u2, y), 16 * C * tok),
+               ("wkv_sweep<gr+gu+gw, two-sided>", bwd(1), 20 * C * tok),
+               ("wkv_sweep<gv, two-sided>", bwd(2), 16 * C * tok),
+               ("wkv_sweep<gk, two-sided>", bwd(4), 20 * C * tok)]
+
+    def cpu_baseline(t_cpu=128):
+        from oracle import wkv5a as A
+        gg = torch.Generator().manual_seed(42)
+        rn = lambda *s, lo=-1.0: torch.rand(*s, generator=gg) * (1.0 - lo) + lo
+        a = [rn(B, t_cpu, C), rn(B, t_cpu, C), rn(B, t_cpu, C), rn(H, N, lo=-8.0), rn(H, N), rn(H, N, lo=-8.0), rn(H, N), rn(B, t_cpu, C)]
+        t0 = time.perf_counter()
+        A.grads(B, t_cpu, C, H, *a, dtype=torch.float32)
+        dt = time.perf_counter() - t0
+        return B * t_cpu / dt / 1e6, f"wkv5a fwd+bwd, fp32 autograd of the recurrent form, B{B} H{H} N{N}, T_cpu={t_cpu} ({dt:.1f} s)"
+
+    cfg = {"workload": f"wkv5a fp32 fwd+bwd B{B} T{T} C{C} H{H} N{N}", "B": B, "T": T, "C": C, "H": H, "N": N,
+           "algorithmic_bytes_per_token": 44 * C}
+    return step, tok, kernels, cfg, cpu_baseline, 44 * C * tok
+
+
 def make_rwkv7(dev):
     from rwkv_cuda_amd import synth
     from rwkv_cuda_amd._call import call
@@ -353,11 +404,12 @@ WORKLOADS = {
     "wkv6_state": lambda dev: make_wkv6(dev, True),
     "wkv5": make_wkv5,
     "wkv5_fp32": make_wkv5_fp32,
+    "wkv5a": make_wkv5a,
     "rwkv7": make_rwkv7,
     "wkv4": make_wkv4,
     "timex": make_timex,
 }
-DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_fp32": "f32", "rwkv7": "bf16", "wkv4": "f32", "timex": "f32"}
+DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "wkv4": "f32", "timex": "f32"}
 
 
 def main():

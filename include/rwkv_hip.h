@@ -124,6 +124,23 @@ int rwkv_wkv5f32_backward(void* stream, int B, int T, int C, int H,
                           float* gr, float* gk, float* gv, float* gw, float* gu);
 
 /* ---------------------------------------------------------------------------------------
+ * wkv5a: RWKV-5 wkv with two-sided decay and bonus, fp32.  Replaces cuda_forward / cuda_backward of
+ * wkv5a/cuda/wkv5a_op.cpp:6-7 (kernels: wkv5a_cuda_v1a2.cu:7-222; DTYPE = float, :5).
+ *   State element [i = value channel][j = key channel] decays by eew1[j] * eew2[i] and the current
+ *   token's bonus is u1[j] + u2[i].  eewX = exp(-exp(wX_raw)), ewX = -exp(wX_raw), fp32 [H,N]
+ *   (wkv5a/run.py:123-126); gw1,gu1,gw2,gu2[B,C] fp32 per-batch partials w.r.t. the raw parameters
+ *   (summed over the batch by the wrapper, wkv5a/run.py:150-153).  Head size 64.  No workspace.
+ * ------------------------------------------------------------------------------------- */
+int rwkv_wkv5a_forward(void* stream, int B, int T, int C, int H,
+                       const float* r, const float* k, const float* v,
+                       const float* eew1, const float* u1, const float* eew2, const float* u2, float* y);
+int rwkv_wkv5a_backward(void* stream, int B, int T, int C, int H,
+                        const float* r, const float* k, const float* v,
+                        const float* eew1, const float* ew1, const float* u1,
+                        const float* eew2, const float* ew2, const float* u2, const float* gy,
+                        float* gr, float* gk, float* gv, float* gw1, float* gu1, float* gw2, float* gu2);
+
+/* ---------------------------------------------------------------------------------------
  * RWKV-6 wkv, bf16 I/O, per-token decay.  Replaces cuda_forward / cuda_backward of
  * wkv6/cuda/wkv6_op.cpp:5-6 (kernels: wkv6_cuda_v1.cu:6-223).
  *   w = ew = -exp(w_raw), fp32 [B,T,C] (wkv6/run.py:147); the kernel applies exp(ew).

@@ -16,6 +16,7 @@ Modules
   wkv4     RWKV-4 wkv (fp32)                       wkv/run.py, wkv/cuda/wkv_cuda_v2.cu
   timex    depthwise_conv1d                        depthwise_conv1d/run.py, cuda/timex_cuda_v0.cu
   wkv56    wkv5 / wkv6 / wkv6_state (bf16 I/O)     wkv5/run.py, wkv6/run.py, wkv6_state/run.py (+ kernels)
+  wkv5a    wkv5 with two-sided decay/bonus (fp32)   wkv5a/run.py (+ wkv5a_cuda_v1a2.cu)
   rwkv7    rwkv7 clamp-w with state passing        rwkv7_fast_fused/rwkv7_cuda_benchmark_state_passing.py (+ kernel)
 """
 

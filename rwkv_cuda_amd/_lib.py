@@ -87,6 +87,8 @@ SIGNATURES = {
     "rwkv_wkv5_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_P, _Z]),
     "rwkv_wkv5f32_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
     "rwkv_wkv5f32_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12),
+    "rwkv_wkv5a_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 8),
+    "rwkv_wkv5a_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 17),
     "rwkv_wkv6_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
     "rwkv_wkv6_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv6_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z]),

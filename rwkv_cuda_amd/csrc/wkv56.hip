@@ -45,6 +45,10 @@ struct Args {
     const void* w;        // W_HEAD: const float* eew[H*N]; W_EW: const float* ew[B*T*C]; W_RAW: const uint16_t* raw
     const float* ew_head; // W_HEAD, GK only: -exp(w_raw) [H*N]
     uint16_t *y, *gr, *gk, *gv, *gw, *gu, *gs;
+    // two-sided decay and bonus (wkv5a): decay w[j] * w2[i], bonus u[j] + u2[i], i = value channel
+    const float *w2, *ew2_head;
+    const uint16_t* u2;
+    uint16_t *gw2, *gu2;
     float* rdr;           // workspace [B,T,C] fp32: r * dr'
 };
 
@@ -61,6 +65,8 @@ template <int PASS> struct Smem {
     float part[NW][TC][N];
     float dot[TC];
     float u[N];
+    float dot2[TC], dot3[TC];      // two-sided mode only
+    float u2[N], w2[N];
 };
 
 // eight consecutive elements as they come from memory: bf16 in one 16-byte load, fp32 in two
@@ -146,7 +152,7 @@ DEVINL void ld8f(const float* src, float (&f)[8]) {
 }
 
 // registers -> LDS (fp32), plus the per-step scalar `dot`
-template <int PASS, int WMODE, bool F32>
+template <int PASS, int WMODE, bool F32, bool TWO>
 DEVINL void commit(Smem<PASS>& S, const Staged<F32>& p, const Args& a, int c0, int st, int sj) {
     const bool ok = (c0 + st) < a.T;
     float fr[8], fk[8], fv[8], fg[8];
@@ -187,11 +193,36 @@ DEVINL void commit(Smem<PASS>& S, const Staged<F32>& p, const Args& a, int c0, i
     }
     d = group_sum<8>(d);
     if ((threadIdx.x & 7) == 0) S.dot[st] = d;
+    if constexpr (TWO) {
+        // the bonus (u[j] + u2[i]) splits into the one-sided term above and a second scalar per step
+        float d2 = 0.f;
+        if constexpr (PASS == P_FWD || PASS == P_GV) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) d2 = fmaf(fr[e], fk[e], d2);                   // sum_j r k
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) d2 = fmaf(fv[e] * S.u2[sj + e], fg[e], d2);    // sum_i u2 v gy
+        }
+        d2 = group_sum<8>(d2);
+        if ((threadIdx.x & 7) == 0) S.dot2[st] = d2;
+        if constexpr (PASS == P_GR) {
+            float d3 = 0.f, g2[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                d3 = fmaf(fr[e], fk[e], d3);                                           // sum_j r k, for gu2
+                g2[e] = fg[e] * S.w2[sj + e];                                          // w2[i] gy[i], for gw
+            }
+            d3 = group_sum<8>(d3);
+            if ((threadIdx.x & 7) == 0) S.dot3[st] = d3;
+            st8(&S.w[st][sj], g2);                         // the per-token decay rows are free in this mode
+        }
+    }
 }
 
-template <int PASS, int WMODE, bool F32 = false>
+template <int PASS, int WMODE, bool F32 = false, bool TWO = false>
 __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     static_assert(!F32 || WMODE == W_HEAD, "fp32 I/O exists for wkv5 only");
+    static_assert(!TWO || F32, "the two-sided op is fp32 only, as in the reference (wkv5a_cuda_v1a2.cu:5)");
     constexpr bool REV = (PASS == P_GK || PASS == P_GV);
     constexpr bool SHAPE_F = (PASS == P_FWD || PASS == P_GV);
     __shared__ Smem<PASS> S;
@@ -205,6 +236,12 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     const bool stateful = a.s0 != nullptr;
 
     if (tid < N) S.u[tid] = load1<F32>(a.u, h * N + tid);
+    if constexpr (TWO) {
+        if (tid < N) {
+            S.u2[tid] = load1<F32>(a.u2, h * N + tid);
+            S.w2[tid] = a.w2[h * N + tid];
+        }
+    }
 
     // ---- state registers
     float St[JW];
@@ -229,6 +266,30 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
         const float* eew = static_cast<const float*>(a.w) + h * N;
         w_const = SHAPE_F ? eew[rowslot] : eew[lane];
     }
+#pragma unroll
+    for (int e = 0; e < JW; ++e) asm volatile("" : "+v"(St[e]));
+    // Values loaded here are first used inside the step loop.  Left alone, the compiler waits for them there, with a
+    // vmcnt(0) in every chunk that also waits for the next chunk's prefetch (issued just before the steps) and so
+    // serialises load latency with compute.  Pinning them to a register now puts the wait up here, once.
+    asm volatile("" : "+v"(w_const));
+    // time-constant decays that vary along the in-register axis live in registers (a plain multiply instead of a
+    // row-broadcast one): w[j] in shape F, and every element's w[j] * w2[i] of the two-sided op
+    constexpr bool REGW = TWO || (WMODE == W_HEAD && SHAPE_F);
+    float wreg[REGW ? JW : 1];
+    if constexpr (TWO) {
+        const float* w1 = static_cast<const float*>(a.w) + h * N;
+        const float* w2 = a.w2 + h * N;
+#pragma unroll
+        for (int e = 0; e < JW; ++e) wreg[e] = SHAPE_F ? w1[q * JW + e] * w2[lane] : w1[lane] * w2[q * JW + e];
+    } else if constexpr (REGW) {
+        const float* eew = static_cast<const float*>(a.w) + h * N;
+#pragma unroll
+        for (int e = 0; e < JW; ++e) wreg[e] = eew[q * JW + e];
+    }
+    if constexpr (REGW) {
+#pragma unroll
+        for (int e = 0; e < JW; ++e) asm volatile("" : "+v"(wreg[e]));
+    }
 
     float gu_acc[8];
 #pragma unroll
@@ -242,17 +303,26 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     float Q[DIRECT_GW ? JW : 1];
 #pragma unroll
     for (int e = 0; e < (DIRECT_GW ? JW : 1); ++e) Q[e] = 0.f;
+    // two-sided: with gW[i,j] = sum_t gy_t[i] r_t[j] Q_t[i,j], gw1[j] = sum_i w2[i] gW[i,j] stays a per-lane sum
+    // (the broadcast operand becomes w2[i] gy[i]); gw2[i] = sum_j w1[j] gW[i,j] is kept per state element in A and
+    // summed over the lanes once, at the end.
+    constexpr bool GW2 = TWO && PASS == P_GR;
+    float A[GW2 ? JW : 1], gu2_acc[8];
+#pragma unroll
+    for (int e = 0; e < (GW2 ? JW : 1); ++e) A[e] = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) gu2_acc[e] = 0.f;
 
     const int nchunks = (a.T + TC - 1) / TC;
     const bool stager = tid < NSTAGE;                       // whole waves
     Staged<F32> pre;
     if (stager) prefetch<PASS, WMODE, F32>(pre, a, base, (REV ? nchunks - 1 : 0) * TC, st, sj);
-    __syncthreads();                                        // S.u visible
+    __syncthreads();                                        // S.u (u2, w2) visible
 
     for (int ci = 0; ci < nchunks; ++ci) {
         const int c0 = (REV ? nchunks - 1 - ci : ci) * TC;
         __syncthreads();                                    // previous epilogue is done with LDS
-        if (stager) commit<PASS, WMODE, F32>(S, pre, a, c0, st, sj);
+        if (stager) commit<PASS, WMODE, F32, TWO>(S, pre, a, c0, st, sj);
         __syncthreads();
         if (stager && ci + 1 < nchunks) prefetch<PASS, WMODE, F32>(pre, a, base, (REV ? nchunks - 2 - ci : ci + 1) * TC, st, sj);
 
@@ -268,7 +338,8 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
                 const float x = (PASS == P_FWD) ? S.v[t][lane] : S.g[t][lane];
                 static_for<JW>([&](auto J) {
                     fmac_bc<decltype(J)::value>(acc, av, St[decltype(J)::value]);
-                    mul_bc<decltype(J)::value>(St[decltype(J)::value], wv);
+                    if constexpr (REGW) St[decltype(J)::value] *= wreg[decltype(J)::value];
+                    else mul_bc<decltype(J)::value>(St[decltype(J)::value], wv);
                     fmac_bc<decltype(J)::value>(St[decltype(J)::value], bv, x);
                 });
             } else {
@@ -276,15 +347,21 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
                 const float xv = (PASS == P_GR) ? S.v[t][rowslot] : S.g[t][rowslot];
                 const float bl = (PASS == P_GR) ? S.k[t][lane] : S.r[t][lane];
                 const float wl = (WMODE == W_HEAD) ? w_const : S.w[t][lane];
-                float acc2 = 0.f;
+                float acc2 = 0.f, g2 = 0.f, w1r = 0.f;
+                if constexpr (GW2) {
+                    g2 = S.w[t][rowslot];                       // w2[i] gy[i]
+                    w1r = w_const * S.r[t][lane];               // w1[j] r[j]
+                }
                 static_for<JW>([&](auto I) {
                     constexpr int i = decltype(I)::value;
+                    const float dec = TWO ? wreg[TWO ? i : 0] : wl;
                     fmac_bc<i>(acc, av, St[i]);
                     if constexpr (DIRECT_GW) {
-                        fmac_bc<i>(acc2, av, Q[i]);
-                        Q[i] = fmaf(Q[i], wl, St[i]);
+                        fmac_bc<i>(acc2, GW2 ? g2 : av, Q[i]);
+                        if constexpr (GW2) fmac_bc<i>(A[i], av, Q[i] * w1r);
+                        Q[i] = fmaf(Q[i], dec, St[i]);
                     }
-                    St[i] *= wl;
+                    St[i] *= dec;
                     fmac_bc<i>(St[i], xv, bl);
                 });
                 if constexpr (DIRECT_GW) gw_acc = fmaf(S.r[t][lane], acc2, gw_acc);
@@ -310,20 +387,21 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
         float out[8];
         if constexpr (PASS == P_FWD) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) out[e] = fmaf(S.v[es][sj + e], dot, sum[e]);
+            for (int e = 0; e < 8; ++e) out[e] = fmaf(S.v[es][sj + e], TWO ? fmaf(S.u2[sj + e], S.dot2[es], dot) : dot, sum[e]);
             if (ok) store8<F32>(a.y, off, out);
         } else if constexpr (PASS == P_GV) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) out[e] = fmaf(S.g[es][sj + e], dot, sum[e]);
+            for (int e = 0; e < 8; ++e) out[e] = fmaf(S.g[es][sj + e], TWO ? fmaf(S.u2[sj + e], S.dot2[es], dot) : dot, sum[e]);
             if (ok) store8<F32>(a.gv, off, out);
         } else if constexpr (PASS == P_GR) {
             float rdr[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float rr = S.r[es][sj + e], kk = S.k[es][sj + e];
-                out[e] = fmaf(S.u[sj + e] * kk, dot, sum[e]);
+                out[e] = TWO ? fmaf(kk, fmaf(S.u[sj + e], dot, S.dot2[es]), sum[e]) : fmaf(S.u[sj + e] * kk, dot, sum[e]);
                 rdr[e] = rr * sum[e];
                 gu_acc[e] = fmaf(rr * kk, dot, gu_acc[e]);
+                if constexpr (TWO) gu2_acc[e] = fmaf(S.v[es][sj + e] * S.g[es][sj + e], S.dot3[es], gu2_acc[e]);
             }
             if (ok) {
                 store8<F32>(a.gr, off, out);
@@ -336,7 +414,8 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
             float kdk[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                out[e] = fmaf(S.u[sj + e] * S.r[es][sj + e], dot, sum[e]);
+                out[e] = TWO ? fmaf(S.r[es][sj + e], fmaf(S.u[sj + e], dot, S.dot2[es]), sum[e])
+                             : fmaf(S.u[sj + e] * S.r[es][sj + e], dot, sum[e]);
                 kdk[e] = S.k[es][sj + e] * sum[e];
             }
             if (ok) store8<F32>(a.gk, off, out);
@@ -382,6 +461,26 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
                 for (int w = 0; w < NW; ++w) s += S.part[w][0][tid];
                 const float eew = static_cast<const float*>(a.w)[h * N + tid];   // d eew / d w_raw = eew * ew
                 store1<F32>(a.gw, static_cast<size_t>(b) * a.C + h * N + tid, a.ew_head[h * N + tid] * eew * s);
+            }
+        }
+        if constexpr (TWO) {
+            __syncthreads();
+            if (stager) st8(&S.part[0][st][sj], gu2_acc);
+            __syncthreads();
+            if (tid < N) {
+                float s = 0.f;
+#pragma unroll 8
+                for (int t = 0; t < TC; ++t) s += S.part[0][t][tid];
+                store1<F32>(a.gu2, static_cast<size_t>(b) * a.C + h * N + tid, s);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < JW; ++e) S.part[q][e][lane] = A[GW2 ? e : 0];     // [wave][i within the wave][j]
+            __syncthreads();
+            if (tid < N) {                                                        // tid = i
+                float s = 0.f;
+                for (int j = 0; j < N; ++j) s += S.part[tid / JW][tid % JW][(j + tid) & (N - 1)];
+                store1<F32>(a.gw2, static_cast<size_t>(b) * a.C + h * N + tid, a.ew2_head[h * N + tid] * a.w2[h * N + tid] * s);
             }
         }
     }
@@ -514,6 +613,37 @@ int rwkv_wkv5f32_backward(void* stream, int B, int T, int C, int H, const float*
     if (g_bwd_passes & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
     if (g_bwd_passes & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
     if (g_bwd_passes & RWKV_PASS_GK) hipLaunchKernelGGL((wkv_sweep<P_GK, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
+    return launch_status();
+}
+
+// ---- wkv5a: two-sided decay and bonus, fp32, on the same sweeps
+int rwkv_wkv5a_forward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
+                       const float* eew1, const float* u1, const float* eew2, const float* u2, float* y) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, eew1, u1, eew2, u2, y})) return e;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew1; a.u = as_elems(u1);
+    a.w2 = eew2; a.u2 = as_elems(u2); a.y = out_elems(y);
+    hipLaunchKernelGGL((wkv_sweep<P_FWD, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, static_cast<hipStream_t>(stream), a);
+    return launch_status();
+}
+
+int rwkv_wkv5a_backward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
+                        const float* eew1, const float* ew1, const float* u1, const float* eew2, const float* ew2,
+                        const float* u2, const float* gy, float* gr, float* gk, float* gv, float* gw1, float* gu1,
+                        float* gw2, float* gu2) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, eew1, ew1, u1, eew2, ew2, u2, gy, gr, gk, gv, gw1, gu1, gw2, gu2})) return e;
+    Args a{};
+    a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew1; a.ew_head = ew1;
+    a.u = as_elems(u1); a.w2 = eew2; a.ew2_head = ew2; a.u2 = as_elems(u2); a.gy = as_elems(gy);
+    a.gr = out_elems(gr); a.gk = out_elems(gk); a.gv = out_elems(gv);
+    a.gw = out_elems(gw1); a.gu = out_elems(gu1); a.gw2 = out_elems(gw2); a.gu2 = out_elems(gu2);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // three independent sweeps: gr + gu1 + gu2 + gw1 + gw2, gv, gk
+    if (g_bwd_passes & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);
+    if (g_bwd_passes & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);
+    if (g_bwd_passes & RWKV_PASS_GK) hipLaunchKernelGGL((wkv_sweep<P_GK, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);
     return launch_status();
 }
 

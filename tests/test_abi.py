@@ -20,7 +20,7 @@ def _declared_symbols():
 
 def test_header_and_bindings_agree(lib):
     names = _declared_symbols()
-    assert len(names) == 30
+    assert len(names) == 32
     assert sorted(_lib.SIGNATURES) == names
     for n in names:
         assert hasattr(lib, n), f"{n} declared in rwkv_hip.h but not exported"
@@ -60,6 +60,8 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.rwkv_wkv6state_backward(None, 2, 8, 128, 2, *([p] * 13), p, need - 1) == -4
     assert lib.rwkv_wkv6_backward_workspace_bytes(1, 1, 96, 1) == 0
     assert lib.rwkv_wkv5f32_backward(None, 2, 8, 128, 2, *([p] * 11), None) == -2
+    assert lib.rwkv_wkv5a_forward(None, 1, 8, 96, 1, *([p] * 8)) == -1
+    assert lib.rwkv_wkv5a_backward(None, 2, 8, 128, 2, *([p] * 16), p + 4) == -3
     assert lib.rwkv_wkv4_backward(None, 1, 4, 4, *([p] * 9), None, 0) == -4
     with pytest.raises(_lib.RwkvHipError):
         _lib.check(-1)
