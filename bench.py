@@ -36,6 +36,11 @@ TRAFFIC_MEASURED = {
     "wkv6_fwd_ws": 537e6 + 134e6,
     "wkv6_bwd_a_ws": 671e6 + 432e6,
     "wkv6_bwd_b_ws": 970e6 + 403e6,
+    # profiles/wkv5_ws_kernels_B8_T4096_C2048.md
+    "wkv6_bwd_b_ws<head decay>": 936e6 + 269e6,
+    # profiles/wkv5_fp32_sweep_kernels_B8_T4096_C4096.md, profiles/wkv5a_sweep_kernels_B8_T4096_C4096.md
+    "wkv_sweep<gr+gu+gw, fp32 I/O>": 2148e6 + 537e6,
+    "wkv_sweep<gr+gu+gw, two-sided>": 2148e6 + 537e6,
 }
 
 
