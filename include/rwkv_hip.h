@@ -225,8 +225,8 @@ int rwkv7_statepassing_backward(void* stream, int B, int T, int H,
  *                    cuda_backward of rwkv7_fast_fused/cuda/rwkv7_state_clampw.cpp:10,17.
  *   rwkv7_forward / rwkv7_backward : zero initial state, no state outputs.  Replaces cuda_forward /
  *                    cuda_backward of rwkv7_fast_fused/cuda/rwkv7_clampw.cpp:10,17.
- * Argument order is the reference's after the leading stream; bf16 mode only (the reference's -D_FP32_ build of the
- * same files is not provided). */
+ * Argument order is the reference's after the leading stream.  These are the bf16 mode; the *_f32 entry points below
+ * are the reference's -D_FP32_ build. */
 int rwkv7_state_forward(void* stream, int B, int T, int H,
                         const float* s0, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
                         const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b,
@@ -246,6 +246,35 @@ int rwkv7_backward(void* stream, int B, int T, int H,
                    const float* s, const float* sa,
                    rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv,
                    rwkv_bf16* da, rwkv_bf16* db);
+
+/* fp32 I/O for the three rwkv7 ops: what the reference builds from the same sources with -D_FP32_, where `bf` is float
+ * (rwkv7_clampw.cu:3-7, rwkv7_cuda_benchmark.py:102-126, and the same lines of the _state and _state_passing siblings).
+ * Same arguments as the bf16 entry points with every bf16 tensor fp32; same kernels and fp32 arithmetic. */
+int rwkv7_statepassing_forward_f32(void* stream, int B, int T, int H,
+                                   const float* s0, const float* r, const float* w, const float* k,
+                                   const float* v, const float* a, const float* b,
+                                   float* y, float* sT, float* s, float* sa);
+int rwkv7_statepassing_backward_f32(void* stream, int B, int T, int H,
+                                    const float* r, const float* w, const float* k, const float* v,
+                                    const float* a, const float* b, const float* dy, const float* dsT,
+                                    const float* s, const float* sa, float* ds0,
+                                    float* dr, float* dw, float* dk, float* dv, float* da, float* db);
+int rwkv7_state_forward_f32(void* stream, int B, int T, int H,
+                            const float* s0, const float* r, const float* w, const float* k,
+                            const float* v, const float* a, const float* b, float* y, float* s, float* sa);
+int rwkv7_state_backward_f32(void* stream, int B, int T, int H,
+                             const float* r, const float* w, const float* k, const float* v,
+                             const float* a, const float* b, const float* dy,
+                             const float* s, const float* sa, float* ds0,
+                             float* dr, float* dw, float* dk, float* dv, float* da, float* db);
+int rwkv7_forward_f32(void* stream, int B, int T, int H,
+                      const float* r, const float* w, const float* k, const float* v,
+                      const float* a, const float* b, float* y, float* s, float* sa);
+int rwkv7_backward_f32(void* stream, int B, int T, int H,
+                       const float* r, const float* w, const float* k, const float* v,
+                       const float* a, const float* b, const float* dy,
+                       const float* s, const float* sa,
+                       float* dr, float* dw, float* dk, float* dv, float* da, float* db);
 
 #ifdef __cplusplus
 }

@@ -104,6 +104,12 @@ SIGNATURES = {
     "rwkv7_state_backward": (_I, [_P, _I, _I, _I] + [_P] * 16),
     "rwkv7_forward": (_I, [_P, _I, _I, _I] + [_P] * 9),
     "rwkv7_backward": (_I, [_P, _I, _I, _I] + [_P] * 15),
+    "rwkv7_statepassing_forward_f32": (_I, [_P, _I, _I, _I] + [_P] * 11),
+    "rwkv7_statepassing_backward_f32": (_I, [_P, _I, _I, _I] + [_P] * 17),
+    "rwkv7_state_forward_f32": (_I, [_P, _I, _I, _I] + [_P] * 10),
+    "rwkv7_state_backward_f32": (_I, [_P, _I, _I, _I] + [_P] * 16),
+    "rwkv7_forward_f32": (_I, [_P, _I, _I, _I] + [_P] * 9),
+    "rwkv7_backward_f32": (_I, [_P, _I, _I, _I] + [_P] * 15),
 }
 
 

@@ -28,6 +28,8 @@ constexpr int NT = NW * 64;
 constexpr int JW = 16;
 constexpr float W_SCALE = -0.6065306597f;   // -exp(-0.5)
 
+// Element pointers are typed for the bf16 mode; the fp32 mode (the reference's -D_FP32_ build) stores float pointers in
+// the same fields and its kernels (F32 = true) read them back as such through ldg4 / stg4.
 struct Args7 {
     int T, H;
     const uint16_t *r, *w, *k, *v, *a, *b, *dy;
@@ -47,7 +49,24 @@ DEVINL uint2 pack4(const float (&f)[4]) {
     return q;
 }
 DEVINL void st4(float* dst, const float (&f)[4]) { *reinterpret_cast<float4*>(dst) = make_float4(f[0], f[1], f[2], f[3]); }
-DEVINL uint2 ldg4(const uint16_t* p) { return *reinterpret_cast<const uint2*>(p); }
+// four consecutive elements as they come from memory
+template <bool F32> struct Raw4;
+template <> struct Raw4<false> { uint2 q; };
+template <> struct Raw4<true> { float4 q; };
+template <bool F32> DEVINL Raw4<F32> ldg4(const uint16_t* p, size_t o) {
+    Raw4<F32> x;
+    if constexpr (F32) x.q = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + o);
+    else x.q = *reinterpret_cast<const uint2*>(p + o);
+    return x;
+}
+template <bool F32> DEVINL void widen4(const Raw4<F32>& x, float (&f)[4]) {
+    if constexpr (F32) { f[0] = x.q.x; f[1] = x.q.y; f[2] = x.q.z; f[3] = x.q.w; }
+    else unpack4(x.q, f);
+}
+template <bool F32> DEVINL void stg4(uint16_t* p, size_t o, const float (&f)[4]) {
+    if constexpr (F32) *reinterpret_cast<float4*>(reinterpret_cast<float*>(p) + o) = make_float4(f[0], f[1], f[2], f[3]);
+    else *reinterpret_cast<uint2*>(p + o) = pack4(f);
+}
 DEVINL void ld16(float (&f)[16], const float* src) {          // 16 consecutive floats, 16-byte aligned (LDS)
 #pragma unroll
     for (int e = 0; e < 16; e += 4) {
@@ -62,6 +81,7 @@ struct SmemF {
     float y[CL][N], sa[CL][N];
 };
 
+template <bool F32>
 __global__ __launch_bounds__(NT) void rwkv7_fwd(const Args7 p) {
     __shared__ SmemF S;
     const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6, lo = lane & 15, hi = lane >> 4;
@@ -84,11 +104,11 @@ __global__ __launch_bounds__(NT) void rwkv7_fwd(const Args7 p) {
     }
 
     const int nchunks = T / CL;
-    uint2 gr, gw, gk, gv, ga, gb;
+    Raw4<F32> gr, gw, gk, gv, ga, gb;
     auto prefetch = [&](int c) {
         const size_t o = off(c * CL + st);
-        gr = ldg4(p.r + o); gw = ldg4(p.w + o); gk = ldg4(p.k + o);
-        gv = ldg4(p.v + o); ga = ldg4(p.a + o); gb = ldg4(p.b + o);
+        gr = ldg4<F32>(p.r, o); gw = ldg4<F32>(p.w, o); gk = ldg4<F32>(p.k, o);
+        gv = ldg4<F32>(p.v, o); ga = ldg4<F32>(p.a, o); gb = ldg4<F32>(p.b, o);
     };
     prefetch(0);
 
@@ -96,12 +116,12 @@ __global__ __launch_bounds__(NT) void rwkv7_fwd(const Args7 p) {
         __syncthreads();
         {
             float f[4];
-            unpack4(gr, f); st4(&S.r[st][sj], f);
-            unpack4(gk, f); st4(&S.k[st][sj], f);
-            unpack4(gv, f); st4(&S.v[st][sj], f);
-            unpack4(ga, f); st4(&S.a[st][sj], f);
-            unpack4(gb, f); st4(&S.b[st][sj], f);
-            unpack4(gw, f);
+            widen4<F32>(gr, f); st4(&S.r[st][sj], f);
+            widen4<F32>(gk, f); st4(&S.k[st][sj], f);
+            widen4<F32>(gv, f); st4(&S.v[st][sj], f);
+            widen4<F32>(ga, f); st4(&S.a[st][sj], f);
+            widen4<F32>(gb, f); st4(&S.b[st][sj], f);
+            widen4<F32>(gw, f);
 #pragma unroll
             for (int e = 0; e < 4; ++e) f[e] = __expf(W_SCALE / (1.0f + __expf(-f[e])));
             st4(&S.w[st][sj], f);
@@ -141,7 +161,7 @@ __global__ __launch_bounds__(NT) void rwkv7_fwd(const Args7 p) {
         {
             const size_t o = off(c * CL + st);
             float f[4] = {S.y[st][sj], S.y[st][sj + 1], S.y[st][sj + 2], S.y[st][sj + 3]};
-            *reinterpret_cast<uint2*>(p.y + o) = pack4(f);
+            stg4<F32>(p.y, o, f);
             *reinterpret_cast<float4*>(p.sa + o) = *reinterpret_cast<const float4*>(&S.sa[st][sj]);
         }
     }
@@ -161,6 +181,7 @@ struct SmemB {
     float dSb[2][N];
 };
 
+template <bool F32>
 __global__ __launch_bounds__(NT) void rwkv7_bwd(const Args7 p) {
     __shared__ SmemB S;
     const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6, lo = lane & 15, hi = lane >> 4;
@@ -189,12 +210,12 @@ __global__ __launch_bounds__(NT) void rwkv7_bwd(const Args7 p) {
     }
 
     const int nchunks = T / CL;
-    uint2 gr, gw, gk, gv, ga, gb, gdy;
+    Raw4<F32> gr, gw, gk, gv, ga, gb, gdy;
     float4 gsa;
     auto prefetch = [&](int c) {
         const size_t o = off(c * CL + st);
-        gr = ldg4(p.r + o); gw = ldg4(p.w + o); gk = ldg4(p.k + o); gv = ldg4(p.v + o);
-        ga = ldg4(p.a + o); gb = ldg4(p.b + o); gdy = ldg4(p.dy + o);
+        gr = ldg4<F32>(p.r, o); gw = ldg4<F32>(p.w, o); gk = ldg4<F32>(p.k, o); gv = ldg4<F32>(p.v, o);
+        ga = ldg4<F32>(p.a, o); gb = ldg4<F32>(p.b, o); gdy = ldg4<F32>(p.dy, o);
         gsa = *reinterpret_cast<const float4*>(p.sa + o);
     };
     prefetch(nchunks - 1);
@@ -203,14 +224,14 @@ __global__ __launch_bounds__(NT) void rwkv7_bwd(const Args7 p) {
         __syncthreads();
         {
             float f[4], g[4];
-            unpack4(gr, f); st4(&S.r[st][sj], f);
-            unpack4(gk, f); st4(&S.k[st][sj], f);
-            unpack4(gv, f); st4(&S.v[st][sj], f);
-            unpack4(ga, f); st4(&S.a[st][sj], f);
-            unpack4(gb, f); st4(&S.b[st][sj], f);
-            unpack4(gdy, f); st4(&S.dy[st][sj], f);
+            widen4<F32>(gr, f); st4(&S.r[st][sj], f);
+            widen4<F32>(gk, f); st4(&S.k[st][sj], f);
+            widen4<F32>(gv, f); st4(&S.v[st][sj], f);
+            widen4<F32>(ga, f); st4(&S.a[st][sj], f);
+            widen4<F32>(gb, f); st4(&S.b[st][sj], f);
+            widen4<F32>(gdy, f); st4(&S.dy[st][sj], f);
             *reinterpret_cast<float4*>(&S.sa[st][sj]) = gsa;
-            unpack4(gw, f);
+            widen4<F32>(gw, f);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const float sig = 1.0f / (1.0f + __expf(-f[e]));
@@ -294,7 +315,7 @@ __global__ __launch_bounds__(NT) void rwkv7_bwd(const Args7 p) {
             const size_t o = off(c * CL + st);
             auto put = [&](uint16_t* dst, const float (*src)[N]) {
                 float f[4] = {src[st][sj], src[st][sj + 1], src[st][sj + 2], src[st][sj + 3]};
-                *reinterpret_cast<uint2*>(dst + o) = pack4(f);
+                stg4<F32>(dst, o, f);
             };
             put(p.dr, S.dr); put(p.dw, S.dw); put(p.dk, S.dk);
             put(p.dv, S.dv); put(p.da, S.da); put(p.db, S.db);
@@ -315,25 +336,31 @@ int check7(int B, int T, int H) {
     return RWKV_OK;
 }
 
-int launch7_fwd(void* stream, int B, int T, int H, const float* s0, const rwkv_bf16* r, const rwkv_bf16* w,
-                const rwkv_bf16* k, const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b, rwkv_bf16* y,
+const uint16_t* el(const void* p) { return static_cast<const uint16_t*>(p); }
+uint16_t* el(void* p) { return static_cast<uint16_t*>(p); }
+
+// r..b, y (and dy, dr..db below) are bf16 or, with f32, float
+int launch7_fwd(void* stream, bool f32, int B, int T, int H, const float* s0, const void* r, const void* w,
+                const void* k, const void* v, const void* a, const void* b, void* y,
                 float* sT, float* s, float* sa) {
     Args7 p{};
-    p.T = T; p.H = H; p.s0 = s0; p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b;
-    p.y = y; p.sT = sT; p.s = s; p.sa = sa;
-    hipLaunchKernelGGL(rwkv7_fwd, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
+    p.T = T; p.H = H; p.s0 = s0; p.r = el(r); p.w = el(w); p.k = el(k); p.v = el(v); p.a = el(a); p.b = el(b);
+    p.y = el(y); p.sT = sT; p.s = s; p.sa = sa;
+    if (f32) hipLaunchKernelGGL(rwkv7_fwd<true>, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
+    else hipLaunchKernelGGL(rwkv7_fwd<false>, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
     return launch_status();
 }
 
-int launch7_bwd(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
-                const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b, const rwkv_bf16* dy, const float* dsT,
-                const float* s, const float* sa, float* ds0, rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk,
-                rwkv_bf16* dv, rwkv_bf16* da, rwkv_bf16* db) {
+int launch7_bwd(void* stream, bool f32, int B, int T, int H, const void* r, const void* w, const void* k,
+                const void* v, const void* a, const void* b, const void* dy, const float* dsT,
+                const float* s, const float* sa, float* ds0, void* dr, void* dw, void* dk,
+                void* dv, void* da, void* db) {
     Args7 p{};
-    p.T = T; p.H = H; p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b; p.dy = dy; p.dsT = dsT;
-    p.s = const_cast<float*>(s); p.sa = const_cast<float*>(sa);
-    p.ds0 = ds0; p.dr = dr; p.dw = dw; p.dk = dk; p.dv = dv; p.da = da; p.db = db;
-    hipLaunchKernelGGL(rwkv7_bwd, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
+    p.T = T; p.H = H; p.r = el(r); p.w = el(w); p.k = el(k); p.v = el(v); p.a = el(a); p.b = el(b); p.dy = el(dy);
+    p.dsT = dsT; p.s = const_cast<float*>(s); p.sa = const_cast<float*>(sa);
+    p.ds0 = ds0; p.dr = el(dr); p.dw = el(dw); p.dk = el(dk); p.dv = el(dv); p.da = el(da); p.db = el(db);
+    if (f32) hipLaunchKernelGGL(rwkv7_bwd<true>, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
+    else hipLaunchKernelGGL(rwkv7_bwd<false>, dim3(H, B), dim3(NT), 0, static_cast<hipStream_t>(stream), p);
     return launch_status();
 }
 
@@ -349,7 +376,7 @@ int rwkv7_statepassing_forward(void* stream, int B, int T, int H, const float* s
                                const rwkv_bf16* b, rwkv_bf16* y, float* sT, float* s, float* sa) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({s0, r, w, k, v, a, b, y, sT, s, sa})) return e;
-    return launch7_fwd(stream, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa);
+    return launch7_fwd(stream, false, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa);
 }
 
 int rwkv7_statepassing_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w,
@@ -359,7 +386,7 @@ int rwkv7_statepassing_backward(void* stream, int B, int T, int H, const rwkv_bf
                                 rwkv_bf16* da, rwkv_bf16* db) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db})) return e;
-    return launch7_bwd(stream, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db);
+    return launch7_bwd(stream, false, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db);
 }
 
 // Initial state with its gradient, no final state: the same kernels without the sT store and with dsT = 0.
@@ -368,7 +395,7 @@ int rwkv7_state_forward(void* stream, int B, int T, int H, const float* s0, cons
                         rwkv_bf16* y, float* s, float* sa) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({s0, r, w, k, v, a, b, y, s, sa})) return e;
-    return launch7_fwd(stream, B, T, H, s0, r, w, k, v, a, b, y, nullptr, s, sa);
+    return launch7_fwd(stream, false, B, T, H, s0, r, w, k, v, a, b, y, nullptr, s, sa);
 }
 
 int rwkv7_state_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w,
@@ -377,7 +404,7 @@ int rwkv7_state_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, 
                          rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv, rwkv_bf16* da, rwkv_bf16* db) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({r, w, k, v, a, b, dy, s, sa, ds0, dr, dw, dk, dv, da, db})) return e;
-    return launch7_bwd(stream, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, ds0, dr, dw, dk, dv, da, db);
+    return launch7_bwd(stream, false, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, ds0, dr, dw, dk, dv, da, db);
 }
 
 // No state on either side: zero initial state, no final state, no state gradients.
@@ -385,7 +412,7 @@ int rwkv7_forward(void* stream, int B, int T, int H, const rwkv_bf16* r, const r
                   const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b, rwkv_bf16* y, float* s, float* sa) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({r, w, k, v, a, b, y, s, sa})) return e;
-    return launch7_fwd(stream, B, T, H, nullptr, r, w, k, v, a, b, y, nullptr, s, sa);
+    return launch7_fwd(stream, false, B, T, H, nullptr, r, w, k, v, a, b, y, nullptr, s, sa);
 }
 
 int rwkv7_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
@@ -394,7 +421,58 @@ int rwkv7_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const 
                    rwkv_bf16* db) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({r, w, k, v, a, b, dy, s, sa, dr, dw, dk, dv, da, db})) return e;
-    return launch7_bwd(stream, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, nullptr, dr, dw, dk, dv, da, db);
+    return launch7_bwd(stream, false, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, nullptr, dr, dw, dk, dv, da, db);
+}
+
+// ---- fp32 I/O: what the reference builds from the same sources with -D_FP32_ (rwkv7_cuda_benchmark.py:102-126 and the
+// same lines of its _state and _state_passing siblings).  Same kernels, same fp32 arithmetic; only loads and stores differ.
+int rwkv7_statepassing_forward_f32(void* stream, int B, int T, int H, const float* s0, const float* r, const float* w,
+                                   const float* k, const float* v, const float* a, const float* b, float* y,
+                                   float* sT, float* s, float* sa) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({s0, r, w, k, v, a, b, y, sT, s, sa})) return e;
+    return launch7_fwd(stream, true, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa);
+}
+
+int rwkv7_statepassing_backward_f32(void* stream, int B, int T, int H, const float* r, const float* w, const float* k,
+                                    const float* v, const float* a, const float* b, const float* dy, const float* dsT,
+                                    const float* s, const float* sa, float* ds0, float* dr, float* dw, float* dk,
+                                    float* dv, float* da, float* db) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db})) return e;
+    return launch7_bwd(stream, true, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db);
+}
+
+int rwkv7_state_forward_f32(void* stream, int B, int T, int H, const float* s0, const float* r, const float* w,
+                            const float* k, const float* v, const float* a, const float* b, float* y, float* s,
+                            float* sa) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({s0, r, w, k, v, a, b, y, s, sa})) return e;
+    return launch7_fwd(stream, true, B, T, H, s0, r, w, k, v, a, b, y, nullptr, s, sa);
+}
+
+int rwkv7_state_backward_f32(void* stream, int B, int T, int H, const float* r, const float* w, const float* k,
+                             const float* v, const float* a, const float* b, const float* dy, const float* s,
+                             const float* sa, float* ds0, float* dr, float* dw, float* dk, float* dv, float* da,
+                             float* db) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({r, w, k, v, a, b, dy, s, sa, ds0, dr, dw, dk, dv, da, db})) return e;
+    return launch7_bwd(stream, true, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, ds0, dr, dw, dk, dv, da, db);
+}
+
+int rwkv7_forward_f32(void* stream, int B, int T, int H, const float* r, const float* w, const float* k,
+                      const float* v, const float* a, const float* b, float* y, float* s, float* sa) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({r, w, k, v, a, b, y, s, sa})) return e;
+    return launch7_fwd(stream, true, B, T, H, nullptr, r, w, k, v, a, b, y, nullptr, s, sa);
+}
+
+int rwkv7_backward_f32(void* stream, int B, int T, int H, const float* r, const float* w, const float* k,
+                       const float* v, const float* a, const float* b, const float* dy, const float* s,
+                       const float* sa, float* dr, float* dw, float* dk, float* dv, float* da, float* db) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({r, w, k, v, a, b, dy, s, sa, dr, dw, dk, dv, da, db})) return e;
+    return launch7_bwd(stream, true, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, nullptr, dr, dw, dk, dv, da, db);
 }
 
 }  // extern "C"

@@ -20,7 +20,7 @@ def _declared_symbols():
 
 def test_header_and_bindings_agree(lib):
     names = _declared_symbols()
-    assert len(names) == 32
+    assert len(names) == 38
     assert sorted(_lib.SIGNATURES) == names
     for n in names:
         assert hasattr(lib, n), f"{n} declared in rwkv_hip.h but not exported"
@@ -44,6 +44,9 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.rwkv7_state_forward(None, 1, 24, 1, *([p] * 10)) == -1
     assert lib.rwkv7_forward(None, 1, 16, 1, *([p] * 8), None) == -2
     assert lib.rwkv7_backward(None, 0, 16, 1, *([p] * 15)) == -1
+    assert lib.rwkv7_statepassing_forward_f32(None, 1, 24, 1, *([p] * 11)) == -1
+    assert lib.rwkv7_state_backward_f32(None, 1, 16, 1, *([p] * 15), p + 8) == -3
+    assert lib.rwkv7_backward_f32(None, 1, 16, 1, *([p] * 14), None) == -2
     assert lib.rwkv_timex_forward(None, p, p, p, 0.0, 1, 1, 6) == -1                 # T % 4
     assert lib.rwkv_timex_backward_sum(None, p, p, p, p, p, 2, 1, 48) == -1           # T % 32
     assert lib.rwkv_timex_backward_sum(None, p, p, p, p, p, 2, 1, 2048) == -1         # T > 1024

@@ -118,3 +118,63 @@ def test_rwkv7_long_sequence_is_no_worse_than_the_reference_kernel(lib):
     got = _run(args)
     for name, a, e, g in zip(NAMES, ref, emu, got):
         assert_no_worse("rwkv7 T2048 " + name, a, e, g)
+
+
+def _fp32_inputs(B, T, H, seed):
+    """The bf16 test inputs plus an fp32 perturbation below bf16 resolution, so that the fp32 mode is
+    seen to read all 32 bits of every element."""
+    g = torch.Generator().manual_seed(seed + 1000)
+    args = synth.rwkv7_inputs(B, T, H, 64, seed=seed)
+    jig = lambda x: x.float() * (1 + 1e-3 * torch.rand(x.shape, generator=g))
+    s0, r, w, k, v, a, b, dy, dsT = args
+    return (s0, jig(r), jig(w), jig(k), jig(v), jig(a), jig(b), jig(dy), dsT)
+
+
+def assert_fp32_mode(name, ref64, emu, got):
+    """fp32 mode: the error against fp64 may not exceed twice that of the reference kernel's arithmetic
+    (fp32, in-chunk inversion, checkpoints every 16 steps) emulated on the CPU.  The two differ only
+    in summation order, so their errors are independent samples of the same size; 2x covers that."""
+    e_hip = err_ratio(ref64, got.detach().double().cpu())
+    e_emu = err_ratio(ref64, emu.double())
+    print(f"  {name}: hip {e_hip:.3e}  reference-kernel arithmetic {e_emu:.3e}", flush=True)
+    assert e_hip <= 2.0 * e_emu + 1e-6, f"{name}: {e_hip:.3e} vs {e_emu:.3e}"
+    assert e_hip < 1e-3, name                       # and far below what a bf16 rounding anywhere would leave
+
+
+@pytest.mark.parametrize("B,T,H", [(2, 32, 2), (1, 256, 1)])
+def test_rwkv7_fp32_mode(lib, B, T, H):
+    """The reference's -D_FP32_ build (rwkv7_cuda_benchmark_state_passing.py:105-131): every tensor fp32."""
+    print(f"\nrwkv7 fp32 mode B={B} T={T} H={H}", flush=True)
+    args = _fp32_inputs(B, T, H, seed=35)
+    ref = O.grads(*args)
+    emu = O.backward_hand(*args, dtype=torch.float32, invert=True)
+    got = _run(args)
+    assert got[0].dtype == torch.float32 and got[3].dtype == torch.float32
+    for name, a, e, g in zip(NAMES, ref, emu, got):
+        assert_fp32_mode(name, a, e, g)
+
+
+def test_rwkv7_fp32_mode_siblings(lib):
+    B, T, H, N = 2, 32, 2, 64
+    s0, r, w, k, v, a, b, dy, dsT = _fp32_inputs(B, T, H, seed=36)
+    flat = lambda x: x.contiguous().view(B, T, H * N)
+    args = (s0, r, w, k, v, a, b, dy, torch.zeros_like(dsT))
+    ref, emu = O.grads(*args), O.backward_hand(*args, dtype=torch.float32, invert=True)
+    t = [x.to(DEV).requires_grad_(True) for x in (s0, r, w, k, v, a, b)]
+    y = R.RWKV7_STATE_CLAMPW_CUDA(t[0], *(flat(x) for x in t[1:]))
+    y.backward(flat(dy.to(DEV)))
+    torch.cuda.synchronize()
+    got = [y.detach().view(B, T, H, N), None] + [x.grad for x in t]
+    for name, a_, e, g in zip(NAMES, ref, emu, got):
+        if g is not None:
+            assert_fp32_mode("fp32 state op " + name, a_, e, g)
+    args = (torch.zeros_like(s0), r, w, k, v, a, b, dy, torch.zeros_like(dsT))
+    ref, emu = O.grads(*args), O.backward_hand(*args, dtype=torch.float32, invert=True)
+    t = [x.to(DEV).requires_grad_(True) for x in (r, w, k, v, a, b)]
+    y = R.RWKV7_CLAMPW_CUDA(*(flat(x) for x in t))
+    y.backward(flat(dy.to(DEV)))
+    torch.cuda.synchronize()
+    got = [y.detach().view(B, T, H, N), None, None] + [x.grad for x in t]
+    for name, a_, e, g in zip(NAMES, ref, emu, got):
+        if g is not None:
+            assert_fp32_mode("fp32 stateless op " + name, a_, e, g)
