@@ -177,7 +177,13 @@ DEVINL void commit(Smem<PASS>& S, const Staged<F32>& p, const Args& a, int c0, i
 #pragma unroll
         for (int e = 0; e < 8; ++e) dec[e] = ok ? __expf(fw[e]) : 1.0f;  // rows past T leave the state alone
         st8(&S.w[st][sj], dec);
-        if constexpr (PASS == P_GK) st8(&S.f[st][sj], fw);
+        if constexpr (PASS == P_GK) {
+            // the factor of the decay gradient; zero once the decay is below e^-30, where the true gradient has vanished and
+            // the factor would only amplify the rounding noise of G (the original kernel gives an exact zero there too)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) fw[e] = fw[e] < -30.0f ? 0.f : fw[e];
+            st8(&S.f[st][sj], fw);
+        }
     }
     if constexpr (PASS == P_GK && !F32) {
         *reinterpret_cast<float4*>(&S.rdr[st][sj]) = p.rdr0;
@@ -486,7 +492,10 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     }
     if constexpr (PASS == P_GK) {
         if constexpr (WMODE == W_HEAD && SCAN_GW) {
-            if (tid < N) store1<F32>(a.gw, static_cast<size_t>(b) * a.C + h * N + tid, a.ew_head[h * N + tid] * gw_acc);
+            if (tid < N) {
+                const float f = a.ew_head[h * N + tid];
+                store1<F32>(a.gw, static_cast<size_t>(b) * a.C + h * N + tid, (f < -30.0f ? 0.f : f) * gw_acc);
+            }
         }
         if (a.gs != nullptr) {
 #pragma unroll

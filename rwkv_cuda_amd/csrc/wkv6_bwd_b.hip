@@ -231,7 +231,7 @@ DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base
             *reinterpret_cast<float2*>(&O.rdr[pt0 + e][2 * jp]) = x.d[e];
             O.V[pt0 + e][jp] = x.v[e];
             O.GY[pt0 + e][jp] = x.g[e];
-            *reinterpret_cast<float2*>(&O.lam[pt0 + e][2 * jp]) = make_float2(x.lam[e][0] * LN2, x.lam[e][1] * LN2);
+            *reinterpret_cast<float2*>(&O.lam[pt0 + e][2 * jp]) = make_float2(gw_factor(x.lam[e][0] * LN2), gw_factor(x.lam[e][1] * LN2));
         }
         if (wid == 3 && th == 0) {
             float cm[2] = {0.f, 0.f}, ch[2] = {0.f, 0.f};
@@ -528,7 +528,7 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const float s = row_sum_to_last(gw_acc[v]) + pxv[v];
-            if (l16 == 15) a.gw[bh * N + j4 + v] = f2bf(ev[v] * s);
+            if (l16 == 15) a.gw[bh * N + j4 + v] = f2bf(gw_factor(ev[v]) * s);
         }
     }
     if (a.gs != nullptr) {

@@ -138,6 +138,14 @@ constexpr int FS = 72;            // row stride (dwords) of an fp32 [token][chan
 constexpr int AS = 24;            // row stride (dwords) of a tile plane [row][32 permuted positions]
 constexpr float LN2 = 0.69314718055994530942f;
 
+// The factor that turns G into the raw-decay gradient: gw = lam G with lam = -exp(w_raw) = log(decay).  G comes from the
+// P recurrence and carries rounding noise of a few 1e-6 |P| whatever the decay, while its true value is decay * (...).  Once
+// the decay is below e^-30 the true gw is under 3e-12 of the other gradients, but lam would amplify the noise without bound
+// (w_raw = 15 -> lam = -3e6).  The factor is therefore zero from there on, which is also what the original kernel
+// produces, exactly, once its fp32 decay has underflowed.
+constexpr float LAM_CUT = -30.0f;
+DEVINL float gw_factor(float lam) { return lam < LAM_CUT ? 0.f : lam; }
+
 template <int CTRL, int ROW_MASK> DEVINL float dpp_add(float x) {
     return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xf, true));
 }

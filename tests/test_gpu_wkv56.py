@@ -256,3 +256,58 @@ def test_wkv5_both_algorithms_and_strong_decays(lib, algo):
         for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y] + [x.grad for x in t]):
             assert torch.isfinite(g).all(), name
             assert_no_worse(name, a, e, g)
+
+
+def _low_rank_decay(B, T, C, seed):
+    """w = w0 + (x @ ww1) @ ww2 as the reference's wkv6 checks build it (wkv6_state/run.py:183-186,214): at C = 128
+    it spans about -18 .. +15, so a seventh of the decays exp(-exp(w)) are exactly zero in fp32 and others are 1."""
+    g = torch.Generator().manual_seed(seed)
+    U = lambda lo, hi, *s: (torch.rand(*s, generator=g) * (hi - lo) + lo).to(BF).float()
+    return (U(-3, 1, 1, 1, C) + (U(-1, 1, B, T, C) @ U(-1, 1, C, 3)) @ U(-1, 1, 3, C)).to(BF)
+
+
+@pytest.mark.parametrize("algo", [0, 1])
+def test_decay_gradient_where_the_decay_has_vanished(lib, algo):
+    """gw = -exp(w_raw) G, and G comes from a recurrence whose rounding noise does not shrink with the decay: at
+    w_raw = 15 the factor is 3e6 and would turn 1e-6 of noise into O(1) gradients where the true value (and the
+    reference kernel's) is an exact zero."""
+    B, T, H = 2, 64, 2
+    C = H * 64
+    r, k, v, _, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=51, state=True)
+    w = _low_rank_decay(B, T, C, seed=52)
+    assert float(w.max()) > 8 and float(w.min()) < -8
+    gone = w.float() > 4.5                                   # exp(-exp(4.5)) < 1e-39
+    lib.rwkv_wkv6_set_algorithm(algo)
+    try:
+        for state in (None, s0):
+            print(f"\nlow-rank decays algo={algo} state={state is not None}", flush=True)
+            ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=state)
+            emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=state)
+            t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u)]
+            if state is None:
+                y = wkv6.RUN_CUDA(B, T, C, H, *t)
+            else:
+                t.append(state.to(DEV).requires_grad_(True))
+                y = wkv6_state.RUN_CUDA(B, T, C, H, *t)
+            y.backward(gy.to(DEV))
+            torch.cuda.synchronize()
+            for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, emu, [y] + [x.grad for x in t]):
+                assert_no_worse(name, a, e, g)
+            assert float(t[3].grad.float().cpu()[gone].abs().max()) == 0.0
+        # wkv5: per-channel decays up to w_raw = 6 (the state of those channels is wiped every step)
+        r, k, v, w5, u, gy = synth.wkv5_inputs(B, T, C, H, seed=53)
+        w5 = w5.float()
+        w5[0, 5:12] = 6.0
+        w5[1, 30] = 4.0
+        w5 = w5.to(BF)
+        ref = O.wkv5_grads(B, T, C, H, r, k, v, w5, u, gy)
+        emu = O.emulate_wkv5_bf16(B, T, C, H, r, k, v, w5, u, gy)
+        t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w5, u)]
+        y = wkv5_bf16.RUN_CUDA(B, T, C, H, *t)
+        y.backward(gy.to(DEV))
+        torch.cuda.synchronize()
+        for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y] + [x.grad for x in t]):
+            assert_no_worse("wkv5 " + name, a, e, g)
+        assert float(t[3].grad.float().cpu()[0, 5:12].abs().max()) == 0.0
+    finally:
+        lib.rwkv_wkv6_set_algorithm(0)
