@@ -57,3 +57,42 @@ def test_wkv6_state_chunked_equals_sweeps(lib, seed):
             diff = float((c.float() - s.float()).abs().max()) / peak
             print(f"  {name}: chunked vs sweeps, max difference / peak {diff:.3e}", flush=True)
             assert diff < 2.0 ** -6, (name, diff)
+
+
+REGIMES = ["wide", "alternating", "tiny", "zero_k", "big_u", "large_inputs"]
+
+
+@pytest.mark.parametrize("regime", REGIMES)
+@pytest.mark.parametrize("algo", [0, 1])
+def test_wkv6_state_input_regimes(lib, algo, regime):
+    """Input regimes away from the benchmark's: decays spread over exp(-exp(-18..12)) (every chunk on the exact path,
+    many decays exactly 0 or 1), decays alternating between almost 0 and almost 1 token by token, no decay at all,
+    k = 0 (the state never changes), a bonus of order 10, inputs of order 8."""
+    rng = random.Random(REGIMES.index(regime))
+    B, H, T = rng.randint(1, 2), rng.randint(1, 2), rng.choice([5, 33, 64, 100])
+    C = H * 64
+    print(f"\nregime {regime} algo={algo} B={B} T={T} H={H}", flush=True)
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=300 + REGIMES.index(regime), state=True)
+    g = torch.Generator().manual_seed(7)
+    if regime == "wide":
+        w = (torch.rand(B, T, C, generator=g) * 30 - 18).to(BF)
+    elif regime == "alternating":
+        w = torch.full((B, T, C), -6.0)
+        w[:, ::2] = 3.5
+        w[:, :, ::3] = -1.0
+        w = w.to(BF)
+    elif regime == "tiny":
+        w = torch.full((B, T, C), -25.0).to(BF)
+    elif regime == "zero_k":
+        k = torch.zeros_like(k)
+    elif regime == "big_u":
+        u = (u.float() * 30).to(BF)
+    elif regime == "large_inputs":
+        r, k, v, gy, s0 = ((x.float() * 16).to(BF) for x in (r, k, v, gy, s0))
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    d = [x.to(DEV) for x in (r, k, v, w, u, s0, gy)]
+    got = _run(lib, algo, B, T, C, H, d)
+    for name, a, e, q in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, emu, got):
+        assert torch.isfinite(q.float()).all(), name
+        assert_no_worse(name, a, e, q)
