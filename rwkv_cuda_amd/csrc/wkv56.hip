@@ -19,6 +19,10 @@
 // The decay gradient needs no third recurrence: with P_t[j] = sum_i dS_t[i,j] S_t[i,j],
 //   G_t = w_t * sum_i dS_{t+1} S_t = P_{t+1} - k_t dk'_t,   P_t = G_t + r_t dr'_t,   P_T = 0,
 // where dr', dk' are the bonus-free parts of gr, gk; gw_raw = -exp(w_raw) * G.
+//
+// The same kernels with fp32 loads and stores (F32) are the fp32 wkv5 op (wkv5/cuda/wkv5_op.cpp); there GR carries
+// Q = dS/dw and makes gw itself, without the P recurrence and its workspace.  With TWO they are wkv5a
+// (wkv5a_cuda_v1a2.cu): decay w1[j] w2[i] and bonus u1[j] + u2[i] per state element.
 #include "common.h"
 
 namespace rwkv {
@@ -426,22 +430,22 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
             }
             if (ok) store8<F32>(a.gk, off, out);
             if constexpr (SCAN_GW) {
-            if (stager) st8(&S.k[st][sj], kdk);              // k is no longer needed: keep k*dk' there
-            __syncthreads();
-            if (tid < N) {                                   // per-channel scan over the chunk, t descending
-                for (int t = TC - 1; t >= 0; --t) {
-                    float G = P - S.k[t][tid];
-                    if (!stateful && (c0 + t) == 0) G = 0.f; // S_0 = 0: exact zero, as the reference leaves it
-                    P = G + S.rdr[t][tid];
-                    if constexpr (WMODE == W_HEAD) gw_acc += G;
-                    else S.part[0][t][tid] = S.f[t][tid] * G;
-                }
-            }
-            if constexpr (WMODE != W_HEAD) {
+                if (stager) st8(&S.k[st][sj], kdk);              // k is no longer needed: keep k*dk' there
                 __syncthreads();
-                ld8f(&S.part[0][es][sj], out);
-                if (ok) store8<F32>(a.gw, off, out);
-            }
+                if (tid < N) {                                   // per-channel scan over the chunk, t descending
+                    for (int t = TC - 1; t >= 0; --t) {
+                        float G = P - S.k[t][tid];
+                        if (!stateful && (c0 + t) == 0) G = 0.f; // S_0 = 0: exact zero, as the reference leaves it
+                        P = G + S.rdr[t][tid];
+                        if constexpr (WMODE == W_HEAD) gw_acc += G;
+                        else S.part[0][t][tid] = S.f[t][tid] * G;
+                    }
+                }
+                if constexpr (WMODE != W_HEAD) {
+                    __syncthreads();
+                    ld8f(&S.part[0][es][sj], out);
+                    if (ok) store8<F32>(a.gw, off, out);
+                }
             }
         }
     }
