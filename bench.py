@@ -282,13 +282,17 @@ def make_wkv5a(dev):
     return step, tok, kernels, cfg, cpu_baseline, 44 * C * tok
 
 
-def make_rwkv7(dev):
+def make_rwkv7(dev, fp32=False):
+    """fp32=True: the reference's -D_FP32_ mode (every bf16 tensor fp32), same kernels with fp32 loads and stores."""
     from rwkv_cuda_amd import synth
     from rwkv_cuda_amd._call import call
     B, T, H, N = 8, 4096, 64, 64
     C = H * N
     TS = T // 4                                                   # four chained T=1024 calls
+    sfx, eb = ("_f32", 4) if fp32 else ("", 2)                    # entry-point suffix, bytes per element
     s0, r, w, k, v, a, b, dy, dsT = (x.to(dev) for x in synth.rwkv7_inputs(B, T, H, N, seed=42))
+    if fp32:
+        r, w, k, v, a, b, dy = (x.float() for x in (r, w, k, v, a, b, dy))
     seg = [[x[:, i * TS:(i + 1) * TS].contiguous() for x in (r, w, k, v, a, b, dy)] for i in range(4)]
     f32 = dict(device=dev, dtype=torch.float32)
     ys = [torch.empty_like(s[0]) for s in seg]
@@ -303,21 +307,21 @@ def make_rwkv7(dev):
         st = s0
         for i in range(4):
             rr, ww, kk, vv, aa, bb, _ = seg[i]
-            call("rwkv7_statepassing_forward", dev, B, TS, H, st, rr, ww, kk, vv, aa, bb, ys[i], sTs[i], ss[i], sas[i])
+            call("rwkv7_statepassing_forward" + sfx, dev, B, TS, H, st, rr, ww, kk, vv, aa, bb, ys[i], sTs[i], ss[i], sas[i])
             st = sTs[i]
 
     def bwd():
         g = dsT
         for i in (3, 2, 1, 0):
             rr, ww, kk, vv, aa, bb, dd = seg[i]
-            call("rwkv7_statepassing_backward", dev, B, TS, H, rr, ww, kk, vv, aa, bb, dd, g, ss[i], sas[i], ds[i], *grads[i])
+            call("rwkv7_statepassing_backward" + sfx, dev, B, TS, H, rr, ww, kk, vv, aa, bb, dd, g, ss[i], sas[i], ds[i], *grads[i])
             g = ds[i]
 
     def step():
         fwd()
         bwd()
 
-    kernels = [("rwkv7 forward x4 (T=1024 each)", fwd, 14 * C * tok), ("rwkv7 backward x4", bwd, 26 * C * tok)]
+    kernels = [("rwkv7 forward x4 (T=1024 each)", fwd, 7 * eb * C * tok), ("rwkv7 backward x4", bwd, 13 * eb * C * tok)]
 
     def cpu_baseline(t_cpu=64):
         from oracle import rwkv7 as O
@@ -327,9 +331,9 @@ def make_rwkv7(dev):
         dt = time.perf_counter() - t0
         return B * t_cpu / dt / 1e6, f"rwkv7 fwd+bwd, fp32 autograd of the einsum step, B{B} H{H} N{N}, T_cpu={t_cpu} ({dt:.1f} s)"
 
-    cfg = {"workload": f"rwkv7 state-passing bf16 fwd+bwd B{B} T{T} (4 x {TS}) C{C} H{H} N{N}", "B": B, "T": T, "C": C,
-           "H": H, "N": N, "algorithmic_bytes_per_token": 40 * C}
-    return step, tok, kernels, cfg, cpu_baseline, 40 * C * tok
+    cfg = {"workload": f"rwkv7 state-passing {'fp32' if fp32 else 'bf16'} fwd+bwd B{B} T{T} (4 x {TS}) C{C} H{H} N{N}", "B": B, "T": T,
+           "C": C, "H": H, "N": N, "algorithmic_bytes_per_token": 20 * eb * C}
+    return step, tok, kernels, cfg, cpu_baseline, 20 * eb * C * tok
 
 
 def make_wkv4(dev):
@@ -411,10 +415,11 @@ WORKLOADS = {
     "wkv5_fp32": make_wkv5_fp32,
     "wkv5a": make_wkv5a,
     "rwkv7": make_rwkv7,
+    "rwkv7_fp32": lambda dev: make_rwkv7(dev, fp32=True),
     "wkv4": make_wkv4,
     "timex": make_timex,
 }
-DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "wkv4": "f32", "timex": "f32"}
+DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "timex": "f32"}
 
 
 def main():
