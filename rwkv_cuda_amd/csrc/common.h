@@ -89,6 +89,32 @@ DEVINL float allreduce_rows(float x) {
 #endif
 }
 
+// The same two swaps applied to distinct values do more work per instruction.  permlane16_swap(a, b) leaves
+// a = [a0, b0, a2, b2] and b = [a1, b1, a3, b3] (by row), permlane32_swap(s, t) leaves s = [s0, s1, t0, t1] and
+// t = [s2, s3, t2, t3].
+
+// Row sums of four values in three swaps: row 0 of the result holds sum(a), row 1 sum(b), row 2 sum(c), row 3 sum(d).
+DEVINL float reduce4_rows(float a, float b, float c, float d) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\ts_nop 1"
+                 : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+    float s = a + b, t = c + d;                   // [a01, b01, a23, b23], [c01, d01, c23, d23]
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(s), "+v"(t));
+    return s + t;
+}
+
+// Row sums of two values, each result in all four rows, in three swaps instead of four.
+DEVINL void allreduce2_rows(float& x, float& y) {
+    float a = x, b = y;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    float s = a + b;                              // [x01, y01, x23, y23]
+    float t = s;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(s), "+v"(t));
+    float u = s + t;                              // [X, Y, X, Y]
+    float w = u;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(u), "+v"(w));
+    x = u; y = w;                                 // [X, X, X, X], [Y, Y, Y, Y]
+}
+
 // ----------------------------------------------------------------------------- host checks
 extern thread_local int g_last_hip_error;
 

@@ -177,7 +177,9 @@ __global__ __launch_bounds__(NT) void rwkv7_fwd(const Args7 p) {
 struct SmemB {
     float r[CL][N], w[CL][N], k[CL][N], v[CL][N], a[CL][N], b[CL][N], dy[CL][N], sa[CL][N];
     float wf[CL][N];                       // d w / d w_raw = W_SCALE * w * sig * (1 - sig)
-    float dr[CL][N], dw[CL][N], dk[CL][N], dv[CL][N], da[CL][N], db[CL][N];
+    float dr[CL][N], dw[CL][N], dk[CL][N], db[CL][N];      // in this order: row h of a wave's four-way reduction goes to array h
+    float dv[CL][N];
+    float da[CL][4][N];                    // one partial per lane row, summed when the chunk is stored: no reduction in the step
     float dSb[2][N];
 };
 
@@ -281,22 +283,18 @@ __global__ __launch_bounds__(NT) void rwkv7_bwd(const Args7 p) {
                 fmac_bc<e>(dvp, kv, dSH[e]);
                 fmac_bc<e>(dSbp, bv, dSH[e]);
             });
-            const float dSb = allreduce_rows(dSbp);
-            const float dv = allreduce_rows(dvp);
+            float dSb = dSbp, dv = dvp;
+            allreduce2_rows(dSb, dv);
             static_for<JW>([&](auto E) {
                 constexpr int e = decltype(E)::value;
                 mul_bc<e>(dSH[e], wv);                    // dS <- dS w_j + dSb_i a_j
                 fmac_bc<e>(dSH[e], av, dSb);
             });
-            const float dr = allreduce_rows(drp), dw = allreduce_rows(dwp);
-            const float dk = allreduce_rows(dkp), db = allreduce_rows(dbp);
+            // dr, dw, dk, db: the four column sums reduced together, lane row h ends up with the h-th of them
+            (&S.dr[0][0])[(hi * CL + t) * N + own] = reduce4_rows(drp, dwp * S.wf[t][own], dkp, dbp);
             if (hi == 0) {
                 S.dSb[par][own] = dSb;
                 S.dv[t][own] = dv;
-                S.dr[t][own] = dr;
-                S.dw[t][own] = dw * S.wf[t][own];
-                S.dk[t][own] = dk;
-                S.db[t][own] = db;
             }
             __syncthreads();
             const float dSbv = S.dSb[par][lane];
@@ -307,8 +305,7 @@ __global__ __launch_bounds__(NT) void rwkv7_bwd(const Args7 p) {
                 dST[e] *= wj;                             // dS <- dS w_j + dSb_i a_j
                 fmac_bc<e>(dST[e], dSbv, aj);
             });
-            const float da = allreduce_rows(dap);
-            if (hi == 0) S.da[t][own] = da;
+            S.da[t][hi][own] = dap;
         }
         __syncthreads();
         {
@@ -318,7 +315,11 @@ __global__ __launch_bounds__(NT) void rwkv7_bwd(const Args7 p) {
                 stg4<F32>(dst, o, f);
             };
             put(p.dr, S.dr); put(p.dw, S.dw); put(p.dk, S.dk);
-            put(p.dv, S.dv); put(p.da, S.da); put(p.db, S.db);
+            put(p.dv, S.dv); put(p.db, S.db);
+            float f[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f[e] = (S.da[st][0][sj + e] + S.da[st][1][sj + e]) + (S.da[st][2][sj + e] + S.da[st][3][sj + e]);
+            stg4<F32>(p.da, o, f);
         }
     }
     if (p.ds0 != nullptr) {
