@@ -358,7 +358,7 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
                         vg = fmaf(gg[mm][v], vv[mm][v], vg);
                         D[mm][v] = fmaf(D[mm][v], wj, vv[mm][v] * kj);
                     }
-                dr = allreduce_rows(dr); vg = allreduce_rows(vg);
+                allreduce2_rows(dr, vg);
                 if (g == 0) S.Yx[ih][t][j_own] = dr;
                 if (q == 0 && lane == 0) S.Vx[ih][t] = vg;
             }

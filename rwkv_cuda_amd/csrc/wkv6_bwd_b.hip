@@ -437,7 +437,7 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                         vg = fmaf(vv[m][v], gg[m][v], vg);
                         D[m][v] = fmaf(D[m][v], wj, gg[m][v] * rj);
                     }
-                dkp = allreduce_rows(dkp); vg = allreduce_rows(vg);
+                allreduce2_rows(dkp, vg);
                 const float Gt = P - kj * dkp;
                 P = Gt + rdrj;
                 if (g == 0 && tg < T) {
