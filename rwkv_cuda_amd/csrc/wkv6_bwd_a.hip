@@ -340,27 +340,32 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
             }
         } else {
             // ------------------------------------------------------------ exact path: 32 sequential steps
-            for (int t = 0; t < L; ++t) {
-                float vv[2][4], gg[2][4];
+            for (int t4 = 0; t4 < L; t4 += 4) {
+                float dr[4], vg[4];                     // four steps, then their sums over the lane rows in one go
 #pragma unroll
-                for (int mm = 0; mm < 2; ++mm) {
-                    unpack4(*reinterpret_cast<const uint2*>(&O.V[t][i0[mm] >> 1]), vv[mm]);
-                    unpack4(*reinterpret_cast<const uint2*>(&O.GY[t][i0[mm] >> 1]), gg[mm]);
-                }
-                const uint32_t kq = O.Kr[t][j_own >> 1];
-                const float kj = (j_own & 1) ? bf_hi(kq) : bf_lo(kq), wj = O.Ea[t][j_own];
-                float dr = 0.f, vg = 0.f;
+                for (int s = 0; s < 4; ++s) {
+                    const int t = t4 + s;
+                    float vv[2][4], gg[2][4];
 #pragma unroll
-                for (int mm = 0; mm < 2; ++mm)
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        dr = fmaf(gg[mm][v], D[mm][v], dr);
-                        vg = fmaf(gg[mm][v], vv[mm][v], vg);
-                        D[mm][v] = fmaf(D[mm][v], wj, vv[mm][v] * kj);
+                    for (int mm = 0; mm < 2; ++mm) {
+                        unpack4(*reinterpret_cast<const uint2*>(&O.V[t][i0[mm] >> 1]), vv[mm]);
+                        unpack4(*reinterpret_cast<const uint2*>(&O.GY[t][i0[mm] >> 1]), gg[mm]);
                     }
-                allreduce2_rows(dr, vg);
-                if (g == 0) S.Yx[ih][t][j_own] = dr;
-                if (q == 0 && lane == 0) S.Vx[ih][t] = vg;
+                    const uint32_t kq = O.Kr[t][j_own >> 1];
+                    const float kj = (j_own & 1) ? bf_hi(kq) : bf_lo(kq), wj = O.Ea[t][j_own];
+                    dr[s] = 0.f; vg[s] = 0.f;
+#pragma unroll
+                    for (int mm = 0; mm < 2; ++mm)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            dr[s] = fmaf(gg[mm][v], D[mm][v], dr[s]);
+                            vg[s] = fmaf(gg[mm][v], vv[mm][v], vg[s]);
+                            D[mm][v] = fmaf(D[mm][v], wj, vv[mm][v] * kj);
+                        }
+                }
+                S.Yx[ih][t4 + g][j_own] = reduce4_rows(dr[0], dr[1], dr[2], dr[3]);     // lane row g holds step t4 + g
+                const float vgs = reduce4_rows(vg[0], vg[1], vg[2], vg[3]);
+                if (q == 0 && l16 == 0) S.Vx[ih][t4 + g] = vgs;
             }
         }
         __syncthreads();

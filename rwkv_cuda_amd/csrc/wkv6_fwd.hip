@@ -416,25 +416,29 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
                 const float4 y = *reinterpret_cast<const float4*>(&S.u[j0[m]]);
                 uv[m][0] = y.x; uv[m][1] = y.y; uv[m][2] = y.z; uv[m][3] = y.w;
             }
-            for (int t = 0; t < L; ++t) {
-                const uint32_t vv = O.V[t][i_own >> 1];
-                const float vi = (l16 & 1) ? bf_hi(vv) : bf_lo(vv);
-                float yp = 0.f;
+            for (int t4 = 0; t4 < L; t4 += 4) {
+                float yp[4];                            // four steps, then their sums over the lane rows in one go
 #pragma unroll
-                for (int m = 0; m < 2; ++m) {
-                    const float4 r4 = *reinterpret_cast<const float4*>(&R[t * N + j0[m]]);
-                    const float4 k4 = *reinterpret_cast<const float4*>(&K[t * N + j0[m]]);
-                    const float4 w4 = *reinterpret_cast<const float4*>(&O.Wx[t][j0[m]]);
-                    const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, ww[4] = {w4.x, w4.y, w4.z, w4.w};
+                for (int s = 0; s < 4; ++s) {
+                    const int t = t4 + s;
+                    const uint32_t vv = O.V[t][i_own >> 1];
+                    const float vi = (l16 & 1) ? bf_hi(vv) : bf_lo(vv);
+                    yp[s] = 0.f;
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const float kv = kk[v] * vi;
-                        yp = fmaf(rr[v], fmaf(uv[m][v], kv, D[m][v]), yp);
-                        D[m][v] = fmaf(D[m][v], ww[v], kv);
+                    for (int m = 0; m < 2; ++m) {
+                        const float4 r4 = *reinterpret_cast<const float4*>(&R[t * N + j0[m]]);
+                        const float4 k4 = *reinterpret_cast<const float4*>(&K[t * N + j0[m]]);
+                        const float4 w4 = *reinterpret_cast<const float4*>(&O.Wx[t][j0[m]]);
+                        const float rr[4] = {r4.x, r4.y, r4.z, r4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, ww[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            const float kv = kk[v] * vi;
+                            yp[s] = fmaf(rr[v], fmaf(uv[m][v], kv, D[m][v]), yp[s]);
+                            D[m][v] = fmaf(D[m][v], ww[v], kv);
+                        }
                     }
                 }
-                const float y = allreduce_rows(yp);
-                if (g == 0) S.Yx[i & 1][jh][t][i_own] = y;
+                S.Yx[i & 1][jh][t4 + g][i_own] = reduce4_rows(yp[0], yp[1], yp[2], yp[3]);   // lane row g holds step t4 + g
             }
         }
         __syncthreads();
