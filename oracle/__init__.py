@@ -18,6 +18,7 @@ Modules
   wkv56    wkv5 / wkv6 / wkv6_state (bf16 I/O)     wkv5/run.py, wkv6/run.py, wkv6_state/run.py (+ kernels)
   wkv5a    wkv5 with two-sided decay/bonus (fp32)   wkv5a/run.py (+ wkv5a_cuda_v1a2.cu)
   rwkv7    rwkv7 clamp-w with state passing        rwkv7_fast_fused/rwkv7_cuda_benchmark_state_passing.py (+ kernel)
+  rwkv7_chunked  the same recurrence in chunked (matrix-product) form, forward and backward; pinned against rwkv7
 """
 
 import torch
