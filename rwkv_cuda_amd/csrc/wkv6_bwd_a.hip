@@ -36,6 +36,8 @@ struct alignas(16) SmemA2 {
     uint32_t BmH[L][AS], BmL[L][AS];   // Bm[t][s] (s < t) as [t][position of s], hi and lo
     uint4 sel[2][64];                  // selection operands per lane, tile parity 0 and 1
     float4 Xch[NSTATE][64];            // partial (GY S)^T tile handed to the partner wave
+    float outR[2][L][N + 4];              // r dr' and gr of the chunk just finished, [token][channel]: stored one phase later as
+    uint32_t outG[2][L][N / 2 + 2];       // whole rows (a lane of the state waves holds one token and four channels)
     float Yx[2][L][N];                 // exact path: partial dr' of the two value-channel halves;  at the end: gu partial sums
     float Vx[2][L];                    // exact path: partial gy . v
     float vgy[L];                      // gy_t . v_t
@@ -289,12 +291,28 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
     float gu_acc[4] = {0.f, 0.f, 0.f, 0.f};            // chunked path: lane = token of tile ih, rows j4 + v
     float gu_x[4] = {0.f, 0.f, 0.f, 0.f};              // exact path: token xt, channels xj + e
 
+    // The outputs of a chunk leave one phase after they were formed, read back from LDS as whole rows: wave sw takes tokens
+    // 4 sw .. 4 sw + 3, 16 lanes per token (128 B of gr, 256 B of r dr' per row).  Stored straight from the accumulator
+    // layout they would be 8- and 16-byte pieces of sixteen different rows per instruction, which measured 8 % slower.
+    bool staged = false;
+    auto flush = [&](const int c0p, const int pb) __attribute__((always_inline)) {
+        const int row = 4 * sw + g, tg = c0p + row;
+        const uint2 y = *reinterpret_cast<const uint2*>(&S.outG[pb][row][2 * l16]);
+        const float4 x = *reinterpret_cast<const float4*>(&S.outR[pb][row][4 * l16]);
+        if (tg < T) {
+            const uint32_t o = static_cast<uint32_t>(tg) * C + 4 * l16;
+            store8(a.gr + base, o * 2, y);
+            store16(a.rdr + base, o * 4, f32x4{x.x, x.y, x.z, x.w});
+        }
+    };
+
     __syncthreads();
     __syncthreads();
     for (int i = 0; i < nchunks; ++i) {
         const int c0 = i * L;
         const SetA& O = S.set[i & 1];
         const bool exact = __builtin_amdgcn_readfirstlane(O.exact) != 0;
+        bool staged_now = false;
         {
             constexpr int pck = WMODE == W_HEAD ? PCK : 4 * PCK;      // wkv5 sums G over time and needs the shorter walk
             if (i > 0 && i % pck == 0) {               // S at the start of chunk i, for the second sweep's P (see PCK)
@@ -370,7 +388,7 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
         }
         __syncthreads();
         if (!exact) {
-            const int t = 16 * ih + l16, tg = c0 + t;
+            const int t = 16 * ih + l16;
             const float4 p = S.Xch[sw ^ 4][lane];
             const bf16x8 bh_ = lds_op(&S.BmH[t][4 * g]);
             f32x4 dr = own + f32x4{p.x, p.y, p.z, p.w};
@@ -393,11 +411,9 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
                 rd[v] = rr[v] * drp;
                 gu_acc[v] = fmaf(rr[v], kv, gu_acc[v]);
             }
-            if (tg < T) {
-                const uint32_t o = static_cast<uint32_t>(tg) * C + j4;
-                store8(a.gr + base, o * 2, make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3])));
-                store16(a.rdr + base, o * 4, f32x4{rd[0], rd[1], rd[2], rd[3]});
-            }
+            *reinterpret_cast<uint2*>(&S.outG[i & 1][t][j4 >> 1]) = make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3]));
+            *reinterpret_cast<float4*>(&S.outR[i & 1][t][j4]) = make_float4(rd[0], rd[1], rd[2], rd[3]);
+            staged_now = true;
         } else {
             // exact path: add the two halves; token xt, key channels xj .. xj+3
             const float4 p0 = *reinterpret_cast<const float4*>(&S.Yx[0][xt][xj]);
@@ -422,8 +438,11 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
                 store16(a.rdr + base, o * 4, f32x4{rd[0], rd[1], rd[2], rd[3]});
             }
         }
+        if (staged) flush(c0 - L, (i & 1) ^ 1);             // the chunk before: its rows were complete at the last barrier
+        staged = staged_now;
         __syncthreads();
     }
+    if (staged) flush((nchunks - 1) * L, (nchunks - 1) & 1);
     // gu: the chunked path sums over the 16 tokens of a row of lanes; the exact path's sums go by (token, channel) rows
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
