@@ -34,8 +34,8 @@ ALGO = "chunked"
 TRAFFIC_MEASURED = {
     # profiles/wkv6_ws_kernels_B8_T4096_C2048.md  (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB)
     "wkv6_fwd_ws": 537e6 + 134e6,
-    "wkv6_bwd_a_ws": 671e6 + 432e6,
-    "wkv6_bwd_b_ws": 970e6 + 403e6,
+    "wkv6_bwd_a_ws": 683e6 + 432e6,
+    "wkv6_bwd_b_ws": 990e6 + 403e6,
     # profiles/wkv5_ws_kernels_B8_T4096_C2048.md
     "wkv6_bwd_b_ws<head decay>": 936e6 + 269e6,
     # profiles/wkv5_fp32_sweep_kernels_B8_T4096_C4096.md, profiles/wkv5a_sweep_kernels_B8_T4096_C4096.md
