@@ -37,7 +37,7 @@ TRAFFIC_MEASURED = {
     "wkv6_bwd_a_ws": 683e6 + 432e6,
     "wkv6_bwd_b_ws": 990e6 + 403e6,
     # profiles/wkv5_ws_kernels_B8_T4096_C2048.md
-    "wkv6_bwd_b_ws<head decay>": 936e6 + 269e6,
+    "wkv6_bwd_b_ws<head decay>": 957e6 + 269e6,
     # profiles/wkv5_fp32_sweep_kernels_B8_T4096_C4096.md, profiles/wkv5a_sweep_kernels_B8_T4096_C4096.md
     "wkv_sweep<gr+gu+gw, fp32 I/O>": 2148e6 + 537e6,
     "wkv_sweep<gr+gu+gw, two-sided>": 2148e6 + 537e6,
