@@ -28,6 +28,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
 PREWARM_S = 0.3                # seconds of untimed load before the warmup steps (clock ramp)
 ALGO = "chunked"
+FLAGS = 0                      # RWKV_FLAG_SWEEPS when --algo sweeps: passed per call to the *_ex entry points
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), keyed
 # by kernel label at the headline shape; None = not measured for the current kernels.
@@ -84,29 +85,27 @@ def make_wkv6(dev, state):
         gs = new(B, H, N, N)
 
         def step():
-            call("rwkv_wkv6state_forward", dev, B, T, C, H, r, k, v, w, u, s0, y)
-            call("rwkv_wkv6state_backward", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes)
+            call("rwkv_wkv6state_forward_ex", dev, B, T, C, H, r, k, v, w, u, s0, y, FLAGS)
+            call("rwkv_wkv6state_backward_ex", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes, FLAGS)
             return torch.sum(gu, 0).view(H, N)
 
-        kernels = [("wkv6state forward", lambda: call("rwkv_wkv6state_forward", dev, B, T, C, H, r, k, v, w, u, s0, y), 10 * C * tok),
-                   ("wkv6state backward (3 kernels)", lambda: call("rwkv_wkv6state_backward", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes), 18 * C * tok)]
+        kernels = [("wkv6state forward", lambda: call("rwkv_wkv6state_forward_ex", dev, B, T, C, H, r, k, v, w, u, s0, y, FLAGS), 10 * C * tok),
+                   ("wkv6state backward (3 kernels)", lambda: call("rwkv_wkv6state_backward_ex", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes, FLAGS), 18 * C * tok)]
         name = "wkv6_state"
     else:
         def step():
             # what WKV_6.forward / backward do: raw bf16 decay straight into the kernels, per-batch gu summed by torch
-            call("rwkv_wkv6raw_forward", dev, B, T, C, H, r, k, v, w, u, y)
-            call("rwkv_wkv6raw_backward", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+            call("rwkv_wkv6raw_forward_ex", dev, B, T, C, H, r, k, v, w, u, y, FLAGS)
+            call("rwkv_wkv6raw_backward_ex", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes, FLAGS)
             return torch.sum(gu, 0).view(H, N)                      # wrapper reduction, wkv6/run.py:169
 
         def bwd(mask):
             def run():
-                lib.rwkv_wkv6_set_backward_passes(mask)
-                call("rwkv_wkv6raw_backward", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
-                lib.rwkv_wkv6_set_backward_passes(7)
+                call("rwkv_wkv6raw_backward_ex", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes, mask | FLAGS)
             return run
 
         # algorithmic bytes per kernel: tensors it must read once + outputs it must write once, 2 B per element
-        fwd = lambda: call("rwkv_wkv6raw_forward", dev, B, T, C, H, r, k, v, w, u, y)
+        fwd = lambda: call("rwkv_wkv6raw_forward_ex", dev, B, T, C, H, r, k, v, w, u, y, FLAGS)
         if ALGO == "chunked":
             kernels = [("wkv6_fwd_ws", fwd, 10 * C * tok),                    # r k v w -> y
                        ("wkv6_bwd_a_ws", bwd(1), 12 * C * tok),               # r k v w gy -> gr (+ fp32 workspace)
@@ -152,18 +151,16 @@ def make_wkv5(dev):
     def step():
         ew_ = (-torch.exp(w.float())).contiguous()
         eew_ = torch.exp(ew_).contiguous()
-        call("rwkv_wkv5_forward", dev, B, T, C, H, r, k, v, eew_, u, y)
-        call("rwkv_wkv5_backward", dev, B, T, C, H, r, k, v, eew_, ew_, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+        call("rwkv_wkv5_forward_ex", dev, B, T, C, H, r, k, v, eew_, u, y, FLAGS)
+        call("rwkv_wkv5_backward_ex", dev, B, T, C, H, r, k, v, eew_, ew_, u, gy, gr, gk, gv, gw, gu, ws, nbytes, FLAGS)
         return torch.sum(gw, 0), torch.sum(gu, 0)
 
     def bwd(mask):
         def run():
-            lib.rwkv_wkv6_set_backward_passes(mask)
-            call("rwkv_wkv5_backward", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
-            lib.rwkv_wkv6_set_backward_passes(7)
+            call("rwkv_wkv5_backward_ex", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes, mask | FLAGS)
         return run
 
-    kernels = [("wkv6_fwd_ws<head decay>", lambda: call("rwkv_wkv5_forward", dev, B, T, C, H, r, k, v, eew, u, y), 8 * C * tok),
+    kernels = [("wkv6_fwd_ws<head decay>", lambda: call("rwkv_wkv5_forward_ex", dev, B, T, C, H, r, k, v, eew, u, y, FLAGS), 8 * C * tok),
                ("wkv6_bwd_a_ws<head decay>", bwd(1), 10 * C * tok),           # r k v gy -> gr (+ fp32 workspace)
                ("wkv6_bwd_b_ws<head decay>", bwd(4), 12 * C * tok)]           # r k v gy -> gk gv
 
@@ -206,9 +203,7 @@ def make_wkv5_fp32(dev):
 
     def bwd(mask):
         def run():
-            lib.rwkv_wkv6_set_backward_passes(mask)
-            call("rwkv_wkv5f32_backward", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu)
-            lib.rwkv_wkv6_set_backward_passes(7)
+            call("rwkv_wkv5f32_backward_ex", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, mask | FLAGS)
         return run
 
     kernels = [("wkv_sweep<fwd, fp32 I/O>", lambda: call("rwkv_wkv5f32_forward", dev, B, T, C, H, r, k, v, eew, u, y), 16 * C * tok),
@@ -257,9 +252,7 @@ def make_wkv5a(dev):
 
     def bwd(mask):
         def run():
-            lib.rwkv_wkv6_set_backward_passes(mask)
-            call("rwkv_wkv5a_backward", dev, B, T, C, H, r, k, v, eew1, ew1, u1, eew2, ew2, u2, gy, gr, gk, gv, gw1, gu1, gw2, gu2)
-            lib.rwkv_wkv6_set_backward_passes(7)
+            call("rwkv_wkv5a_backward_ex", dev, B, T, C, H, r, k, v, eew1, ew1, u1, eew2, ew2, u2, gy, gr, gk, gv, gw1, gu1, gw2, gu2, mask | FLAGS)
         return run
 
     kernels = [("wkv_sweep<fwd, two-sided>", lambda: call("rwkv_wkv5a_forward", dev, B, T, C, H, r, k, v, eew1, u1, eew2, u2, y), 16 * C * tok),
@@ -443,9 +436,9 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     from rwkv_cuda_amd import _lib
-    global ALGO
+    global ALGO, FLAGS
     ALGO = args.algo
-    _lib.check(_lib.load().rwkv_wkv6_set_algorithm(0 if args.algo == "chunked" else 1))
+    FLAGS = 0x100 if args.algo == "sweeps" else 0
     step, tok, kernels, cfg, cpu_baseline, step_bytes = WORKLOADS[args.workload](dev)
 
     if args.calibrate_copy:

@@ -48,12 +48,20 @@ int rwkv_last_hip_error(void);
 /* ABI version of this header (bumped when a signature changes). */
 int rwkv_abi_version(void);
 
-/* Which kernels serve wkv6 / wkv6_state (process-wide; meant for tests and profiling, no counterpart
- * in the reference).  CHUNKED (default): chunked formulation on the matrix cores.  SWEEPS: the
- * sequential fp32 recurrence kernels, which also serve wkv5. */
-#define RWKV_ALGO_CHUNKED 0
-#define RWKV_ALGO_SWEEPS 1
-int rwkv_wkv6_set_algorithm(int algo);
+/* Per-call options of the *_ex entry points below (no counterpart in the reference).  Every *_ex function is its
+ * reference-signature sibling plus a trailing `flags` word; the sibling is the same call with flags = 0.  Nothing here is
+ * process-wide: two threads may run different algorithms or pass subsets at the same time.
+ *   RWKV_FLAG_SWEEPS : wkv5 / wkv6 / wkv6_state run the sequential fp32 recurrence kernels instead of the chunked
+ *                      matrix-core kernels (second algorithm; the parity anchor of the chunked kernels).
+ *   RWKV_PASS_*      : restrict a backward to a subset of its kernels so that a profiler can time one kernel per call
+ *                      (no pass bit set = all of them).  Sequential kernels: GR (gr, gu, workspace), GV (gv), GK (gk, gw,
+ *                      gs; reads the workspace GR left).  Chunked kernels: GR selects the first sweep (gr, gu, workspace),
+ *                      GK the second (gk, gv, gw, gs); GV alone is empty.  Outputs of the passes left out are not written. */
+#define RWKV_PASS_GR 1u
+#define RWKV_PASS_GV 2u
+#define RWKV_PASS_GK 4u
+#define RWKV_PASS_ALL 7u
+#define RWKV_FLAG_SWEEPS 0x100u
 
 /* ---------------------------------------------------------------------------------------
  * RWKV-4 wkv, fp32.  Replaces cuda_forward / cuda_backward of wkv/cuda/wkv_op.cpp:3-4
@@ -99,12 +107,20 @@ int rwkv_timex_backward_sum(void* stream, const float* w, const float* k, const 
 int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H,
                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                       const float* eew, const rwkv_bf16* u, rwkv_bf16* y);
+int rwkv_wkv5_forward_ex(void* stream, int B, int T, int C, int H,
+                      const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                      const float* eew, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags);
 size_t rwkv_wkv5_backward_workspace_bytes(int B, int T, int C, int H);
 int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H,
                        const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                        const float* eew, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                        void* workspace, size_t workspace_bytes);
+int rwkv_wkv5_backward_ex(void* stream, int B, int T, int C, int H,
+                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                       const float* eew, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
+                       rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                       void* workspace, size_t workspace_bytes, unsigned flags);
 
 /* ---------------------------------------------------------------------------------------
  * RWKV-5 wkv, fp32 I/O.  Replaces cuda_forward / cuda_backward of wkv5/cuda/wkv5_op.cpp:3-4
@@ -122,6 +138,10 @@ int rwkv_wkv5f32_backward(void* stream, int B, int T, int C, int H,
                           const float* r, const float* k, const float* v,
                           const float* eew, const float* ew, const float* u, const float* gy,
                           float* gr, float* gk, float* gv, float* gw, float* gu);
+int rwkv_wkv5f32_backward_ex(void* stream, int B, int T, int C, int H,
+                          const float* r, const float* k, const float* v,
+                          const float* eew, const float* ew, const float* u, const float* gy,
+                          float* gr, float* gk, float* gv, float* gw, float* gu, unsigned flags);
 
 /* ---------------------------------------------------------------------------------------
  * wkv5a: RWKV-5 wkv with two-sided decay and bonus, fp32.  Replaces cuda_forward / cuda_backward of
@@ -139,6 +159,11 @@ int rwkv_wkv5a_backward(void* stream, int B, int T, int C, int H,
                         const float* eew1, const float* ew1, const float* u1,
                         const float* eew2, const float* ew2, const float* u2, const float* gy,
                         float* gr, float* gk, float* gv, float* gw1, float* gu1, float* gw2, float* gu2);
+int rwkv_wkv5a_backward_ex(void* stream, int B, int T, int C, int H,
+                        const float* r, const float* k, const float* v,
+                        const float* eew1, const float* ew1, const float* u1,
+                        const float* eew2, const float* ew2, const float* u2, const float* gy,
+                        float* gr, float* gk, float* gv, float* gw1, float* gu1, float* gw2, float* gu2, unsigned flags);
 
 /* ---------------------------------------------------------------------------------------
  * RWKV-6 wkv, bf16 I/O, per-token decay.  Replaces cuda_forward / cuda_backward of
@@ -150,12 +175,20 @@ int rwkv_wkv5a_backward(void* stream, int B, int T, int C, int H,
 int rwkv_wkv6_forward(void* stream, int B, int T, int C, int H,
                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                       const float* ew, const rwkv_bf16* u, rwkv_bf16* y);
+int rwkv_wkv6_forward_ex(void* stream, int B, int T, int C, int H,
+                      const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                      const float* ew, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags);
 size_t rwkv_wkv6_backward_workspace_bytes(int B, int T, int C, int H);
 int rwkv_wkv6_backward(void* stream, int B, int T, int C, int H,
                        const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                        const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                        void* workspace, size_t workspace_bytes);
+int rwkv_wkv6_backward_ex(void* stream, int B, int T, int C, int H,
+                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                       const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
+                       rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                       void* workspace, size_t workspace_bytes, unsigned flags);
 
 /* RWKV-6 wkv without state, taking the RAW bf16 decay parameter w[B,T,C] (the kernels apply exp(-exp(w)) and
  * return gw w.r.t. w): the wrapper-side pre-transform ew = -exp(w.float()) of wkv6/run.py:147 folded into the
@@ -164,21 +197,19 @@ int rwkv_wkv6_backward(void* stream, int B, int T, int C, int H,
 int rwkv_wkv6raw_forward(void* stream, int B, int T, int C, int H,
                          const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                          const rwkv_bf16* w, const rwkv_bf16* u, rwkv_bf16* y);
+int rwkv_wkv6raw_forward_ex(void* stream, int B, int T, int C, int H,
+                         const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                         const rwkv_bf16* w, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags);
 int rwkv_wkv6raw_backward(void* stream, int B, int T, int C, int H,
                           const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                           const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* gy,
                           rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                           void* workspace, size_t workspace_bytes);
-
-/* Restrict the wkv6 / wkv6raw / wkv6state backward to a subset of its kernels, so that a profiler can time one
- * kernel per call (process-wide; no counterpart in the reference; RWKV_PASS_ALL restores normal operation).
- * Sequential kernels: GR (gr, gu, workspace), GV (gv), GK (gk, gw, gs; reads the workspace GR left).
- * Chunked kernels: GR selects the first sweep (gr, gu, workspace), GK the second (gk, gv, gw, gs); GV alone is empty. */
-#define RWKV_PASS_GR 1u
-#define RWKV_PASS_GV 2u
-#define RWKV_PASS_GK 4u
-#define RWKV_PASS_ALL 7u
-int rwkv_wkv6_set_backward_passes(unsigned passes);
+int rwkv_wkv6raw_backward_ex(void* stream, int B, int T, int C, int H,
+                          const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                          const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* gy,
+                          rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                          void* workspace, size_t workspace_bytes, unsigned flags);
 
 /* ---------------------------------------------------------------------------------------
  * RWKV-6 wkv with initial state.  Replaces cuda_forward / cuda_backward of
@@ -189,12 +220,20 @@ int rwkv_wkv6_set_backward_passes(unsigned passes);
 int rwkv_wkv6state_forward(void* stream, int B, int T, int C, int H,
                            const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                            const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, rwkv_bf16* y);
+int rwkv_wkv6state_forward_ex(void* stream, int B, int T, int C, int H,
+                           const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                           const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, rwkv_bf16* y, unsigned flags);
 size_t rwkv_wkv6state_backward_workspace_bytes(int B, int T, int C, int H);
 int rwkv_wkv6state_backward(void* stream, int B, int T, int C, int H,
                             const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                             const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, const rwkv_bf16* gy,
                             rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                             rwkv_bf16* gs, void* workspace, size_t workspace_bytes);
+int rwkv_wkv6state_backward_ex(void* stream, int B, int T, int C, int H,
+                            const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                            const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, const rwkv_bf16* gy,
+                            rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                            rwkv_bf16* gs, void* workspace, size_t workspace_bytes, unsigned flags);
 
 /* ---------------------------------------------------------------------------------------
  * RWKV-7 "clamp-w" with state passing, bf16 I/O, fp32 states.  Replaces cuda_forward /

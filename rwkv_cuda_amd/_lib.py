@@ -6,6 +6,7 @@ PyTorch fallback: if the library cannot be loaded the import of an op fails loud
 """
 
 import ctypes
+import hashlib
 import os
 import re
 import subprocess
@@ -15,6 +16,7 @@ _ROOT = os.path.dirname(_HERE)
 _CSRC = os.path.join(_HERE, "csrc")
 _INCLUDE = os.path.join(_ROOT, "include")
 LIB_PATH = os.path.join(_HERE, "librwkv_hip.so")
+HASH_PATH = LIB_PATH + ".srchash"        # digest of the sources the library was built from (content, not mtime)
 
 SOURCES = ["abi.hip", "wkv56.hip", "wkv6_fwd.hip", "wkv6_bwd_a.hip", "wkv6_bwd_b.hip", "wkv4.hip", "timex.hip", "rwkv7.hip"]
 
@@ -35,6 +37,14 @@ HIPCC_FLAGS = [
 SPILL_LIMIT = {"wkv6_fwd_ws": 0, "wkv6_bwd_a_ws": 0, "wkv6_bwd_b_wsILi0E": 3, "wkv6_bwd_b_wsILi1E": 1, "wkv6_bwd_b_wsILi2E": 1}
 
 _lib = None
+
+
+def source_hash():
+    h = hashlib.sha256()
+    for path in sorted(os.path.join(_CSRC, f) for f in os.listdir(_CSRC)) + [os.path.join(_INCLUDE, "rwkv_hip.h")]:
+        with open(path, "rb") as f:
+            h.update(os.path.basename(path).encode() + b"\0" + f.read())
+    return h.hexdigest()
 
 
 def build(verbose=False):
@@ -62,6 +72,8 @@ def build(verbose=False):
                     raise RuntimeError(f"{kernel}: {m.group(1)} spilled VGPRs (limit {limit}); its asm-loaded registers must stay in registers")
     if verbose and out.strip():
         print(out, flush=True)
+    with open(HASH_PATH, "w") as f:
+        f.write(source_hash() + "\n")
     return LIB_PATH
 
 
@@ -69,13 +81,13 @@ _P = ctypes.c_void_p
 _I = ctypes.c_int
 _F = ctypes.c_float
 _Z = ctypes.c_size_t
+_U = ctypes.c_uint
 
 # name -> (restype, argtypes): one row per symbol in include/rwkv_hip.h
 SIGNATURES = {
     "rwkv_strerror": (ctypes.c_char_p, [_I]),
     "rwkv_last_hip_error": (_I, []),
     "rwkv_abi_version": (_I, []),
-    "rwkv_wkv6_set_algorithm": (_I, [_I]),
     "rwkv_wkv4_forward": (_I, [_P, _I, _I, _I] + [_P] * 5),
     "rwkv_wkv4_backward_workspace_bytes": (_Z, [_I, _I, _I]),
     "rwkv_wkv4_backward": (_I, [_P, _I, _I, _I] + [_P] * 9 + [_P, _Z]),
@@ -83,21 +95,30 @@ SIGNATURES = {
     "rwkv_timex_backward": (_I, [_P] * 6 + [_I, _I, _I]),
     "rwkv_timex_backward_sum": (_I, [_P] * 6 + [_I, _I, _I]),
     "rwkv_wkv5_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
+    "rwkv_wkv5_forward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 6 + [_U]),
     "rwkv_wkv5_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv5_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_P, _Z]),
+    "rwkv_wkv5_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_P, _Z] + [_U]),
     "rwkv_wkv5f32_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
     "rwkv_wkv5f32_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12),
+    "rwkv_wkv5f32_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_U]),
     "rwkv_wkv5a_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 8),
     "rwkv_wkv5a_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 17),
+    "rwkv_wkv5a_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 17 + [_U]),
     "rwkv_wkv6_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
+    "rwkv_wkv6_forward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 6 + [_U]),
     "rwkv_wkv6_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv6_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z]),
+    "rwkv_wkv6_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z] + [_U]),
     "rwkv_wkv6raw_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
+    "rwkv_wkv6raw_forward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 6 + [_U]),
     "rwkv_wkv6raw_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z]),
-    "rwkv_wkv6_set_backward_passes": (_I, [ctypes.c_uint]),
+    "rwkv_wkv6raw_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z] + [_U]),
     "rwkv_wkv6state_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 7),
+    "rwkv_wkv6state_forward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 7 + [_U]),
     "rwkv_wkv6state_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv6state_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, _Z]),
+    "rwkv_wkv6state_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, _Z] + [_U]),
     "rwkv7_statepassing_forward": (_I, [_P, _I, _I, _I] + [_P] * 11),
     "rwkv7_statepassing_backward": (_I, [_P, _I, _I, _I] + [_P] * 17),
     "rwkv7_state_forward": (_I, [_P, _I, _I, _I] + [_P] * 10),
@@ -120,6 +141,11 @@ def load():
         return _lib
     if not os.path.exists(LIB_PATH):
         build()
+    elif os.path.exists(HASH_PATH):
+        # a library built from other sources than the ones beside it would silently run yesterday's kernels
+        with open(HASH_PATH) as f:
+            if f.read().strip() != source_hash():
+                raise RuntimeError(f"{LIB_PATH} was built from different sources: rebuild it (python __graft_entry__.py)")
     lib = ctypes.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)        # AttributeError here = header and library disagree

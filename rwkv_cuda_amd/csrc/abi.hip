@@ -3,7 +3,6 @@
 
 namespace rwkv {
 thread_local int g_last_hip_error = 0;
-int g_wkv6_algorithm = RWKV_ALGO_CHUNKED;
 }
 
 extern "C" {
@@ -22,12 +21,6 @@ const char* rwkv_strerror(int status) {
 
 int rwkv_last_hip_error(void) { return rwkv::g_last_hip_error; }
 
-int rwkv_abi_version(void) { return 1; }
-
-int rwkv_wkv6_set_algorithm(int algo) {
-    if (algo != RWKV_ALGO_CHUNKED && algo != RWKV_ALGO_SWEEPS) return RWKV_ERR_SHAPE;
-    rwkv::g_wkv6_algorithm = algo;
-    return RWKV_OK;
-}
+int rwkv_abi_version(void) { return 2; }
 
 }  // extern "C"

@@ -144,6 +144,5 @@ int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
                             const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
                             const uint16_t* s0, const uint16_t* gy, uint16_t* gk, uint16_t* gv, uint16_t* gw,
                             uint16_t* gs, const float* rdr);
-extern int g_wkv6_algorithm;     // RWKV_ALGO_*
 
 }  // namespace rwkv

@@ -26,7 +26,6 @@
 #include "common.h"
 
 namespace rwkv {
-extern unsigned g_bwd_passes;
 namespace {
 
 constexpr int N = 64;            // head size
@@ -511,10 +510,13 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
 // The chunked matrix-core kernels serve all three decay conventions; the sequential sweeps remain as the second algorithm.
 // They address one batch row with 32-bit byte offsets (up to 4 bytes per element), so rows of 2^30 elements or more
 // take the sweeps.
-bool use_chunked(const Args& a) { return g_wkv6_algorithm == RWKV_ALGO_CHUNKED && static_cast<long long>(a.T) * a.C < (1LL << 30); }
+bool use_chunked(const Args& a, unsigned flags) { return !(flags & RWKV_FLAG_SWEEPS) && static_cast<long long>(a.T) * a.C < (1LL << 30); }
 
-template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a) {
-    if (use_chunked(a))
+// pass mask of a flags word: no bit set means every pass
+unsigned passes_of(unsigned flags) { return (flags & RWKV_PASS_ALL) ? (flags & RWKV_PASS_ALL) : RWKV_PASS_ALL; }
+
+template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a, unsigned flags) {
+    if (use_chunked(a, flags))
         return launch_wkv6_fwd_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, a.w, a.u, a.s0, a.y);
     hipLaunchKernelGGL((wkv_sweep<P_FWD, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
     return launch_status();
@@ -522,8 +524,9 @@ template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a) {
 
 // GR and GV are independent; GK consumes GR's workspace.  All three run on `st` in order.
 // `passes` is a bit mask (RWKV_PASS_*) so that a profiler can time one kernel at a time.
-template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a, unsigned passes = RWKV_PASS_ALL) {
-    const bool chunked = use_chunked(a);
+template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a, unsigned flags) {
+    const bool chunked = use_chunked(a, flags);
+    const unsigned passes = passes_of(flags);
     const void* w = (WMODE == W_HEAD) ? static_cast<const void*>(a.ew_head) : a.w;   // wkv5: the log decay
     if ((passes & RWKV_PASS_GR) && chunked) {
         if (int e = launch_wkv6_bwd_a_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, w, a.u, a.s0, a.gy, a.gr, a.gu, a.rdr)) return e;
@@ -559,40 +562,30 @@ size_t ws_bytes(int B, int T, int C, int H) {
 
 using namespace rwkv;
 
-namespace rwkv {
-unsigned g_bwd_passes = RWKV_PASS_ALL;
-}
-
 extern "C" {
 
-int rwkv_wkv6_set_backward_passes(unsigned passes) {
-    if (passes == 0 || passes > RWKV_PASS_ALL) return RWKV_ERR_SHAPE;
-    g_bwd_passes = passes;
-    return RWKV_OK;
-}
-
-int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
-                      const rwkv_bf16* v, const float* eew, const rwkv_bf16* u, rwkv_bf16* y) {
+int rwkv_wkv5_forward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                      const rwkv_bf16* v, const float* eew, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, eew, u, y})) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = eew; a.u = u; a.y = y;
-    return launch_fwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a);
+    return launch_fwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a, flags);
 }
 
 size_t rwkv_wkv5_backward_workspace_bytes(int B, int T, int C, int H) { return ws_bytes(B, T, C, H); }
 
-int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+int rwkv_wkv5_backward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                        const rwkv_bf16* v, const float* eew, const float* ew, const rwkv_bf16* u,
                        const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw,
-                       rwkv_bf16* gu, void* workspace, size_t workspace_bytes) {
+                       rwkv_bf16* gu, void* workspace, size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu})) return e;
     if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = eew; a.ew_head = ew; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
-    return launch_bwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a, g_bwd_passes);
+    return launch_bwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a, flags);
 }
 
 // ---- wkv5, fp32 I/O: the sequential fp32 sweeps only (the chunked kernels work to bf16-I/O accuracy)
@@ -612,9 +605,9 @@ int rwkv_wkv5f32_forward(void* stream, int B, int T, int C, int H, const float* 
     return launch_status();
 }
 
-int rwkv_wkv5f32_backward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
+int rwkv_wkv5f32_backward_ex(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
                           const float* eew, const float* ew, const float* u, const float* gy, float* gr, float* gk,
-                          float* gv, float* gw, float* gu) {
+                          float* gv, float* gw, float* gu, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu})) return e;
     Args a{};
@@ -623,9 +616,9 @@ int rwkv_wkv5f32_backward(void* stream, int B, int T, int C, int H, const float*
     a.gw = out_elems(gw); a.gu = out_elems(gu);
     hipStream_t st = static_cast<hipStream_t>(stream);
     // three independent sweeps: gr + gu + gw, gv, gk
-    if (g_bwd_passes & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
-    if (g_bwd_passes & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
-    if (g_bwd_passes & RWKV_PASS_GK) hipLaunchKernelGGL((wkv_sweep<P_GK, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
+    if (passes_of(flags) & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
+    if (passes_of(flags) & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
+    if (passes_of(flags) & RWKV_PASS_GK) hipLaunchKernelGGL((wkv_sweep<P_GK, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
     return launch_status();
 }
 
@@ -641,10 +634,10 @@ int rwkv_wkv5a_forward(void* stream, int B, int T, int C, int H, const float* r,
     return launch_status();
 }
 
-int rwkv_wkv5a_backward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
+int rwkv_wkv5a_backward_ex(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
                         const float* eew1, const float* ew1, const float* u1, const float* eew2, const float* ew2,
                         const float* u2, const float* gy, float* gr, float* gk, float* gv, float* gw1, float* gu1,
-                        float* gw2, float* gu2) {
+                        float* gw2, float* gu2, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, eew1, ew1, u1, eew2, ew2, u2, gy, gr, gk, gv, gw1, gu1, gw2, gu2})) return e;
     Args a{};
@@ -654,82 +647,144 @@ int rwkv_wkv5a_backward(void* stream, int B, int T, int C, int H, const float* r
     a.gw = out_elems(gw1); a.gu = out_elems(gu1); a.gw2 = out_elems(gw2); a.gu2 = out_elems(gu2);
     hipStream_t st = static_cast<hipStream_t>(stream);
     // three independent sweeps: gr + gu1 + gu2 + gw1 + gw2, gv, gk
-    if (g_bwd_passes & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);
-    if (g_bwd_passes & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);
-    if (g_bwd_passes & RWKV_PASS_GK) hipLaunchKernelGGL((wkv_sweep<P_GK, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);
+    if (passes_of(flags) & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);
+    if (passes_of(flags) & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);
+    if (passes_of(flags) & RWKV_PASS_GK) hipLaunchKernelGGL((wkv_sweep<P_GK, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);
     return launch_status();
 }
 
-int rwkv_wkv6_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
-                      const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, rwkv_bf16* y) {
+int rwkv_wkv6_forward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                      const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, ew, u, y})) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.y = y;
-    return launch_fwd<W_EW>(static_cast<hipStream_t>(stream), B, a);
+    return launch_fwd<W_EW>(static_cast<hipStream_t>(stream), B, a, flags);
 }
 
 size_t rwkv_wkv6_backward_workspace_bytes(int B, int T, int C, int H) { return ws_bytes(B, T, C, H); }
 
-int rwkv_wkv6_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+int rwkv_wkv6_backward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                        const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
-                       void* workspace, size_t workspace_bytes) {
-    const unsigned passes = g_bwd_passes;
+                       void* workspace, size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, ew, u, gy, gr, gk, gv, gw, gu})) return e;
     if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
-    return launch_bwd<W_EW>(static_cast<hipStream_t>(stream), B, a, passes);
+    return launch_bwd<W_EW>(static_cast<hipStream_t>(stream), B, a, flags);
 }
 
-int rwkv_wkv6raw_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
-                         const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, rwkv_bf16* y) {
+int rwkv_wkv6raw_forward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                         const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, w, u, y})) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.y = y;
-    return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a);
+    return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, flags);
 }
 
-int rwkv_wkv6raw_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+int rwkv_wkv6raw_backward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                           const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* gy,
                           rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
-                          void* workspace, size_t workspace_bytes) {
+                          void* workspace, size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, w, u, gy, gr, gk, gv, gw, gu})) return e;
     if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
-    return launch_bwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, g_bwd_passes);
+    return launch_bwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, flags);
 }
 
-int rwkv_wkv6state_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+int rwkv_wkv6state_forward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                            const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s,
-                           rwkv_bf16* y) {
+                           rwkv_bf16* y, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, w, u, s, y})) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.y = y;
-    return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a);
+    return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, flags);
 }
 
 size_t rwkv_wkv6state_backward_workspace_bytes(int B, int T, int C, int H) { return ws_bytes(B, T, C, H); }
 
-int rwkv_wkv6state_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+int rwkv_wkv6state_backward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                             const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s,
                             const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw,
-                            rwkv_bf16* gu, rwkv_bf16* gs, void* workspace, size_t workspace_bytes) {
+                            rwkv_bf16* gu, rwkv_bf16* gs, void* workspace, size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, w, u, s, gy, gr, gk, gv, gw, gu, gs})) return e;
     if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.gs = gs; a.rdr = static_cast<float*>(workspace);
-    return launch_bwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, g_bwd_passes);
+    return launch_bwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, flags);
+}
+
+// ---- the reference-signature entry points: default kernels, every pass
+int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                      const rwkv_bf16* v, const float* eew, const rwkv_bf16* u, rwkv_bf16* y) {
+    return rwkv_wkv5_forward_ex(stream, B, T, C, H, r, k, v, eew, u, y, 0u);
+}
+
+int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                       const rwkv_bf16* v, const float* eew, const float* ew, const rwkv_bf16* u,
+                       const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw,
+                       rwkv_bf16* gu, void* workspace, size_t workspace_bytes) {
+    return rwkv_wkv5_backward_ex(stream, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, workspace, workspace_bytes, 0u);
+}
+
+int rwkv_wkv5f32_backward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
+                          const float* eew, const float* ew, const float* u, const float* gy, float* gr, float* gk,
+                          float* gv, float* gw, float* gu) {
+    return rwkv_wkv5f32_backward_ex(stream, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, 0u);
+}
+
+int rwkv_wkv5a_backward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
+                        const float* eew1, const float* ew1, const float* u1, const float* eew2, const float* ew2,
+                        const float* u2, const float* gy, float* gr, float* gk, float* gv, float* gw1, float* gu1,
+                        float* gw2, float* gu2) {
+    return rwkv_wkv5a_backward_ex(stream, B, T, C, H, r, k, v, eew1, ew1, u1, eew2, ew2, u2, gy, gr, gk, gv, gw1, gu1, gw2, gu2, 0u);
+}
+
+int rwkv_wkv6_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                      const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, rwkv_bf16* y) {
+    return rwkv_wkv6_forward_ex(stream, B, T, C, H, r, k, v, ew, u, y, 0u);
+}
+
+int rwkv_wkv6_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                       const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
+                       rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                       void* workspace, size_t workspace_bytes) {
+    return rwkv_wkv6_backward_ex(stream, B, T, C, H, r, k, v, ew, u, gy, gr, gk, gv, gw, gu, workspace, workspace_bytes, 0u);
+}
+
+int rwkv_wkv6raw_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                         const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, rwkv_bf16* y) {
+    return rwkv_wkv6raw_forward_ex(stream, B, T, C, H, r, k, v, w, u, y, 0u);
+}
+
+int rwkv_wkv6raw_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                          const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* gy,
+                          rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                          void* workspace, size_t workspace_bytes) {
+    return rwkv_wkv6raw_backward_ex(stream, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, workspace_bytes, 0u);
+}
+
+int rwkv_wkv6state_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                           const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s,
+                           rwkv_bf16* y) {
+    return rwkv_wkv6state_forward_ex(stream, B, T, C, H, r, k, v, w, u, s, y, 0u);
+}
+
+int rwkv_wkv6state_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
+                            const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s,
+                            const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw,
+                            rwkv_bf16* gu, rwkv_bf16* gs, void* workspace, size_t workspace_bytes) {
+    return rwkv_wkv6state_backward_ex(stream, B, T, C, H, r, k, v, w, u, s, gy, gr, gk, gv, gw, gu, gs, workspace, workspace_bytes, 0u);
 }
 
 }  // extern "C"

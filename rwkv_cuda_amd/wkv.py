@@ -27,10 +27,10 @@ class WKV(torch.autograd.Function):
         w, u, k, v = ctx.saved_tensors
         gy = gy.contiguous()
         dev = check_tensors((gy,), torch.float32, ("gy",))
-        gw = torch.zeros((B, C), device=dev)
-        gu = torch.zeros((B, C), device=dev)
-        gk = torch.empty((B, T, C), device=dev)
-        gv = torch.empty((B, T, C), device=dev)
+        gw = torch.zeros((B, C), device=dev, dtype=torch.float32)
+        gu = torch.zeros((B, C), device=dev, dtype=torch.float32)
+        gk = torch.empty((B, T, C), device=dev, dtype=torch.float32)
+        gv = torch.empty((B, T, C), device=dev, dtype=torch.float32)
         nbytes = _lib.load().rwkv_wkv4_backward_workspace_bytes(B, T, C)
         ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
         call("rwkv_wkv4_backward", dev, B, T, C, w, u, k, v, gy, gw, gu, gk, gv, ws, nbytes)

@@ -2,7 +2,7 @@
 
 import torch
 
-from . import _lib
+from . import _lib, options
 from ._call import call, check_tensors, require
 
 HEAD_SIZE = 64
@@ -19,11 +19,12 @@ class WKV_5(torch.autograd.Function):
             require(HEAD_SIZE == C // H and C == H * HEAD_SIZE, "head size must be 64")
             require(r.numel() == B * T * C and w.numel() == C, "shape mismatch")
             ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
+            ctx.flags = options.current_flags()
             ew = (-torch.exp(w.float())).contiguous()
             eew = (torch.exp(ew)).contiguous()
             ctx.save_for_backward(r, k, v, eew, ew, u)
             y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
-            call("rwkv_wkv5_forward", dev, B, T, C, H, r, k, v, eew, u, y)
+            call("rwkv_wkv5_forward_ex", dev, B, T, C, H, r, k, v, eew, u, y, ctx.flags)
             return y
 
     @staticmethod
@@ -38,7 +39,7 @@ class WKV_5(torch.autograd.Function):
             gw, gu = new(B, C), new(B, C)
             nbytes = _lib.load().rwkv_wkv5_backward_workspace_bytes(B, T, C, H)
             ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
-            call("rwkv_wkv5_backward", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+            call("rwkv_wkv5_backward_ex", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes, ctx.flags)
             gw = torch.sum(gw, 0).view(H, C // H)
             gu = torch.sum(gu, 0).view(H, C // H)
             return (None, None, None, None, gr, gk, gv, gw, gu)

@@ -2,7 +2,7 @@
 
 import torch
 
-from . import _lib
+from . import _lib, options
 from ._call import call, check_tensors, require
 
 HEAD_SIZE = 64
@@ -21,9 +21,10 @@ class WKV_6(torch.autograd.Function):
             require(HEAD_SIZE == C // H and C == H * HEAD_SIZE, "head size must be 64")
             require(r.numel() == B * T * C, "shape mismatch")
             ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
+            ctx.flags = options.current_flags()
             ctx.save_for_backward(r, k, v, w, u)
             y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
-            call("rwkv_wkv6raw_forward", dev, B, T, C, H, r, k, v, w, u, y)
+            call("rwkv_wkv6raw_forward_ex", dev, B, T, C, H, r, k, v, w, u, y, ctx.flags)
             return y
 
     @staticmethod
@@ -38,7 +39,7 @@ class WKV_6(torch.autograd.Function):
             gu = new(B, C)
             nbytes = _lib.load().rwkv_wkv6_backward_workspace_bytes(B, T, C, H)
             ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
-            call("rwkv_wkv6raw_backward", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes)
+            call("rwkv_wkv6raw_backward_ex", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes, ctx.flags)
             gu = torch.sum(gu, 0).view(H, C // H)
             return (None, None, None, None, gr, gk, gv, gw, gu)
 

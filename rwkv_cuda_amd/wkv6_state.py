@@ -2,7 +2,7 @@
 
 import torch
 
-from . import _lib
+from . import _lib, options
 from ._call import call, check_tensors, require
 
 HEAD_SIZE = 64
@@ -19,9 +19,10 @@ class WKV_6STATE(torch.autograd.Function):
             require(HEAD_SIZE == C // H and C == H * HEAD_SIZE, "head size must be 64")
             require(r.numel() == B * T * C and s.numel() == B * H * HEAD_SIZE * HEAD_SIZE, "shape mismatch")
             ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
+            ctx.flags = options.current_flags()
             ctx.save_for_backward(r, k, v, w, u, s)
             y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
-            call("rwkv_wkv6state_forward", dev, B, T, C, H, r, k, v, w, u, s, y)
+            call("rwkv_wkv6state_forward_ex", dev, B, T, C, H, r, k, v, w, u, s, y, ctx.flags)
             return y
 
     @staticmethod
@@ -37,8 +38,8 @@ class WKV_6STATE(torch.autograd.Function):
             gs = new(B, H, C // H, C // H)
             nbytes = _lib.load().rwkv_wkv6state_backward_workspace_bytes(B, T, C, H)
             ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
-            call("rwkv_wkv6state_backward", dev, B, T, C, H, r, k, v, w, u, s, gy,
-                 gr, gk, gv, gw, gu, gs, ws, nbytes)
+            call("rwkv_wkv6state_backward_ex", dev, B, T, C, H, r, k, v, w, u, s, gy,
+                 gr, gk, gv, gw, gu, gs, ws, nbytes, ctx.flags)
             gu = torch.sum(gu, 0).view(H, C // H)
             return (None, None, None, None, gr, gk, gv, gw, gu, gs)
 

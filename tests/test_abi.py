@@ -20,14 +20,14 @@ def _declared_symbols():
 
 def test_header_and_bindings_agree(lib):
     names = _declared_symbols()
-    assert len(names) == 38
+    assert len(names) == len(_lib.SIGNATURES) and len(names) >= 48
     assert sorted(_lib.SIGNATURES) == names
     for n in names:
         assert hasattr(lib, n), f"{n} declared in rwkv_hip.h but not exported"
 
 
 def test_status_text(lib):
-    assert lib.rwkv_abi_version() == 1
+    assert lib.rwkv_abi_version() == 2
     assert lib.rwkv_strerror(0) == b"ok"
     for code in (-1, -2, -3, -4, -5, -99):
         assert len(lib.rwkv_strerror(code)) > 0
@@ -66,6 +66,9 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.rwkv_wkv5a_forward(None, 1, 8, 96, 1, *([p] * 8)) == -1
     assert lib.rwkv_wkv5a_backward(None, 2, 8, 128, 2, *([p] * 16), p + 4) == -3
     assert lib.rwkv_wkv4_backward(None, 1, 4, 4, *([p] * 9), None, 0) == -4
+    # per-call flags: same validation as the plain entry points
+    assert lib.rwkv_wkv6state_backward_ex(None, 2, 8, 128, 2, *([p] * 13), None, 0, 0x100) == -4
+    assert lib.rwkv_wkv6raw_forward_ex(None, 1, 8, 96, 1, p, p, p, p, p, p, 0) == -1
     with pytest.raises(_lib.RwkvHipError):
         _lib.check(-1)
 

@@ -64,7 +64,8 @@ def test_wkv4_extreme_k_stays_finite(lib):
     assert e < 1e-3
 
 
-@pytest.mark.parametrize("B,C,T", [(3, 5, 64), (9, 2, 4), (40, 3, 96), (17, 2, 1024), (32, 768, 768)])
+# the last two: T above the matrix-core kernels' limit (VALU kernels, 1024 threads, near the LDS limit), T % 32 != 0 and T = T_MAX
+@pytest.mark.parametrize("B,C,T", [(3, 5, 64), (9, 2, 4), (40, 3, 96), (17, 2, 1024), (32, 768, 768), (3, 2, 1100), (2, 3, 4096)])
 def test_timex(lib, B, C, T):
     print(f"\ntimex B={B} C={C} T={T}", flush=True)
     w, k, g = synth.timex_inputs(B, C, T, seed=23)

@@ -4,7 +4,7 @@ import torch
 
 from oracle import wkv56 as O
 from oracle import err_ratio
-from rwkv_cuda_amd import _lib, synth, wkv5_bf16, wkv6, wkv6_state
+from rwkv_cuda_amd import _lib, options, synth, wkv5_bf16, wkv6, wkv6_state
 from rwkv_cuda_amd._call import call
 from _gpu_util import DEV, assert_no_worse, garbage
 
@@ -12,6 +12,7 @@ pytestmark = pytest.mark.gpu
 BF = torch.bfloat16
 
 # (B, T, H): T below one staging chunk, not a multiple of it, a multiple, and T = 1
+ALGOS = ["chunked", "sweeps"]
 SHAPES = [(2, 50, 2), (1, 97, 3), (2, 64, 1), (3, 1, 1), (1, 7, 2)]
 
 
@@ -116,6 +117,46 @@ def test_wkv6_full_size_sampled_heads(lib):
             assert e < (4e-3 if name == "gu" else 2.5e-3), (name, e)
 
 
+@pytest.mark.parametrize("entry", ["raw", "ew"])
+def test_wkv6_stateless_full_size_sampled_heads(lib, entry):
+    """The stateless ops at the headline shape B8 T4096 C2048, through the C ABI: rwkv_wkv6raw_* (raw bf16 decay, what
+    WKV_6 and the benchmark call) and rwkv_wkv6_* (fp32 ew = -exp(w), the boundary of wkv6/cuda/wkv6_op.cpp:5-6).
+    Two heads, all batches, full T, against the fp64 oracle; without a state the decay of token 0 feeds nothing."""
+    B, T, H = 8, 4096, 32
+    C = H * 64
+    r, k, v, w, u, gy, _ = synth.wkv6_inputs(B, T, C, H, seed=44)
+    d = [x.to(DEV) for x in (r, k, v, w, u, gy)]
+    wd = d[3] if entry == "raw" else (-torch.exp(d[3].float())).contiguous()
+    name_f, name_b = ("rwkv_wkv6raw_forward", "rwkv_wkv6raw_backward") if entry == "raw" else ("rwkv_wkv6_forward", "rwkv_wkv6_backward")
+    print(f"\nwkv6 stateless full size, entry {entry}", flush=True)
+    y = garbage((B, T, C), BF)
+    call(name_f, d[0].device, B, T, C, H, d[0], d[1], d[2], wd, d[4], y)
+    gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
+    gu = garbage((B, C), BF)
+    n = lib.rwkv_wkv6_backward_workspace_bytes(B, T, C, H)
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+    call(name_b, d[0].device, B, T, C, H, d[0], d[1], d[2], wd, d[4], d[5], gr, gk, gv, gw, gu, ws, n)
+    torch.cuda.synchronize()
+    assert float(gw[:, 0].float().abs().max()) == 0.0 and float(gw[:, T - 1].float().abs().max()) == 0.0
+    gu_sum = gu.float().sum(0).view(H, 64)
+    for h in (3, 28):
+        print(f" head {h}", flush=True)
+        sl = slice(h * 64, (h + 1) * 64)
+        rr, kk, vv, ww, gg = (x[:, :, sl].contiguous().double() for x in (r, k, v, w, gy))
+        uu = u[h:h + 1].double()
+        dec = O.wkv6_decay(ww)
+        yref, _ = O.wkv_recurrent(B, T, 64, 1, rr, kk, vv, dec, uu)
+        rgr, rgk, rgv, G, rgu, _ = O.wkv_backward_hand(B, T, 64, 1, rr, kk, vv, dec, uu, gg)
+        rgw = -torch.exp(ww) * G
+        ref = [yref, rgr, rgk, rgv, rgw, rgu.sum(0)]
+        got = [y[:, :, sl], gr[:, :, sl], gk[:, :, sl], gv[:, :, sl], gw[:, :, sl], gu_sum[h:h + 1]]
+        for name, a, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, got):
+            e = err_ratio(a, g.double().cpu())
+            print(f"  {name}: {e:.3e}", flush=True)
+            # pure bf16 output rounding is 1.7e-3; gu sums 8 bf16 per-batch partials
+            assert e < (4e-3 if name == "gu" else 2.5e-3), (name, e)
+
+
 def test_wkv5_full_size_sampled_heads(lib):
     """wkv5 at B8 T4096 C2048 (per-head constant decay, 128 chunks per sequence): two heads against the fp64 oracle."""
     B, T, H = 8, 4096, 32
@@ -183,18 +224,15 @@ def test_wkv6_fp32_ew_c_abi(lib):
     ew = (-torch.exp(d[3].float())).contiguous()
     for algo in (0, 1):
         print(f"\nwkv6 fp32-ew C-ABI algo={algo}", flush=True)
-        lib.rwkv_wkv6_set_algorithm(algo)
-        try:
-            y = garbage((B, T, C), BF)
-            call("rwkv_wkv6_forward", d[0].device, B, T, C, H, d[0], d[1], d[2], ew, d[4], y)
-            gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
-            gu = garbage((B, C), BF)
-            n = lib.rwkv_wkv6_backward_workspace_bytes(B, T, C, H)
-            ws = torch.empty(n, device=DEV, dtype=torch.uint8)
-            call("rwkv_wkv6_backward", d[0].device, B, T, C, H, d[0], d[1], d[2], ew, d[4], d[5], gr, gk, gv, gw, gu, ws, n)
-            torch.cuda.synchronize()
-        finally:
-            lib.rwkv_wkv6_set_algorithm(0)
+        flags = options.FLAG_SWEEPS if algo else 0
+        y = garbage((B, T, C), BF)
+        call("rwkv_wkv6_forward_ex", d[0].device, B, T, C, H, d[0], d[1], d[2], ew, d[4], y, flags)
+        gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
+        gu = garbage((B, C), BF)
+        n = lib.rwkv_wkv6_backward_workspace_bytes(B, T, C, H)
+        ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+        call("rwkv_wkv6_backward_ex", d[0].device, B, T, C, H, d[0], d[1], d[2], ew, d[4], d[5], gr, gk, gv, gw, gu, ws, n, flags)
+        torch.cuda.synchronize()
         for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y, gr, gk, gv, gw, gu.sum(0).view(H, 64)]):
             assert_no_worse(name, a, e, g)
 
@@ -216,14 +254,11 @@ def test_wkv6_state_both_algorithms_and_extreme_decays(lib, algo):
         ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
         emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
         print(f"\nwkv6_state algo={algo} extreme={extreme}", flush=True)
-        lib.rwkv_wkv6_set_algorithm(algo)
-        try:
-            t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u, s0)]
+        t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u, s0)]
+        with options.algorithm(ALGOS[algo]):
             y = wkv6_state.RUN_CUDA(B, T, C, H, *t)
-            y.backward(gy.to(DEV))
-            torch.cuda.synchronize()
-        finally:
-            lib.rwkv_wkv6_set_algorithm(0)
+        y.backward(gy.to(DEV))               # outside the block: the backward follows the forward's choice
+        torch.cuda.synchronize()
         for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, emu, [y] + [x.grad for x in t]):
             assert torch.isfinite(g).all(), name
             assert_no_worse(name, a, e, g)
@@ -245,14 +280,11 @@ def test_wkv5_both_algorithms_and_strong_decays(lib, algo):
         ref = O.wkv5_grads(B, T, C, H, r, k, v, w, u, gy)
         emu = O.emulate_wkv5_bf16(B, T, C, H, r, k, v, w, u, gy)
         print(f"\nwkv5 algo={algo} strong={strong}", flush=True)
-        lib.rwkv_wkv6_set_algorithm(algo)
-        try:
-            t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u)]
+        t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u)]
+        with options.algorithm(ALGOS[algo]):
             y = wkv5_bf16.RUN_CUDA(B, T, C, H, *t)
             y.backward(gy.to(DEV))
-            torch.cuda.synchronize()
-        finally:
-            lib.rwkv_wkv6_set_algorithm(0)
+        torch.cuda.synchronize()
         for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y] + [x.grad for x in t]):
             assert torch.isfinite(g).all(), name
             assert_no_worse(name, a, e, g)
@@ -277,8 +309,7 @@ def test_decay_gradient_where_the_decay_has_vanished(lib, algo):
     w = _low_rank_decay(B, T, C, seed=52)
     assert float(w.max()) > 8 and float(w.min()) < -8
     gone = w.float() > 4.5                                   # exp(-exp(4.5)) < 1e-39
-    lib.rwkv_wkv6_set_algorithm(algo)
-    try:
+    with options.algorithm(ALGOS[algo]):
         for state in (None, s0):
             print(f"\nlow-rank decays algo={algo} state={state is not None}", flush=True)
             ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=state)
@@ -309,5 +340,3 @@ def test_decay_gradient_where_the_decay_has_vanished(lib, algo):
         for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y] + [x.grad for x in t]):
             assert_no_worse("wkv5 " + name, a, e, g)
         assert float(t[3].grad.float().cpu()[0, 5:12].abs().max()) == 0.0
-    finally:
-        lib.rwkv_wkv6_set_algorithm(0)

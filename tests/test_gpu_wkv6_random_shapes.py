@@ -1,6 +1,6 @@
 """GPU: the chunked matrix-core kernels against the sequential fp32 sweeps on random shapes and decay strengths.
 
-Both algorithms round the same quantities to bf16, so they may differ by one bf16 unit of the value (2^-8 relative);
+Both algorithms round the same quantities to bf16, so they may differ by one bf16 unit of the value (2^-8 relative to the value, under 2^-7 of the tensor's peak);
 a slip in the chunk logic (a partial last chunk, the exact-path switch, state passing) shows up as an error of order one.
 Every result is also checked against the fp64 oracle with the usual bar."""
 import random
@@ -9,7 +9,7 @@ import pytest
 import torch
 
 from oracle import wkv56 as O
-from rwkv_cuda_amd import _lib, synth
+from rwkv_cuda_amd import options, synth
 from rwkv_cuda_amd._call import call
 from _gpu_util import DEV, assert_no_worse, garbage
 
@@ -18,19 +18,16 @@ BF = torch.bfloat16
 
 
 def _run(lib, algo, B, T, C, H, d):
-    _lib.check(lib.rwkv_wkv6_set_algorithm(algo))
-    try:
-        y = garbage((B, T, C), BF)
-        call("rwkv_wkv6state_forward", d[0].device, B, T, C, H, *d[:6], y)
-        gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
-        gu = garbage((B, C), BF)
-        gs = garbage((B, H, 64, 64), BF)
-        n = lib.rwkv_wkv6state_backward_workspace_bytes(B, T, C, H)
-        ws = torch.empty(max(n, 16), device=DEV, dtype=torch.uint8)
-        call("rwkv_wkv6state_backward", d[0].device, B, T, C, H, *d[:6], d[6], gr, gk, gv, gw, gu, gs, ws, n)
-        torch.cuda.synchronize()
-    finally:
-        _lib.check(lib.rwkv_wkv6_set_algorithm(0))
+    flags = options.FLAG_SWEEPS if algo else 0
+    y = garbage((B, T, C), BF)
+    call("rwkv_wkv6state_forward_ex", d[0].device, B, T, C, H, *d[:6], y, flags)
+    gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
+    gu = garbage((B, C), BF)
+    gs = garbage((B, H, 64, 64), BF)
+    n = lib.rwkv_wkv6state_backward_workspace_bytes(B, T, C, H)
+    ws = torch.empty(max(n, 16), device=DEV, dtype=torch.uint8)
+    call("rwkv_wkv6state_backward_ex", d[0].device, B, T, C, H, *d[:6], d[6], gr, gk, gv, gw, gu, gs, ws, n, flags)
+    torch.cuda.synchronize()
     return [y, gr, gk, gv, gw, gu.sum(0).view(H, 64), gs]
 
 
@@ -56,7 +53,7 @@ def test_wkv6_state_chunked_equals_sweeps(lib, seed):
         if peak > 0.0:
             diff = float((c.float() - s.float()).abs().max()) / peak
             print(f"  {name}: chunked vs sweeps, max difference / peak {diff:.3e}", flush=True)
-            assert diff < 2.0 ** -6, (name, diff)
+            assert diff <= 2.0 ** -7, (name, diff)
 
 
 REGIMES = ["wide", "alternating", "tiny", "zero_k", "big_u", "large_inputs"]
