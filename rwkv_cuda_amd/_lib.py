@@ -41,7 +41,9 @@ _lib = None
 
 def source_hash():
     h = hashlib.sha256()
-    for path in sorted(os.path.join(_CSRC, f) for f in os.listdir(_CSRC)) + [os.path.join(_INCLUDE, "rwkv_hip.h")]:
+    # the kernel sources and their headers; csrc/binding.cpp is the torch-side shim, built separately (binding.py)
+    files = sorted(f for f in os.listdir(_CSRC) if f.endswith((".hip", ".h")))
+    for path in [os.path.join(_CSRC, f) for f in files] + [os.path.join(_INCLUDE, "rwkv_hip.h")]:
         with open(path, "rb") as f:
             h.update(os.path.basename(path).encode() + b"\0" + f.read())
     return h.hexdigest()

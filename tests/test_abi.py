@@ -86,3 +86,17 @@ def test_ops_refuse_cpu_tensors():
     x4 = x.view(B, T, H, 64)
     with pytest.raises(AssertionError):
         rwkv7_fast_fused.RWKV7_STATE_PASSING_CLAMPW_CUDA_OP.apply(torch.zeros(B, H, 64, 64), x4, x4, x4, x4, x4, x4)
+
+
+def test_reference_style_extension_loads_and_registers_its_ops(lib):
+    """csrc/binding.cpp: one pybind submodule per reference extension and the TORCH_LIBRARY names of the *_op.cpp files."""
+    from rwkv_cuda_amd import binding
+    ext = binding.load()
+    for name in ("wkv", "timex", "wkv5", "wkv5a", "wkv6", "wkv6state", "rwkv7_clampw", "rwkv7_state_clampw", "rwkv7_statepassing_clampw"):
+        sub = getattr(ext, name)
+        assert callable(sub.forward) and callable(sub.backward)
+    for ns in ("wkv", "timex", "wkv5", "wkv5a", "wkv6", "wkv6b", "rwkv7_clampw", "rwkv7_state_clampw", "rwkv7_statepassing_clampw"):
+        assert getattr(torch.ops, ns).forward is not None and getattr(torch.ops, ns).backward is not None
+    c = torch.zeros(4)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        ext.wkv.forward(1, 1, 4, c, c, c, c, c)
