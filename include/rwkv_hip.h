@@ -80,6 +80,17 @@ int rwkv_wkv4_backward(void* stream, int B, int T, int C,
                        float* gw, float* gu, float* gk, float* gv,
                        void* workspace, size_t workspace_bytes);
 
+/* rwkv_wkv4_backward without a workspace argument and without any allocation.  It has no counterpart in the reference;
+ * it is for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc.  The backward's scratch (B*T*C floats) lives in a file-scope device array of the library,
+ * rwkv_wkv4_backward_noalloc_max_elems() floats (8 MiB) that every GPU the library runs on holds until the process
+ * ends; B*T*C beyond that returns RWKV_ERR_WORKSPACE.  All calls on one GPU share that one array: calls that overlap
+ * in time on the same GPU (two streams, two threads) race; serialise them.  Results are those of rwkv_wkv4_backward. */
+size_t rwkv_wkv4_backward_noalloc_max_elems(void);
+int rwkv_wkv4_backward_noalloc(void* stream, int B, int T, int C,
+                               const float* w, const float* u, const float* k, const float* v, const float* gy,
+                               float* gw, float* gu, float* gk, float* gv);
+
 /* ---------------------------------------------------------------------------------------
  * depthwise_conv1d ("TimeX"), fp32.  Replaces cuda_forward / cuda_backward of
  * depthwise_conv1d/cuda/timex_op.cpp:3-4 (kernels: timex_cuda_v3.cu:7-150).

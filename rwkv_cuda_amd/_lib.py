@@ -93,6 +93,8 @@ SIGNATURES = {
     "rwkv_wkv4_forward": (_I, [_P, _I, _I, _I] + [_P] * 5),
     "rwkv_wkv4_backward_workspace_bytes": (_Z, [_I, _I, _I]),
     "rwkv_wkv4_backward": (_I, [_P, _I, _I, _I] + [_P] * 9 + [_P, _Z]),
+    "rwkv_wkv4_backward_noalloc_max_elems": (_Z, []),
+    "rwkv_wkv4_backward_noalloc": (_I, [_P, _I, _I, _I] + [_P] * 9),
     "rwkv_timex_forward": (_I, [_P, _P, _P, _P, _F, _I, _I, _I]),
     "rwkv_timex_backward": (_I, [_P] * 6 + [_I, _I, _I]),
     "rwkv_timex_backward_sum": (_I, [_P] * 6 + [_I, _I, _I]),

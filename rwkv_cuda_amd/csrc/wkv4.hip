@@ -11,6 +11,8 @@
 // whose lanes of a wave are 64 consecutive channels (256 contiguous bytes per tensor and step).
 #include <math.h>
 
+#include <atomic>
+
 #include "common.h"
 
 namespace rwkv {
@@ -355,6 +357,30 @@ int check4(int B, int T, int C) {
     return RWKV_OK;
 }
 
+// Scratch of the entry point that allocates nothing: the backward's per-step intermediates (B*T*C floats) live in this
+// file-scope device array instead of a caller's workspace.  Each GPU the library runs on holds its own copy, at its own
+// address, until the process ends.  `scratch` itself is only a host-side handle: the device address comes from
+// hipGetSymbolAddress, once per device, and that address is what the kernels receive.
+constexpr size_t NOALLOC_MAX_FLOATS = size_t(1) << 21;           // 8 MiB: B*T*C <= 2 097 152 (B4 T512 C768 needs 1 572 864)
+static __device__ __align__(256) float scratch[NOALLOC_MAX_FLOATS];
+constexpr int MAX_DEVICES = 64;
+std::atomic<float*> g_scratch_ptr[MAX_DEVICES];                  // written once per device; every writer stores the same value
+
+int scratch_of_current_device(float** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return RWKV_ERR_LAUNCH;
+    float* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        void* sym = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || sym == nullptr) { g_last_hip_error = static_cast<int>(e); return RWKV_ERR_LAUNCH; }
+        p = static_cast<float*>(sym);
+        g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+    *out = p;
+    return RWKV_OK;
+}
+
 }  // namespace
 }  // namespace rwkv
 
@@ -398,6 +424,18 @@ int rwkv_wkv4_backward(void* stream, int B, int T, int C, const float* w, const 
     hipLaunchKernelGGL(wkv4_bwd_seg, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
                        T, C, (T + NSEG - 1) / NSEG, w, u, k, v, gy, gw, gu, gk, gv, static_cast<float*>(workspace));
     return launch_status();
+}
+
+size_t rwkv_wkv4_backward_noalloc_max_elems(void) { return NOALLOC_MAX_FLOATS; }
+
+int rwkv_wkv4_backward_noalloc(void* stream, int B, int T, int C, const float* w, const float* u, const float* k,
+                               const float* v, const float* gy, float* gw, float* gu, float* gk, float* gv) {
+    if (int e = check4(B, T, C)) return e;
+    if (static_cast<unsigned long long>(B) * T * C > NOALLOC_MAX_FLOATS) return RWKV_ERR_WORKSPACE;
+    float* ws = nullptr;
+    if (int e = scratch_of_current_device(&ws)) return e;
+    // every element of the scratch that the kernels read they have written earlier in the same launch: nothing to clear
+    return rwkv_wkv4_backward(stream, B, T, C, w, u, k, v, gy, gw, gu, gk, gv, ws, static_cast<size_t>(B) * T * C * sizeof(float));
 }
 
 }  // extern "C"

@@ -1,0 +1,46 @@
+"""GPU: the entry point that allocates nothing (rwkv_wkv4_backward_noalloc) against rwkv_wkv4_backward, through the
+C ABI, on two calls in a row, the second with a smaller input (the shared scratch keeps the first call's contents)."""
+import pytest
+import torch
+
+from rwkv_cuda_amd import synth
+from rwkv_cuda_amd._call import call
+from _gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(lib, B, T, C, seed):
+    w_raw, u, k, v, gy = (x.to(DEV) for x in synth.wkv4_inputs(B, T, C, seed=seed))
+    w = -torch.exp(w_raw)
+    out = []
+    for noalloc in (False, True):
+        gw = torch.zeros(B, C, device=DEV, dtype=torch.float32)
+        gu = torch.zeros(B, C, device=DEV, dtype=torch.float32)
+        gk = torch.full((B, T, C), 7.0, device=DEV, dtype=torch.float32)
+        gv = torch.full((B, T, C), -7.0, device=DEV, dtype=torch.float32)
+        if noalloc:
+            call("rwkv_wkv4_backward_noalloc", gy.device, B, T, C, w, u, k, v, gy, gw, gu, gk, gv)
+        else:
+            n = lib.rwkv_wkv4_backward_workspace_bytes(B, T, C)
+            ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+            call("rwkv_wkv4_backward", gy.device, B, T, C, w, u, k, v, gy, gw, gu, gk, gv, ws, n)
+        torch.cuda.synchronize()
+        out.append((gw, gu, gk, gv))
+    return out
+
+
+def test_noalloc_equals_workspace_entry_point_twice(lib):
+    assert lib.rwkv_wkv4_backward_noalloc_max_elems() == 1 << 21
+    for B, T, C, seed in ((4, 512, 768, 5), (2, 37, 80, 6)):      # the second call is smaller than the first
+        print(f"\nwkv4 noalloc B={B} T={T} C={C}", flush=True)
+        ref, got = _both(lib, B, T, C, seed)
+        for name, a, g in zip(("gw", "gu", "gk", "gv"), ref, got):
+            assert torch.equal(a, g), name                         # same kernels, same order of operations: bit-identical
+
+
+def test_noalloc_rejects_sizes_beyond_its_scratch(lib):
+    B, T, C = 4, 1024, 768                                         # 3 145 728 elements > 2 097 152
+    z = torch.zeros(16, device=DEV, dtype=torch.float32)
+    status = lib.rwkv_wkv4_backward_noalloc(None, B, T, C, *([z.data_ptr()] * 9))
+    assert status == -4
