@@ -270,6 +270,21 @@ int rwkv7_statepassing_backward(void* stream, int B, int T, int H,
                                 rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv,
                                 rwkv_bf16* da, rwkv_bf16* db);
 
+/* The state-passing op with the per-call flags word (RWKV_FLAG_SWEEPS: the step-by-step recurrence kernels instead of
+ * the chunked matrix-core kernels; the two families lay `s` out differently, so a backward must be given the flags of
+ * its forward).  Here s0 and sT (forward), dsT and ds0 (backward) may be NULL: a missing s0 / dsT is zero, a missing
+ * sT / ds0 is not written.  No counterpart in the reference. */
+int rwkv7_statepassing_forward_ex(void* stream, int B, int T, int H,
+                                  const float* s0, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
+                                  const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b,
+                                  rwkv_bf16* y, float* sT, float* s, float* sa, unsigned flags);
+int rwkv7_statepassing_backward_ex(void* stream, int B, int T, int H,
+                                   const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k, const rwkv_bf16* v,
+                                   const rwkv_bf16* a, const rwkv_bf16* b, const rwkv_bf16* dy, const float* dsT,
+                                   const float* s, const float* sa, float* ds0,
+                                   rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv,
+                                   rwkv_bf16* da, rwkv_bf16* db, unsigned flags);
+
 /* The two siblings of the state-passing op, served by the same kernels:
  *   rwkv7_state_*  : initial state s0 and its gradient ds0, no final state.  Replaces cuda_forward /
  *                    cuda_backward of rwkv7_fast_fused/cuda/rwkv7_state_clampw.cpp:10,17.

@@ -18,7 +18,7 @@ _INCLUDE = os.path.join(_ROOT, "include")
 LIB_PATH = os.path.join(_HERE, "librwkv_hip.so")
 HASH_PATH = LIB_PATH + ".srchash"        # digest of the sources the library was built from (content, not mtime)
 
-SOURCES = ["abi.hip", "wkv56.hip", "wkv6_fwd.hip", "wkv6_bwd_a.hip", "wkv6_bwd_b.hip", "wkv4.hip", "timex.hip", "rwkv7.hip"]
+SOURCES = ["abi.hip", "wkv56.hip", "wkv6_fwd.hip", "wkv6_bwd_a.hip", "wkv6_bwd_b.hip", "wkv4.hip", "timex.hip", "rwkv7.hip", "rwkv7_chunk.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -125,6 +125,8 @@ SIGNATURES = {
     "rwkv_wkv6state_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, _Z] + [_U]),
     "rwkv7_statepassing_forward": (_I, [_P, _I, _I, _I] + [_P] * 11),
     "rwkv7_statepassing_backward": (_I, [_P, _I, _I, _I] + [_P] * 17),
+    "rwkv7_statepassing_forward_ex": (_I, [_P, _I, _I, _I] + [_P] * 11 + [_U]),
+    "rwkv7_statepassing_backward_ex": (_I, [_P, _I, _I, _I] + [_P] * 17 + [_U]),
     "rwkv7_state_forward": (_I, [_P, _I, _I, _I] + [_P] * 10),
     "rwkv7_state_backward": (_I, [_P, _I, _I, _I] + [_P] * 16),
     "rwkv7_forward": (_I, [_P, _I, _I, _I] + [_P] * 9),

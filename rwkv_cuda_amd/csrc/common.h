@@ -145,4 +145,11 @@ int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
                             const uint16_t* s0, const uint16_t* gy, uint16_t* gk, uint16_t* gv, uint16_t* gw,
                             uint16_t* gs, const float* rdr);
 
+// rwkv7_chunk.hip: chunked rwkv7 kernels (bf16 I/O); s0, sT, dsT, ds0 may be null
+int launch7c_fwd(hipStream_t st, int B, int T, int H, const float* s0, const uint16_t* r, const uint16_t* w, const uint16_t* k,
+                 const uint16_t* v, const uint16_t* a, const uint16_t* b, uint16_t* y, float* sT, float* s, float* sa);
+int launch7c_bwd(hipStream_t st, int B, int T, int H, const uint16_t* r, const uint16_t* w, const uint16_t* k, const uint16_t* v,
+                 const uint16_t* a, const uint16_t* b, const uint16_t* dy, const float* dsT, const float* s, const float* sa,
+                 float* ds0, uint16_t* dr, uint16_t* dw, uint16_t* dk, uint16_t* dv, uint16_t* da, uint16_t* db);
+
 }  // namespace rwkv

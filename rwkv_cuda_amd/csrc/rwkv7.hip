@@ -365,6 +365,24 @@ int launch7_bwd(void* stream, bool f32, int B, int T, int H, const void* r, cons
     return launch_status();
 }
 
+
+// bf16 mode: the chunked matrix-core kernels (rwkv7_chunk.hip) unless RWKV_FLAG_SWEEPS asks for the step kernels above.
+// The two families lay out the scratch tensor `s` differently, so a backward must get the flags of its forward.
+constexpr unsigned DEFAULT7 = 0u;                   // what the entry points without a flags argument run: the chunked kernels
+int bf16_fwd(void* stream, unsigned flags, int B, int T, int H, const float* s0, const rwkv_bf16* r, const rwkv_bf16* w,
+             const rwkv_bf16* k, const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b, rwkv_bf16* y, float* sT,
+             float* s, float* sa) {
+    if (flags & RWKV_FLAG_SWEEPS) return launch7_fwd(stream, false, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa);
+    return launch7c_fwd(static_cast<hipStream_t>(stream), B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa);
+}
+int bf16_bwd(void* stream, unsigned flags, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
+             const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b, const rwkv_bf16* dy, const float* dsT,
+             const float* s, const float* sa, float* ds0, rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv,
+             rwkv_bf16* da, rwkv_bf16* db) {
+    if (flags & RWKV_FLAG_SWEEPS) return launch7_bwd(stream, false, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db);
+    return launch7c_bwd(static_cast<hipStream_t>(stream), B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db);
+}
+
 }  // namespace
 }  // namespace rwkv
 
@@ -377,7 +395,7 @@ int rwkv7_statepassing_forward(void* stream, int B, int T, int H, const float* s
                                const rwkv_bf16* b, rwkv_bf16* y, float* sT, float* s, float* sa) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({s0, r, w, k, v, a, b, y, sT, s, sa})) return e;
-    return launch7_fwd(stream, false, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa);
+    return bf16_fwd(stream, DEFAULT7, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa);
 }
 
 int rwkv7_statepassing_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w,
@@ -387,7 +405,7 @@ int rwkv7_statepassing_backward(void* stream, int B, int T, int H, const rwkv_bf
                                 rwkv_bf16* da, rwkv_bf16* db) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db})) return e;
-    return launch7_bwd(stream, false, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db);
+    return bf16_bwd(stream, DEFAULT7, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db);
 }
 
 // Initial state with its gradient, no final state: the same kernels without the sT store and with dsT = 0.
@@ -396,7 +414,7 @@ int rwkv7_state_forward(void* stream, int B, int T, int H, const float* s0, cons
                         rwkv_bf16* y, float* s, float* sa) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({s0, r, w, k, v, a, b, y, s, sa})) return e;
-    return launch7_fwd(stream, false, B, T, H, s0, r, w, k, v, a, b, y, nullptr, s, sa);
+    return bf16_fwd(stream, DEFAULT7, B, T, H, s0, r, w, k, v, a, b, y, nullptr, s, sa);
 }
 
 int rwkv7_state_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w,
@@ -405,7 +423,7 @@ int rwkv7_state_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, 
                          rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv, rwkv_bf16* da, rwkv_bf16* db) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({r, w, k, v, a, b, dy, s, sa, ds0, dr, dw, dk, dv, da, db})) return e;
-    return launch7_bwd(stream, false, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, ds0, dr, dw, dk, dv, da, db);
+    return bf16_bwd(stream, DEFAULT7, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, ds0, dr, dw, dk, dv, da, db);
 }
 
 // No state on either side: zero initial state, no final state, no state gradients.
@@ -413,7 +431,7 @@ int rwkv7_forward(void* stream, int B, int T, int H, const rwkv_bf16* r, const r
                   const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b, rwkv_bf16* y, float* s, float* sa) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({r, w, k, v, a, b, y, s, sa})) return e;
-    return launch7_fwd(stream, false, B, T, H, nullptr, r, w, k, v, a, b, y, nullptr, s, sa);
+    return bf16_fwd(stream, DEFAULT7, B, T, H, nullptr, r, w, k, v, a, b, y, nullptr, s, sa);
 }
 
 int rwkv7_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,
@@ -422,7 +440,29 @@ int rwkv7_backward(void* stream, int B, int T, int H, const rwkv_bf16* r, const 
                    rwkv_bf16* db) {
     if (int e = check7(B, T, H)) return e;
     if (int e = check_ptrs({r, w, k, v, a, b, dy, s, sa, dr, dw, dk, dv, da, db})) return e;
-    return launch7_bwd(stream, false, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, nullptr, dr, dw, dk, dv, da, db);
+    return bf16_bwd(stream, DEFAULT7, B, T, H, r, w, k, v, a, b, dy, nullptr, s, sa, nullptr, dr, dw, dk, dv, da, db);
+}
+
+// The state-passing op with per-call flags; s0, sT (forward) and dsT, ds0 (backward) may be NULL, which makes these two
+// entry points cover the state-only and the stateless siblings as well.
+int rwkv7_statepassing_forward_ex(void* stream, int B, int T, int H, const float* s0, const rwkv_bf16* r,
+                                  const rwkv_bf16* w, const rwkv_bf16* k, const rwkv_bf16* v, const rwkv_bf16* a,
+                                  const rwkv_bf16* b, rwkv_bf16* y, float* sT, float* s, float* sa, unsigned flags) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({r, w, k, v, a, b, y, s, sa})) return e;
+    if (!aligned16(s0) || !aligned16(sT)) return RWKV_ERR_ALIGN;
+    return bf16_fwd(stream, flags, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa);
+}
+
+int rwkv7_statepassing_backward_ex(void* stream, int B, int T, int H, const rwkv_bf16* r, const rwkv_bf16* w,
+                                   const rwkv_bf16* k, const rwkv_bf16* v, const rwkv_bf16* a, const rwkv_bf16* b,
+                                   const rwkv_bf16* dy, const float* dsT, const float* s, const float* sa,
+                                   float* ds0, rwkv_bf16* dr, rwkv_bf16* dw, rwkv_bf16* dk, rwkv_bf16* dv,
+                                   rwkv_bf16* da, rwkv_bf16* db, unsigned flags) {
+    if (int e = check7(B, T, H)) return e;
+    if (int e = check_ptrs({r, w, k, v, a, b, dy, s, sa, dr, dw, dk, dv, da, db})) return e;
+    if (!aligned16(dsT) || !aligned16(ds0)) return RWKV_ERR_ALIGN;
+    return bf16_bwd(stream, flags, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db);
 }
 
 // ---- fp32 I/O: what the reference builds from the same sources with -D_FP32_ (rwkv7_cuda_benchmark.py:102-126 and the

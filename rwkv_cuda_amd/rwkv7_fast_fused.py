@@ -6,6 +6,7 @@ rwkv7_fast_fused/rwkv7_cuda_benchmark.py:76-100 (RWKV7_CLAMPW_CUDA_OP, ..._CUDA:
 
 import torch
 
+from . import options
 from ._call import call, check_tensors, require
 
 HEAD_SIZE = 64
@@ -36,7 +37,13 @@ class RWKV7_STATE_PASSING_CLAMPW_CUDA_OP(torch.autograd.Function):
         sT = torch.empty_like(s0)
         s = torch.empty(B, H, T // CHUNK_LEN, N, N, dtype=torch.float32, device=dev)
         sa = torch.empty(B, T, H, N, dtype=torch.float32, device=dev)
-        call("rwkv7_statepassing_forward" + sfx, dev, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa)
+        # bf16 mode: chunked matrix-core kernels unless options.algorithm("sweeps") is active; the backward must follow the
+        # forward's choice (the two kernel families lay `s` out differently), so the flags ride on the context
+        ctx.flags = options.current_flags()
+        if sfx:
+            call("rwkv7_statepassing_forward_f32", dev, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa)
+        else:
+            call("rwkv7_statepassing_forward_ex", dev, B, T, H, s0, r, w, k, v, a, b, y, sT, s, sa, ctx.flags)
         ctx.save_for_backward(r, w, k, v, a, b, s, sa)
         return y.view(B, T, H * N), sT
 
@@ -50,8 +57,10 @@ class RWKV7_STATE_PASSING_CLAMPW_CUDA_OP(torch.autograd.Function):
         dev = check_tensors((dy,), dt, ("dy",))
         check_tensors((dsT,), torch.float32, ("dsT",))
         ds0, dr, dw, dk, dv, da, db = [torch.empty_like(x) for x in [dsT, r, w, k, v, a, b]]
-        call("rwkv7_statepassing_backward" + sfx, dev, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa,
-             ds0, dr, dw, dk, dv, da, db)
+        if sfx:
+            call("rwkv7_statepassing_backward_f32", dev, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db)
+        else:
+            call("rwkv7_statepassing_backward_ex", dev, B, T, H, r, w, k, v, a, b, dy, dsT, s, sa, ds0, dr, dw, dk, dv, da, db, ctx.flags)
         return ds0, dr, dw, dk, dv, da, db
 
 

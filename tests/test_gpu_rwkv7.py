@@ -4,7 +4,7 @@ import torch
 
 from oracle import rwkv7 as O
 from oracle import err_ratio
-from rwkv_cuda_amd import synth, rwkv7_fast_fused as R
+from rwkv_cuda_amd import options, synth, rwkv7_fast_fused as R
 from _gpu_util import DEV, assert_no_worse
 
 pytestmark = pytest.mark.gpu
@@ -28,13 +28,16 @@ def _run(args, splits=1):
     return [y.detach().view(B, T, H, N), S.detach()] + [x.grad for x in t]
 
 
+@pytest.mark.parametrize("algo", ["chunked", "sweeps"])
 @pytest.mark.parametrize("B,T,H", [(2, 32, 2), (1, 64, 3), (3, 16, 1)])
-def test_rwkv7_small(lib, B, T, H):
-    print(f"\nrwkv7 B={B} T={T} H={H}", flush=True)
+def test_rwkv7_small(lib, B, T, H, algo):
+    """Both kernel families: the chunked matrix-core kernels (default) and the step-by-step recurrence."""
+    print(f"\nrwkv7 B={B} T={T} H={H} {algo}", flush=True)
     args = synth.rwkv7_inputs(B, T, H, 64, seed=31)
     ref = O.grads(*args)
     emu = O.emulate_bf16(*args)
-    got = _run(args)
+    with options.algorithm(algo):
+        got = _run(args)
     for name, a, e, g in zip(NAMES, ref, emu, got):
         assert_no_worse(name, a, e, g)
 

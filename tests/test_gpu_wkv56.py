@@ -340,3 +340,50 @@ def test_decay_gradient_where_the_decay_has_vanished(lib, algo):
         for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y] + [x.grad for x in t]):
             assert_no_worse("wkv5 " + name, a, e, g)
         assert float(t[3].grad.float().cpu()[0, 5:12].abs().max()) == 0.0
+
+
+def test_two_threads_run_different_algorithms_concurrently(lib):
+    """The kernel choice is a per-call argument: one thread runs the chunked kernels and another the sequential sweeps
+    at the same time, on two streams, and each gets exactly what it gets when it runs alone."""
+    import threading
+    B, T, H = 2, 200, 2
+    C = H * 64
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=71, state=True)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    d = [x.to(DEV) for x in (r, k, v, w, u, s0, gy)]
+    n = lib.rwkv_wkv6state_backward_workspace_bytes(B, T, C, H)
+
+    def run(flags, stream, reps, out):
+        with torch.cuda.stream(stream):
+            for _ in range(reps):
+                ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+                y, gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(5))
+                gu, gs = garbage((B, C), BF), garbage((B, H, 64, 64), BF)
+                call("rwkv_wkv6state_forward_ex", d[0].device, B, T, C, H, *d[:6], y, flags)
+                call("rwkv_wkv6state_backward_ex", d[0].device, B, T, C, H, *d[:6], d[6], gr, gk, gv, gw, gu, gs, ws, n, flags)
+                out.append([y, gr, gk, gv, gw, gu, gs])
+            stream.synchronize()
+
+    torch.cuda.synchronize()
+    alone = {}
+    for flags in (0, options.FLAG_SWEEPS):
+        res = []
+        run(flags, torch.cuda.Stream(), 1, res)
+        alone[flags] = res[0]
+    results = {0: [], options.FLAG_SWEEPS: []}
+    threads = [threading.Thread(target=run, args=(f, torch.cuda.Stream(), 6, results[f])) for f in results]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    for flags, runs in results.items():
+        assert len(runs) == 6
+        for got in runs:
+            for name, a, b in zip(("y", "gr", "gk", "gv", "gw", "gu", "gs"), alone[flags], got):
+                assert torch.equal(a, b), (flags, name)
+        got = runs[-1]
+        got[5] = got[5].sum(0).view(H, 64)
+        for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, emu, got):
+            assert_no_worse(f"flags {flags:#x} {name}", a, e, g)
