@@ -135,9 +135,11 @@ DEVINL Factors chunk_factors(const float (&lam)[4], const float (*part)[N], int 
         // c_t - c_m and c_{t+1} - c_m
         const float xt = q < 2 ? -(suf[e] + gap) : gap + pre[e];
         const float xn = q < 2 ? -(suf[e + 1] + gap) : gap + pre[e + 1];
-        f.ea[e] = exp_acc(xt);
-        f.er[e] = exp_acc(xn);
-        f.eb[e] = exp_acc(-xn);
+        // the middle-referenced factors always come in pairs whose exponents cancel only partly, so the extra digits of
+        // exp_acc would be lost anyway; the start- and end-referenced ones carry the fp32 states and keep them
+        f.ea[e] = __expf(xt);
+        f.er[e] = __expf(xn);
+        f.eb[e] = __expf(-xn);
         f.es[e] = exp_acc(before + pre[e]);
         f.ee[e] = exp_acc(suf[e + 1] + after);
     }
@@ -154,6 +156,7 @@ struct SmemCF {
     float As[CL][PS];                  // a referred to the start of the chunk: e^{c_t}
     float Yo[CL][PS], Uo[CL][PS];
     float ABt[CL][TS], AK[CL][TS], RB[CL][TS], RK[CL][TS];
+    float M[CL][TS];                   // (I - AB)^{-1}, rows by the wave that made AB
     float part[4][N];
     float d1[N], dec[N];
 };
@@ -234,8 +237,15 @@ __global__ __launch_bounds__(NT, 2) void rwkv7c_fwd(const Args7c p) {
                 const int t = 4 * g + v;
                 acc[v] = (q < 2 ? l16 < t : l16 <= t) ? acc[v] : 0.f;
             }
-            if (q == 0) st4(&S.ABt[l16][4 * g], acc);
-            else {
+            if (q == 0) {
+                st4(&S.ABt[l16][4 * g], acc);
+                // this wave wrote AB itself (LDS keeps a wave's accesses in order): the inverse once, for all four waves
+                float m[CL];
+                inverse_rows(S.ABt, l16, m);
+                if (g == 0)
+#pragma unroll
+                    for (int s4 = 0; s4 < CL; s4 += 4) st4(&S.M[l16][s4], f32x4{m[s4], m[s4 + 1], m[s4 + 2], m[s4 + 3]});
+            } else {
                 float (*Tl)[TS] = q == 1 ? S.AK : (q == 2 ? S.RB : S.RK);
 #pragma unroll
                 for (int v = 0; v < 4; ++v) Tl[4 * g + v][l16] = acc[v];
@@ -259,11 +269,12 @@ __global__ __launch_bounds__(NT, 2) void rwkv7c_fwd(const Args7c p) {
             for (int v = 0; v < 4; ++v) W = mm(ak[v], vop[v], W);
         }
         // ---------------------------------------------------------------- U = (I - AB)^{-1} W
-        float m[CL];
-        inverse_rows(S.ABt, l16, m);
         f32x4 U = ZERO4;
+        {
+            const f32x4 mr = ld4(&S.M[l16][4 * g]);   // M[t = l16][s = 4 g + v]
 #pragma unroll
-        for (int v = 0; v < 4; ++v) U = mm(by_group(g, m[v], m[4 + v], m[8 + v], m[12 + v]), W[v], U);
+            for (int v = 0; v < 4; ++v) U = mm(mr[v], W[v], U);
+        }
         // ---------------------------------------------------------------- Y = R' (d1 S0^T) + RB U + RK V
         f32x4 Sd[4];
 #pragma unroll
@@ -337,18 +348,22 @@ constexpr int NTB = 12 * 64;       // waves 0..3 role A, 4..7 role B, 8..11 role
 // Everything that is a function of one chunk's inputs alone; two copies: the P waves fill one while the A and B waves work on the other.
 struct PlanesB {
     float Ap[CL][PS], Rp[CL][PS], Bp[CL][PS], Kp[CL][PS];   // referred to the middle of the chunk (tiles, dA' .. dK')
-    float As[CL][PS], Rs[CL][PS];                            // a e^{c_t}, r e^{c_{t+1}}: the state-gradient update     (later: da, dr)
-    float Bd[CL][PS], Kd[CL][PS];                            // b, k times e^{c_L - c_{s+1}}: dU, dV, S_T               (later: db, dv)
-    float V[CL][PS], dY[CL][PS], U[CL][PS];                  //                                                          (U later: dw)
+    float As[CL][PS], Rs[CL][PS];                            // a e^{c_t}, r e^{c_{t+1}}: the state-gradient update
+    float Bd[CL][PS], Kd[CL][PS];                            // b, k times e^{c_L - c_{s+1}}: dU, dV, S_T
+    float V[CL][PS], dY[CL][PS], U[CL][PS];
     float EA[CL][PS], ER[CL][PS], DWF[CL][PS];               // e^{c_t - c_m}, e^{c_{t+1} - c_m}, W_SCALE sig (1 - sig)
     float part[4][N];
     float d1[N], d2[N], dec[N];
 };
+constexpr int PK = 72;            // row stride (bf16 elements) of a parked output
 struct SmemCB {
     PlanesB pl[2];
-    float dW[CL][PS];                                        //                                                          (later: dk)
+    float dW[CL][PS];
+    float M[CL][TS];                                         // (I - AB)^{-1}
     float AB[CL][TS], AK[CL][TS], RB[CL][TS], RK[CL][TS];
     float dAB[CL][TS], dAK[CL][TS], dRB[CL][TS], dRK[CL][TS];
+    uint16_t park[5][CL][PK];                                // da, dr, db, dk, dw of the chunk whose phase 4 ran last, [token][channel]
+    uint16_t parkv[2][CL][PK];                               // dv, which is ready one visit earlier than the other five
 };
 
 // tile[t][s] = sum_c X[t][c] Y[s][c] over 64 channels, masked to s < t (strict) or s <= t, stored as [t][s]
@@ -368,93 +383,111 @@ DEVINL void causal_tile(const float (*X)[PS], const float (*Y)[PS], float (*Tl)[
     }
 }
 
-// Per visit (chunks in descending order) every wave passes the same four barriers:
-//   A, B:  phase 1 | B | phase 2 | B | phase 3 | B | phase 4 | B
-//   P:     row stores of the previous visit, raw inputs -> decay sums | B | factors, planes of the NEXT visit | B | - | B | - | B
+// Per visit i (chunks in descending order) every wave passes three barriers; role B trails role A by one phase, so that
+// both always have matrix work in the same phase:
+//          phase 1                          | phase 2                                   | phase 3
+//   A:     tile, M, tile-free parts of (i)   | dU, dW, dV, state update of (i)           | dAB, dAK of (i)
+//   B:     tile parts + epilogue of (i - 1)  | dY S0, U dS, V dS, dRB, dRK of (i)        | dW S0, state update of (i)
+//   P:     raw inputs -> decay sums (i + 1)  | row stores (i - 1); factors, planes (i+1) | -
 
 // ---- role P: elementwise preparation (lane = channel, tokens 4 wp + e) one visit ahead, and the row-wise output stores
 struct Prep7 { uint32_t nx[7][4]; float nsa[4]; };
+struct Conv7 { float sg[4], uu[4]; uint32_t pk[6][2]; };      // sigmoid(w), sa, and r k v a b dy as bf16 pairs (tokens 2 z, 2 z + 1)
 DEVINL void bwd_fetch(const Args7c& p, Prep7& x, size_t row0, int wp, int lane, int H, int h) {
     // wave-uniform base (scalar registers) plus a 32-bit lane offset: no 64-bit address per tensor and token in vector registers
+    // (the lane part is hidden from the optimiser: it would otherwise turn every tensor-and-token address into a 64-bit
+    // induction variable of the chunk loop, 64 vector registers)
     const size_t base = (row0 * H + h) * N;
+    uint32_t lo = lane;
+    asm volatile("" : "+v"(lo));
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        const uint32_t o = static_cast<uint32_t>((4 * wp + e) * H) * N + lane;
+        const uint32_t o = static_cast<uint32_t>((4 * wp + e) * H) * N + lo;
         x.nx[0][e] = (p.w + base)[o]; x.nx[1][e] = (p.r + base)[o]; x.nx[2][e] = (p.k + base)[o]; x.nx[3][e] = (p.v + base)[o];
         x.nx[4][e] = (p.a + base)[o]; x.nx[5][e] = (p.b + base)[o]; x.nx[6][e] = (p.dy + base)[o];
         x.nsa[e] = (p.sa + base)[o];
     }
 }
-// first half: up to the barrier that publishes the decay sums; second half: the planes
-DEVINL void bwd_prep(PlanesB& O, const Args7c& p, Prep7& x, bool more, size_t next_row0, int wp, int lane, int H, int h) {
-    float lam[4], sg[4], rr[4], kk[4], vv[4], aa[4], bb[4], gg[4], uu[4];
+// first half of the preparation: the decay of each token, this wave's decay sum; the other inputs are kept packed so that the
+// registers of x are free for the next fetch
+DEVINL void bwd_convert(PlanesB& O, const Prep7& x, Conv7& y, int wp, int lane) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        sg[e] = sigmoid_fast(bf2f(x.nx[0][e]));
-        lam[e] = W_SCALE * sg[e];
-        rr[e] = bf2f(x.nx[1][e]); kk[e] = bf2f(x.nx[2][e]); vv[e] = bf2f(x.nx[3][e]); aa[e] = bf2f(x.nx[4][e]); bb[e] = bf2f(x.nx[5][e]);
-        gg[e] = bf2f(x.nx[6][e]); uu[e] = x.nsa[e];
-    }
-    O.part[wp][lane] = (lam[0] + lam[1]) + (lam[2] + lam[3]);
-    if (more) bwd_fetch(p, x, next_row0, wp, lane, H, h);
-    __syncthreads();
+    for (int e = 0; e < 4; ++e) { y.sg[e] = sigmoid_fast(bf2f(x.nx[0][e])); y.uu[e] = x.nsa[e]; }
+#pragma unroll
+    for (int k = 0; k < 6; ++k)
+#pragma unroll
+        for (int z = 0; z < 2; ++z) y.pk[k][z] = x.nx[k + 1][2 * z] | (x.nx[k + 1][2 * z + 1] << 16);
+    O.part[wp][lane] = W_SCALE * ((y.sg[0] + y.sg[1]) + (y.sg[2] + y.sg[3]));
+}
+// second half (after a barrier): the in-chunk factors and every plane
+DEVINL void bwd_planes(PlanesB& O, const Conv7& y, int wp, int lane) {
     float cm, cl;
+    const float lam[4] = {W_SCALE * y.sg[0], W_SCALE * y.sg[1], W_SCALE * y.sg[2], W_SCALE * y.sg[3]};
     const Factors f = chunk_factors(lam, O.part, wp, lane, cm, cl);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const int t = 4 * wp + e;
-        O.Ap[t][lane] = aa[e] * f.ea[e];
-        O.Rp[t][lane] = rr[e] * f.er[e];
-        O.Bp[t][lane] = bb[e] * f.eb[e];
-        O.Kp[t][lane] = kk[e] * f.eb[e];
-        O.As[t][lane] = aa[e] * f.es[e];
-        O.Rs[t][lane] = rr[e] * (f.es[e] * __expf(lam[e]));
-        O.Bd[t][lane] = bb[e] * f.ee[e];
-        O.Kd[t][lane] = kk[e] * f.ee[e];
-        O.V[t][lane] = vv[e];
-        O.dY[t][lane] = gg[e];
-        O.U[t][lane] = uu[e];
+        auto in = [&](int k) __attribute__((always_inline)) { return (e & 1) ? bf_hi(y.pk[k][e >> 1]) : bf_lo(y.pk[k][e >> 1]); };
+        const float rr = in(0), kk = in(1), vv = in(2), aa = in(3), bb = in(4), gg = in(5);
+        O.Ap[t][lane] = aa * f.ea[e];
+        O.Rp[t][lane] = rr * f.er[e];
+        O.Bp[t][lane] = bb * f.eb[e];
+        O.Kp[t][lane] = kk * f.eb[e];
+        O.As[t][lane] = aa * f.es[e];
+        O.Rs[t][lane] = rr * (f.es[e] * __expf(lam[e]));
+        O.Bd[t][lane] = bb * f.ee[e];
+        O.Kd[t][lane] = kk * f.ee[e];
+        O.V[t][lane] = vv;
+        O.dY[t][lane] = gg;
+        O.U[t][lane] = y.uu[e];
         O.EA[t][lane] = f.ea[e];
         O.ER[t][lane] = f.er[e];
-        O.DWF[t][lane] = W_SCALE * sg[e] * (1.f - sg[e]);
+        O.DWF[t][lane] = W_SCALE * y.sg[e] * (1.f - y.sg[e]);
     }
     if (wp == 0) { O.d1[lane] = exp_acc(cm); O.d2[lane] = exp_acc(cl - cm); O.dec[lane] = exp_acc(cl); }
-    __syncthreads();
 }
-// da dr db dk dv dw of one chunk leave the planes they were parked in as whole rows (256 threads, four channels each)
-DEVINL void bwd_store_rows(const SmemCB& S, const PlanesB& O, const Args7c& p, size_t row0, int tp, int H, int h) {
+// da dr db dk dw (and dv) of one chunk leave their parking places as whole rows (256 threads, four channels each)
+DEVINL void bwd_store_rows(const SmemCB& S, int vbuf, const Args7c& p, size_t row0, int tp, int H, int h) {
     const int t = tp >> 4, c4 = (tp & 15) * 4;
     const size_t base = (row0 * H + h) * N;
-    const uint32_t o = static_cast<uint32_t>(t * H) * N + c4;
-    auto put = [&](uint16_t* dst, const float* src) __attribute__((always_inline)) {
-        const f32x4 x = ld4(src);
-        *reinterpret_cast<uint2*>(dst + base + o) = make_uint2(pack_bf2(x[0], x[1]), pack_bf2(x[2], x[3]));
+    uint32_t o = static_cast<uint32_t>(t * H) * N + c4;
+    asm volatile("" : "+v"(o));
+    auto put = [&](uint16_t* dst, const uint16_t* src) __attribute__((always_inline)) {
+        *reinterpret_cast<uint2*>(dst + base + o) = *reinterpret_cast<const uint2*>(src);
     };
-    put(p.da, &O.As[t][c4]); put(p.dr, &O.Rs[t][c4]); put(p.db, &O.Bd[t][c4]); put(p.dk, &S.dW[t][c4]);
-    put(p.dv, &O.Kd[t][c4]); put(p.dw, &O.U[t][c4]);
+    put(p.da, &S.park[0][t][c4]); put(p.dr, &S.park[1][t][c4]); put(p.db, &S.park[2][t][c4]); put(p.dk, &S.park[3][t][c4]);
+    put(p.dw, &S.park[4][t][c4]); put(p.dv, &S.parkv[vbuf][t][c4]);
 }
 DEVINL void bwd_role_p(SmemCB& S, const Args7c& p, int tid, int w, size_t tok0, int nch, int H, int h) {
     const int lane = tid & 63, wp = w - 8, tp = tid - 8 * 64;
     Prep7 x;
+    Conv7 y;
     bwd_fetch(p, x, tok0 + static_cast<size_t>(nch - 1) * CL, wp, lane, H, h);
-    bwd_prep(S.pl[0], p, x, nch > 1, tok0 + static_cast<size_t>(nch > 1 ? nch - 2 : 0) * CL, wp, lane, H, h);      // visit 0, before the loop
+    bwd_convert(S.pl[0], x, y, wp, lane);            // visit 0, before the loop
+    if (nch > 1) bwd_fetch(p, x, tok0 + static_cast<size_t>(nch - 2) * CL, wp, lane, H, h);
+    __syncthreads();
+    bwd_planes(S.pl[0], y, wp, lane);
+    __syncthreads();
     STAMP_INIT;
-    for (int i = 0; i < nch; ++i) {                  // during visit i (chunk nch - 1 - i): store visit i - 1, prepare visit i + 1
-        if (i > 0) bwd_store_rows(S, S.pl[(i - 1) & 1], p, tok0 + static_cast<size_t>(nch - i) * CL, tp, H, h);
-        if (i + 1 < nch) {
-            const int cn = nch - 2 - i;              // chunk of visit i + 1
-            bwd_prep(S.pl[(i + 1) & 1], p, x, cn > 0, tok0 + static_cast<size_t>(cn > 0 ? cn - 1 : 0) * CL, wp, lane, H, h);
-        } else {
-            __syncthreads();
-            __syncthreads();
+    for (int i = 0; i < nch; ++i) {                  // visit i is chunk nch - 1 - i
+        const bool next = i + 1 < nch;
+        if (next) {
+            bwd_convert(S.pl[(i + 1) & 1], x, y, wp, lane);
+            if (i + 2 < nch) bwd_fetch(p, x, tok0 + static_cast<size_t>(nch - 3 - i) * CL, wp, lane, H, h);
         }
         STAMP(0);
         __syncthreads();
-        __syncthreads();
         STAMP(1);
+        if (i > 0) bwd_store_rows(S, (i - 1) & 1, p, tok0 + static_cast<size_t>(nch - i) * CL, tp, H, h);
+        if (next) bwd_planes(S.pl[(i + 1) & 1], y, wp, lane);
+        STAMP(2);
+        __syncthreads();
+        __syncthreads();
+        STAMP(3);
     }
     STAMP_DUMP(w);
-    bwd_store_rows(S, S.pl[(nch - 1) & 1], p, tok0, tp, H, h);
+    __syncthreads();                                 // role B finishes the last chunk
+    bwd_store_rows(S, (nch - 1) & 1, p, tok0, tp, H, h);
 }
 
 DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, int nch) {
@@ -469,10 +502,8 @@ DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
     STAMP_INIT;
     for (int i = 0; i < nch; ++i) {
         const PlanesB& O = S.pl[i & 1];
-        PlanesB& Ow = S.pl[i & 1];
-        // ---------------------------------------------------------------- phase 1: a causal tile; the parts of dU, dV, dS that need no tile
-        causal_tile(q < 2 ? O.Ap : O.Rp, (q & 1) ? O.Kp : O.Bp, q == 0 ? S.AB : (q == 1 ? S.AK : (q == 2 ? S.RB : S.RK)), q < 2, l16, g);
-        // (a chain of dependent matrix instructions runs at half the rate of independent ones: partial sums per 16 key channels)
+        // ---------------------------------------------------------------- phase 1: the parts of dU, dV, dS that need no tile; a causal tile; M
+        // (a chain of dependent matrix instructions runs slower than independent ones: two partial sums each)
         f32x4 dyop, dUp[2] = {ZERO4, ZERO4}, dVp[2] = {ZERO4, ZERO4}, accA[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) dyop[v] = O.dY[4 * g + v][own];           // dY[tau = 4 g + v][i]
@@ -488,19 +519,25 @@ DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
             }
             accA[jt] = acc;
         }
+        causal_tile(q < 2 ? O.Ap : O.Rp, (q & 1) ? O.Kp : O.Bp, q == 0 ? S.AB : (q == 1 ? S.AK : (q == 2 ? S.RB : S.RK)), q < 2, l16, g);
+        if (q == 0) {                                // this wave wrote AB itself: LDS keeps a wave's accesses in order
+            float m[CL];
+            inverse_cols(S.AB, l16, m);
+            if (g == 0)
+#pragma unroll
+                for (int t = 0; t < CL; ++t) S.M[t][l16] = m[t];
+        }
         f32x4 dU = dUp[0] + dUp[1], dV = dVp[0] + dVp[1];
         STAMP(0);
         __syncthreads();
         STAMP(1);
-        // ---------------------------------------------------------------- phase 2: dU, the solve, dW, dV, the gradient state
+        // ---------------------------------------------------------------- phase 2: dU, dW = M^T dU, dV, the gradient state
         {
 #pragma unroll
             for (int v = 0; v < 4; ++v) dU = mm(S.RB[4 * g + v][l16], dyop[v], dU);
-            float m[CL];
-            inverse_cols(S.AB, l16, m);
             f32x4 dW = ZERO4;
 #pragma unroll
-            for (int v = 0; v < 4; ++v) dW = mm(by_group(g, m[v], m[4 + v], m[8 + v], m[12 + v]), dU[v], dW);
+            for (int v = 0; v < 4; ++v) dW = mm(S.M[4 * g + v][l16], dU[v], dW);
 #pragma unroll
             for (int v = 0; v < 4; ++v) S.dW[4 * g + v][own] = dW[v];
 #pragma unroll
@@ -508,7 +545,7 @@ DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
 #pragma unroll
             for (int v = 0; v < 4; ++v) dV = mm(S.RK[4 * g + v][l16], dyop[v], dV);
 #pragma unroll
-            for (int v = 0; v < 4; ++v) Ow.Kd[4 * g + v][own] = dV[v];           // Kd is dead: dv waits here for the row stores
+            for (int v = 0; v < 4; ++v) S.parkv[i & 1][4 * g + v][own] = f2bf(dV[v]);
 #pragma unroll
             for (int jt = 0; jt < 4; ++jt) {
                 f32x4 acc = accA[jt];
@@ -524,10 +561,10 @@ DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
         if (q < 2) causal_tile(S.dW, q == 0 ? O.U : O.V, q == 0 ? S.dAB : S.dAK, true, l16, g);
         STAMP(4);
         __syncthreads();
-        __syncthreads();
         STAMP(5);
     }
     STAMP_DUMP(w);
+    __syncthreads();
     if (p.ds0 != nullptr) {
         float* dst = p.ds0 + bh * N * N + static_cast<size_t>(own) * N + 4 * g;
 #pragma unroll
@@ -546,13 +583,61 @@ DEVINL void bwd_role_b(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
             dS[ib][v] = p.dsT != nullptr ? p.dsT[bh * N * N + static_cast<size_t>(16 * ib + 4 * g + v) * N + own] : 0.f;
     auto fetch_state = [&](int c) __attribute__((always_inline)) {
         const float* slot = p.s + (bh * nch + c) * N * N;
-        const uint32_t o = static_cast<uint32_t>(4 * g) * N + own;
+        uint32_t o = static_cast<uint32_t>(4 * g) * N + own;
+        asm volatile("" : "+v"(o));
 #pragma unroll
         for (int ib = 0; ib < 4; ++ib)
 #pragma unroll
             for (int v = 0; v < 4; ++v) S0b[ib][v] = slot[o + (16 * ib + v) * N];
     };
-    float Pj = 0.f;                                  // P at the end of the chunk being visited
+    float Pj = 0.f;                                  // P at the end of the chunk whose phase 4 comes next
+    f32x4 xA = ZERO4, xR = ZERO4, xB = ZERO4, xK = ZERO4;     // state parts of dA', dR', dB', dK', carried into the next visit's phase 1
+    // tile parts, scaling, decay gradient of the chunk whose planes are O; results parked as bf16
+    auto finish = [&](const PlanesB& O) __attribute__((always_inline)) {
+        const float d1j = O.d1[own], d2j = O.d2[own];
+        f32x4 bp, kp, ap, rp;                        // planes at [s or t = 4 g + v][j]
+#pragma unroll
+        for (int v = 0; v < 4; ++v) { bp[v] = O.Bp[4 * g + v][own]; kp[v] = O.Kp[4 * g + v][own]; ap[v] = O.Ap[4 * g + v][own]; rp[v] = O.Rp[4 * g + v][own]; }
+        f32x4 tA = ZERO4, tR = ZERO4, tB = ZERO4, tK = ZERO4;
+        const f32x4 dab = ld4(&S.dAB[l16][4 * g]), dak = ld4(&S.dAK[l16][4 * g]), drb = ld4(&S.dRB[l16][4 * g]), drk = ld4(&S.dRK[l16][4 * g]);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            tA = mm(dab[v], bp[v], tA); tR = mm(drb[v], bp[v], tR);
+            tB = mm(S.dAB[4 * g + v][l16], ap[v], tB); tK = mm(S.dAK[4 * g + v][l16], ap[v], tK);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            tA = mm(dak[v], kp[v], tA); tR = mm(drk[v], kp[v], tR);
+            tB = mm(S.dRB[4 * g + v][l16], rp[v], tB); tK = mm(S.dRK[4 * g + v][l16], rp[v], tK);
+        }
+        float del[4], ada[4], dwf[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int t = 4 * g + v;
+            const float dAp = fmaf(d1j, xA[v], tA[v]), dRp = fmaf(d1j, xR[v], tR[v]);
+            const float dBp = fmaf(d2j, xB[v], tB[v]), dKp = fmaf(d2j, xK[v], tK[v]);
+            const float ea = O.EA[t][own], er = O.ER[t][own];
+            const float eb = __frcp_rn(er);
+            S.park[0][t][own] = f2bf(dAp * ea);
+            S.park[1][t][own] = f2bf(dRp * er);
+            S.park[2][t][own] = f2bf(dBp * eb);
+            S.park[3][t][own] = f2bf(dKp * eb);
+            ada[v] = ap[v] * dAp;
+            del[v] = fmaf(rp[v], dRp, -fmaf(bp[v], dBp, kp[v] * dKp));      // r dr - b db - k dk
+            dwf[v] = O.DWF[t][own];
+        }
+        // G_t = P_{t+1} + del_t,  P_t = G_t + a da:  suffix sums over t = 4 g + v, later lane groups first
+        const float tot = (del[0] + ada[0]) + (del[1] + ada[1]) + (del[2] + ada[2]) + (del[3] + ada[3]);
+        const float t1 = __shfl_down(tot, 16, 64), t2 = __shfl_down(tot, 32, 64), t3 = __shfl_down(tot, 48, 64);
+        float Pn = Pj + (g < 3 ? t1 : 0.f) + (g < 2 ? t2 : 0.f) + (g < 1 ? t3 : 0.f);     // P after this lane's last token
+#pragma unroll
+        for (int v = 3; v >= 0; --v) {
+            const float G = Pn + del[v];
+            Pn = G + ada[v];
+            S.park[4][4 * g + v][own] = f2bf(G * dwf[v]);
+        }
+        Pj = __shfl(Pn, l16, 64);                    // lane group 0 holds P at the start of the chunk
+    };
     fetch_state(nch - 1);
     __syncthreads();
     __syncthreads();
@@ -560,8 +645,12 @@ DEVINL void bwd_role_b(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
     for (int i = 0; i < nch; ++i) {
         const int c = nch - 1 - i;
         const PlanesB& O = S.pl[i & 1];
-        PlanesB& Ow = S.pl[i & 1];
-        // ---------------------------------------------------------------- phase 1: dY S0, U dS, V dS; dRB, dRK
+        // ---------------------------------------------------------------- phase 1: finish the previous visit's chunk
+        if (i > 0) finish(S.pl[(i - 1) & 1]);
+        STAMP(0);
+        __syncthreads();
+        STAMP(1);
+        // ---------------------------------------------------------------- phase 2: dY S0, U dS, V dS; dRB, dRK
         if (i == 0 && p.dsT != nullptr) {
             // P at the end of the call: sum_i dsT o S_T with S_T = S0 dec + U^T (B' d2) + V^T (K' d2) of the last chunk
             const float decj = O.dec[own];
@@ -580,7 +669,6 @@ DEVINL void bwd_role_b(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
             pp += __shfl_xor(pp, 32, 64);
             Pj = pp;
         }
-        f32x4 xA, xR, xB, xK;
         {
             f32x4 pr[2] = {ZERO4, ZERO4}, pb[2] = {ZERO4, ZERO4}, pk[2] = {ZERO4, ZERO4};   // two partial sums each: independent chains
 #pragma unroll
@@ -596,10 +684,9 @@ DEVINL void bwd_role_b(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
             xR = pr[0] + pr[1]; xB = pb[0] + pb[1]; xK = pk[0] + pk[1];
         }
         if (q >= 2) causal_tile(O.dY, q == 2 ? O.U : O.V, q == 2 ? S.dRB : S.dRK, false, l16, g);
-        STAMP(0);
+        STAMP(2);
         __syncthreads();
-        __syncthreads();
-        STAMP(1);
+        STAMP(3);
         // ---------------------------------------------------------------- phase 3: dW S0; the gradient state
         {
             const float decj = O.dec[own];
@@ -622,61 +709,13 @@ DEVINL void bwd_role_b(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
             xA = pa[0] + pa[1];
             if (c > 0) fetch_state(c - 1);
         }
-        STAMP(2);
-        __syncthreads();
-        STAMP(3);
-        // ---------------------------------------------------------------- phase 4: tile parts, scaling, decay gradient
-        {
-            const float d1j = O.d1[own], d2j = O.d2[own];
-            f32x4 bp, kp, ap, rp;                    // planes at [s or t = 4 g + v][j]
-#pragma unroll
-            for (int v = 0; v < 4; ++v) { bp[v] = O.Bp[4 * g + v][own]; kp[v] = O.Kp[4 * g + v][own]; ap[v] = O.Ap[4 * g + v][own]; rp[v] = O.Rp[4 * g + v][own]; }
-            f32x4 tA = ZERO4, tR = ZERO4, tB = ZERO4, tK = ZERO4;
-            const f32x4 dab = ld4(&S.dAB[l16][4 * g]), dak = ld4(&S.dAK[l16][4 * g]), drb = ld4(&S.dRB[l16][4 * g]), drk = ld4(&S.dRK[l16][4 * g]);
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                tA = mm(dab[v], bp[v], tA); tR = mm(drb[v], bp[v], tR);
-                tB = mm(S.dAB[4 * g + v][l16], ap[v], tB); tK = mm(S.dAK[4 * g + v][l16], ap[v], tK);
-            }
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                tA = mm(dak[v], kp[v], tA); tR = mm(drk[v], kp[v], tR);
-                tB = mm(S.dRB[4 * g + v][l16], rp[v], tB); tK = mm(S.dRK[4 * g + v][l16], rp[v], tK);
-            }
-            float del[4], ada[4], dwf[4];
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int t = 4 * g + v;
-                const float dAp = fmaf(d1j, xA[v], tA[v]), dRp = fmaf(d1j, xR[v], tR[v]);
-                const float dBp = fmaf(d2j, xB[v], tB[v]), dKp = fmaf(d2j, xK[v], tK[v]);
-                const float ea = O.EA[t][own], er = O.ER[t][own];
-                const float eb = __frcp_rn(er);
-                // outputs are parked in planes that are dead by now; the P waves store them as whole rows during the next visit
-                Ow.As[t][own] = dAp * ea;
-                Ow.Rs[t][own] = dRp * er;
-                Ow.Bd[t][own] = dBp * eb;
-                S.dW[t][own] = dKp * eb;
-                ada[v] = ap[v] * dAp;
-                del[v] = fmaf(rp[v], dRp, -fmaf(bp[v], dBp, kp[v] * dKp));      // r dr - b db - k dk
-                dwf[v] = O.DWF[t][own];
-            }
-            // G_t = P_{t+1} + del_t,  P_t = G_t + a da:  suffix sums over t = 4 g + v, later lane groups first
-            const float tot = (del[0] + ada[0]) + (del[1] + ada[1]) + (del[2] + ada[2]) + (del[3] + ada[3]);
-            const float t1 = __shfl_down(tot, 16, 64), t2 = __shfl_down(tot, 32, 64), t3 = __shfl_down(tot, 48, 64);
-            float Pn = Pj + (g < 3 ? t1 : 0.f) + (g < 2 ? t2 : 0.f) + (g < 1 ? t3 : 0.f);     // P after this lane's last token
-#pragma unroll
-            for (int v = 3; v >= 0; --v) {
-                const float G = Pn + del[v];
-                Pn = G + ada[v];
-                Ow.U[4 * g + v][own] = G * dwf[v];
-            }
-            Pj = __shfl(Pn, l16, 64);                // lane group 0 holds P at the start of the chunk
-        }
         STAMP(4);
         __syncthreads();
         STAMP(5);
     }
     STAMP_DUMP(w);
+    finish(S.pl[(nch - 1) & 1]);
+    __syncthreads();
 }
 
 __global__ __launch_bounds__(NTB, 3) void rwkv7c_bwd(const Args7c p) {
