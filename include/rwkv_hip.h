@@ -91,6 +91,18 @@ int rwkv_wkv4_backward_noalloc(void* stream, int B, int T, int C,
                                const float* w, const float* u, const float* k, const float* v, const float* gy,
                                float* gw, float* gu, float* gk, float* gv);
 
+/* The whole of WKV.forward / WKV.backward (wkv/run.py:89-117) behind two calls: w_raw[C] is the raw parameter (the kernels
+ * apply w = -exp(w_raw), :95), and gw, gu [C] come out summed over the batch (:115-116; no zero-fill by the caller).  The
+ * backward launches the sweep kernel and one small reduction kernel; the order of every sum is fixed.  Workspace: the
+ * B*T*C floats of rwkv_wkv4_backward plus 2*B*C floats of per-batch partials. */
+int rwkv_wkv4raw_forward(void* stream, int B, int T, int C,
+                         const float* w_raw, const float* u, const float* k, const float* v, float* y);
+size_t rwkv_wkv4raw_backward_workspace_bytes(int B, int T, int C);
+int rwkv_wkv4raw_backward(void* stream, int B, int T, int C,
+                          const float* w_raw, const float* u, const float* k, const float* v, const float* gy,
+                          float* gw, float* gu, float* gk, float* gv,
+                          void* workspace, size_t workspace_bytes);
+
 /* ---------------------------------------------------------------------------------------
  * depthwise_conv1d ("TimeX"), fp32.  Replaces cuda_forward / cuda_backward of
  * depthwise_conv1d/cuda/timex_op.cpp:3-4 (kernels: timex_cuda_v3.cu:7-150).
@@ -132,6 +144,20 @@ int rwkv_wkv5_backward_ex(void* stream, int B, int T, int C, int H,
                        const float* eew, const float* ew, const rwkv_bf16* u, const rwkv_bf16* gy,
                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                        void* workspace, size_t workspace_bytes, unsigned flags);
+
+/* WKV_5.forward / backward (wkv5_bf16/run.py:44-88) with the wrapper's steps folded in.  w_raw[H,N] is the raw bf16
+ * parameter; the forward writes decay[2*C] fp32 = [exp(-exp(w_raw)) | -exp(w_raw)] (:63-64), which the caller keeps for the
+ * backward; gw, gu [H,N] bf16 come out summed over the batch exactly as torch.sum over the bf16 per-batch partials gives
+ * them (:86-87).  `flags` as for the *_ex entry points. */
+int rwkv_wkv5raw_forward(void* stream, int B, int T, int C, int H,
+                         const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                         const rwkv_bf16* w_raw, const rwkv_bf16* u, rwkv_bf16* y, float* decay, unsigned flags);
+size_t rwkv_wkv5raw_backward_workspace_bytes(int B, int T, int C, int H);
+int rwkv_wkv5raw_backward(void* stream, int B, int T, int C, int H,
+                          const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                          const float* decay, const rwkv_bf16* u, const rwkv_bf16* gy,
+                          rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                          void* workspace, size_t workspace_bytes, unsigned flags);
 
 /* ---------------------------------------------------------------------------------------
  * RWKV-5 wkv, fp32 I/O.  Replaces cuda_forward / cuda_backward of wkv5/cuda/wkv5_op.cpp:3-4
@@ -221,6 +247,16 @@ int rwkv_wkv6raw_backward_ex(void* stream, int B, int T, int C, int H,
                           const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* gy,
                           rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                           void* workspace, size_t workspace_bytes, unsigned flags);
+
+/* The backward of WKV_6 (s = gs = NULL) and WKV_6STATE with the wrapper's torch.sum(gu, 0) (wkv6/run.py:169,
+ * wkv6_state/run.py:123) folded in: raw bf16 w, gu[H,N] summed over the batch as torch.sum over the bf16 per-batch
+ * partials gives it.  The forward is rwkv_wkv6raw_forward / rwkv_wkv6state_forward.  `flags` as for the *_ex entry points. */
+size_t rwkv_wkv6f_backward_workspace_bytes(int B, int T, int C, int H);
+int rwkv_wkv6f_backward(void* stream, int B, int T, int C, int H,
+                        const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                        const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, const rwkv_bf16* gy,
+                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                        rwkv_bf16* gs, void* workspace, size_t workspace_bytes, unsigned flags);
 
 /* ---------------------------------------------------------------------------------------
  * RWKV-6 wkv with initial state.  Replaces cuda_forward / cuda_backward of

@@ -93,6 +93,9 @@ SIGNATURES = {
     "rwkv_wkv4_forward": (_I, [_P, _I, _I, _I] + [_P] * 5),
     "rwkv_wkv4_backward_workspace_bytes": (_Z, [_I, _I, _I]),
     "rwkv_wkv4_backward": (_I, [_P, _I, _I, _I] + [_P] * 9 + [_P, _Z]),
+    "rwkv_wkv4raw_forward": (_I, [_P, _I, _I, _I] + [_P] * 5),
+    "rwkv_wkv4raw_backward_workspace_bytes": (_Z, [_I, _I, _I]),
+    "rwkv_wkv4raw_backward": (_I, [_P, _I, _I, _I] + [_P] * 9 + [_P, _Z]),
     "rwkv_wkv4_backward_noalloc_max_elems": (_Z, []),
     "rwkv_wkv4_backward_noalloc": (_I, [_P, _I, _I, _I] + [_P] * 9),
     "rwkv_timex_forward": (_I, [_P, _P, _P, _P, _F, _I, _I, _I]),
@@ -103,6 +106,11 @@ SIGNATURES = {
     "rwkv_wkv5_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv5_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_P, _Z]),
     "rwkv_wkv5_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_P, _Z] + [_U]),
+    "rwkv_wkv5raw_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 7 + [_U]),
+    "rwkv_wkv5raw_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "rwkv_wkv5raw_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z, _U]),
+    "rwkv_wkv6f_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "rwkv_wkv6f_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, _Z, _U]),
     "rwkv_wkv5f32_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
     "rwkv_wkv5f32_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12),
     "rwkv_wkv5f32_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_U]),

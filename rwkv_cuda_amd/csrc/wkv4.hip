@@ -21,6 +21,7 @@ namespace {
 constexpr int NT = 64;
 constexpr float O_INIT = -65500.0f;
 
+template <bool RAW>
 __global__ __launch_bounds__(NT) void wkv4_fwd(int BC, int T, int C, const float* __restrict__ w_,
                                               const float* __restrict__ u_, const float* __restrict__ k_,
                                               const float* __restrict__ v_, float* __restrict__ y_) {
@@ -28,7 +29,7 @@ __global__ __launch_bounds__(NT) void wkv4_fwd(int BC, int T, int C, const float
     if (idx >= BC) return;
     const int b = idx / C, c = idx % C;
     const size_t off = static_cast<size_t>(b) * T * C + c;
-    const float u = u_[c], w = w_[c];
+    const float u = u_[c], w = RAW ? -expf(w_[c]) : w_[c];           // RAW: the wrapper's w = -exp(w_raw) done here
     const float* __restrict__ k = k_ + off;
     const float* __restrict__ v = v_ + off;
     float* __restrict__ y = y_ + off;
@@ -68,6 +69,7 @@ DEVINL State3 combine(const State3 a, const State3 b) {
     return {ea * a.p + eb * b.p, ea * a.q + eb * b.q, no};
 }
 
+template <bool RAW>
 __global__ __launch_bounds__(NTS) void wkv4_fwd_seg(int T, int C, int S, const float* __restrict__ w_,
                                                    const float* __restrict__ u_, const float* __restrict__ k_,
                                                    const float* __restrict__ v_, float* __restrict__ y_) {
@@ -77,7 +79,7 @@ __global__ __launch_bounds__(NTS) void wkv4_fwd_seg(int T, int C, int S, const f
     const bool live = c < C;
     const int cc = live ? c : C - 1;
     const size_t off = static_cast<size_t>(b) * T * C + cc;
-    const float u = u_[cc], w = w_[cc];
+    const float u = u_[cc], w = RAW ? -expf(w_[cc]) : w_[cc];        // RAW: the wrapper's w = -exp(w_raw) done here
     const float* __restrict__ k = k_ + off;
     const float* __restrict__ v = v_ + off;
     float* __restrict__ y = y_ + off;
@@ -128,6 +130,7 @@ __global__ __launch_bounds__(NTS) void wkv4_fwd_seg(int T, int C, int S, const f
     }
 }
 
+template <bool RAW>
 __global__ __launch_bounds__(NT) void wkv4_bwd(int BC, int T, int C, const float* __restrict__ w_,
                                               const float* __restrict__ u_, const float* __restrict__ k_,
                                               const float* __restrict__ v_, const float* __restrict__ gy_,
@@ -138,7 +141,7 @@ __global__ __launch_bounds__(NT) void wkv4_bwd(int BC, int T, int C, const float
     if (idx >= BC) return;
     const int b = idx / C, c = idx % C;
     const size_t off = static_cast<size_t>(b) * T * C + c;
-    const float u = u_[c], w = w_[c];
+    const float u = u_[c], w = RAW ? -expf(w_[c]) : w_[c];           // RAW: the wrapper's w = -exp(w_raw) done here
     const float* __restrict__ k = k_ + off;
     const float* __restrict__ v = v_ + off;
     const float* __restrict__ gy = gy_ + off;
@@ -189,8 +192,13 @@ __global__ __launch_bounds__(NT) void wkv4_bwd(int BC, int T, int C, const float
         o = no;
     }
     // the caller's buffers are accumulated into, as the reference does (wkv_cuda_v2.cu:112-113)
-    gw_[static_cast<size_t>(b) * C + c] += gw * w;
-    gu_[static_cast<size_t>(b) * C + c] += gu;
+    if constexpr (RAW) {                            // per-batch partials in the library's own scratch: plain stores
+        gw_[static_cast<size_t>(b) * C + c] = gw * w;
+        gu_[static_cast<size_t>(b) * C + c] = gu;
+    } else {
+        gw_[static_cast<size_t>(b) * C + c] += gw * w;
+        gu_[static_cast<size_t>(b) * C + c] += gu;
+    }
 }
 
 // Backward in the same time-parallel form.  The ascending sweep also carries dp/dw and dq/dw; a state that is n steps
@@ -205,6 +213,7 @@ DEVINL State5 combine(const State5 a, const State5 b) {
     return {ea * a.p + eb * b.p, ea * a.q + eb * b.q, ea * a.dp + eb * b.dp, ea * a.dq + eb * b.dq, no};
 }
 
+template <bool RAW>
 __global__ __launch_bounds__(NTS) void wkv4_bwd_seg(int T, int C, int S, const float* __restrict__ w_,
                                                    const float* __restrict__ u_, const float* __restrict__ k_,
                                                    const float* __restrict__ v_, const float* __restrict__ gy_,
@@ -217,7 +226,7 @@ __global__ __launch_bounds__(NTS) void wkv4_bwd_seg(int T, int C, int S, const f
     const bool live = c < C;
     const int cc = live ? c : C - 1;
     const size_t off = static_cast<size_t>(b) * T * C + cc;
-    const float u = u_[cc], w = w_[cc];
+    const float u = u_[cc], w = RAW ? -expf(w_[cc]) : w_[cc];        // RAW: the wrapper's w = -exp(w_raw) done here
     const float* __restrict__ k = k_ + off;
     const float* __restrict__ v = v_ + off;
     const float* __restrict__ gy = gy_ + off;
@@ -346,9 +355,24 @@ __global__ __launch_bounds__(NTS) void wkv4_bwd_seg(int T, int C, int S, const f
         float a = 0.f, bsum = 0.f;
         for (int z = 0; z < NSEG; ++z) { a += part[z * CH + cl].x; bsum += part[z * CH + cl].y; }
         // the caller's buffers are accumulated into, as the reference does (wkv_cuda_v2.cu:112-113)
-        gw_[static_cast<size_t>(b) * C + c] += a * w;
-        gu_[static_cast<size_t>(b) * C + c] += bsum;
+        if constexpr (RAW) {                        // per-batch partials in the library's own scratch: plain stores
+            gw_[static_cast<size_t>(b) * C + c] = a * w;
+            gu_[static_cast<size_t>(b) * C + c] = bsum;
+        } else {
+            gw_[static_cast<size_t>(b) * C + c] += a * w;
+            gu_[static_cast<size_t>(b) * C + c] += bsum;
+        }
     }
+}
+
+// out[c] = sum_b part[b][c], in the fixed order b = 0, 1, ...: the wrapper's torch.sum(gw, dim=0) (wkv/run.py:115-116)
+__global__ __launch_bounds__(256) void wkv4_batch_sum(int B, int C, const float* __restrict__ pw, const float* __restrict__ pu,
+                                                      float* __restrict__ gw, float* __restrict__ gu) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    float a = 0.f, b2 = 0.f;
+    for (int b = 0; b < B; ++b) { a += pw[static_cast<size_t>(b) * C + c]; b2 += pu[static_cast<size_t>(b) * C + c]; }
+    gw[c] = a; gu[c] = b2;
 }
 
 int check4(int B, int T, int C) {
@@ -394,11 +418,11 @@ int rwkv_wkv4_forward(void* stream, int B, int T, int C, const float* w, const f
     if (int e = check_ptrs({w, u, k, v, y})) return e;
     if (B > 65535) {                            // beyond the grid's y range: the one-lane-per-scan kernel
         const int BC = B * C;
-        hipLaunchKernelGGL(wkv4_fwd, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
+        hipLaunchKernelGGL(wkv4_fwd<false>, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
                            BC, T, C, w, u, k, v, y);
         return launch_status();
     }
-    hipLaunchKernelGGL(wkv4_fwd_seg, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
+    hipLaunchKernelGGL(wkv4_fwd_seg<false>, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
                        T, C, (T + NSEG - 1) / NSEG, w, u, k, v, y);
     return launch_status();
 }
@@ -417,12 +441,55 @@ int rwkv_wkv4_backward(void* stream, int B, int T, int C, const float* w, const 
         return RWKV_ERR_WORKSPACE;
     if (B > 65535) {                            // beyond the grid's y range: the one-lane-per-scan kernel
         const int BC = B * C;
-        hipLaunchKernelGGL(wkv4_bwd, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
+        hipLaunchKernelGGL(wkv4_bwd<false>, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
                            BC, T, C, w, u, k, v, gy, gw, gu, gk, gv, static_cast<float*>(workspace));
         return launch_status();
     }
-    hipLaunchKernelGGL(wkv4_bwd_seg, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
+    hipLaunchKernelGGL(wkv4_bwd_seg<false>, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
                        T, C, (T + NSEG - 1) / NSEG, w, u, k, v, gy, gw, gu, gk, gv, static_cast<float*>(workspace));
+    return launch_status();
+}
+
+// ---- the whole of WKV.forward / WKV.backward (wkv/run.py:89-117) behind two entry points: raw w, summed gw and gu
+int rwkv_wkv4raw_forward(void* stream, int B, int T, int C, const float* w_raw, const float* u, const float* k,
+                         const float* v, float* y) {
+    if (int e = check4(B, T, C)) return e;
+    if (int e = check_ptrs({w_raw, u, k, v, y})) return e;
+    if (B > 65535) {
+        const int BC = B * C;
+        hipLaunchKernelGGL(wkv4_fwd<true>, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
+                           BC, T, C, w_raw, u, k, v, y);
+        return launch_status();
+    }
+    hipLaunchKernelGGL(wkv4_fwd_seg<true>, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
+                       T, C, (T + NSEG - 1) / NSEG, w_raw, u, k, v, y);
+    return launch_status();
+}
+
+size_t rwkv_wkv4raw_backward_workspace_bytes(int B, int T, int C) {
+    if (check4(B, T, C) != RWKV_OK) return 0;
+    return (static_cast<size_t>(B) * T * C + 2 * static_cast<size_t>(B) * C) * sizeof(float);
+}
+
+int rwkv_wkv4raw_backward(void* stream, int B, int T, int C, const float* w_raw, const float* u, const float* k,
+                          const float* v, const float* gy, float* gw, float* gu, float* gk, float* gv,
+                          void* workspace, size_t workspace_bytes) {
+    if (int e = check4(B, T, C)) return e;
+    if (int e = check_ptrs({w_raw, u, k, v, gy, gw, gu, gk, gv})) return e;
+    if (workspace == nullptr || !aligned16(workspace) || workspace_bytes < rwkv_wkv4raw_backward_workspace_bytes(B, T, C))
+        return RWKV_ERR_WORKSPACE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    float* ze = static_cast<float*>(workspace);
+    float* pw = ze + static_cast<size_t>(B) * T * C;
+    float* pu = pw + static_cast<size_t>(B) * C;
+    if (B > 65535) {
+        const int BC = B * C;
+        hipLaunchKernelGGL(wkv4_bwd<true>, dim3((BC + NT - 1) / NT), dim3(NT), 0, st, BC, T, C, w_raw, u, k, v, gy, pw, pu, gk, gv, ze);
+    } else {
+        hipLaunchKernelGGL(wkv4_bwd_seg<true>, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, st,
+                           T, C, (T + NSEG - 1) / NSEG, w_raw, u, k, v, gy, pw, pu, gk, gv, ze);
+    }
+    hipLaunchKernelGGL(wkv4_batch_sum, dim3((C + 255) / 256), dim3(256), 0, st, B, C, pw, pu, gw, gu);
     return launch_status();
 }
 

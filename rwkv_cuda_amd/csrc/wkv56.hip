@@ -557,6 +557,31 @@ size_t ws_bytes(int B, int T, int C, int H) {
     return static_cast<size_t>(B) * T * C * sizeof(float) + static_cast<size_t>(B) * H * npck * 64 * 64 * sizeof(float);
 }
 
+// ---- wrapper-side steps of WKV_5 / WKV_6 (wkv5_bf16/run.py:63-64,86-87; wkv6/run.py:169) as two small kernels
+// ew = -exp(w_raw), eew = exp(ew) in fp32 from the raw bf16 decay parameter [H*N]; decay = [eew | ew]
+__global__ __launch_bounds__(256) void wkv5_decay_transform(int C, const uint16_t* __restrict__ w_raw, float* __restrict__ decay) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const float ew = -expf(bf2f(w_raw[c]));
+    decay[c] = expf(ew);
+    decay[C + c] = ew;
+}
+// out[c] = bf16(sum_b float(part[b][c])) for one or two [B,C] bf16 arrays: torch.sum(x, 0) of the per-batch partials
+__global__ __launch_bounds__(256) void bf16_batch_sum(int B, int C, const uint16_t* __restrict__ p0, uint16_t* __restrict__ o0,
+                                                      const uint16_t* __restrict__ p1, uint16_t* __restrict__ o1) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    float a = 0.f, b2 = 0.f;
+    for (int b = 0; b < B; ++b) {
+        a += bf2f(p0[static_cast<size_t>(b) * C + c]);
+        if (p1 != nullptr) b2 += bf2f(p1[static_cast<size_t>(b) * C + c]);
+    }
+    o0[c] = f2bf(a);
+    if (p1 != nullptr) o1[c] = f2bf(b2);
+}
+
+size_t round16(size_t x) { return (x + 15) & ~static_cast<size_t>(15); }
+
 }  // namespace
 }  // namespace rwkv
 
@@ -722,6 +747,61 @@ int rwkv_wkv6state_backward_ex(void* stream, int B, int T, int C, int H, const r
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.gs = gs; a.rdr = static_cast<float*>(workspace);
     return launch_bwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, flags);
+}
+
+// ---- the whole of WKV_5 / WKV_6 / WKV_6STATE forward and backward behind the C ABI: raw decay parameter in, parameter
+//      gradients summed over the batch out (no torch kernel is left in the autograd step)
+int rwkv_wkv5raw_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                         const rwkv_bf16* w_raw, const rwkv_bf16* u, rwkv_bf16* y, float* decay, unsigned flags) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, w_raw, u, y, decay})) return e;
+    hipLaunchKernelGGL(wkv5_decay_transform, dim3((C + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), C, w_raw, decay);
+    return rwkv_wkv5_forward_ex(stream, B, T, C, H, r, k, v, decay, u, y, flags);
+}
+
+size_t rwkv_wkv5raw_backward_workspace_bytes(int B, int T, int C, int H) {
+    const size_t n = ws_bytes(B, T, C, H);
+    return n == 0 ? 0 : round16(n) + round16(2 * static_cast<size_t>(B) * C * sizeof(uint16_t));
+}
+
+int rwkv_wkv5raw_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                          const float* decay, const rwkv_bf16* u, const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk,
+                          rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu, void* workspace, size_t workspace_bytes, unsigned flags) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({decay, gw, gu})) return e;
+    if (workspace == nullptr || workspace_bytes < rwkv_wkv5raw_backward_workspace_bytes(B, T, C, H) || !aligned16(workspace))
+        return RWKV_ERR_WORKSPACE;
+    const size_t n = round16(ws_bytes(B, T, C, H));
+    uint16_t* pw = reinterpret_cast<uint16_t*>(static_cast<char*>(workspace) + n);      // per-batch gw, then per-batch gu
+    uint16_t* pu = pw + static_cast<size_t>(B) * C;
+    if (int e = rwkv_wkv5_backward_ex(stream, B, T, C, H, r, k, v, decay, decay + C, u, gy, gr, gk, gv, pw, pu, workspace, n, flags)) return e;
+    hipLaunchKernelGGL(bf16_batch_sum, dim3((C + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), B, C, pw, gw, pu, gu);
+    return launch_status();
+}
+
+size_t rwkv_wkv6f_backward_workspace_bytes(int B, int T, int C, int H) {
+    const size_t n = ws_bytes(B, T, C, H);
+    return n == 0 ? 0 : round16(n) + round16(static_cast<size_t>(B) * C * sizeof(uint16_t));
+}
+
+int rwkv_wkv6f_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                        const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, const rwkv_bf16* gy, rwkv_bf16* gr,
+                        rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu, rwkv_bf16* gs, void* workspace,
+                        size_t workspace_bytes, unsigned flags) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({gu})) return e;
+    if ((s == nullptr) != (gs == nullptr)) return RWKV_ERR_NULL;           // state and its gradient come together
+    if (workspace == nullptr || workspace_bytes < rwkv_wkv6f_backward_workspace_bytes(B, T, C, H) || !aligned16(workspace))
+        return RWKV_ERR_WORKSPACE;
+    const size_t n = round16(ws_bytes(B, T, C, H));
+    uint16_t* pu = reinterpret_cast<uint16_t*>(static_cast<char*>(workspace) + n);      // per-batch gu
+    const int e = s != nullptr
+        ? rwkv_wkv6state_backward_ex(stream, B, T, C, H, r, k, v, w, u, s, gy, gr, gk, gv, gw, pu, gs, workspace, n, flags)
+        : rwkv_wkv6raw_backward_ex(stream, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, pu, workspace, n, flags);
+    if (e) return e;
+    hipLaunchKernelGGL(bf16_batch_sum, dim3((C + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), B, C, pu, gu,
+                       static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(nullptr));
+    return launch_status();
 }
 
 // ---- the reference-signature entry points: default kernels, every pass

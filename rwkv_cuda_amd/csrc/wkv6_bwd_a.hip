@@ -59,7 +59,7 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
     // channel pair (2 jp, 2 jp + 1), tokens 4 wid + 2 th + {0, 1}
     const int jp = lane & 31, th = lane >> 5, pt0 = 4 * wid + 2 * th;
     const bool second = wid >= 4;
-    struct Raw { uint32_t r[2], k[2], v[2], g[2], w[2][WMODE == W_EW ? 2 : 1]; float lam[2][2], other[2], kp[2][2]; };
+    struct Raw { uint32_t r[2], k[2], v[2], g[2], w[2]; uint2 wq[2]; float lam[2][2], other[2], kp[2][2]; };
     Raw ring[STA];
     // Loads are asm so that the wait before their first use can leave the younger batches in flight; every call issues the
     // same ten loads (chunk index clamped), which keeps the count fixed.
@@ -73,31 +73,30 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
         for (int e = 0; e < 2; ++e) {
             const int t = c * L + pt0 + e;
             const uint32_t o = (static_cast<uint32_t>(t < T ? t : T - 1) * C + 2 * jp) * 2;    // byte offset of the channel pair
-            asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(x.r[e]) : "v"(o), "s"(rb));
-            asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(x.k[e]) : "v"(o), "s"(kb));
-            asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(x.v[e]) : "v"(o), "s"(vb));
-            asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(x.g[e]) : "v"(o), "s"(gb));
+            asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(x.r[e]) : "v"(o), "s"(rb) : "memory");
+            asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(x.k[e]) : "v"(o), "s"(kb) : "memory");
+            asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(x.v[e]) : "v"(o), "s"(vb) : "memory");
+            asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(x.g[e]) : "v"(o), "s"(gb) : "memory");
             if constexpr (WMODE == W_RAW) {
-                asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(x.w[e][0]) : "v"(o), "s"(wb32));
+                asm volatile("global_load_dword %0, %1, %2 nt" : "=&v"(x.w[e]) : "v"(o), "s"(wb32) : "memory");
             } else if constexpr (WMODE == W_EW) {
-                uint2 y;
-                asm volatile("global_load_dwordx2 %0, %1, %2 nt" : "=&v"(y) : "v"(2 * o), "s"(wbf));
-                x.w[e][0] = y.x; x.w[e][1] = y.y;
+                // straight into the ring: a copy here would read the register before the load has landed
+                asm volatile("global_load_dwordx2 %0, %1, %2 nt" : "=&v"(x.wq[e]) : "v"(2 * o), "s"(wbf) : "memory");
             }
         }
     };
     constexpr int NLOADS = WMODE == W_HEAD ? 8 : 10;   // loads per prefetch call
     auto arrived = [&](Raw& x, auto younger) __attribute__((always_inline)) {
         if constexpr (WMODE == W_RAW)
-            asm volatile("s_waitcnt vmcnt(%10)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
-                         "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[1][0]) : "n"(decltype(younger)::value * NLOADS));
+            asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0]), "+v"(x.w[1]) : [n] "n"(decltype(younger)::value * NLOADS) : "memory");
         else if constexpr (WMODE == W_EW)
-            asm volatile("s_waitcnt vmcnt(%12)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
-                         "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.w[0][0]), "+v"(x.w[0][1]), "+v"(x.w[1][0]), "+v"(x.w[1][1])
-                         : "n"(decltype(younger)::value * NLOADS));
+            asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.g[0]), "+v"(x.g[1]), "+v"(x.wq[0]), "+v"(x.wq[1])
+                         : [n] "n"(decltype(younger)::value * NLOADS) : "memory");
         else
-            asm volatile("s_waitcnt vmcnt(%8)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
-                         "+v"(x.g[0]), "+v"(x.g[1]) : "n"(decltype(younger)::value * NLOADS));
+            asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.g[0]), "+v"(x.g[1]) : [n] "n"(decltype(younger)::value * NLOADS) : "memory");
     };
     // wkv5: one decay per channel for the whole sequence, given as ew = -exp(w_raw) = log of the decay
     float lamc[2] = {0.f, 0.f};
@@ -115,16 +114,16 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
             for (int e = 0; e < 2; ++e)
                 if (c0 + pt0 + e >= T) {
                     x.r[e] = 0; x.k[e] = 0; x.v[e] = 0; x.g[e] = 0;
-                    if constexpr (WMODE == W_RAW) x.w[e][0] = 0xff80ff80u;   // w = -inf  ->  lam = -exp(w) = 0
-                    if constexpr (WMODE == W_EW) { x.w[e][0] = 0u; x.w[e][1] = 0u; }
+                    if constexpr (WMODE == W_RAW) x.w[e] = 0xff80ff80u;   // w = -inf  ->  lam = -exp(w) = 0
+                    if constexpr (WMODE == W_EW) x.wq[e] = make_uint2(0u, 0u);
                 }
         }
 #pragma unroll
         for (int e = 0; e < 2; ++e)
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
-                if constexpr (WMODE == W_RAW) x.lam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e][0]) : bf_lo(x.w[e][0])));
-                else if constexpr (WMODE == W_EW) x.lam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+                if constexpr (WMODE == W_RAW) x.lam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e]) : bf_lo(x.w[e])));
+                else if constexpr (WMODE == W_EW) x.lam[e][z] = LOG2E * __uint_as_float(z ? x.wq[e].y : x.wq[e].x);
                 else x.lam[e][z] = (c0 + pt0 + e < T) ? lamc[z] : 0.f;
             }
         float s2[2];

@@ -63,7 +63,7 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + 2 * jp);
         uj[0] = bf_lo(x); uj[1] = bf_hi(x);
     }
-    struct Raw { uint32_t r[2], k[2], v[2], w[2][WMODE == W_EW ? 2 : 1]; float lam[2][2], other[2], kp[2][2]; };
+    struct Raw { uint32_t r[2], k[2], v[2], w[2]; uint2 wq[2]; float lam[2][2], other[2], kp[2][2]; };
     // fp32 decays take two more registers per token: one stage less keeps the ring in registers
     constexpr int NST = WMODE == W_EW ? STAGES - 1 : STAGES;
     Raw ring[NST];
@@ -78,15 +78,14 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         for (int e = 0; e < 2; ++e) {
             const int t = c * L + pt0 + e;
             const uint32_t o = (static_cast<uint32_t>(t < T ? t : T - 1) * C + 2 * jp) * 2;    // byte offset of the channel pair
-            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.r[e]) : "v"(o), "s"(rb));
-            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.k[e]) : "v"(o), "s"(kb));
-            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.v[e]) : "v"(o), "s"(vb));
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.r[e]) : "v"(o), "s"(rb) : "memory");
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.k[e]) : "v"(o), "s"(kb) : "memory");
+            asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.v[e]) : "v"(o), "s"(vb) : "memory");
             if constexpr (WMODE == W_RAW) {
-                asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.w[e][0]) : "v"(o), "s"(wb32));
+                asm volatile("global_load_dword %0, %1, %2" : "=&v"(x.w[e]) : "v"(o), "s"(wb32) : "memory");
             } else if constexpr (WMODE == W_EW) {
-                uint2 y;
-                asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(y) : "v"(2 * o), "s"(wbf));
-                x.w[e][0] = y.x; x.w[e][1] = y.y;
+                // straight into the ring: a copy here would read the register before the load has landed
+                asm volatile("global_load_dwordx2 %0, %1, %2" : "=&v"(x.wq[e]) : "v"(2 * o), "s"(wbf) : "memory");
             }
         }
     };
@@ -94,14 +93,14 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
     constexpr int NLOADS = WMODE == W_HEAD ? 6 : 8;    // loads per prefetch call
     auto arrived = [&](Raw& x, auto younger) __attribute__((always_inline)) {
         if constexpr (WMODE == W_EW)
-            asm volatile("s_waitcnt vmcnt(%10)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
-                         "+v"(x.w[0][0]), "+v"(x.w[0][1]), "+v"(x.w[1][0]), "+v"(x.w[1][1]) : "n"(decltype(younger)::value * NLOADS));
+            asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.wq[0]), "+v"(x.wq[1]) : [n] "n"(decltype(younger)::value * NLOADS) : "memory");
         else if constexpr (WMODE == W_RAW)
-            asm volatile("s_waitcnt vmcnt(%8)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
-                         "+v"(x.w[0][0]), "+v"(x.w[1][0]) : "n"(decltype(younger)::value * NLOADS));
+            asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1]),
+                         "+v"(x.w[0]), "+v"(x.w[1]) : [n] "n"(decltype(younger)::value * NLOADS) : "memory");
         else
-            asm volatile("s_waitcnt vmcnt(%6)" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1])
-                         : "n"(decltype(younger)::value * NLOADS));
+            asm volatile("s_waitcnt vmcnt(%[n])" : "+v"(x.r[0]), "+v"(x.r[1]), "+v"(x.k[0]), "+v"(x.k[1]), "+v"(x.v[0]), "+v"(x.v[1])
+                         : [n] "n"(decltype(younger)::value * NLOADS) : "memory");
     };
     // wkv5: one decay per channel for the whole sequence, given as eew = exp(-exp(w_raw)); lam = log2(eew)
     float lamc[2] = {0.f, 0.f};
@@ -143,16 +142,16 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
             for (int e = 0; e < 2; ++e)
                 if (c0 + pt0 + e >= T) {
                     x.r[e] = 0; x.k[e] = 0; x.v[e] = 0;
-                    if constexpr (WMODE == W_RAW) x.w[e][0] = 0xff80ff80u;   // w = -inf  ->  lam = -exp(w) = 0
-                    if constexpr (WMODE == W_EW) { x.w[e][0] = 0u; x.w[e][1] = 0u; }
+                    if constexpr (WMODE == W_RAW) x.w[e] = 0xff80ff80u;   // w = -inf  ->  lam = -exp(w) = 0
+                    if constexpr (WMODE == W_EW) x.wq[e] = make_uint2(0u, 0u);
                 }
         }
 #pragma unroll
         for (int e = 0; e < 2; ++e)
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
-                if constexpr (WMODE == W_RAW) x.lam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e][0]) : bf_lo(x.w[e][0])));
-                else if constexpr (WMODE == W_EW) x.lam[e][z] = LOG2E * __uint_as_float(x.w[e][z]);
+                if constexpr (WMODE == W_RAW) x.lam[e][z] = -LOG2E * exp2_fast(LOG2E * (z ? bf_hi(x.w[e]) : bf_lo(x.w[e])));
+                else if constexpr (WMODE == W_EW) x.lam[e][z] = LOG2E * __uint_as_float(z ? x.wq[e].y : x.wq[e].x);
                 else x.lam[e][z] = (c0 + pt0 + e < T) ? lamc[z] : 0.f;
             }
         float s2[2];

@@ -12,13 +12,13 @@ class WKV(torch.autograd.Function):
     @staticmethod
     def forward(ctx, B, T, C, w, u, k, v):
         ctx.B, ctx.T, ctx.C = B, T, C
-        w = -torch.exp(w.contiguous())
-        u, k, v = u.contiguous(), k.contiguous(), v.contiguous()
+        # w = -exp(w) of the reference wrapper (:95) happens inside the kernels (rwkv_wkv4raw_*)
+        w, u, k, v = w.contiguous(), u.contiguous(), k.contiguous(), v.contiguous()
         dev = check_tensors((w, u, k, v), torch.float32, "wukv")
         require(k.numel() == B * T * C and w.numel() == C, "shape mismatch")
         ctx.save_for_backward(w, u, k, v)
         y = torch.empty((B, T, C), device=dev, dtype=torch.float32)
-        call("rwkv_wkv4_forward", dev, B, T, C, w, u, k, v, y)
+        call("rwkv_wkv4raw_forward", dev, B, T, C, w, u, k, v, y)
         return y
 
     @staticmethod
@@ -27,15 +27,13 @@ class WKV(torch.autograd.Function):
         w, u, k, v = ctx.saved_tensors
         gy = gy.contiguous()
         dev = check_tensors((gy,), torch.float32, ("gy",))
-        gw = torch.zeros((B, C), device=dev, dtype=torch.float32)
-        gu = torch.zeros((B, C), device=dev, dtype=torch.float32)
+        gw = torch.empty((C,), device=dev, dtype=torch.float32)      # summed over the batch by the library (:115-116)
+        gu = torch.empty((C,), device=dev, dtype=torch.float32)
         gk = torch.empty((B, T, C), device=dev, dtype=torch.float32)
         gv = torch.empty((B, T, C), device=dev, dtype=torch.float32)
-        nbytes = _lib.load().rwkv_wkv4_backward_workspace_bytes(B, T, C)
+        nbytes = _lib.load().rwkv_wkv4raw_backward_workspace_bytes(B, T, C)
         ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
-        call("rwkv_wkv4_backward", dev, B, T, C, w, u, k, v, gy, gw, gu, gk, gv, ws, nbytes)
-        gw = torch.sum(gw, dim=0)
-        gu = torch.sum(gu, dim=0)
+        call("rwkv_wkv4raw_backward", dev, B, T, C, w, u, k, v, gy, gw, gu, gk, gv, ws, nbytes)
         return (None, None, None, gw, gu, gk, gv)
 
 

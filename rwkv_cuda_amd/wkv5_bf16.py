@@ -20,28 +20,26 @@ class WKV_5(torch.autograd.Function):
             require(r.numel() == B * T * C and w.numel() == C, "shape mismatch")
             ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
             ctx.flags = options.current_flags()
-            ew = (-torch.exp(w.float())).contiguous()
-            eew = (torch.exp(ew)).contiguous()
-            ctx.save_for_backward(r, k, v, eew, ew, u)
+            # ew = -exp(w.float()), eew = exp(ew) (:63-64) are made by the library into `decay` = [eew | ew]
+            decay = torch.empty(2 * C, device=dev, dtype=torch.float32)
             y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
-            call("rwkv_wkv5_forward_ex", dev, B, T, C, H, r, k, v, eew, u, y, ctx.flags)
+            call("rwkv_wkv5raw_forward", dev, B, T, C, H, r, k, v, w, u, y, decay, ctx.flags)
+            ctx.save_for_backward(r, k, v, decay, u)
             return y
 
     @staticmethod
     def backward(ctx, gy):
         with torch.no_grad():
             B, T, C, H = ctx.B, ctx.T, ctx.C, ctx.H
-            r, k, v, eew, ew, u = ctx.saved_tensors
+            r, k, v, decay, u = ctx.saved_tensors
             gy = gy.contiguous()
             dev = check_tensors((gy,), torch.bfloat16, ("gy",))
             new = lambda *shape: torch.empty(shape, device=dev, dtype=torch.bfloat16)
             gr, gk, gv = new(B, T, C), new(B, T, C), new(B, T, C)
-            gw, gu = new(B, C), new(B, C)
-            nbytes = _lib.load().rwkv_wkv5_backward_workspace_bytes(B, T, C, H)
+            gw, gu = new(H, C // H), new(H, C // H)           # summed over the batch by the library (:86-87)
+            nbytes = _lib.load().rwkv_wkv5raw_backward_workspace_bytes(B, T, C, H)
             ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
-            call("rwkv_wkv5_backward_ex", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes, ctx.flags)
-            gw = torch.sum(gw, 0).view(H, C // H)
-            gu = torch.sum(gu, 0).view(H, C // H)
+            call("rwkv_wkv5raw_backward", dev, B, T, C, H, r, k, v, decay, u, gy, gr, gk, gv, gw, gu, ws, nbytes, ctx.flags)
             return (None, None, None, None, gr, gk, gv, gw, gu)
 
 

@@ -36,11 +36,10 @@ class WKV_6(torch.autograd.Function):
             dev = check_tensors((gy,), torch.bfloat16, ("gy",))
             new = lambda *shape: torch.empty(shape, device=dev, dtype=torch.bfloat16)
             gr, gk, gv, gw = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C)
-            gu = new(B, C)
-            nbytes = _lib.load().rwkv_wkv6_backward_workspace_bytes(B, T, C, H)
+            gu = new(H, C // H)                               # summed over the batch by the library (:169)
+            nbytes = _lib.load().rwkv_wkv6f_backward_workspace_bytes(B, T, C, H)
             ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
-            call("rwkv_wkv6raw_backward_ex", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes, ctx.flags)
-            gu = torch.sum(gu, 0).view(H, C // H)
+            call("rwkv_wkv6f_backward", dev, B, T, C, H, r, k, v, w, u, None, gy, gr, gk, gv, gw, gu, None, ws, nbytes, ctx.flags)
             return (None, None, None, None, gr, gk, gv, gw, gu)
 
 

@@ -34,13 +34,12 @@ class WKV_6STATE(torch.autograd.Function):
             dev = check_tensors((gy,), torch.bfloat16, ("gy",))
             new = lambda *shape: torch.empty(shape, device=dev, dtype=torch.bfloat16)
             gr, gk, gv, gw = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C)
-            gu = new(B, C)
+            gu = new(H, C // H)                               # summed over the batch by the library (:123)
             gs = new(B, H, C // H, C // H)
-            nbytes = _lib.load().rwkv_wkv6state_backward_workspace_bytes(B, T, C, H)
+            nbytes = _lib.load().rwkv_wkv6f_backward_workspace_bytes(B, T, C, H)
             ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
-            call("rwkv_wkv6state_backward_ex", dev, B, T, C, H, r, k, v, w, u, s, gy,
+            call("rwkv_wkv6f_backward", dev, B, T, C, H, r, k, v, w, u, s, gy,
                  gr, gk, gv, gw, gu, gs, ws, nbytes, ctx.flags)
-            gu = torch.sum(gu, 0).view(H, C // H)
             return (None, None, None, None, gr, gk, gv, gw, gu, gs)
 
 
