@@ -78,26 +78,27 @@ def make_wkv6(dev, state):
     r, k, v, w, u, gy, s0 = (x.to(dev) if x is not None else None for x in synth.wkv6_inputs(B, T, C, H, seed=42, state=state))
     new = lambda *s: torch.empty(s, device=dev, dtype=bf)
     y, gr, gk, gv, gw, gu = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C), new(B, C)
-    nbytes = lib.rwkv_wkv6_backward_workspace_bytes(B, T, C, H)
+    gu_sum = new(H, N)
+    nbytes = lib.rwkv_wkv6f_backward_workspace_bytes(B, T, C, H)
     ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
     tok = B * T
     if state:
         gs = new(B, H, N, N)
 
         def step():
+            # what WKV_6STATE.forward / backward do; the wrapper's torch.sum(gu, 0) (wkv6_state/run.py:123) runs inside the library
             call("rwkv_wkv6state_forward_ex", dev, B, T, C, H, r, k, v, w, u, s0, y, FLAGS)
-            call("rwkv_wkv6state_backward_ex", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes, FLAGS)
-            return torch.sum(gu, 0).view(H, N)
+            call("rwkv_wkv6f_backward", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu_sum, gs, ws, nbytes, FLAGS)
 
         kernels = [("wkv6state forward", lambda: call("rwkv_wkv6state_forward_ex", dev, B, T, C, H, r, k, v, w, u, s0, y, FLAGS), 10 * C * tok),
                    ("wkv6state backward (3 kernels)", lambda: call("rwkv_wkv6state_backward_ex", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes, FLAGS), 18 * C * tok)]
         name = "wkv6_state"
     else:
         def step():
-            # what WKV_6.forward / backward do: raw bf16 decay straight into the kernels, per-batch gu summed by torch
+            # what WKV_6.forward / backward do: raw bf16 decay straight into the kernels; the wrapper's torch.sum(gu, 0)
+            # (wkv6/run.py:169) runs inside the library (one small kernel after the two sweeps)
             call("rwkv_wkv6raw_forward_ex", dev, B, T, C, H, r, k, v, w, u, y, FLAGS)
-            call("rwkv_wkv6raw_backward_ex", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes, FLAGS)
-            return torch.sum(gu, 0).view(H, N)                      # wrapper reduction, wkv6/run.py:169
+            call("rwkv_wkv6f_backward", dev, B, T, C, H, r, k, v, w, u, None, gy, gr, gk, gv, gw, gu_sum, None, ws, nbytes, FLAGS)
 
         def bwd(mask):
             def run():
@@ -142,18 +143,19 @@ def make_wkv5(dev):
     r, k, v, w, u, gy = (x.to(dev) for x in synth.wkv5_inputs(B, T, C, H, seed=42))
     new = lambda *s: torch.empty(s, device=dev, dtype=bf)
     y, gr, gk, gv, gw, gu = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C), new(B, C), new(B, C)
-    nbytes = lib.rwkv_wkv5_backward_workspace_bytes(B, T, C, H)
+    gw_sum, gu_sum = new(H, N), new(H, N)
+    decay = torch.empty(2 * C, device=dev, dtype=torch.float32)
+    nbytes = lib.rwkv_wkv5raw_backward_workspace_bytes(B, T, C, H)
     ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
     tok = B * T
     ew = (-torch.exp(w.float())).contiguous()
     eew = torch.exp(ew).contiguous()
 
     def step():
-        ew_ = (-torch.exp(w.float())).contiguous()
-        eew_ = torch.exp(ew_).contiguous()
-        call("rwkv_wkv5_forward_ex", dev, B, T, C, H, r, k, v, eew_, u, y, FLAGS)
-        call("rwkv_wkv5_backward_ex", dev, B, T, C, H, r, k, v, eew_, ew_, u, gy, gr, gk, gv, gw, gu, ws, nbytes, FLAGS)
-        return torch.sum(gw, 0), torch.sum(gu, 0)
+        # what WKV_5.forward / backward do; the decay transforms (wkv5_bf16/run.py:63-64) and the sums over the batch
+        # (:86-87) run inside the library
+        call("rwkv_wkv5raw_forward", dev, B, T, C, H, r, k, v, w, u, y, decay, FLAGS)
+        call("rwkv_wkv5raw_backward", dev, B, T, C, H, r, k, v, decay, u, gy, gr, gk, gv, gw_sum, gu_sum, ws, nbytes, FLAGS)
 
     def bwd(mask):
         def run():
@@ -300,21 +302,29 @@ def make_rwkv7(dev, fp32=False):
         st = s0
         for i in range(4):
             rr, ww, kk, vv, aa, bb, _ = seg[i]
-            call("rwkv7_statepassing_forward" + sfx, dev, B, TS, H, st, rr, ww, kk, vv, aa, bb, ys[i], sTs[i], ss[i], sas[i])
+            if fp32:
+                call("rwkv7_statepassing_forward_f32", dev, B, TS, H, st, rr, ww, kk, vv, aa, bb, ys[i], sTs[i], ss[i], sas[i])
+            else:
+                call("rwkv7_statepassing_forward_ex", dev, B, TS, H, st, rr, ww, kk, vv, aa, bb, ys[i], sTs[i], ss[i], sas[i], FLAGS)
             st = sTs[i]
 
     def bwd():
         g = dsT
         for i in (3, 2, 1, 0):
             rr, ww, kk, vv, aa, bb, dd = seg[i]
-            call("rwkv7_statepassing_backward" + sfx, dev, B, TS, H, rr, ww, kk, vv, aa, bb, dd, g, ss[i], sas[i], ds[i], *grads[i])
+            if fp32:
+                call("rwkv7_statepassing_backward_f32", dev, B, TS, H, rr, ww, kk, vv, aa, bb, dd, g, ss[i], sas[i], ds[i], *grads[i])
+            else:
+                call("rwkv7_statepassing_backward_ex", dev, B, TS, H, rr, ww, kk, vv, aa, bb, dd, g, ss[i], sas[i], ds[i], *grads[i], FLAGS)
             g = ds[i]
 
     def step():
         fwd()
         bwd()
 
-    kernels = [("rwkv7 forward x4 (T=1024 each)", fwd, 7 * eb * C * tok), ("rwkv7 backward x4", bwd, 13 * eb * C * tok)]
+    chunked = not fp32 and ALGO == "chunked"
+    kernels = [("rwkv7c_fwd x4 (T=1024 each)" if chunked else "rwkv7_fwd x4 (T=1024 each)", fwd, 7 * eb * C * tok),
+               ("rwkv7c_bwd x4" if chunked else "rwkv7_bwd x4", bwd, 13 * eb * C * tok)]
 
     def cpu_baseline(t_cpu=64):
         from oracle import rwkv7 as O
@@ -336,21 +346,19 @@ def make_wkv4(dev):
     B, T, C = 4, 512, 768
     w_raw, u, k, v, gy = (x.to(dev) for x in synth.wkv4_inputs(B, T, C, seed=42))
     y, gk, gv = (torch.empty(B, T, C, device=dev) for _ in range(3))
-    nbytes = lib.rwkv_wkv4_backward_workspace_bytes(B, T, C)
+    nbytes = lib.rwkv_wkv4raw_backward_workspace_bytes(B, T, C)
     ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
     tok = B * T
-    w_keep = -torch.exp(w_raw)
-    gwz, guz = torch.zeros(B, C, device=dev), torch.zeros(B, C, device=dev)
+    gw, gu = torch.empty(C, device=dev), torch.empty(C, device=dev)
 
     def step():
-        w = -torch.exp(w_raw)
-        call("rwkv_wkv4_forward", dev, B, T, C, w, u, k, v, y)
-        gw, gu = torch.zeros(B, C, device=dev), torch.zeros(B, C, device=dev)
-        call("rwkv_wkv4_backward", dev, B, T, C, w, u, k, v, gy, gw, gu, gk, gv, ws, nbytes)
-        return gw.sum(0), gu.sum(0)
+        # what WKV.forward / backward do; w = -exp(w_raw), the zero-fills and the sums over the batch (wkv/run.py:95,110-116)
+        # run inside the library
+        call("rwkv_wkv4raw_forward", dev, B, T, C, w_raw, u, k, v, y)
+        call("rwkv_wkv4raw_backward", dev, B, T, C, w_raw, u, k, v, gy, gw, gu, gk, gv, ws, nbytes)
 
-    kernels = [("wkv4 forward", lambda: call("rwkv_wkv4_forward", dev, B, T, C, w_keep, u, k, v, y), 12 * C * tok),
-               ("wkv4 backward", lambda: call("rwkv_wkv4_backward", dev, B, T, C, w_keep, u, k, v, gy, gwz, guz, gk, gv, ws, nbytes), 20 * C * tok)]
+    kernels = [("wkv4_fwd_seg", lambda: call("rwkv_wkv4raw_forward", dev, B, T, C, w_raw, u, k, v, y), 12 * C * tok),
+               ("wkv4_bwd_seg + wkv4_batch_sum", lambda: call("rwkv_wkv4raw_backward", dev, B, T, C, w_raw, u, k, v, gy, gw, gu, gk, gv, ws, nbytes), 20 * C * tok)]
 
     def cpu_baseline():
         from oracle import wkv4 as O
@@ -423,7 +431,7 @@ def main():
     ap.add_argument("--workload", default="wkv6", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--algo", default="chunked", choices=["chunked", "sweeps"],
-                    help="wkv6 kernels: chunked MFMA formulation (default) or the sequential fp32 sweeps")
+                    help="wkv5 / wkv6 / rwkv7 kernels: chunked matrix-core formulation (default) or the sequential fp32 recurrence")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy, so that a rocprofv3 --pmc run holds a kernel of known traffic")
     args = ap.parse_args()
@@ -460,13 +468,27 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # EXACTLY K timed steps between two synchronisations (the contract's figure), with a HIP event after every step so
+    # that the spread over the steps can be reported too (an event record costs no kernel and ~1 us of host time)
+    marks = _events(args.steps + 1)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         step()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = 1e3 * dt / args.steps
     mtok = tok / (dt / args.steps) / 1e6
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    ms_min, ms_median = per_step[0], per_step[len(per_step) // 2]
+
+    # what a plain copy reaches on this device (read 1 GiB + write 1 GiB per launch): the achievable HBM rate beside the 8 TB/s peak
+    src = torch.empty(1 << 28, device=dev, dtype=torch.float32).normal_()
+    dst = torch.empty_like(src)
+    copy_ms = time_gpu(lambda: dst.copy_(src), 10, 3)
+    copy_gbps = 2 * src.numel() * 4 / (copy_ms * 1e-3) / 1e9
+    del src, dst
 
     # per-kernel timing, HIP events on the launch stream
     per_kernel = []
@@ -477,21 +499,27 @@ def main():
         if flops:                                # a kernel bound by the fp32 matrix cores, not by HBM
             per_kernel[-1].update(algorithmic_flops=flops[0], TFLOPs=round(flops[0] / (ms * 1e-3) / 1e12, 2))
     dom = max(per_kernel, key=lambda d: d["ms"])
+    traffic = TRAFFIC_MEASURED.get(dom["kernel"]) if ALGO == "chunked" else None
+    step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(dom["GBps"] / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_MEASURED.get(dom["kernel"]),
+                "frac": round(dom["GBps"] / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "traffic_over_algorithmic": round(traffic / dom["algorithmic_bytes"], 3) if traffic else None,
                 "launch_ms": dom["ms"], "algorithmic_bytes": dom["algorithmic_bytes"],
-                "whole_step_frac": round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                "whole_step_frac": round(step_gbps / HBM_PEAK_GBS, 4),
+                "hbm_copy_GBps": round(copy_gbps, 1), "frac_of_copy": round(dom["GBps"] / copy_gbps, 4),
+                "whole_step_frac_of_copy": round(step_gbps / copy_gbps, 4)}
     if "TFLOPs" in dom:
         roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["TFLOPs"], "peak": FP32_MFMA_PEAK_TFLOPS,
                     "unit": "TFLOP/s", "frac": round(dom["TFLOPs"] / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
                     "launch_ms": dom["ms"], "algorithmic_flops": dom["algorithmic_flops"],
-                    "hbm_frac": round(dom["GBps"] / HBM_PEAK_GBS, 4)}
+                    "hbm_frac": round(dom["GBps"] / HBM_PEAK_GBS, 4), "hbm_copy_GBps": round(copy_gbps, 1)}
 
     out = {
         "metric": "WKV6 bf16 fwd+bwd Mtokens/s @B8 T4096 C2048; % HBM peak achieved" if args.workload == "wkv6"
                   else f"{args.workload} fwd+bwd Mtokens/s; % HBM peak achieved",
         "value": round(mtok, 3), "unit": "Mtokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4), "prewarm_s": PREWARM_S, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 4), "ms_per_step_min": round(ms_min, 4), "ms_per_step_median": round(ms_median, 4),
+        "prewarm_s": PREWARM_S, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": DTYPES[args.workload], "data": "synthetic", "config": cfg,
         "pct_hbm_peak": round(100 * step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
         "roofline": roofline, "kernels": per_kernel,
