@@ -38,10 +38,21 @@ TRAFFIC_MEASURED = {
     "wkv6_bwd_a_ws": 683e6 + 432e6,
     "wkv6_bwd_b_ws": 990e6 + 403e6,
     # profiles/wkv5_ws_kernels_B8_T4096_C2048.md
+    "wkv6_fwd_ws<head decay>": 403e6 + 134e6,
+    "wkv6_bwd_a_ws<head decay>": 548e6 + 533e6,
     "wkv6_bwd_b_ws<head decay>": 957e6 + 269e6,
     # profiles/wkv5_fp32_sweep_kernels_B8_T4096_C4096.md, profiles/wkv5a_sweep_kernels_B8_T4096_C4096.md
     "wkv_sweep<gr+gu+gw, fp32 I/O>": 2148e6 + 537e6,
     "wkv_sweep<gr+gu+gw, two-sided>": 2148e6 + 537e6,
+    # profiles/rwkv7_chunk_kernels_B8_T4096_C4096.md (four calls of T = 1024)
+    "rwkv7c_fwd x4 (T=1024 each)": 4 * (411.2e6 + 746.6e6),
+    "rwkv7c_bwd x4": 4 * (1149.7e6 + 411.0e6),
+    # profiles/wkv4_seg_kernels_B4_T512_C768.md
+    "wkv4_fwd_seg": 29.7e6 + 6.3e6,
+    "wkv4_bwd_seg + wkv4_batch_sum": 186.6e6 + 31.5e6,
+    # profiles/timex_mfma_kernels_B32_C768_T768.md
+    "timex_conv_mfma (forward)": 77.9e6 + 75.5e6,
+    "timex backward (timex_conv_mfma + timex_gw_sum_mfma)": (77.9e6 + 75.5e6) + (151.1e6 + 2.4e6),
 }
 
 
@@ -510,7 +521,8 @@ def main():
                 "whole_step_frac_of_copy": round(step_gbps / copy_gbps, 4)}
     if "TFLOPs" in dom:
         roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["TFLOPs"], "peak": FP32_MFMA_PEAK_TFLOPS,
-                    "unit": "TFLOP/s", "frac": round(dom["TFLOPs"] / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                    "unit": "TFLOP/s", "frac": round(dom["TFLOPs"] / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": traffic,
+                    "traffic_over_algorithmic": round(traffic / dom["algorithmic_bytes"], 3) if traffic else None,
                     "launch_ms": dom["ms"], "algorithmic_flops": dom["algorithmic_flops"],
                     "hbm_frac": round(dom["GBps"] / HBM_PEAK_GBS, 4), "hbm_copy_GBps": round(copy_gbps, 1)}
 
