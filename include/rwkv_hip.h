@@ -13,11 +13,14 @@
  *     (workspace, workspace_bytes) pair whose size the matching *_workspace_bytes()
  *     function reports.  No entry point allocates or frees device memory, and none
  *     synchronises: work is enqueued on `stream` and the call returns.
- *   - T is a run-time argument (the reference bakes -D_T_ into wkv6 / wkv6_state);
- *     the head size N = C / H must be 64.
+ *   - T and the head size N = C / H are run-time values (the reference bakes -D_T_ and -D_N_ into its kernels).
+ *     wkv5 (bf16), wkv6 and wkv6_state take any N from 1 to 128 (C a multiple of H); 64 runs on the matrix-core
+ *     kernels, every other size on one-thread-per-state-row kernels.  The fp32 wkv5 op takes N <= 64, wkv5a and
+ *     rwkv7 N = 64 only.
  *
  * bf16 tensors are passed as uint16_t* (raw bfloat16 bits).  All tensors are dense and
- * contiguous in the layouts named per function and must be 16-byte aligned.
+ * contiguous in the layouts named per function and must be 16-byte aligned (head sizes other than 64: any alignment
+ * of the element type).
  * Pointers are device pointers on the current HIP device.
  */
 #ifndef RWKV_HIP_H
@@ -34,7 +37,7 @@ typedef uint16_t rwkv_bf16;
 
 enum {
     RWKV_OK = 0,
-    RWKV_ERR_SHAPE = -1,     /* a dimension is <= 0, C != H*64, T not a multiple of the chunk, ... */
+    RWKV_ERR_SHAPE = -1,     /* a dimension is <= 0, an unsupported head size C / H, T not a multiple of the chunk, ... */
     RWKV_ERR_NULL = -2,      /* a required pointer is NULL */
     RWKV_ERR_ALIGN = -3,     /* a pointer is not 16-byte aligned */
     RWKV_ERR_WORKSPACE = -4, /* workspace missing or smaller than *_workspace_bytes() */

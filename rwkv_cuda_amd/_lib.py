@@ -34,7 +34,10 @@ HIPCC_FLAGS = [
 # The backward sweep B keeps one index of its state waves' epilogue in scratch, outside the loops (three values in the
 # wkv5 instantiation, ILi0E, one of them reloaded once per chunk by a state wave); anything beyond these counts fails the
 # build.
-SPILL_LIMIT = {"wkv6_fwd_ws": 0, "wkv6_bwd_a_ws": 0, "wkv6_bwd_b_wsILi0E": 3, "wkv6_bwd_b_wsILi1E": 1, "wkv6_bwd_b_wsILi2E": 1}
+# The row-per-thread kernels for other head sizes (wkv_rows) keep a whole state row in registers; an instantiation that
+# no longer fits gave wrong results on the GPU (fp32 decay-gradient sweep at 128), so none may spill.
+SPILL_LIMIT = {"wkv6_fwd_ws": 0, "wkv6_bwd_a_ws": 0, "wkv6_bwd_b_wsILi0E": 3, "wkv6_bwd_b_wsILi1E": 1, "wkv6_bwd_b_wsILi2E": 1,
+               "wkv_rows": 0}
 
 _lib = None
 
@@ -71,7 +74,7 @@ def build(verbose=False):
             for name, limit in SPILL_LIMIT.items():
                 if name in kernel and int(m.group(1)) > limit:
                     os.remove(LIB_PATH)
-                    raise RuntimeError(f"{kernel}: {m.group(1)} spilled VGPRs (limit {limit}); its asm-loaded registers must stay in registers")
+                    raise RuntimeError(f"{kernel}: {m.group(1)} spilled VGPRs (limit {limit}); see SPILL_LIMIT")
     if verbose and out.strip():
         print(out, flush=True)
     with open(HASH_PATH, "w") as f:

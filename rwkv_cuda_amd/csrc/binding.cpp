@@ -113,7 +113,7 @@ void wkv5_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor
     c10::hip::HIPGuardMasqueradingAsCUDA guard(r.device());
     if (dt == BF) {
         const size_t n = rwkv_wkv5_backward_workspace_bytes(B, T, C, H);
-        TORCH_CHECK(n > 0, "wkv5.backward: bad shape (C must be H*64)");
+        TORCH_CHECK(n > 0, "wkv5.backward: bad shape (C must be a multiple of H, head size at most 128)");
         Tensor ws = scratch(r, n);
         ok(rwkv_wkv5_backward(stream_of(r), B, T, C, H, bp(r), bp(k), bp(v), fp(w), fp(ww), bp(u), bp(gy), bp(gr), bp(gk), bp(gv),
                               bp(gw), bp(gu), ws.data_ptr(), n), "wkv5.backward");
@@ -161,7 +161,7 @@ void wkv6_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor
     chk(gw, BF, B * T * C, "gw"); chk(gu, BF, B * C, "gu");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(r.device());
     const size_t n = rwkv_wkv6_backward_workspace_bytes(B, T, C, H);
-    TORCH_CHECK(n > 0, "wkv6.backward: bad shape (C must be H*64)");
+    TORCH_CHECK(n > 0, "wkv6.backward: bad shape (C must be a multiple of H, head size at most 128)");
     Tensor ws = scratch(r, n);
     ok(rwkv_wkv6_backward(stream_of(r), B, T, C, H, bp(r), bp(k), bp(v), fp(w), bp(u), bp(gy), bp(gr), bp(gk), bp(gv), bp(gw), bp(gu),
                           ws.data_ptr(), n), "wkv6.backward");
@@ -171,7 +171,7 @@ void wkv6_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor
 void wkv6b_forward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor& k, Tensor& v, Tensor& w, Tensor& u, Tensor& s, Tensor& y) {
     const Checker chk{r, "wkv6b.forward"};
     chk(r, BF, B * T * C, "r"); chk(k, BF, B * T * C, "k"); chk(v, BF, B * T * C, "v"); chk(w, BF, B * T * C, "w"); chk(u, BF, C, "u");
-    chk(s, BF, B * C * 64, "s"); chk(y, BF, B * T * C, "y");
+    chk(s, BF, B * C * (C / H), "s"); chk(y, BF, B * T * C, "y");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(r.device());
     ok(rwkv_wkv6state_forward(stream_of(r), B, T, C, H, bp(r), bp(k), bp(v), bp(w), bp(u), bp(s), bp(y)), "wkv6b.forward");
 }
@@ -179,11 +179,11 @@ void wkv6b_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tenso
                     Tensor& gy, Tensor& gr, Tensor& gk, Tensor& gv, Tensor& gw, Tensor& gu, Tensor& gs) {
     const Checker chk{r, "wkv6b.backward"};
     chk(r, BF, B * T * C, "r"); chk(k, BF, B * T * C, "k"); chk(v, BF, B * T * C, "v"); chk(w, BF, B * T * C, "w"); chk(u, BF, C, "u");
-    chk(s, BF, B * C * 64, "s"); chk(gy, BF, B * T * C, "gy"); chk(gr, BF, B * T * C, "gr"); chk(gk, BF, B * T * C, "gk");
-    chk(gv, BF, B * T * C, "gv"); chk(gw, BF, B * T * C, "gw"); chk(gu, BF, B * C, "gu"); chk(gs, BF, B * C * 64, "gs");
+    chk(s, BF, B * C * (C / H), "s"); chk(gy, BF, B * T * C, "gy"); chk(gr, BF, B * T * C, "gr"); chk(gk, BF, B * T * C, "gk");
+    chk(gv, BF, B * T * C, "gv"); chk(gw, BF, B * T * C, "gw"); chk(gu, BF, B * C, "gu"); chk(gs, BF, B * C * (C / H), "gs");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(r.device());
     const size_t n = rwkv_wkv6state_backward_workspace_bytes(B, T, C, H);
-    TORCH_CHECK(n > 0, "wkv6b.backward: bad shape (C must be H*64)");
+    TORCH_CHECK(n > 0, "wkv6b.backward: bad shape (C must be a multiple of H, head size at most 128)");
     Tensor ws = scratch(r, n);
     ok(rwkv_wkv6state_backward(stream_of(r), B, T, C, H, bp(r), bp(k), bp(v), bp(w), bp(u), bp(s), bp(gy), bp(gr), bp(gk), bp(gv),
                                bp(gw), bp(gu), bp(gs), ws.data_ptr(), n), "wkv6b.backward");

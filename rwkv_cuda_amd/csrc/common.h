@@ -120,9 +120,10 @@ extern thread_local int g_last_hip_error;
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-inline int check_ptrs(std::initializer_list<const void*> ps) {
+// need_align: the kernels that will run use 16-byte loads and stores (those for other head sizes than 64 do not)
+inline int check_ptrs(std::initializer_list<const void*> ps, bool need_align = true) {
     for (const void* p : ps) if (p == nullptr) return RWKV_ERR_NULL;
-    for (const void* p : ps) if (!aligned16(p)) return RWKV_ERR_ALIGN;
+    if (need_align) for (const void* p : ps) if (!aligned16(p)) return RWKV_ERR_ALIGN;
     return RWKV_OK;
 }
 

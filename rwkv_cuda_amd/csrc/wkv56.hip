@@ -507,6 +507,190 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
     }
 }
 
+// ----------------------------------------------------------------------------------------------------------------------
+// Head sizes other than 64 (the reference builds its kernels with -D_N_=HEAD_SIZE: wkv5_bf16/run.py:21 ships 128, the
+// self-checks of wkv5/run.py, wkv6/run.py and wkv6_state/run.py use 2, 4 and 8).  One workgroup per (batch, head), one
+// thread per channel of the "row" axis, and that row of the state in registers: thread i keeps S[i][.] in FWD and GV,
+// thread j keeps S[.][j] in GR and GK, so every sum of the recurrence is a private loop and the vectors indexed by the
+// in-register axis are LDS broadcast reads.  Same passes, formulas, rounding points and workspace as the sweeps above; hn
+// (the head size, 1..NP) is a run-time value, NP the padded size the registers are unrolled for.
+constexpr int GTC = 16;          // time steps per staged chunk
+
+// The step loops below are unrolled over a whole state row.  Left alone, the compiler issues all of a row's LDS reads
+// first and the arithmetic afterwards, which keeps three more rows alive in registers (spills at NP = 128).  Passing the
+// running sum and the eight state elements just updated through an empty asm statement with a memory clobber ends the
+// live ranges of a block's operands before the next block's reads are issued.
+DEVINL void row_fence(float& acc, float* s8) {
+    asm volatile("" : "+v"(acc), "+v"(s8[0]), "+v"(s8[1]), "+v"(s8[2]), "+v"(s8[3]), "+v"(s8[4]), "+v"(s8[5]), "+v"(s8[6]), "+v"(s8[7]) : : "memory");
+}
+
+template <int NP> struct SmemRows {
+    float r[GTC][NP], k[GTC][NP], v[GTC][NP], g[GTC][NP], w[GTC][NP], f[GTC][NP], rdr[GTC][NP];
+    float dot[GTC];
+    float u[NP], wh[NP];
+};
+
+template <int NP, int PASS, int WMODE, bool F32>
+__global__ __launch_bounds__(NP < 64 ? 64 : NP) void wkv_rows(const Args a, const int hn) {
+    static_assert(!F32 || WMODE == W_HEAD, "fp32 I/O exists for wkv5 only");
+    constexpr bool REV = (PASS == P_GK || PASS == P_GV);
+    constexpr bool ROW_I = (PASS == P_FWD || PASS == P_GV);     // thread = value channel, registers = key channels
+    constexpr bool DIRECT_GW = F32 && PASS == P_GR;             // as in wkv_sweep: the fp32 op carries Q = dS/dw
+    constexpr bool SCAN_GW = !F32 && PASS == P_GK;
+    __shared__ SmemRows<NP> S;
+
+    const int me = threadIdx.x;
+    const bool lane_ok = me < NP;                               // NP < 64: the rest of the wave idles
+    const bool live = me < hn;
+    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
+    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * hn;
+    const size_t bh = static_cast<size_t>(b) * a.H + h;
+    const bool stateful = a.s0 != nullptr;
+
+    if (lane_ok) {
+        S.u[me] = live ? load1<F32>(a.u, h * hn + me) : 0.f;
+        S.wh[me] = (WMODE == W_HEAD && live) ? static_cast<const float*>(a.w)[h * hn + me] : 1.f;
+    }
+    float St[NP], Q[DIRECT_GW ? NP : 1];
+#pragma unroll
+    for (int o = 0; o < NP; ++o) St[o] = 0.f;
+#pragma unroll
+    for (int o = 0; o < (DIRECT_GW ? NP : 1); ++o) Q[o] = 0.f;
+    if (stateful && live) {
+        if constexpr (PASS == P_FWD) {
+#pragma unroll
+            for (int o = 0; o < NP; ++o) if (o < hn) St[o] = bf2f(a.s0[(bh * hn + me) * hn + o]);
+        } else if constexpr (PASS == P_GR) {
+#pragma unroll
+            for (int o = 0; o < NP; ++o) if (o < hn) St[o] = bf2f(a.s0[(bh * hn + o) * hn + me]);
+        }
+    }
+    const float w_own = (WMODE == W_HEAD && live) ? static_cast<const float*>(a.w)[h * hn + me] : 1.f;
+    float gu_acc = 0.f, gw_acc = 0.f, P = 0.f;
+
+    const int nchunks = (a.T + GTC - 1) / GTC;
+    for (int ci = 0; ci < nchunks; ++ci) {
+        const int c0 = (REV ? nchunks - 1 - ci : ci) * GTC;
+        __syncthreads();                                        // the previous chunk is done with LDS
+        if (lane_ok) {
+#pragma unroll 2
+            for (int t = 0; t < GTC; ++t) {
+                const bool ok = live && (c0 + t) < a.T;         // rows past T and padded channels: no input, no decay
+                const size_t off = base + static_cast<size_t>(c0 + t) * a.C + me;
+                S.r[t][me] = ok ? load1<F32>(a.r, off) : 0.f;
+                S.k[t][me] = ok ? load1<F32>(a.k, off) : 0.f;
+                if constexpr (PASS != P_GV) S.v[t][me] = ok ? load1<F32>(a.v, off) : 0.f;
+                if constexpr (PASS != P_FWD) S.g[t][me] = ok ? load1<F32>(a.gy, off) : 0.f;
+                if constexpr (WMODE != W_HEAD) {
+                    float ew = 0.f;
+                    if (ok) ew = (WMODE == W_RAW) ? -__expf(bf2f(static_cast<const uint16_t*>(a.w)[off])) : static_cast<const float*>(a.w)[off];
+                    S.w[t][me] = ok ? __expf(ew) : 1.0f;
+                    if constexpr (PASS == P_GK) S.f[t][me] = ew < -30.0f ? 0.f : ew;    // see wkv_sweep's commit()
+                } else {
+                    S.w[t][me] = ok ? w_own : 1.0f;
+                }
+                if constexpr (SCAN_GW) S.rdr[t][me] = ok ? a.rdr[off] : 0.f;
+            }
+        }
+        __syncthreads();
+        if (me < GTC) {                                         // the scalar of each step: sum_j u r k, or sum_i v gy
+            float d = 0.f;
+#pragma unroll 4
+            for (int o = 0; o < NP; ++o)
+                d = ROW_I ? fmaf(S.r[me][o] * S.u[o], S.k[me][o], d) : fmaf(S.v[me][o], S.g[me][o], d);
+            S.dot[me] = d;
+        }
+        __syncthreads();
+
+#pragma unroll 1
+        for (int tt = 0; tt < GTC; ++tt) {
+            const int t = REV ? GTC - 1 - tt : tt, tg = c0 + t;
+            const bool ok = live && tg < a.T;
+            const size_t off = base + static_cast<size_t>(tg) * a.C + me;
+            const float dot = S.dot[t];
+            float acc = 0.f, acc2 = 0.f;
+            if constexpr (ROW_I) {
+                const float x = lane_ok ? ((PASS == P_FWD) ? S.v[t][me] : S.g[t][me]) : 0.f;
+#pragma unroll
+                for (int o = 0; o < NP; ++o) {
+                    const float av = (PASS == P_FWD) ? S.r[t][o] : S.k[t][o];
+                    const float bv = (PASS == P_FWD) ? S.k[t][o] : S.r[t][o];
+                    acc = fmaf(av, St[o], acc);
+                    St[o] = fmaf(St[o], S.w[t][o], bv * x);
+                    if (o % 8 == 7) row_fence(acc, &St[o - 7]);
+                }
+                if (ok) store1<F32>(PASS == P_FWD ? a.y : a.gv, off, fmaf(x, dot, acc));
+            } else {
+                const float bl = lane_ok ? ((PASS == P_GR) ? S.k[t][me] : S.r[t][me]) : 0.f;
+                const float wl = lane_ok ? S.w[t][me] : 1.f;
+#pragma unroll
+                for (int o = 0; o < NP; ++o) {
+                    const float av = (PASS == P_GR) ? S.g[t][o] : S.v[t][o];
+                    const float xv = (PASS == P_GR) ? S.v[t][o] : S.g[t][o];
+                    acc = fmaf(av, St[o], acc);
+                    if constexpr (DIRECT_GW) {
+                        acc2 = fmaf(av, Q[o], acc2);
+                        Q[o] = fmaf(Q[o], wl, St[o]);
+                    }
+                    St[o] = fmaf(St[o], wl, xv * bl);
+                    if (o % 8 == 7) {
+                        row_fence(acc, &St[o - 7]);
+                        if constexpr (DIRECT_GW) row_fence(acc2, &Q[o - 7]);
+                    }
+                }
+                const float rr = lane_ok ? S.r[t][me] : 0.f, kk = lane_ok ? S.k[t][me] : 0.f, uu = lane_ok ? S.u[me] : 0.f;
+                if constexpr (PASS == P_GR) {
+                    gu_acc = fmaf(rr * kk, dot, gu_acc);
+                    if constexpr (DIRECT_GW) gw_acc = fmaf(rr, acc2, gw_acc);
+                    if (ok) {
+                        store1<F32>(a.gr, off, fmaf(uu * kk, dot, acc));
+                        if constexpr (!F32) a.rdr[off] = rr * acc;
+                    }
+                } else {
+                    if (ok) store1<F32>(a.gk, off, fmaf(uu * rr, dot, acc));
+                    if constexpr (SCAN_GW) {
+                        float G = P - kk * acc;
+                        if (!stateful && tg == 0) G = 0.f;      // S_0 = 0: exact zero, as the reference leaves it
+                        P = G + (lane_ok ? S.rdr[t][me] : 0.f);
+                        if constexpr (WMODE == W_HEAD) gw_acc += G;
+                        else if (ok) store1<F32>(a.gw, off, S.f[t][me] * G);
+                    }
+                }
+            }
+        }
+    }
+
+    const size_t pc = static_cast<size_t>(b) * a.C + static_cast<size_t>(h) * hn + me;
+    if constexpr (PASS == P_GR) {
+        if (live) {
+            store1<F32>(a.gu, pc, gu_acc);
+            if constexpr (DIRECT_GW) store1<F32>(a.gw, pc, a.ew_head[h * hn + me] * w_own * gw_acc);   // d eew / d w_raw = eew * ew
+        }
+    }
+    if constexpr (PASS == P_GK) {
+        if constexpr (WMODE == W_HEAD && SCAN_GW) {
+            if (live) {
+                const float f = a.ew_head[h * hn + me];
+                store1<F32>(a.gw, pc, (f < -30.0f ? 0.f : f) * gw_acc);
+            }
+        }
+        if (a.gs != nullptr && live) {
+#pragma unroll
+            for (int o = 0; o < NP; ++o) if (o < hn) a.gs[(bh * hn + o) * hn + me] = f2bf(St[o]);
+        }
+    }
+}
+
+constexpr int MAX_HEAD = 128;
+
+template <int PASS, int WMODE, bool F32> void launch_rows(hipStream_t st, int B, const Args& a) {
+    const int hn = a.C / a.H;
+    if (hn <= 8) hipLaunchKernelGGL((wkv_rows<8, PASS, WMODE, F32>), dim3(B * a.H), dim3(64), 0, st, a, hn);
+    else if (hn <= 32) hipLaunchKernelGGL((wkv_rows<32, PASS, WMODE, F32>), dim3(B * a.H), dim3(64), 0, st, a, hn);
+    else if (hn <= 64) hipLaunchKernelGGL((wkv_rows<64, PASS, WMODE, F32>), dim3(B * a.H), dim3(64), 0, st, a, hn);
+    else if constexpr (!F32) hipLaunchKernelGGL((wkv_rows<128, PASS, WMODE, F32>), dim3(B * a.H), dim3(128), 0, st, a, hn);
+}
+
 // The chunked matrix-core kernels serve all three decay conventions; the sequential sweeps remain as the second algorithm.
 // They address one batch row with 32-bit byte offsets (up to 4 bytes per element), so rows of 2^30 elements or more
 // take the sweeps.
@@ -516,6 +700,10 @@ bool use_chunked(const Args& a, unsigned flags) { return !(flags & RWKV_FLAG_SWE
 unsigned passes_of(unsigned flags) { return (flags & RWKV_PASS_ALL) ? (flags & RWKV_PASS_ALL) : RWKV_PASS_ALL; }
 
 template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a, unsigned flags) {
+    if (a.C != a.H * N) {                              // another head size: the row-per-thread kernels
+        launch_rows<P_FWD, WMODE, false>(st, B, a);
+        return launch_status();
+    }
     if (use_chunked(a, flags))
         return launch_wkv6_fwd_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, a.w, a.u, a.s0, a.y);
     hipLaunchKernelGGL((wkv_sweep<P_FWD, WMODE>), dim3(B * a.H), dim3(NT), 0, st, a);
@@ -525,8 +713,14 @@ template <int WMODE> int launch_fwd(hipStream_t st, int B, const Args& a, unsign
 // GR and GV are independent; GK consumes GR's workspace.  All three run on `st` in order.
 // `passes` is a bit mask (RWKV_PASS_*) so that a profiler can time one kernel at a time.
 template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a, unsigned flags) {
-    const bool chunked = use_chunked(a, flags);
     const unsigned passes = passes_of(flags);
+    if (a.C != a.H * N) {                              // another head size: GR and GV are independent, GK reads GR's workspace
+        if (passes & RWKV_PASS_GR) launch_rows<P_GR, WMODE, false>(st, B, a);
+        if (passes & RWKV_PASS_GV) launch_rows<P_GV, WMODE, false>(st, B, a);
+        if (passes & RWKV_PASS_GK) launch_rows<P_GK, WMODE, false>(st, B, a);
+        return launch_status();
+    }
+    const bool chunked = use_chunked(a, flags);
     const void* w = (WMODE == W_HEAD) ? static_cast<const void*>(a.ew_head) : a.w;   // wkv5: the log decay
     if ((passes & RWKV_PASS_GR) && chunked) {
         if (int e = launch_wkv6_bwd_a_chunk(st, WMODE, B, a.T, a.C, a.H, a.r, a.k, a.v, w, a.u, a.s0, a.gy, a.gr, a.gu, a.rdr)) return e;
@@ -542,9 +736,13 @@ template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a, unsign
     return launch_status();
 }
 
-int check_dims(int B, int T, int C, int H) {
+// head size 64 takes the kernels this file and wkv6_*.hip are written for, any other size up to 128 the row-per-thread
+// kernels (wkv_rows); wkv5a exists for 64 only, and the fp32 wkv5 op up to 64 (its decay-gradient sweep keeps two state
+// rows per thread, which at 128 no longer fit the register file)
+int check_dims(int B, int T, int C, int H, bool only64 = false, int max_head = MAX_HEAD) {
     if (B <= 0 || T <= 0 || C <= 0 || H <= 0) return RWKV_ERR_SHAPE;
-    if (C != H * N) return RWKV_ERR_SHAPE;
+    if (C % H != 0 || C / H > max_head) return RWKV_ERR_SHAPE;
+    if (only64 && C != H * N) return RWKV_ERR_SHAPE;
     if (static_cast<long long>(B) * H > 0x7fffffffLL) return RWKV_ERR_SHAPE;
     return RWKV_OK;
 }
@@ -592,7 +790,7 @@ extern "C" {
 int rwkv_wkv5_forward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                       const rwkv_bf16* v, const float* eew, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, eew, u, y})) return e;
+    if (int e = check_ptrs({r, k, v, eew, u, y}, C == H * N)) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = eew; a.u = u; a.y = y;
     return launch_fwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a, flags);
@@ -605,7 +803,7 @@ int rwkv_wkv5_backward_ex(void* stream, int B, int T, int C, int H, const rwkv_b
                        const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw,
                        rwkv_bf16* gu, void* workspace, size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu})) return e;
+    if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu}, C == H * N)) return e;
     if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = eew; a.ew_head = ew; a.u = u; a.gy = gy;
@@ -621,25 +819,32 @@ uint16_t* out_elems(float* p) { return reinterpret_cast<uint16_t*>(p); }
 
 int rwkv_wkv5f32_forward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
                          const float* eew, const float* u, float* y) {
-    if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, eew, u, y})) return e;
+    if (int e = check_dims(B, T, C, H, false, N)) return e;
+    if (int e = check_ptrs({r, k, v, eew, u, y}, C == H * N)) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew; a.u = as_elems(u);
     a.y = out_elems(y);
-    hipLaunchKernelGGL((wkv_sweep<P_FWD, W_HEAD, true>), dim3(B * H), dim3(NT), 0, static_cast<hipStream_t>(stream), a);
+    if (C != H * N) launch_rows<P_FWD, W_HEAD, true>(static_cast<hipStream_t>(stream), B, a);
+    else hipLaunchKernelGGL((wkv_sweep<P_FWD, W_HEAD, true>), dim3(B * H), dim3(NT), 0, static_cast<hipStream_t>(stream), a);
     return launch_status();
 }
 
 int rwkv_wkv5f32_backward_ex(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
                           const float* eew, const float* ew, const float* u, const float* gy, float* gr, float* gk,
                           float* gv, float* gw, float* gu, unsigned flags) {
-    if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu})) return e;
+    if (int e = check_dims(B, T, C, H, false, N)) return e;
+    if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu}, C == H * N)) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew; a.ew_head = ew;
     a.u = as_elems(u); a.gy = as_elems(gy); a.gr = out_elems(gr); a.gk = out_elems(gk); a.gv = out_elems(gv);
     a.gw = out_elems(gw); a.gu = out_elems(gu);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (C != H * N) {
+        if (passes_of(flags) & RWKV_PASS_GR) launch_rows<P_GR, W_HEAD, true>(st, B, a);
+        if (passes_of(flags) & RWKV_PASS_GV) launch_rows<P_GV, W_HEAD, true>(st, B, a);
+        if (passes_of(flags) & RWKV_PASS_GK) launch_rows<P_GK, W_HEAD, true>(st, B, a);
+        return launch_status();
+    }
     // three independent sweeps: gr + gu + gw, gv, gk
     if (passes_of(flags) & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
     if (passes_of(flags) & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, W_HEAD, true>), dim3(B * H), dim3(NT), 0, st, a);
@@ -650,7 +855,7 @@ int rwkv_wkv5f32_backward_ex(void* stream, int B, int T, int C, int H, const flo
 // ---- wkv5a: two-sided decay and bonus, fp32, on the same sweeps
 int rwkv_wkv5a_forward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
                        const float* eew1, const float* u1, const float* eew2, const float* u2, float* y) {
-    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_dims(B, T, C, H, true)) return e;
     if (int e = check_ptrs({r, k, v, eew1, u1, eew2, u2, y})) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew1; a.u = as_elems(u1);
@@ -663,7 +868,7 @@ int rwkv_wkv5a_backward_ex(void* stream, int B, int T, int C, int H, const float
                         const float* eew1, const float* ew1, const float* u1, const float* eew2, const float* ew2,
                         const float* u2, const float* gy, float* gr, float* gk, float* gv, float* gw1, float* gu1,
                         float* gw2, float* gu2, unsigned flags) {
-    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_dims(B, T, C, H, true)) return e;
     if (int e = check_ptrs({r, k, v, eew1, ew1, u1, eew2, ew2, u2, gy, gr, gk, gv, gw1, gu1, gw2, gu2})) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew1; a.ew_head = ew1;
@@ -681,7 +886,7 @@ int rwkv_wkv5a_backward_ex(void* stream, int B, int T, int C, int H, const float
 int rwkv_wkv6_forward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                       const rwkv_bf16* v, const float* ew, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, ew, u, y})) return e;
+    if (int e = check_ptrs({r, k, v, ew, u, y}, C == H * N)) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.y = y;
     return launch_fwd<W_EW>(static_cast<hipStream_t>(stream), B, a, flags);
@@ -694,7 +899,7 @@ int rwkv_wkv6_backward_ex(void* stream, int B, int T, int C, int H, const rwkv_b
                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                        void* workspace, size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, ew, u, gy, gr, gk, gv, gw, gu})) return e;
+    if (int e = check_ptrs({r, k, v, ew, u, gy, gr, gk, gv, gw, gu}, C == H * N)) return e;
     if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.gy = gy;
@@ -705,7 +910,7 @@ int rwkv_wkv6_backward_ex(void* stream, int B, int T, int C, int H, const rwkv_b
 int rwkv_wkv6raw_forward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                          const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, w, u, y})) return e;
+    if (int e = check_ptrs({r, k, v, w, u, y}, C == H * N)) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.y = y;
     return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, flags);
@@ -716,7 +921,7 @@ int rwkv_wkv6raw_backward_ex(void* stream, int B, int T, int C, int H, const rwk
                           rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                           void* workspace, size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, w, u, gy, gr, gk, gv, gw, gu})) return e;
+    if (int e = check_ptrs({r, k, v, w, u, gy, gr, gk, gv, gw, gu}, C == H * N)) return e;
     if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.gy = gy;
@@ -728,7 +933,7 @@ int rwkv_wkv6state_forward_ex(void* stream, int B, int T, int C, int H, const rw
                            const rwkv_bf16* v, const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s,
                            rwkv_bf16* y, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, w, u, s, y})) return e;
+    if (int e = check_ptrs({r, k, v, w, u, s, y}, C == H * N)) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.y = y;
     return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, flags);
@@ -741,7 +946,7 @@ int rwkv_wkv6state_backward_ex(void* stream, int B, int T, int C, int H, const r
                             const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw,
                             rwkv_bf16* gu, rwkv_bf16* gs, void* workspace, size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, w, u, s, gy, gr, gk, gv, gw, gu, gs})) return e;
+    if (int e = check_ptrs({r, k, v, w, u, s, gy, gr, gk, gv, gw, gu, gs}, C == H * N)) return e;
     if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.gy = gy;
@@ -754,7 +959,7 @@ int rwkv_wkv6state_backward_ex(void* stream, int B, int T, int C, int H, const r
 int rwkv_wkv5raw_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                          const rwkv_bf16* w_raw, const rwkv_bf16* u, rwkv_bf16* y, float* decay, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, w_raw, u, y, decay})) return e;
+    if (int e = check_ptrs({r, k, v, w_raw, u, y, decay}, C == H * N)) return e;
     hipLaunchKernelGGL(wkv5_decay_transform, dim3((C + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), C, w_raw, decay);
     return rwkv_wkv5_forward_ex(stream, B, T, C, H, r, k, v, decay, u, y, flags);
 }
@@ -768,7 +973,7 @@ int rwkv_wkv5raw_backward(void* stream, int B, int T, int C, int H, const rwkv_b
                           const float* decay, const rwkv_bf16* u, const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk,
                           rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu, void* workspace, size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({decay, gw, gu})) return e;
+    if (int e = check_ptrs({decay, gw, gu}, C == H * N)) return e;
     if (workspace == nullptr || workspace_bytes < rwkv_wkv5raw_backward_workspace_bytes(B, T, C, H) || !aligned16(workspace))
         return RWKV_ERR_WORKSPACE;
     const size_t n = round16(ws_bytes(B, T, C, H));
@@ -789,7 +994,7 @@ int rwkv_wkv6f_backward(void* stream, int B, int T, int C, int H, const rwkv_bf1
                         rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu, rwkv_bf16* gs, void* workspace,
                         size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({gu})) return e;
+    if (int e = check_ptrs({gu}, C == H * N)) return e;
     if ((s == nullptr) != (gs == nullptr)) return RWKV_ERR_NULL;           // state and its gradient come together
     if (workspace == nullptr || workspace_bytes < rwkv_wkv6f_backward_workspace_bytes(B, T, C, H) || !aligned16(workspace))
         return RWKV_ERR_WORKSPACE;

@@ -4,7 +4,8 @@ import torch
 
 from ._call import call, check_tensors, require
 
-HEAD_SIZE = 64
+HEAD_SIZE = 64          # the size the matrix-core kernels are written for; any size up to MAX_HEAD_SIZE runs
+MAX_HEAD_SIZE = 128
 
 
 class WKV_5(torch.autograd.Function):
@@ -16,7 +17,7 @@ class WKV_5(torch.autograd.Function):
     def forward(ctx, B, T, C, H, r, k, v, w, u):
         with torch.no_grad():
             dev = check_tensors((r, k, v, w, u), torch.float32, "rkvwu")
-            require(HEAD_SIZE == C // H and C == H * HEAD_SIZE, "head size must be 64")
+            require(C % H == 0 and C // H <= MAX_HEAD_SIZE, "C must be a multiple of H with a head size of at most 128")
             require(r.numel() == B * T * C and w.numel() == C and u.numel() == C, "shape mismatch")
             ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
             ctx.wshape, ctx.ushape = w.shape, u.shape

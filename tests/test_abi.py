@@ -37,9 +37,9 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     p = 0x1000  # never dereferenced: every call below fails validation first
     # shapes
     assert lib.rwkv_wkv6_forward(None, 0, 8, 64, 1, p, p, p, p, p, p) == -1
-    assert lib.rwkv_wkv6_forward(None, 1, 8, 96, 1, p, p, p, p, p, p) == -1          # C != H*64
-    assert lib.rwkv_wkv5_forward(None, 1, 8, 128, 1, p, p, p, p, p, p) == -1
-    assert lib.rwkv_wkv5f32_forward(None, 1, 8, 128, 1, p, p, p, p, p, p) == -1
+    assert lib.rwkv_wkv6_forward(None, 1, 8, 97, 2, p, p, p, p, p, p) == -1          # C not a multiple of H
+    assert lib.rwkv_wkv5_forward(None, 1, 8, 129, 1, p, p, p, p, p, p) == -1         # head size above 128
+    assert lib.rwkv_wkv5f32_forward(None, 1, 8, 258, 2, p, p, p, p, p, p) == -1
     assert lib.rwkv7_statepassing_forward(None, 1, 24, 1, *([p] * 11)) == -1         # T % 16
     assert lib.rwkv7_state_forward(None, 1, 24, 1, *([p] * 10)) == -1
     assert lib.rwkv7_forward(None, 1, 16, 1, *([p] * 8), None) == -2
@@ -61,7 +61,7 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert need == 2 * 8 * 128 * 4 + 2 * 2 * 1 * 64 * 64 * 4      # r*dr' and one stored state per (b,h) for the single chunk
     assert lib.rwkv_wkv6state_backward(None, 2, 8, 128, 2, *([p] * 13), None, 0) == -4
     assert lib.rwkv_wkv6state_backward(None, 2, 8, 128, 2, *([p] * 13), p, need - 1) == -4
-    assert lib.rwkv_wkv6_backward_workspace_bytes(1, 1, 96, 1) == 0
+    assert lib.rwkv_wkv6_backward_workspace_bytes(1, 1, 129, 1) == 0
     assert lib.rwkv_wkv5f32_backward(None, 2, 8, 128, 2, *([p] * 11), None) == -2
     assert lib.rwkv_wkv5a_forward(None, 1, 8, 96, 1, *([p] * 8)) == -1
     assert lib.rwkv_wkv5a_backward(None, 2, 8, 128, 2, *([p] * 16), p + 4) == -3
@@ -70,7 +70,7 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.rwkv_wkv4_backward_noalloc(None, 4, 1024, 768, *([p] * 9)) == -4
     # per-call flags: same validation as the plain entry points
     assert lib.rwkv_wkv6state_backward_ex(None, 2, 8, 128, 2, *([p] * 13), None, 0, 0x100) == -4
-    assert lib.rwkv_wkv6raw_forward_ex(None, 1, 8, 96, 1, p, p, p, p, p, p, 0) == -1
+    assert lib.rwkv_wkv6raw_forward_ex(None, 1, 8, 130, 1, p, p, p, p, p, p, 0) == -1
     with pytest.raises(_lib.RwkvHipError):
         _lib.check(-1)
 

@@ -1,0 +1,146 @@
+"""GPU: head sizes other than 64.
+
+The reference compiles its kernels with -D_N_=HEAD_SIZE: wkv5_bf16/run.py:21 ships 128, the self-checks of
+wkv5/run.py:366, wkv6/run.py:35 and wkv6_state/run.py:39 use 2 and 4, wkv5a/run.py:60 lists 17.  Here head size 64 takes
+the matrix-core kernels and every other size up to 128 the row-per-thread kernels of csrc/wkv56.hip (`wkv_rows`); the bar
+is the one of the 64-wide kernels: fp64 oracle, bf16 ops no worse than the reference kernel's arithmetic, fp32 ops 1e-5."""
+import pytest
+import torch
+
+from oracle import wkv56 as O
+from oracle import err_ratio
+from rwkv_cuda_amd import synth, wkv5_bf16, wkv6, wkv6_state
+from rwkv_cuda_amd._call import call
+from _gpu_util import DEV, assert_no_worse, garbage
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+SIZES = [2, 4, 8, 17, 32, 48, 128]
+
+
+@pytest.mark.parametrize("N", SIZES)
+def test_wkv5_bf16_any_head_size(lib, N):
+    B, T, H = 2, 37, 3
+    C = H * N
+    print(f"\nwkv5 bf16 N={N} B={B} T={T} H={H}", flush=True)
+    r, k, v, w, u, gy = synth.wkv5_inputs(B, T, C, H, seed=200 + N)
+    ref = O.wkv5_grads(B, T, C, H, r, k, v, w, u, gy)
+    emu = O.emulate_wkv5_bf16(B, T, C, H, r, k, v, w, u, gy)
+    t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u)]
+    y = wkv5_bf16.RUN_CUDA(B, T, C, H, *t)
+    y.backward(gy.to(DEV))
+    torch.cuda.synchronize()
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y] + [x.grad for x in t]):
+        assert_no_worse(f"wkv5 N={N} {name}", a, e.reshape(a.shape), g.reshape(a.shape))
+
+
+@pytest.mark.parametrize("state", [False, True])
+@pytest.mark.parametrize("N", SIZES)
+def test_wkv6_any_head_size(lib, N, state):
+    B, T, H = 2, 41, 2
+    C = H * N
+    print(f"\nwkv6 N={N} state={state} B={B} T={T} H={H}", flush=True)
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=300 + N, state=state)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    ins = (r, k, v, w, u, s0) if state else (r, k, v, w, u)
+    t = [x.to(DEV).requires_grad_(True) for x in ins]
+    y = (wkv6_state if state else wkv6).RUN_CUDA(B, T, C, H, *t)
+    y.backward(gy.to(DEV))
+    torch.cuda.synchronize()
+    names = ["y", "gr", "gk", "gv", "gw", "gu"] + (["gs"] if state else [])
+    for name, a, e, g in zip(names, ref, emu, [y] + [x.grad for x in t]):
+        assert_no_worse(f"wkv6 N={N} {name}", a, e.reshape(a.shape), g.reshape(a.shape))
+    if not state:
+        assert float(t[3].grad[:, 0].abs().max()) == 0.0          # no state before the first token: an exact zero
+
+
+@pytest.mark.parametrize("N", [2, 17, 128])
+def test_wkv6_fp32_ew_interface_any_head_size(lib, N):
+    """The reference's own signature (fp32 ew = -exp(w), per-batch gu; wkv6/cuda/wkv6_op.cpp:5-6) with garbage-filled outputs."""
+    B, T, H = 2, 19, 2
+    C = H * N
+    r, k, v, w, u, gy, _ = synth.wkv6_inputs(B, T, C, H, seed=400 + N)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, per_batch=True)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy)
+    d = [x.to(DEV) for x in (r, k, v, w, u, gy)]
+    ew = (-torch.exp(d[3].float())).contiguous()
+    y, gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(5))
+    gu = garbage((B, C), BF)
+    n = lib.rwkv_wkv6_backward_workspace_bytes(B, T, C, H)
+    assert n >= B * T * C * 4
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+    call("rwkv_wkv6_forward", d[0].device, B, T, C, H, d[0], d[1], d[2], ew, d[4], y)
+    call("rwkv_wkv6_backward", d[0].device, B, T, C, H, d[0], d[1], d[2], ew, d[4], d[5], gr, gk, gv, gw, gu, ws, n)
+    torch.cuda.synchronize()
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw"], ref, emu, [y, gr, gk, gv, gw]):
+        assert_no_worse(f"wkv6 ew N={N} {name}", a, e, g)
+    gu_ref = ref[5]
+    e = err_ratio(gu_ref.sum(0).reshape(-1), gu.double().cpu().sum(0).reshape(-1))
+    print(f"  gu (summed over the batch): {e:.3e}", flush=True)
+    assert e < 6e-3
+
+
+@pytest.mark.parametrize("N", [2, 4, 17, 48])
+def test_wkv5_fp32_any_head_size(lib, N):
+    B, T, H = 2, 53, 2
+    C = H * N
+    g = torch.Generator().manual_seed(500 + N)
+    rnd = lambda *s: torch.rand(*s, generator=g) * 2 - 1
+    r, k, v, w, u, gy = rnd(B, T, C), rnd(B, T, C), rnd(B, T, C), rnd(C), rnd(C), rnd(B, T, C)
+    ref = O.wkv5_grads(B, T, C, H, r, k, v, w, u, gy, per_batch=True)
+    ew = -torch.exp(w)
+    d = [x.to(DEV) for x in (r, k, v, torch.exp(ew), ew, u, gy)]
+    f32 = torch.float32
+    y = garbage((B, T, C), f32)
+    call("rwkv_wkv5f32_forward", d[0].device, B, T, C, H, d[0], d[1], d[2], d[3], d[5], y)
+    gr, gk, gv = (garbage((B, T, C), f32) for _ in range(3))
+    gw, gu = garbage((B, C), f32), garbage((B, C), f32)
+    call("rwkv_wkv5f32_backward", d[0].device, B, T, C, H, *d, gr, gk, gv, gw, gu)
+    torch.cuda.synchronize()
+    for name, a, got in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, [y, gr, gk, gv, gw, gu]):
+        e = err_ratio(a, got.double().cpu().reshape(a.shape))
+        print(f"  wkv5 fp32 N={N} {name}: {e:.3e}", flush=True)
+        assert e <= 1e-5, (name, e)
+
+
+def test_wkv5_bf16_reference_default_shape_sampled_heads(lib):
+    """wkv5_bf16/run.py:17-22 as shipped: B8 T4096 C4096, head size 128.  Two heads against the fp64 oracle."""
+    B, T, N = 8, 4096, 128
+    C, H = 4096, 32
+    r, k, v, w, u, gy = synth.wkv5_inputs(B, T, C, H, seed=44)
+    t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u)]
+    print("\nwkv5 bf16 head size 128, full size launch", flush=True)
+    y = wkv5_bf16.RUN_CUDA(B, T, C, H, *t)
+    y.backward(gy.to(DEV))
+    torch.cuda.synchronize()
+    got_all = [y.detach()] + [x.grad for x in t]
+    for h in (3, 29):
+        print(f" head {h}", flush=True)
+        sl = slice(h * N, (h + 1) * N)
+        rr, kk, vv, gg = (x[:, :, sl].contiguous().double() for x in (r, k, v, gy))
+        uu, wr = u[h:h + 1].double(), w[h:h + 1].double()
+        dec = O.wkv6_decay(wr).reshape(1, 1, N).expand(B, T, N).contiguous()
+        yref, _ = O.wkv_recurrent(B, T, N, 1, rr, kk, vv, dec, uu)
+        gr, gk, gv, G, gu, _ = O.wkv_backward_hand(B, T, N, 1, rr, kk, vv, dec, uu, gg)
+        gw = (-torch.exp(wr) * G.sum((0, 1)).reshape(1, N))
+        ref = [yref, gr, gk, gv, gw, gu.sum(0)]
+        got = [got_all[0][:, :, sl], got_all[1][:, :, sl], got_all[2][:, :, sl], got_all[3][:, :, sl],
+               got_all[4][h:h + 1], got_all[5][h:h + 1]]
+        for name, a, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, got):
+            e = err_ratio(a, g.double().cpu())
+            print(f"  {name}: {e:.3e}", flush=True)
+            assert e < (4e-3 if name in ("gu", "gw") else 2.5e-3), (name, e)
+
+
+def test_head_size_limits(lib):
+    x = torch.zeros(2 * 8 * 258, device=DEV, dtype=BF)
+    f = torch.zeros(2 * 258, device=DEV)
+    # 129 > 128, and C not a multiple of H
+    assert lib.rwkv_wkv6raw_forward(None, 2, 8, 129, 1, *(x.data_ptr(),) * 6) == -1
+    assert lib.rwkv_wkv6raw_forward(None, 2, 8, 130, 4, *(x.data_ptr(),) * 6) == -1
+    # the fp32 op: up to 64 (wkv5/run.py benchmarks 64 and checks with 2)
+    assert lib.rwkv_wkv5f32_forward(None, 2, 8, 128, 1, *(f.data_ptr(),) * 6) == -1
+    # the two-sided op exists for head size 64 only, as built here
+    assert lib.rwkv_wkv5a_forward(None, 2, 8, 32, 1, x.data_ptr(), x.data_ptr(), x.data_ptr(), f.data_ptr(), f.data_ptr(),
+                                  f.data_ptr(), f.data_ptr(), x.data_ptr()) == -1
