@@ -144,11 +144,13 @@ def make_wkv6(dev, state):
     return step, tok, kernels, cfg, cpu_baseline, 28 * C * tok
 
 
-def make_wkv5(dev):
+def make_wkv5(dev, H=32, N=64):
+    """N = 64: the matrix-core kernels at B8 T4096 C2048; N = 128: wkv5_bf16/run.py:17-22 as shipped (B8 T4096 C4096),
+    which runs on the one-thread-per-state-row kernels."""
     from rwkv_cuda_amd import _lib, synth
     from rwkv_cuda_amd._call import call
     lib = _lib.load()
-    B, T, H, N = 8, 4096, 32, 64
+    B, T = 8, 4096
     C = H * N
     bf = torch.bfloat16
     r, k, v, w, u, gy = (x.to(dev) for x in synth.wkv5_inputs(B, T, C, H, seed=42))
@@ -173,9 +175,13 @@ def make_wkv5(dev):
             call("rwkv_wkv5_backward_ex", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes, mask | FLAGS)
         return run
 
-    kernels = [("wkv6_fwd_ws<head decay>", lambda: call("rwkv_wkv5_forward_ex", dev, B, T, C, H, r, k, v, eew, u, y, FLAGS), 8 * C * tok),
-               ("wkv6_bwd_a_ws<head decay>", bwd(1), 10 * C * tok),           # r k v gy -> gr (+ fp32 workspace)
-               ("wkv6_bwd_b_ws<head decay>", bwd(4), 12 * C * tok)]           # r k v gy -> gk gv
+    if N == 64:
+        kernels = [("wkv6_fwd_ws<head decay>", lambda: call("rwkv_wkv5_forward_ex", dev, B, T, C, H, r, k, v, eew, u, y, FLAGS), 8 * C * tok),
+                   ("wkv6_bwd_a_ws<head decay>", bwd(1), 10 * C * tok),           # r k v gy -> gr (+ fp32 workspace)
+                   ("wkv6_bwd_b_ws<head decay>", bwd(4), 12 * C * tok)]           # r k v gy -> gk gv
+    else:
+        kernels = [("wkv_rows<FWD>", lambda: call("rwkv_wkv5_forward_ex", dev, B, T, C, H, r, k, v, eew, u, y, FLAGS), 8 * C * tok),
+                   ("wkv_rows<GR>", bwd(1), 10 * C * tok), ("wkv_rows<GV>", bwd(2), 8 * C * tok), ("wkv_rows<GK>", bwd(4), 10 * C * tok)]
 
     def cpu_baseline(t_cpu=256):
         from oracle import wkv56 as O
@@ -424,6 +430,7 @@ WORKLOADS = {
     "wkv6": lambda dev: make_wkv6(dev, False),
     "wkv6_state": lambda dev: make_wkv6(dev, True),
     "wkv5": make_wkv5,
+    "wkv5_n128": lambda dev: make_wkv5(dev, H=32, N=128),
     "wkv5_fp32": make_wkv5_fp32,
     "wkv5a": make_wkv5a,
     "rwkv7": make_rwkv7,
@@ -431,7 +438,7 @@ WORKLOADS = {
     "wkv4": make_wkv4,
     "timex": make_timex,
 }
-DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "timex": "f32"}
+DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_n128": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "timex": "f32"}
 
 
 def main():

@@ -509,136 +509,194 @@ __global__ __launch_bounds__(NT) void wkv_sweep(const Args a) {
 
 // ----------------------------------------------------------------------------------------------------------------------
 // Head sizes other than 64 (the reference builds its kernels with -D_N_=HEAD_SIZE: wkv5_bf16/run.py:21 ships 128, the
-// self-checks of wkv5/run.py, wkv6/run.py and wkv6_state/run.py use 2, 4 and 8).  One workgroup per (batch, head), one
-// thread per channel of the "row" axis, and that row of the state in registers: thread i keeps S[i][.] in FWD and GV,
-// thread j keeps S[.][j] in GR and GK, so every sum of the recurrence is a private loop and the vectors indexed by the
-// in-register axis are LDS broadcast reads.  Same passes, formulas, rounding points and workspace as the sweeps above; hn
-// (the head size, 1..NP) is a run-time value, NP the padded size the registers are unrolled for.
+// self-checks of wkv5/run.py, wkv6/run.py and wkv6_state/run.py use 2, 4 and 8).  One workgroup per (batch, head).  A row
+// of the state (S[i][.] in FWD and GV, S[.][j] in GR and GK) is kept in the registers of PARTS adjacent lanes, EL elements
+// each, so every sum of the recurrence is a private loop over LDS-broadcast vectors plus one or two cross-lane adds.
+// Same passes, formulas, rounding points and workspace as the sweeps above; hn (the head size, 1..NP) is a run-time
+// value, NP the padded size the registers are unrolled for.
 constexpr int GTC = 16;          // time steps per staged chunk
 
-// The step loops below are unrolled over a whole state row.  Left alone, the compiler issues all of a row's LDS reads
-// first and the arithmetic afterwards, which keeps three more rows alive in registers (spills at NP = 128).  Passing the
+// The step loops below are unrolled over a thread's part of a state row.  Left alone, the compiler issues all of the LDS
+// reads first and the arithmetic afterwards, which keeps three more copies of the row alive in registers.  Passing the
 // running sum and the eight state elements just updated through an empty asm statement with a memory clobber ends the
 // live ranges of a block's operands before the next block's reads are issued.
 DEVINL void row_fence(float& acc, float* s8) {
     asm volatile("" : "+v"(acc), "+v"(s8[0]), "+v"(s8[1]), "+v"(s8[2]), "+v"(s8[3]), "+v"(s8[4]), "+v"(s8[5]), "+v"(s8[6]), "+v"(s8[7]) : : "memory");
 }
 
-template <int NP> struct SmemRows {
-    float r[GTC][NP], k[GTC][NP], v[GTC][NP], g[GTC][NP], w[GTC][NP], f[GTC][NP], rdr[GTC][NP];
-    float dot[GTC];
-    float u[NP], wh[NP];
+template <int NP, int PARTS> struct RowGeom {
+    static constexpr int EL = NP / PARTS;                    // state elements per thread
+    static constexpr int SLOT = EL + (PARTS > 1 ? 4 : 0);    // a part's slice of a staged vector; the 16-byte skew keeps the
+    static constexpr int LEN = PARTS * SLOT;                 // PARTS broadcast reads of a wave on different banks
+    static constexpr int NTHREADS = NP * PARTS < 64 ? 64 : NP * PARTS;
+    static_assert(EL % 8 == 0, "row_fence takes blocks of eight");
+    static __device__ __forceinline__ int at(int n) { return (n / EL) * SLOT + n % EL; }   // where channel n of a vector sits
 };
 
-template <int NP, int PASS, int WMODE, bool F32>
-__global__ __launch_bounds__(NP < 64 ? 64 : NP) void wkv_rows(const Args a, const int hn) {
+template <int NP, int PARTS> struct SmemRows {
+    static constexpr int LEN = RowGeom<NP, PARTS>::LEN;
+    alignas(16) float r[GTC][LEN], k[GTC][LEN], v[GTC][LEN], g[GTC][LEN], w[GTC][LEN], f[GTC][LEN], rdr[GTC][LEN];
+    float dot[GTC];
+    alignas(16) float u[LEN];
+};
+
+// sum over the PARTS adjacent lanes that share a row; every one of them gets the total
+template <int PARTS> DEVINL float parts_sum(float x) {
+    if constexpr (PARTS >= 2) x += __shfl_xor(x, 1, 64);
+    if constexpr (PARTS >= 4) x += __shfl_xor(x, 2, 64);
+    static_assert(PARTS == 1 || PARTS == 2 || PARTS == 4, "adjacent lanes of one quad");
+    return x;
+}
+
+template <int NP, int PARTS, int PASS, int WMODE, bool F32>
+__global__ __launch_bounds__((RowGeom<NP, PARTS>::NTHREADS)) void wkv_rows(const Args a, const int hn) {
     static_assert(!F32 || WMODE == W_HEAD, "fp32 I/O exists for wkv5 only");
+    using G = RowGeom<NP, PARTS>;
+    constexpr int EL = G::EL, SLOT = G::SLOT;
     constexpr bool REV = (PASS == P_GK || PASS == P_GV);
-    constexpr bool ROW_I = (PASS == P_FWD || PASS == P_GV);     // thread = value channel, registers = key channels
+    constexpr bool ROW_I = (PASS == P_FWD || PASS == P_GV);     // row = value channel, registers = key channels
     constexpr bool DIRECT_GW = F32 && PASS == P_GR;             // as in wkv_sweep: the fp32 op carries Q = dS/dw
     constexpr bool SCAN_GW = !F32 && PASS == P_GK;
-    __shared__ SmemRows<NP> S;
+    __shared__ SmemRows<NP, PARTS> S;
 
-    const int me = threadIdx.x;
-    const bool lane_ok = me < NP;                               // NP < 64: the rest of the wave idles
-    const bool live = me < hn;
+    const int tid = threadIdx.x;
+    const int row = tid / PARTS, part = tid % PARTS;            // threads beyond NP * PARTS (NP * PARTS < 64) only idle
+    const bool in_rows = row < NP;
+    const int rrow = in_rows ? row : 0;                         // a valid row to read for idle threads
+    const bool live = in_rows && row < hn;                      // this thread's row is a channel of the head
+    const bool writer = live && part == 0;
+    const int own = G::at(rrow);                                // where this row's element of a staged vector sits
+    const int sl = part * SLOT;                                 // where this thread's slice of a staged vector starts
+    const int o0 = part * EL;                                   // first in-register channel of this thread
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
     const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * hn;
     const size_t bh = static_cast<size_t>(b) * a.H + h;
     const bool stateful = a.s0 != nullptr;
+    // the staging role: thread (channel cn, group sg) moves SPT steps of channel cn in every chunk
+    constexpr int SG = G::NTHREADS / NP, SPT = GTC / SG;
+    static_assert(SG * NP == G::NTHREADS && SPT * SG == GTC && SPT >= 1, "the workgroup tiles a chunk");
+    const int cn = tid % NP, t_first = (tid / NP) * SPT;
+    const bool chan = cn < hn;
+    const int cat = G::at(cn);
 
-    if (lane_ok) {
-        S.u[me] = live ? load1<F32>(a.u, h * hn + me) : 0.f;
-        S.wh[me] = (WMODE == W_HEAD && live) ? static_cast<const float*>(a.w)[h * hn + me] : 1.f;
-    }
-    float St[NP], Q[DIRECT_GW ? NP : 1];
+    if (tid < NP) S.u[cat] = chan ? load1<F32>(a.u, h * hn + cn) : 0.f;
+    const float w_chan = (WMODE == W_HEAD && chan) ? static_cast<const float*>(a.w)[h * hn + cn] : 1.f;     // stager's channel
+    const float w_row = (WMODE == W_HEAD && live) ? static_cast<const float*>(a.w)[h * hn + row] : 1.f;     // this row's channel
+    float St[EL], Q[DIRECT_GW ? EL : 1];
 #pragma unroll
-    for (int o = 0; o < NP; ++o) St[o] = 0.f;
+    for (int e = 0; e < EL; ++e) St[e] = 0.f;
 #pragma unroll
-    for (int o = 0; o < (DIRECT_GW ? NP : 1); ++o) Q[o] = 0.f;
+    for (int e = 0; e < (DIRECT_GW ? EL : 1); ++e) Q[e] = 0.f;
     if (stateful && live) {
         if constexpr (PASS == P_FWD) {
 #pragma unroll
-            for (int o = 0; o < NP; ++o) if (o < hn) St[o] = bf2f(a.s0[(bh * hn + me) * hn + o]);
+            for (int e = 0; e < EL; ++e) if (o0 + e < hn) St[e] = bf2f(a.s0[(bh * hn + row) * hn + o0 + e]);
         } else if constexpr (PASS == P_GR) {
 #pragma unroll
-            for (int o = 0; o < NP; ++o) if (o < hn) St[o] = bf2f(a.s0[(bh * hn + o) * hn + me]);
+            for (int e = 0; e < EL; ++e) if (o0 + e < hn) St[e] = bf2f(a.s0[(bh * hn + o0 + e) * hn + row]);
         }
     }
-    const float w_own = (WMODE == W_HEAD && live) ? static_cast<const float*>(a.w)[h * hn + me] : 1.f;
     float gu_acc = 0.f, gw_acc = 0.f, P = 0.f;
 
     const int nchunks = (a.T + GTC - 1) / GTC;
+    // Inputs of a chunk are fetched into registers, unconverted, while the steps of the chunk before run, and go to LDS at
+    // the top of their own chunk: the first use, and with it the compiler's wait, comes after the step loop.
+    using Elem = typename std::conditional<F32, float, uint16_t>::type;
+    Elem pre_r[SPT], pre_k[SPT], pre_v[SPT], pre_g[SPT];
+    uint32_t pre_w[SPT];
+    float pre_d[SPT];
+    auto widen = [](Elem x) __attribute__((always_inline)) -> float {
+        if constexpr (F32) return x; else return bf2f(x);
+    };
+    auto prefetch = [&](const int c0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < SPT; ++i) {
+            const int tg = c0 + t_first + i;
+            const bool ok = chan && tg < a.T;
+            const size_t off = base + static_cast<size_t>(ok ? tg : 0) * a.C + (chan ? cn : 0);   // an address that exists
+            pre_r[i] = reinterpret_cast<const Elem*>(a.r)[off];
+            pre_k[i] = reinterpret_cast<const Elem*>(a.k)[off];
+            if constexpr (PASS != P_GV) pre_v[i] = reinterpret_cast<const Elem*>(a.v)[off];
+            if constexpr (PASS != P_FWD) pre_g[i] = reinterpret_cast<const Elem*>(a.gy)[off];
+            if constexpr (WMODE == W_RAW) pre_w[i] = static_cast<const uint16_t*>(a.w)[off];
+            if constexpr (WMODE == W_EW) pre_w[i] = static_cast<const uint32_t*>(a.w)[off];
+            if constexpr (SCAN_GW) pre_d[i] = a.rdr[off];
+        }
+    };
+    prefetch((REV ? nchunks - 1 : 0) * GTC);
     for (int ci = 0; ci < nchunks; ++ci) {
         const int c0 = (REV ? nchunks - 1 - ci : ci) * GTC;
         __syncthreads();                                        // the previous chunk is done with LDS
-        if (lane_ok) {
-#pragma unroll 2
-            for (int t = 0; t < GTC; ++t) {
-                const bool ok = live && (c0 + t) < a.T;         // rows past T and padded channels: no input, no decay
-                const size_t off = base + static_cast<size_t>(c0 + t) * a.C + me;
-                S.r[t][me] = ok ? load1<F32>(a.r, off) : 0.f;
-                S.k[t][me] = ok ? load1<F32>(a.k, off) : 0.f;
-                if constexpr (PASS != P_GV) S.v[t][me] = ok ? load1<F32>(a.v, off) : 0.f;
-                if constexpr (PASS != P_FWD) S.g[t][me] = ok ? load1<F32>(a.gy, off) : 0.f;
-                if constexpr (WMODE != W_HEAD) {
-                    float ew = 0.f;
-                    if (ok) ew = (WMODE == W_RAW) ? -__expf(bf2f(static_cast<const uint16_t*>(a.w)[off])) : static_cast<const float*>(a.w)[off];
-                    S.w[t][me] = ok ? __expf(ew) : 1.0f;
-                    if constexpr (PASS == P_GK) S.f[t][me] = ew < -30.0f ? 0.f : ew;    // see wkv_sweep's commit()
-                } else {
-                    S.w[t][me] = ok ? w_own : 1.0f;
-                }
-                if constexpr (SCAN_GW) S.rdr[t][me] = ok ? a.rdr[off] : 0.f;
+#pragma unroll
+        for (int i = 0; i < SPT; ++i) {                         // registers (fetched during the previous chunk's steps) -> LDS
+            const int t = t_first + i;
+            const bool ok = chan && (c0 + t) < a.T;             // rows past T and padded channels: no input, no decay
+            S.r[t][cat] = ok ? widen(pre_r[i]) : 0.f;
+            S.k[t][cat] = ok ? widen(pre_k[i]) : 0.f;
+            if constexpr (PASS != P_GV) S.v[t][cat] = ok ? widen(pre_v[i]) : 0.f;
+            if constexpr (PASS != P_FWD) S.g[t][cat] = ok ? widen(pre_g[i]) : 0.f;
+            if constexpr (WMODE != W_HEAD) {
+                float ew = 0.f;
+                if (ok) ew = (WMODE == W_RAW) ? -__expf(bf2f(static_cast<uint16_t>(pre_w[i]))) : __uint_as_float(pre_w[i]);
+                S.w[t][cat] = ok ? __expf(ew) : 1.0f;
+                if constexpr (PASS == P_GK) S.f[t][cat] = ew < -30.0f ? 0.f : ew;    // see wkv_sweep's commit()
+            } else {
+                S.w[t][cat] = ok ? w_chan : 1.0f;
             }
+            if constexpr (SCAN_GW) S.rdr[t][cat] = ok ? pre_d[i] : 0.f;
         }
         __syncthreads();
-        if (me < GTC) {                                         // the scalar of each step: sum_j u r k, or sum_i v gy
+        if (tid < GTC) {                                        // the scalar of each step: sum_j u r k, or sum_i v gy
             float d = 0.f;
-#pragma unroll 4
-            for (int o = 0; o < NP; ++o)
-                d = ROW_I ? fmaf(S.r[me][o] * S.u[o], S.k[me][o], d) : fmaf(S.v[me][o], S.g[me][o], d);
-            S.dot[me] = d;
+            for (int n = 0; n < NP; ++n) {
+                const int at = G::at(n);
+                d = ROW_I ? fmaf(S.r[tid][at] * S.u[at], S.k[tid][at], d) : fmaf(S.v[tid][at], S.g[tid][at], d);
+            }
+            S.dot[tid] = d;
         }
         __syncthreads();
+        if (ci + 1 < nchunks) prefetch((REV ? nchunks - 2 - ci : ci + 1) * GTC);
 
 #pragma unroll 1
         for (int tt = 0; tt < GTC; ++tt) {
             const int t = REV ? GTC - 1 - tt : tt, tg = c0 + t;
-            const bool ok = live && tg < a.T;
-            const size_t off = base + static_cast<size_t>(tg) * a.C + me;
+            const bool ok = writer && tg < a.T;
+            const size_t off = base + static_cast<size_t>(tg) * a.C + row;
             const float dot = S.dot[t];
             float acc = 0.f, acc2 = 0.f;
             if constexpr (ROW_I) {
-                const float x = lane_ok ? ((PASS == P_FWD) ? S.v[t][me] : S.g[t][me]) : 0.f;
+                const float x = (PASS == P_FWD) ? S.v[t][own] : S.g[t][own];
 #pragma unroll
-                for (int o = 0; o < NP; ++o) {
-                    const float av = (PASS == P_FWD) ? S.r[t][o] : S.k[t][o];
-                    const float bv = (PASS == P_FWD) ? S.k[t][o] : S.r[t][o];
-                    acc = fmaf(av, St[o], acc);
-                    St[o] = fmaf(St[o], S.w[t][o], bv * x);
-                    if (o % 8 == 7) row_fence(acc, &St[o - 7]);
+                for (int e = 0; e < EL; ++e) {
+                    const float av = (PASS == P_FWD) ? S.r[t][sl + e] : S.k[t][sl + e];
+                    const float bv = (PASS == P_FWD) ? S.k[t][sl + e] : S.r[t][sl + e];
+                    acc = fmaf(av, St[e], acc);
+                    St[e] = fmaf(St[e], S.w[t][sl + e], bv * x);
+                    if (e % 8 == 7) row_fence(acc, &St[e - 7]);
                 }
+                acc = parts_sum<PARTS>(acc);
                 if (ok) store1<F32>(PASS == P_FWD ? a.y : a.gv, off, fmaf(x, dot, acc));
             } else {
-                const float bl = lane_ok ? ((PASS == P_GR) ? S.k[t][me] : S.r[t][me]) : 0.f;
-                const float wl = lane_ok ? S.w[t][me] : 1.f;
+                const float bl = (PASS == P_GR) ? S.k[t][own] : S.r[t][own];
+                const float wl = S.w[t][own];
 #pragma unroll
-                for (int o = 0; o < NP; ++o) {
-                    const float av = (PASS == P_GR) ? S.g[t][o] : S.v[t][o];
-                    const float xv = (PASS == P_GR) ? S.v[t][o] : S.g[t][o];
-                    acc = fmaf(av, St[o], acc);
+                for (int e = 0; e < EL; ++e) {
+                    const float av = (PASS == P_GR) ? S.g[t][sl + e] : S.v[t][sl + e];
+                    const float xv = (PASS == P_GR) ? S.v[t][sl + e] : S.g[t][sl + e];
+                    acc = fmaf(av, St[e], acc);
                     if constexpr (DIRECT_GW) {
-                        acc2 = fmaf(av, Q[o], acc2);
-                        Q[o] = fmaf(Q[o], wl, St[o]);
+                        acc2 = fmaf(av, Q[e], acc2);
+                        Q[e] = fmaf(Q[e], wl, St[e]);
                     }
-                    St[o] = fmaf(St[o], wl, xv * bl);
-                    if (o % 8 == 7) {
-                        row_fence(acc, &St[o - 7]);
-                        if constexpr (DIRECT_GW) row_fence(acc2, &Q[o - 7]);
+                    St[e] = fmaf(St[e], wl, xv * bl);
+                    if (e % 8 == 7) {
+                        row_fence(acc, &St[e - 7]);
+                        if constexpr (DIRECT_GW) row_fence(acc2, &Q[e - 7]);
                     }
                 }
-                const float rr = lane_ok ? S.r[t][me] : 0.f, kk = lane_ok ? S.k[t][me] : 0.f, uu = lane_ok ? S.u[me] : 0.f;
+                acc = parts_sum<PARTS>(acc);
+                if constexpr (DIRECT_GW) acc2 = parts_sum<PARTS>(acc2);
+                const float rr = S.r[t][own], kk = S.k[t][own], uu = S.u[own];
                 if constexpr (PASS == P_GR) {
                     gu_acc = fmaf(rr * kk, dot, gu_acc);
                     if constexpr (DIRECT_GW) gw_acc = fmaf(rr, acc2, gw_acc);
@@ -649,34 +707,34 @@ __global__ __launch_bounds__(NP < 64 ? 64 : NP) void wkv_rows(const Args a, cons
                 } else {
                     if (ok) store1<F32>(a.gk, off, fmaf(uu * rr, dot, acc));
                     if constexpr (SCAN_GW) {
-                        float G = P - kk * acc;
-                        if (!stateful && tg == 0) G = 0.f;      // S_0 = 0: exact zero, as the reference leaves it
-                        P = G + (lane_ok ? S.rdr[t][me] : 0.f);
-                        if constexpr (WMODE == W_HEAD) gw_acc += G;
-                        else if (ok) store1<F32>(a.gw, off, S.f[t][me] * G);
+                        float Gt = P - kk * acc;
+                        if (!stateful && tg == 0) Gt = 0.f;     // S_0 = 0: exact zero, as the reference leaves it
+                        P = Gt + S.rdr[t][own];
+                        if constexpr (WMODE == W_HEAD) gw_acc += Gt;
+                        else if (ok) store1<F32>(a.gw, off, S.f[t][own] * Gt);
                     }
                 }
             }
         }
     }
 
-    const size_t pc = static_cast<size_t>(b) * a.C + static_cast<size_t>(h) * hn + me;
+    const size_t pc = static_cast<size_t>(b) * a.C + static_cast<size_t>(h) * hn + row;
     if constexpr (PASS == P_GR) {
-        if (live) {
+        if (writer) {
             store1<F32>(a.gu, pc, gu_acc);
-            if constexpr (DIRECT_GW) store1<F32>(a.gw, pc, a.ew_head[h * hn + me] * w_own * gw_acc);   // d eew / d w_raw = eew * ew
+            if constexpr (DIRECT_GW) store1<F32>(a.gw, pc, a.ew_head[h * hn + row] * w_row * gw_acc);     // d eew / d w_raw = eew * ew
         }
     }
     if constexpr (PASS == P_GK) {
         if constexpr (WMODE == W_HEAD && SCAN_GW) {
-            if (live) {
-                const float f = a.ew_head[h * hn + me];
+            if (writer) {
+                const float f = a.ew_head[h * hn + row];
                 store1<F32>(a.gw, pc, (f < -30.0f ? 0.f : f) * gw_acc);
             }
         }
         if (a.gs != nullptr && live) {
 #pragma unroll
-            for (int o = 0; o < NP; ++o) if (o < hn) a.gs[(bh * hn + o) * hn + me] = f2bf(St[o]);
+            for (int e = 0; e < EL; ++e) if (o0 + e < hn) a.gs[(bh * hn + o0 + e) * hn + row] = f2bf(St[e]);
         }
     }
 }
@@ -685,10 +743,11 @@ constexpr int MAX_HEAD = 128;
 
 template <int PASS, int WMODE, bool F32> void launch_rows(hipStream_t st, int B, const Args& a) {
     const int hn = a.C / a.H;
-    if (hn <= 8) hipLaunchKernelGGL((wkv_rows<8, PASS, WMODE, F32>), dim3(B * a.H), dim3(64), 0, st, a, hn);
-    else if (hn <= 32) hipLaunchKernelGGL((wkv_rows<32, PASS, WMODE, F32>), dim3(B * a.H), dim3(64), 0, st, a, hn);
-    else if (hn <= 64) hipLaunchKernelGGL((wkv_rows<64, PASS, WMODE, F32>), dim3(B * a.H), dim3(64), 0, st, a, hn);
-    else if constexpr (!F32) hipLaunchKernelGGL((wkv_rows<128, PASS, WMODE, F32>), dim3(B * a.H), dim3(128), 0, st, a, hn);
+    const dim3 grid(B * a.H);
+    if (hn <= 8) hipLaunchKernelGGL((wkv_rows<8, 1, PASS, WMODE, F32>), grid, dim3(RowGeom<8, 1>::NTHREADS), 0, st, a, hn);
+    else if (hn <= 32) hipLaunchKernelGGL((wkv_rows<32, 2, PASS, WMODE, F32>), grid, dim3(RowGeom<32, 2>::NTHREADS), 0, st, a, hn);
+    else if (hn <= 64) hipLaunchKernelGGL((wkv_rows<64, 4, PASS, WMODE, F32>), grid, dim3(RowGeom<64, 4>::NTHREADS), 0, st, a, hn);
+    else hipLaunchKernelGGL((wkv_rows<128, 4, PASS, WMODE, F32>), grid, dim3(RowGeom<128, 4>::NTHREADS), 0, st, a, hn);
 }
 
 // The chunked matrix-core kernels serve all three decay conventions; the sequential sweeps remain as the second algorithm.
@@ -737,8 +796,7 @@ template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a, unsign
 }
 
 // head size 64 takes the kernels this file and wkv6_*.hip are written for, any other size up to 128 the row-per-thread
-// kernels (wkv_rows); wkv5a exists for 64 only, and the fp32 wkv5 op up to 64 (its decay-gradient sweep keeps two state
-// rows per thread, which at 128 no longer fit the register file)
+// kernels (wkv_rows); wkv5a exists for 64 only
 int check_dims(int B, int T, int C, int H, bool only64 = false, int max_head = MAX_HEAD) {
     if (B <= 0 || T <= 0 || C <= 0 || H <= 0) return RWKV_ERR_SHAPE;
     if (C % H != 0 || C / H > max_head) return RWKV_ERR_SHAPE;
@@ -819,7 +877,7 @@ uint16_t* out_elems(float* p) { return reinterpret_cast<uint16_t*>(p); }
 
 int rwkv_wkv5f32_forward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
                          const float* eew, const float* u, float* y) {
-    if (int e = check_dims(B, T, C, H, false, N)) return e;
+    if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, eew, u, y}, C == H * N)) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew; a.u = as_elems(u);
@@ -832,7 +890,7 @@ int rwkv_wkv5f32_forward(void* stream, int B, int T, int C, int H, const float* 
 int rwkv_wkv5f32_backward_ex(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
                           const float* eew, const float* ew, const float* u, const float* gy, float* gr, float* gk,
                           float* gv, float* gw, float* gu, unsigned flags) {
-    if (int e = check_dims(B, T, C, H, false, N)) return e;
+    if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu}, C == H * N)) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew; a.ew_head = ew;

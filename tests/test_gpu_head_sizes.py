@@ -81,7 +81,7 @@ def test_wkv6_fp32_ew_interface_any_head_size(lib, N):
     assert e < 6e-3
 
 
-@pytest.mark.parametrize("N", [2, 4, 17, 48])
+@pytest.mark.parametrize("N", [2, 4, 17, 48, 128])
 def test_wkv5_fp32_any_head_size(lib, N):
     B, T, H = 2, 53, 2
     C = H * N
@@ -139,8 +139,7 @@ def test_head_size_limits(lib):
     # 129 > 128, and C not a multiple of H
     assert lib.rwkv_wkv6raw_forward(None, 2, 8, 129, 1, *(x.data_ptr(),) * 6) == -1
     assert lib.rwkv_wkv6raw_forward(None, 2, 8, 130, 4, *(x.data_ptr(),) * 6) == -1
-    # the fp32 op: up to 64 (wkv5/run.py benchmarks 64 and checks with 2)
-    assert lib.rwkv_wkv5f32_forward(None, 2, 8, 128, 1, *(f.data_ptr(),) * 6) == -1
+    assert lib.rwkv_wkv5f32_forward(None, 2, 8, 129, 1, *(f.data_ptr(),) * 6) == -1
     # the two-sided op exists for head size 64 only, as built here
     assert lib.rwkv_wkv5a_forward(None, 2, 8, 32, 1, x.data_ptr(), x.data_ptr(), x.data_ptr(), f.data_ptr(), f.data_ptr(),
                                   f.data_ptr(), f.data_ptr(), x.data_ptr()) == -1
