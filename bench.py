@@ -37,6 +37,7 @@ TRAFFIC_MEASURED = {
     "wkv6_fwd_ws": 537e6 + 134e6,
     "wkv6_bwd_a_ws": 683e6 + 432e6,
     "wkv6_bwd_b_ws": 990e6 + 403e6,
+    "wkv6state forward": 537e6 + 134e6, "wkv6state backward (3 kernels)": 683e6 + 432e6 + 990e6 + 403e6,
     # profiles/wkv5_ws_kernels_B8_T4096_C2048.md
     "wkv6_fwd_ws<head decay>": 403e6 + 134e6,
     "wkv6_bwd_a_ws<head decay>": 548e6 + 533e6,
@@ -47,6 +48,9 @@ TRAFFIC_MEASURED = {
     # profiles/rwkv7_chunk_kernels_B8_T4096_C4096.md (four calls of T = 1024)
     "rwkv7c_fwd x4 (T=1024 each)": 4 * (411.2e6 + 746.6e6),
     "rwkv7c_bwd x4": 4 * (1149.7e6 + 411.0e6),
+    # profiles/wkv5_rows_kernels_B8_T4096_C4096_N128.md
+    "wkv_rows<FWD>": 805.4e6 + 268.4e6, "wkv_rows<GR>": 1073.8e6 + 805.4e6,
+    "wkv_rows<GV>": 805.4e6 + 268.4e6, "wkv_rows<GK>": 1610.8e6 + 268.5e6,
     # profiles/wkv4_seg_kernels_B4_T512_C768.md
     "wkv4_fwd_seg": 29.7e6 + 6.3e6,
     "wkv4_bwd_seg + wkv4_batch_sum": 186.6e6 + 31.5e6,
