@@ -14,9 +14,9 @@
  *     function reports.  No entry point allocates or frees device memory, and none
  *     synchronises: work is enqueued on `stream` and the call returns.
  *   - T and the head size N = C / H are run-time values (the reference bakes -D_T_ and -D_N_ into its kernels).
- *     wkv5 (bf16 and fp32), wkv6 and wkv6_state take any N from 1 to 128 (C a multiple of H); 64 runs on the kernels
+ *     wkv5 (bf16 and fp32), wkv5a, wkv6 and wkv6_state take any N from 1 to 128 (C a multiple of H); 64 runs on the kernels
  *     written for it, every other size on kernels that keep one state row in the registers of one to four lanes.
- *     wkv5a and rwkv7 take N = 64 only.
+ *     rwkv7 takes N = 64 only.
  *
  * bf16 tensors are passed as uint16_t* (raw bfloat16 bits).  All tensors are dense and
  * contiguous in the layouts named per function and must be 16-byte aligned (head sizes other than 64: any alignment

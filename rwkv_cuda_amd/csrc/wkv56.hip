@@ -533,31 +533,37 @@ template <int NP, int PARTS> struct RowGeom {
     static __device__ __forceinline__ int at(int n) { return (n / EL) * SLOT + n % EL; }   // where channel n of a vector sits
 };
 
-template <int NP, int PARTS> struct SmemRows {
+// staged vectors of one chunk; the ones a pass does not use shrink to one row
+template <int NP, int PARTS, int PASS, bool F32, bool TWO> struct SmemRows {
     static constexpr int LEN = RowGeom<NP, PARTS>::LEN;
-    alignas(16) float r[GTC][LEN], k[GTC][LEN], v[GTC][LEN], g[GTC][LEN], w[GTC][LEN], f[GTC][LEN], rdr[GTC][LEN];
-    float dot[GTC];
-    alignas(16) float u[LEN];
+    static constexpr bool kF = (PASS == P_GK && !F32) || (TWO && PASS == P_GR);     // gw factor, or w2[i] gy[i]
+    alignas(16) float r[GTC][LEN], k[GTC][LEN], w[GTC][LEN];
+    alignas(16) float v[PASS != P_GV ? GTC : 1][LEN], g[PASS != P_FWD ? GTC : 1][LEN];
+    alignas(16) float f[kF ? GTC : 1][LEN], rdr[(PASS == P_GK && !F32) ? GTC : 1][LEN];
+    float dot[GTC], dot2[TWO ? GTC : 1], dot3[TWO ? GTC : 1];
+    alignas(16) float u[LEN], u2[TWO ? LEN : 4], w2[TWO ? LEN : 4];
 };
 
 // sum over the PARTS adjacent lanes that share a row; every one of them gets the total
 template <int PARTS> DEVINL float parts_sum(float x) {
     if constexpr (PARTS >= 2) x += __shfl_xor(x, 1, 64);
     if constexpr (PARTS >= 4) x += __shfl_xor(x, 2, 64);
-    static_assert(PARTS == 1 || PARTS == 2 || PARTS == 4, "adjacent lanes of one quad");
+    if constexpr (PARTS >= 8) x += __shfl_xor(x, 4, 64);
+    static_assert(PARTS == 1 || PARTS == 2 || PARTS == 4 || PARTS == 8, "adjacent lanes");
     return x;
 }
 
-template <int NP, int PARTS, int PASS, int WMODE, bool F32>
+template <int NP, int PARTS, int PASS, int WMODE, bool F32, bool TWO = false>
 __global__ __launch_bounds__((RowGeom<NP, PARTS>::NTHREADS)) void wkv_rows(const Args a, const int hn) {
     static_assert(!F32 || WMODE == W_HEAD, "fp32 I/O exists for wkv5 only");
+    static_assert(!TWO || F32, "the two-sided op is fp32 only");
     using G = RowGeom<NP, PARTS>;
     constexpr int EL = G::EL, SLOT = G::SLOT;
     constexpr bool REV = (PASS == P_GK || PASS == P_GV);
     constexpr bool ROW_I = (PASS == P_FWD || PASS == P_GV);     // row = value channel, registers = key channels
     constexpr bool DIRECT_GW = F32 && PASS == P_GR;             // as in wkv_sweep: the fp32 op carries Q = dS/dw
     constexpr bool SCAN_GW = !F32 && PASS == P_GK;
-    __shared__ SmemRows<NP, PARTS> S;
+    __shared__ SmemRows<NP, PARTS, PASS, F32, TWO> S;
 
     const int tid = threadIdx.x;
     const int row = tid / PARTS, part = tid % PARTS;            // threads beyond NP * PARTS (NP * PARTS < 64) only idle
@@ -579,7 +585,13 @@ __global__ __launch_bounds__((RowGeom<NP, PARTS>::NTHREADS)) void wkv_rows(const
     const bool chan = cn < hn;
     const int cat = G::at(cn);
 
-    if (tid < NP) S.u[cat] = chan ? load1<F32>(a.u, h * hn + cn) : 0.f;
+    if (tid < NP) {
+        S.u[cat] = chan ? load1<F32>(a.u, h * hn + cn) : 0.f;
+        if constexpr (TWO) {
+            S.u2[cat] = chan ? load1<F32>(a.u2, h * hn + cn) : 0.f;
+            S.w2[cat] = chan ? a.w2[h * hn + cn] : 1.f;
+        }
+    }
     const float w_chan = (WMODE == W_HEAD && chan) ? static_cast<const float*>(a.w)[h * hn + cn] : 1.f;     // stager's channel
     const float w_row = (WMODE == W_HEAD && live) ? static_cast<const float*>(a.w)[h * hn + row] : 1.f;     // this row's channel
     float St[EL], Q[DIRECT_GW ? EL : 1];
@@ -587,6 +599,16 @@ __global__ __launch_bounds__((RowGeom<NP, PARTS>::NTHREADS)) void wkv_rows(const
     for (int e = 0; e < EL; ++e) St[e] = 0.f;
 #pragma unroll
     for (int e = 0; e < (DIRECT_GW ? EL : 1); ++e) Q[e] = 0.f;
+    // two-sided: state element [i][j] decays by w1[j] w2[i]; A collects gw2 per state element
+    constexpr bool GW2 = TWO && PASS == P_GR;
+    float A[GW2 ? EL : 1];
+    float u2_row = 0.f, w2_row = 1.f, gu2_acc = 0.f;
+    if constexpr (TWO) {
+        u2_row = live ? load1<F32>(a.u2, h * hn + row) : 0.f;
+        w2_row = live ? a.w2[h * hn + row] : 1.f;
+#pragma unroll
+        for (int e = 0; e < (GW2 ? EL : 1); ++e) A[e] = 0.f;
+    }
     if (stateful && live) {
         if constexpr (PASS == P_FWD) {
 #pragma unroll
@@ -644,17 +666,27 @@ __global__ __launch_bounds__((RowGeom<NP, PARTS>::NTHREADS)) void wkv_rows(const
                 S.w[t][cat] = ok ? w_chan : 1.0f;
             }
             if constexpr (SCAN_GW) S.rdr[t][cat] = ok ? pre_d[i] : 0.f;
+            if constexpr (GW2) S.f[t][cat] = ok ? widen(pre_g[i]) * S.w2[cat] : 0.f;    // w2[i] gy[i]: the operand of gw1
         }
         __syncthreads();
         if (tid < GTC) {                                        // the scalar of each step: sum_j u r k, or sum_i v gy
-            float d = 0.f;
+            float d = 0.f, d2 = 0.f, d3 = 0.f;
             for (int n = 0; n < NP; ++n) {
                 const int at = G::at(n);
                 d = ROW_I ? fmaf(S.r[tid][at] * S.u[at], S.k[tid][at], d) : fmaf(S.v[tid][at], S.g[tid][at], d);
+                if constexpr (TWO) {                            // the bonus u1[j] + u2[i] needs a second scalar, gu2 a third
+                    d2 = ROW_I ? fmaf(S.r[tid][at], S.k[tid][at], d2) : fmaf(S.v[tid][at] * S.u2[at], S.g[tid][at], d2);
+                    if constexpr (PASS == P_GR) d3 = fmaf(S.r[tid][at], S.k[tid][at], d3);
+                }
             }
             S.dot[tid] = d;
+            if constexpr (TWO) { S.dot2[tid] = d2; S.dot3[tid] = d3; }
         }
         __syncthreads();
+        if constexpr (GW2) {                                    // gu2[i] = sum_t v_i gy_i sum_j r_j k_j, by the staging threads
+#pragma unroll
+            for (int i = 0; i < SPT; ++i) gu2_acc = fmaf(S.v[t_first + i][cat] * S.g[t_first + i][cat], S.dot3[t_first + i], gu2_acc);
+        }
         if (ci + 1 < nchunks) prefetch((REV ? nchunks - 2 - ci : ci + 1) * GTC);
 
 #pragma unroll 1
@@ -671,27 +703,32 @@ __global__ __launch_bounds__((RowGeom<NP, PARTS>::NTHREADS)) void wkv_rows(const
                     const float av = (PASS == P_FWD) ? S.r[t][sl + e] : S.k[t][sl + e];
                     const float bv = (PASS == P_FWD) ? S.k[t][sl + e] : S.r[t][sl + e];
                     acc = fmaf(av, St[e], acc);
-                    St[e] = fmaf(St[e], S.w[t][sl + e], bv * x);
+                    St[e] = fmaf(St[e], TWO ? S.w[t][sl + e] * w2_row : S.w[t][sl + e], bv * x);
                     if (e % 8 == 7) row_fence(acc, &St[e - 7]);
                 }
                 acc = parts_sum<PARTS>(acc);
-                if (ok) store1<F32>(PASS == P_FWD ? a.y : a.gv, off, fmaf(x, dot, acc));
+                const float bonus = TWO ? fmaf(u2_row, S.dot2[t], dot) : dot;
+                if (ok) store1<F32>(PASS == P_FWD ? a.y : a.gv, off, fmaf(x, bonus, acc));
             } else {
                 const float bl = (PASS == P_GR) ? S.k[t][own] : S.r[t][own];
                 const float wl = S.w[t][own];
+                const float w1r = GW2 ? wl * S.r[t][own] : 0.f;                 // w1[j] r[j]
 #pragma unroll
                 for (int e = 0; e < EL; ++e) {
                     const float av = (PASS == P_GR) ? S.g[t][sl + e] : S.v[t][sl + e];
                     const float xv = (PASS == P_GR) ? S.v[t][sl + e] : S.g[t][sl + e];
+                    const float de = TWO ? wl * S.w2[sl + e] : wl;
                     acc = fmaf(av, St[e], acc);
                     if constexpr (DIRECT_GW) {
-                        acc2 = fmaf(av, Q[e], acc2);
-                        Q[e] = fmaf(Q[e], wl, St[e]);
+                        acc2 = fmaf(GW2 ? S.f[t][sl + e] : av, Q[e], acc2);
+                        if constexpr (GW2) A[e] = fmaf(av, Q[e] * w1r, A[e]);
+                        Q[e] = fmaf(Q[e], de, St[e]);
                     }
-                    St[e] = fmaf(St[e], wl, xv * bl);
+                    St[e] = fmaf(St[e], de, xv * bl);
                     if (e % 8 == 7) {
                         row_fence(acc, &St[e - 7]);
                         if constexpr (DIRECT_GW) row_fence(acc2, &Q[e - 7]);
+                        if constexpr (GW2) row_fence(acc, &A[e - 7]);
                     }
                 }
                 acc = parts_sum<PARTS>(acc);
@@ -701,11 +738,11 @@ __global__ __launch_bounds__((RowGeom<NP, PARTS>::NTHREADS)) void wkv_rows(const
                     gu_acc = fmaf(rr * kk, dot, gu_acc);
                     if constexpr (DIRECT_GW) gw_acc = fmaf(rr, acc2, gw_acc);
                     if (ok) {
-                        store1<F32>(a.gr, off, fmaf(uu * kk, dot, acc));
+                        store1<F32>(a.gr, off, TWO ? fmaf(kk, fmaf(uu, dot, S.dot2[t]), acc) : fmaf(uu * kk, dot, acc));
                         if constexpr (!F32) a.rdr[off] = rr * acc;
                     }
                 } else {
-                    if (ok) store1<F32>(a.gk, off, fmaf(uu * rr, dot, acc));
+                    if (ok) store1<F32>(a.gk, off, TWO ? fmaf(rr, fmaf(uu, dot, S.dot2[t]), acc) : fmaf(uu * rr, dot, acc));
                     if constexpr (SCAN_GW) {
                         float Gt = P - kk * acc;
                         if (!stateful && tg == 0) Gt = 0.f;     // S_0 = 0: exact zero, as the reference leaves it
@@ -724,6 +761,31 @@ __global__ __launch_bounds__((RowGeom<NP, PARTS>::NTHREADS)) void wkv_rows(const
             store1<F32>(a.gu, pc, gu_acc);
             if constexpr (DIRECT_GW) store1<F32>(a.gw, pc, a.ew_head[h * hn + row] * w_row * gw_acc);     // d eew / d w_raw = eew * ew
         }
+        if constexpr (GW2) {
+            // gu2: the staging groups' partial sums, one row of LDS per group
+            __syncthreads();
+            S.r[tid / NP][cat] = gu2_acc;
+            __syncthreads();
+            if (tid < NP && chan) {
+                float sum = 0.f;
+                for (int q = 0; q < SG; ++q) sum += S.r[q][cat];
+                store1<F32>(a.gu2, static_cast<size_t>(b) * a.C + static_cast<size_t>(h) * hn + cn, sum);
+            }
+            // gw2[i] = ew2[i] w2[i] sum_j A_j[i]: rows j pass through LDS sixteen at a time and are added in order
+            float tot = 0.f;
+            for (int r0 = 0; r0 < NP; r0 += GTC) {
+                __syncthreads();
+                if (in_rows && row >= r0 && row < r0 + GTC) {
+#pragma unroll
+                    for (int e = 0; e < EL; ++e) S.k[row - r0][sl + e] = A[GW2 ? e : 0];
+                }
+                __syncthreads();
+                if (tid < NP)
+                    for (int q = 0; q < (NP < GTC ? NP : GTC); ++q) tot += S.k[q][cat];
+            }
+            if (tid < NP && chan)
+                store1<F32>(a.gw2, static_cast<size_t>(b) * a.C + static_cast<size_t>(h) * hn + cn, a.ew2_head[h * hn + cn] * a.w2[h * hn + cn] * tot);
+        }
     }
     if constexpr (PASS == P_GK) {
         if constexpr (WMODE == W_HEAD && SCAN_GW) {
@@ -741,13 +803,14 @@ __global__ __launch_bounds__((RowGeom<NP, PARTS>::NTHREADS)) void wkv_rows(const
 
 constexpr int MAX_HEAD = 128;
 
-template <int PASS, int WMODE, bool F32> void launch_rows(hipStream_t st, int B, const Args& a) {
+template <int PASS, int WMODE, bool F32, bool TWO = false> void launch_rows(hipStream_t st, int B, const Args& a) {
     const int hn = a.C / a.H;
     const dim3 grid(B * a.H);
-    if (hn <= 8) hipLaunchKernelGGL((wkv_rows<8, 1, PASS, WMODE, F32>), grid, dim3(RowGeom<8, 1>::NTHREADS), 0, st, a, hn);
-    else if (hn <= 32) hipLaunchKernelGGL((wkv_rows<32, 2, PASS, WMODE, F32>), grid, dim3(RowGeom<32, 2>::NTHREADS), 0, st, a, hn);
-    else if (hn <= 64) hipLaunchKernelGGL((wkv_rows<64, 4, PASS, WMODE, F32>), grid, dim3(RowGeom<64, 4>::NTHREADS), 0, st, a, hn);
-    else hipLaunchKernelGGL((wkv_rows<128, 4, PASS, WMODE, F32>), grid, dim3(RowGeom<128, 4>::NTHREADS), 0, st, a, hn);
+    if (hn <= 8) hipLaunchKernelGGL((wkv_rows<8, 1, PASS, WMODE, F32, TWO>), grid, dim3(RowGeom<8, 1>::NTHREADS), 0, st, a, hn);
+    else if (hn <= 32) hipLaunchKernelGGL((wkv_rows<32, 2, PASS, WMODE, F32, TWO>), grid, dim3(RowGeom<32, 2>::NTHREADS), 0, st, a, hn);
+    else if (hn <= 64) hipLaunchKernelGGL((wkv_rows<64, 4, PASS, WMODE, F32, TWO>), grid, dim3(RowGeom<64, 4>::NTHREADS), 0, st, a, hn);
+    else if constexpr (TWO) hipLaunchKernelGGL((wkv_rows<128, 8, PASS, WMODE, F32, TWO>), grid, dim3(RowGeom<128, 8>::NTHREADS), 0, st, a, hn);
+    else hipLaunchKernelGGL((wkv_rows<128, 4, PASS, WMODE, F32, TWO>), grid, dim3(RowGeom<128, 4>::NTHREADS), 0, st, a, hn);
 }
 
 // The chunked matrix-core kernels serve all three decay conventions; the sequential sweeps remain as the second algorithm.
@@ -795,12 +858,10 @@ template <int WMODE> int launch_bwd(hipStream_t st, int B, const Args& a, unsign
     return launch_status();
 }
 
-// head size 64 takes the kernels this file and wkv6_*.hip are written for, any other size up to 128 the row-per-thread
-// kernels (wkv_rows); wkv5a exists for 64 only
-int check_dims(int B, int T, int C, int H, bool only64 = false, int max_head = MAX_HEAD) {
+// head size 64 takes the kernels this file and wkv6_*.hip are written for, any other size up to 128 the row kernels (wkv_rows)
+int check_dims(int B, int T, int C, int H) {
     if (B <= 0 || T <= 0 || C <= 0 || H <= 0) return RWKV_ERR_SHAPE;
-    if (C % H != 0 || C / H > max_head) return RWKV_ERR_SHAPE;
-    if (only64 && C != H * N) return RWKV_ERR_SHAPE;
+    if (C % H != 0 || C / H > MAX_HEAD) return RWKV_ERR_SHAPE;
     if (static_cast<long long>(B) * H > 0x7fffffffLL) return RWKV_ERR_SHAPE;
     return RWKV_OK;
 }
@@ -913,11 +974,15 @@ int rwkv_wkv5f32_backward_ex(void* stream, int B, int T, int C, int H, const flo
 // ---- wkv5a: two-sided decay and bonus, fp32, on the same sweeps
 int rwkv_wkv5a_forward(void* stream, int B, int T, int C, int H, const float* r, const float* k, const float* v,
                        const float* eew1, const float* u1, const float* eew2, const float* u2, float* y) {
-    if (int e = check_dims(B, T, C, H, true)) return e;
-    if (int e = check_ptrs({r, k, v, eew1, u1, eew2, u2, y})) return e;
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, eew1, u1, eew2, u2, y}, C == H * N)) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew1; a.u = as_elems(u1);
     a.w2 = eew2; a.u2 = as_elems(u2); a.y = out_elems(y);
+    if (C != H * N) {
+        launch_rows<P_FWD, W_HEAD, true, true>(static_cast<hipStream_t>(stream), B, a);
+        return launch_status();
+    }
     hipLaunchKernelGGL((wkv_sweep<P_FWD, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, static_cast<hipStream_t>(stream), a);
     return launch_status();
 }
@@ -926,14 +991,20 @@ int rwkv_wkv5a_backward_ex(void* stream, int B, int T, int C, int H, const float
                         const float* eew1, const float* ew1, const float* u1, const float* eew2, const float* ew2,
                         const float* u2, const float* gy, float* gr, float* gk, float* gv, float* gw1, float* gu1,
                         float* gw2, float* gu2, unsigned flags) {
-    if (int e = check_dims(B, T, C, H, true)) return e;
-    if (int e = check_ptrs({r, k, v, eew1, ew1, u1, eew2, ew2, u2, gy, gr, gk, gv, gw1, gu1, gw2, gu2})) return e;
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, eew1, ew1, u1, eew2, ew2, u2, gy, gr, gk, gv, gw1, gu1, gw2, gu2}, C == H * N)) return e;
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = as_elems(r); a.k = as_elems(k); a.v = as_elems(v); a.w = eew1; a.ew_head = ew1;
     a.u = as_elems(u1); a.w2 = eew2; a.ew2_head = ew2; a.u2 = as_elems(u2); a.gy = as_elems(gy);
     a.gr = out_elems(gr); a.gk = out_elems(gk); a.gv = out_elems(gv);
     a.gw = out_elems(gw1); a.gu = out_elems(gu1); a.gw2 = out_elems(gw2); a.gu2 = out_elems(gu2);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (C != H * N) {
+        if (passes_of(flags) & RWKV_PASS_GR) launch_rows<P_GR, W_HEAD, true, true>(st, B, a);
+        if (passes_of(flags) & RWKV_PASS_GV) launch_rows<P_GV, W_HEAD, true, true>(st, B, a);
+        if (passes_of(flags) & RWKV_PASS_GK) launch_rows<P_GK, W_HEAD, true, true>(st, B, a);
+        return launch_status();
+    }
     // three independent sweeps: gr + gu1 + gu2 + gw1 + gw2, gv, gk
     if (passes_of(flags) & RWKV_PASS_GR) hipLaunchKernelGGL((wkv_sweep<P_GR, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);
     if (passes_of(flags) & RWKV_PASS_GV) hipLaunchKernelGGL((wkv_sweep<P_GV, W_HEAD, true, true>), dim3(B * H), dim3(NT), 0, st, a);

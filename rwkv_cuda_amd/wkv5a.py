@@ -4,7 +4,7 @@ import torch
 
 from ._call import call, check_tensors, require
 
-HEAD_SIZE = 64
+MAX_HEAD_SIZE = 128      # 64 runs on the kernels written for it, other sizes on the row kernels
 
 
 class WKV_5A(torch.autograd.Function):
@@ -20,7 +20,7 @@ class WKV_5A(torch.autograd.Function):
             require(r.dim() == 3 and w1.dim() == 2, "r,k,v are [B,T,C]; w1,u1,w2,u2 are [H,N]")
             B, T, C = r.shape
             H = w1.shape[0]
-            require(C == H * HEAD_SIZE and w1.shape[1] == HEAD_SIZE, "head size must be 64")
+            require(C % H == 0 and w1.shape[1] == C // H and C // H <= MAX_HEAD_SIZE, "w1 is [H, C/H] with a head size of at most 128")
             require(k.shape == r.shape and v.shape == r.shape, "shape mismatch")
             require(u1.shape == w1.shape and w2.shape == w1.shape and u2.shape == w1.shape, "shape mismatch")
             ctx.dims = (B, T, C, H)

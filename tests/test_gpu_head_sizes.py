@@ -9,7 +9,8 @@ import torch
 
 from oracle import wkv56 as O
 from oracle import err_ratio
-from rwkv_cuda_amd import synth, wkv5_bf16, wkv6, wkv6_state
+from oracle import wkv5a as A5
+from rwkv_cuda_amd import synth, wkv5_bf16, wkv5a, wkv6, wkv6_state
 from rwkv_cuda_amd._call import call
 from _gpu_util import DEV, assert_no_worse, garbage
 
@@ -104,6 +105,26 @@ def test_wkv5_fp32_any_head_size(lib, N):
         assert e <= 1e-5, (name, e)
 
 
+@pytest.mark.parametrize("N", [1, 4, 17, 48, 128])
+def test_wkv5a_any_head_size(lib, N):
+    """wkv5a/run.py:38-72 lists head sizes 4, 17, 64 and 128 for its jobs."""
+    B, T, H = 2, 45, 2
+    C = H * N
+    g = torch.Generator().manual_seed(600 + N)
+    rnd = lambda *s, lo=-1.0, hi=1.0: torch.rand(*s, generator=g) * (hi - lo) + lo
+    r, k, v, gy = rnd(B, T, C), rnd(B, T, C), rnd(B, T, C), rnd(B, T, C)
+    w1, u1, w2, u2 = rnd(H, N, lo=-8.0), rnd(H, N), rnd(H, N, lo=-8.0), rnd(H, N)
+    ref = A5.grads(B, T, C, H, r, k, v, w1, u1, w2, u2, gy)
+    t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w1, u1, w2, u2)]
+    y = wkv5a.CUDA_1(*t)
+    y.backward(gy.to(DEV))
+    torch.cuda.synchronize()
+    for name, a, got in zip(["y", "gr", "gk", "gv", "gw1", "gu1", "gw2", "gu2"], ref, [y] + [x.grad for x in t]):
+        e = err_ratio(a, got.detach().double().cpu().reshape(a.shape))
+        print(f"  wkv5a N={N} {name}: {e:.3e}", flush=True)
+        assert e <= 1e-5, (name, e)
+
+
 def test_wkv5_bf16_reference_default_shape_sampled_heads(lib):
     """wkv5_bf16/run.py:17-22 as shipped: B8 T4096 C4096, head size 128.  Two heads against the fp64 oracle."""
     B, T, N = 8, 4096, 128
@@ -140,6 +161,5 @@ def test_head_size_limits(lib):
     assert lib.rwkv_wkv6raw_forward(None, 2, 8, 129, 1, *(x.data_ptr(),) * 6) == -1
     assert lib.rwkv_wkv6raw_forward(None, 2, 8, 130, 4, *(x.data_ptr(),) * 6) == -1
     assert lib.rwkv_wkv5f32_forward(None, 2, 8, 129, 1, *(f.data_ptr(),) * 6) == -1
-    # the two-sided op exists for head size 64 only, as built here
-    assert lib.rwkv_wkv5a_forward(None, 2, 8, 32, 1, x.data_ptr(), x.data_ptr(), x.data_ptr(), f.data_ptr(), f.data_ptr(),
-                                  f.data_ptr(), f.data_ptr(), x.data_ptr()) == -1
+    assert lib.rwkv_wkv5a_forward(None, 2, 8, 129, 1, f.data_ptr(), f.data_ptr(), f.data_ptr(), f.data_ptr(), f.data_ptr(),
+                                  f.data_ptr(), f.data_ptr(), f.data_ptr()) == -1
