@@ -56,6 +56,22 @@ def test_wkv6_any_head_size(lib, N, state):
         assert float(t[3].grad[:, 0].abs().max()) == 0.0          # no state before the first token: an exact zero
 
 
+@pytest.mark.parametrize("T", [1, 16, 33])
+def test_wkv6_state_short_sequences_head_size_8(lib, T):
+    """One step, exactly one staged chunk of 16 steps, and two chunks and a step."""
+    B, H, N = 3, 2, 8
+    C = H * N
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=700 + T, state=True)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    t = [x.to(DEV).requires_grad_(True) for x in (r, k, v, w, u, s0)]
+    y = wkv6_state.RUN_CUDA(B, T, C, H, *t)
+    y.backward(gy.to(DEV))
+    torch.cuda.synchronize()
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, emu, [y] + [x.grad for x in t]):
+        assert_no_worse(f"wkv6_state N=8 T={T} {name}", a, e.reshape(a.shape), g.reshape(a.shape))
+
+
 @pytest.mark.parametrize("N", [2, 17, 128])
 def test_wkv6_fp32_ew_interface_any_head_size(lib, N):
     """The reference's own signature (fp32 ew = -exp(w), per-batch gu; wkv6/cuda/wkv6_op.cpp:5-6) with garbage-filled outputs."""
