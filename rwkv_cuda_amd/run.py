@@ -228,8 +228,15 @@ def main(argv=None):
     ap.add_argument("job", nargs="?", default="check", choices=["check", "benchmark"])
     ap.add_argument("--B", type=int)
     ap.add_argument("--T", type=int)
-    ap.add_argument("--H", type=int, help="heads (channels = 64 H; for wkv and depthwise_conv1d: channels / 64)")
+    ap.add_argument("--H", type=int, help="heads (channels = head size x H; for wkv and depthwise_conv1d: channels / 64)")
+    ap.add_argument("--N", type=int, help="head size for wkv5, wkv5_bf16, wkv5a, wkv6, wkv6_state (default 64; 1..128, as the "
+                                          "reference's -D_N_: its checks use 2 and 4, wkv5_bf16/run.py ships 128)")
     args = ap.parse_args(argv)
+    if args.N is not None:
+        if not 1 <= args.N <= 128 or (args.N != 64 and args.op not in ("wkv5", "wkv5_bf16", "wkv5a", "wkv6", "wkv6_state")):
+            ap.error("--N: 1..128 for wkv5, wkv5_bf16, wkv5a, wkv6, wkv6_state; the other ops have head size 64")
+        global N
+        N = args.N
     if not torch.cuda.is_available():
         raise SystemExit("rwkv_cuda_amd.run needs a HIP device: the kernels have no CPU path")
     dev = torch.device("cuda:0")

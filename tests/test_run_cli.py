@@ -54,3 +54,22 @@ def test_benchmark_job_prints_the_profiler_tables(lib):
     run.benchmark("wkv6_state", torch.device("cuda:0"), 2, 256, 2, out=lines.append)
     text = "\n".join(lines)
     assert "HIP forward" in text and "HIP backward" in text
+
+
+def test_head_size_option_is_validated():
+    with pytest.raises(SystemExit):
+        run.main(["rwkv7", "check", "--N", "4"])          # rwkv7 has head size 64 only
+    with pytest.raises(SystemExit):
+        run.main(["wkv6", "check", "--N", "129"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("op,n", [("wkv6_state", 4), ("wkv6", 4), ("wkv5", 2), ("wkv5_bf16", 128), ("wkv5a", 4)])
+def test_check_job_at_the_reference_drivers_head_sizes(lib, op, n):
+    """The head sizes the reference's own check jobs use (wkv6_state/run.py:39, wkv6/run.py:35, wkv5/run.py:366,
+    wkv5_bf16/run.py:21, wkv5a/run.py:43)."""
+    old = run.N
+    try:
+        assert run.main([op, "check", "--N", str(n), "--T", "40"]) == 0
+    finally:
+        run.N = old
