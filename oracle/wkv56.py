@@ -252,3 +252,76 @@ def emulate_wkv6_bf16(B, T, C, H, r, k, v, w_raw, u, gy, s0=None):
     if s0 is not None:
         res.append(rb(out[6]))
     return res
+
+
+def emulate_wkv6state_kernel_order(B, T, C, H, r, k, v, w_raw, u, gy, s0):
+    """The reference wkv6_state kernels restated sweep by sweep in fp32, in their own order of operations
+    (wkv6_state/cuda/wkv6state_cuda_v1a.cu): forward :6-65; backward_111 :67-188 (gr + gu ascending, gk descending, gv
+    descending, gs ascending through the running product of the decays); backward_222 :190-293, which makes the decay
+    gradient from a descending sweep that stores one scalar per step (`sbbbb`), the initial state, and an ascending
+    sweep that carries a running sum.  Outputs are rounded to bf16 where the kernels round (:63,119,121,143,166,187,
+    251,292) and gu is summed over the batch in bf16 (wkv6_state/run.py:123).  Vectorised over batch, head and the
+    kernels' thread index; the loop over time is explicit.  Needs T >= 3 (the kernel's sweeps address t-2)."""
+    assert T >= 3
+    N = C // H
+    f = torch.float32
+    rb = lambda x: x.to(torch.bfloat16)
+    R, K, V, G = (x.to(f).reshape(B, T, H, N) for x in (r, k, v, gy))
+    Wraw = w_raw.to(f).reshape(B, T, H, N)
+    W = torch.exp(-torch.exp(Wraw))                                  # the decay of each step and key channel
+    U = u.to(f).reshape(1, H, N)
+    S0 = s0.to(f).reshape(B, H, N, N)                                # [value][key]
+    y, gr, gk, gv, gw = (torch.zeros(B, T, H, N, dtype=f) for _ in range(5))
+    # forward: a thread per value channel i, registers over the key channel j
+    S = S0.clone()
+    for t in range(T):
+        x = V[:, t, :, :, None] * K[:, t, :, None, :]                # k[j] v[i] as [i][j]
+        y[:, t] = (R[:, t, :, None, :] * (U[:, :, None, :] * x + S)).sum(-1)
+        S = S * W[:, t, :, None, :] + x
+    # backward_111, first sweep: a thread per key channel i, registers over the value channel j; state[j] = S[j][i]
+    S = S0.clone()
+    gu = torch.zeros(B, H, N, dtype=f)
+    for t in range(T):
+        x = V[:, t, :, :, None] * K[:, t, :, None, :]                # [value j][key i]
+        gr[:, t] = ((U[:, :, None, :] * x + S) * G[:, t, :, :, None]).sum(-2)
+        gu += R[:, t] * (x * G[:, t, :, :, None]).sum(-2)
+        S = S * W[:, t, :, None, :] + x
+    # second sweep, descending: gk
+    D = torch.zeros(B, H, N, N, dtype=f)                             # [value j][key i]
+    for t in range(T - 1, -1, -1):
+        x = G[:, t, :, :, None] * R[:, t, :, None, :]
+        gk[:, t] = ((U[:, :, None, :] * x + D) * V[:, t, :, :, None]).sum(-2)
+        D = x + D * W[:, t, :, None, :]
+    # third sweep, descending: gv, a thread per value channel i, registers over the key channel j
+    D = torch.zeros(B, H, N, N, dtype=f)                             # [value i][key j]
+    for t in range(T - 1, -1, -1):
+        x = G[:, t, :, :, None] * R[:, t, :, None, :]
+        gv[:, t] = ((U[:, :, None, :] * x + D) * K[:, t, :, None, :]).sum(-1)
+        D = x + D * W[:, t, :, None, :]
+    # fourth sweep, ascending: gs[i][j] = sum_t gy_t[i] r_t[j] prod_{z<t} w_z[j]
+    gs = torch.zeros(B, H, N, N, dtype=f)
+    run = torch.ones(B, H, N, dtype=f)
+    for t in range(T):
+        gs += G[:, t, :, :, None] * (run * R[:, t])[:, :, None, :]
+        run = run * W[:, t]
+    # backward_222: a thread per key channel i, registers over the value channel j
+    A = torch.zeros(B, H, N, N, dtype=f)                             # `saaaa`, [value j][key i]
+    sb = torch.zeros(B, T, H, N, dtype=f)                            # `sbbbb`, T - 1 entries used
+    for t in range(T - 1, 1, -1):
+        A = (A + G[:, t, :, :, None] * R[:, t, :, None, :]) * W[:, t - 1, :, None, :]
+        sb[:, t - 1] = (A * V[:, t - 2, :, :, None]).sum(-2) * K[:, t - 2]
+    A = (A + G[:, 1, :, :, None] * R[:, 1, :, None, :]) * W[:, 0, :, None, :]
+    sb[:, 0] = (A * S0).sum(-2)
+    lam = -torch.exp(Wraw)                                           # d(log decay) / d(w_raw)
+    sss = sb[:, 0].clone()
+    gw[:, 0] = sss * lam[:, 0]
+    Cc = S0 * W[:, 0, :, None, :]                                    # `scccc`
+    sss = sss + (sb[:, 1] - (Cc * G[:, 1, :, :, None]).sum(-2) * R[:, 1])
+    gw[:, 1] = sss * lam[:, 1]
+    for t in range(2, T - 1):
+        Cc = (Cc + V[:, t - 2, :, :, None] * K[:, t - 2, :, None, :]) * W[:, t - 1, :, None, :]
+        sss = sss + (sb[:, t] - (Cc * G[:, t, :, :, None]).sum(-2) * R[:, t])
+        gw[:, t] = sss * lam[:, t]
+    gw[:, T - 1] = 0.0
+    flat = lambda x: rb(x.reshape(B, T, C))
+    return [flat(y), flat(gr), flat(gk), flat(gv), flat(gw), rb(gu).sum(0).reshape(H, N), rb(gs)]
