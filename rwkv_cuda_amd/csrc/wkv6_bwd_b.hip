@@ -51,7 +51,6 @@ struct alignas(16) SmemB2 {
     float u[N];
     float pc[N];                       // P per channel, when it changes layout around an exact chunk
     float part[2][NPREP][N];
-    alignas(8) uint8_t flag[2][NPREP]; // per prep wave: some channel decays too fast for the mid-point factors
 };
 
 // ---------------------------------------------------------------------------------------------------- prep waves
@@ -148,21 +147,19 @@ DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base
         }
         const float s4a = s2[0] + x.other[0], s4b = s2[1] + x.other[1];
         *reinterpret_cast<float2*>(&S.part[pb][wid][2 * jp]) = make_float2(s4a, s4b);   // both half-waves hold the same sums
-        // A chunk whose decays could overflow the mid-point factors is redone exactly (see wkv6_chunk.h).
-        const bool fast_decay = (-s4a > 0.25f * RANGE_LIMIT * LOG2E) || (-s4b > 0.25f * RANGE_LIMIT * LOG2E);
-        const unsigned long long any = __ballot(fast_decay);
-        if (lane == 0) S.flag[pb][wid] = any != 0ull ? 1 : 0;
     };
 
     // ---- operands of visit ci into set ci & 1, first part: R' planes, Eb, plain r (K' values stay in registers)
     auto operands_a = [&](const int ci, Raw& x) __attribute__((always_inline)) -> bool {
         SetB& O = S.set[ci & 1];
         const int pb = ci & 1;
-        const uint2 f8 = *reinterpret_cast<const uint2*>(&S.flag[pb][0]);
-        float2 pe[4];
+        float2 pe[4], po[4];
 #pragma unroll
-        for (int w4 = 0; w4 < 4; ++w4) pe[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * second + w4][2 * jp]);
-        const bool exact = __builtin_amdgcn_readfirstlane(f8.x | f8.y) != 0;     // the same in every wave: a scalar
+        for (int w4 = 0; w4 < 4; ++w4) {
+            pe[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * second + w4][2 * jp]);
+            po[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * !second + w4][2 * jp]);
+        }
+        const bool exact = chunk_needs_exact_path(pe, po);                       // the same in every wave: a scalar
         if (tid == 0) O.exact = exact;
         float near[2];
         near[0] = second ? (th ? x.other[0] : 0.f) : (th ? 0.f : x.other[0]);

@@ -146,6 +146,17 @@ constexpr float LN2 = 0.69314718055994530942f;
 constexpr float LAM_CUT = -30.0f;
 DEVINL float gw_factor(float lam) { return lam < LAM_CUT ? 0.f : lam; }
 
+// A chunk takes the step-by-step path when the mid-point factors of some channel could leave the range that the hi / lo
+// bf16 operands are designed for: the decay exponent summed over either half of the chunk beyond RANGE_LIMIT.  Every
+// prep wave holds every channel (a lane per channel pair), so each of them takes this decision from the eight partial sums
+// by itself and all arrive at the same answer.  other[] = the four partial sums of the half this wave does not prepare.
+DEVINL bool chunk_needs_exact_path(const float2 (&own)[4], const float2 (&other)[4]) {
+    const float ax = (own[0].x + own[1].x) + (own[2].x + own[3].x), ay = (own[0].y + own[1].y) + (own[2].y + own[3].y);
+    const float bx = (other[0].x + other[1].x) + (other[2].x + other[3].x), by = (other[0].y + other[1].y) + (other[2].y + other[3].y);
+    const float worst = fminf(fminf(ax, ay), fminf(bx, by));            // exponents are <= 0, in log2 units
+    return __ballot(-worst > RANGE_LIMIT * LOG2E) != 0ull;
+}
+
 template <int CTRL, int ROW_MASK> DEVINL float dpp_add(float x) {
     return x + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, ROW_MASK, 0xf, true));
 }

@@ -44,7 +44,6 @@ struct alignas(16) SmemF {
     float Yx[2][2][L][N];              // exact path: partial y of the two key-channel halves, double buffered
     float u[N];
     float part[2][NPREP][N];           // sums of lam over each eighth of a chunk
-    alignas(8) uint8_t flag[2][NPREP]; // per prep wave: some channel decays too fast for the mid-point factors
 };
 
 // ---------------------------------------------------------------------------------------------------- prep waves
@@ -162,11 +161,6 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         }
         const float s4a = s2[0] + x.other[0], s4b = s2[1] + x.other[1];
         *reinterpret_cast<float2*>(&S.part[pb][wid][2 * jp]) = make_float2(s4a, s4b);   // both half-waves hold the same sums
-        // A chunk whose decays could overflow the mid-point factors is redone exactly.  A half-chunk sum beyond the limit
-        // implies an eighth beyond limit/4, so this local test is sufficient (and conservative).
-        const bool fast_decay = (-s4a > 0.25f * RANGE_LIMIT * LOG2E) || (-s4b > 0.25f * RANGE_LIMIT * LOG2E);
-        const unsigned long long any = __ballot(fast_decay);
-        if (lane == 0) S.flag[pb][wid] = any != 0ull ? 1 : 0;
     };
 
     // ---- operands of chunk c into set c & 1, first part: R' planes (and the K' values kept in registers for the second
@@ -178,12 +172,14 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
         bool exact = exact_head;
         float near[2] = {0.f, 0.f};
         if (!hf) {
-            const uint2 f8 = *reinterpret_cast<const uint2*>(&S.flag[pb][0]);
             // sums of lam over the eighths of this thread's half-chunk; those between this wave's eighth and the middle count
-            float2 pe[4];
+            float2 pe[4], po[4];
 #pragma unroll
-            for (int w4 = 0; w4 < 4; ++w4) pe[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * second + w4][2 * jp]);
-            exact = __builtin_amdgcn_readfirstlane(f8.x | f8.y) != 0;            // the same in every wave: a scalar
+            for (int w4 = 0; w4 < 4; ++w4) {
+                pe[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * second + w4][2 * jp]);
+                po[w4] = *reinterpret_cast<const float2*>(&S.part[pb][4 * !second + w4][2 * jp]);
+            }
+            exact = chunk_needs_exact_path(pe, po);                              // the same in every wave: a scalar
             near[0] = second ? (th ? x.other[0] : 0.f) : (th ? 0.f : x.other[0]);
             near[1] = second ? (th ? x.other[1] : 0.f) : (th ? 0.f : x.other[1]);
             // eighths between this wave's and the middle: first half w_own+1..3, second half 0..w_own-1 (scalar branches)

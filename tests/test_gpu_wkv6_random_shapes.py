@@ -38,10 +38,14 @@ def test_wkv6_state_chunked_equals_sweeps(lib, seed):
     C = H * 64
     print(f"\nseed {seed}: B={B} T={T} H={H}", flush=True)
     r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=100 + seed, state=True)
-    if seed % 2:                                   # some tokens and channels decay fast enough for the exact path
+    if seed % 2:
+        # Single tokens whose decay is strong.  w_raw = 4.5 (the state loses e^-90 in one step) is beyond what the mid-point
+        # factors of a half-chunk may span, so that chunk takes the exact path: about one hit per two chunks and head, exact
+        # and chunked chunks alternate.  w_raw = 2.5 (e^-12) stays on the chunked path with factors of e^+-12.
         g = torch.Generator().manual_seed(seed)
-        mask = torch.rand(B, T, C, generator=g) < 0.0004    # about one hit per chunk and head: exact and chunked chunks alternate
-        w = torch.where(mask, torch.full_like(w, 2.5), w)
+        pick = torch.rand(B, T, C, generator=g)
+        w = torch.where(pick < 0.0002, torch.full_like(w, 4.5), w)
+        w = torch.where((pick >= 0.0002) & (pick < 0.0006), torch.full_like(w, 2.5), w)
     ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
     emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
     d = [x.to(DEV) for x in (r, k, v, w, u, s0, gy)]
