@@ -51,9 +51,9 @@ TRAFFIC_MEASURED = {
     # profiles/wkv5_rows_kernels_B8_T4096_C4096_N128.md
     "wkv_rows<FWD>": 805.4e6 + 268.4e6, "wkv_rows<GR>": 1073.8e6 + 805.4e6,
     "wkv_rows<GV>": 805.4e6 + 268.4e6, "wkv_rows<GK>": 1610.8e6 + 268.5e6,
-    # profiles/wkv4_seg_kernels_B4_T512_C768.md
-    "wkv4_fwd_seg": 29.7e6 + 6.3e6,
-    "wkv4_bwd_seg + wkv4_batch_sum": 186.6e6 + 31.5e6,
+    # profiles/wkv4_reg_kernels_B4_T512_C768.md
+    "wkv4_fwd_reg": 12.7e6 + 6.3e6,
+    "wkv4_bwd_reg + wkv4_batch_sum": 19.1e6 + 12.6e6,
     # profiles/timex_mfma_kernels_B32_C768_T768.md
     "timex_conv_mfma (forward)": 77.9e6 + 75.5e6,
     "timex backward (timex_conv_mfma + timex_gw_sum_mfma)": (77.9e6 + 75.5e6) + (151.1e6 + 2.4e6),
@@ -378,8 +378,8 @@ def make_wkv4(dev):
         call("rwkv_wkv4raw_forward", dev, B, T, C, w_raw, u, k, v, y)
         call("rwkv_wkv4raw_backward", dev, B, T, C, w_raw, u, k, v, gy, gw, gu, gk, gv, ws, nbytes)
 
-    kernels = [("wkv4_fwd_seg", lambda: call("rwkv_wkv4raw_forward", dev, B, T, C, w_raw, u, k, v, y), 12 * C * tok),
-               ("wkv4_bwd_seg + wkv4_batch_sum", lambda: call("rwkv_wkv4raw_backward", dev, B, T, C, w_raw, u, k, v, gy, gw, gu, gk, gv, ws, nbytes), 20 * C * tok)]
+    kernels = [("wkv4_fwd_reg", lambda: call("rwkv_wkv4raw_forward", dev, B, T, C, w_raw, u, k, v, y), 12 * C * tok),
+               ("wkv4_bwd_reg + wkv4_batch_sum", lambda: call("rwkv_wkv4raw_backward", dev, B, T, C, w_raw, u, k, v, gy, gw, gu, gk, gv, ws, nbytes), 20 * C * tok)]
 
     def cpu_baseline():
         from oracle import wkv4 as O

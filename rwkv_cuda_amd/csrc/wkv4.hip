@@ -21,6 +21,25 @@ namespace {
 constexpr int NT = 64;
 constexpr float O_INIT = -65500.0f;
 
+// e^x in six instructions, good to about 1.5 ulp over the whole range (underflow gives 0; the arguments here are finite
+// and their results never overflow; the reference builds its kernel with --use_fast_math, wkv/run.py:87): 2^(x log2 e) by the hardware's own exp2, plus the first-order correction for what
+// the rounded product and the rounded constant lost.
+DEVINL float exp32(float x) {
+    constexpr float L2E_HI = 1.44269502e+00f, L2E_LO = 1.92596299e-08f, LN2 = 0.693147182f;
+    const float t = x * L2E_HI;
+    const float lo = fmaf(x, L2E_LO, fmaf(x, L2E_HI, -t));
+    const float r = __builtin_amdgcn_exp2f(t);
+    return fmaf(r, lo * LN2, r);
+}
+
+// e^{a - max(a,b)} and e^{b - max(a,b)}: one of the two is e^0, so one exponential serves both
+struct ExpPair { float no, ea, eb; };
+DEVINL ExpPair exp_pair(float a, float b) {
+    const float e = exp32(-fabsf(a - b));
+    const bool first = a >= b;
+    return {fmaxf(a, b), first ? 1.0f : e, first ? e : 1.0f};
+}
+
 template <bool RAW>
 __global__ __launch_bounds__(NT) void wkv4_fwd(int BC, int T, int C, const float* __restrict__ w_,
                                               const float* __restrict__ u_, const float* __restrict__ k_,
@@ -38,12 +57,13 @@ __global__ __launch_bounds__(NT) void wkv4_fwd(int BC, int T, int C, const float
     for (int t = 0; t < T; ++t) {
         const size_t ii = static_cast<size_t>(t) * C;
         const float kt = k[ii], vt = v[ii];
-        float no = fmaxf(o, u + kt);
-        float A = expf(o - no), Bq = expf(u + kt - no);
+        ExpPair e = exp_pair(o, u + kt);
+        float no = e.no, A = e.ea, Bq = e.eb;
         y[ii] = (A * p + Bq * vt) / (A * q + Bq);
-        no = fmaxf(w + o, kt);
-        A = expf(w + o - no);
-        Bq = expf(kt - no);
+        e = exp_pair(w + o, kt);
+        no = e.no;
+        A = e.ea;
+        Bq = e.eb;
         p = A * p + Bq * vt;
         q = A * q + Bq;
         o = no;
@@ -64,8 +84,8 @@ struct State3 { float p, q, o; };
 
 // a: the older state, exponent already lowered by the decay over the steps of b
 DEVINL State3 combine(const State3 a, const State3 b) {
-    const float no = fmaxf(a.o, b.o);
-    const float ea = expf(a.o - no), eb = expf(b.o - no);
+    const ExpPair e = exp_pair(a.o, b.o);
+    const float no = e.no, ea = e.ea, eb = e.eb;
     return {ea * a.p + eb * b.p, ea * a.q + eb * b.q, no};
 }
 
@@ -89,8 +109,8 @@ __global__ __launch_bounds__(NTS) void wkv4_fwd_seg(int T, int C, int S, const f
     for (int t = t0; t < t1; ++t) {
         const size_t ii = static_cast<size_t>(t) * C;
         const float kt = k[ii], vt = v[ii];
-        const float no = fmaxf(w + x.o, kt);
-        const float A = expf(w + x.o - no), Bq = expf(kt - no);
+        const ExpPair e = exp_pair(w + x.o, kt);
+        const float no = e.no, A = e.ea, Bq = e.eb;
         x.p = A * x.p + Bq * vt;
         x.q = A * x.q + Bq;
         x.o = no;
@@ -118,12 +138,13 @@ __global__ __launch_bounds__(NTS) void wkv4_fwd_seg(int T, int C, int S, const f
     for (int t = t0; t < t1; ++t) {
         const size_t ii = static_cast<size_t>(t) * C;
         const float kt = k[ii], vt = v[ii];
-        float no = fmaxf(x.o, u + kt);
-        float A = expf(x.o - no), Bq = expf(u + kt - no);
+        ExpPair e = exp_pair(x.o, u + kt);
+        float no = e.no, A = e.ea, Bq = e.eb;
         if (live) y[ii] = (A * x.p + Bq * vt) / (A * x.q + Bq);
-        no = fmaxf(w + x.o, kt);
-        A = expf(w + x.o - no);
-        Bq = expf(kt - no);
+        e = exp_pair(w + x.o, kt);
+        no = e.no;
+        A = e.ea;
+        Bq = e.eb;
         x.p = A * x.p + Bq * vt;
         x.q = A * x.q + Bq;
         x.o = no;
@@ -154,8 +175,8 @@ __global__ __launch_bounds__(NT) void wkv4_bwd(int BC, int T, int C, const float
     for (int t = 0; t < T; ++t) {
         const size_t ii = static_cast<size_t>(t) * C;
         const float kt = k[ii], vt = v[ii], gt = gy[ii];
-        float no = fmaxf(o, kt + u);
-        float A = expf(o - no), Bq = expf(kt + u - no);
+        ExpPair e = exp_pair(o, kt + u);
+        float no = e.no, A = e.ea, Bq = e.eb;
         const float num = A * p + Bq * vt;
         const float iden = 1.0f / (A * q + Bq);
         const float y = num * iden;
@@ -164,9 +185,10 @@ __global__ __launch_bounds__(NT) void wkv4_bwd(int BC, int T, int C, const float
         ze[ii] = kt + u - no;
         gw += gt * (dpdw - dqdw * y) * iden * A;
         gu += gt * (vt - y) * Bq * iden;
-        no = fmaxf(w + o, kt);
-        A = expf(w + o - no);
-        Bq = expf(kt - no);
+        e = exp_pair(w + o, kt);
+        no = e.no;
+        A = e.ea;
+        Bq = e.eb;
         dpdw = A * (p + dpdw);
         dqdw = A * (q + dqdw);
         p = A * p + Bq * vt;
@@ -180,13 +202,14 @@ __global__ __launch_bounds__(NT) void wkv4_bwd(int BC, int T, int C, const float
         const size_t ii = static_cast<size_t>(t) * C;
         const float kt = k[ii], vt = v[ii], gt = gy[ii];
         const float y = gv[ii], z = gk[ii], zexp = ze[ii];
-        float A = gt * z * expf(zexp);
-        float Bq = expf(kt + o);
+        float A = gt * z * exp32(zexp);
+        float Bq = exp32(kt + o);
         gk[ii] = A * (vt - y) + Bq * (gp * vt + gq);
         gv[ii] = A + Bq * gp;
-        const float no = fmaxf(w + o, zexp - kt - u);
-        A = expf(w + o - no);
-        Bq = gt * z * expf(zexp - kt - u - no);
+        const ExpPair e2 = exp_pair(w + o, zexp - kt - u);
+        const float no = e2.no;
+        A = e2.ea;
+        Bq = gt * z * e2.eb;
         gp = A * gp + Bq;
         gq = A * gq - Bq * y;
         o = no;
@@ -208,8 +231,8 @@ __global__ __launch_bounds__(NT) void wkv4_bwd(int BC, int T, int C, const float
 struct State5 { float p, q, dp, dq, o; };
 
 DEVINL State5 combine(const State5 a, const State5 b) {
-    const float no = fmaxf(a.o, b.o);
-    const float ea = expf(a.o - no), eb = expf(b.o - no);
+    const ExpPair e = exp_pair(a.o, b.o);
+    const float no = e.no, ea = e.ea, eb = e.eb;
     return {ea * a.p + eb * b.p, ea * a.q + eb * b.q, ea * a.dp + eb * b.dp, ea * a.dq + eb * b.dq, no};
 }
 
@@ -242,8 +265,8 @@ __global__ __launch_bounds__(NTS) void wkv4_bwd_seg(int T, int C, int S, const f
     for (int t = t0; t < t1; ++t) {
         const size_t ii = static_cast<size_t>(t) * C;
         const float kt = k[ii], vt = v[ii];
-        const float no = fmaxf(w + x.o, kt);
-        const float A = expf(w + x.o - no), Bq = expf(kt - no);
+        const ExpPair e = exp_pair(w + x.o, kt);
+        const float no = e.no, A = e.ea, Bq = e.eb;
         x.dp = A * (x.p + x.dp);
         x.dq = A * (x.q + x.dq);
         x.p = A * x.p + Bq * vt;
@@ -277,8 +300,8 @@ __global__ __launch_bounds__(NTS) void wkv4_bwd_seg(int T, int C, int S, const f
     for (int t = t0; t < t1; ++t) {
         const size_t ii = static_cast<size_t>(t) * C;
         const float kt = k[ii], vt = v[ii], gt = gy[ii];
-        float no = fmaxf(x.o, kt + u);
-        float A = expf(x.o - no), Bq = expf(kt + u - no);
+        ExpPair e = exp_pair(x.o, kt + u);
+        float no = e.no, A = e.ea, Bq = e.eb;
         const float num = A * x.p + Bq * vt;
         const float iden = 1.0f / (A * x.q + Bq);
         const float y = num * iden;
@@ -287,9 +310,10 @@ __global__ __launch_bounds__(NTS) void wkv4_bwd_seg(int T, int C, int S, const f
         ze[ii] = kt + u - no;
         gw += gt * (x.dp - x.dq * y) * iden * A;
         gu += gt * (vt - y) * Bq * iden;
-        no = fmaxf(w + x.o, kt);
-        A = expf(w + x.o - no);
-        Bq = expf(kt - no);
+        e = exp_pair(w + x.o, kt);
+        no = e.no;
+        A = e.ea;
+        Bq = e.eb;
         x.dp = A * (x.p + x.dp);
         x.dq = A * (x.q + x.dq);
         x.p = A * x.p + Bq * vt;
@@ -303,8 +327,8 @@ __global__ __launch_bounds__(NTS) void wkv4_bwd_seg(int T, int C, int S, const f
         const size_t ii = static_cast<size_t>(t) * C;
         const float kt = k[ii], gt = gy[ii];
         const float y = gv[ii], z = gk[ii], zexp = ze[ii];
-        const float no = fmaxf(w + g.o, zexp - kt - u);
-        const float A = expf(w + g.o - no), Bq = gt * z * expf(zexp - kt - u - no);
+        const ExpPair e = exp_pair(w + g.o, zexp - kt - u);
+        const float no = e.no, A = e.ea, Bq = gt * z * e.eb;
         g.p = A * g.p + Bq;
         g.q = A * g.q - Bq * y;
         g.o = no;
@@ -335,13 +359,14 @@ __global__ __launch_bounds__(NTS) void wkv4_bwd_seg(int T, int C, int S, const f
         const size_t ii = static_cast<size_t>(t) * C;
         const float kt = k[ii], vt = v[ii], gt = gy[ii];
         const float y = gv[ii], z = gk[ii], zexp = ze[ii];
-        float A = gt * z * expf(zexp);
-        float Bq = expf(kt + g.o);
+        float A = gt * z * exp32(zexp);
+        float Bq = exp32(kt + g.o);
         gk[ii] = A * (vt - y) + Bq * (g.p * vt + g.q);
         gv[ii] = A + Bq * g.p;
-        const float no = fmaxf(w + g.o, zexp - kt - u);
-        A = expf(w + g.o - no);
-        Bq = gt * z * expf(zexp - kt - u - no);
+        const ExpPair e2 = exp_pair(w + g.o, zexp - kt - u);
+        const float no = e2.no;
+        A = e2.ea;
+        Bq = gt * z * e2.eb;
         g.p = A * g.p + Bq;
         g.q = A * g.q - Bq * y;
         g.o = no;
@@ -365,6 +390,256 @@ __global__ __launch_bounds__(NTS) void wkv4_bwd_seg(int T, int C, int S, const f
     }
 }
 
+// ---------------------------------------------------------------------------------------- time-parallel, inputs in registers
+// Up to NSEG * 16 = 1024 steps (the reference's own limit, wkv/run.py:149,153) a segment is at most 16 steps long,
+// and a lane can hold its segment's k, v, gy and, in the backward, what the ascending sweep hands to the descending one
+// (y_t, 1/den_t, zexp_t) in registers: every input is fetched once, all loads of a segment are in flight together
+// instead of one dependent load per step and sweep, and the backward needs no workspace.  The arithmetic and its order
+// are those of wkv4_fwd_seg / wkv4_bwd_seg, so the results are the same bit for bit.
+//   CHR channels x NSEG segments per workgroup; SM = the most steps a segment may have (8 with 16 channels, 16 with 8).
+// Workgroups are handed to the chip's 8 XCDs in turn, each with an L2 of its own, and a workgroup's 16 channels are half of
+// a 128-byte line: numbered as launched, the two workgroups that share every line would sit on different XCDs and each
+// L2 would fetch the whole line.  Workgroup x of XCD d takes piece d * (n / 8) + x instead, so neighbours share an L2.
+DEVINL int paired_workgroup(int launched, int n) {
+    return n % 16 == 0 ? (launched % 8) * (n / 8) + launched / 8 : launched;
+}
+
+template <bool RAW, int CHR, int SM>
+__global__ __launch_bounds__(CHR * NSEG) void wkv4_fwd_reg(int T, int C, int S, const float* __restrict__ w_,
+                                                          const float* __restrict__ u_, const float* __restrict__ k_,
+                                                          const float* __restrict__ v_, float* __restrict__ y_) {
+    __shared__ State3 X[2][NSEG][CHR];
+    const int cl = threadIdx.x % CHR, s = threadIdx.x / CHR;
+    const int q = paired_workgroup(blockIdx.x, gridDim.x), nx = (C + CHR - 1) / CHR;
+    const int c = (q % nx) * CHR + cl, b = q / nx;
+    const bool live = c < C;
+    const int cc = live ? c : C - 1;
+    const float u = u_[cc], w = RAW ? -expf(w_[cc]) : w_[cc];        // RAW: the wrapper's w = -exp(w_raw) done here
+    const int t0 = min(s * S, T), n = live ? min(t0 + S, T) - t0 : 0;
+    const size_t off = (static_cast<size_t>(b) * T + t0) * C + cc;
+    const float* __restrict__ k = k_ + off;
+    const float* __restrict__ v = v_ + off;
+    float* __restrict__ y = y_ + off;
+
+    float kk[SM], vv[SM];
+#pragma unroll
+    for (int j = 0; j < SM; ++j) {
+        kk[j] = 0.f; vv[j] = 0.f;
+        if (j < n) { kk[j] = k[static_cast<size_t>(j) * C]; vv[j] = v[static_cast<size_t>(j) * C]; }
+    }
+    State3 x = {0.f, 0.f, O_INIT};
+#pragma unroll
+    for (int j = 0; j < SM; ++j) {
+        if (j < n) {
+            const ExpPair e = exp_pair(w + x.o, kk[j]);
+            const float no = e.no, A = e.ea, Bq = e.eb;
+            x.p = A * x.p + Bq * vv[j];
+            x.q = A * x.q + Bq;
+            x.o = no;
+        }
+    }
+    X[0][s][cl] = x;
+    __syncthreads();
+    int cur = 0;
+#pragma unroll
+    for (int d = 1; d < NSEG; d *= 2) {
+        State3 mine = X[cur][s][cl];
+        if (s >= d) {
+            State3 older = X[cur][s - d][cl];
+            older.o += static_cast<float>(d * S) * w;
+            mine = combine(older, mine);
+        }
+        X[cur ^ 1][s][cl] = mine;
+        cur ^= 1;
+        __syncthreads();
+    }
+    x = State3{0.f, 0.f, O_INIT};
+    if (s > 0) x = X[cur][s - 1][cl];
+#pragma unroll
+    for (int j = 0; j < SM; ++j) {
+        if (j < n) {
+            ExpPair e = exp_pair(x.o, u + kk[j]);
+            float no = e.no, A = e.ea, Bq = e.eb;
+            y[static_cast<size_t>(j) * C] = (A * x.p + Bq * vv[j]) / (A * x.q + Bq);
+            e = exp_pair(w + x.o, kk[j]);
+            no = e.no;
+            A = e.ea;
+            Bq = e.eb;
+            x.p = A * x.p + Bq * vv[j];
+            x.q = A * x.q + Bq;
+            x.o = no;
+        }
+    }
+}
+
+template <bool RAW, int CHR, int SM>
+__global__ __launch_bounds__(CHR * NSEG) void wkv4_bwd_reg(int T, int C, int S, const float* __restrict__ w_,
+                                                          const float* __restrict__ u_, const float* __restrict__ k_,
+                                                          const float* __restrict__ v_, const float* __restrict__ gy_,
+                                                          float* __restrict__ gw_, float* __restrict__ gu_,
+                                                          float* __restrict__ gk_, float* __restrict__ gv_) {
+    __shared__ State5 X[2][NSEG][CHR];
+    const int cl = threadIdx.x % CHR, s = threadIdx.x / CHR;
+    const int q = paired_workgroup(blockIdx.x, gridDim.x), nx = (C + CHR - 1) / CHR;
+    const int c = (q % nx) * CHR + cl, b = q / nx;
+    const bool live = c < C;
+    const int cc = live ? c : C - 1;
+    const float u = u_[cc], w = RAW ? -expf(w_[cc]) : w_[cc];        // RAW: the wrapper's w = -exp(w_raw) done here
+    // lanes past C have no steps: they only keep the barriers company
+    const int t0 = min(s * S, T), n = live ? min(t0 + S, T) - t0 : 0;
+    const size_t off = (static_cast<size_t>(b) * T + t0) * C + cc;
+    const float* __restrict__ k = k_ + off;
+    const float* __restrict__ v = v_ + off;
+    const float* __restrict__ gy = gy_ + off;
+    float* __restrict__ gk = gk_ + off;
+    float* __restrict__ gv = gv_ + off;
+    const float span = static_cast<float>(S);
+
+    float kk[SM], vv[SM], gg[SM], yy[SM], zz[SM], ze[SM];
+#pragma unroll
+    for (int j = 0; j < SM; ++j) {
+        kk[j] = 0.f; vv[j] = 0.f; gg[j] = 0.f;
+        if (j < n) {
+            kk[j] = k[static_cast<size_t>(j) * C]; vv[j] = v[static_cast<size_t>(j) * C]; gg[j] = gy[static_cast<size_t>(j) * C];
+        }
+    }
+
+    // ---- ascending: the segment alone
+    State5 x = {0.f, 0.f, 0.f, 0.f, O_INIT};
+#pragma unroll
+    for (int j = 0; j < SM; ++j) {
+        if (j < n) {
+            const ExpPair e = exp_pair(w + x.o, kk[j]);
+            const float no = e.no, A = e.ea, Bq = e.eb;
+            x.dp = A * (x.p + x.dp);
+            x.dq = A * (x.q + x.dq);
+            x.p = A * x.p + Bq * vv[j];
+            x.q = A * x.q + Bq;
+            x.o = no;
+        }
+    }
+    X[0][s][cl] = x;
+    __syncthreads();
+    int cur = 0;
+#pragma unroll
+    for (int d = 1; d < NSEG; d *= 2) {
+        State5 mine = X[cur][s][cl];
+        if (s >= d) {
+            State5 older = X[cur][s - d][cl];
+            const float m = static_cast<float>(d) * span;
+            older.dp += m * older.p;
+            older.dq += m * older.q;
+            older.o += m * w;
+            mine = combine(older, mine);
+        }
+        X[cur ^ 1][s][cl] = mine;
+        cur ^= 1;
+        __syncthreads();
+    }
+    x = State5{0.f, 0.f, 0.f, 0.f, O_INIT};
+    if (s > 0) x = X[cur][s - 1][cl];
+    __syncthreads();                               // X is reused below
+
+    // ---- ascending, from the true state: y, 1/den and zexp stay in registers for the descending sweep
+    float gw = 0.f, gu = 0.f;
+#pragma unroll
+    for (int j = 0; j < SM; ++j) {
+        yy[j] = 0.f; zz[j] = 0.f; ze[j] = 0.f;
+        if (j < n) {
+            const float kt = kk[j], vt = vv[j], gt = gg[j];
+            ExpPair e = exp_pair(x.o, kt + u);
+            float no = e.no, A = e.ea, Bq = e.eb;
+            const float num = A * x.p + Bq * vt;
+            const float iden = 1.0f / (A * x.q + Bq);
+            const float y = num * iden;
+            yy[j] = y;
+            zz[j] = iden;
+            ze[j] = kt + u - no;
+            gw += gt * (x.dp - x.dq * y) * iden * A;
+            gu += gt * (vt - y) * Bq * iden;
+            e = exp_pair(w + x.o, kt);
+            no = e.no;
+            A = e.ea;
+            Bq = e.eb;
+            x.dp = A * (x.p + x.dp);
+            x.dq = A * (x.q + x.dq);
+            x.p = A * x.p + Bq * vt;
+            x.q = A * x.q + Bq;
+            x.o = no;
+        }
+    }
+
+    // ---- descending: the segment alone (p, q stand for gp, gq)
+    State3 g = {0.f, 0.f, O_INIT};
+#pragma unroll
+    for (int j = SM - 1; j >= 0; --j) {
+        if (j < n) {
+            const ExpPair e = exp_pair(w + g.o, ze[j] - kk[j] - u);
+            const float no = e.no, A = e.ea, Bq = gg[j] * zz[j] * e.eb;
+            g.p = A * g.p + Bq;
+            g.q = A * g.q - Bq * yy[j];
+            g.o = no;
+        }
+    }
+    State3 (*G)[NSEG][CHR] = reinterpret_cast<State3 (*)[NSEG][CHR]>(&X[0][0][0]);  // [2][NSEG][CHR], inside X
+    const int rs = NSEG - 1 - s;                   // position in the descending order
+    G[0][rs][cl] = g;
+    __syncthreads();
+    cur = 0;
+#pragma unroll
+    for (int d = 1; d < NSEG; d *= 2) {
+        State3 mine = G[cur][rs][cl];
+        if (rs >= d) {
+            State3 older = G[cur][rs - d][cl];
+            older.o += static_cast<float>(d) * span * w;
+            mine = combine(older, mine);
+        }
+        G[cur ^ 1][rs][cl] = mine;
+        cur ^= 1;
+        __syncthreads();
+    }
+    g = State3{0.f, 0.f, O_INIT};
+    if (rs > 0) g = G[cur][rs - 1][cl];
+    __syncthreads();
+
+    // ---- descending, from the true state
+#pragma unroll
+    for (int j = SM - 1; j >= 0; --j) {
+        if (j < n) {
+            const float kt = kk[j], vt = vv[j], gt = gg[j];
+            const float y = yy[j], z = zz[j], zexp = ze[j];
+            float A = gt * z * exp32(zexp);
+            float Bq = exp32(kt + g.o);
+            gk[static_cast<size_t>(j) * C] = A * (vt - y) + Bq * (g.p * vt + g.q);
+            gv[static_cast<size_t>(j) * C] = A + Bq * g.p;
+            const ExpPair e2 = exp_pair(w + g.o, zexp - kt - u);
+            const float no = e2.no;
+            A = e2.ea;
+            Bq = gt * z * e2.eb;
+            g.p = A * g.p + Bq;
+            g.q = A * g.q - Bq * y;
+            g.o = no;
+        }
+    }
+
+    // ---- gw, gu: the segments' sums, added in time order
+    float2* part = reinterpret_cast<float2*>(&X[0][0][0]);                         // [NSEG][CHR]
+    part[s * CHR + cl] = make_float2(gw, gu);
+    __syncthreads();
+    if (s == 0 && live) {
+        float a = 0.f, bsum = 0.f;
+        for (int z = 0; z < NSEG; ++z) { a += part[z * CHR + cl].x; bsum += part[z * CHR + cl].y; }
+        // the caller's buffers are accumulated into, as the reference does (wkv_cuda_v2.cu:112-113)
+        if constexpr (RAW) {                        // per-batch partials in the library's own scratch: plain stores
+            gw_[static_cast<size_t>(b) * C + c] = a * w;
+            gu_[static_cast<size_t>(b) * C + c] = bsum;
+        } else {
+            gw_[static_cast<size_t>(b) * C + c] += a * w;
+            gu_[static_cast<size_t>(b) * C + c] += bsum;
+        }
+    }
+}
+
 // out[c] = sum_b part[b][c], in the fixed order b = 0, 1, ...: the wrapper's torch.sum(gw, dim=0) (wkv/run.py:115-116)
 __global__ __launch_bounds__(256) void wkv4_batch_sum(int B, int C, const float* __restrict__ pw, const float* __restrict__ pu,
                                                       float* __restrict__ gw, float* __restrict__ gu) {
@@ -373,6 +648,48 @@ __global__ __launch_bounds__(256) void wkv4_batch_sum(int B, int C, const float*
     float a = 0.f, b2 = 0.f;
     for (int b = 0; b < B; ++b) { a += pw[static_cast<size_t>(b) * C + c]; b2 += pu[static_cast<size_t>(b) * C + c]; }
     gw[c] = a; gu[c] = b2;
+}
+
+// Which form runs: one lane per scan beyond the grid's y range, inputs in registers while a segment has at most 16
+// steps, the form that parks the ascending sweep's results in memory beyond that.
+template <bool RAW, int CHR, int SM, typename... Ptrs>
+void launch4_fwd_reg(hipStream_t st, int B, int T, int C, int S, Ptrs... p) {
+    hipLaunchKernelGGL((wkv4_fwd_reg<RAW, CHR, SM>), dim3(((C + CHR - 1) / CHR) * B), dim3(CHR * NSEG), 0, st, T, C, S, p...);
+}
+template <bool RAW, int CHR, int SM, typename... Ptrs>
+void launch4_bwd_reg(hipStream_t st, int B, int T, int C, int S, Ptrs... p) {
+    hipLaunchKernelGGL((wkv4_bwd_reg<RAW, CHR, SM>), dim3(((C + CHR - 1) / CHR) * B), dim3(CHR * NSEG), 0, st, T, C, S, p...);
+}
+
+template <bool RAW>
+void launch4_fwd(hipStream_t st, int B, int T, int C, const float* w, const float* u, const float* k, const float* v, float* y) {
+    const int S = (T + NSEG - 1) / NSEG;
+    if (B > 65535) {
+        const int BC = B * C;
+        hipLaunchKernelGGL((wkv4_fwd<RAW>), dim3((BC + NT - 1) / NT), dim3(NT), 0, st, BC, T, C, w, u, k, v, y);
+    } else if (S <= 8) {
+        launch4_fwd_reg<RAW, 16, 8>(st, B, T, C, S, w, u, k, v, y);
+    } else if (S <= 16) {
+        launch4_fwd_reg<RAW, 8, 16>(st, B, T, C, S, w, u, k, v, y);
+    } else {
+        hipLaunchKernelGGL((wkv4_fwd_seg<RAW>), dim3((C + CH - 1) / CH, B), dim3(NTS), 0, st, T, C, S, w, u, k, v, y);
+    }
+}
+
+template <bool RAW>
+void launch4_bwd(hipStream_t st, int B, int T, int C, const float* w, const float* u, const float* k, const float* v,
+                 const float* gy, float* gw, float* gu, float* gk, float* gv, float* ze) {
+    const int S = (T + NSEG - 1) / NSEG;
+    if (B > 65535) {
+        const int BC = B * C;
+        hipLaunchKernelGGL((wkv4_bwd<RAW>), dim3((BC + NT - 1) / NT), dim3(NT), 0, st, BC, T, C, w, u, k, v, gy, gw, gu, gk, gv, ze);
+    } else if (S <= 8) {
+        launch4_bwd_reg<RAW, 16, 8>(st, B, T, C, S, w, u, k, v, gy, gw, gu, gk, gv);
+    } else if (S <= 16) {
+        launch4_bwd_reg<RAW, 8, 16>(st, B, T, C, S, w, u, k, v, gy, gw, gu, gk, gv);
+    } else {
+        hipLaunchKernelGGL((wkv4_bwd_seg<RAW>), dim3((C + CH - 1) / CH, B), dim3(NTS), 0, st, T, C, S, w, u, k, v, gy, gw, gu, gk, gv, ze);
+    }
 }
 
 int check4(int B, int T, int C) {
@@ -416,14 +733,7 @@ int rwkv_wkv4_forward(void* stream, int B, int T, int C, const float* w, const f
                       const float* v, float* y) {
     if (int e = check4(B, T, C)) return e;
     if (int e = check_ptrs({w, u, k, v, y})) return e;
-    if (B > 65535) {                            // beyond the grid's y range: the one-lane-per-scan kernel
-        const int BC = B * C;
-        hipLaunchKernelGGL(wkv4_fwd<false>, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
-                           BC, T, C, w, u, k, v, y);
-        return launch_status();
-    }
-    hipLaunchKernelGGL(wkv4_fwd_seg<false>, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
-                       T, C, (T + NSEG - 1) / NSEG, w, u, k, v, y);
+    launch4_fwd<false>(static_cast<hipStream_t>(stream), B, T, C, w, u, k, v, y);
     return launch_status();
 }
 
@@ -439,14 +749,7 @@ int rwkv_wkv4_backward(void* stream, int B, int T, int C, const float* w, const 
     if (int e = check_ptrs({w, u, k, v, gy, gw, gu, gk, gv})) return e;
     if (workspace == nullptr || !aligned16(workspace) || workspace_bytes < rwkv_wkv4_backward_workspace_bytes(B, T, C))
         return RWKV_ERR_WORKSPACE;
-    if (B > 65535) {                            // beyond the grid's y range: the one-lane-per-scan kernel
-        const int BC = B * C;
-        hipLaunchKernelGGL(wkv4_bwd<false>, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
-                           BC, T, C, w, u, k, v, gy, gw, gu, gk, gv, static_cast<float*>(workspace));
-        return launch_status();
-    }
-    hipLaunchKernelGGL(wkv4_bwd_seg<false>, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
-                       T, C, (T + NSEG - 1) / NSEG, w, u, k, v, gy, gw, gu, gk, gv, static_cast<float*>(workspace));
+    launch4_bwd<false>(static_cast<hipStream_t>(stream), B, T, C, w, u, k, v, gy, gw, gu, gk, gv, static_cast<float*>(workspace));
     return launch_status();
 }
 
@@ -455,14 +758,7 @@ int rwkv_wkv4raw_forward(void* stream, int B, int T, int C, const float* w_raw, 
                          const float* v, float* y) {
     if (int e = check4(B, T, C)) return e;
     if (int e = check_ptrs({w_raw, u, k, v, y})) return e;
-    if (B > 65535) {
-        const int BC = B * C;
-        hipLaunchKernelGGL(wkv4_fwd<true>, dim3((BC + NT - 1) / NT), dim3(NT), 0, static_cast<hipStream_t>(stream),
-                           BC, T, C, w_raw, u, k, v, y);
-        return launch_status();
-    }
-    hipLaunchKernelGGL(wkv4_fwd_seg<true>, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, static_cast<hipStream_t>(stream),
-                       T, C, (T + NSEG - 1) / NSEG, w_raw, u, k, v, y);
+    launch4_fwd<true>(static_cast<hipStream_t>(stream), B, T, C, w_raw, u, k, v, y);
     return launch_status();
 }
 
@@ -482,13 +778,7 @@ int rwkv_wkv4raw_backward(void* stream, int B, int T, int C, const float* w_raw,
     float* ze = static_cast<float*>(workspace);
     float* pw = ze + static_cast<size_t>(B) * T * C;
     float* pu = pw + static_cast<size_t>(B) * C;
-    if (B > 65535) {
-        const int BC = B * C;
-        hipLaunchKernelGGL(wkv4_bwd<true>, dim3((BC + NT - 1) / NT), dim3(NT), 0, st, BC, T, C, w_raw, u, k, v, gy, pw, pu, gk, gv, ze);
-    } else {
-        hipLaunchKernelGGL(wkv4_bwd_seg<true>, dim3((C + CH - 1) / CH, B), dim3(NTS), 0, st,
-                           T, C, (T + NSEG - 1) / NSEG, w_raw, u, k, v, gy, pw, pu, gk, gv, ze);
-    }
+    launch4_bwd<true>(st, B, T, C, w_raw, u, k, v, gy, pw, pu, gk, gv, ze);
     hipLaunchKernelGGL(wkv4_batch_sum, dim3((C + 255) / 256), dim3(256), 0, st, B, C, pw, pu, gw, gu);
     return launch_status();
 }
