@@ -640,6 +640,264 @@ __global__ __launch_bounds__(CHR * NSEG) void wkv4_bwd_reg(int T, int C, int S, 
     }
 }
 
+// ------------------------------------------------------------------------------- longer sequences: blocks of 512 steps
+// Beyond NSEG * 16 steps a workgroup walks over blocks of NSEG * 8 steps and hands the state from block to block: inside
+// a block everything is as in the register kernels, and the state in front of a segment is the block's entering state,
+// aged by the steps in between, combined with the segments of the block before it.  The backward first walks up with
+// the ascending sweep's summaries only (k, v read, nothing written) to learn the state entering every block, keeps those
+// in LDS, then walks down block by block doing both sweeps.  k and v are read twice, gy once, nothing is parked in memory.
+constexpr int BLK_S = 8, BLK_T = NSEG * BLK_S, BLK_CH = 16;
+constexpr int BLK_MAX = 64;            // blocks whose entering states fit in LDS: T <= 32768
+
+DEVINL State3 aged(State3 a, float steps, float w) { a.o += steps * w; return a; }
+DEVINL State5 aged(State5 a, float steps, float w) {
+    a.dp += steps * a.p;
+    a.dq += steps * a.q;
+    a.o += steps * w;
+    return a;
+}
+
+template <bool RAW>
+__global__ __launch_bounds__(BLK_CH * NSEG) void wkv4_fwd_blk(int T, int C, const float* __restrict__ w_,
+                                                             const float* __restrict__ u_, const float* __restrict__ k_,
+                                                             const float* __restrict__ v_, float* __restrict__ y_) {
+    __shared__ State3 X[2][NSEG][BLK_CH];
+    const int cl = threadIdx.x % BLK_CH, s = threadIdx.x / BLK_CH;
+    const int q = paired_workgroup(blockIdx.x, gridDim.x), nx = (C + BLK_CH - 1) / BLK_CH;
+    const int c = (q % nx) * BLK_CH + cl, b = q / nx;
+    const bool live = c < C;
+    const int cc = live ? c : C - 1;
+    const float u = u_[cc], w = RAW ? -expf(w_[cc]) : w_[cc];        // RAW: the wrapper's w = -exp(w_raw) done here
+    const int nblk = (T + BLK_T - 1) / BLK_T;
+    State3 carry = {0.f, 0.f, O_INIT};             // the state entering the block; every lane of a channel holds it
+
+    for (int blk = 0; blk < nblk; ++blk) {
+        const int t0 = min(blk * BLK_T + s * BLK_S, T), n = live ? min(t0 + BLK_S, T) - t0 : 0;
+        const size_t off = (static_cast<size_t>(b) * T + t0) * C + cc;
+        const float* __restrict__ k = k_ + off;
+        const float* __restrict__ v = v_ + off;
+        float* __restrict__ y = y_ + off;
+        float kk[BLK_S], vv[BLK_S];
+#pragma unroll
+        for (int j = 0; j < BLK_S; ++j) {
+            kk[j] = 0.f; vv[j] = 0.f;
+            if (j < n) { kk[j] = k[static_cast<size_t>(j) * C]; vv[j] = v[static_cast<size_t>(j) * C]; }
+        }
+        State3 x = {0.f, 0.f, O_INIT};
+#pragma unroll
+        for (int j = 0; j < BLK_S; ++j) {
+            if (j < n) {
+                const ExpPair e = exp_pair(w + x.o, kk[j]);
+                x.p = e.ea * x.p + e.eb * vv[j];
+                x.q = e.ea * x.q + e.eb;
+                x.o = e.no;
+            }
+        }
+        X[0][s][cl] = x;
+        __syncthreads();
+        int cur = 0;
+#pragma unroll
+        for (int d = 1; d < NSEG; d *= 2) {
+            State3 mine = X[cur][s][cl];
+            if (s >= d) mine = combine(aged(X[cur][s - d][cl], static_cast<float>(d * BLK_S), w), mine);
+            X[cur ^ 1][s][cl] = mine;
+            cur ^= 1;
+            __syncthreads();
+        }
+        x = aged(carry, static_cast<float>(s * BLK_S), w);
+        if (s > 0) x = combine(x, X[cur][s - 1][cl]);
+        carry = combine(aged(carry, static_cast<float>(BLK_T), w), X[cur][NSEG - 1][cl]);
+#pragma unroll
+        for (int j = 0; j < BLK_S; ++j) {
+            if (j < n) {
+                ExpPair e = exp_pair(x.o, u + kk[j]);
+                y[static_cast<size_t>(j) * C] = (e.ea * x.p + e.eb * vv[j]) / (e.ea * x.q + e.eb);
+                e = exp_pair(w + x.o, kk[j]);
+                x.p = e.ea * x.p + e.eb * vv[j];
+                x.q = e.ea * x.q + e.eb;
+                x.o = e.no;
+            }
+        }
+        __syncthreads();                           // X is written again by the next block
+    }
+}
+
+template <bool RAW>
+__global__ __launch_bounds__(BLK_CH * NSEG) void wkv4_bwd_blk(int T, int C, const float* __restrict__ w_,
+                                                             const float* __restrict__ u_, const float* __restrict__ k_,
+                                                             const float* __restrict__ v_, const float* __restrict__ gy_,
+                                                             float* __restrict__ gw_, float* __restrict__ gu_,
+                                                             float* __restrict__ gk_, float* __restrict__ gv_) {
+    __shared__ State5 X[2][NSEG][BLK_CH];
+    __shared__ State5 ENTER[BLK_MAX][BLK_CH];      // the ascending sweep's state entering each block
+    const int cl = threadIdx.x % BLK_CH, s = threadIdx.x / BLK_CH;
+    const int q = paired_workgroup(blockIdx.x, gridDim.x), nx = (C + BLK_CH - 1) / BLK_CH;
+    const int c = (q % nx) * BLK_CH + cl, b = q / nx;
+    const bool live = c < C;
+    const int cc = live ? c : C - 1;
+    const float u = u_[cc], w = RAW ? -expf(w_[cc]) : w_[cc];        // RAW: the wrapper's w = -exp(w_raw) done here
+    const int nblk = (T + BLK_T - 1) / BLK_T;
+    const size_t row = static_cast<size_t>(b) * T;
+
+    // the segment alone, from the empty state, then the scan over the block's segments: X[cur] holds the inclusive prefixes
+    auto summaries = [&](const float (&kk)[BLK_S], const float (&vv)[BLK_S], int n) -> int {
+        State5 x = {0.f, 0.f, 0.f, 0.f, O_INIT};
+#pragma unroll
+        for (int j = 0; j < BLK_S; ++j) {
+            if (j < n) {
+                const ExpPair e = exp_pair(w + x.o, kk[j]);
+                x.dp = e.ea * (x.p + x.dp);
+                x.dq = e.ea * (x.q + x.dq);
+                x.p = e.ea * x.p + e.eb * vv[j];
+                x.q = e.ea * x.q + e.eb;
+                x.o = e.no;
+            }
+        }
+        X[0][s][cl] = x;
+        __syncthreads();
+        int cur = 0;
+#pragma unroll
+        for (int d = 1; d < NSEG; d *= 2) {
+            State5 mine = X[cur][s][cl];
+            if (s >= d) mine = combine(aged(X[cur][s - d][cl], static_cast<float>(d * BLK_S), w), mine);
+            X[cur ^ 1][s][cl] = mine;
+            cur ^= 1;
+            __syncthreads();
+        }
+        return cur;
+    };
+
+    // ---- up: the state entering every block
+    State5 carry = {0.f, 0.f, 0.f, 0.f, O_INIT};
+    for (int blk = 0; blk < nblk; ++blk) {
+        if (s == 0) ENTER[blk][cl] = carry;
+        if (blk == nblk - 1) break;
+        const int t0 = min(blk * BLK_T + s * BLK_S, T), n = live ? min(t0 + BLK_S, T) - t0 : 0;
+        const size_t off = (row + t0) * C + cc;
+        float kk[BLK_S], vv[BLK_S];
+#pragma unroll
+        for (int j = 0; j < BLK_S; ++j) {
+            kk[j] = 0.f; vv[j] = 0.f;
+            if (j < n) { kk[j] = k_[off + static_cast<size_t>(j) * C]; vv[j] = v_[off + static_cast<size_t>(j) * C]; }
+        }
+        const int cur = summaries(kk, vv, n);
+        carry = combine(aged(carry, static_cast<float>(BLK_T), w), X[cur][NSEG - 1][cl]);
+        __syncthreads();                           // X is written again by the next block
+    }
+    __syncthreads();
+
+    // ---- down: both sweeps of a block, the descending sweep's state handed from block to block
+    State3 gcarry = {0.f, 0.f, O_INIT};
+    float gw = 0.f, gu = 0.f;
+    const int rs = NSEG - 1 - s;                   // position in the descending order
+    for (int blk = nblk - 1; blk >= 0; --blk) {
+        const int t0 = min(blk * BLK_T + s * BLK_S, T), n = live ? min(t0 + BLK_S, T) - t0 : 0;
+        const size_t off = (row + t0) * C + cc;
+        float* __restrict__ gk = gk_ + off;
+        float* __restrict__ gv = gv_ + off;
+        float kk[BLK_S], vv[BLK_S], gg[BLK_S], yy[BLK_S], zz[BLK_S], ze[BLK_S];
+#pragma unroll
+        for (int j = 0; j < BLK_S; ++j) {
+            kk[j] = 0.f; vv[j] = 0.f; gg[j] = 0.f;
+            if (j < n) {
+                kk[j] = k_[off + static_cast<size_t>(j) * C]; vv[j] = v_[off + static_cast<size_t>(j) * C];
+                gg[j] = gy_[off + static_cast<size_t>(j) * C];
+            }
+        }
+        int cur = summaries(kk, vv, n);
+        State5 x = aged(ENTER[blk][cl], static_cast<float>(s * BLK_S), w);
+        if (s > 0) x = combine(x, X[cur][s - 1][cl]);
+        __syncthreads();                           // X is reused below
+
+        // ascending, from the true state
+#pragma unroll
+        for (int j = 0; j < BLK_S; ++j) {
+            yy[j] = 0.f; zz[j] = 0.f; ze[j] = 0.f;
+            if (j < n) {
+                const float kt = kk[j], vt = vv[j], gt = gg[j];
+                ExpPair e = exp_pair(x.o, kt + u);
+                const float num = e.ea * x.p + e.eb * vt;
+                const float iden = 1.0f / (e.ea * x.q + e.eb);
+                const float y = num * iden;
+                yy[j] = y;
+                zz[j] = iden;
+                ze[j] = kt + u - e.no;
+                gw += gt * (x.dp - x.dq * y) * iden * e.ea;
+                gu += gt * (vt - y) * e.eb * iden;
+                e = exp_pair(w + x.o, kt);
+                x.dp = e.ea * (x.p + x.dp);
+                x.dq = e.ea * (x.q + x.dq);
+                x.p = e.ea * x.p + e.eb * vt;
+                x.q = e.ea * x.q + e.eb;
+                x.o = e.no;
+            }
+        }
+        // descending: the segment alone (p, q stand for gp, gq)
+        State3 g = {0.f, 0.f, O_INIT};
+#pragma unroll
+        for (int j = BLK_S - 1; j >= 0; --j) {
+            if (j < n) {
+                const ExpPair e = exp_pair(w + g.o, ze[j] - kk[j] - u);
+                const float Bq = gg[j] * zz[j] * e.eb;
+                g.p = e.ea * g.p + Bq;
+                g.q = e.ea * g.q - Bq * yy[j];
+                g.o = e.no;
+            }
+        }
+        State3 (*G)[NSEG][BLK_CH] = reinterpret_cast<State3 (*)[NSEG][BLK_CH]>(&X[0][0][0]);    // [2][NSEG][BLK_CH], inside X
+        G[0][rs][cl] = g;
+        __syncthreads();
+        cur = 0;
+#pragma unroll
+        for (int d = 1; d < NSEG; d *= 2) {
+            State3 mine = G[cur][rs][cl];
+            if (rs >= d) mine = combine(aged(G[cur][rs - d][cl], static_cast<float>(d * BLK_S), w), mine);
+            G[cur ^ 1][rs][cl] = mine;
+            cur ^= 1;
+            __syncthreads();
+        }
+        g = aged(gcarry, static_cast<float>(rs * BLK_S), w);
+        if (rs > 0) g = combine(g, G[cur][rs - 1][cl]);
+        gcarry = combine(aged(gcarry, static_cast<float>(BLK_T), w), G[cur][NSEG - 1][cl]);
+        __syncthreads();                           // X is written again by the next block
+
+        // descending, from the true state
+#pragma unroll
+        for (int j = BLK_S - 1; j >= 0; --j) {
+            if (j < n) {
+                const float kt = kk[j], vt = vv[j], gt = gg[j];
+                const float y = yy[j], z = zz[j], zexp = ze[j];
+                const float A = gt * z * exp32(zexp);
+                const float Bq = exp32(kt + g.o);
+                gk[static_cast<size_t>(j) * C] = A * (vt - y) + Bq * (g.p * vt + g.q);
+                gv[static_cast<size_t>(j) * C] = A + Bq * g.p;
+                const ExpPair e = exp_pair(w + g.o, zexp - kt - u);
+                const float B2 = gt * z * e.eb;
+                g.p = e.ea * g.p + B2;
+                g.q = e.ea * g.q - B2 * y;
+                g.o = e.no;
+            }
+        }
+    }
+
+    // ---- gw, gu: the segments' sums, added in time order
+    float2* part = reinterpret_cast<float2*>(&X[0][0][0]);                         // [NSEG][BLK_CH]
+    part[s * BLK_CH + cl] = make_float2(gw, gu);
+    __syncthreads();
+    if (s == 0 && live) {
+        float a = 0.f, bsum = 0.f;
+        for (int z = 0; z < NSEG; ++z) { a += part[z * BLK_CH + cl].x; bsum += part[z * BLK_CH + cl].y; }
+        // the caller's buffers are accumulated into, as the reference does (wkv_cuda_v2.cu:112-113)
+        if constexpr (RAW) {                        // per-batch partials in the library's own scratch: plain stores
+            gw_[static_cast<size_t>(b) * C + c] = a * w;
+            gu_[static_cast<size_t>(b) * C + c] = bsum;
+        } else {
+            gw_[static_cast<size_t>(b) * C + c] += a * w;
+            gu_[static_cast<size_t>(b) * C + c] += bsum;
+        }
+    }
+}
+
 // out[c] = sum_b part[b][c], in the fixed order b = 0, 1, ...: the wrapper's torch.sum(gw, dim=0) (wkv/run.py:115-116)
 __global__ __launch_bounds__(256) void wkv4_batch_sum(int B, int C, const float* __restrict__ pw, const float* __restrict__ pu,
                                                       float* __restrict__ gw, float* __restrict__ gu) {
@@ -651,7 +909,8 @@ __global__ __launch_bounds__(256) void wkv4_batch_sum(int B, int C, const float*
 }
 
 // Which form runs: one lane per scan beyond the grid's y range, inputs in registers while a segment has at most 16
-// steps, the form that parks the ascending sweep's results in memory beyond that.
+// steps, blocks of 512 steps with the state handed on up to 32768 steps, and beyond that the form that parks the ascending
+// sweep's results in memory.
 template <bool RAW, int CHR, int SM, typename... Ptrs>
 void launch4_fwd_reg(hipStream_t st, int B, int T, int C, int S, Ptrs... p) {
     hipLaunchKernelGGL((wkv4_fwd_reg<RAW, CHR, SM>), dim3(((C + CHR - 1) / CHR) * B), dim3(CHR * NSEG), 0, st, T, C, S, p...);
@@ -671,6 +930,8 @@ void launch4_fwd(hipStream_t st, int B, int T, int C, const float* w, const floa
         launch4_fwd_reg<RAW, 16, 8>(st, B, T, C, S, w, u, k, v, y);
     } else if (S <= 16) {
         launch4_fwd_reg<RAW, 8, 16>(st, B, T, C, S, w, u, k, v, y);
+    } else if (T <= BLK_T * BLK_MAX) {
+        hipLaunchKernelGGL((wkv4_fwd_blk<RAW>), dim3(((C + BLK_CH - 1) / BLK_CH) * B), dim3(BLK_CH * NSEG), 0, st, T, C, w, u, k, v, y);
     } else {
         hipLaunchKernelGGL((wkv4_fwd_seg<RAW>), dim3((C + CH - 1) / CH, B), dim3(NTS), 0, st, T, C, S, w, u, k, v, y);
     }
@@ -687,6 +948,8 @@ void launch4_bwd(hipStream_t st, int B, int T, int C, const float* w, const floa
         launch4_bwd_reg<RAW, 16, 8>(st, B, T, C, S, w, u, k, v, gy, gw, gu, gk, gv);
     } else if (S <= 16) {
         launch4_bwd_reg<RAW, 8, 16>(st, B, T, C, S, w, u, k, v, gy, gw, gu, gk, gv);
+    } else if (T <= BLK_T * BLK_MAX) {
+        hipLaunchKernelGGL((wkv4_bwd_blk<RAW>), dim3(((C + BLK_CH - 1) / BLK_CH) * B), dim3(BLK_CH * NSEG), 0, st, T, C, w, u, k, v, gy, gw, gu, gk, gv);
     } else {
         hipLaunchKernelGGL((wkv4_bwd_seg<RAW>), dim3((C + CH - 1) / CH, B), dim3(NTS), 0, st, T, C, S, w, u, k, v, gy, gw, gu, gk, gv, ze);
     }

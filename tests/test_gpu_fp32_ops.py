@@ -23,11 +23,12 @@ def _check(name, ref, got):
     assert a <= TOL and b <= TOL, (name, a, b)
 
 
-# T <= 512: inputs in registers, 16 channels a workgroup; 513..1024: 8 channels a workgroup; beyond: the form that parks
-# the ascending sweep's results in memory.  Each boundary from both sides, ragged last segments, channel counts that
-# leave a workgroup partly empty.
+# T <= 512: inputs in registers, 16 channels a workgroup; 513..1024: 8 channels a workgroup; up to 32768: blocks of 512
+# steps with the state handed on; beyond: the form that parks the ascending sweep's results in memory.  Each boundary
+# from both sides, ragged last segments and last blocks, channel counts that leave a workgroup partly empty.
 @pytest.mark.parametrize("B,T,C", [(2, 37, 70), (1, 1, 3), (3, 333, 50), (1, 4100, 20), (4, 512, 768),
-                                   (2, 511, 17), (2, 513, 17), (1, 1000, 9), (2, 1024, 40), (2, 1025, 40), (1, 64, 8), (1, 65, 33)])
+                                   (2, 511, 17), (2, 513, 17), (1, 1000, 9), (2, 1024, 40), (2, 1025, 40), (1, 64, 8), (1, 65, 33),
+                                   (2, 1536, 33), (1, 2048, 16), (1, 2049, 7), (1, 33000, 3)])
 def test_wkv4(lib, B, T, C):
     print(f"\nwkv4 B={B} T={T} C={C}", flush=True)
     w_raw, u, k, v, gy = synth.wkv4_inputs(B, T, C, seed=21)
