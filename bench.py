@@ -150,7 +150,7 @@ def make_wkv6(dev, state):
 
 def make_wkv5(dev, H=32, N=64):
     """N = 64: the matrix-core kernels at B8 T4096 C2048; N = 128: wkv5_bf16/run.py:17-22 as shipped (B8 T4096 C4096),
-    which runs on the one-thread-per-state-row kernels."""
+    which runs on the same kernels with every head taken as four heads of 64 (two launches per kernel, fp32 terms added)."""
     from rwkv_cuda_amd import _lib, synth
     from rwkv_cuda_amd._call import call
     lib = _lib.load()
@@ -164,6 +164,8 @@ def make_wkv5(dev, H=32, N=64):
     decay = torch.empty(2 * C, device=dev, dtype=torch.float32)
     nbytes = lib.rwkv_wkv5raw_backward_workspace_bytes(B, T, C, H)
     ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+    fbytes = lib.rwkv_wkv5_forward_workspace_bytes(B, T, C, H)            # 0 unless N = 128
+    fws = torch.empty(max(fbytes, 16), device=dev, dtype=torch.uint8)
     tok = B * T
     ew = (-torch.exp(w.float())).contiguous()
     eew = torch.exp(ew).contiguous()
@@ -171,7 +173,7 @@ def make_wkv5(dev, H=32, N=64):
     def step():
         # what WKV_5.forward / backward do; the decay transforms (wkv5_bf16/run.py:63-64) and the sums over the batch
         # (:86-87) run inside the library
-        call("rwkv_wkv5raw_forward", dev, B, T, C, H, r, k, v, w, u, y, decay, FLAGS)
+        call("rwkv_wkv5raw_forward_ws", dev, B, T, C, H, r, k, v, w, u, y, decay, fws, fbytes, FLAGS)
         call("rwkv_wkv5raw_backward", dev, B, T, C, H, r, k, v, decay, u, gy, gr, gk, gv, gw_sum, gu_sum, ws, nbytes, FLAGS)
 
     def bwd(mask):
@@ -184,8 +186,9 @@ def make_wkv5(dev, H=32, N=64):
                    ("wkv6_bwd_a_ws<head decay>", bwd(1), 10 * C * tok),           # r k v gy -> gr (+ fp32 workspace)
                    ("wkv6_bwd_b_ws<head decay>", bwd(4), 12 * C * tok)]           # r k v gy -> gk gv
     else:
-        kernels = [("wkv_rows<FWD>", lambda: call("rwkv_wkv5_forward_ex", dev, B, T, C, H, r, k, v, eew, u, y, FLAGS), 8 * C * tok),
-                   ("wkv_rows<GR>", bwd(1), 10 * C * tok), ("wkv_rows<GV>", bwd(2), 8 * C * tok), ("wkv_rows<GK>", bwd(4), 10 * C * tok)]
+        kernels = [("wkv6_fwd_ws<head decay, split> x2 + split_sum", lambda: call("rwkv_wkv5_forward_ws", dev, B, T, C, H, r, k, v, eew, u, y, fws, fbytes, FLAGS), 8 * C * tok),
+                   ("wkv6_bwd_a_ws<head decay, split> x2 + split_sum", bwd(1), 10 * C * tok),
+                   ("wkv6_bwd_b_ws<head decay, split> x2 + split_sum x2", bwd(4), 12 * C * tok)]
 
     def cpu_baseline(t_cpu=256):
         from oracle import wkv56 as O

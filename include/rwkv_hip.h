@@ -128,7 +128,8 @@ int rwkv_timex_backward_sum(void* stream, const float* w, const float* k, const 
  *   r,k,v,y,gy,gr,gk,gv[B,T,C] bf16; eew = exp(-exp(w_raw)) and ew = -exp(w_raw), fp32 [H,N]
  *   (wkv5_bf16/run.py:63-64); u[H,N] bf16; gw,gu[B,C] bf16 per-batch partials (fully written).
  *   Backward workspace (wkv5, wkv6, wkv6_state alike): B*T*C floats (r * dr' between the two sweeps) followed by one
- *   64x64 fp32 forward state per (b,h) and 128 tokens; private to the library, no initialisation needed.
+ *   64x64 fp32 forward state per (b,h) and 128 tokens; private to the library, no initialisation needed.  wkv5 with heads
+ *   of 128 channels asks for more (fp32 terms of gr, gk, gv, gw, gu): take the size from the function below.
  * ------------------------------------------------------------------------------------- */
 int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H,
                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
@@ -136,6 +137,15 @@ int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H,
 int rwkv_wkv5_forward_ex(void* stream, int B, int T, int C, int H,
                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                       const float* eew, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags);
+/* The forward with a workspace.  It has no counterpart in the reference (whose forward takes none): heads of 128 channels
+ * run on the matrix-core kernels as four heads of 64 whose fp32 terms are added afterwards, and those terms need
+ * rwkv_wkv5_forward_workspace_bytes() of scratch (2*B*T*C floats; 0 for every other head size, which then needs no
+ * workspace and runs exactly as rwkv_wkv5_forward_ex).  Without it heads of 128 take the one-row-per-lane kernels. */
+size_t rwkv_wkv5_forward_workspace_bytes(int B, int T, int C, int H);
+int rwkv_wkv5_forward_ws(void* stream, int B, int T, int C, int H,
+                         const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                         const float* eew, const rwkv_bf16* u, rwkv_bf16* y,
+                         void* workspace, size_t workspace_bytes, unsigned flags);
 size_t rwkv_wkv5_backward_workspace_bytes(int B, int T, int C, int H);
 int rwkv_wkv5_backward(void* stream, int B, int T, int C, int H,
                        const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
@@ -155,6 +165,10 @@ int rwkv_wkv5_backward_ex(void* stream, int B, int T, int C, int H,
 int rwkv_wkv5raw_forward(void* stream, int B, int T, int C, int H,
                          const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
                          const rwkv_bf16* w_raw, const rwkv_bf16* u, rwkv_bf16* y, float* decay, unsigned flags);
+int rwkv_wkv5raw_forward_ws(void* stream, int B, int T, int C, int H,
+                            const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                            const rwkv_bf16* w_raw, const rwkv_bf16* u, rwkv_bf16* y, float* decay,
+                            void* workspace, size_t workspace_bytes, unsigned flags);   /* see rwkv_wkv5_forward_ws */
 size_t rwkv_wkv5raw_backward_workspace_bytes(int B, int T, int C, int H);
 int rwkv_wkv5raw_backward(void* stream, int B, int T, int C, int H,
                           const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,

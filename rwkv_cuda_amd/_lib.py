@@ -107,6 +107,9 @@ SIGNATURES = {
     "rwkv_timex_backward_sum": (_I, [_P] * 6 + [_I, _I, _I]),
     "rwkv_wkv5_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
     "rwkv_wkv5_forward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 6 + [_U]),
+    "rwkv_wkv5_forward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "rwkv_wkv5_forward_ws": (_I, [_P, _I, _I, _I, _I] + [_P] * 6 + [_P, _Z, _U]),
+    "rwkv_wkv5raw_forward_ws": (_I, [_P, _I, _I, _I, _I] + [_P] * 7 + [_P, _Z, _U]),
     "rwkv_wkv5_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv5_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_P, _Z]),
     "rwkv_wkv5_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_P, _Z] + [_U]),

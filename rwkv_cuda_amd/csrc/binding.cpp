@@ -99,7 +99,12 @@ void wkv5_forward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor&
     TORCH_CHECK(dt == BF || dt == F32, "wkv5.forward: r must be bfloat16 or float32");
     chk(r, dt, B * T * C, "r"); chk(k, dt, B * T * C, "k"); chk(v, dt, B * T * C, "v"); chk(w, F32, C, "w"); chk(u, dt, C, "u"); chk(y, dt, B * T * C, "y");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(r.device());
-    if (dt == BF) ok(rwkv_wkv5_forward(stream_of(r), B, T, C, H, bp(r), bp(k), bp(v), fp(w), bp(u), bp(y)), "wkv5.forward");
+    if (dt == BF) {
+        // heads of 128 channels need scratch for the fp32 terms of their four heads of 64; every other size needs none
+        const size_t n = rwkv_wkv5_forward_workspace_bytes(B, T, C, H);
+        Tensor ws = scratch(r, n > 0 ? n : 16);
+        ok(rwkv_wkv5_forward_ws(stream_of(r), B, T, C, H, bp(r), bp(k), bp(v), fp(w), bp(u), bp(y), ws.data_ptr(), n, 0u), "wkv5.forward");
+    }
     else ok(rwkv_wkv5f32_forward(stream_of(r), B, T, C, H, fp(r), fp(k), fp(v), fp(w), fp(u), fp(y)), "wkv5.forward");
 }
 void wkv5_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor& k, Tensor& v, Tensor& w, Tensor& ww, Tensor& u,

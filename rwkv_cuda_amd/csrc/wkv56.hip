@@ -899,6 +899,73 @@ __global__ __launch_bounds__(256) void bf16_batch_sum(int B, int C, const uint16
 
 size_t round16(size_t x) { return (x + 15) & ~static_cast<size_t>(15); }
 
+// ---- wkv5 with heads of 128 channels on the matrix-core kernels: every head as four heads of 64, two launches per kernel,
+//      each leaving one fp32 term of every output element (see ArgsB in wkv6_chunk.h); the terms are added here
+constexpr int N_SPLIT = 2 * N;
+bool use_split(int T, int C, int H, unsigned flags) {
+    return C == H * N_SPLIT && !(flags & RWKV_FLAG_SWEEPS) && static_cast<long long>(T) * C < (1LL << 30);
+}
+// out[i] = bf16(p0[i] + p1[i]), four elements per thread (n is a multiple of 64)
+__global__ __launch_bounds__(256) void split_sum(size_t n4, const float4* __restrict__ p0, const float4* __restrict__ p1, uint2* __restrict__ out) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= n4) return;
+    const float4 a = p0[i], b = p1[i];
+    out[i] = make_uint2(static_cast<uint32_t>(f2bf(a.x + b.x)) | (static_cast<uint32_t>(f2bf(a.y + b.y)) << 16),
+                        static_cast<uint32_t>(f2bf(a.z + b.z)) | (static_cast<uint32_t>(f2bf(a.w + b.w)) << 16));
+}
+void launch_split_sum(hipStream_t st, size_t n, const float* p0, const float* p1, uint16_t* out) {
+    const size_t n4 = n / 4;
+    hipLaunchKernelGGL(split_sum, dim3(static_cast<unsigned>((n4 + 255) / 256)), dim3(256), 0, st, n4,
+                       reinterpret_cast<const float4*>(p0), reinterpret_cast<const float4*>(p1), reinterpret_cast<uint2*>(out));
+}
+// forward: two terms of y
+size_t fwd_split_bytes(int B, int T, int C) { return 2 * static_cast<size_t>(B) * T * C * sizeof(float); }
+// backward: r dr' [B,T,C], the stored states of 2 H heads of 64, two terms each of gr, gk, gv [B,T,C] and of gu, gw [B,C]
+size_t bwd_split_floats_before_terms(int B, int T, int C, int H) {
+    const size_t nchunks = (static_cast<size_t>(T) + 31) / 32, npck = (nchunks + 3) / 4;
+    return static_cast<size_t>(B) * T * C + static_cast<size_t>(B) * 2 * H * npck * 64 * 64;
+}
+size_t bwd_split_bytes(int B, int T, int C, int H) {
+    return (bwd_split_floats_before_terms(B, T, C, H) + 6 * static_cast<size_t>(B) * T * C + 4 * static_cast<size_t>(B) * C) * sizeof(float);
+}
+int launch_fwd_split(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
+                     const float* eew, const uint16_t* u, uint16_t* y, float* ws) {
+    const size_t n = static_cast<size_t>(B) * T * C;
+    for (int cross = 0; cross < 2; ++cross)
+        if (int e = launch_wkv5_fwd_split(st, cross, B, T, C, H, r, k, v, eew, u, ws + cross * n)) return e;
+    launch_split_sum(st, n, ws, ws + n, y);
+    return launch_status();
+}
+int launch_bwd_split(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
+                     const float* ew, const uint16_t* u, const uint16_t* gy, uint16_t* gr, uint16_t* gk, uint16_t* gv,
+                     uint16_t* gw, uint16_t* gu, float* ws, unsigned flags) {
+    const unsigned passes = passes_of(flags);
+    const size_t n = static_cast<size_t>(B) * T * C, m = static_cast<size_t>(B) * C;
+    float* rdr = ws;
+    float* gr32 = ws + bwd_split_floats_before_terms(B, T, C, H);
+    float* gk32 = gr32 + 2 * n;
+    float* gv32 = gk32 + 2 * n;
+    float* gu32 = gv32 + 2 * n;
+    float* gw32 = gu32 + 2 * m;
+    // the second sweep of a launch reads the r dr' its own first sweep has left: first, second, first, second
+    for (int cross = 0; cross < 2; ++cross) {
+        if (passes & RWKV_PASS_GR)
+            if (int e = launch_wkv5_bwd_a_split(st, cross, B, T, C, H, r, k, v, ew, u, gy, gr32 + cross * n, gu32 + cross * m, rdr)) return e;
+        if (passes & RWKV_PASS_GK)
+            if (int e = launch_wkv5_bwd_b_split(st, cross, B, T, C, H, r, k, v, ew, u, gy, gk32 + cross * n, gv32 + cross * n, gw32 + cross * m, rdr)) return e;
+    }
+    if (passes & RWKV_PASS_GR) {
+        launch_split_sum(st, n, gr32, gr32 + n, gr);
+        launch_split_sum(st, m, gu32, gu32 + m, gu);
+    }
+    if (passes & RWKV_PASS_GK) {
+        launch_split_sum(st, n, gk32, gk32 + n, gk);
+        launch_split_sum(st, n, gv32, gv32 + n, gv);
+        launch_split_sum(st, m, gw32, gw32 + m, gw);
+    }
+    return launch_status();
+}
+
 }  // namespace
 }  // namespace rwkv
 
@@ -915,15 +982,36 @@ int rwkv_wkv5_forward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf
     return launch_fwd<W_HEAD>(static_cast<hipStream_t>(stream), B, a, flags);
 }
 
-size_t rwkv_wkv5_backward_workspace_bytes(int B, int T, int C, int H) { return ws_bytes(B, T, C, H); }
+size_t rwkv_wkv5_forward_workspace_bytes(int B, int T, int C, int H) {
+    if (check_dims(B, T, C, H) != RWKV_OK) return 0;
+    return use_split(T, C, H, 0u) ? fwd_split_bytes(B, T, C) : 0;
+}
+
+int rwkv_wkv5_forward_ws(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                         const float* eew, const rwkv_bf16* u, rwkv_bf16* y, void* workspace, size_t workspace_bytes, unsigned flags) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (!use_split(T, C, H, flags)) return rwkv_wkv5_forward_ex(stream, B, T, C, H, r, k, v, eew, u, y, flags);
+    if (int e = check_ptrs({r, k, v, eew, u, y})) return e;
+    if (workspace == nullptr || workspace_bytes < fwd_split_bytes(B, T, C) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
+    return launch_fwd_split(static_cast<hipStream_t>(stream), B, T, C, H, r, k, v, eew, u, y, static_cast<float*>(workspace));
+}
+
+size_t rwkv_wkv5_backward_workspace_bytes(int B, int T, int C, int H) {
+    if (check_dims(B, T, C, H) != RWKV_OK) return 0;
+    return use_split(T, C, H, 0u) ? bwd_split_bytes(B, T, C, H) : ws_bytes(B, T, C, H);
+}
 
 int rwkv_wkv5_backward_ex(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                        const rwkv_bf16* v, const float* eew, const float* ew, const rwkv_bf16* u,
                        const rwkv_bf16* gy, rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw,
                        rwkv_bf16* gu, void* workspace, size_t workspace_bytes, unsigned flags) {
     if (int e = check_dims(B, T, C, H)) return e;
-    if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu}, C == H * N)) return e;
-    if (workspace == nullptr || workspace_bytes < ws_bytes(B, T, C, H) || !aligned16(workspace)) return RWKV_ERR_WORKSPACE;
+    if (int e = check_ptrs({r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu}, C == H * N || C == H * N_SPLIT)) return e;
+    if (workspace == nullptr || workspace_bytes < rwkv_wkv5_backward_workspace_bytes(B, T, C, H) || !aligned16(workspace))
+        return RWKV_ERR_WORKSPACE;
+    if (use_split(T, C, H, flags))
+        return launch_bwd_split(static_cast<hipStream_t>(stream), B, T, C, H, r, k, v, ew, u, gy, gr, gk, gv, gw, gu,
+                                static_cast<float*>(workspace), flags);
     Args a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = eew; a.ew_head = ew; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.rdr = static_cast<float*>(workspace);
@@ -1093,8 +1181,17 @@ int rwkv_wkv5raw_forward(void* stream, int B, int T, int C, int H, const rwkv_bf
     return rwkv_wkv5_forward_ex(stream, B, T, C, H, r, k, v, decay, u, y, flags);
 }
 
+int rwkv_wkv5raw_forward_ws(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                            const rwkv_bf16* w_raw, const rwkv_bf16* u, rwkv_bf16* y, float* decay, void* workspace,
+                            size_t workspace_bytes, unsigned flags) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, w_raw, u, y, decay}, C == H * N || C == H * N_SPLIT)) return e;
+    hipLaunchKernelGGL(wkv5_decay_transform, dim3((C + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream), C, w_raw, decay);
+    return rwkv_wkv5_forward_ws(stream, B, T, C, H, r, k, v, decay, u, y, workspace, workspace_bytes, flags);
+}
+
 size_t rwkv_wkv5raw_backward_workspace_bytes(int B, int T, int C, int H) {
-    const size_t n = ws_bytes(B, T, C, H);
+    const size_t n = rwkv_wkv5_backward_workspace_bytes(B, T, C, H);
     return n == 0 ? 0 : round16(n) + round16(2 * static_cast<size_t>(B) * C * sizeof(uint16_t));
 }
 
@@ -1105,7 +1202,7 @@ int rwkv_wkv5raw_backward(void* stream, int B, int T, int C, int H, const rwkv_b
     if (int e = check_ptrs({decay, gw, gu}, C == H * N)) return e;
     if (workspace == nullptr || workspace_bytes < rwkv_wkv5raw_backward_workspace_bytes(B, T, C, H) || !aligned16(workspace))
         return RWKV_ERR_WORKSPACE;
-    const size_t n = round16(ws_bytes(B, T, C, H));
+    const size_t n = round16(rwkv_wkv5_backward_workspace_bytes(B, T, C, H));
     uint16_t* pw = reinterpret_cast<uint16_t*>(static_cast<char*>(workspace) + n);      // per-batch gw, then per-batch gu
     uint16_t* pu = pw + static_cast<size_t>(B) * C;
     if (int e = rwkv_wkv5_backward_ex(stream, B, T, C, H, r, k, v, decay, decay + C, u, gy, gr, gk, gv, pw, pu, workspace, n, flags)) return e;

@@ -47,14 +47,15 @@ struct alignas(16) SmemA2 {
 };
 
 // ---------------------------------------------------------------------------------------------------- prep waves
-template <int WMODE>
-DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base, const int nchunks) {
+// base, h: where r, k, w, u (and gu) of this workgroup sit; vbase: where v, gy sit (the same place unless the head is split)
+template <int WMODE, bool SPLIT>
+DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base, const size_t vbase, const int h, const int nchunks) {
     const int lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
     const uint16_t* __restrict__ rb = a.r + base;
     const uint16_t* __restrict__ kb = a.k + base;
-    const uint16_t* __restrict__ vb = a.v + base;
-    const uint16_t* __restrict__ gb = a.gy + base;
+    const uint16_t* __restrict__ vb = a.v + vbase;
+    const uint16_t* __restrict__ gb = a.gy + vbase;
     // channel pair (2 jp, 2 jp + 1), tokens 4 wid + 2 th + {0, 1}
     const int jp = lane & 31, th = lane >> 5, pt0 = 4 * wid + 2 * th;
     const bool second = wid >= 4;
@@ -100,7 +101,7 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
     // wkv5: one decay per channel for the whole sequence, given as ew = -exp(w_raw) = log of the decay
     float lamc[2] = {0.f, 0.f};
     if constexpr (WMODE == W_HEAD) {
-        const float2 e2 = *reinterpret_cast<const float2*>(static_cast<const float*>(a.w) + (blockIdx.x % a.H) * N + 2 * jp);
+        const float2 e2 = *reinterpret_cast<const float2*>(static_cast<const float*>(a.w) + h * N + 2 * jp);
         lamc[0] = LOG2E * e2.x; lamc[1] = LOG2E * e2.y;
     }
     static_for<STA>([&](auto Z) { prefetch(decltype(Z)::value, ring[decltype(Z)::value]); });
@@ -261,12 +262,14 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
     if (tid < N) {
         float s = S.gfast[0][tid] + S.gfast[1][tid];
         for (int t = 0; t < L; ++t) s += S.Yx[0][t][tid];
-        a.gu[static_cast<size_t>(blockIdx.x / a.H) * C + (blockIdx.x % a.H) * N + tid] = f2bf(s);
+        const size_t at = static_cast<size_t>(blockIdx.x / a.H) * C + h * N + tid;
+        if constexpr (SPLIT) a.gu32[at] = s;
+        else a.gu[at] = f2bf(s);
     }
 }
 
 // ---------------------------------------------------------------------------------------------------- state waves
-template <int WMODE>
+template <int WMODE, bool SPLIT>
 DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t base, const size_t bh, const int nchunks) {
     const int lane = tid & 63, sw = __builtin_amdgcn_readfirstlane(tid >> 6) - NPREP, q = sw & 3, ih = sw >> 2, l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
@@ -299,7 +302,7 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
         const float4 x = *reinterpret_cast<const float4*>(&S.outR[pb][row][4 * l16]);
         if (tg < T) {
             const uint32_t o = static_cast<uint32_t>(tg) * C + 4 * l16;
-            store8(a.gr + base, o * 2, y);
+            if constexpr (!SPLIT) store8(a.gr + base, o * 2, y);      // split heads: gr has left in fp32 already
             store16(a.rdr + base, o * 4, f32x4{x.x, x.y, x.z, x.w});
         }
     };
@@ -409,7 +412,11 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
                 rd[v] = rr[v] * drp;
                 gu_acc[v] = fmaf(rr[v], kv, gu_acc[v]);
             }
-            *reinterpret_cast<uint2*>(&S.outG[i & 1][t][j4 >> 1]) = make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3]));
+            if constexpr (SPLIT) {
+                if (c0 + t < T) store16(a.gr32 + base, (static_cast<uint32_t>(c0 + t) * C + j4) * 4, f32x4{gr[0], gr[1], gr[2], gr[3]});
+            } else {
+                *reinterpret_cast<uint2*>(&S.outG[i & 1][t][j4 >> 1]) = make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3]));
+            }
             *reinterpret_cast<float4*>(&S.outR[i & 1][t][j4]) = make_float4(rd[0], rd[1], rd[2], rd[3]);
             staged_now = true;
         } else {
@@ -432,7 +439,8 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
             }
             if (c0 + xt < T) {
                 const uint32_t o = static_cast<uint32_t>(c0 + xt) * C + xj;
-                store8(a.gr + base, o * 2, make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3])));
+                if constexpr (SPLIT) store16(a.gr32 + base, o * 4, f32x4{gr[0], gr[1], gr[2], gr[3]});
+                else store8(a.gr + base, o * 2, make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3])));
                 store16(a.rdr + base, o * 4, f32x4{rd[0], rd[1], rd[2], rd[3]});
             }
         }
@@ -451,27 +459,29 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
     __syncthreads();
 }
 
-template <int WMODE>
+template <int WMODE, bool SPLIT = false>
 __global__ __launch_bounds__(NTA) void wkv6_bwd_a_ws(const ArgsB a) {
     __shared__ SmemA2 S;
     const int tid = threadIdx.x;
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
-    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
+    const int hk = SPLIT ? h ^ a.cross : h;            // the block of 64 channels that r, k, w, u come from and gr, gu go to
+    const size_t vbase = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
+    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(hk) * N;
     const size_t bh = static_cast<size_t>(b) * a.H + h;
     const int nchunks = (a.T + L - 1) / L;
     // positions of the tile that are never written (t < 16 <= s) must read as zero
     for (int i = tid; i < 2 * L * AS; i += NTA) (&S.BmH[0][0])[i] = 0;
-    if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
+    if (tid < N) S.u[tid] = bf2f(a.u[hk * N + tid]);
     if (tid < 128) {
         // One-hot B operand of the transposing products, per lane (column r = l16, K-slot group g), for tile parity p:
         // column r <-> channel 8 (r>>2) + 4 p + (r&3) of a 32-channel half.
         const int p = tid >> 6, ln = tid & 63, c16 = ln & 15, gg = ln >> 4;
         S.sel[p][ln] = one_hot(gg == (c16 >> 2), 4 * p + (c16 & 3));
     }
-    if (__builtin_amdgcn_readfirstlane(tid >> 6) < NPREP) bwa_prep<WMODE>(S, a, tid, base, nchunks);
+    if (__builtin_amdgcn_readfirstlane(tid >> 6) < NPREP) bwa_prep<WMODE, SPLIT>(S, a, tid, base, vbase, hk, nchunks);
     // The state waves carry the chunk-to-chunk dependence; the prep waves work ahead and have slack.  Issue priority goes
     // to the state waves (the hardware otherwise favours the oldest waves of a SIMD, which are the prep waves).
-    else { __builtin_amdgcn_s_setprio(2); bwa_state<WMODE>(S, a, tid, base, bh, nchunks); }
+    else { __builtin_amdgcn_s_setprio(2); bwa_state<WMODE, SPLIT>(S, a, tid, base, bh, nchunks); }
 }
 
 }  // namespace
@@ -485,6 +495,17 @@ int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_bwd_a_ws<W_RAW>, dim3(B * H), dim3(NTA), 0, st, a);
     else if (wmode == W_EW) hipLaunchKernelGGL(wkv6_bwd_a_ws<W_EW>, dim3(B * H), dim3(NTA), 0, st, a);
     else hipLaunchKernelGGL(wkv6_bwd_a_ws<W_HEAD>, dim3(B * H), dim3(NTA), 0, st, a);
+    return launch_status();
+}
+
+// wkv5 with heads of 128 channels: the first sweep of one of the two launches described at ArgsB (H counts the heads of 128)
+int launch_wkv5_bwd_a_split(hipStream_t st, int cross, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k,
+                            const uint16_t* v, const float* ew, const uint16_t* u, const uint16_t* gy, float* gr32, float* gu32,
+                            float* rdr) {
+    ArgsB a{};
+    a.T = T; a.C = C; a.H = 2 * H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.s0 = nullptr; a.gy = gy;
+    a.rdr = rdr; a.cross = cross; a.gr32 = gr32; a.gu32 = gu32;
+    hipLaunchKernelGGL((wkv6_bwd_a_ws<W_HEAD, true>), dim3(B * 2 * H), dim3(NTA), 0, st, a);
     return launch_status();
 }
 

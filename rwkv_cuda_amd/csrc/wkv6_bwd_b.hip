@@ -54,14 +54,15 @@ struct alignas(16) SmemB2 {
 };
 
 // ---------------------------------------------------------------------------------------------------- prep waves
+// base, h: where r, k, w, u and r dr' of this workgroup sit; vbase: where v, gy sit (the same place unless the head is split)
 template <int WMODE>
-DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base, const int h, const int nchunks) {
+DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base, const size_t vbase, const int h, const int nchunks) {
     const int lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
     const uint16_t* __restrict__ rb = a.r + base;
     const uint16_t* __restrict__ kb = a.k + base;
-    const uint16_t* __restrict__ vb = a.v + base;
-    const uint16_t* __restrict__ gb = a.gy + base;
+    const uint16_t* __restrict__ vb = a.v + vbase;
+    const uint16_t* __restrict__ gb = a.gy + vbase;
     // channel pair (2 jp, 2 jp + 1), tokens 4 wid + 2 th + {0, 1}
     const int jp = lane & 31, th = lane >> 5, pt0 = 4 * wid + 2 * th;
     const bool second = wid >= 4;
@@ -320,8 +321,9 @@ DEVINL void bwd_prep(SmemB2& S, const ArgsB& a, const int tid, const size_t base
 }
 
 // ---------------------------------------------------------------------------------------------------- D waves: gk, gw, gs
-template <int WMODE>
-DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t base, const size_t bh, const int nchunks) {
+// bh: this workgroup (stored states, s0, gs); bhk: the (batch, head) its key channels belong to (w, gw)
+template <int WMODE, bool SPLIT>
+DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t base, const size_t bh, const size_t bhk, const int nchunks) {
     const int lane = tid & 63, q = (__builtin_amdgcn_readfirstlane(tid >> 6) - NPREP) & 3, l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
     const bool stateful = a.s0 != nullptr;
@@ -438,7 +440,8 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 const float Gt = P - kj * dkp;
                 P = Gt + rdrj;
                 if (g == 0 && tg < T) {
-                    a.gk[base + static_cast<size_t>(tg) * C + j_own] = f2bf(fmaf(uj * rj, vg, dkp));
+                    if constexpr (SPLIT) a.gk32[base + static_cast<size_t>(tg) * C + j_own] = fmaf(uj * rj, vg, dkp);
+                    else a.gk[base + static_cast<size_t>(tg) * C + j_own] = f2bf(fmaf(uj * rj, vg, dkp));
                     if constexpr (WMODE != W_HEAD) a.gw[base + static_cast<size_t>(tg) * C + j_own] = f2bf((!stateful && tg == 0) ? 0.f : lmj * Gt);
                 }
                 if constexpr (WMODE == W_HEAD) gw_lane += (tg == 0 || tg >= T) ? 0.f : Gt;
@@ -457,6 +460,7 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 u4[0] = z.x; u4[1] = z.y; u4[2] = z.z; u4[3] = z.w;
             }
             float tot1[4] = {0.f, 0.f, 0.f, 0.f};
+            [[maybe_unused]] f32x4 out_k32[2];
             uint2 out_k[2], out_w[2];                   // stored after both tiles: a store in between would make every later
                                                         // register reload from scratch wait for its acknowledgement
 #pragma unroll
@@ -490,7 +494,8 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                     if constexpr (WMODE == W_HEAD) gw_acc[v] += (tg == 0 || tg >= T) ? 0.f : Gt;
                     if (st == 1) tot1[v] = tot; else Pend[v] += tot + tot1[v];
                 }
-                out_k[st] = make_uint2(pack_bf2(gk[0], gk[1]), pack_bf2(gk[2], gk[3]));
+                if constexpr (SPLIT) out_k32[st] = f32x4{gk[0], gk[1], gk[2], gk[3]};
+                else out_k[st] = make_uint2(pack_bf2(gk[0], gk[1]), pack_bf2(gk[2], gk[3]));
                 out_w[st] = make_uint2(pack_bf2(gw[0], gw[1]), pack_bf2(gw[2], gw[3]));
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -499,7 +504,8 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 const int tg = c0 + 16 * st + l16;
                 if (tg < T) {
                     const uint32_t off = (static_cast<uint32_t>(tg) * C + j4) * 2;
-                    store8(a.gk + base, off, out_k[st]);
+                    if constexpr (SPLIT) store16(a.gk32 + base, 2 * off, out_k32[st]);
+                    else store8(a.gk + base, off, out_k[st]);
                     if constexpr (WMODE != W_HEAD) store8(a.gw + base, off, out_w[st]);
                 }
             }
@@ -520,12 +526,15 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
     if constexpr (WMODE == W_HEAD) {                   // gw[b][h][j] = ew_j sum_t G_t[j]
         if (g == 0) S.pc[j_own] = gw_lane;
         const float4 px = *reinterpret_cast<const float4*>(&S.pc[j4]);
-        const float4 e4 = *reinterpret_cast<const float4*>(static_cast<const float*>(a.w) + (bh % a.H) * N + j4);
+        const float4 e4 = *reinterpret_cast<const float4*>(static_cast<const float*>(a.w) + (bhk % a.H) * N + j4);
         const float pxv[4] = {px.x, px.y, px.z, px.w}, ev[4] = {e4.x, e4.y, e4.z, e4.w};
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const float s = row_sum_to_last(gw_acc[v]) + pxv[v];
-            if (l16 == 15) a.gw[bh * N + j4 + v] = f2bf(gw_factor(ev[v]) * s);
+            if (l16 == 15) {
+                if constexpr (SPLIT) a.gw32[bhk * N + j4 + v] = gw_factor(ev[v]) * s;
+                else a.gw[bhk * N + j4 + v] = f2bf(gw_factor(ev[v]) * s);
+            }
         }
     }
     if (a.gs != nullptr) {
@@ -538,7 +547,7 @@ DEVINL void bwd_state_d(SmemB2& S, const ArgsB& a, const int tid, const size_t b
 }
 
 // ---------------------------------------------------------------------------------------------------- E waves: gv
-template <int WMODE>
+template <int WMODE, bool SPLIT>
 DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t base, const int nchunks) {
     const int lane = tid & 63, q = (__builtin_amdgcn_readfirstlane(tid >> 6) - NPREP) & 3, l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
@@ -615,7 +624,10 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 }
                 gvp = allreduce_rows(gvp);
                 const int tg = c0 + t;
-                if (g == 0 && tg < T) a.gv[base + static_cast<size_t>(tg) * C + i_own] = f2bf(gvp);
+                if (g == 0 && tg < T) {
+                    if constexpr (SPLIT) a.gv32[base + static_cast<size_t>(tg) * C + i_own] = gvp;
+                    else a.gv[base + static_cast<size_t>(tg) * C + i_own] = f2bf(gvp);
+                }
             }
         }
         __syncthreads();
@@ -625,7 +637,10 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
                 const int s = 16 * st + l16, tg = c0 + s;
                 f32x4 y = mfma(gto, lds_op(&S.AmH[s][4 * g]), dvin[st]);
                 y = mfma(gto, lds_op(&S.AmL[s][4 * g]), y);
-                if (tg < T) store8(a.gv + base, (static_cast<uint32_t>(tg) * C + i4) * 2, make_uint2(pack_bf2(y[0], y[1]), pack_bf2(y[2], y[3])));
+                if (tg < T) {
+                    if constexpr (SPLIT) store16(a.gv32 + base, (static_cast<uint32_t>(tg) * C + i4) * 4, y);
+                    else store8(a.gv + base, (static_cast<uint32_t>(tg) * C + i4) * 2, make_uint2(pack_bf2(y[0], y[1]), pack_bf2(y[2], y[3])));
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
             // ------------------------------------------------------------ dS^T = diag(dec) dS^T + diag(d1) R'^T GY
@@ -643,17 +658,19 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
     }
 }
 
-template <int WMODE>
+template <int WMODE, bool SPLIT = false>
 __global__ __launch_bounds__(NTB) void wkv6_bwd_b_ws(const ArgsB a) {
     __shared__ SmemB2 S;
     const int tid = threadIdx.x;
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
-    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
-    const size_t bh = static_cast<size_t>(b) * a.H + h;
+    const int hk = SPLIT ? h ^ a.cross : h;            // the block of 64 channels that r, k, w, u come from and gk, gw go to
+    const size_t vbase = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
+    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(hk) * N;
+    const size_t bh = static_cast<size_t>(b) * a.H + h, bhk = static_cast<size_t>(b) * a.H + hk;
     const int nchunks = (a.T + L - 1) / L;
     // positions of the tiles that are never written (s >= 16 > tau) must read as zero
     for (int i = tid; i < 4 * L * AS; i += NTB) (&S.AmH[0][0])[i] = 0;
-    if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
+    if (tid < N) S.u[tid] = bf2f(a.u[hk * N + tid]);
     if (tid < 128) {
         // One-hot B operand of the transposing products, per lane (column r = l16, K-slot group g), for tile parity p:
         // column r <-> channel 8 (r>>2) + 4 p + (r&3) of a 32-channel half.
@@ -661,9 +678,9 @@ __global__ __launch_bounds__(NTB) void wkv6_bwd_b_ws(const ArgsB a) {
         S.sel[p][ln] = one_hot(gg == (c16 >> 2), 4 * p + (c16 & 3));
     }
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6);
-    if (wid < NPREP) bwd_prep<WMODE>(S, a, tid, base, h, nchunks);
-    else if (wid < NPREP + 4) bwd_state_d<WMODE>(S, a, tid, base, bh, nchunks);
-    else bwd_state_e<WMODE>(S, a, tid, base, nchunks);
+    if (wid < NPREP) bwd_prep<WMODE>(S, a, tid, base, vbase, hk, nchunks);
+    else if (wid < NPREP + 4) bwd_state_d<WMODE, SPLIT>(S, a, tid, base, bh, bhk, nchunks);
+    else bwd_state_e<WMODE, SPLIT>(S, a, tid, vbase, nchunks);
 }
 
 }  // namespace
@@ -678,6 +695,17 @@ int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_bwd_b_ws<W_RAW>, dim3(B * H), dim3(NTB), 0, st, a);
     else if (wmode == W_EW) hipLaunchKernelGGL(wkv6_bwd_b_ws<W_EW>, dim3(B * H), dim3(NTB), 0, st, a);
     else hipLaunchKernelGGL(wkv6_bwd_b_ws<W_HEAD>, dim3(B * H), dim3(NTB), 0, st, a);
+    return launch_status();
+}
+
+// wkv5 with heads of 128 channels: the second sweep of one of the two launches described at ArgsB (H counts the heads of 128)
+int launch_wkv5_bwd_b_split(hipStream_t st, int cross, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k,
+                            const uint16_t* v, const float* ew, const uint16_t* u, const uint16_t* gy, float* gk32, float* gv32,
+                            float* gw32, const float* rdr) {
+    ArgsB a{};
+    a.T = T; a.C = C; a.H = 2 * H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.s0 = nullptr; a.gy = gy;
+    a.gs = nullptr; a.rdr = const_cast<float*>(rdr); a.cross = cross; a.gk32 = gk32; a.gv32 = gv32; a.gw32 = gw32;
+    hipLaunchKernelGGL((wkv6_bwd_b_ws<W_HEAD, true>), dim3(B * 2 * H), dim3(NTB), 0, st, a);
     return launch_status();
 }
 

@@ -58,6 +58,9 @@ struct ArgsC {
     const uint16_t *r, *k, *v, *u, *s0;
     const void* w;
     uint16_t* y;
+    // SPLIT kernels only (see below)
+    int cross;
+    float* y32;
 };
 
 struct ArgsB {
@@ -66,7 +69,19 @@ struct ArgsB {
     const void* w;
     uint16_t *gr, *gk, *gv, *gw, *gu, *gs;
     float* rdr;                   // workspace [B,T,C] fp32
+    // SPLIT kernels only (see below)
+    int cross;
+    float *gr32, *gk32, *gv32, *gw32, *gu32;
 };
+
+// A head of 128 channels as four heads of 64 (SPLIT = true, wkv5 only).  With the key channels j and the value channels
+// i of the head cut into halves J and I, everything the op computes is a sum over blocks of the state S[i in I][j in J]:
+//     y_I = sum_J wkv(r_J, k_J, v_I; w_J, u_J)     gv_I = sum_J ...     gr_J, gk_J, gw_J, gu_J = sum_I ...
+// and each term is exactly the 64-channel problem.  A launch treats the tensor as 2 H heads of 64: workgroup h takes its
+// v, gy (and y, gv) from block h and its r, k, w, u (and gr, gk, gw, gu) from block h ^ cross.  cross = 0 gives the
+// diagonal blocks (I = J), cross = 1 the other two, so every output element gets exactly one term from each launch; the
+// terms are written in fp32 (y32, gr32, ...: [B,T,C] like the tensors, gw32 / gu32 [B,C]) and added afterwards, which
+// keeps the single bf16 rounding of the outputs.
 
 // Operand format.  An fp32 value x is used as hi = bf16(x), lo = bf16(x - hi).  Along the K axis of an MFMA a lane holds
 // 8 slots = 4 consecutive elements e0..e3 as  P = [h0 h1 h2 h3 | l0 l1 l2 l3]  (dwords H01, H23, L01, L23).  With the

@@ -47,13 +47,14 @@ struct alignas(16) SmemF {
 };
 
 // ---------------------------------------------------------------------------------------------------- prep waves
+// base, h: where r, k, w, u of this workgroup sit; vbase: where v sits (the same place unless the head is split)
 template <int WMODE>
-DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base, const int h, const int nchunks) {
+DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base, const size_t vbase, const int h, const int nchunks) {
     const int lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
     const uint16_t* __restrict__ rb = a.r + base;
     const uint16_t* __restrict__ kb = a.k + base;
-    const uint16_t* __restrict__ vb = a.v + base;
+    const uint16_t* __restrict__ vb = a.v + vbase;
     // channel pair (2 jp, 2 jp + 1), tokens 4 wid + 2 th + {0, 1}
     const int jp = lane & 31, th = lane >> 5, pt0 = 4 * wid + 2 * th;
     const bool second = wid >= 4;
@@ -313,7 +314,7 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
 }
 
 // ---------------------------------------------------------------------------------------------------- state waves
-template <int WMODE>
+template <int WMODE, bool SPLIT>
 DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base, const size_t bh, const int nchunks) {
     const int lane = tid & 63, sw = __builtin_amdgcn_readfirstlane(tid >> 6) - NPREP, q = sw & 3, jh = sw >> 2, l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
@@ -345,16 +346,25 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
             Y = mfma(Vop, lds_op(&S.AmH[c & 1][16 * jh + l16][4 * g]), Y);
             Y = mfma(Vop, lds_op(&S.AmL[c & 1][16 * jh + l16][4 * g]), Y);
             const int t = c * L + 16 * jh + l16;
-            if (t < T)
-                *reinterpret_cast<uint2*>(a.y + base + static_cast<size_t>(t) * C + 16 * q + 4 * g) =
-                    make_uint2(pack_bf2(Y[0], Y[1]), pack_bf2(Y[2], Y[3]));
+            if (t < T) {
+                if constexpr (SPLIT)
+                    *reinterpret_cast<float4*>(a.y32 + base + static_cast<size_t>(t) * C + 16 * q + 4 * g) = make_float4(Y[0], Y[1], Y[2], Y[3]);
+                else
+                    *reinterpret_cast<uint2*>(a.y + base + static_cast<size_t>(t) * C + 16 * q + 4 * g) =
+                        make_uint2(pack_bf2(Y[0], Y[1]), pack_bf2(Y[2], Y[3]));
+            }
         } else {                                       // exact path: add the two halves and store
             const int idx = tid - NPREP * 64, t = idx >> 4, i4 = (idx & 15) * 4;
             const float4 p0 = *reinterpret_cast<const float4*>(&S.Yx[c & 1][0][t][i4]);
             const float4 p1 = *reinterpret_cast<const float4*>(&S.Yx[c & 1][1][t][i4]);
-            if (c * L + t < T)
-                *reinterpret_cast<uint2*>(a.y + base + static_cast<size_t>(c * L + t) * C + i4) =
-                    make_uint2(pack_bf2(p0.x + p1.x, p0.y + p1.y), pack_bf2(p0.z + p1.z, p0.w + p1.w));
+            if (c * L + t < T) {
+                if constexpr (SPLIT)
+                    *reinterpret_cast<float4*>(a.y32 + base + static_cast<size_t>(c * L + t) * C + i4) =
+                        make_float4(p0.x + p1.x, p0.y + p1.y, p0.z + p1.z, p0.w + p1.w);
+                else
+                    *reinterpret_cast<uint2*>(a.y + base + static_cast<size_t>(c * L + t) * C + i4) =
+                        make_uint2(pack_bf2(p0.x + p1.x, p0.y + p1.y), pack_bf2(p0.z + p1.z, p0.w + p1.w));
+            }
         }
     };
 
@@ -443,7 +453,7 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
     finish(nchunks - 1, exact_prev);
 }
 
-template <int WMODE>
+template <int WMODE, bool SPLIT = false>
 __global__ __launch_bounds__(NTF) void wkv6_fwd_ws(const ArgsC a) {
     __shared__ SmemF S;
     const int tid = threadIdx.x;
@@ -453,9 +463,17 @@ __global__ __launch_bounds__(NTF) void wkv6_fwd_ws(const ArgsC a) {
     const int nchunks = (a.T + L - 1) / L;
     // positions of A that no tile ever writes (t < 16 <= s) must read as zero
     for (int i = tid; i < 2 * L * OS; i += NTF) { (&S.AmH[0][0][0])[i] = 0; (&S.AmL[0][0][0])[i] = 0; }
-    if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
-    if (__builtin_amdgcn_readfirstlane(tid >> 6) < NPREP) fwd_prep<WMODE>(S, a, tid, base, h, nchunks);
-    else fwd_state<WMODE>(S, a, tid, base, bh, nchunks);
+    if constexpr (SPLIT) {
+        const int hk = h ^ a.cross;                    // the block of 64 channels that r, k, w, u come from
+        const size_t kbase = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(hk) * N;
+        if (tid < N) S.u[tid] = bf2f(a.u[hk * N + tid]);
+        if (__builtin_amdgcn_readfirstlane(tid >> 6) < NPREP) fwd_prep<WMODE>(S, a, tid, kbase, base, hk, nchunks);
+        else fwd_state<WMODE, true>(S, a, tid, base, bh, nchunks);
+    } else {
+        if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
+        if (__builtin_amdgcn_readfirstlane(tid >> 6) < NPREP) fwd_prep<WMODE>(S, a, tid, base, base, h, nchunks);
+        else fwd_state<WMODE, false>(S, a, tid, base, bh, nchunks);
+    }
 }
 
 }  // namespace
@@ -468,6 +486,16 @@ int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H,
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_fwd_ws<W_RAW>, dim3(B * H), dim3(NTF), 0, st, a);
     else if (wmode == W_EW) hipLaunchKernelGGL(wkv6_fwd_ws<W_EW>, dim3(B * H), dim3(NTF), 0, st, a);
     else hipLaunchKernelGGL(wkv6_fwd_ws<W_HEAD>, dim3(B * H), dim3(NTF), 0, st, a);
+    return launch_status();
+}
+
+// wkv5 with heads of 128 channels: one of the two launches described at ArgsB (H counts the heads of 128)
+int launch_wkv5_fwd_split(hipStream_t st, int cross, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k,
+                          const uint16_t* v, const float* eew, const uint16_t* u, float* y32) {
+    ArgsC a{};
+    a.T = T; a.C = C; a.H = 2 * H; a.r = r; a.k = k; a.v = v; a.w = eew; a.u = u; a.s0 = nullptr; a.y = nullptr;
+    a.cross = cross; a.y32 = y32;
+    hipLaunchKernelGGL((wkv6_fwd_ws<W_HEAD, true>), dim3(B * 2 * H), dim3(NTF), 0, st, a);
     return launch_status();
 }
 

@@ -24,7 +24,10 @@ class WKV_5(torch.autograd.Function):
             # ew = -exp(w.float()), eew = exp(ew) (:63-64) are made by the library into `decay` = [eew | ew]
             decay = torch.empty(2 * C, device=dev, dtype=torch.float32)
             y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
-            call("rwkv_wkv5raw_forward", dev, B, T, C, H, r, k, v, w, u, y, decay, ctx.flags)
+            # heads of 128 channels run as four heads of 64 whose fp32 terms need scratch; every other size needs none
+            nbytes = _lib.load().rwkv_wkv5_forward_workspace_bytes(B, T, C, H)
+            ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
+            call("rwkv_wkv5raw_forward_ws", dev, B, T, C, H, r, k, v, w, u, y, decay, ws, nbytes, ctx.flags)
             ctx.save_for_backward(r, k, v, decay, u)
             return y
 

@@ -163,6 +163,34 @@ def test_remaining_extensions_match_ctypes(lib, ext):
         assert torch.equal(a, b), name
 
 
+def test_wkv5_head_size_128_through_the_shim(lib, ext):
+    """wkv5_bf16/run.py:21 ships head size 128: the shim allocates the forward's scratch itself (the reference's forward
+    takes none) and must give what the C ABI gives with a caller's workspace."""
+    B, T, H = 2, 70, 2
+    C = H * 128
+    r, k, v, w5, u, gy = (x.to(DEV) for x in synth.wkv5_inputs(B, T, C, H, seed=67))
+    ew = (-torch.exp(w5.float())).contiguous().view(-1)
+    eew = torch.exp(ew).contiguous()
+    res = []
+    for via in (False, True):
+        y, gr, gk, gv = (garbage((B, T, C), BF) for _ in range(4))
+        gw, gu = garbage((B, C), BF), garbage((B, C), BF)
+        if via:
+            ext.wkv5.forward(B, T, C, H, r, k, v, eew, u.view(-1), y)
+            torch.ops.wkv5.backward(B, T, C, H, r, k, v, eew, ew, u.view(-1), gy, gr, gk, gv, gw, gu)
+        else:
+            nf = lib.rwkv_wkv5_forward_workspace_bytes(B, T, C, H)
+            n = lib.rwkv_wkv5_backward_workspace_bytes(B, T, C, H)
+            assert nf > 0 and n > nf
+            fws, ws = torch.empty(nf, device=DEV, dtype=torch.uint8), torch.empty(n, device=DEV, dtype=torch.uint8)
+            call("rwkv_wkv5_forward_ws", r.device, B, T, C, H, r, k, v, eew, u, y, fws, nf, 0)
+            call("rwkv_wkv5_backward", r.device, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, n)
+        torch.cuda.synchronize()
+        res.append((y, gr, gk, gv, gw, gu))
+    for name, a, b in zip("y gr gk gv gw gu".split(), *res):
+        assert torch.equal(a, b), name
+
+
 def test_shim_rejects_wrong_dtype_and_cpu_tensors(ext):
     x = torch.zeros(2, 16, 64, device=DEV, dtype=torch.float32)          # bf16 expected
     u = torch.zeros(64, device=DEV, dtype=BF)

@@ -2,8 +2,9 @@
 
 The reference compiles its kernels with -D_N_=HEAD_SIZE: wkv5_bf16/run.py:21 ships 128, the self-checks of
 wkv5/run.py:366, wkv6/run.py:35 and wkv6_state/run.py:39 use 2 and 4, wkv5a/run.py:60 lists 17.  Here head size 64 takes
-the matrix-core kernels and every other size up to 128 the row-per-thread kernels of csrc/wkv56.hip (`wkv_rows`); the bar
-is the one of the 64-wide kernels: fp64 oracle, bf16 ops no worse than the reference kernel's arithmetic, fp32 ops 1e-5."""
+the matrix-core kernels, bf16 wkv5 with head size 128 the same kernels with every head as four heads of 64, and every other
+case up to 128 the row-per-thread kernels of csrc/wkv56.hip (`wkv_rows`); the bar is the one of the 64-wide kernels: fp64
+oracle, bf16 ops no worse than the reference kernel's arithmetic, fp32 ops 1e-5."""
 import pytest
 import torch
 
@@ -17,6 +18,7 @@ from _gpu_util import DEV, assert_no_worse, garbage
 pytestmark = pytest.mark.gpu
 BF = torch.bfloat16
 SIZES = [2, 4, 8, 17, 32, 48, 128]
+SWEEPS = 0x100                      # RWKV_FLAG_SWEEPS
 
 
 @pytest.mark.parametrize("N", SIZES)
@@ -168,6 +170,77 @@ def test_wkv5_bf16_reference_default_shape_sampled_heads(lib):
             e = err_ratio(a, g.double().cpu())
             print(f"  {name}: {e:.3e}", flush=True)
             assert e < (4e-3 if name in ("gu", "gw") else 2.5e-3), (name, e)
+
+
+def _wkv5_c_abi(lib, B, T, C, H, r, k, v, w, u, gy, flags, with_forward_workspace):
+    """rwkv_wkv5_forward_ws / rwkv_wkv5_backward_ex: the reference's argument lists (eew, ew in fp32, per-batch gw, gu)."""
+    ew = -torch.exp(w.float().reshape(-1))
+    d = [x.to(DEV) for x in (r, k, v, torch.exp(ew), ew, u, gy)]
+    y, gr, gk, gv = (garbage((B, T, C), BF) for _ in range(4))
+    gw, gu = garbage((B, C), BF), garbage((B, C), BF)
+    if with_forward_workspace:
+        n = lib.rwkv_wkv5_forward_workspace_bytes(B, T, C, H)
+        ws = torch.empty(max(n, 16), device=DEV, dtype=torch.uint8)
+        call("rwkv_wkv5_forward_ws", DEV, B, T, C, H, d[0], d[1], d[2], d[3], d[5], y, ws, n, flags)
+    else:
+        call("rwkv_wkv5_forward_ex", DEV, B, T, C, H, d[0], d[1], d[2], d[3], d[5], y, flags)
+    n = lib.rwkv_wkv5_backward_workspace_bytes(B, T, C, H)
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+    call("rwkv_wkv5_backward_ex", DEV, B, T, C, H, *d, gr, gk, gv, gw, gu, ws, n, flags)
+    torch.cuda.synchronize()
+    return [y, gr, gk, gv, gw, gu]
+
+
+@pytest.mark.parametrize("B,T,H", [(2, 37, 3), (1, 1, 1), (3, 160, 2), (1, 515, 1)])
+def test_wkv5_bf16_head_size_128_both_kernel_families(lib, B, T, H):
+    """Heads of 128 as four heads of 64 on the matrix cores (forward with its workspace), and on the row kernels (the
+    forward without a workspace; RWKV_FLAG_SWEEPS for the backward): each against the oracle, per-batch gw and gu."""
+    N = 128
+    C = H * N
+    assert lib.rwkv_wkv5_forward_workspace_bytes(B, T, C, H) == 2 * B * T * C * 4
+    assert lib.rwkv_wkv5_forward_workspace_bytes(B, T, H * 64, H) == 0
+    r, k, v, w, u, gy = synth.wkv5_inputs(B, T, C, H, seed=500 + T)
+    ref = O.wkv5_grads(B, T, C, H, r, k, v, w, u, gy)
+    emu = O.emulate_wkv5_bf16(B, T, C, H, r, k, v, w, u, gy)
+    for flags, fws, what in ((0, True, "four heads of 64"), (SWEEPS, False, "row kernels")):
+        print(f"\nwkv5 bf16 N=128 B={B} T={T} H={H}: {what}", flush=True)
+        got = _wkv5_c_abi(lib, B, T, C, H, r, k, v, w, u, gy, flags, fws)
+        got[4], got[5] = torch.sum(got[4], 0), torch.sum(got[5], 0)       # as the wrapper does (wkv5_bf16/run.py:86-87)
+        names = ["y", "gr", "gk", "gv", "gw", "gu"]
+        if T == 1:                                                        # one step: the decay feeds nothing
+            assert float(got[4].float().abs().max()) == 0.0
+        for name, a, e, g in zip(names, ref, emu, got):
+            assert_no_worse(f"wkv5 N=128 {what} {name}", a, e.reshape(a.shape), g.reshape(a.shape))
+
+
+def test_wkv5_bf16_head_size_128_fast_decay_takes_the_step_by_step_path(lib):
+    """A channel that decays by e^-20 per step sends the blocks holding it down the kernels' exact path; the other blocks of
+    the same head stay on the matrix cores."""
+    B, T, H, N = 2, 100, 2, 128
+    C = H * N
+    r, k, v, w, u, gy = synth.wkv5_inputs(B, T, C, H, seed=77)
+    w = w.clone()
+    w[0, 70] = 3.0                                     # second key block of head 0
+    w[1, 3] = 2.5                                      # first key block of head 1
+    ref = O.wkv5_grads(B, T, C, H, r, k, v, w, u, gy)
+    emu = O.emulate_wkv5_bf16(B, T, C, H, r, k, v, w, u, gy)
+    got = _wkv5_c_abi(lib, B, T, C, H, r, k, v, w, u, gy, 0, True)
+    got[4], got[5] = torch.sum(got[4], 0), torch.sum(got[5], 0)
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, got):
+        assert_no_worse(f"wkv5 N=128 fast decay {name}", a, e.reshape(a.shape), g.reshape(a.shape))
+
+
+def test_wkv5_bf16_head_size_128_workspace_is_checked(lib):
+    B, T, H, C = 1, 40, 1, 128
+    x = torch.zeros(B * T * C, device=DEV, dtype=BF)
+    f = torch.zeros(C, device=DEV)
+    small = torch.empty(64, device=DEV, dtype=torch.uint8)
+    p = x.data_ptr()
+    assert lib.rwkv_wkv5_forward_ws(None, B, T, C, H, p, p, p, f.data_ptr(), p, p, small.data_ptr(), 64, 0) == -4
+    assert lib.rwkv_wkv5_forward_ws(None, B, T, C, H, p, p, p, f.data_ptr(), p, p, None, 0, 0) == -4
+    # the row kernels need none
+    assert lib.rwkv_wkv5_forward_ws(None, B, T, C, H, p, p, p, f.data_ptr(), p, p, None, 0, SWEEPS) == 0
+    torch.cuda.synchronize()
 
 
 def test_head_size_limits(lib):
