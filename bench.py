@@ -48,9 +48,10 @@ TRAFFIC_MEASURED = {
     # profiles/rwkv7_chunk_kernels_B8_T4096_C4096.md (four calls of T = 1024)
     "rwkv7c_fwd x4 (T=1024 each)": 4 * (411.2e6 + 746.6e6),
     "rwkv7c_bwd x4": 4 * (1149.7e6 + 411.0e6),
-    # profiles/wkv5_rows_kernels_B8_T4096_C4096_N128.md
-    "wkv_rows<FWD>": 805.4e6 + 268.4e6, "wkv_rows<GR>": 1073.8e6 + 805.4e6,
-    "wkv_rows<GV>": 805.4e6 + 268.4e6, "wkv_rows<GK>": 1610.8e6 + 268.5e6,
+    # profiles/wkv5_split_kernels_B8_T4096_C4096_N128.md (both launches of a kernel and the sums that follow them)
+    "wkv6_fwd_ws<head decay, split> x2": (805.7e6 + 536.9e6) + (1342.5e6 + 268.5e6),
+    "wkv6_bwd_a_ws<head decay, split> x2": (1095.4e6 + 1334.3e6) + (1638.6e6 + 1065.4e6),
+    "wkv6_bwd_b_ws<head decay, split> x2 + split_sum x2": 2 * (1911.1e6 + 1076.0e6) + 2 * (1073.7e6 + 268.4e6),
     # profiles/wkv4_reg_kernels_B4_T512_C768.md
     "wkv4_fwd_reg": 12.7e6 + 6.3e6,
     "wkv4_bwd_reg + wkv4_batch_sum": 19.1e6 + 12.6e6,
@@ -186,8 +187,8 @@ def make_wkv5(dev, H=32, N=64):
                    ("wkv6_bwd_a_ws<head decay>", bwd(1), 10 * C * tok),           # r k v gy -> gr (+ fp32 workspace)
                    ("wkv6_bwd_b_ws<head decay>", bwd(4), 12 * C * tok)]           # r k v gy -> gk gv
     else:
-        kernels = [("wkv6_fwd_ws<head decay, split> x2 + split_sum", lambda: call("rwkv_wkv5_forward_ws", dev, B, T, C, H, r, k, v, eew, u, y, fws, fbytes, FLAGS), 8 * C * tok),
-                   ("wkv6_bwd_a_ws<head decay, split> x2 + split_sum", bwd(1), 10 * C * tok),
+        kernels = [("wkv6_fwd_ws<head decay, split> x2", lambda: call("rwkv_wkv5_forward_ws", dev, B, T, C, H, r, k, v, eew, u, y, fws, fbytes, FLAGS), 8 * C * tok),
+                   ("wkv6_bwd_a_ws<head decay, split> x2", bwd(1), 10 * C * tok),
                    ("wkv6_bwd_b_ws<head decay, split> x2 + split_sum x2", bwd(4), 12 * C * tok)]
 
     def cpu_baseline(t_cpu=256):

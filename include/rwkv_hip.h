@@ -139,7 +139,7 @@ int rwkv_wkv5_forward_ex(void* stream, int B, int T, int C, int H,
                       const float* eew, const rwkv_bf16* u, rwkv_bf16* y, unsigned flags);
 /* The forward with a workspace.  It has no counterpart in the reference (whose forward takes none): heads of 128 channels
  * run on the matrix-core kernels as four heads of 64 whose fp32 terms are added afterwards, and those terms need
- * rwkv_wkv5_forward_workspace_bytes() of scratch (2*B*T*C floats; 0 for every other head size, which then needs no
+ * rwkv_wkv5_forward_workspace_bytes() of scratch (B*T*C floats; 0 for every other head size, which then needs no
  * workspace and runs exactly as rwkv_wkv5_forward_ex).  Without it heads of 128 take the one-row-per-lane kernels. */
 size_t rwkv_wkv5_forward_workspace_bytes(int B, int T, int C, int H);
 int rwkv_wkv5_forward_ws(void* stream, int B, int T, int C, int H,

@@ -146,12 +146,14 @@ int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
                             const uint16_t* s0, const uint16_t* gy, uint16_t* gk, uint16_t* gv, uint16_t* gw,
                             uint16_t* gs, const float* rdr);
 // wkv5 with heads of 128 channels as four heads of 64 (see ArgsB in wkv6_chunk.h): one launch of each kernel per value
-// of `cross`, results in fp32
+// of `cross`.  Forward and first sweep: the first launch (cross = 0) leaves fp32 terms, the second adds them to its own
+// and writes the bf16 outputs.  Second sweep: both launches leave fp32 terms (its waves have no registers to spare for
+// the first launch's terms), which the caller adds.
 int launch_wkv5_fwd_split(hipStream_t st, int cross, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k,
-                          const uint16_t* v, const float* eew, const uint16_t* u, float* y32);
+                          const uint16_t* v, const float* eew, const uint16_t* u, float* y32, uint16_t* y);
 int launch_wkv5_bwd_a_split(hipStream_t st, int cross, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k,
                             const uint16_t* v, const float* ew, const uint16_t* u, const uint16_t* gy, float* gr32, float* gu32,
-                            float* rdr);
+                            uint16_t* gr, uint16_t* gu, float* rdr);
 int launch_wkv5_bwd_b_split(hipStream_t st, int cross, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k,
                             const uint16_t* v, const float* ew, const uint16_t* u, const uint16_t* gy, float* gk32, float* gv32,
                             float* gw32, const float* rdr);

@@ -918,22 +918,21 @@ void launch_split_sum(hipStream_t st, size_t n, const float* p0, const float* p1
     hipLaunchKernelGGL(split_sum, dim3(static_cast<unsigned>((n4 + 255) / 256)), dim3(256), 0, st, n4,
                        reinterpret_cast<const float4*>(p0), reinterpret_cast<const float4*>(p1), reinterpret_cast<uint2*>(out));
 }
-// forward: two terms of y
-size_t fwd_split_bytes(int B, int T, int C) { return 2 * static_cast<size_t>(B) * T * C * sizeof(float); }
-// backward: r dr' [B,T,C], the stored states of 2 H heads of 64, two terms each of gr, gk, gv [B,T,C] and of gu, gw [B,C]
+// forward: the first launch's term of y
+size_t fwd_split_bytes(int B, int T, int C) { return static_cast<size_t>(B) * T * C * sizeof(float); }
+// backward: r dr' [B,T,C], the stored states of 2 H heads of 64, then fp32 terms: the first launch's gr [B,T,C], both
+// launches' gk and gv, the first launch's gu [B,C], both launches' gw
 size_t bwd_split_floats_before_terms(int B, int T, int C, int H) {
     const size_t nchunks = (static_cast<size_t>(T) + 31) / 32, npck = (nchunks + 3) / 4;
     return static_cast<size_t>(B) * T * C + static_cast<size_t>(B) * 2 * H * npck * 64 * 64;
 }
 size_t bwd_split_bytes(int B, int T, int C, int H) {
-    return (bwd_split_floats_before_terms(B, T, C, H) + 6 * static_cast<size_t>(B) * T * C + 4 * static_cast<size_t>(B) * C) * sizeof(float);
+    return (bwd_split_floats_before_terms(B, T, C, H) + 5 * static_cast<size_t>(B) * T * C + 3 * static_cast<size_t>(B) * C) * sizeof(float);
 }
 int launch_fwd_split(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
                      const float* eew, const uint16_t* u, uint16_t* y, float* ws) {
-    const size_t n = static_cast<size_t>(B) * T * C;
     for (int cross = 0; cross < 2; ++cross)
-        if (int e = launch_wkv5_fwd_split(st, cross, B, T, C, H, r, k, v, eew, u, ws + cross * n)) return e;
-    launch_split_sum(st, n, ws, ws + n, y);
+        if (int e = launch_wkv5_fwd_split(st, cross, B, T, C, H, r, k, v, eew, u, ws, y)) return e;
     return launch_status();
 }
 int launch_bwd_split(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
@@ -943,20 +942,16 @@ int launch_bwd_split(hipStream_t st, int B, int T, int C, int H, const uint16_t*
     const size_t n = static_cast<size_t>(B) * T * C, m = static_cast<size_t>(B) * C;
     float* rdr = ws;
     float* gr32 = ws + bwd_split_floats_before_terms(B, T, C, H);
-    float* gk32 = gr32 + 2 * n;
+    float* gk32 = gr32 + n;
     float* gv32 = gk32 + 2 * n;
     float* gu32 = gv32 + 2 * n;
-    float* gw32 = gu32 + 2 * m;
+    float* gw32 = gu32 + m;
     // the second sweep of a launch reads the r dr' its own first sweep has left: first, second, first, second
     for (int cross = 0; cross < 2; ++cross) {
         if (passes & RWKV_PASS_GR)
-            if (int e = launch_wkv5_bwd_a_split(st, cross, B, T, C, H, r, k, v, ew, u, gy, gr32 + cross * n, gu32 + cross * m, rdr)) return e;
+            if (int e = launch_wkv5_bwd_a_split(st, cross, B, T, C, H, r, k, v, ew, u, gy, gr32, gu32, gr, gu, rdr)) return e;
         if (passes & RWKV_PASS_GK)
             if (int e = launch_wkv5_bwd_b_split(st, cross, B, T, C, H, r, k, v, ew, u, gy, gk32 + cross * n, gv32 + cross * n, gw32 + cross * m, rdr)) return e;
-    }
-    if (passes & RWKV_PASS_GR) {
-        launch_split_sum(st, n, gr32, gr32 + n, gr);
-        launch_split_sum(st, m, gu32, gu32 + m, gu);
     }
     if (passes & RWKV_PASS_GK) {
         launch_split_sum(st, n, gk32, gk32 + n, gk);

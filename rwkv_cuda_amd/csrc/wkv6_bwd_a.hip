@@ -48,7 +48,9 @@ struct alignas(16) SmemA2 {
 
 // ---------------------------------------------------------------------------------------------------- prep waves
 // base, h: where r, k, w, u (and gu) of this workgroup sit; vbase: where v, gy sit (the same place unless the head is split)
-template <int WMODE, bool SPLIT>
+// SPLIT: 0 = whole heads; 1 = first launch of a split head (gr, gu leave as fp32 terms); 2 = second launch (the first
+// launch's terms are added and gr, gu leave in bf16)
+template <int WMODE, int SPLIT>
 DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base, const size_t vbase, const int h, const int nchunks) {
     const int lane = tid & 63, wid = __builtin_amdgcn_readfirstlane(tid >> 6), l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
@@ -263,13 +265,14 @@ DEVINL void bwa_prep(SmemA2& S, const ArgsB& a, const int tid, const size_t base
         float s = S.gfast[0][tid] + S.gfast[1][tid];
         for (int t = 0; t < L; ++t) s += S.Yx[0][t][tid];
         const size_t at = static_cast<size_t>(blockIdx.x / a.H) * C + h * N + tid;
-        if constexpr (SPLIT) a.gu32[at] = s;
+        if constexpr (SPLIT == 1) a.gu32[at] = s;
+        else if constexpr (SPLIT == 2) a.gu[at] = f2bf(s + a.gu32[at]);
         else a.gu[at] = f2bf(s);
     }
 }
 
 // ---------------------------------------------------------------------------------------------------- state waves
-template <int WMODE, bool SPLIT>
+template <int WMODE, int SPLIT>
 DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t base, const size_t bh, const int nchunks) {
     const int lane = tid & 63, sw = __builtin_amdgcn_readfirstlane(tid >> 6) - NPREP, q = sw & 3, ih = sw >> 2, l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
@@ -302,7 +305,7 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
         const float4 x = *reinterpret_cast<const float4*>(&S.outR[pb][row][4 * l16]);
         if (tg < T) {
             const uint32_t o = static_cast<uint32_t>(tg) * C + 4 * l16;
-            if constexpr (!SPLIT) store8(a.gr + base, o * 2, y);      // split heads: gr has left in fp32 already
+            if constexpr (SPLIT != 1) store8(a.gr + base, o * 2, y);  // first launch of a split head: gr has left as an fp32 term
             store16(a.rdr + base, o * 4, f32x4{x.x, x.y, x.z, x.w});
         }
     };
@@ -322,6 +325,11 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
                 store16(slot, (sw * 64 + lane) * 32, D[0]);
                 store16(slot, (sw * 64 + lane) * 32 + 16, D[1]);
             }
+        }
+        [[maybe_unused]] f32x4 term = zero4;           // SPLIT == 2: the first launch's term of this lane's gr
+        if constexpr (SPLIT == 2) {
+            const int tg = c0 + 16 * ih + l16;
+            term = *reinterpret_cast<const f32x4*>(a.gr32 + base + static_cast<size_t>(tg < T ? tg : T - 1) * C + j4);
         }
         f32x4 own;                                     // (GY S)^T of this half of i: rows j4 + v, token 16 ih + l16
         bf16x8 ktH, ktL;                               // K'^T of the own key channels: lane = j_own, K slots = tokens
@@ -412,9 +420,10 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
                 rd[v] = rr[v] * drp;
                 gu_acc[v] = fmaf(rr[v], kv, gu_acc[v]);
             }
-            if constexpr (SPLIT) {
+            if constexpr (SPLIT == 1) {
                 if (c0 + t < T) store16(a.gr32 + base, (static_cast<uint32_t>(c0 + t) * C + j4) * 4, f32x4{gr[0], gr[1], gr[2], gr[3]});
             } else {
+                if constexpr (SPLIT == 2) { gr[0] += term[0]; gr[1] += term[1]; gr[2] += term[2]; gr[3] += term[3]; }
                 *reinterpret_cast<uint2*>(&S.outG[i & 1][t][j4 >> 1]) = make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3]));
             }
             *reinterpret_cast<float4*>(&S.outR[i & 1][t][j4]) = make_float4(rd[0], rd[1], rd[2], rd[3]);
@@ -439,7 +448,11 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
             }
             if (c0 + xt < T) {
                 const uint32_t o = static_cast<uint32_t>(c0 + xt) * C + xj;
-                if constexpr (SPLIT) store16(a.gr32 + base, o * 4, f32x4{gr[0], gr[1], gr[2], gr[3]});
+                if constexpr (SPLIT == 2) {            // rare path: read the first launch's term here
+                    const f32x4 f = *reinterpret_cast<const f32x4*>(a.gr32 + base + o);
+                    gr[0] += f[0]; gr[1] += f[1]; gr[2] += f[2]; gr[3] += f[3];
+                }
+                if constexpr (SPLIT == 1) store16(a.gr32 + base, o * 4, f32x4{gr[0], gr[1], gr[2], gr[3]});
                 else store8(a.gr + base, o * 2, make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3])));
                 store16(a.rdr + base, o * 4, f32x4{rd[0], rd[1], rd[2], rd[3]});
             }
@@ -459,12 +472,12 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
     __syncthreads();
 }
 
-template <int WMODE, bool SPLIT = false>
+template <int WMODE, int SPLIT = 0>
 __global__ __launch_bounds__(NTA) void wkv6_bwd_a_ws(const ArgsB a) {
     __shared__ SmemA2 S;
     const int tid = threadIdx.x;
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
-    const int hk = SPLIT ? h ^ a.cross : h;            // the block of 64 channels that r, k, w, u come from and gr, gu go to
+    const int hk = SPLIT != 0 ? h ^ a.cross : h;       // the block of 64 channels that r, k, w, u come from and gr, gu go to
     const size_t vbase = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
     const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(hk) * N;
     const size_t bh = static_cast<size_t>(b) * a.H + h;
@@ -501,11 +514,13 @@ int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
 // wkv5 with heads of 128 channels: the first sweep of one of the two launches described at ArgsB (H counts the heads of 128)
 int launch_wkv5_bwd_a_split(hipStream_t st, int cross, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k,
                             const uint16_t* v, const float* ew, const uint16_t* u, const uint16_t* gy, float* gr32, float* gu32,
-                            float* rdr) {
+                            uint16_t* gr, uint16_t* gu, float* rdr) {
     ArgsB a{};
     a.T = T; a.C = C; a.H = 2 * H; a.r = r; a.k = k; a.v = v; a.w = ew; a.u = u; a.s0 = nullptr; a.gy = gy;
-    a.rdr = rdr; a.cross = cross; a.gr32 = gr32; a.gu32 = gu32;
-    hipLaunchKernelGGL((wkv6_bwd_a_ws<W_HEAD, true>), dim3(B * 2 * H), dim3(NTA), 0, st, a);
+    a.rdr = rdr; a.cross = cross; a.gr32 = gr32; a.gu32 = gu32; a.gr = gr; a.gu = gu;
+    // the first launch leaves its terms in gr32, gu32; the second adds them to its own and writes gr, gu
+    if (cross == 0) hipLaunchKernelGGL((wkv6_bwd_a_ws<W_HEAD, 1>), dim3(B * 2 * H), dim3(NTA), 0, st, a);
+    else hipLaunchKernelGGL((wkv6_bwd_a_ws<W_HEAD, 2>), dim3(B * 2 * H), dim3(NTA), 0, st, a);
     return launch_status();
 }
 

@@ -314,7 +314,9 @@ DEVINL void fwd_prep(SmemF& S, const ArgsC& a, const int tid, const size_t base,
 }
 
 // ---------------------------------------------------------------------------------------------------- state waves
-template <int WMODE, bool SPLIT>
+// SPLIT: 0 = whole heads; 1 = first launch of a split head (y leaves as an fp32 term); 2 = second launch (the first
+// launch's term is added and y leaves in bf16)
+template <int WMODE, int SPLIT>
 DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base, const size_t bh, const int nchunks) {
     const int lane = tid & 63, sw = __builtin_amdgcn_readfirstlane(tid >> 6) - NPREP, q = sw & 3, jh = sw >> 2, l16 = lane & 15, g = lane >> 4;
     const int T = a.T, C = a.C;
@@ -337,6 +339,13 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
 
     bf16x8 Vop = op4(make_uint4(0, 0, 0, 0));          // v of the chunk in flight: lane = value channel, K slots = tokens
     f32x4 Yk = zero4;                                  // y^T rows 16q + 4g + v, tokens 16 jh + l16: this half of the key channels
+    [[maybe_unused]] float4 term = make_float4(0.f, 0.f, 0.f, 0.f);   // SPLIT == 2: the first launch's term of the tile in flight
+    auto fetch_term = [&](const int c) __attribute__((always_inline)) {
+        if constexpr (SPLIT == 2) {
+            const int t = c * L + 16 * jh + l16;
+            term = *reinterpret_cast<const float4*>(a.y32 + base + static_cast<size_t>(t < T ? t : T - 1) * C + 16 * q + 4 * g);
+        }
+    };
 
     // y of chunk c (tokens 16 jh + l16): own half + partner's half + A V
     auto finish = [&](const int c, const bool was_exact) __attribute__((always_inline)) {
@@ -346,8 +355,9 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
             Y = mfma(Vop, lds_op(&S.AmH[c & 1][16 * jh + l16][4 * g]), Y);
             Y = mfma(Vop, lds_op(&S.AmL[c & 1][16 * jh + l16][4 * g]), Y);
             const int t = c * L + 16 * jh + l16;
+            if constexpr (SPLIT == 2) { Y[0] += term.x; Y[1] += term.y; Y[2] += term.z; Y[3] += term.w; }
             if (t < T) {
-                if constexpr (SPLIT)
+                if constexpr (SPLIT == 1)
                     *reinterpret_cast<float4*>(a.y32 + base + static_cast<size_t>(t) * C + 16 * q + 4 * g) = make_float4(Y[0], Y[1], Y[2], Y[3]);
                 else
                     *reinterpret_cast<uint2*>(a.y + base + static_cast<size_t>(t) * C + 16 * q + 4 * g) =
@@ -358,12 +368,16 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
             const float4 p0 = *reinterpret_cast<const float4*>(&S.Yx[c & 1][0][t][i4]);
             const float4 p1 = *reinterpret_cast<const float4*>(&S.Yx[c & 1][1][t][i4]);
             if (c * L + t < T) {
-                if constexpr (SPLIT)
-                    *reinterpret_cast<float4*>(a.y32 + base + static_cast<size_t>(c * L + t) * C + i4) =
-                        make_float4(p0.x + p1.x, p0.y + p1.y, p0.z + p1.z, p0.w + p1.w);
+                float4 s4 = make_float4(p0.x + p1.x, p0.y + p1.y, p0.z + p1.z, p0.w + p1.w);
+                if constexpr (SPLIT == 2) {            // this thread's elements are not those of `term`: read here (rare path)
+                    const float4 f = *reinterpret_cast<const float4*>(a.y32 + base + static_cast<size_t>(c * L + t) * C + i4);
+                    s4 = make_float4(s4.x + f.x, s4.y + f.y, s4.z + f.z, s4.w + f.w);
+                }
+                if constexpr (SPLIT == 1)
+                    *reinterpret_cast<float4*>(a.y32 + base + static_cast<size_t>(c * L + t) * C + i4) = s4;
                 else
                     *reinterpret_cast<uint2*>(a.y + base + static_cast<size_t>(c * L + t) * C + i4) =
-                        make_uint2(pack_bf2(p0.x + p1.x, p0.y + p1.y), pack_bf2(p0.z + p1.z, p0.w + p1.w));
+                        make_uint2(pack_bf2(s4.x, s4.y), pack_bf2(s4.z, s4.w));
             }
         }
     };
@@ -375,6 +389,7 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
         const OperandSet& O = S.set[i & 1];
         const bool exact = __builtin_amdgcn_readfirstlane(O.exact) != 0;
         if (i > 0) finish(i - 1, exact_prev);
+        fetch_term(i);                                 // used by finish(i), one iteration from here
         if (!exact) {
             // ------------------------------------------------------------ y^T = (d1 S) R'^T over this wave's key channels
             const float4 da = *reinterpret_cast<const float4*>(&O.d1[j0[0]]);
@@ -453,7 +468,7 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
     finish(nchunks - 1, exact_prev);
 }
 
-template <int WMODE, bool SPLIT = false>
+template <int WMODE, int SPLIT = 0>
 __global__ __launch_bounds__(NTF) void wkv6_fwd_ws(const ArgsC a) {
     __shared__ SmemF S;
     const int tid = threadIdx.x;
@@ -463,16 +478,16 @@ __global__ __launch_bounds__(NTF) void wkv6_fwd_ws(const ArgsC a) {
     const int nchunks = (a.T + L - 1) / L;
     // positions of A that no tile ever writes (t < 16 <= s) must read as zero
     for (int i = tid; i < 2 * L * OS; i += NTF) { (&S.AmH[0][0][0])[i] = 0; (&S.AmL[0][0][0])[i] = 0; }
-    if constexpr (SPLIT) {
+    if constexpr (SPLIT != 0) {
         const int hk = h ^ a.cross;                    // the block of 64 channels that r, k, w, u come from
         const size_t kbase = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(hk) * N;
         if (tid < N) S.u[tid] = bf2f(a.u[hk * N + tid]);
         if (__builtin_amdgcn_readfirstlane(tid >> 6) < NPREP) fwd_prep<WMODE>(S, a, tid, kbase, base, hk, nchunks);
-        else fwd_state<WMODE, true>(S, a, tid, base, bh, nchunks);
+        else fwd_state<WMODE, SPLIT>(S, a, tid, base, bh, nchunks);
     } else {
         if (tid < N) S.u[tid] = bf2f(a.u[h * N + tid]);
         if (__builtin_amdgcn_readfirstlane(tid >> 6) < NPREP) fwd_prep<WMODE>(S, a, tid, base, base, h, nchunks);
-        else fwd_state<WMODE, false>(S, a, tid, base, bh, nchunks);
+        else fwd_state<WMODE, 0>(S, a, tid, base, bh, nchunks);
     }
 }
 
@@ -491,11 +506,13 @@ int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H,
 
 // wkv5 with heads of 128 channels: one of the two launches described at ArgsB (H counts the heads of 128)
 int launch_wkv5_fwd_split(hipStream_t st, int cross, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k,
-                          const uint16_t* v, const float* eew, const uint16_t* u, float* y32) {
+                          const uint16_t* v, const float* eew, const uint16_t* u, float* y32, uint16_t* y) {
     ArgsC a{};
-    a.T = T; a.C = C; a.H = 2 * H; a.r = r; a.k = k; a.v = v; a.w = eew; a.u = u; a.s0 = nullptr; a.y = nullptr;
+    a.T = T; a.C = C; a.H = 2 * H; a.r = r; a.k = k; a.v = v; a.w = eew; a.u = u; a.s0 = nullptr; a.y = y;
     a.cross = cross; a.y32 = y32;
-    hipLaunchKernelGGL((wkv6_fwd_ws<W_HEAD, true>), dim3(B * 2 * H), dim3(NTF), 0, st, a);
+    // the first launch leaves its term in y32, the second adds it to its own and writes y
+    if (cross == 0) hipLaunchKernelGGL((wkv6_fwd_ws<W_HEAD, 1>), dim3(B * 2 * H), dim3(NTF), 0, st, a);
+    else hipLaunchKernelGGL((wkv6_fwd_ws<W_HEAD, 2>), dim3(B * 2 * H), dim3(NTF), 0, st, a);
     return launch_status();
 }
 
