@@ -72,8 +72,9 @@ int rwkv_abi_version(void);
  *   w[C]  = -exp(w_raw) (the wrapper's pre-transform, wkv/run.py:95), u[C], k,v,y,gy,gk,gv[B,T,C].
  *   gw,gu[B,C] are per-batch partials that the kernel ADDS into (caller zero-fills, as
  *   wkv/run.py:110-111 does); gw already carries the factor w of the w_raw chain rule.
- *   The backward keeps its per-step intermediates in gk, gv and the workspace (B*T*C floats)
- *   where the reference uses per-thread arrays of 4096 floats, so T is not limited.
+ *   Where the reference keeps the backward's per-step intermediates in per-thread arrays of 4096 floats, here they stay
+ *   in registers up to T = 32768 and go to gk, gv and the workspace (B*T*C floats) beyond, so T is not limited; the
+ *   workspace is asked for at every T.
  * ------------------------------------------------------------------------------------- */
 int rwkv_wkv4_forward(void* stream, int B, int T, int C,
                       const float* w, const float* u, const float* k, const float* v, float* y);
@@ -85,7 +86,7 @@ int rwkv_wkv4_backward(void* stream, int B, int T, int C,
 
 /* rwkv_wkv4_backward without a workspace argument and without any allocation.  It has no counterpart in the reference;
  * it is for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
- * that forbid hipMalloc.  The backward's scratch (B*T*C floats) lives in a file-scope device array of the library,
+ * that forbid hipMalloc.  The backward's scratch (B*T*C floats, touched only beyond T = 32768) lives in a file-scope device array of the library,
  * rwkv_wkv4_backward_noalloc_max_elems() floats (8 MiB) that every GPU the library runs on holds until the process
  * ends; B*T*C beyond that returns RWKV_ERR_WORKSPACE.  All calls on one GPU share that one array: calls that overlap
  * in time on the same GPU (two streams, two threads) race; serialise them.  Results are those of rwkv_wkv4_backward. */
