@@ -79,9 +79,10 @@ struct ArgsB {
 //     y_I = sum_J wkv(r_J, k_J, v_I; w_J, u_J)     gv_I = sum_J ...     gr_J, gk_J, gw_J, gu_J = sum_I ...
 // and each term is exactly the 64-channel problem.  A launch treats the tensor as 2 H heads of 64: workgroup h takes its
 // v, gy (and y, gv) from block h and its r, k, w, u (and gr, gk, gw, gu) from block h ^ cross.  cross = 0 gives the
-// diagonal blocks (I = J), cross = 1 the other two, so every output element gets exactly one term from each launch; the
-// terms are written in fp32 (y32, gr32, ...: [B,T,C] like the tensors, gw32 / gu32 [B,C]) and added afterwards, which
-// keeps the single bf16 rounding of the outputs.
+// diagonal blocks (I = J), cross = 1 the other two, so every output element gets exactly one term from each launch.  The
+// first launch writes its terms in fp32 (y32, gr32, ...: [B,T,C] like the tensors, gw32 / gu32 [B,C]); the second
+// launch of the forward and of the first sweep reads them back, adds its own and writes the bf16 outputs, while both
+// launches of the second sweep write terms that the caller adds.  Either way an output is rounded to bf16 once.
 
 // Operand format.  An fp32 value x is used as hi = bf16(x), lo = bf16(x - hi).  Along the K axis of an MFMA a lane holds
 // 8 slots = 4 consecutive elements e0..e3 as  P = [h0 h1 h2 h3 | l0 l1 l2 l3]  (dwords H01, H23, L01, L23).  With the
