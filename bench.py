@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: WKV6 bf16 forward+backward at B=8, T=4096, C=2048 (H=32, N=64) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wkv6|wkv6_state|wkv5|rwkv7|wkv4|timex]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wkv6|wkv6_state|wkv5|wkv5_n128|rwkv7|wkv4|wkv4_b32|timex|...]
 
 A "step" is one forward + one backward of the operator over one batch of synthetic inputs that are
 already resident in HBM, through the same C-ABI calls and the same wrapper-side torch work
@@ -55,6 +55,9 @@ TRAFFIC_MEASURED = {
     # profiles/wkv4_reg_kernels_B4_T512_C768.md
     "wkv4_fwd_reg": 12.7e6 + 6.3e6,
     "wkv4_bwd_reg + wkv4_batch_sum": 19.1e6 + 12.6e6,
+    # profiles/wkv4_reg_kernels_B32_T768_C768.md
+    "wkv4_fwd_reg B32 T768": 152.5e6 + 78.4e6,
+    "wkv4_bwd_reg + wkv4_batch_sum B32 T768": 227.2e6 + 151.7e6,
     # profiles/timex_mfma_kernels_B32_C768_T768.md
     "timex_conv_mfma (forward)": 77.9e6 + 75.5e6,
     "timex backward (timex_conv_mfma + timex_gw_sum_mfma)": (77.9e6 + 75.5e6) + (151.1e6 + 2.4e6),
@@ -364,11 +367,12 @@ def make_rwkv7(dev, fp32=False):
     return step, tok, kernels, cfg, cpu_baseline, 20 * eb * C * tok
 
 
-def make_wkv4(dev):
+def make_wkv4(dev, B=4, T=512):
+    """B4 T512: the configuration of the contract; B32 T768: the shape of the reference's own check (wkv/run.py:152-154)."""
     from rwkv_cuda_amd import _lib, synth
     from rwkv_cuda_amd._call import call
     lib = _lib.load()
-    B, T, C = 4, 512, 768
+    C = 768
     w_raw, u, k, v, gy = (x.to(dev) for x in synth.wkv4_inputs(B, T, C, seed=42))
     y, gk, gv = (torch.empty(B, T, C, device=dev) for _ in range(3))
     nbytes = lib.rwkv_wkv4raw_backward_workspace_bytes(B, T, C)
@@ -382,8 +386,9 @@ def make_wkv4(dev):
         call("rwkv_wkv4raw_forward", dev, B, T, C, w_raw, u, k, v, y)
         call("rwkv_wkv4raw_backward", dev, B, T, C, w_raw, u, k, v, gy, gw, gu, gk, gv, ws, nbytes)
 
-    kernels = [("wkv4_fwd_reg", lambda: call("rwkv_wkv4raw_forward", dev, B, T, C, w_raw, u, k, v, y), 12 * C * tok),
-               ("wkv4_bwd_reg + wkv4_batch_sum", lambda: call("rwkv_wkv4raw_backward", dev, B, T, C, w_raw, u, k, v, gy, gw, gu, gk, gv, ws, nbytes), 20 * C * tok)]
+    tag = "" if (B, T) == (4, 512) else f" B{B} T{T}"
+    kernels = [("wkv4_fwd_reg" + tag, lambda: call("rwkv_wkv4raw_forward", dev, B, T, C, w_raw, u, k, v, y), 12 * C * tok),
+               ("wkv4_bwd_reg + wkv4_batch_sum" + tag, lambda: call("rwkv_wkv4raw_backward", dev, B, T, C, w_raw, u, k, v, gy, gw, gu, gk, gv, ws, nbytes), 20 * C * tok)]
 
     def cpu_baseline():
         from oracle import wkv4 as O
@@ -444,9 +449,10 @@ WORKLOADS = {
     "rwkv7": make_rwkv7,
     "rwkv7_fp32": lambda dev: make_rwkv7(dev, fp32=True),
     "wkv4": make_wkv4,
+    "wkv4_b32": lambda dev: make_wkv4(dev, B=32, T=768),
     "timex": make_timex,
 }
-DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_n128": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "timex": "f32"}
+DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_n128": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "wkv4_b32": "f32", "timex": "f32"}
 
 
 def main():
