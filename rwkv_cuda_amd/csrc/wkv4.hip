@@ -898,14 +898,22 @@ __global__ __launch_bounds__(BLK_CH * NSEG) void wkv4_bwd_blk(int T, int C, cons
     }
 }
 
-// out[c] = sum_b part[b][c], in the fixed order b = 0, 1, ...: the wrapper's torch.sum(gw, dim=0) (wkv/run.py:115-116)
+// out[c] = sum_b part[b][c]: the wrapper's torch.sum(gw, dim=0) (wkv/run.py:115-116), in a fixed order: four lanes per
+// channel take every fourth batch row each, and their sums are added in lane order
 __global__ __launch_bounds__(256) void wkv4_batch_sum(int B, int C, const float* __restrict__ pw, const float* __restrict__ pu,
                                                       float* __restrict__ gw, float* __restrict__ gu) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= C) return;
+    __shared__ float2 part[4][64];
+    const int cl = threadIdx.x & 63, q = threadIdx.x >> 6, c = blockIdx.x * 64 + cl;
     float a = 0.f, b2 = 0.f;
-    for (int b = 0; b < B; ++b) { a += pw[static_cast<size_t>(b) * C + c]; b2 += pu[static_cast<size_t>(b) * C + c]; }
-    gw[c] = a; gu[c] = b2;
+    if (c < C)
+        for (int b = q; b < B; b += 4) { a += pw[static_cast<size_t>(b) * C + c]; b2 += pu[static_cast<size_t>(b) * C + c]; }
+    part[q][cl] = make_float2(a, b2);
+    __syncthreads();
+    if (q == 0 && c < C) {
+        const float2 x0 = part[0][cl], x1 = part[1][cl], x2 = part[2][cl], x3 = part[3][cl];
+        gw[c] = ((x0.x + x1.x) + x2.x) + x3.x;
+        gu[c] = ((x0.y + x1.y) + x2.y) + x3.y;
+    }
 }
 
 // Which form runs: one lane per scan beyond the grid's y range, inputs in registers while a segment has at most 16
@@ -1042,7 +1050,7 @@ int rwkv_wkv4raw_backward(void* stream, int B, int T, int C, const float* w_raw,
     float* pw = ze + static_cast<size_t>(B) * T * C;
     float* pu = pw + static_cast<size_t>(B) * C;
     launch4_bwd<true>(st, B, T, C, w_raw, u, k, v, gy, pw, pu, gk, gv, ze);
-    hipLaunchKernelGGL(wkv4_batch_sum, dim3((C + 255) / 256), dim3(256), 0, st, B, C, pw, pu, gw, gu);
+    hipLaunchKernelGGL(wkv4_batch_sum, dim3((C + 63) / 64), dim3(256), 0, st, B, C, pw, pu, gw, gu);
     return launch_status();
 }
 
