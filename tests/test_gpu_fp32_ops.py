@@ -41,6 +41,29 @@ def test_wkv4(lib, B, T, C):
         _check(name, a, g)
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_wkv4_random_shapes(lib, seed):
+    """Shapes drawn at random across the four kernel forms, through the reference-signature entry points (w = -exp(w_raw)
+    in, per-batch gw, gu added into zeroed buffers) instead of the fused ones that the autograd wrapper uses."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    B = int(torch.randint(1, 5, (1,), generator=g))
+    T = int(torch.randint(1, [40, 600, 1100, 2600][seed % 4], (1,), generator=g))
+    C = int(torch.randint(1, 90, (1,), generator=g))
+    print(f"\nwkv4 random B={B} T={T} C={C}", flush=True)
+    w_raw, u, k, v, gy = synth.wkv4_inputs(B, T, C, seed=seed)
+    ref = O4.grads(B, T, C, w_raw, u, k, v, gy)
+    d = [x.to(DEV) for x in (-torch.exp(w_raw), u, k, v, gy)]
+    y, gk, gv = (garbage((B, T, C), torch.float32) for _ in range(3))
+    gw, gu = torch.zeros(B, C, device=DEV), torch.zeros(B, C, device=DEV)
+    n = lib.rwkv_wkv4_backward_workspace_bytes(B, T, C)
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+    call("rwkv_wkv4_forward", d[0].device, B, T, C, d[0], d[1], d[2], d[3], y)
+    call("rwkv_wkv4_backward", d[0].device, B, T, C, *d, gw, gu, gk, gv, ws, n)
+    torch.cuda.synchronize()
+    for name, a, got in zip(["y", "gw", "gu", "gk", "gv"], ref, [y, gw.sum(0), gu.sum(0), gk, gv]):
+        _check(name, a, got)
+
+
 def test_wkv4_more_batch_rows_than_a_grid_dimension(lib):
     """B > 65535 takes the one-lane-per-scan kernels (the time-parallel ones put B on the grid's y axis)."""
     B, T, C = 65536, 3, 1
