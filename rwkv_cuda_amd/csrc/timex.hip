@@ -221,6 +221,173 @@ __global__ __launch_bounds__(TXT) void timex_conv_mfma(const float* __restrict__
     }
 }
 
+// ------------------------------------------------------------------------------------ matrix-core path, bf16 x 3 products
+// The same product with every fp32 operand x cut into three bf16 terms, x = h + m + l (24 mantissa bits together), and
+//     x y = h h' + h m' + m h' + m m' + h l' + l h'          (the terms left out are below 2^-24 of the product)
+// on v_mfma_f32_32x32x16_bf16: six instructions of 16 matrix passes where the fp32 instruction needs eight of 16 passes
+// for the same 32 x 32 x 16 block, i.e. 2.7 times the arithmetic rate at fp32 accuracy (accumulation is fp32 either way).
+// Operand layout of the instruction: lane = (row or column l & 31, K half l >> 5) holds the eight consecutive K slots
+// 8 (l >> 5) .. + 7; accumulator as above.  K slot s of a step is input step 16 ks + s of the 32-step tile.
+//   rows : three planes [32 batch rows][T + 16] bf16; a lane's eight slots are 16 aligned bytes.
+//   taps : the A operand of row t and slot u is line[base(t) + u] for a line that depends only on the direction
+//          (forward: the kernel row in tap order followed by zeros; mirror: 31 zeros, then the reversed kernel row), so a
+//          lane reads eight consecutive bf16 starting at an arbitrary element.  Two copies of every plane, the second
+//          shifted by one element, make that four aligned dwords whatever the parity of the start.
+// LDS: 3 x 32 x (T + 16) x 2 + 6 x (T + 96) x 2 bytes = 160 896 of 163 840 at T = 768, the longest T this form takes.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+constexpr int T_BF3_MAX = 768;
+constexpr int PFQ3 = MROWS * (T_BF3_MAX / 4) / TXT;
+__host__ __device__ inline int bf3_row_stride(int T) { return T + 16; }          // elements; (T + 16) / 2 dwords = 8 or 24 mod 32
+__host__ __device__ inline int bf3_line_len(int T) { return T + 96; }           // (T + 96) / 2 dwords = 16 mod 32: the shifted copy sits 16 banks away
+__host__ __device__ inline size_t bf3_lds_bytes(int T) {
+    return (3 * static_cast<size_t>(MROWS) * bf3_row_stride(T) + 6 * static_cast<size_t>(bf3_line_len(T))) * sizeof(uint16_t);
+}
+struct Bf3 { uint16_t h, m, l; };
+DEVINL Bf3 split3(float x) {
+    Bf3 r;
+    r.h = f2bf(x);
+    const float x1 = x - bf2f(r.h);
+    r.m = f2bf(x1);
+    r.l = f2bf(x1 - bf2f(r.m));
+    return r;
+}
+
+template <bool MIRROR>
+__global__ __launch_bounds__(TXT) void timex_conv_bf3(const float* __restrict__ w, const float* __restrict__ in,
+                                                      float* __restrict__ out, float eps, int B, int C, int T) {
+    extern __shared__ float lds[];
+    const int rs = bf3_row_stride(T), xl = bf3_line_len(T);
+    uint16_t* rp = reinterpret_cast<uint16_t*>(lds);                    // [3][32][rs]
+    uint16_t* al = rp + 3 * MROWS * rs;                                 // [3 planes][2 copies][xl]
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int ln = lane & 31, kh = lane >> 5;
+    const int q4n = T >> 2, total = MROWS * q4n, nt = T >> 5;
+    const int nbg = (B + MROWS - 1) / MROWS, nunits = C * nbg;
+    float4 x[PFQ3];
+    float wr[2];
+    // piece s of this thread is 16-byte piece idx = s TXT + tid of the unit's rows, (row, piece in the row) = (idx / q4n,
+    // idx % q4n): one division here, then steps of TXT
+    const int r_first = tid / q4n, q_first = tid - r_first * q4n, r_step = TXT / q4n, q_step = TXT - r_step * q4n;
+    auto fetch_unit = [&](const int unit) __attribute__((always_inline)) {
+        const int c = unit / nbg, b0 = (unit - c * nbg) * MROWS;
+        int r = r_first, q4 = q_first;
+#pragma unroll
+        for (int s = 0; s < PFQ3; ++s) {
+            const bool live = s * TXT + tid < total && b0 + r < B;
+            x[s] = *reinterpret_cast<const float4*>(in + (static_cast<size_t>(live ? b0 + r : b0) * C + c) * T + (live ? 4 * q4 : 0));
+            r += r_step; q4 += q_step;
+            if (q4 >= q4n) { q4 -= q4n; ++r; }
+        }
+#pragma unroll
+        for (int s = 0; s < 2; ++s) wr[s] = w[static_cast<size_t>(c) * T + min(s * TXT + tid, T - 1)];
+    };
+    auto store_unit = [&](const int unit) __attribute__((always_inline)) {
+        const int c = unit / nbg, b0 = (unit - c * nbg) * MROWS;
+        int r = r_first, q4 = q_first;
+#pragma unroll
+        for (int s = 0; s < PFQ3; ++s) {
+            if (s * TXT + tid < total) {
+                const float4 v = b0 + r < B ? x[s] : make_float4(0.f, 0.f, 0.f, 0.f);
+                const Bf3 a0 = split3(v.x), a1 = split3(v.y), a2 = split3(v.z), a3 = split3(v.w);
+                uint16_t* d = rp + r * rs + 4 * q4;
+                *reinterpret_cast<uint2*>(d) = make_uint2(a0.h | (static_cast<uint32_t>(a1.h) << 16), a2.h | (static_cast<uint32_t>(a3.h) << 16));
+                *reinterpret_cast<uint2*>(d + MROWS * rs) = make_uint2(a0.m | (static_cast<uint32_t>(a1.m) << 16), a2.m | (static_cast<uint32_t>(a3.m) << 16));
+                *reinterpret_cast<uint2*>(d + 2 * MROWS * rs) = make_uint2(a0.l | (static_cast<uint32_t>(a1.l) << 16), a2.l | (static_cast<uint32_t>(a3.l) << 16));
+            }
+            r += r_step; q4 += q_step;
+            if (q4 >= q4n) { q4 -= q4n; ++r; }
+        }
+        // tap tau of the kernel row sits at line position tau (forward) or 31 + (T - 1 - tau) (mirror); the rest is zero
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const int tau = s * TXT + tid;
+            if (tau < T) {
+                const Bf3 a = split3(wr[s]);
+                const int pos = MIRROR ? 31 + (T - 1 - tau) : tau;
+                const uint16_t pl[3] = {a.h, a.m, a.l};
+#pragma unroll
+                for (int p = 0; p < 3; ++p) {
+                    al[(2 * p) * xl + pos] = pl[p];
+                    if (pos >= 1) al[(2 * p + 1) * xl + pos - 1] = pl[p];
+                }
+            }
+        }
+        (void)c;
+    };
+    // the zero parts of the line never change: clear everything once (the taps are rewritten for every unit)
+    for (int i = tid; i < 6 * xl; i += TXT) al[i] = 0;
+    __syncthreads();
+    int unit = blockIdx.x;
+    if (unit < nunits) fetch_unit(unit);
+
+    for (; unit < nunits; unit += gridDim.x) {
+        const int c = unit / nbg, b0 = (unit - c * nbg) * MROWS;
+        store_unit(unit);
+        __syncthreads();
+        if (unit + static_cast<int>(gridDim.x) < nunits) fetch_unit(unit + gridDim.x);
+        for (int p = wv; 2 * p < nt; p += TXW) {
+#pragma unroll 1
+            for (int side = 0; side < 2; ++side) {
+                const int ot = side == 0 ? p : nt - 1 - p;
+                if (side == 1 && ot == p) break;
+                f32x16 acc, acc1;                              // two chains: consecutive MFMAs are independent
+#pragma unroll
+                for (int v = 0; v < 16; ++v) { acc[v] = MIRROR ? 0.f : eps; acc1[v] = 0.f; }
+                const int n_in = MIRROR ? nt - ot : ot + 1;
+                // A step is 16 input steps: the six products of one K block.  From one step to the next both operands move on
+                // by 16 elements: the tap window because the lag falls by 16 (forward) or grows by 16 (mirror) together with
+                // the slot base, the rows because the input step does.
+                //   forward: row t = 32 ot + ln, slot u: tap T-1-(t-u)            -> line[T-1-32 ot-ln + u]
+                //   mirror : row u = 32 ot + ln, slot t: lag 32 (it-ot) + slot-ln -> line[31-ln + 32 (it-ot) + slot]
+                const int start0 = (MIRROR ? 31 - ln : T - 1 - 32 * ot - ln) + 8 * kh;
+                const uint32_t* ap0 = reinterpret_cast<const uint32_t*>(al + (start0 & 1) * xl) + (start0 >> 1);
+                const uint16_t* bp0 = rp + ln * rs + (MIRROR ? 32 * ot : 0) + 8 * kh;
+                auto fetch = [&](int j2, bf16x8 (&fa)[3], bf16x8 (&fb)[3]) __attribute__((always_inline)) {
+#pragma unroll
+                    for (int pq = 0; pq < 3; ++pq) {
+                        const uint32_t* a4 = ap0 + 8 * j2 + pq * xl;   // a plane is 2 xl elements = xl dwords
+                        fa[pq] = __builtin_bit_cast(bf16x8, make_uint4(a4[0], a4[1], a4[2], a4[3]));
+                        fb[pq] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(bp0 + 16 * j2 + pq * MROWS * rs));
+                    }
+                };
+                auto products = [&](const bf16x8 (&fa)[3], const bf16x8 (&fb)[3]) __attribute__((always_inline)) {
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0], fb[0], acc, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0], fb[1], acc1, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1], fb[0], acc, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1], fb[1], acc1, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0], fb[2], acc, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[2], fb[0], acc1, 0, 0, 0);
+                };
+                // two register sets take turns; the step after the last one is fetched too and never used (it lies inside
+                // the workgroup's LDS: the line has 64 spare elements, the rows are followed by the line)
+                bf16x8 a[3], b[3], a2[3], b2[3];
+                fetch(0, a, b);
+                // (the fences keep the reads of the next step in front of the products of this one: left to itself the
+                // scheduler sinks them behind the products and then waits for them at once)
+                for (int j2 = 0; j2 < 2 * n_in; j2 += 2) {
+                    fetch(j2 + 1, a2, b2);
+                    __builtin_amdgcn_sched_barrier(0);
+                    products(a, b);
+                    __builtin_amdgcn_sched_barrier(0);
+                    fetch(j2 + 2, a, b);
+                    __builtin_amdgcn_sched_barrier(0);
+                    products(a2, b2);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[v] += acc1[v];
+                if (b0 + ln < B) {
+                    float* o = out + (static_cast<size_t>(b0 + ln) * C + c) * T + 32 * ot + 4 * kh;
+#pragma unroll
+                    for (int v4 = 0; v4 < 4; ++v4)
+                        *reinterpret_cast<float4*>(o + 8 * v4) = make_float4(acc[4 * v4], acc[4 * v4 + 1], acc[4 * v4 + 2], acc[4 * v4 + 3]);
+                }
+            }
+        }
+        __syncthreads();               // every wave is done with this unit's rows
+    }
+}
+
 // Kernel gradient summed over the batch: gws[c][T-1-lag] = sum_b sum_t g[b,c,t] k[b,c,t-lag], i.e. the sum of the lag-th
 // sub-diagonal of M = G^T K (contraction over the batch).  Batch rows are staged ROWS at a time; MFMA number kk contracts
 // rows 2kk and 2kk+1 (K slot = l >> 5), even and odd kk into separate accumulators so that consecutive MFMAs are
@@ -354,6 +521,7 @@ int check_tx(int B, int C, int T) {
 
 // The matrix-core path pays off once the 32 columns of a product are mostly real batch rows.
 bool use_mfma(int B, int T) { return T % 32 == 0 && T <= T_MFMA_MAX && B >= 8; }
+bool use_bf3(int B, int T) { return use_mfma(B, T) && T <= T_BF3_MAX; }
 int conv_grid(int B, int C) {
     const long long units = static_cast<long long>(C) * ((B + MROWS - 1) / MROWS);
     return static_cast<int>(units < NCU ? units : NCU);
@@ -375,7 +543,12 @@ using namespace rwkv;
 
 // gk = the mirrored convolution of gwk with w.
 int launch_gk(void* stream, const float* w, const float* gwk, float* gk, int B, int C, int T) {
-    if (use_mfma(B, T)) {
+    if (use_bf3(B, T)) {
+        const size_t lds = bf3_lds_bytes(T);
+        if (int e = raise_lds_limit(timex_conv_bf3<true>, lds)) return e;
+        hipLaunchKernelGGL(timex_conv_bf3<true>, dim3(conv_grid(B, C)), dim3(TXT), lds,
+                           static_cast<hipStream_t>(stream), w, gwk, gk, 0.0f, B, C, T);
+    } else if (use_mfma(B, T)) {
         const size_t lds = mfma_lds_bytes(T);
         if (int e = raise_lds_limit(timex_conv_mfma<true>, lds)) return e;
         hipLaunchKernelGGL(timex_conv_mfma<true>, dim3(conv_grid(B, C)), dim3(TXT), lds,
@@ -394,6 +567,13 @@ extern "C" {
 int rwkv_timex_forward(void* stream, const float* w, const float* k, float* x, float eps, int B, int C, int T) {
     if (int e = check_tx(B, C, T)) return e;
     if (int e = check_ptrs({w, k, x})) return e;
+    if (use_bf3(B, T)) {
+        const size_t lds = bf3_lds_bytes(T);
+        if (int e = raise_lds_limit(timex_conv_bf3<false>, lds)) return e;
+        hipLaunchKernelGGL(timex_conv_bf3<false>, dim3(conv_grid(B, C)), dim3(TXT), lds,
+                           static_cast<hipStream_t>(stream), w, k, x, eps, B, C, T);
+        return launch_status();
+    }
     if (use_mfma(B, T)) {
         const size_t lds = mfma_lds_bytes(T);
         if (int e = raise_lds_limit(timex_conv_mfma<false>, lds)) return e;
