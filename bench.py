@@ -60,7 +60,7 @@ TRAFFIC_MEASURED = {
     "wkv4_bwd_reg + wkv4_batch_sum B32 T768": 227.2e6 + 151.7e6,
     # profiles/timex_mfma_kernels_B32_C768_T768.md
     "timex_conv_bf3 (forward)": 77.9e6 + 75.5e6,
-    "timex backward (timex_conv_bf3 + timex_gw_sum_mfma)": (77.9e6 + 75.5e6) + (151.1e6 + 2.4e6),
+    "timex backward (timex_conv_bf3 + timex_gw_sum_bf3)": (77.9e6 + 75.5e6) + (151.1e6 + 2.4e6),
 }
 
 
@@ -423,7 +423,7 @@ def make_timex(dev):
     # T = 768, three times the ratio of the fp32 matrix peak to the HBM peak, so these kernels are bound by the former.
     conv_flops = B * C * T * (T + 1)
     kernels = [("timex_conv_bf3 (forward)", lambda: call("rwkv_timex_forward", dev, w, k, x, 0.0, B, C, T), fwd_bytes, conv_flops),
-               ("timex backward (timex_conv_bf3 + timex_gw_sum_mfma)",
+               ("timex backward (timex_conv_bf3 + timex_gw_sum_bf3)",
                 lambda: call("rwkv_timex_backward_sum", dev, w, k, g, gw, gk, B, C, T), bwd_bytes, 2 * conv_flops)]
 
     def cpu_baseline(bs=4):

@@ -242,13 +242,18 @@ __host__ __device__ inline int bf3_line_len(int T) { return T + 96; }           
 __host__ __device__ inline size_t bf3_lds_bytes(int T) {
     return (3 * static_cast<size_t>(MROWS) * bf3_row_stride(T) + 6 * static_cast<size_t>(bf3_line_len(T))) * sizeof(uint16_t);
 }
+// x = h + m + l with each term the leading eight mantissa bits of what the terms before it leave (truncation: two AND and
+// two exact subtractions; what l drops is below 2^-24 |x|)
 struct Bf3 { uint16_t h, m, l; };
 DEVINL Bf3 split3(float x) {
+    const uint32_t hb = __float_as_uint(x) & 0xffff0000u;
+    const float x1 = x - __uint_as_float(hb);
+    const uint32_t mb = __float_as_uint(x1) & 0xffff0000u;
+    const float x2 = x1 - __uint_as_float(mb);
     Bf3 r;
-    r.h = f2bf(x);
-    const float x1 = x - bf2f(r.h);
-    r.m = f2bf(x1);
-    r.l = f2bf(x1 - bf2f(r.m));
+    r.h = static_cast<uint16_t>(hb >> 16);
+    r.m = static_cast<uint16_t>(mb >> 16);
+    r.l = static_cast<uint16_t>(__float_as_uint(x2) >> 16);
     return r;
 }
 
@@ -510,6 +515,135 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_mfma(const float* __restrict
     }
 }
 
+// The same sum with three-term bf16 products (see timex_conv_bf3), 16 batch rows per pass: one v_mfma_f32_32x32x16_bf16
+// block per pair of tiles and product.  Both operands hold eight consecutive batch rows per lane, so the planes are kept
+// transposed, [step][16 rows] bf16: 32 bytes per step, and the 64 lanes of an operand read cover one contiguous KiB.
+// A finished tile's diagonals are summed in registers: lane p of a half-wave collects, for every row t it holds, the
+// element of column (t - p) mod 32 (one ds_bpermute per accumulator register), which belongs to diagonal p if t >= p and
+// to diagonal p - 32 otherwise.
+// LDS: 2 x 3 x T x 32 + 2 T x 4 bytes = 153 600 at T = 768.
+constexpr int GB3_ROWS = 16;
+__host__ __device__ inline size_t gw_bf3_lds_bytes(int T) { return 6 * static_cast<size_t>(T) * GB3_ROWS * sizeof(uint16_t) + 2 * static_cast<size_t>(T) * sizeof(float); }
+
+__global__ __launch_bounds__(TXT) void timex_gw_sum_bf3(const float* __restrict__ k, const float* __restrict__ g,
+                                                        float* __restrict__ gws, int B, int C, int T) {
+    extern __shared__ float lds[];
+    uint16_t* gp = reinterpret_cast<uint16_t*>(lds);           // [3][T][16]
+    uint16_t* kp = gp + 3 * T * GB3_ROWS;                      // [3][T][16]
+    float* diag = reinterpret_cast<float*>(kp + 3 * T * GB3_ROWS);   // [T/32 lag tiles][64]: entry l of tile d is the sum for lag 32 d + l - 31
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int ln = lane & 31, kh = lane >> 5;
+    const int nt = T >> 5, q4n = T >> 2;
+    const int plane = T * GB3_ROWS;                            // elements
+
+    // Staging: thread (row r = tid & 15, piece q = tid >> 4, + 32 per round) reads 16 bytes of its row.  The bank of a
+    // step's cell depends on the step within its group of four and on the row only, so the cells of a group are stored
+    // rotated by the group number: step 4 q + e sits in cell 4 q + ((e + q) & 3), and the lanes of a store instruction
+    // (one e, many q) spread over all banks.  A reading lane applies the same rotation to its step, once.
+    constexpr int PF = GB3_ROWS * (T_BF3_MAX / 4) / TXT;       // pieces per thread and tensor: 6
+    const int npass = (B + GB3_ROWS - 1) / GB3_ROWS;
+    const int nmine = (C > static_cast<int>(blockIdx.x) ? (C - 1 - static_cast<int>(blockIdx.x)) / static_cast<int>(gridDim.x) + 1 : 0) * npass;
+    const int r_own = tid & 15, q_own = tid >> 4;
+    float4 xg[PF], xk[PF];
+    auto fetch_unit = [&](const int u) __attribute__((always_inline)) {
+        const int c = blockIdx.x + (u / npass) * gridDim.x, b0 = (u % npass) * GB3_ROWS;
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+            const int q4 = s * 32 + q_own;
+            const bool live = q4 < q4n && b0 + r_own < B;
+            const size_t off = (static_cast<size_t>(live ? b0 + r_own : b0) * C + c) * T + (live ? 4 * q4 : 0);
+            xg[s] = *reinterpret_cast<const float4*>(g + off);
+            xk[s] = *reinterpret_cast<const float4*>(k + off);
+        }
+    };
+    auto put = [&](uint16_t* dst, const float4& x4, const int q4, const bool real) __attribute__((always_inline)) {
+        const float xs[4] = {real ? x4.x : 0.f, real ? x4.y : 0.f, real ? x4.z : 0.f, real ? x4.w : 0.f};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const Bf3 y = split3(xs[e]);
+            uint16_t* d = dst + (4 * q4 + ((e + q4) & 3)) * GB3_ROWS + r_own;
+            d[0] = y.h; d[plane] = y.m; d[2 * plane] = y.l;
+        }
+    };
+    auto store_unit = [&](const int u) __attribute__((always_inline)) {
+        const int b0 = (u % npass) * GB3_ROWS;
+        const bool real = b0 + r_own < B;
+#pragma unroll
+        for (int s = 0; s < PF; ++s) {
+            const int q4 = s * 32 + q_own;
+            if (q4 < q4n) { put(gp, xg[s], q4, real); put(kp, xk[s], q4, real); }
+        }
+    };
+    if (nmine > 0) fetch_unit(0);
+
+    for (int u = 0; u < nmine; ++u) {
+        const int pass = u % npass;
+        if (pass == 0)
+            for (int i = tid; i < 2 * T; i += TXT) diag[i] = 0.f;
+        store_unit(u);
+        __syncthreads();
+        if (u + 1 < nmine) fetch_unit(u + 1);
+        for (int p = wv; 2 * p < nt; p += TXW) {
+#pragma unroll 1
+            for (int side = 0; side < 2; ++side) {
+                const int d = side == 0 ? p : nt - 1 - p;
+                if (side == 1 && d == p) break;
+                f32x16 acc0, acc1;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.f;
+                // tile tt of g against tile tt - d of k: both move on by one tile (32 steps of 32 bytes) per iteration
+                const int cell = (ln & ~3) | (((ln & 3) + (ln >> 2)) & 3);     // where step ln of a tile sits (8 groups per tile)
+                const uint16_t* ga0 = gp + (32 * d + cell) * GB3_ROWS + 8 * kh;
+                const uint16_t* kb0 = kp + cell * GB3_ROWS + 8 * kh;
+                auto fetch = [&](int i, bf16x8 (&fa)[3], bf16x8 (&fb)[3]) __attribute__((always_inline)) {
+#pragma unroll
+                    for (int pq = 0; pq < 3; ++pq) {
+                        fa[pq] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(ga0 + i * 32 * GB3_ROWS + pq * plane));
+                        fb[pq] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(kb0 + i * 32 * GB3_ROWS + pq * plane));
+                    }
+                };
+                auto products = [&](const bf16x8 (&fa)[3], const bf16x8 (&fb)[3]) __attribute__((always_inline)) {
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0], fb[0], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0], fb[1], acc1, 0, 0, 0);
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1], fb[0], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1], fb[1], acc1, 0, 0, 0);
+                    acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0], fb[2], acc0, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[2], fb[0], acc1, 0, 0, 0);
+                };
+                const int n = nt - d;                          // tile pairs of this lag tile
+                // one register set: the other wave of the SIMD runs its products while this one waits for its operands (a
+                // second set, with the next unit's rows held across this loop, does not fit in 256 registers)
+                for (int i = 0; i < n; ++i) {
+                    bf16x8 a[3], b[3];
+                    fetch(i, a, b);
+                    products(a, b);
+                }
+                // accumulator v: t = 8 (v/4) + 4 kh + (v&3), u = ln, of tiles d apart
+                float pos = 0.f, neg = 0.f;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int t = 8 * (v >> 2) + 4 * kh + (v & 3);
+                    const float y = __shfl(acc0[v] + acc1[v], (kh << 5) | ((t - ln) & 31), 64);
+                    if (t >= ln) pos += y; else neg += y;
+                }
+                pos += __shfl_xor(pos, 32, 64);
+                neg += __shfl_xor(neg, 32, 64);
+                if (kh == 0) diag[64 * d + 31 + ln] += pos;    // lag tile d belongs to this wave alone
+                else if (ln >= 1) diag[64 * d + ln - 1] += neg;
+            }
+        }
+        __syncthreads();
+        if (pass == npass - 1) {
+            const int c = blockIdx.x + (u / npass) * gridDim.x;
+            for (int x = tid; x < T; x += TXT) {        // lag = 32 d + e comes from tile d (diagonal e) and tile d + 1 (diagonal e - 32)
+                const int lag = T - 1 - x, d = lag >> 5, e = lag & 31;
+                gws[static_cast<size_t>(c) * T + x] = diag[64 * d + 31 + e] + (d + 1 < nt ? diag[64 * (d + 1) + e - 1] : 0.f);
+            }
+            __syncthreads();           // diag is cleared for the next channel only after it has been read
+        }
+    }
+}
+
 constexpr int T_MAX = 4096;
 
 int check_tx(int B, int C, int T) {
@@ -604,11 +738,17 @@ int rwkv_timex_backward_sum(void* stream, const float* w, const float* k, const 
     if (int e = check_tx(B, C, T)) return e;
     if (T % 32 != 0 || T > T_MFMA_MAX) return RWKV_ERR_SHAPE;
     if (int e = check_ptrs({w, k, gwk, gw_sum, gk})) return e;
+    if (int e = launch_gk(stream, w, gwk, gk, B, C, T)) return e;
+    if (use_bf3(B, T)) {
+        const size_t lds_gw = gw_bf3_lds_bytes(T);
+        if (int e = raise_lds_limit(timex_gw_sum_bf3, lds_gw)) return e;
+        hipLaunchKernelGGL(timex_gw_sum_bf3, dim3(C < NCU ? C : NCU), dim3(TXT), lds_gw, static_cast<hipStream_t>(stream), k, gwk, gw_sum, B, C, T);
+        return launch_status();
+    }
     const bool wide = T <= T_GW_WIDE;
     const size_t lds_gw = gw_lds_floats(T, wide ? 16 : 8) * sizeof(float);
     auto kernel = wide ? timex_gw_sum_mfma<16> : timex_gw_sum_mfma<8>;
     if (int e = raise_lds_limit(kernel, lds_gw)) return e;
-    if (int e = launch_gk(stream, w, gwk, gk, B, C, T)) return e;
     hipLaunchKernelGGL(kernel, dim3(C < NCU ? C : NCU), dim3(TXT), lds_gw, static_cast<hipStream_t>(stream), k, gwk, gw_sum, B, C, T);
     return launch_status();
 }
