@@ -26,6 +26,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
+# depthwise_conv1d up to T = 768 forms every fp32 product from six bf16 matrix products (three bf16 terms per operand):
+# its ceiling in algorithmic (fp32) flops is a sixth of the bf16 rate
+BF3_PRODUCTS = 6
 PREWARM_S = 0.3                # seconds of untimed load before the warmup steps (clock ramp)
 ALGO = "chunked"
 FLAGS = 0                      # RWKV_FLAG_SWEEPS when --algo sweeps: passed per call to the *_ex entry points
@@ -58,9 +62,9 @@ TRAFFIC_MEASURED = {
     # profiles/wkv4_reg_kernels_B32_T768_C768.md
     "wkv4_fwd_reg B32 T768": 152.5e6 + 78.4e6,
     "wkv4_bwd_reg + wkv4_batch_sum B32 T768": 227.2e6 + 151.7e6,
-    # profiles/timex_mfma_kernels_B32_C768_T768.md
-    "timex_conv_bf3 (forward)": 77.9e6 + 75.5e6,
-    "timex backward (timex_conv_bf3 + timex_gw_sum_bf3)": (77.9e6 + 75.5e6) + (151.1e6 + 2.4e6),
+    # profiles/timex_bf3_kernels_B32_C768_T768.md
+    "timex_conv_bf3 (forward)": 78.0e6 + 75.5e6,
+    "timex backward (timex_conv_bf3 + timex_gw_sum_bf3)": (78.0e6 + 75.5e6) + (151.2e6 + 2.4e6),
 }
 
 
@@ -452,7 +456,7 @@ WORKLOADS = {
     "wkv4_b32": lambda dev: make_wkv4(dev, B=32, T=768),
     "timex": make_timex,
 }
-DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_n128": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "wkv4_b32": "f32", "timex": "f32"}
+DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_n128": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "wkv4_b32": "f32", "timex": "bf16x3 (every fp32 operand as three bf16 terms, fp32 accumulation)"}
 
 
 def main():
@@ -528,7 +532,7 @@ def main():
         ms = time_gpu(fn, max(5, args.steps), 2)
         per_kernel.append({"kernel": label, "ms": round(ms, 4), "algorithmic_bytes": nbytes,
                            "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)})
-        if flops:                                # a kernel bound by the fp32 matrix cores, not by HBM
+        if flops:                                # a kernel bound by the matrix cores, not by HBM
             per_kernel[-1].update(algorithmic_flops=flops[0], TFLOPs=round(flops[0] / (ms * 1e-3) / 1e12, 2))
     dom = max(per_kernel, key=lambda d: d["ms"])
     traffic = TRAFFIC_MEASURED.get(dom["kernel"]) if ALGO == "chunked" else None
@@ -541,8 +545,11 @@ def main():
                 "hbm_copy_GBps": round(copy_gbps, 1), "frac_of_copy": round(dom["GBps"] / copy_gbps, 4),
                 "whole_step_frac_of_copy": round(step_gbps / copy_gbps, 4)}
     if "TFLOPs" in dom:
-        roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["TFLOPs"], "peak": FP32_MFMA_PEAK_TFLOPS,
-                    "unit": "TFLOP/s", "frac": round(dom["TFLOPs"] / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": traffic,
+        peak = BF16_MFMA_PEAK_TFLOPS / BF3_PRODUCTS
+        roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["TFLOPs"], "peak": round(peak, 1),
+                    "peak_is": "bf16 dense 2500 TFLOP/s / 6 bf16 products per fp32 product",
+                    "unit": "TFLOP/s", "frac": round(dom["TFLOPs"] / peak, 4),
+                    "frac_of_fp32_matrix_peak": round(dom["TFLOPs"] / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": traffic,
                     "traffic_over_algorithmic": round(traffic / dom["algorithmic_bytes"], 3) if traffic else None,
                     "launch_ms": dom["ms"], "algorithmic_flops": dom["algorithmic_flops"],
                     "hbm_frac": round(dom["GBps"] / HBM_PEAK_GBS, 4), "hbm_copy_GBps": round(copy_gbps, 1)}
