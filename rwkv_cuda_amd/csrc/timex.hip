@@ -238,7 +238,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 constexpr int T_BF3_MAX = 768;
 constexpr int PFQ3 = MROWS * (T_BF3_MAX / 4) / TXT;
 __host__ __device__ inline int bf3_row_stride(int T) { return T + 16; }          // elements; (T + 16) / 2 dwords = 8 or 24 mod 32
-__host__ __device__ inline int bf3_line_len(int T) { return T + 96; }           // (T + 96) / 2 dwords = 16 mod 32: the shifted copy sits 16 banks away
+__host__ __device__ inline int bf3_line_len(int T) { return T + ((T & 32) ? 64 : 96); }   // half of it = 16 mod 32 dwords: the shifted copy sits 16 banks away
 __host__ __device__ inline size_t bf3_lds_bytes(int T) {
     return (3 * static_cast<size_t>(MROWS) * bf3_row_stride(T) + 6 * static_cast<size_t>(bf3_line_len(T))) * sizeof(uint16_t);
 }
@@ -364,7 +364,7 @@ __global__ __launch_bounds__(TXT) void timex_conv_bf3(const float* __restrict__ 
                     acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[2], fb[0], acc1, 0, 0, 0);
                 };
                 // two register sets take turns; the step after the last one is fetched too and never used (it lies inside
-                // the workgroup's LDS: the line has 64 spare elements, the rows are followed by the line)
+                // the workgroup's LDS: the line has at least 64 spare elements, the rows are followed by the line)
                 bf16x8 a[3], b[3], a2[3], b2[3];
                 fetch(0, a, b);
                 // (the fences keep the reads of the next step in front of the products of this one: left to itself the
