@@ -524,6 +524,12 @@ def main():
     dst = torch.empty_like(src)
     copy_ms = time_gpu(lambda: dst.copy_(src), 10, 3)
     copy_gbps = 2 * src.numel() * 4 / (copy_ms * 1e-3) / 1e9
+    # the same 1 GiB as a read-only stream (a sum reduction: 1 GiB in, a few KB out) and as a write-only stream (a fill):
+    # a kernel that mostly reads is priced against the first, one that mostly writes against the second
+    read_ms = time_gpu(lambda: torch.sum(src), 10, 3)
+    write_ms = time_gpu(lambda: dst.fill_(1.0), 10, 3)
+    read_gbps = src.numel() * 4 / (read_ms * 1e-3) / 1e9
+    write_gbps = src.numel() * 4 / (write_ms * 1e-3) / 1e9
     del src, dst
 
     # per-kernel timing, HIP events on the launch stream
@@ -543,7 +549,8 @@ def main():
                 "launch_ms": dom["ms"], "algorithmic_bytes": dom["algorithmic_bytes"],
                 "whole_step_frac": round(step_gbps / HBM_PEAK_GBS, 4),
                 "hbm_copy_GBps": round(copy_gbps, 1), "frac_of_copy": round(dom["GBps"] / copy_gbps, 4),
-                "whole_step_frac_of_copy": round(step_gbps / copy_gbps, 4)}
+                "whole_step_frac_of_copy": round(step_gbps / copy_gbps, 4),
+                "hbm_read_GBps": round(read_gbps, 1), "hbm_write_GBps": round(write_gbps, 1)}
     if "TFLOPs" in dom:
         peak = BF16_MFMA_PEAK_TFLOPS / BF3_PRODUCTS
         roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["TFLOPs"], "peak": round(peak, 1),

@@ -276,6 +276,28 @@ int rwkv_wkv6f_backward(void* stream, int B, int T, int C, int H,
                         rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
                         rwkv_bf16* gs, void* workspace, size_t workspace_bytes, unsigned flags);
 
+/* WKV_6 (s = gs = NULL) and WKV_6STATE with states handed from the forward to the backward.  The forward also writes,
+ * into `saved` (rwkv_wkv6f_saved_bytes; fp32 [B*H][ceil(T/64)][64][64]), the state entering every 64th token; the backward
+ * reads them and produces every gradient in ONE reverse sweep instead of two sweeps and an fp32 [B,T,C] hand-over.  The
+ * reference's wkv6 operators keep nothing between their two calls; the precedents are its rwkv7 forward, which keeps `s`
+ * and `sa` for its backward (rwkv7_statepassing_clampw.cu:67-73), and wkv5_bf16/cuda/wkv5_cuda_v3.cu:12-30 (chunk states).
+ * Results are those of the pair above to the rounding of the outputs.  With another head size than 64, or with
+ * RWKV_FLAG_SWEEPS / RWKV_PASS_*, rwkv_wkv6f_saved_bytes is 0 for sizes the kernels do not take, `saved` may be NULL and
+ * both calls run the kernels above.  The workspace also serves the two-sweep kernels, which redo any (batch, head) whose
+ * decay over 16 tokens exceeds e^-60. */
+size_t rwkv_wkv6f_saved_bytes(int B, int T, int C, int H);
+int rwkv_wkv6f_forward(void* stream, int B, int T, int C, int H,
+                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                       const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, rwkv_bf16* y,
+                       void* saved, size_t saved_bytes, unsigned flags);
+size_t rwkv_wkv6f_backward_saved_workspace_bytes(int B, int T, int C, int H);
+int rwkv_wkv6f_backward_saved(void* stream, int B, int T, int C, int H,
+                              const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                              const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, const rwkv_bf16* gy,
+                              rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                              rwkv_bf16* gs, const void* saved, size_t saved_bytes,
+                              void* workspace, size_t workspace_bytes, unsigned flags);
+
 /* ---------------------------------------------------------------------------------------
  * RWKV-6 wkv with initial state.  Replaces cuda_forward / cuda_backward of
  * wkv6_state/cuda/wkv6state_op.cpp:5-6 (kernels: wkv6state_cuda_v1a.cu:6-308).

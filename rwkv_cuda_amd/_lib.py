@@ -18,10 +18,10 @@ _INCLUDE = os.path.join(_ROOT, "include")
 LIB_PATH = os.path.join(_HERE, "librwkv_hip.so")
 HASH_PATH = LIB_PATH + ".srchash"        # digest of the sources the library was built from (content, not mtime)
 
-SOURCES = ["abi.hip", "wkv56.hip", "wkv6_fwd.hip", "wkv6_bwd_a.hip", "wkv6_bwd_b.hip", "wkv4.hip", "timex.hip", "rwkv7.hip", "rwkv7_chunk.hip"]
+SOURCES = ["abi.hip", "wkv56.hip", "wkv6_fwd.hip", "wkv6_bwd_a.hip", "wkv6_bwd_b.hip", "wkv6_bwd_f.hip", "wkv4.hip", "timex.hip", "rwkv7.hip", "rwkv7_chunk.hip"]
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed fp32 VALU ops stay off on this target
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
@@ -53,19 +53,38 @@ def source_hash():
     return h.hexdigest()
 
 
+def _compile_one(args):
+    hipcc, src, obj = args
+    cmd = [hipcc] + HIPCC_FLAGS + ["-c", "-I", _INCLUDE, "-I", _CSRC, "-o", obj, src]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    return " ".join(cmd), res.returncode, res.stdout
+
+
 def build(verbose=False):
-    """Compile every HIP source into one shared library, in-tree."""
+    """Compile every HIP source (one hipcc process per file, side by side) and link them into one shared library, in-tree."""
+    from concurrent.futures import ThreadPoolExecutor
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    srcs = [os.path.join(_CSRC, s) for s in SOURCES if os.path.exists(os.path.join(_CSRC, s))]
-    cmd = [hipcc] + HIPCC_FLAGS + ["-I", _INCLUDE, "-I", _CSRC, "-o", LIB_PATH] + srcs
+    objdir = os.path.join(_HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    jobs = [(hipcc, os.path.join(_CSRC, s), os.path.join(objdir, s + ".o")) for s in SOURCES]
+    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
+        results = list(pool.map(_compile_one, jobs))
+    lines = []
+    for cmd, rc, text in results:
+        if verbose:
+            print(cmd, flush=True)
+        if rc != 0:
+            raise RuntimeError("hipcc failed:\n" + "\n".join(l for l in text.splitlines() if "is not a recognized feature" not in l and "kernel-resource-usage" not in l))
+        lines += text.splitlines()
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + [j[2] for j in jobs]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    lines = res.stdout.splitlines()
-    out = "\n".join(l for l in lines if "is not a recognized feature" not in l and "kernel-resource-usage" not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
+        raise RuntimeError("link failed:\n" + res.stdout)
+    out = "\n".join(l for l in lines if "is not a recognized feature" not in l and "kernel-resource-usage" not in l)
     kernel = None
+    report = []
     for l in lines:
         m = re.search(r"remark: Function Name: (\S+)", l)
         if m:
@@ -118,6 +137,10 @@ SIGNATURES = {
     "rwkv_wkv5raw_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 11 + [_P, _Z, _U]),
     "rwkv_wkv6f_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv6f_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, _Z, _U]),
+    "rwkv_wkv6f_saved_bytes": (_Z, [_I, _I, _I, _I]),
+    "rwkv_wkv6f_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 7 + [_P, _Z, _U]),
+    "rwkv_wkv6f_backward_saved_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "rwkv_wkv6f_backward_saved": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, _Z, _P, _Z, _U]),
     "rwkv_wkv5f32_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
     "rwkv_wkv5f32_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12),
     "rwkv_wkv5f32_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_U]),

@@ -21,6 +21,6 @@ const char* rwkv_strerror(int status) {
 
 int rwkv_last_hip_error(void) { return rwkv::g_last_hip_error; }
 
-int rwkv_abi_version(void) { return 2; }
+int rwkv_abi_version(void) { return 3; }
 
 }  // extern "C"

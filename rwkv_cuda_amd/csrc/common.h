@@ -137,14 +137,20 @@ inline int launch_status() {
 // wkv6_chunk.hip: chunked MFMA kernels.  wmode: 1 = fp32 ew [B,T,C], 2 = raw bf16 w.
 int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                           const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
-                          const uint16_t* s0, uint16_t* y);
+                          const uint16_t* s0, uint16_t* y, float* saved = nullptr);
 int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                             const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
-                            const uint16_t* s0, const uint16_t* gy, uint16_t* gr, uint16_t* gu, float* rdr);
+                            const uint16_t* s0, const uint16_t* gy, uint16_t* gr, uint16_t* gu, float* rdr,
+                            const int* only_flagged = nullptr);
 int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                             const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
                             const uint16_t* s0, const uint16_t* gy, uint16_t* gk, uint16_t* gv, uint16_t* gw,
-                            uint16_t* gs, const float* rdr);
+                            uint16_t* gs, const float* rdr, const int* only_flagged = nullptr);
+// wkv6_bwd_f.hip: the whole backward in one reverse sweep from the states the forward saved (raw bf16 decay);
+// flags [B*H][4] names the (batch, head) pairs that have to be redone by the two sweeps above
+int launch_wkv6_bwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
+                          const uint16_t* w, const uint16_t* u, const uint16_t* gy, uint16_t* gr, uint16_t* gk, uint16_t* gv,
+                          uint16_t* gw, uint16_t* gu, uint16_t* gs, const float* saved, int* flags);
 // wkv5 with heads of 128 channels as four heads of 64 (see ArgsB in wkv6_chunk.h): one launch of each kernel per value
 // of `cross`.  Forward and first sweep: the first launch (cross = 0) leaves fp32 terms, the second adds them to its own
 // and writes the bf16 outputs.  Second sweep: both launches leave fp32 terms (its waves have no registers to spare for

@@ -323,26 +323,17 @@ __global__ __launch_bounds__(NT, 2) void rwkv7c_fwd(const Args7c p) {
 }
 
 // ---------------------------------------------------------------------------------------------------- backward
-// One workgroup of eight waves per (batch, head), two roles; wave w: q = w & 3.
+// One workgroup of twelve waves per (batch, head), three roles with their own loops; wave w: q = w & 3.
 //   waves 0..3 ("A", value-channel tile q): dSa[jt][v] = dS[i = 16 q + l16][j = 16 jt + 4 g + v]   (rows j, columns i): the B operand
 //                of the contractions over the key channel, (B' d2) dS^T and (K' d2) dS^T; they make the causal tiles, dU, the
 //                triangular solve, dW, dV and ds0.
 //   waves 4..7 ("B", key-channel tile q):   dSb[ib][v] = dS[i = 16 ib + 4 g + v][j = 16 q + l16]   (rows i, columns j): the B operand
 //                of the contractions over the value channel, U dS and V dS, next to S0 of the chunk loaded from `s` in the same
 //                layout (dW S0, dY S0); they make dA', dR', dB', dK' (register v <-> token 4 g + v, lane <-> key channel), scale
-//                them, scan the decay gradient and park the results.
+//                them, scan the decay gradient and park the results; they run one phase behind the A waves.
+//   waves 8..11 ("P"): fetch the next chunk's seven input rows and `sa`, convert them, build the operand planes
+//                (double-buffered) and store the finished gradient rows (LDS-staged, whole rows).
 // The gradient state is therefore kept twice (both copies get the same update); nothing is transposed through LDS.
-// All eight waves share the elementwise preparation (lane = channel, tokens 2 w and 2 w + 1) and the row-wise output stores.
-#ifdef RWKV7_TIMING
-__device__ unsigned long long g_dbg[12][8];
-#define STAMP(k) do { const unsigned long long now_ = __builtin_readcyclecounter(); tacc[k] += now_ - tlast; tlast = now_; } while (0)
-#define STAMP_INIT unsigned long long tacc[8] = {0, 0, 0, 0, 0, 0, 0, 0}; unsigned long long tlast = __builtin_readcyclecounter()
-#define STAMP_DUMP(w) do { if ((tid & 63) == 0 && blockIdx.x == 0 && blockIdx.y == 0) for (int k_ = 0; k_ < 8; ++k_) g_dbg[w][k_] = tacc[k_]; } while (0)
-#else
-#define STAMP(k)
-#define STAMP_INIT
-#define STAMP_DUMP(w)
-#endif
 constexpr int NTB = 12 * 64;       // waves 0..3 role A, 4..7 role B, 8..11 role P
 
 // Everything that is a function of one chunk's inputs alone; two copies: the P waves fill one while the A and B waves work on the other.
@@ -468,24 +459,18 @@ DEVINL void bwd_role_p(SmemCB& S, const Args7c& p, int tid, int w, size_t tok0, 
     __syncthreads();
     bwd_planes(S.pl[0], y, wp, lane);
     __syncthreads();
-    STAMP_INIT;
     for (int i = 0; i < nch; ++i) {                  // visit i is chunk nch - 1 - i
         const bool next = i + 1 < nch;
         if (next) {
             bwd_convert(S.pl[(i + 1) & 1], x, y, wp, lane);
             if (i + 2 < nch) bwd_fetch(p, x, tok0 + static_cast<size_t>(nch - 3 - i) * CL, wp, lane, H, h);
         }
-        STAMP(0);
         __syncthreads();
-        STAMP(1);
         if (i > 0) bwd_store_rows(S, (i - 1) & 1, p, tok0 + static_cast<size_t>(nch - i) * CL, tp, H, h);
         if (next) bwd_planes(S.pl[(i + 1) & 1], y, wp, lane);
-        STAMP(2);
         __syncthreads();
         __syncthreads();
-        STAMP(3);
     }
-    STAMP_DUMP(w);
     __syncthreads();                                 // role B finishes the last chunk
     bwd_store_rows(S, (nch - 1) & 1, p, tok0, tp, H, h);
 }
@@ -499,7 +484,6 @@ DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
         dS[jt] = p.dsT != nullptr ? ld4(p.dsT + bh * N * N + static_cast<size_t>(own) * N + 16 * jt + 4 * g) : ZERO4;
     __syncthreads();
     __syncthreads();
-    STAMP_INIT;
     for (int i = 0; i < nch; ++i) {
         const PlanesB& O = S.pl[i & 1];
         // ---------------------------------------------------------------- phase 1: the parts of dU, dV, dS that need no tile; a causal tile; M
@@ -528,9 +512,7 @@ DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
                 for (int t = 0; t < CL; ++t) S.M[t][l16] = m[t];
         }
         f32x4 dU = dUp[0] + dUp[1], dV = dVp[0] + dVp[1];
-        STAMP(0);
         __syncthreads();
-        STAMP(1);
         // ---------------------------------------------------------------- phase 2: dU, dW = M^T dU, dV, the gradient state
         {
 #pragma unroll
@@ -554,16 +536,11 @@ DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
                 dS[jt] = dS[jt] * ld4(&O.dec[16 * jt + 4 * g]) + acc;
             }
         }
-        STAMP(2);
         __syncthreads();
-        STAMP(3);
         // ---------------------------------------------------------------- phase 3: dAB, dAK (they need dW)
         if (q < 2) causal_tile(S.dW, q == 0 ? O.U : O.V, q == 0 ? S.dAB : S.dAK, true, l16, g);
-        STAMP(4);
         __syncthreads();
-        STAMP(5);
     }
-    STAMP_DUMP(w);
     __syncthreads();
     if (p.ds0 != nullptr) {
         float* dst = p.ds0 + bh * N * N + static_cast<size_t>(own) * N + 4 * g;
@@ -641,15 +618,12 @@ DEVINL void bwd_role_b(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
     fetch_state(nch - 1);
     __syncthreads();
     __syncthreads();
-    STAMP_INIT;
     for (int i = 0; i < nch; ++i) {
         const int c = nch - 1 - i;
         const PlanesB& O = S.pl[i & 1];
         // ---------------------------------------------------------------- phase 1: finish the previous visit's chunk
         if (i > 0) finish(S.pl[(i - 1) & 1]);
-        STAMP(0);
         __syncthreads();
-        STAMP(1);
         // ---------------------------------------------------------------- phase 2: dY S0, U dS, V dS; dRB, dRK
         if (i == 0 && p.dsT != nullptr) {
             // P at the end of the call: sum_i dsT o S_T with S_T = S0 dec + U^T (B' d2) + V^T (K' d2) of the last chunk
@@ -684,9 +658,7 @@ DEVINL void bwd_role_b(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
             xR = pr[0] + pr[1]; xB = pb[0] + pb[1]; xK = pk[0] + pk[1];
         }
         if (q >= 2) causal_tile(O.dY, q == 2 ? O.U : O.V, q == 2 ? S.dRB : S.dRK, false, l16, g);
-        STAMP(2);
         __syncthreads();
-        STAMP(3);
         // ---------------------------------------------------------------- phase 3: dW S0; the gradient state
         {
             const float decj = O.dec[own];
@@ -709,11 +681,8 @@ DEVINL void bwd_role_b(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
             xA = pa[0] + pa[1];
             if (c > 0) fetch_state(c - 1);
         }
-        STAMP(4);
         __syncthreads();
-        STAMP(5);
     }
-    STAMP_DUMP(w);
     finish(S.pl[(nch - 1) & 1]);
     __syncthreads();
 }
@@ -733,9 +702,6 @@ __global__ __launch_bounds__(NTB, 3) void rwkv7c_bwd(const Args7c p) {
 
 }  // namespace
 
-#ifdef RWKV7_TIMING
-extern "C" int rwkv7_dbg_read(unsigned long long* out) { return static_cast<int>(hipMemcpyFromSymbol(out, HIP_SYMBOL(g_dbg), sizeof(g_dbg))); }
-#endif
 
 int launch7c_fwd(hipStream_t st, int B, int T, int H, const float* s0, const uint16_t* r, const uint16_t* w, const uint16_t* k,
                  const uint16_t* v, const uint16_t* a, const uint16_t* b, uint16_t* y, float* sT, float* s, float* sa) {

@@ -1230,6 +1230,67 @@ int rwkv_wkv6f_backward(void* stream, int B, int T, int C, int H, const rwkv_bf1
     return launch_status();
 }
 
+// ---- WKV_6 / WKV_6STATE with states handed from the forward to the backward: the forward keeps the state entering
+//      every second chunk, and the backward is one reverse sweep (wkv6_bwd_f.hip).  Head size 64 and the chunked
+//      kernels only; otherwise `saved` has no bytes and both calls are the ones above.
+bool fused_ok(int T, int C, int H, unsigned flags) {
+    return C == H * N && !(flags & (RWKV_FLAG_SWEEPS | RWKV_PASS_ALL)) && static_cast<long long>(T) * C < (1LL << 30);
+}
+
+size_t rwkv_wkv6f_saved_bytes(int B, int T, int C, int H) {
+    if (check_dims(B, T, C, H) != RWKV_OK || C != H * N || static_cast<long long>(T) * C >= (1LL << 30)) return 0;
+    const size_t nchunks = (static_cast<size_t>(T) + 31) / 32, nseg = (nchunks + 1) / 2;
+    return static_cast<size_t>(B) * H * nseg * 64 * 64 * sizeof(float);
+}
+
+int rwkv_wkv6f_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                       const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, rwkv_bf16* y, void* saved, size_t saved_bytes,
+                       unsigned flags) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, w, u, y}, C == H * N)) return e;
+    if (s != nullptr && C == H * N && !aligned16(s)) return RWKV_ERR_ALIGN;
+    if (!fused_ok(T, C, H, flags) || saved == nullptr) {
+        Args a{};
+        a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s; a.y = y;
+        return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, flags);
+    }
+    if (saved_bytes < rwkv_wkv6f_saved_bytes(B, T, C, H) || !aligned16(saved)) return RWKV_ERR_WORKSPACE;
+    return launch_wkv6_fwd_chunk(static_cast<hipStream_t>(stream), W_RAW, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved));
+}
+
+size_t rwkv_wkv6f_backward_saved_workspace_bytes(int B, int T, int C, int H) {
+    const size_t n = rwkv_wkv6f_backward_workspace_bytes(B, T, C, H);
+    return n == 0 ? 0 : round16(n) + round16(static_cast<size_t>(B) * H * 4 * sizeof(int));
+}
+
+int rwkv_wkv6f_backward_saved(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                              const rwkv_bf16* w, const rwkv_bf16* u, const rwkv_bf16* s, const rwkv_bf16* gy, rwkv_bf16* gr,
+                              rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu, rwkv_bf16* gs, const void* saved,
+                              size_t saved_bytes, void* workspace, size_t workspace_bytes, unsigned flags) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (workspace == nullptr || workspace_bytes < rwkv_wkv6f_backward_saved_workspace_bytes(B, T, C, H) || !aligned16(workspace))
+        return RWKV_ERR_WORKSPACE;
+    if (!fused_ok(T, C, H, flags) || saved == nullptr)
+        return rwkv_wkv6f_backward(stream, B, T, C, H, r, k, v, w, u, s, gy, gr, gk, gv, gw, gu, gs, workspace, workspace_bytes, flags);
+    if (int e = check_ptrs({r, k, v, w, u, gy, gr, gk, gv, gw, gu})) return e;
+    if ((s == nullptr) != (gs == nullptr)) return RWKV_ERR_NULL;
+    if (s != nullptr && (!aligned16(s) || !aligned16(gs))) return RWKV_ERR_ALIGN;
+    if (saved_bytes < rwkv_wkv6f_saved_bytes(B, T, C, H) || !aligned16(saved)) return RWKV_ERR_WORKSPACE;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t n = round16(ws_bytes(B, T, C, H));
+    char* wsb = static_cast<char*>(workspace);
+    float* rdr = static_cast<float*>(workspace);
+    uint16_t* pu = reinterpret_cast<uint16_t*>(wsb + n);                                  // per-batch gu
+    int* flg = reinterpret_cast<int*>(wsb + round16(rwkv_wkv6f_backward_workspace_bytes(B, T, C, H)));
+    if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, pu, gs, static_cast<const float*>(saved), flg)) return e;
+    // (batch, head) pairs with a decay the mid-point factors cannot carry: the two sweeps redo them, all others return at once
+    if (int e = launch_wkv6_bwd_a_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, gy, gr, pu, rdr, flg)) return e;
+    if (int e = launch_wkv6_bwd_b_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, gy, gk, gv, gw, gs, rdr, flg)) return e;
+    hipLaunchKernelGGL(bf16_batch_sum, dim3((C + 255) / 256), dim3(256), 0, st, B, C, pu, gu,
+                       static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(nullptr));
+    return launch_status();
+}
+
 // ---- the reference-signature entry points: default kernels, every pass
 int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                       const rwkv_bf16* v, const float* eew, const rwkv_bf16* u, rwkv_bf16* y) {

@@ -475,6 +475,7 @@ DEVINL void bwa_state(SmemA2& S, const ArgsB& a, const int tid, const size_t bas
 template <int WMODE, int SPLIT = 0>
 __global__ __launch_bounds__(NTA) void wkv6_bwd_a_ws(const ArgsB a) {
     __shared__ SmemA2 S;
+    if (skip_unflagged(a.only_flagged, blockIdx.x)) return;
     const int tid = threadIdx.x;
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
     const int hk = SPLIT != 0 ? h ^ a.cross : h;       // the block of 64 channels that r, k, w, u come from and gr, gu go to
@@ -501,10 +502,11 @@ __global__ __launch_bounds__(NTA) void wkv6_bwd_a_ws(const ArgsB a) {
 
 int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                             const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
-                            const uint16_t* s0, const uint16_t* gy, uint16_t* gr, uint16_t* gu, float* rdr) {
+                            const uint16_t* s0, const uint16_t* gy, uint16_t* gr, uint16_t* gu, float* rdr,
+                            const int* only_flagged) {
     ArgsB a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.gy = gy;
-    a.gr = gr; a.gu = gu; a.rdr = rdr;
+    a.gr = gr; a.gu = gu; a.rdr = rdr; a.only_flagged = only_flagged;
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_bwd_a_ws<W_RAW>, dim3(B * H), dim3(NTA), 0, st, a);
     else if (wmode == W_EW) hipLaunchKernelGGL(wkv6_bwd_a_ws<W_EW>, dim3(B * H), dim3(NTA), 0, st, a);
     else hipLaunchKernelGGL(wkv6_bwd_a_ws<W_HEAD>, dim3(B * H), dim3(NTA), 0, st, a);

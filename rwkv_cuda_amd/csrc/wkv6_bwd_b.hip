@@ -661,6 +661,7 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
 template <int WMODE, bool SPLIT = false>
 __global__ __launch_bounds__(NTB) void wkv6_bwd_b_ws(const ArgsB a) {
     __shared__ SmemB2 S;
+    if (skip_unflagged(a.only_flagged, blockIdx.x)) return;
     const int tid = threadIdx.x;
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
     const int hk = SPLIT ? h ^ a.cross : h;            // the block of 64 channels that r, k, w, u come from and gk, gw go to
@@ -688,10 +689,10 @@ __global__ __launch_bounds__(NTB) void wkv6_bwd_b_ws(const ArgsB a) {
 int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                             const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
                             const uint16_t* s0, const uint16_t* gy, uint16_t* gk, uint16_t* gv, uint16_t* gw,
-                            uint16_t* gs, const float* rdr) {
+                            uint16_t* gs, const float* rdr, const int* only_flagged) {
     ArgsB a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.gy = gy;
-    a.gk = gk; a.gv = gv; a.gw = gw; a.gs = gs; a.rdr = const_cast<float*>(rdr);
+    a.gk = gk; a.gv = gv; a.gw = gw; a.gs = gs; a.rdr = const_cast<float*>(rdr); a.only_flagged = only_flagged;
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_bwd_b_ws<W_RAW>, dim3(B * H), dim3(NTB), 0, st, a);
     else if (wmode == W_EW) hipLaunchKernelGGL(wkv6_bwd_b_ws<W_EW>, dim3(B * H), dim3(NTB), 0, st, a);
     else hipLaunchKernelGGL(wkv6_bwd_b_ws<W_HEAD>, dim3(B * H), dim3(NTB), 0, st, a);

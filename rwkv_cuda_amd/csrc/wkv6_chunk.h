@@ -61,6 +61,9 @@ struct ArgsC {
     // SPLIT kernels only (see below)
     int cross;
     float* y32;
+    // when not null: [B*H][ceil(chunks / 2)][64][64] fp32, the state entering every even chunk, [value][key], for the
+    // one-sweep backward (wkv6_bwd_f.hip)
+    float* saved;
 };
 
 struct ArgsB {
@@ -72,7 +75,15 @@ struct ArgsB {
     // SPLIT kernels only (see below)
     int cross;
     float *gr32, *gk32, *gv32, *gw32, *gu32;
+    // when not null: [B*H][4]; a workgroup runs only if one of its four words is not zero (the (batch, head) pairs that
+    // the one-sweep backward has handed back)
+    const int* only_flagged;
 };
+DEVINL bool skip_unflagged(const int* f, const int bh) {
+    if (f == nullptr) return false;
+    const int4 x = *reinterpret_cast<const int4*>(f + 4 * bh);
+    return (x.x | x.y | x.z | x.w) == 0;
+}
 
 // A head of 128 channels as four heads of 64 (SPLIT = true, wkv5 only).  With the key channels j and the value channels
 // i of the head cut into halves J and I, everything the op computes is a sum over blocks of the state S[i in I][j in J]:

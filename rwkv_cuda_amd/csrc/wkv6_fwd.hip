@@ -390,6 +390,13 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
         const bool exact = __builtin_amdgcn_readfirstlane(O.exact) != 0;
         if (i > 0) finish(i - 1, exact_prev);
         fetch_term(i);                                 // used by finish(i), one iteration from here
+        if constexpr (SPLIT == 0) {
+            if (a.saved != nullptr && !(i & 1)) {      // the state entering every even chunk, for the one-sweep backward
+                float* dst = a.saved + ((bh * ((nchunks + 1) / 2) + (i >> 1)) * N + i_own) * N + j0[0];
+                *reinterpret_cast<float4*>(dst) = make_float4(D[0][0], D[0][1], D[0][2], D[0][3]);
+                *reinterpret_cast<float4*>(dst + 4) = make_float4(D[1][0], D[1][1], D[1][2], D[1][3]);
+            }
+        }
         if (!exact) {
             // ------------------------------------------------------------ y^T = (d1 S) R'^T over this wave's key channels
             const float4 da = *reinterpret_cast<const float4*>(&O.d1[j0[0]]);
@@ -495,9 +502,9 @@ __global__ __launch_bounds__(NTF) void wkv6_fwd_ws(const ArgsC a) {
 
 int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                           const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
-                          const uint16_t* s0, uint16_t* y) {
+                          const uint16_t* s0, uint16_t* y, float* saved) {
     ArgsC a{};
-    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y;
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y; a.saved = saved;
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_fwd_ws<W_RAW>, dim3(B * H), dim3(NTF), 0, st, a);
     else if (wmode == W_EW) hipLaunchKernelGGL(wkv6_fwd_ws<W_EW>, dim3(B * H), dim3(NTF), 0, st, a);
     else hipLaunchKernelGGL(wkv6_fwd_ws<W_HEAD>, dim3(B * H), dim3(NTF), 0, st, a);
