@@ -10,23 +10,24 @@
 // S0 = the forward state entering the chunk: the forward kernel stores it for every second chunk (fp32, [value][key]);
 // the state of the odd chunk in between is rebuilt here with one update, S <- S dec + d2 V^T K'.
 //
-// One workgroup of 16 waves per (batch, head), four roles of four waves each; wave w of a role owns 16 channels:
+// One workgroup of 12 waves per (batch, head), three roles of four waves each; wave w of a role owns 16 channels:
 //   P  (prep)   channels 16w..16w+15 of r, k, w, v, gy for all 32 tokens of a chunk: lane = 16 * (channel quad) + token,
-//               so the two time scans of a half-chunk are four DPP adds inside a 16-lane row and no prep wave ever needs
-//               another one's sums.  Writes the bf16 hi / lo planes of R', K', plain v, gy, and the exponents cc_t = log2 ea_t.
-//   SW (state)  forward state S[i][j], key channels j = 16w..: lane = j, registers = i.  X, gr, gu, the running sum of r dr'.
-//   DW (dstate) gradient state dS[i][j], key channels j = 16w..: lane = j, registers = i.  Z, gk, gw, gs, dS update.
-//   EW (dstate^T) dS[i][j], value channels i = 16w..: lane = i, registers = j.  gv, dS update, and the causal tiles A, Bm of
+//               so the time scans of a half-chunk are four DPP adds inside a 16-lane row and no prep wave ever needs
+//               another one's sums.  Writes the bf16 hi / lo planes of R', K', plain v, gy; keeps r, k and the exponents
+//               cc_t = log2 ea_t of the chunks in flight in registers and, three iterations later, turns the X and Z of
+//               that chunk into gr, gk, gw (and gu) and stores them: all elementwise work sits where the inputs are.
+//   SD (states) forward state S[i][j] and gradient state dS[i][j], key channels j = 16w..: lane = j, registers = i.
+//               X, Z, gs, the dS update, P at the anchors.
+//   E  (dstate^T) dS[i][j], value channels i = 16w..: lane = i, registers = j.  gv, dS update, and the causal tiles A, Bm of
 //               the next chunk.
 // A state is the accumulator of its update product and, as it stands, the A operand of the products that read it
 // (K slots <-> channels in accumulator order).  Operands with the tokens along K come from the natural [token][channel]
 // planes through ds_read_b64_tr_b16: 16 lanes read a 4 x 16 block and each ends up with one column of it.
 // The accumulators of X, Z, gv have lane = token and four consecutive channels in registers -- the layout of the prep
-// waves -- so gr, gk, gw, gv are finished in registers and stored from there.
+// waves: X and Z cross to prep wave w through LDS lane for lane, gv is stored from registers.
 //
 // Pipeline (one barrier per chunk): in iteration `it` the P waves prepare chunk n-1-it, the EW waves make the tiles of
-// chunk n-it, SW / DW / EW do the products of chunk n+1-it, and DW finishes gw of chunk n+2-it (it needs SW's running sum
-// of r dr', which crosses through LDS).
+// chunk n-it, the SD and E waves do the products of chunk n+1-it, and the P waves finish chunk n+2-it.
 //
 // A chunk in which some channel decays by more than e^-60 over either half cannot use the mid-point factors.  Such a
 // (batch, head) is flagged in `flags` and the caller reruns it with the two-sweep kernels, which have a step-by-step path.
@@ -35,7 +36,7 @@
 namespace rwkv {
 namespace {
 
-constexpr int NTG = 16 * 64;
+constexpr int NTG = 12 * 64;           // 3 waves per SIMD: 168 registers per lane
 constexpr int CS = 72;             // row stride (dwords) of an fp32 [token][channel] array
 
 struct alignas(16) SlotG {
@@ -45,14 +46,13 @@ struct alignas(16) SlotG {
 };
 struct alignas(16) TilesG {
     uint32_t AH[L][AS], AL[L][AS], BH[L][AS], BL[L][AS];   // [t][s] bf16 hi / lo
-    float vg[L];                            // v_t . gy_t
 };
 struct alignas(16) SmemG {
     SlotG slot[3];
-    float cc[2][L][CS];                     // cc_t = c_t - c_m (log2 units)
     TilesG tile[2];
-    float prx[2][L][CS];                    // sum of r dr' over the later tokens, anchor to anchor
-    float pex[N];                           // P at the last anchor
+    float xz[2][2][L][CS];                  // [chunk parity][X, Z][token][key channel]: from SD wave w to P wave w
+    float vg[4][L];                         // v_t . gy_t of the chunks in flight
+    float pex[2][N];                        // P = sum_i dS S at the last two anchors
 };
 static_assert(sizeof(SmemG) <= 160 * 1024, "LDS");
 
@@ -106,7 +106,7 @@ struct ArgsG {
     int* flags;                    // [B*H][4]
 };
 
-// state entering even chunk e of this (batch, head), in the layout of the SW / DW waves: lane <-> key channel 16w + l16,
+// state entering even chunk e of this (batch, head), in the layout of the SD waves: lane <-> key channel 16w + l16,
 // x[tile][v] <-> value channel 16 tile + 4g + v
 DEVINL void load_state(const float* __restrict__ p, f32x4 (&x)[4], const int g) {
 #pragma unroll
@@ -120,52 +120,70 @@ template <int WMODE>
 DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n) {
     const int jq = lane >> 4, tp = lane & 15, ch = 16 * w + 4 * jq;
     const int T = a.T, C = a.C;
-    const uint16_t* __restrict__ rb = a.r + base + ch;
-    const uint16_t* __restrict__ kb = a.k + base + ch;
-    const uint16_t* __restrict__ vb = a.v + base + ch;
-    const uint16_t* __restrict__ gb = a.gy + base + ch;
-    const uint16_t* __restrict__ wb = static_cast<const uint16_t*>(a.w) + base + ch;
+    // wave-uniform bases plus one 32-bit per-lane offset: the addresses stay out of the vector registers
+    const uint16_t* __restrict__ rb = a.r + base;
+    const uint16_t* __restrict__ kb = a.k + base;
+    const uint16_t* __restrict__ vb = a.v + base;
+    const uint16_t* __restrict__ gb = a.gy + base;
+    const uint16_t* __restrict__ wb = static_cast<const uint16_t*>(a.w) + base;
     float uj[4];
     {
         const uint2 x = *reinterpret_cast<const uint2*>(a.u + h * N + ch);
         uj[0] = bf_lo(x.x); uj[1] = bf_hi(x.x); uj[2] = bf_lo(x.y); uj[3] = bf_hi(x.y);
     }
-    struct Raw { uint2 r[2], k[2], v[2], g[2], w[2]; };
+    // r, k, w are needed by the arithmetic of a preparation and are fetched two chunks ahead; v, gy are only copied
+    // into their planes at its end and are fetched one chunk ahead
+    struct Raw { uint2 r[2], k[2], w[2]; };
+    struct RawVG { uint2 v[2], g[2]; };
     Raw ring[2];
+    RawVG vgn;
+    auto row_of = [&](const int c, const int e) __attribute__((always_inline)) {
+        const int t = c * L + tp + 16 * e;
+        return static_cast<uint32_t>(t < T ? t : T - 1) * C + ch;
+    };
     auto fetch = [&](const int c, Raw& x) __attribute__((always_inline)) {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const int t = c * L + tp + 16 * e;
-            const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C;
+            const uint32_t o = row_of(c, e);
             x.r[e] = *reinterpret_cast<const uint2*>(rb + o);
             x.k[e] = *reinterpret_cast<const uint2*>(kb + o);
-            x.v[e] = *reinterpret_cast<const uint2*>(vb + o);
-            x.g[e] = *reinterpret_cast<const uint2*>(gb + o);
             x.w[e] = *reinterpret_cast<const uint2*>(wb + o);
         }
     };
-    float cch[2][4] = {};                  // cc of the chunk prepared one iteration ago, written one iteration late
+    auto fetch_vg = [&](const int c, RawVG& x) __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const uint32_t o = row_of(c, e);
+            x.v[e] = *reinterpret_cast<const uint2*>(vb + o);
+            x.g[e] = *reinterpret_cast<const uint2*>(gb + o);
+        }
+    };
+    // what the finishing of a chunk needs from its preparation, three iterations earlier
+    struct Held { uint2 r[2], k[2]; float cc[2][4]; };
+    Held hq[3] = {};
     bool any_exact = false;
+    float carry[4] = {0.f, 0.f, 0.f, 0.f}, gu_acc[4] = {0.f, 0.f, 0.f, 0.f};
 
-    auto prep = [&](const int c, Raw& x) __attribute__((always_inline)) {
+    auto prep = [&](const int c, Raw& x, Held& hd) __attribute__((always_inline)) {
         SlotG& O = S.slot[c % 3];
         float lam[2][4], rf[2][4], kf[2][4];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const bool live = c * L + tp + 16 * e < T;
-            if (!live) { x.r[e] = make_uint2(0, 0); x.k[e] = make_uint2(0, 0); x.v[e] = make_uint2(0, 0); x.g[e] = make_uint2(0, 0); }
+            if (!live) { x.r[e] = make_uint2(0, 0); x.k[e] = make_uint2(0, 0); }
             float wf[4];
             unpack4(x.w[e], wf); unpack4(x.r[e], rf[e]); unpack4(x.k[e], kf[e]);
 #pragma unroll
             for (int z = 0; z < 4; ++z) lam[e][z] = live ? -LOG2E * exp2_fast(LOG2E * wf[z]) : 0.f;
+            hd.r[e] = x.r[e]; hd.k[e] = x.k[e];
         }
-        float cc[2][4], l1[4], l2[4];
+        float l1[4], l2[4];
 #pragma unroll
         for (int z = 0; z < 4; ++z) {
             const float s0 = row_suffix_sum(lam[0][z]);        // sum over tokens tp..15
             const float p1 = row_prefix_sum(lam[1][z]);        // sum over tokens 16..16+tp
-            cc[0][z] = -s0;
-            cc[1][z] = p1 - lam[1][z];
+            hd.cc[0][z] = -s0;
+            hd.cc[1][z] = p1 - lam[1][z];
             l1[z] = bc<0>(s0);
             l2[z] = bc<15>(p1);
         }
@@ -189,8 +207,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             ruk[e] = 0.f;
 #pragma unroll
             for (int z = 0; z < 4; ++z) {
-                rp[z] = rf[e][z] * exp2_fast(cc[e][z]);
-                kp[z] = kf[e][z] * exp2_fast(-(cc[e][z] + lam[e][z]));
+                rp[z] = rf[e][z] * exp2_fast(hd.cc[e][z]);
+                kp[z] = kf[e][z] * exp2_fast(-(hd.cc[e][z] + lam[e][z]));
                 ruk[e] = fmaf(rf[e][z] * uj[z], kf[e][z], ruk[e]);
             }
             const HL r0 = hilo2(rp[0], rp[1]), r1 = hilo2(rp[2], rp[3]), k0 = hilo2(kp[0], kp[1]), k1 = hilo2(kp[2], kp[3]);
@@ -198,17 +216,80 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             *reinterpret_cast<uint2*>(&O.RpL[t][8 * w + 2 * jq]) = make_uint2(r0.l, r1.l);
             *reinterpret_cast<uint2*>(&O.KpH[t][8 * w + 2 * jq]) = make_uint2(k0.h, k1.h);
             *reinterpret_cast<uint2*>(&O.KpL[t][8 * w + 2 * jq]) = make_uint2(k0.l, k1.l);
-            *reinterpret_cast<uint2*>(&O.V[t][8 * w + 2 * jq]) = x.v[e];
-            *reinterpret_cast<uint2*>(&O.GY[t][8 * w + 2 * jq]) = x.g[e];
         }
         allreduce2_rows(ruk[0], ruk[1]);                       // sums over the four channel quads of this wave
         if (jq == 0) { O.ruk[w][tp] = ruk[0]; O.ruk[w][tp + 16] = ruk[1]; }
+    };
+    // v, gy of chunk c into their planes.  This comes first in an iteration: the loads it waits for are then older than
+    // everything else in flight except the r, k, w of the next chunk, which the wait can count.
+    auto copy_vg = [&](const int c, const RawVG& y) __attribute__((always_inline)) {
+        SlotG& O = S.slot[c % 3];
 #pragma unroll
-        for (int e = 0; e < 2; ++e)
-#pragma unroll
-            for (int z = 0; z < 4; ++z) cch[e][z] = cc[e][z];
+        for (int e = 0; e < 2; ++e) {
+            const bool live = c * L + tp + 16 * e < T;
+            *reinterpret_cast<uint2*>(&O.V[tp + 16 * e][8 * w + 2 * jq]) = live ? y.v[e] : make_uint2(0, 0);
+            *reinterpret_cast<uint2*>(&O.GY[tp + 16 * e][8 * w + 2 * jq]) = live ? y.g[e] : make_uint2(0, 0);
+        }
     };
 
+    // gr, gk, gw of chunk c from X, Z (left by SD wave w in the last iteration) and what prep kept
+    auto finish = [&](const int c, const Held& hd) __attribute__((always_inline)) {
+        const float4 e4 = *reinterpret_cast<const float4*>(&S.slot[c % 3].l2[ch]);
+        const float l2v[4] = {e4.x, e4.y, e4.z, e4.w};
+        float q[2][4], kdk[2][4], lam[2][4];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int t = tp + 16 * e, tg = c * L + t;
+            const float4 x4 = *reinterpret_cast<const float4*>(&S.xz[c & 1][0][t][ch]);
+            const float4 z4 = *reinterpret_cast<const float4*>(&S.xz[c & 1][1][t][ch]);
+            const float X[4] = {x4.x, x4.y, x4.z, x4.w}, Z[4] = {z4.x, z4.y, z4.z, z4.w};
+            const float vg = S.vg[c & 3][t];
+            float rf[4], kf[4], gr[4], gk[4];
+            unpack4(hd.r[e], rf); unpack4(hd.k[e], kf);
+#pragma unroll
+            for (int z = 0; z < 4; ++z) {
+                const float cc = hd.cc[e][z];
+                const float nx = row_next(cc);
+                const float ccn = tp == 15 ? (e ? l2v[z] : 0.f) : nx;
+                const float drp = exp2_fast(cc) * X[z], dkp = exp2_fast(-ccn) * Z[z];
+                const float uvg = uj[z] * vg;
+                gr[z] = fmaf(uvg, kf[z], drp);
+                gk[z] = fmaf(uvg, rf[z], dkp);
+                kdk[e][z] = kf[z] * dkp;
+                q[e][z] = fmaf(rf[z], drp, -kdk[e][z]);
+                gu_acc[z] = fmaf(rf[z] * kf[z], vg, gu_acc[z]);
+                lam[e][z] = gw_factor((ccn - cc) * LN2);
+            }
+            if (tg < T) {
+                const uint32_t o = static_cast<uint32_t>(tg) * C + ch;
+                *reinterpret_cast<uint2*>(a.gr + base + o) = make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3]));
+                *reinterpret_cast<uint2*>(a.gk + base + o) = make_uint2(pack_bf2(gk[0], gk[1]), pack_bf2(gk[2], gk[3]));
+            }
+        }
+        float gw[2][4];
+#pragma unroll
+        for (int z = 0; z < 4; ++z) {
+            const float s1 = row_suffix_sum(q[1][z]) + carry[z];           // P_t of the second half
+            const float s0 = row_suffix_sum(q[0][z]) + bc<0>(s1);
+            gw[1][z] = lam[1][z] * ((s1 - q[1][z]) - kdk[1][z]);          // lam (P_{t+1} - k dk')
+            gw[0][z] = lam[0][z] * ((s0 - q[0][z]) - kdk[0][z]);
+            carry[z] = bc<0>(s0);
+        }
+        if (!(c & 1)) {
+            // the chunk began at an anchor: from here on P counts from its exact value there
+            const float4 p4 = *reinterpret_cast<const float4*>(&S.pex[(c >> 1) & 1][ch]);
+            carry[0] = p4.x; carry[1] = p4.y; carry[2] = p4.z; carry[3] = p4.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int tg = c * L + tp + 16 * e;
+            if (tg < T)
+                *reinterpret_cast<uint2*>(a.gw + base + (static_cast<uint32_t>(tg) * C + ch)) =
+                    make_uint2(pack_bf2(gw[e][0], gw[e][1]), pack_bf2(gw[e][2], gw[e][3]));
+        }
+    };
+
+    fetch_vg(n - 1, vgn);
     fetch(n - 1, ring[0]);
     fetch(n >= 2 ? n - 2 : 0, ring[1]);
     for (int it0 = 0; it0 <= n + 2; it0 += 2)
@@ -217,54 +298,47 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             const int it = it0 + z;
             if (it <= n + 2) {
                 const int cp = n - 1 - it;
-                if (it >= 1 && cp + 1 >= 0) {
-                    float (*cw)[CS] = S.cc[(cp + 1) & 1];
-                    *reinterpret_cast<float4*>(&cw[tp][ch]) = make_float4(cch[0][0], cch[0][1], cch[0][2], cch[0][3]);
-                    *reinterpret_cast<float4*>(&cw[tp + 16][ch]) = make_float4(cch[1][0], cch[1][1], cch[1][2], cch[1][3]);
-                }
-                if (cp >= 0) {
-                    prep(cp, ring[z]);
-                    if (cp >= 2) fetch(cp - 2, ring[z]);
-                }
+                // The same loads in every iteration (chunk index clamped): the wait for a chunk's registers is then the
+                // count of loads issued after them on every path, and never has to cover the newest ones.
+                if (cp >= 0) copy_vg(cp, vgn);
+                fetch_vg(cp >= 1 ? cp - 1 : 0, vgn);
+                __builtin_amdgcn_sched_barrier(0);
+                if (it >= 3) finish(cp + 3, hq[2]);
+                __builtin_amdgcn_sched_barrier(0);
+                hq[2] = hq[1]; hq[1] = hq[0];
+                if (cp >= 0) prep(cp, ring[z], hq[0]);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(cp >= 2 ? cp - 2 : 0, ring[z]);
                 __syncthreads();
             }
         });
     if (lane == 0) a.flags[bh * 4 + w] = any_exact ? 1 : 0;
+    // gu of this batch row: sum over the tokens (lanes of a row)
+#pragma unroll
+    for (int z = 0; z < 4; ++z) gu_acc[z] = row_sum_to_last(gu_acc[z]);
+    if (tp == 15)
+        *reinterpret_cast<uint2*>(a.gu + bh * N + ch) = make_uint2(pack_bf2(gu_acc[0], gu_acc[1]), pack_bf2(gu_acc[2], gu_acc[3]));
 }
 
-// ---------------------------------------------------------------------------------------------------- SW waves
+// ---------------------------------------------------------------------------------------------------- SD waves
 template <int WMODE>
-DEVINL void role_s(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n) {
+DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t bh, const int n) {
     const int g = lane >> 4, l16 = lane & 15, j = 16 * w + l16;
-    const int T = a.T, C = a.C;
     const int nseg = (n + 1) / 2;
     const float* __restrict__ sv = a.saved + bh * nseg * (N * N) + j;
-    float uj[4];
-    {
-        const uint2 x = *reinterpret_cast<const uint2*>(a.u + h * N + 16 * w + 4 * g);
-        uj[0] = bf_lo(x.x); uj[1] = bf_hi(x.x); uj[2] = bf_lo(x.y); uj[3] = bf_hi(x.y);
-    }
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
-    f32x4 Sa[4], Sn[4];
-    int ea_seg = nseg - 1;                 // segment held in Sa
-    load_state(sv + static_cast<size_t>(ea_seg) * (N * N), Sa, g);
-    if (ea_seg >= 1) load_state(sv + static_cast<size_t>(ea_seg - 1) * (N * N), Sn, g);
-    else {
-#pragma unroll
-        for (int tl = 0; tl < 4; ++tl) Sn[tl] = zero4;
-    }
-    float carry[4] = {0.f, 0.f, 0.f, 0.f}, gu_acc[4] = {0.f, 0.f, 0.f, 0.f};
-
-    for (int it = 0; it <= n + 2; ++it) {
-        const int c = n + 1 - it;
-        if (it >= 2 && c >= 0) {
-            const SlotG& O = S.slot[c % 3];
-            const TilesG& Tl = S.tile[c & 1];
+    f32x4 D[4] = {zero4, zero4, zero4, zero4};
+    // one chunk: X and Z of chunk c, the update of dS, and P at an anchor; Sa = the saved state of the chunk's segment
+    auto chunk = [&](const int c, const f32x4 (&Sa)[4]) __attribute__((always_inline)) {
+        const SlotG& O = S.slot[c % 3];
+        const TilesG& Tl = S.tile[c & 1];
+        const float d1 = O.d1[j], d2 = O.d2[j], dec = O.dec[j];
+        {
             f32x4 Sc[4];
             if (c & 1) {
                 // state entering the odd chunk: one update of the saved state with the chunk below
                 const SlotG& Q = S.slot[(c - 1) % 3];
-                const float dec = Q.dec[j], d2 = Q.d2[j];
+                const float qdec = Q.dec[j], qd2 = Q.d2[j];
                 const bf16x8 kh = tr_pair(&Q.KpH[8 * g][8 * w], OS, l16), kl = tr_pair(&Q.KpL[8 * g][8 * w], OS, l16);
 #pragma unroll
                 for (int tl = 0; tl < 4; ++tl) {
@@ -272,15 +346,15 @@ DEVINL void role_s(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                     f32x4 U = mfma(vop, kh, zero4);
                     U = mfma(vop, kl, U);
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) Sc[tl][v] = fmaf(Sa[tl][v], dec, d2 * U[v]);
+                    for (int v = 0; v < 4; ++v) Sc[tl][v] = fmaf(Sa[tl][v], qdec, qd2 * U[v]);
                 }
             } else {
 #pragma unroll
                 for (int tl = 0; tl < 4; ++tl) Sc[tl] = Sa[tl];
             }
-            // ------------------------------------------------------------ X^T[j][t] = (S d1)^T GY^T + K'^T Bm^T
+            // -------------------------------------------------------- X^T[j][t] = (S d1)^T GY^T + K'^T Bm^T
             bf16x8 sh[2], sl[2];
-            split16(Sc, O.d1[j], sh, sl);
+            split16(Sc, d1, sh, sl);
             f32x4 X[2] = {zero4, zero4};
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt)
@@ -290,203 +364,79 @@ DEVINL void role_s(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                     X[tt] = mfma(sh[ks], gop, X[tt]);
                     X[tt] = mfma(sl[ks], gop, X[tt]);
                 }
-            {
-                const bf16x8 kh = tr_pair(&O.KpH[8 * g][8 * w], OS, l16), kl = tr_pair(&O.KpL[8 * g][8 * w], OS, l16);
-#pragma unroll
-                for (int tt = 0; tt < 2; ++tt) {
-                    const bf16x8 bh_ = lds_op(&Tl.BH[16 * tt + l16][4 * g]), bl_ = lds_op(&Tl.BL[16 * tt + l16][4 * g]);
-                    X[tt] = mfma(kh, bh_, X[tt]);
-                    X[tt] = mfma(kh, bl_, X[tt]);
-                    X[tt] = mfma(kl, bh_, X[tt]);
-                }
-            }
-            // ------------------------------------------------------------ gr, r dr' and its running sum, gu
-            float rdr[2][4];
+            const bf16x8 kh = tr_pair(&O.KpH[8 * g][8 * w], OS, l16), kl = tr_pair(&O.KpL[8 * g][8 * w], OS, l16);
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
-                const int t = 16 * tt + l16, tg = c * L + t;
-                const float4 c4 = *reinterpret_cast<const float4*>(&S.cc[c & 1][t][16 * w + 4 * g]);
-                const float4 e4 = *reinterpret_cast<const float4*>(&O.l2[16 * w + 4 * g]);
-                const float cc[4] = {c4.x, c4.y, c4.z, c4.w};
-                const float end[4] = {tt ? e4.x : 0.f, tt ? e4.y : 0.f, tt ? e4.z : 0.f, tt ? e4.w : 0.f};
-                float rp[4], rl[4], kp[4], kl4[4];
-                unpack4(*reinterpret_cast<const uint2*>(&O.RpH[t][8 * w + 2 * g]), rp);
-                unpack4(*reinterpret_cast<const uint2*>(&O.RpL[t][8 * w + 2 * g]), rl);
-                unpack4(*reinterpret_cast<const uint2*>(&O.KpH[t][8 * w + 2 * g]), kp);
-                unpack4(*reinterpret_cast<const uint2*>(&O.KpL[t][8 * w + 2 * g]), kl4);
-                const float vg = Tl.vg[t];
-                float gr[4];
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float nx = row_next(cc[v]);
-                    const float ccn = l16 == 15 ? end[v] : nx;
-                    const float Rp = rp[v] + rl[v], Kp = kp[v] + kl4[v];
-                    const float kk = Kp * exp2_fast(ccn);                  // k_t
-                    gr[v] = fmaf(exp2_fast(cc[v]), X[tt][v], uj[v] * kk * vg);
-                    rdr[tt][v] = Rp * X[tt][v];
-                    gu_acc[v] = fmaf(Rp * Kp, exp2_fast(ccn - cc[v]) * vg, gu_acc[v]);
-                }
-                if (tg < T)
-                    *reinterpret_cast<uint2*>(a.gr + base + static_cast<size_t>(tg) * C + 16 * w + 4 * g) =
-                        make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3]));
-            }
-            float x0[4], x1[4];
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const float s1 = row_suffix_sum(rdr[1][v]) + carry[v];
-                const float s0 = row_suffix_sum(rdr[0][v]) + bc<0>(s1);
-                x1[v] = s1 - rdr[1][v];                                    // sum over the tokens after t
-                x0[v] = s0 - rdr[0][v];
-                carry[v] = (c & 1) ? bc<0>(s0) : 0.f;                      // the sum starts again where P is taken exactly
-            }
-            *reinterpret_cast<float4*>(&S.prx[c & 1][l16][16 * w + 4 * g]) = make_float4(x0[0], x0[1], x0[2], x0[3]);
-            *reinterpret_cast<float4*>(&S.prx[c & 1][16 + l16][16 * w + 4 * g]) = make_float4(x1[0], x1[1], x1[2], x1[3]);
-            if (!(c & 1)) {
-                // next segment: its saved state has been on its way for two chunks
-#pragma unroll
-                for (int tl = 0; tl < 4; ++tl) Sa[tl] = Sn[tl];
-                ea_seg -= 1;
-                if (ea_seg >= 1) load_state(sv + static_cast<size_t>(ea_seg - 1) * (N * N), Sn, g);
+                const bf16x8 bh_ = lds_op(&Tl.BH[16 * tt + l16][4 * g]), bl_ = lds_op(&Tl.BL[16 * tt + l16][4 * g]);
+                X[tt] = mfma(kh, bh_, X[tt]);
+                X[tt] = mfma(kh, bl_, X[tt]);
+                X[tt] = mfma(kl, bh_, X[tt]);
+                *reinterpret_cast<float4*>(&S.xz[c & 1][0][16 * tt + l16][16 * w + 4 * g]) = make_float4(X[tt][0], X[tt][1], X[tt][2], X[tt][3]);
             }
         }
+        // ------------------------------------------------------------ Z^T[j][s] = (dS d2)^T V^T + R'^T Bm
+        bf16x8 dh[2], dl[2];
+        split16(D, d2, dh, dl);
+        f32x4 Z[2] = {zero4, zero4};
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const bf16x8 vop = acc_order_op(&O.V[16 * tt + l16][0], ks, g);
+                Z[tt] = mfma(dh[ks], vop, Z[tt]);
+                Z[tt] = mfma(dl[ks], vop, Z[tt]);
+            }
+        const bf16x8 rh = tr_pair(&O.RpH[8 * g][8 * w], OS, l16), rl = tr_pair(&O.RpL[8 * g][8 * w], OS, l16);
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            const bf16x8 bh_ = tr_pair(&Tl.BH[8 * g][8 * tt], AS, l16), bl_ = tr_pair(&Tl.BL[8 * g][8 * tt], AS, l16);
+            Z[tt] = mfma(rh, bh_, Z[tt]);
+            Z[tt] = mfma(rh, bl_, Z[tt]);
+            Z[tt] = mfma(rl, bh_, Z[tt]);
+            *reinterpret_cast<float4*>(&S.xz[c & 1][1][16 * tt + l16][16 * w + 4 * g]) = make_float4(Z[tt][0], Z[tt][1], Z[tt][2], Z[tt][3]);
+        }
+        // ------------------------------------------------------------ dS <- dS dec + d1 GY^T R'
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) {
+            const bf16x8 gop = tr_pair(&O.GY[8 * g][8 * tl], OS, l16);
+            f32x4 U = mfma(gop, rh, zero4);
+            U = mfma(gop, rl, U);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) D[tl][v] = fmaf(D[tl][v], dec, d1 * U[v]);
+        }
+        if (!(c & 1)) {
+            // anchor: P = sum_i dS S with the saved state entering this chunk
+            float p = 0.f;
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) p = fmaf(D[tl][v], Sa[tl][v], p);
+            p = allreduce_rows(p);
+            if (g == 0) S.pex[(c >> 1) & 1][j] = p;
+        }
+    };
+    // a segment = an even chunk and the odd chunk above it, taken in reverse; one barrier per chunk
+    auto segment = [&](const int sg, const f32x4 (&Sa)[4]) __attribute__((always_inline)) {
+        if (2 * sg + 1 < n) { chunk(2 * sg + 1, Sa); __syncthreads(); }
+        chunk(2 * sg, Sa);
         __syncthreads();
+    };
+    // The saved states alternate between two register sets with fixed roles, each refilled as soon as its segment is
+    // done, two chunks before it is read again: no value that is still in flight is ever copied.
+    f32x4 SA[4], SB[4];
+    const int top = nseg - 1;
+    // (every refill is issued on every path, with the segment index clamped, so that the waits can count them)
+    load_state(sv + static_cast<size_t>(top) * (N * N), SA, g);
+    load_state(sv + static_cast<size_t>(top >= 1 ? top - 1 : 0) * (N * N), SB, g);
+    __syncthreads();                       // iterations 0 and 1: nothing prepared yet
+    __syncthreads();
+    for (int sg = top; sg >= 0; sg -= 2) {
+        segment(sg, SA);
+        load_state(sv + static_cast<size_t>(sg >= 2 ? sg - 2 : 0) * (N * N), SA, g);
+        if (sg >= 1) segment(sg - 1, SB);
+        load_state(sv + static_cast<size_t>(sg >= 3 ? sg - 3 : 0) * (N * N), SB, g);
     }
-    // gu of this batch row: sum over the tokens (lanes of a row)
-#pragma unroll
-    for (int v = 0; v < 4; ++v) gu_acc[v] = row_sum_to_last(gu_acc[v]);
-    if (l16 == 15)
-        *reinterpret_cast<uint2*>(a.gu + bh * N + 16 * w + 4 * g) = make_uint2(pack_bf2(gu_acc[0], gu_acc[1]), pack_bf2(gu_acc[2], gu_acc[3]));
-}
-
-// ---------------------------------------------------------------------------------------------------- DW waves
-template <int WMODE>
-DEVINL void role_d(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n) {
-    const int g = lane >> 4, l16 = lane & 15, j = 16 * w + l16;
-    const int T = a.T, C = a.C;
-    const int nseg = (n + 1) / 2;
-    const float* __restrict__ sv = a.saved + bh * nseg * (N * N) + j;
-    float uj[4];
-    {
-        const uint2 x = *reinterpret_cast<const uint2*>(a.u + h * N + 16 * w + 4 * g);
-        uj[0] = bf_lo(x.x); uj[1] = bf_hi(x.x); uj[2] = bf_lo(x.y); uj[3] = bf_hi(x.y);
-    }
-    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
-    f32x4 D[4] = {zero4, zero4, zero4, zero4};
-    f32x4 S0[4];
-    int seg = nseg - 1;                    // segment whose saved state is in S0
-    load_state(sv + static_cast<size_t>(seg) * (N * N), S0, g);
-    float carry[4] = {0.f, 0.f, 0.f, 0.f};
-    float pk[2][4] = {}, lamh[2][4] = {};  // of the chunk whose gw is still to be finished
-
-    for (int it = 0; it <= n + 2; ++it) {
-        const int c = n + 1 - it;
-        if (it >= 3 && c + 1 >= 0) {
-            // ------------------------------------------------------------ gw of chunk c + 1
-            const int cf = c + 1;
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                const int t = 16 * tt + l16, tg = cf * L + t;
-                const float4 p4 = *reinterpret_cast<const float4*>(&S.prx[cf & 1][t][16 * w + 4 * g]);
-                const float pr[4] = {p4.x, p4.y, p4.z, p4.w};
-                float gw[4];
-#pragma unroll
-                for (int v = 0; v < 4; ++v) gw[v] = lamh[tt][v] * (pr[v] - pk[tt][v]);
-                if (tg < T)
-                    *reinterpret_cast<uint2*>(a.gw + base + static_cast<size_t>(tg) * C + 16 * w + 4 * g) =
-                        make_uint2(pack_bf2(gw[0], gw[1]), pack_bf2(gw[2], gw[3]));
-            }
-            if (!(cf & 1)) {
-                // chunk cf began at an anchor: from here on P counts from its exact value there
-                const float4 p4 = *reinterpret_cast<const float4*>(&S.pex[16 * w + 4 * g]);
-                carry[0] = -p4.x; carry[1] = -p4.y; carry[2] = -p4.z; carry[3] = -p4.w;
-            }
-        }
-        if (it >= 2 && c >= 0) {
-            const SlotG& O = S.slot[c % 3];
-            const TilesG& Tl = S.tile[c & 1];
-            const float d1 = O.d1[j], d2 = O.d2[j], dec = O.dec[j];
-            // ------------------------------------------------------------ Z^T[j][s] = (dS d2)^T V^T + R'^T Bm
-            bf16x8 dh[2], dl[2];
-            split16(D, d2, dh, dl);
-            f32x4 Z[2] = {zero4, zero4};
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    const bf16x8 vop = acc_order_op(&O.V[16 * tt + l16][0], ks, g);
-                    Z[tt] = mfma(dh[ks], vop, Z[tt]);
-                    Z[tt] = mfma(dl[ks], vop, Z[tt]);
-                }
-            const bf16x8 rh = tr_pair(&O.RpH[8 * g][8 * w], OS, l16), rl = tr_pair(&O.RpL[8 * g][8 * w], OS, l16);
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                const bf16x8 bh_ = tr_pair(&Tl.BH[8 * g][8 * tt], AS, l16), bl_ = tr_pair(&Tl.BL[8 * g][8 * tt], AS, l16);
-                Z[tt] = mfma(rh, bh_, Z[tt]);
-                Z[tt] = mfma(rh, bl_, Z[tt]);
-                Z[tt] = mfma(rl, bh_, Z[tt]);
-            }
-            // ------------------------------------------------------------ gk, k dk' and its running sum, lam for gw
-            float kdk[2][4];
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                const int t = 16 * tt + l16, tg = c * L + t;
-                const float4 c4 = *reinterpret_cast<const float4*>(&S.cc[c & 1][t][16 * w + 4 * g]);
-                const float4 e4 = *reinterpret_cast<const float4*>(&O.l2[16 * w + 4 * g]);
-                const float cc[4] = {c4.x, c4.y, c4.z, c4.w};
-                const float end[4] = {tt ? e4.x : 0.f, tt ? e4.y : 0.f, tt ? e4.z : 0.f, tt ? e4.w : 0.f};
-                float rp[4], rl4[4], kp[4], kl4[4];
-                unpack4(*reinterpret_cast<const uint2*>(&O.RpH[t][8 * w + 2 * g]), rp);
-                unpack4(*reinterpret_cast<const uint2*>(&O.RpL[t][8 * w + 2 * g]), rl4);
-                unpack4(*reinterpret_cast<const uint2*>(&O.KpH[t][8 * w + 2 * g]), kp);
-                unpack4(*reinterpret_cast<const uint2*>(&O.KpL[t][8 * w + 2 * g]), kl4);
-                const float vg = Tl.vg[t];
-                float gk[4];
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float nx = row_next(cc[v]);
-                    const float ccn = l16 == 15 ? end[v] : nx;
-                    const float Rp = rp[v] + rl4[v], Kp = kp[v] + kl4[v];
-                    const float rr = Rp * exp2_fast(-cc[v]);               // r_s
-                    gk[v] = fmaf(exp2_fast(-ccn), Z[tt][v], uj[v] * rr * vg);
-                    kdk[tt][v] = Kp * Z[tt][v];
-                    lamh[tt][v] = gw_factor((ccn - cc[v]) * LN2);
-                }
-                if (tg < T)
-                    *reinterpret_cast<uint2*>(a.gk + base + static_cast<size_t>(tg) * C + 16 * w + 4 * g) =
-                        make_uint2(pack_bf2(gk[0], gk[1]), pack_bf2(gk[2], gk[3]));
-            }
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const float s1 = row_suffix_sum(kdk[1][v]) + carry[v];
-                const float s0 = row_suffix_sum(kdk[0][v]) + bc<0>(s1);
-                pk[1][v] = s1;                                             // sum over the tokens from t on
-                pk[0][v] = s0;
-                carry[v] = bc<0>(s0);
-            }
-            // ------------------------------------------------------------ dS <- dS dec + d1 GY^T R'
-#pragma unroll
-            for (int tl = 0; tl < 4; ++tl) {
-                const bf16x8 gop = tr_pair(&O.GY[8 * g][8 * tl], OS, l16);
-                f32x4 U = mfma(gop, rh, zero4);
-                U = mfma(gop, rl, U);
-#pragma unroll
-                for (int v = 0; v < 4; ++v) D[tl][v] = fmaf(D[tl][v], dec, d1 * U[v]);
-            }
-            if (!(c & 1)) {
-                // anchor: P = sum_i dS S with the saved state entering this chunk
-                float p = 0.f;
-#pragma unroll
-                for (int tl = 0; tl < 4; ++tl)
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) p = fmaf(D[tl][v], S0[tl][v], p);
-                p = allreduce_rows(p);
-                if (g == 0) S.pex[j] = p;
-                seg -= 1;
-                if (seg >= 0) load_state(sv + static_cast<size_t>(seg) * (N * N), S0, g);
-            }
-        }
-        __syncthreads();
-    }
+    __syncthreads();                       // iteration n + 2: the P waves finish chunk 0
     if (a.gs != nullptr) {
 #pragma unroll
         for (int tl = 0; tl < 4; ++tl)
@@ -526,7 +476,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int sl = 4 * g + v;
-                if (sl == l16) Tl.vg[t] = bm[v];
+                if (sl == l16) S.vg[c & 3][t] = bm[v];
                 am[v] = (sl < l16) ? am[v] : (sl == l16 ? d : 0.f);
                 bm[v] = (sl < l16) ? bm[v] : 0.f;
             }
@@ -605,8 +555,7 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG a) {
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
     if (wid < 4) role_prep<WMODE>(S, a, lane, w, base, h, bh, n);
-    else if (wid < 8) role_s<WMODE>(S, a, lane, w, base, h, bh, n);
-    else if (wid < 12) role_d<WMODE>(S, a, lane, w, base, h, bh, n);
+    else if (wid < 8) role_sd<WMODE>(S, a, lane, w, bh, n);
     else role_e<WMODE>(S, a, lane, w, base, n);
 }
 
