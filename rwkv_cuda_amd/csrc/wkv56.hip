@@ -1260,7 +1260,7 @@ int rwkv_wkv6f_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16
 
 size_t rwkv_wkv6f_backward_saved_workspace_bytes(int B, int T, int C, int H) {
     const size_t n = rwkv_wkv6f_backward_workspace_bytes(B, T, C, H);
-    return n == 0 ? 0 : round16(n) + round16(static_cast<size_t>(B) * H * 4 * sizeof(int));
+    return n == 0 ? 0 : round16(n) + round16(static_cast<size_t>(B) * H * 8 * sizeof(int));
 }
 
 int rwkv_wkv6f_backward_saved(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,

@@ -10,8 +10,9 @@
 // S0 = the forward state entering the chunk: the forward kernel stores it for every second chunk (fp32, [value][key]);
 // the state of the odd chunk in between is rebuilt here with one update, S <- S dec + d2 V^T K'.
 //
-// One workgroup of 12 waves per (batch, head), three roles of four waves each; wave w of a role owns 16 channels:
-//   P  (prep)   channels 16w..16w+15 of r, k, w, v, gy for all 32 tokens of a chunk: lane = 16 * (channel quad) + token,
+// One workgroup of 16 waves per (batch, head) in three roles: eight P waves with 8 channels each, four SD and four E waves
+// with 16 channels each:
+//   P  (prep)   channels 8w..8w+7 of r, k, w, v, gy for all 32 tokens of a chunk: lane = 16 * (channel pair) + token,
 //               so the time scans of a half-chunk are four DPP adds inside a 16-lane row and no prep wave ever needs
 //               another one's sums.  Writes the bf16 hi / lo planes of R', K', plain v, gy; keeps r, k and the exponents
 //               cc_t = log2 ea_t of the chunks in flight in registers and, three iterations later, turns the X and Z of
@@ -24,7 +25,7 @@
 // (K slots <-> channels in accumulator order).  Operands with the tokens along K come from the natural [token][channel]
 // planes through ds_read_b64_tr_b16: 16 lanes read a 4 x 16 block and each ends up with one column of it.
 // The accumulators of X, Z, gv have lane = token and four consecutive channels in registers -- the layout of the prep
-// waves: X and Z cross to prep wave w through LDS lane for lane, gv is stored from registers.
+// waves: X and Z cross to the prep waves through LDS, gv is stored from registers.
 //
 // Pipeline (one barrier per chunk): in iteration `it` the P waves prepare chunk n-1-it, the EW waves make the tiles of
 // chunk n-it, the SD and E waves do the products of chunk n+1-it, and the P waves finish chunk n+2-it.
@@ -36,13 +37,13 @@
 namespace rwkv {
 namespace {
 
-constexpr int NTG = 12 * 64;           // 3 waves per SIMD: 168 registers per lane
+constexpr int NTG = 16 * 64;
 constexpr int CS = 72;             // row stride (dwords) of an fp32 [token][channel] array
 
 struct alignas(16) SlotG {
     uint32_t RpH[L][OS], RpL[L][OS], KpH[L][OS], KpL[L][OS], V[L][OS], GY[L][OS];
     float d1[N], d2[N], dec[N], l2[N];     // 2^{c_m}, 2^{c_L - c_m}, 2^{c_L}, cc_32 = c_L - c_m
-    float ruk[4][L];                        // sum of r u k over the 16 channels of each prep wave
+    float ruk[8][L];                        // sum of r u k over the 8 channels of each prep wave
 };
 struct alignas(16) TilesG {
     uint32_t AH[L][AS], AL[L][AS], BH[L][AS], BL[L][AS];   // [t][s] bf16 hi / lo
@@ -50,7 +51,7 @@ struct alignas(16) TilesG {
 struct alignas(16) SmemG {
     SlotG slot[3];
     TilesG tile[2];
-    float xz[2][2][L][CS];                  // [chunk parity][X, Z][token][key channel]: from SD wave w to P wave w
+    float xz[2][2][L][CS];                  // [chunk parity][X, Z][token][key channel]: from the SD waves to the P waves
     float vg[4][L];                         // v_t . gy_t of the chunks in flight
     float pex[2][N];                        // P = sum_i dS S at the last two anchors
 };
@@ -103,7 +104,7 @@ struct ArgsG {
     const void* w;
     uint16_t *gr, *gk, *gv, *gw, *gu, *gs;
     const float* saved;            // [B*H][ceil(n/2)][64][64]: the forward state entering every even chunk
-    int* flags;                    // [B*H][4]
+    int* flags;                    // [B*H][8]
 };
 
 // state entering even chunk e of this (batch, head), in the layout of the SD waves: lane <-> key channel 16w + l16,
@@ -116,9 +117,10 @@ DEVINL void load_state(const float* __restrict__ p, f32x4 (&x)[4], const int g) 
 }
 
 // ---------------------------------------------------------------------------------------------------- P waves
+// wave w (0..7): channels 8w..8w+7; lane = 16 * (channel pair) + token: a thread has two channels of tokens tp and tp + 16
 template <int WMODE>
 DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n) {
-    const int jq = lane >> 4, tp = lane & 15, ch = 16 * w + 4 * jq;
+    const int jq = lane >> 4, tp = lane & 15, ch = 8 * w + 2 * jq, cd = 4 * w + jq;      // cd: dword column of the pair in a bf16 plane
     const int T = a.T, C = a.C;
     // wave-uniform bases plus one 32-bit per-lane offset: the addresses stay out of the vector registers
     const uint16_t* __restrict__ rb = a.r + base;
@@ -126,15 +128,15 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     const uint16_t* __restrict__ vb = a.v + base;
     const uint16_t* __restrict__ gb = a.gy + base;
     const uint16_t* __restrict__ wb = static_cast<const uint16_t*>(a.w) + base;
-    float uj[4];
+    float uj[2];
     {
-        const uint2 x = *reinterpret_cast<const uint2*>(a.u + h * N + ch);
-        uj[0] = bf_lo(x.x); uj[1] = bf_hi(x.x); uj[2] = bf_lo(x.y); uj[3] = bf_hi(x.y);
+        const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + ch);
+        uj[0] = bf_lo(x); uj[1] = bf_hi(x);
     }
     // r, k, w are needed by the arithmetic of a preparation and are fetched two chunks ahead; v, gy are only copied
-    // into their planes at its end and are fetched one chunk ahead
-    struct Raw { uint2 r[2], k[2], w[2]; };
-    struct RawVG { uint2 v[2], g[2]; };
+    // into their planes and are fetched one chunk ahead
+    struct Raw { uint32_t r[2], k[2], w[2]; };
+    struct RawVG { uint32_t v[2], g[2]; };
     Raw ring[2];
     RawVG vgn;
     auto row_of = [&](const int c, const int e) __attribute__((always_inline)) {
@@ -145,41 +147,54 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const uint32_t o = row_of(c, e);
-            x.r[e] = *reinterpret_cast<const uint2*>(rb + o);
-            x.k[e] = *reinterpret_cast<const uint2*>(kb + o);
-            x.w[e] = *reinterpret_cast<const uint2*>(wb + o);
+            x.r[e] = *reinterpret_cast<const uint32_t*>(rb + o);
+            x.k[e] = *reinterpret_cast<const uint32_t*>(kb + o);
+            x.w[e] = *reinterpret_cast<const uint32_t*>(wb + o);
         }
     };
     auto fetch_vg = [&](const int c, RawVG& x) __attribute__((always_inline)) {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const uint32_t o = row_of(c, e);
-            x.v[e] = *reinterpret_cast<const uint2*>(vb + o);
-            x.g[e] = *reinterpret_cast<const uint2*>(gb + o);
+            x.v[e] = *reinterpret_cast<const uint32_t*>(vb + o);
+            x.g[e] = *reinterpret_cast<const uint32_t*>(gb + o);
         }
     };
     // what the finishing of a chunk needs from its preparation, three iterations earlier
-    struct Held { uint2 r[2], k[2]; float cc[2][4]; };
+    struct Held { uint32_t r[2], k[2]; float cc[2][2]; };
     Held hq[3] = {};
     bool any_exact = false;
-    float carry[4] = {0.f, 0.f, 0.f, 0.f}, gu_acc[4] = {0.f, 0.f, 0.f, 0.f};
+    float carry[2] = {0.f, 0.f}, gu_acc[2] = {0.f, 0.f};
+    // Only the last chunk of the sequence can be cut short (PARTIAL): its rows past T carry no input and no decay.
 
-    auto prep = [&](const int c, Raw& x, Held& hd) __attribute__((always_inline)) {
+    // v, gy of chunk c into their planes.  This comes first in an iteration: the loads it waits for are then older than
+    // everything else in flight except the r, k, w of the next chunk, which the wait can count.
+    auto copy_vg = [&](const int c, const RawVG& y, auto PARTIAL) __attribute__((always_inline)) {
         SlotG& O = S.slot[c % 3];
-        float lam[2][4], rf[2][4], kf[2][4];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const bool live = c * L + tp + 16 * e < T;
-            if (!live) { x.r[e] = make_uint2(0, 0); x.k[e] = make_uint2(0, 0); }
-            float wf[4];
-            unpack4(x.w[e], wf); unpack4(x.r[e], rf[e]); unpack4(x.k[e], kf[e]);
+            const bool live = !decltype(PARTIAL)::value || c * L + tp + 16 * e < T;
+            O.V[tp + 16 * e][cd] = live ? y.v[e] : 0u;
+            O.GY[tp + 16 * e][cd] = live ? y.g[e] : 0u;
+        }
+    };
+
+    auto prep = [&](const int c, Raw& x, Held& hd, auto PARTIAL) __attribute__((always_inline)) {
+        SlotG& O = S.slot[c % 3];
+        float lam[2][2], rf[2][2], kf[2][2];
 #pragma unroll
-            for (int z = 0; z < 4; ++z) lam[e][z] = live ? -LOG2E * exp2_fast(LOG2E * wf[z]) : 0.f;
+        for (int e = 0; e < 2; ++e) {
+            const bool live = !decltype(PARTIAL)::value || c * L + tp + 16 * e < T;
+            if (!live) { x.r[e] = 0u; x.k[e] = 0u; }
+            rf[e][0] = bf_lo(x.r[e]); rf[e][1] = bf_hi(x.r[e]);
+            kf[e][0] = bf_lo(x.k[e]); kf[e][1] = bf_hi(x.k[e]);
+            lam[e][0] = live ? -LOG2E * exp2_fast(LOG2E * bf_lo(x.w[e])) : 0.f;
+            lam[e][1] = live ? -LOG2E * exp2_fast(LOG2E * bf_hi(x.w[e])) : 0.f;
             hd.r[e] = x.r[e]; hd.k[e] = x.k[e];
         }
-        float l1[4], l2[4];
+        float l1[2], l2[2];
 #pragma unroll
-        for (int z = 0; z < 4; ++z) {
+        for (int z = 0; z < 2; ++z) {
             const float s0 = row_suffix_sum(lam[0][z]);        // sum over tokens tp..15
             const float p1 = row_prefix_sum(lam[1][z]);        // sum over tokens 16..16+tp
             hd.cc[0][z] = -s0;
@@ -188,66 +203,47 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             l2[z] = bc<15>(p1);
         }
         {
-            bool bad = false;
-#pragma unroll
-            for (int z = 0; z < 4; ++z) bad = bad || (-l1[z] > RANGE_LIMIT * LOG2E) || (-l2[z] > RANGE_LIMIT * LOG2E);
+            const bool bad = (-l1[0] > RANGE_LIMIT * LOG2E) || (-l2[0] > RANGE_LIMIT * LOG2E) || (-l1[1] > RANGE_LIMIT * LOG2E) || (-l2[1] > RANGE_LIMIT * LOG2E);
             any_exact = any_exact || (__ballot(bad) != 0ull);
         }
         if (tp == 0) {
-            *reinterpret_cast<float4*>(&O.d1[ch]) = make_float4(exp2_fast(l1[0]), exp2_fast(l1[1]), exp2_fast(l1[2]), exp2_fast(l1[3]));
-            *reinterpret_cast<float4*>(&O.d2[ch]) = make_float4(exp2_fast(l2[0]), exp2_fast(l2[1]), exp2_fast(l2[2]), exp2_fast(l2[3]));
-            *reinterpret_cast<float4*>(&O.dec[ch]) = make_float4(exp2_fast(l1[0] + l2[0]), exp2_fast(l1[1] + l2[1]), exp2_fast(l1[2] + l2[2]), exp2_fast(l1[3] + l2[3]));
-            *reinterpret_cast<float4*>(&O.l2[ch]) = make_float4(l2[0], l2[1], l2[2], l2[3]);
+            const float a0 = exp2_fast(l1[0]), a1 = exp2_fast(l1[1]), b0 = exp2_fast(l2[0]), b1 = exp2_fast(l2[1]);
+            *reinterpret_cast<float2*>(&O.d1[ch]) = make_float2(a0, a1);
+            *reinterpret_cast<float2*>(&O.d2[ch]) = make_float2(b0, b1);
+            *reinterpret_cast<float2*>(&O.dec[ch]) = make_float2(a0 * b0, a1 * b1);
+            *reinterpret_cast<float2*>(&O.l2[ch]) = make_float2(l2[0], l2[1]);
         }
         float ruk[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int t = tp + 16 * e;
-            float rp[4], kp[4];
-            ruk[e] = 0.f;
-#pragma unroll
-            for (int z = 0; z < 4; ++z) {
-                rp[z] = rf[e][z] * exp2_fast(hd.cc[e][z]);
-                kp[z] = kf[e][z] * exp2_fast(-(hd.cc[e][z] + lam[e][z]));
-                ruk[e] = fmaf(rf[e][z] * uj[z], kf[e][z], ruk[e]);
-            }
-            const HL r0 = hilo2(rp[0], rp[1]), r1 = hilo2(rp[2], rp[3]), k0 = hilo2(kp[0], kp[1]), k1 = hilo2(kp[2], kp[3]);
-            *reinterpret_cast<uint2*>(&O.RpH[t][8 * w + 2 * jq]) = make_uint2(r0.h, r1.h);
-            *reinterpret_cast<uint2*>(&O.RpL[t][8 * w + 2 * jq]) = make_uint2(r0.l, r1.l);
-            *reinterpret_cast<uint2*>(&O.KpH[t][8 * w + 2 * jq]) = make_uint2(k0.h, k1.h);
-            *reinterpret_cast<uint2*>(&O.KpL[t][8 * w + 2 * jq]) = make_uint2(k0.l, k1.l);
+            const float rp0 = rf[e][0] * exp2_fast(hd.cc[e][0]), rp1 = rf[e][1] * exp2_fast(hd.cc[e][1]);
+            const float kp0 = kf[e][0] * exp2_fast(-(hd.cc[e][0] + lam[e][0])), kp1 = kf[e][1] * exp2_fast(-(hd.cc[e][1] + lam[e][1]));
+            ruk[e] = fmaf(rf[e][0] * uj[0], kf[e][0], rf[e][1] * uj[1] * kf[e][1]);
+            const HL r0 = hilo2(rp0, rp1), k0 = hilo2(kp0, kp1);
+            O.RpH[t][cd] = r0.h; O.RpL[t][cd] = r0.l;
+            O.KpH[t][cd] = k0.h; O.KpL[t][cd] = k0.l;
         }
-        allreduce2_rows(ruk[0], ruk[1]);                       // sums over the four channel quads of this wave
+        allreduce2_rows(ruk[0], ruk[1]);                       // sums over the four channel pairs of this wave
         if (jq == 0) { O.ruk[w][tp] = ruk[0]; O.ruk[w][tp + 16] = ruk[1]; }
     };
-    // v, gy of chunk c into their planes.  This comes first in an iteration: the loads it waits for are then older than
-    // everything else in flight except the r, k, w of the next chunk, which the wait can count.
-    auto copy_vg = [&](const int c, const RawVG& y) __attribute__((always_inline)) {
-        SlotG& O = S.slot[c % 3];
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const bool live = c * L + tp + 16 * e < T;
-            *reinterpret_cast<uint2*>(&O.V[tp + 16 * e][8 * w + 2 * jq]) = live ? y.v[e] : make_uint2(0, 0);
-            *reinterpret_cast<uint2*>(&O.GY[tp + 16 * e][8 * w + 2 * jq]) = live ? y.g[e] : make_uint2(0, 0);
-        }
-    };
 
-    // gr, gk, gw of chunk c from X, Z (left by SD wave w in the last iteration) and what prep kept
-    auto finish = [&](const int c, const Held& hd) __attribute__((always_inline)) {
-        const float4 e4 = *reinterpret_cast<const float4*>(&S.slot[c % 3].l2[ch]);
-        const float l2v[4] = {e4.x, e4.y, e4.z, e4.w};
-        float q[2][4], kdk[2][4], lam[2][4];
+    // gr, gk, gw of chunk c from X, Z (left by the SD waves in the last iteration) and what prep kept
+    auto finish = [&](const int c, const Held& hd, auto PARTIAL) __attribute__((always_inline)) {
+        const float2 e2 = *reinterpret_cast<const float2*>(&S.slot[c % 3].l2[ch]);
+        const float l2v[2] = {e2.x, e2.y};
+        float q[2][2], kdk[2][2], lam[2][2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int t = tp + 16 * e, tg = c * L + t;
-            const float4 x4 = *reinterpret_cast<const float4*>(&S.xz[c & 1][0][t][ch]);
-            const float4 z4 = *reinterpret_cast<const float4*>(&S.xz[c & 1][1][t][ch]);
-            const float X[4] = {x4.x, x4.y, x4.z, x4.w}, Z[4] = {z4.x, z4.y, z4.z, z4.w};
+            const float2 x2 = *reinterpret_cast<const float2*>(&S.xz[c & 1][0][t][ch]);
+            const float2 z2 = *reinterpret_cast<const float2*>(&S.xz[c & 1][1][t][ch]);
+            const float X[2] = {x2.x, x2.y}, Z[2] = {z2.x, z2.y};
             const float vg = S.vg[c & 3][t];
-            float rf[4], kf[4], gr[4], gk[4];
-            unpack4(hd.r[e], rf); unpack4(hd.k[e], kf);
+            const float rf[2] = {bf_lo(hd.r[e]), bf_hi(hd.r[e])}, kf[2] = {bf_lo(hd.k[e]), bf_hi(hd.k[e])};
+            float gr[2], gk[2];
 #pragma unroll
-            for (int z = 0; z < 4; ++z) {
+            for (int z = 0; z < 2; ++z) {
                 const float cc = hd.cc[e][z];
                 const float nx = row_next(cc);
                 const float ccn = tp == 15 ? (e ? l2v[z] : 0.f) : nx;
@@ -260,15 +256,15 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
                 gu_acc[z] = fmaf(rf[z] * kf[z], vg, gu_acc[z]);
                 lam[e][z] = gw_factor((ccn - cc) * LN2);
             }
-            if (tg < T) {
+            if (!decltype(PARTIAL)::value || tg < T) {
                 const uint32_t o = static_cast<uint32_t>(tg) * C + ch;
-                *reinterpret_cast<uint2*>(a.gr + base + o) = make_uint2(pack_bf2(gr[0], gr[1]), pack_bf2(gr[2], gr[3]));
-                *reinterpret_cast<uint2*>(a.gk + base + o) = make_uint2(pack_bf2(gk[0], gk[1]), pack_bf2(gk[2], gk[3]));
+                *reinterpret_cast<uint32_t*>(a.gr + base + o) = pack_bf2(gr[0], gr[1]);
+                *reinterpret_cast<uint32_t*>(a.gk + base + o) = pack_bf2(gk[0], gk[1]);
             }
         }
-        float gw[2][4];
+        float gw[2][2];
 #pragma unroll
-        for (int z = 0; z < 4; ++z) {
+        for (int z = 0; z < 2; ++z) {
             const float s1 = row_suffix_sum(q[1][z]) + carry[z];           // P_t of the second half
             const float s0 = row_suffix_sum(q[0][z]) + bc<0>(s1);
             gw[1][z] = lam[1][z] * ((s1 - q[1][z]) - kdk[1][z]);          // lam (P_{t+1} - k dk')
@@ -277,18 +273,20 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         }
         if (!(c & 1)) {
             // the chunk began at an anchor: from here on P counts from its exact value there
-            const float4 p4 = *reinterpret_cast<const float4*>(&S.pex[(c >> 1) & 1][ch]);
-            carry[0] = p4.x; carry[1] = p4.y; carry[2] = p4.z; carry[3] = p4.w;
+            const float2 p2 = *reinterpret_cast<const float2*>(&S.pex[(c >> 1) & 1][ch]);
+            carry[0] = p2.x; carry[1] = p2.y;
         }
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int tg = c * L + tp + 16 * e;
-            if (tg < T)
-                *reinterpret_cast<uint2*>(a.gw + base + (static_cast<uint32_t>(tg) * C + ch)) =
-                    make_uint2(pack_bf2(gw[e][0], gw[e][1]), pack_bf2(gw[e][2], gw[e][3]));
+            if (!decltype(PARTIAL)::value || tg < T)
+                *reinterpret_cast<uint32_t*>(a.gw + base + (static_cast<uint32_t>(tg) * C + ch)) = pack_bf2(gw[e][0], gw[e][1]);
         }
     };
 
+    const bool cut = (T % L) != 0;         // the last chunk is cut short
+    const std::true_type part{};
+    const std::false_type full{};
     fetch_vg(n - 1, vgn);
     fetch(n - 1, ring[0]);
     fetch(n >= 2 ? n - 2 : 0, ring[1]);
@@ -300,110 +298,155 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
                 const int cp = n - 1 - it;
                 // The same loads in every iteration (chunk index clamped): the wait for a chunk's registers is then the
                 // count of loads issued after them on every path, and never has to cover the newest ones.
-                if (cp >= 0) copy_vg(cp, vgn);
+                if (cp >= 0) { if (cut && it == 0) copy_vg(cp, vgn, part); else copy_vg(cp, vgn, full); }
                 fetch_vg(cp >= 1 ? cp - 1 : 0, vgn);
                 __builtin_amdgcn_sched_barrier(0);
-                if (it >= 3) finish(cp + 3, hq[2]);
+                if (it >= 3) { if (cut && it == 3) finish(cp + 3, hq[2], part); else finish(cp + 3, hq[2], full); }
                 __builtin_amdgcn_sched_barrier(0);
                 hq[2] = hq[1]; hq[1] = hq[0];
-                if (cp >= 0) prep(cp, ring[z], hq[0]);
+                if (cp >= 0) { if (cut && it == 0) prep(cp, ring[z], hq[0], part); else prep(cp, ring[z], hq[0], full); }
                 __builtin_amdgcn_sched_barrier(0);
                 fetch(cp >= 2 ? cp - 2 : 0, ring[z]);
                 __syncthreads();
             }
         });
-    if (lane == 0) a.flags[bh * 4 + w] = any_exact ? 1 : 0;
+    if (lane == 0) a.flags[bh * 8 + w] = any_exact ? 1 : 0;
     // gu of this batch row: sum over the tokens (lanes of a row)
 #pragma unroll
-    for (int z = 0; z < 4; ++z) gu_acc[z] = row_sum_to_last(gu_acc[z]);
-    if (tp == 15)
-        *reinterpret_cast<uint2*>(a.gu + bh * N + ch) = make_uint2(pack_bf2(gu_acc[0], gu_acc[1]), pack_bf2(gu_acc[2], gu_acc[3]));
+    for (int z = 0; z < 2; ++z) gu_acc[z] = row_sum_to_last(gu_acc[z]);
+    if (tp == 15) *reinterpret_cast<uint32_t*>(a.gu + bh * N + ch) = pack_bf2(gu_acc[0], gu_acc[1]);
 }
 
 // ---------------------------------------------------------------------------------------------------- SD waves
 template <int WMODE>
 DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t bh, const int n) {
-    const int g = lane >> 4, l16 = lane & 15, j = 16 * w + l16;
+    // g, l16 and j are redefined behind an empty asm in every iteration: LDS addresses are then formed where they are
+    // used instead of being kept, dozens of them, in registers across the loop
+    int g = lane >> 4, l16 = lane & 15, j = 16 * w + l16;
     const int nseg = (n + 1) / 2;
     const float* __restrict__ sv = a.saved + bh * nseg * (N * N) + j;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     f32x4 D[4] = {zero4, zero4, zero4, zero4};
-    // one chunk: X and Z of chunk c, the update of dS, and P at an anchor; Sa = the saved state of the chunk's segment
-    auto chunk = [&](const int c, const f32x4 (&Sa)[4]) __attribute__((always_inline)) {
+    f32x4 Sa[4];                           // the saved state of the segment at hand (chunks 2 sg, 2 sg + 1)
+
+    // Operands are fetched in batches, each issued as a whole before anything waits for it (the scheduling barriers keep
+    // the batches apart): a wave then waits for LDS a few times per chunk instead of once per product.
+    // X^T[j][t] = (S d1)^T GY^T + K'^T Bm^T for chunk c; S = Sa (even chunk) or one update of it (odd chunk)
+    auto part_x = [&](const int c) __attribute__((always_inline)) {
         const SlotG& O = S.slot[c % 3];
         const TilesG& Tl = S.tile[c & 1];
-        const float d1 = O.d1[j], d2 = O.d2[j], dec = O.dec[j];
-        {
-            f32x4 Sc[4];
-            if (c & 1) {
-                // state entering the odd chunk: one update of the saved state with the chunk below
-                const SlotG& Q = S.slot[(c - 1) % 3];
-                const float qdec = Q.dec[j], qd2 = Q.d2[j];
-                const bf16x8 kh = tr_pair(&Q.KpH[8 * g][8 * w], OS, l16), kl = tr_pair(&Q.KpL[8 * g][8 * w], OS, l16);
+        f32x4 Sc[4];
+        if (c & 1) {
+            // state entering the odd chunk: S dec + d2 V^T K' with the chunk below
+            const SlotG& Q = S.slot[(c - 1) % 3];
+            const float qdec = Q.dec[j], qd2 = Q.d2[j];
+            const bf16x8 qh = tr_pair(&Q.KpH[8 * g][8 * w], OS, l16), ql = tr_pair(&Q.KpL[8 * g][8 * w], OS, l16);
+            bf16x8 vop[4];
 #pragma unroll
-                for (int tl = 0; tl < 4; ++tl) {
-                    const bf16x8 vop = tr_pair(&Q.V[8 * g][8 * tl], OS, l16);
-                    f32x4 U = mfma(vop, kh, zero4);
-                    U = mfma(vop, kl, U);
+            for (int tl = 0; tl < 4; ++tl) vop[tl] = tr_pair(&Q.V[8 * g][8 * tl], OS, l16);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) Sc[tl][v] = fmaf(Sa[tl][v], qdec, qd2 * U[v]);
-                }
-            } else {
+            for (int tl = 0; tl < 4; ++tl) {
+                f32x4 U = mfma(vop[tl], qh, zero4);
+                U = mfma(vop[tl], ql, U);
 #pragma unroll
-                for (int tl = 0; tl < 4; ++tl) Sc[tl] = Sa[tl];
+                for (int v = 0; v < 4; ++v) Sc[tl][v] = fmaf(Sa[tl][v], qdec, qd2 * U[v]);
             }
-            // -------------------------------------------------------- X^T[j][t] = (S d1)^T GY^T + K'^T Bm^T
-            bf16x8 sh[2], sl[2];
-            split16(Sc, d1, sh, sl);
-            f32x4 X[2] = {zero4, zero4};
+        } else {
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    const bf16x8 gop = acc_order_op(&O.GY[16 * tt + l16][0], ks, g);
-                    X[tt] = mfma(sh[ks], gop, X[tt]);
-                    X[tt] = mfma(sl[ks], gop, X[tt]);
-                }
-            const bf16x8 kh = tr_pair(&O.KpH[8 * g][8 * w], OS, l16), kl = tr_pair(&O.KpL[8 * g][8 * w], OS, l16);
-#pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                const bf16x8 bh_ = lds_op(&Tl.BH[16 * tt + l16][4 * g]), bl_ = lds_op(&Tl.BL[16 * tt + l16][4 * g]);
-                X[tt] = mfma(kh, bh_, X[tt]);
-                X[tt] = mfma(kh, bl_, X[tt]);
-                X[tt] = mfma(kl, bh_, X[tt]);
-                *reinterpret_cast<float4*>(&S.xz[c & 1][0][16 * tt + l16][16 * w + 4 * g]) = make_float4(X[tt][0], X[tt][1], X[tt][2], X[tt][3]);
-            }
+            for (int tl = 0; tl < 4; ++tl) Sc[tl] = Sa[tl];
         }
-        // ------------------------------------------------------------ Z^T[j][s] = (dS d2)^T V^T + R'^T Bm
-        bf16x8 dh[2], dl[2];
-        split16(D, d2, dh, dl);
-        f32x4 Z[2] = {zero4, zero4};
+        __builtin_amdgcn_sched_barrier(0);
+        const float d1 = O.d1[j];
+        bf16x8 gop[2][2];
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                const bf16x8 vop = acc_order_op(&O.V[16 * tt + l16][0], ks, g);
-                Z[tt] = mfma(dh[ks], vop, Z[tt]);
-                Z[tt] = mfma(dl[ks], vop, Z[tt]);
+            for (int ks = 0; ks < 2; ++ks) gop[tt][ks] = acc_order_op(&O.GY[16 * tt + l16][0], ks, g);
+        const bf16x8 kh = tr_pair(&O.KpH[8 * g][8 * w], OS, l16), kl = tr_pair(&O.KpL[8 * g][8 * w], OS, l16);
+        bf16x8 bh_[2], bl_[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) { bh_[tt] = lds_op(&Tl.BH[16 * tt + l16][4 * g]); bl_[tt] = lds_op(&Tl.BL[16 * tt + l16][4 * g]); }
+        __builtin_amdgcn_sched_barrier(0);
+        bf16x8 sh[2], sl[2];
+        split16(Sc, d1, sh, sl);
+        f32x4 X[2] = {zero4, zero4};
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                X[tt] = mfma(sh[ks], gop[tt][ks], X[tt]);
+                X[tt] = mfma(sl[ks], gop[tt][ks], X[tt]);
             }
-        const bf16x8 rh = tr_pair(&O.RpH[8 * g][8 * w], OS, l16), rl = tr_pair(&O.RpL[8 * g][8 * w], OS, l16);
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt) {
-            const bf16x8 bh_ = tr_pair(&Tl.BH[8 * g][8 * tt], AS, l16), bl_ = tr_pair(&Tl.BL[8 * g][8 * tt], AS, l16);
-            Z[tt] = mfma(rh, bh_, Z[tt]);
-            Z[tt] = mfma(rh, bl_, Z[tt]);
-            Z[tt] = mfma(rl, bh_, Z[tt]);
-            *reinterpret_cast<float4*>(&S.xz[c & 1][1][16 * tt + l16][16 * w + 4 * g]) = make_float4(Z[tt][0], Z[tt][1], Z[tt][2], Z[tt][3]);
+            X[tt] = mfma(kh, bh_[tt], X[tt]);
+            X[tt] = mfma(kh, bl_[tt], X[tt]);
+            X[tt] = mfma(kl, bh_[tt], X[tt]);
         }
-        // ------------------------------------------------------------ dS <- dS dec + d1 GY^T R'
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+            *reinterpret_cast<float4*>(&S.xz[c & 1][0][16 * tt + l16][16 * w + 4 * g]) = make_float4(X[tt][0], X[tt][1], X[tt][2], X[tt][3]);
+    };
+    // Z^T[j][s] = (dS d2)^T V^T + R'^T Bm, then dS <- dS dec + d1 GY^T R'
+    auto part_z = [&](const int c) __attribute__((always_inline)) {
+        const SlotG& O = S.slot[c % 3];
+        const TilesG& Tl = S.tile[c & 1];
+        const float d1 = O.d1[j], d2 = O.d2[j], dec = O.dec[j];
+        bf16x8 vop[2][2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) vop[tt][ks] = acc_order_op(&O.V[16 * tt + l16][0], ks, g);
+        const bf16x8 rh = tr_pair(&O.RpH[8 * g][8 * w], OS, l16), rl = tr_pair(&O.RpL[8 * g][8 * w], OS, l16);
+        bf16x8 bh_[2], bl_[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) { bh_[tt] = tr_pair(&Tl.BH[8 * g][8 * tt], AS, l16); bl_[tt] = tr_pair(&Tl.BL[8 * g][8 * tt], AS, l16); }
+        __builtin_amdgcn_sched_barrier(0);
+        bf16x8 dh[2], dl[2];
+        split16(D, d2, dh, dl);
+        __builtin_amdgcn_sched_barrier(0);
+        bf16x8 gop[4];
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) gop[tl] = tr_pair(&O.GY[8 * g][8 * tl], OS, l16);
+        __builtin_amdgcn_sched_barrier(0);
+        f32x4 Z[2] = {zero4, zero4};
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                Z[tt] = mfma(dh[ks], vop[tt][ks], Z[tt]);
+                Z[tt] = mfma(dl[ks], vop[tt][ks], Z[tt]);
+            }
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            Z[tt] = mfma(rh, bh_[tt], Z[tt]);
+            Z[tt] = mfma(rh, bl_[tt], Z[tt]);
+            Z[tt] = mfma(rl, bh_[tt], Z[tt]);
+        }
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+            *reinterpret_cast<float4*>(&S.xz[c & 1][1][16 * tt + l16][16 * w + 4 * g]) = make_float4(Z[tt][0], Z[tt][1], Z[tt][2], Z[tt][3]);
 #pragma unroll
         for (int tl = 0; tl < 4; ++tl) {
-            const bf16x8 gop = tr_pair(&O.GY[8 * g][8 * tl], OS, l16);
-            f32x4 U = mfma(gop, rh, zero4);
-            U = mfma(gop, rl, U);
+            f32x4 U = mfma(gop[tl], rh, zero4);
+            U = mfma(gop[tl], rl, U);
 #pragma unroll
             for (int v = 0; v < 4; ++v) D[tl][v] = fmaf(D[tl][v], dec, d1 * U[v]);
         }
+    };
+
+    load_state(sv + static_cast<size_t>(nseg - 1) * (N * N), Sa, g);
+    __syncthreads();                       // iterations 0 and 1: nothing prepared yet
+    __syncthreads();
+#pragma unroll 1
+    for (int c = n - 1; c >= 0; --c) {
+        asm volatile("" : "+v"(g), "+v"(l16), "+v"(j));
+        // Sa of an odd chunk was asked for at the end of the last iteration: what does not need it goes first
+        part_z(c);
+        __builtin_amdgcn_sched_barrier(0);
+        part_x(c);
+        __builtin_amdgcn_sched_barrier(0);
         if (!(c & 1)) {
             // anchor: P = sum_i dS S with the saved state entering this chunk
             float p = 0.f;
@@ -413,28 +456,10 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
                 for (int v = 0; v < 4; ++v) p = fmaf(D[tl][v], Sa[tl][v], p);
             p = allreduce_rows(p);
             if (g == 0) S.pex[(c >> 1) & 1][j] = p;
+            // the next segment's state (index clamped: the load is issued on every path, so that waits can count it)
+            load_state(sv + static_cast<size_t>(c >= 2 ? (c >> 1) - 1 : 0) * (N * N), Sa, g);
         }
-    };
-    // a segment = an even chunk and the odd chunk above it, taken in reverse; one barrier per chunk
-    auto segment = [&](const int sg, const f32x4 (&Sa)[4]) __attribute__((always_inline)) {
-        if (2 * sg + 1 < n) { chunk(2 * sg + 1, Sa); __syncthreads(); }
-        chunk(2 * sg, Sa);
         __syncthreads();
-    };
-    // The saved states alternate between two register sets with fixed roles, each refilled as soon as its segment is
-    // done, two chunks before it is read again: no value that is still in flight is ever copied.
-    f32x4 SA[4], SB[4];
-    const int top = nseg - 1;
-    // (every refill is issued on every path, with the segment index clamped, so that the waits can count them)
-    load_state(sv + static_cast<size_t>(top) * (N * N), SA, g);
-    load_state(sv + static_cast<size_t>(top >= 1 ? top - 1 : 0) * (N * N), SB, g);
-    __syncthreads();                       // iterations 0 and 1: nothing prepared yet
-    __syncthreads();
-    for (int sg = top; sg >= 0; sg -= 2) {
-        segment(sg, SA);
-        load_state(sv + static_cast<size_t>(sg >= 2 ? sg - 2 : 0) * (N * N), SA, g);
-        if (sg >= 1) segment(sg - 1, SB);
-        load_state(sv + static_cast<size_t>(sg >= 3 ? sg - 3 : 0) * (N * N), SB, g);
     }
     __syncthreads();                       // iteration n + 2: the P waves finish chunk 0
     if (a.gs != nullptr) {
@@ -448,7 +473,7 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
 // ---------------------------------------------------------------------------------------------------- EW waves
 template <int WMODE>
 DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int n) {
-    const int g = lane >> 4, l16 = lane & 15;
+    int g = lane >> 4, l16 = lane & 15;    // redefined behind an empty asm in every iteration, see role_sd
     const int T = a.T, C = a.C;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     f32x4 E[4] = {zero4, zero4, zero4, zero4};     // dS[i = 16w + l16][j = 16 tile + 4g + v]
@@ -459,20 +484,25 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
         TilesG& Tl = S.tile[c & 1];
         const int ta = (w == 0) ? 0 : 1, tb = (w == 2) ? 1 : 0;
         f32x4 a0 = zero4, a1 = zero4, bm = zero4;
+        bf16x8 kh[2], kl[2], rh[2], rl[2], vo[2], go[2];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            const bf16x8 kh = lds_op(&O.KpH[16 * tb + l16][16 * ks + 4 * g]), kl = lds_op(&O.KpL[16 * tb + l16][16 * ks + 4 * g]);
-            const bf16x8 rh = lds_op(&O.RpH[16 * ta + l16][16 * ks + 4 * g]), rl = lds_op(&O.RpL[16 * ta + l16][16 * ks + 4 * g]);
-            const bf16x8 vo = lds_op(&O.V[16 * tb + l16][16 * ks + 4 * g]), go = lds_op(&O.GY[16 * ta + l16][16 * ks + 4 * g]);
-            a0 = mfma(kh, rh, a0);
-            a1 = mfma(kh, rl, a1);
-            a1 = mfma(kl, rh, a1);
-            bm = mfma(vo, go, bm);
+            kh[ks] = lds_op(&O.KpH[16 * tb + l16][16 * ks + 4 * g]); kl[ks] = lds_op(&O.KpL[16 * tb + l16][16 * ks + 4 * g]);
+            rh[ks] = lds_op(&O.RpH[16 * ta + l16][16 * ks + 4 * g]); rl[ks] = lds_op(&O.RpL[16 * ta + l16][16 * ks + 4 * g]);
+            vo[ks] = lds_op(&O.V[16 * tb + l16][16 * ks + 4 * g]); go[ks] = lds_op(&O.GY[16 * ta + l16][16 * ks + 4 * g]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            a0 = mfma(kh[ks], rh[ks], a0);
+            a1 = mfma(kh[ks], rl[ks], a1);
+            a1 = mfma(kl[ks], rh[ks], a1);
+            bm = mfma(vo[ks], go[ks], bm);
         }
         f32x4 am = a0 + a1;                                    // [v]: s = 16 tb + 4g + v, t = 16 ta + l16
         if (ta == tb) {
             const int t = 16 * ta + l16;
-            const float d = (O.ruk[0][t] + O.ruk[1][t]) + (O.ruk[2][t] + O.ruk[3][t]);
+            const float d = ((O.ruk[0][t] + O.ruk[1][t]) + (O.ruk[2][t] + O.ruk[3][t])) + ((O.ruk[4][t] + O.ruk[5][t]) + (O.ruk[6][t] + O.ruk[7][t]));
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int sl = 4 * g + v;
@@ -488,38 +518,77 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
         *reinterpret_cast<uint2*>(&Tl.BL[16 * ta + l16][8 * tb + 2 * g]) = make_uint2(y0.l, y1.l);
     };
 
+#pragma unroll 1
     for (int it = 0; it <= n + 2; ++it) {
         const int c = n + 1 - it;
+        asm volatile("" : "+v"(g), "+v"(l16));
         if (it >= 2 && c >= 0) {
             const SlotG& O = S.slot[c % 3];
             const TilesG& Tl = S.tile[c & 1];
+            // Operands are fetched in batches, each issued as a whole before anything waits for it (the scheduling barriers
+            // keep the batches apart): a wave then waits for LDS three times per chunk instead of once per product.
+            // ------------------------------------------------------------ batch 1: d2 and K' (natural rows)
+            float4 dq[4];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                dq[2 * ks] = *reinterpret_cast<const float4*>(&O.d2[32 * ks + 4 * g]);
+                dq[2 * ks + 1] = *reinterpret_cast<const float4*>(&O.d2[32 * ks + 16 + 4 * g]);
+            }
+            bf16x8 kh[2][2], kl[2][2];
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    kh[tt][ks] = acc_order_op(&O.KpH[16 * tt + l16][0], ks, g);
+                    kl[tt][ks] = acc_order_op(&O.KpL[16 * tt + l16][0], ks, g);
+                }
+            __builtin_amdgcn_sched_barrier(0);
             // ------------------------------------------------------------ gv^T[i][s] = (dS d2) K'^T + GY^T A
             bf16x8 dh[2], dl[2];
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
-                const float4 p = *reinterpret_cast<const float4*>(&O.d2[32 * ks + 4 * g]);
-                const float4 q = *reinterpret_cast<const float4*>(&O.d2[32 * ks + 16 + 4 * g]);
+                const float4 p = dq[2 * ks], q = dq[2 * ks + 1];
                 const HL x0 = hilo2(E[2 * ks][0] * p.x, E[2 * ks][1] * p.y), x1 = hilo2(E[2 * ks][2] * p.z, E[2 * ks][3] * p.w);
                 const HL x2 = hilo2(E[2 * ks + 1][0] * q.x, E[2 * ks + 1][1] * q.y), x3 = hilo2(E[2 * ks + 1][2] * q.z, E[2 * ks + 1][3] * q.w);
                 dh[ks] = as_op(x0.h, x1.h, x2.h, x3.h);
                 dl[ks] = as_op(x0.l, x1.l, x2.l, x3.l);
             }
+            __builtin_amdgcn_sched_barrier(0);
+            // ------------------------------------------------------------ batch 2: gy and the A tile with the tokens along K
+            const bf16x8 gyo = tr_pair(&O.GY[8 * g][8 * w], OS, l16);       // lane = value channel 16w + l16, K = tokens
+            bf16x8 ah[2], al[2];
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) { ah[tt] = tr_pair(&Tl.AH[8 * g][8 * tt], AS, l16); al[tt] = tr_pair(&Tl.AL[8 * g][8 * tt], AS, l16); }
+            __builtin_amdgcn_sched_barrier(0);
             f32x4 G[2] = {zero4, zero4};
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
+            for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    const bf16x8 kh = acc_order_op(&O.KpH[16 * tt + l16][0], ks, g), kl = acc_order_op(&O.KpL[16 * tt + l16][0], ks, g);
-                    G[tt] = mfma(dh[ks], kh, G[tt]);
-                    G[tt] = mfma(dh[ks], kl, G[tt]);
-                    G[tt] = mfma(dl[ks], kh, G[tt]);
+                for (int tt = 0; tt < 2; ++tt) {
+                    G[tt] = mfma(dh[ks], kh[tt][ks], G[tt]);
+                    G[tt] = mfma(dh[ks], kl[tt][ks], G[tt]);
+                    G[tt] = mfma(dl[ks], kh[tt][ks], G[tt]);
                 }
-            const bf16x8 gyo = tr_pair(&O.GY[8 * g][8 * w], OS, l16);       // lane = value channel 16w + l16, K = tokens
+            __builtin_amdgcn_sched_barrier(0);
+            // ------------------------------------------------------------ batch 3: R' with the tokens along K, dec, d1
+            bf16x8 rh[4], rl[4];
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) { rh[tl] = tr_pair(&O.RpH[8 * g][8 * tl], OS, l16); rl[tl] = tr_pair(&O.RpL[8 * g][8 * tl], OS, l16); }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
-                const bf16x8 ah = tr_pair(&Tl.AH[8 * g][8 * tt], AS, l16), al = tr_pair(&Tl.AL[8 * g][8 * tt], AS, l16);
-                G[tt] = mfma(gyo, ah, G[tt]);
-                G[tt] = mfma(gyo, al, G[tt]);
+                G[tt] = mfma(gyo, ah[tt], G[tt]);
+                G[tt] = mfma(gyo, al[tt], G[tt]);
+            }
+            f32x4 U[4];
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) {
+                U[tl] = mfma(rh[tl], gyo, zero4);
+                U[tl] = mfma(rl[tl], gyo, U[tl]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
                 const int tg = c * L + 16 * tt + l16;
                 if (tg < T)
                     *reinterpret_cast<uint2*>(a.gv + base + static_cast<size_t>(tg) * C + 16 * w + 4 * g) =
@@ -528,15 +597,13 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
             // ------------------------------------------------------------ dS^T <- dS^T dec + d1 R'^T GY
 #pragma unroll
             for (int tl = 0; tl < 4; ++tl) {
-                const bf16x8 rh = tr_pair(&O.RpH[8 * g][8 * tl], OS, l16), rl = tr_pair(&O.RpL[8 * g][8 * tl], OS, l16);
-                f32x4 U = mfma(rh, gyo, zero4);
-                U = mfma(rl, gyo, U);
                 const float4 de = *reinterpret_cast<const float4*>(&O.dec[16 * tl + 4 * g]);
                 const float4 d1 = *reinterpret_cast<const float4*>(&O.d1[16 * tl + 4 * g]);
-                E[tl][0] = fmaf(E[tl][0], de.x, d1.x * U[0]); E[tl][1] = fmaf(E[tl][1], de.y, d1.y * U[1]);
-                E[tl][2] = fmaf(E[tl][2], de.z, d1.z * U[2]); E[tl][3] = fmaf(E[tl][3], de.w, d1.w * U[3]);
+                E[tl][0] = fmaf(E[tl][0], de.x, d1.x * U[tl][0]); E[tl][1] = fmaf(E[tl][1], de.y, d1.y * U[tl][1]);
+                E[tl][2] = fmaf(E[tl][2], de.z, d1.z * U[tl][2]); E[tl][3] = fmaf(E[tl][3], de.w, d1.w * U[tl][3]);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
         if (it >= 1 && c - 1 >= 0 && w < 3) tiles(c - 1);
         __syncthreads();
     }
@@ -554,8 +621,8 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG a) {
     for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTG) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
-    if (wid < 4) role_prep<WMODE>(S, a, lane, w, base, h, bh, n);
-    else if (wid < 8) role_sd<WMODE>(S, a, lane, w, bh, n);
+    if (wid < 8) role_prep<WMODE>(S, a, lane, wid, base, h, bh, n);
+    else if (wid < 12) role_sd<WMODE>(S, a, lane, w, bh, n);
     else role_e<WMODE>(S, a, lane, w, base, n);
 }
 

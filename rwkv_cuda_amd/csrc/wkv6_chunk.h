@@ -75,14 +75,14 @@ struct ArgsB {
     // SPLIT kernels only (see below)
     int cross;
     float *gr32, *gk32, *gv32, *gw32, *gu32;
-    // when not null: [B*H][4]; a workgroup runs only if one of its four words is not zero (the (batch, head) pairs that
+    // when not null: [B*H][8]; a workgroup runs only if one of its eight words is not zero (the (batch, head) pairs that
     // the one-sweep backward has handed back)
     const int* only_flagged;
 };
 DEVINL bool skip_unflagged(const int* f, const int bh) {
     if (f == nullptr) return false;
-    const int4 x = *reinterpret_cast<const int4*>(f + 4 * bh);
-    return (x.x | x.y | x.z | x.w) == 0;
+    const int4 x = *reinterpret_cast<const int4*>(f + 8 * bh), y = *reinterpret_cast<const int4*>(f + 8 * bh + 4);
+    return (x.x | x.y | x.z | x.w | y.x | y.y | y.z | y.w) == 0;
 }
 
 // A head of 128 channels as four heads of 64 (SPLIT = true, wkv5 only).  With the key channels j and the value channels
