@@ -58,6 +58,7 @@ struct alignas(16) SmemG {
 static_assert(sizeof(SmemG) <= 160 * 1024, "LDS");
 
 typedef short v4s __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef v4s __attribute__((address_space(3))) * lds_v4s_ptr;
 
 // Operand with the rows of an LDS matrix along K: slot (g, e) <-> row row0 + e (e = 0..7), lane l16 <-> column col + l16.
@@ -120,45 +121,47 @@ DEVINL void load_state(const float* __restrict__ p, f32x4 (&x)[4], const int g) 
 // wave w (0..7): channels 8w..8w+7; lane = 16 * (channel pair) + token: a thread has two channels of tokens tp and tp + 16
 template <int WMODE>
 DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n) {
-    const int jq = lane >> 4, tp = lane & 15, ch = 8 * w + 2 * jq, cd = 4 * w + jq;      // cd: dword column of the pair in a bf16 plane
+    // jq, tp (and hl, rw below) are redefined behind an empty asm in every iteration, see role_sd
+    int jq = lane >> 4, tp = lane & 15;
+    const int ch0 = 8 * w + 2 * (lane >> 4);
     const int T = a.T, C = a.C;
-    // wave-uniform bases plus one 32-bit per-lane offset: the addresses stay out of the vector registers
-    const uint16_t* __restrict__ rb = a.r + base;
-    const uint16_t* __restrict__ kb = a.k + base;
-    const uint16_t* __restrict__ vb = a.v + base;
-    const uint16_t* __restrict__ gb = a.gy + base;
-    const uint16_t* __restrict__ wb = static_cast<const uint16_t*>(a.w) + base;
+    // Global memory is touched in another lane order than the arithmetic: a lane moves one 16-byte row piece (this wave's
+    // 8 channels of one token) of one tensor, so that a wave needs three loads and two stores per chunk instead of
+    // sixteen four-byte accesses to sixteen rows each.  The pieces cross to the arithmetic's lane order (and back)
+    // through this wave's own columns of LDS arrays that are free at that moment: the planes of the slot being
+    // prepared on the way in, the X / Z cells just consumed on the way out.  Only this wave touches those columns and
+    // LDS serves a wave's accesses in order, so no barrier is involved.
+    int hl = lane >> 5, rw = lane & 31;
+    const int hl0 = lane >> 5;
+    const uint16_t* __restrict__ pA = (hl0 ? a.k : a.r) + base + 8 * w;                                  // r | k
+    const uint16_t* __restrict__ pB = (hl0 ? a.v : static_cast<const uint16_t*>(a.w)) + base + 8 * w;   // w | v
+    const uint16_t* __restrict__ pC = a.gy + base + 8 * w;                                               // gy (both halves)
+    uint16_t* __restrict__ pS1 = (hl0 ? a.gk : a.gr) + base + 8 * w;                                     // gr | gk
+    uint16_t* __restrict__ pS2 = a.gw + base + 8 * w;                                                    // gw (first half)
     float uj[2];
     {
-        const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + ch);
+        const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + ch0);
         uj[0] = bf_lo(x); uj[1] = bf_hi(x);
     }
-    // r, k, w are needed by the arithmetic of a preparation and are fetched two chunks ahead; v, gy are only copied
-    // into their planes and are fetched one chunk ahead
-    struct Raw { uint32_t r[2], k[2], w[2]; };
-    struct RawVG { uint32_t v[2], g[2]; };
-    Raw ring[2];
-    RawVG vgn;
-    auto row_of = [&](const int c, const int e) __attribute__((always_inline)) {
-        const int t = c * L + tp + 16 * e;
-        return static_cast<uint32_t>(t < T ? t : T - 1) * C + ch;
-    };
+    struct Raw { u32x4 a, b, c; };
+    Raw ring[2];                           // two chunks ahead
     auto fetch = [&](const int c, Raw& x) __attribute__((always_inline)) {
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const uint32_t o = row_of(c, e);
-            x.r[e] = *reinterpret_cast<const uint32_t*>(rb + o);
-            x.k[e] = *reinterpret_cast<const uint32_t*>(kb + o);
-            x.w[e] = *reinterpret_cast<const uint32_t*>(wb + o);
-        }
+        const int t = c * L + rw;
+        const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C;
+        x.a = *reinterpret_cast<const u32x4*>(pA + o);
+        x.b = *reinterpret_cast<const u32x4*>(pB + o);
+        x.c = *reinterpret_cast<const u32x4*>(pC + o);
     };
-    auto fetch_vg = [&](const int c, RawVG& x) __attribute__((always_inline)) {
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const uint32_t o = row_of(c, e);
-            x.v[e] = *reinterpret_cast<const uint32_t*>(vb + o);
-            x.g[e] = *reinterpret_cast<const uint32_t*>(gb + o);
-        }
+    // the pieces of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v and gy in place
+    auto stage_in = [&](const int c, const Raw& x, auto PARTIAL) __attribute__((always_inline)) {
+        SlotG& O = S.slot[c % 3];
+        const bool live = !decltype(PARTIAL)::value || c * L + rw < T;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        uint32_t* da = &O.RpH[rw][4 * w] + hl * (2 * L * OS);        // R' hi | K' hi
+        uint32_t* db = &O.RpL[rw][4 * w] + hl * (3 * L * OS);        // R' lo | V
+        *reinterpret_cast<u32x4*>(da) = live ? x.a : zero;
+        *reinterpret_cast<u32x4*>(db) = (live || !hl) ? x.b : zero;  // w of a dead row is masked where the decay is formed
+        if (!hl) *reinterpret_cast<u32x4*>(&O.GY[rw][4 * w]) = live ? x.c : zero;
     };
     // what the finishing of a chunk needs from its preparation, three iterations earlier
     struct Held { uint32_t r[2], k[2]; float cc[2][2]; };
@@ -167,30 +170,21 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     float carry[2] = {0.f, 0.f}, gu_acc[2] = {0.f, 0.f};
     // Only the last chunk of the sequence can be cut short (PARTIAL): its rows past T carry no input and no decay.
 
-    // v, gy of chunk c into their planes.  This comes first in an iteration: the loads it waits for are then older than
-    // everything else in flight except the r, k, w of the next chunk, which the wait can count.
-    auto copy_vg = [&](const int c, const RawVG& y, auto PARTIAL) __attribute__((always_inline)) {
-        SlotG& O = S.slot[c % 3];
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const bool live = !decltype(PARTIAL)::value || c * L + tp + 16 * e < T;
-            O.V[tp + 16 * e][cd] = live ? y.v[e] : 0u;
-            O.GY[tp + 16 * e][cd] = live ? y.g[e] : 0u;
-        }
-    };
-
-    auto prep = [&](const int c, Raw& x, Held& hd, auto PARTIAL) __attribute__((always_inline)) {
+    auto prep = [&](const int c, Held& hd, auto PARTIAL) __attribute__((always_inline)) {
+        const int ch = 8 * w + 2 * jq, cd = 4 * w + jq;        // cd: dword column of the pair in a bf16 plane
         SlotG& O = S.slot[c % 3];
         float lam[2][2], rf[2][2], kf[2][2];
+        uint32_t xr[2], xk[2], xw[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) { xr[e] = O.RpH[tp + 16 * e][cd]; xk[e] = O.KpH[tp + 16 * e][cd]; xw[e] = O.RpL[tp + 16 * e][cd]; }
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const bool live = !decltype(PARTIAL)::value || c * L + tp + 16 * e < T;
-            if (!live) { x.r[e] = 0u; x.k[e] = 0u; }
-            rf[e][0] = bf_lo(x.r[e]); rf[e][1] = bf_hi(x.r[e]);
-            kf[e][0] = bf_lo(x.k[e]); kf[e][1] = bf_hi(x.k[e]);
-            lam[e][0] = live ? -LOG2E * exp2_fast(LOG2E * bf_lo(x.w[e])) : 0.f;
-            lam[e][1] = live ? -LOG2E * exp2_fast(LOG2E * bf_hi(x.w[e])) : 0.f;
-            hd.r[e] = x.r[e]; hd.k[e] = x.k[e];
+            rf[e][0] = bf_lo(xr[e]); rf[e][1] = bf_hi(xr[e]);
+            kf[e][0] = bf_lo(xk[e]); kf[e][1] = bf_hi(xk[e]);
+            lam[e][0] = live ? -LOG2E * exp2_fast(LOG2E * bf_lo(xw[e])) : 0.f;
+            lam[e][1] = live ? -LOG2E * exp2_fast(LOG2E * bf_hi(xw[e])) : 0.f;
+            hd.r[e] = xr[e]; hd.k[e] = xk[e];
         }
         float l1[2], l2[2];
 #pragma unroll
@@ -230,6 +224,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
 
     // gr, gk, gw of chunk c from X, Z (left by the SD waves in the last iteration) and what prep kept
     auto finish = [&](const int c, const Held& hd, auto PARTIAL) __attribute__((always_inline)) {
+        const int ch = 8 * w + 2 * jq;
         const float2 e2 = *reinterpret_cast<const float2*>(&S.slot[c % 3].l2[ch]);
         const float l2v[2] = {e2.x, e2.y};
         float q[2][2], kdk[2][2], lam[2][2];
@@ -256,11 +251,9 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
                 gu_acc[z] = fmaf(rf[z] * kf[z], vg, gu_acc[z]);
                 lam[e][z] = gw_factor((ccn - cc) * LN2);
             }
-            if (!decltype(PARTIAL)::value || tg < T) {
-                const uint32_t o = static_cast<uint32_t>(tg) * C + ch;
-                *reinterpret_cast<uint32_t*>(a.gr + base + o) = pack_bf2(gr[0], gr[1]);
-                *reinterpret_cast<uint32_t*>(a.gk + base + o) = pack_bf2(gk[0], gk[1]);
-            }
+            // X and Z of this thread are in registers: their cells now carry the results to the lanes that store them
+            reinterpret_cast<uint32_t*>(&S.xz[c & 1][0][t][8 * w])[jq] = pack_bf2(gr[0], gr[1]);
+            reinterpret_cast<uint32_t*>(&S.xz[c & 1][0][t][8 * w + 4])[jq] = pack_bf2(gk[0], gk[1]);
         }
         float gw[2][2];
 #pragma unroll
@@ -277,17 +270,21 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             carry[0] = p2.x; carry[1] = p2.y;
         }
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const int tg = c * L + tp + 16 * e;
-            if (!decltype(PARTIAL)::value || tg < T)
-                *reinterpret_cast<uint32_t*>(a.gw + base + (static_cast<uint32_t>(tg) * C + ch)) = pack_bf2(gw[e][0], gw[e][1]);
+        for (int e = 0; e < 2; ++e) reinterpret_cast<uint32_t*>(&S.xz[c & 1][1][tp + 16 * e][8 * w])[jq] = pack_bf2(gw[e][0], gw[e][1]);
+        // one 16-byte row piece per lane: gr | gk, then gw
+        const u32x4 o1 = *reinterpret_cast<const u32x4*>(&S.xz[c & 1][0][rw][8 * w + 4 * hl]);
+        const u32x4 o2 = *reinterpret_cast<const u32x4*>(&S.xz[c & 1][1][rw][8 * w]);
+        const int tg = c * L + rw;
+        if (!decltype(PARTIAL)::value || tg < T) {
+            const uint32_t o = static_cast<uint32_t>(tg) * C;
+            *reinterpret_cast<u32x4*>(pS1 + o) = o1;
+            if (!hl) *reinterpret_cast<u32x4*>(pS2 + o) = o2;
         }
     };
 
     const bool cut = (T % L) != 0;         // the last chunk is cut short
     const std::true_type part{};
     const std::false_type full{};
-    fetch_vg(n - 1, vgn);
     fetch(n - 1, ring[0]);
     fetch(n >= 2 ? n - 2 : 0, ring[1]);
     for (int it0 = 0; it0 <= n + 2; it0 += 2)
@@ -296,17 +293,17 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             const int it = it0 + z;
             if (it <= n + 2) {
                 const int cp = n - 1 - it;
-                // The same loads in every iteration (chunk index clamped): the wait for a chunk's registers is then the
-                // count of loads issued after them on every path, and never has to cover the newest ones.
-                if (cp >= 0) { if (cut && it == 0) copy_vg(cp, vgn, part); else copy_vg(cp, vgn, full); }
-                fetch_vg(cp >= 1 ? cp - 1 : 0, vgn);
+                asm volatile("" : "+v"(jq), "+v"(tp), "+v"(hl), "+v"(rw));
+                // The same three loads in every iteration (chunk index clamped): the wait for a chunk's registers is then
+                // the count of loads issued after them on every path, and never has to cover the newest ones.
+                if (cp >= 0) { if (cut && it == 0) stage_in(cp, ring[z], part); else stage_in(cp, ring[z], full); }
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(cp >= 2 ? cp - 2 : 0, ring[z]);
                 __builtin_amdgcn_sched_barrier(0);
                 if (it >= 3) { if (cut && it == 3) finish(cp + 3, hq[2], part); else finish(cp + 3, hq[2], full); }
                 __builtin_amdgcn_sched_barrier(0);
                 hq[2] = hq[1]; hq[1] = hq[0];
-                if (cp >= 0) { if (cut && it == 0) prep(cp, ring[z], hq[0], part); else prep(cp, ring[z], hq[0], full); }
-                __builtin_amdgcn_sched_barrier(0);
-                fetch(cp >= 2 ? cp - 2 : 0, ring[z]);
+                if (cp >= 0) { if (cut && it == 0) prep(cp, hq[0], part); else prep(cp, hq[0], full); }
                 __syncthreads();
             }
         });
@@ -314,7 +311,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     // gu of this batch row: sum over the tokens (lanes of a row)
 #pragma unroll
     for (int z = 0; z < 2; ++z) gu_acc[z] = row_sum_to_last(gu_acc[z]);
-    if (tp == 15) *reinterpret_cast<uint32_t*>(a.gu + bh * N + ch) = pack_bf2(gu_acc[0], gu_acc[1]);
+    if (tp == 15) *reinterpret_cast<uint32_t*>(a.gu + bh * N + ch0) = pack_bf2(gu_acc[0], gu_acc[1]);
 }
 
 // ---------------------------------------------------------------------------------------------------- SD waves
