@@ -37,11 +37,9 @@ FLAGS = 0                      # RWKV_FLAG_SWEEPS when --algo sweeps: passed per
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see profiles/), keyed
 # by kernel label at the headline shape; None = not measured for the current kernels.
 TRAFFIC_MEASURED = {
-    # profiles/wkv6_ws_kernels_B8_T4096_C2048.md  (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB)
-    "wkv6_fwd_ws": 537e6 + 134e6,
-    "wkv6_bwd_a_ws": 683e6 + 432e6,
-    "wkv6_bwd_b_ws": 990e6 + 403e6,
-    "wkv6state forward": 537e6 + 134e6, "wkv6state backward (3 kernels)": 683e6 + 432e6 + 990e6 + 403e6,
+    # profiles/wkv6_fused_kernels_B8_T4096_C2048.md  (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB)
+    "wkv6_fwd_ws (keeps states)": 537.2e6 + 402.7e6,
+    "wkv6_bwd_fused (+ gu batch sum)": 940.4e6 + 537.0e6,
     # profiles/wkv5_ws_kernels_B8_T4096_C2048.md
     "wkv6_fwd_ws<head decay>": 403e6 + 134e6,
     "wkv6_bwd_a_ws<head decay>": 548e6 + 533e6,
@@ -102,44 +100,41 @@ def make_wkv6(dev, state):
     new = lambda *s: torch.empty(s, device=dev, dtype=bf)
     y, gr, gk, gv, gw, gu = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C), new(B, C)
     gu_sum = new(H, N)
-    nbytes = lib.rwkv_wkv6f_backward_workspace_bytes(B, T, C, H)
+    nbytes = lib.rwkv_wkv6f_backward_saved_workspace_bytes(B, T, C, H)
     ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+    nsaved = lib.rwkv_wkv6f_saved_bytes(B, T, C, H)
+    saved = torch.empty(nsaved, device=dev, dtype=torch.uint8)   # the states the forward hands to the backward
     tok = B * T
-    if state:
-        gs = new(B, H, N, N)
+    gs = new(B, H, N, N) if state else None
+    name = "wkv6_state" if state else "wkv6"
+    # what WKV_6 / WKV_6STATE.forward and backward do: raw bf16 decay straight into the kernels, the forward keeps the state
+    # entering every 64th token, the backward is one reverse sweep, and the wrapper's torch.sum(gu, 0) (wkv6/run.py:169,
+    # wkv6_state/run.py:123) runs inside the library
+    fwd = lambda: call("rwkv_wkv6f_forward", dev, B, T, C, H, r, k, v, w, u, s0, y, saved, nsaved, FLAGS)
+    bwd_all = lambda: call("rwkv_wkv6f_backward_saved", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu_sum, gs,
+                           saved, nsaved, ws, nbytes, FLAGS)
 
-        def step():
-            # what WKV_6STATE.forward / backward do; the wrapper's torch.sum(gu, 0) (wkv6_state/run.py:123) runs inside the library
-            call("rwkv_wkv6state_forward_ex", dev, B, T, C, H, r, k, v, w, u, s0, y, FLAGS)
-            call("rwkv_wkv6f_backward", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu_sum, gs, ws, nbytes, FLAGS)
+    def step():
+        fwd()
+        bwd_all()
 
-        kernels = [("wkv6state forward", lambda: call("rwkv_wkv6state_forward_ex", dev, B, T, C, H, r, k, v, w, u, s0, y, FLAGS), 10 * C * tok),
-                   ("wkv6state backward (3 kernels)", lambda: call("rwkv_wkv6state_backward_ex", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes, FLAGS), 18 * C * tok)]
-        name = "wkv6_state"
-    else:
-        def step():
-            # what WKV_6.forward / backward do: raw bf16 decay straight into the kernels; the wrapper's torch.sum(gu, 0)
-            # (wkv6/run.py:169) runs inside the library (one small kernel after the two sweeps)
-            call("rwkv_wkv6raw_forward_ex", dev, B, T, C, H, r, k, v, w, u, y, FLAGS)
-            call("rwkv_wkv6f_backward", dev, B, T, C, H, r, k, v, w, u, None, gy, gr, gk, gv, gw, gu_sum, None, ws, nbytes, FLAGS)
-
-        def bwd(mask):
-            def run():
+    def bwd(mask):
+        def run():
+            if state:
+                call("rwkv_wkv6state_backward_ex", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, ws, nbytes, mask | FLAGS)
+            else:
                 call("rwkv_wkv6raw_backward_ex", dev, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, nbytes, mask | FLAGS)
-            return run
+        return run
 
-        # algorithmic bytes per kernel: tensors it must read once + outputs it must write once, 2 B per element
-        fwd = lambda: call("rwkv_wkv6raw_forward_ex", dev, B, T, C, H, r, k, v, w, u, y, FLAGS)
-        if ALGO == "chunked":
-            kernels = [("wkv6_fwd_ws", fwd, 10 * C * tok),                    # r k v w -> y
-                       ("wkv6_bwd_a_ws", bwd(1), 12 * C * tok),               # r k v w gy -> gr (+ fp32 workspace)
-                       ("wkv6_bwd_b_ws", bwd(4), 16 * C * tok)]               # r k v w gy -> gk gv gw
-        else:
-            kernels = [("wkv_sweep<FWD>", fwd, 10 * C * tok),
-                       ("wkv_sweep<GR>", bwd(1), 12 * C * tok),               # r k v w gy -> gr
-                       ("wkv_sweep<GV>", bwd(2), 10 * C * tok),               # r k w gy -> gv
-                       ("wkv_sweep<GK>", bwd(4), 14 * C * tok)]               # r k v w gy -> gk gw
-        name = "wkv6"
+    # algorithmic bytes per kernel: tensors it must read once + outputs it must write once, 2 B per element
+    if ALGO == "chunked":
+        kernels = [("wkv6_fwd_ws (keeps states)", fwd, 10 * C * tok),                      # r k v w -> y
+                   ("wkv6_bwd_fused (+ gu batch sum)", bwd_all, 18 * C * tok)]              # r k v w gy -> gr gk gv gw
+    else:
+        kernels = [("wkv_sweep<FWD>", fwd, 10 * C * tok),
+                   ("wkv_sweep<GR>", bwd(1), 12 * C * tok),               # r k v w gy -> gr
+                   ("wkv_sweep<GV>", bwd(2), 10 * C * tok),               # r k w gy -> gv
+                   ("wkv_sweep<GK>", bwd(4), 14 * C * tok)]               # r k v w gy -> gk gw
 
     def cpu_baseline(t_cpu=256):
         from oracle import wkv56 as O
@@ -524,10 +519,12 @@ def main():
     dst = torch.empty_like(src)
     copy_ms = time_gpu(lambda: dst.copy_(src), 10, 3)
     copy_gbps = 2 * src.numel() * 4 / (copy_ms * 1e-3) / 1e9
-    # the same 1 GiB as a read-only stream (a sum reduction: 1 GiB in, a few KB out) and as a write-only stream (a fill):
+    # the same 1 GiB as a read-only stream and as a write-only stream (rwkv_hbm_probe: 16 bytes per lane, grid-stride):
     # a kernel that mostly reads is priced against the first, one that mostly writes against the second
-    read_ms = time_gpu(lambda: torch.sum(src), 10, 3)
-    write_ms = time_gpu(lambda: dst.fill_(1.0), 10, 3)
+    from rwkv_cuda_amd._call import call as _call
+    nb = src.numel() * 4
+    read_ms = time_gpu(lambda: _call("rwkv_hbm_probe", dev, 0, src, dst, nb), 10, 3)
+    write_ms = time_gpu(lambda: _call("rwkv_hbm_probe", dev, 1, None, dst, nb), 10, 3)
     read_gbps = src.numel() * 4 / (read_ms * 1e-3) / 1e9
     write_gbps = src.numel() * 4 / (write_ms * 1e-3) / 1e9
     del src, dst

@@ -51,6 +51,11 @@ int rwkv_last_hip_error(void);
 /* ABI version of this header (bumped when a signature changes). */
 int rwkv_abi_version(void);
 
+/* A measuring aid (no counterpart in the reference): one pass over `bytes` of device memory as a read-only stream
+ * (mode 0: src is read, 16 bytes of dst may be written), a write-only stream (mode 1: dst) or a copy (mode 2), so that a
+ * benchmark can price kernels against what the memory system delivers for reads and for writes. */
+int rwkv_hbm_probe(void* stream, int mode, const void* src, void* dst, size_t bytes);
+
 /* Per-call options of the *_ex entry points below (no counterpart in the reference).  Every *_ex function is its
  * reference-signature sibling plus a trailing `flags` word; the sibling is the same call with flags = 0.  Nothing here is
  * process-wide: two threads may run different algorithms or pass subsets at the same time.

@@ -113,6 +113,7 @@ SIGNATURES = {
     "rwkv_strerror": (ctypes.c_char_p, [_I]),
     "rwkv_last_hip_error": (_I, []),
     "rwkv_abi_version": (_I, []),
+    "rwkv_hbm_probe": (_I, [_P, _I, _P, _P, _Z]),
     "rwkv_wkv4_forward": (_I, [_P, _I, _I, _I] + [_P] * 5),
     "rwkv_wkv4_backward_workspace_bytes": (_Z, [_I, _I, _I]),
     "rwkv_wkv4_backward": (_I, [_P, _I, _I, _I] + [_P] * 9 + [_P, _Z]),

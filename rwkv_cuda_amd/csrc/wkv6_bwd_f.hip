@@ -269,6 +269,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             const float2 p2 = *reinterpret_cast<const float2*>(&S.pex[(c >> 1) & 1][ch]);
             carry[0] = p2.x; carry[1] = p2.y;
         }
+        // without an initial state nothing has been accumulated before token 0: its decay has no effect at all
+        if (a.gs == nullptr && c == 0 && tp == 0) { gw[0][0] = 0.f; gw[0][1] = 0.f; }
 #pragma unroll
         for (int e = 0; e < 2; ++e) reinterpret_cast<uint32_t*>(&S.xz[c & 1][1][tp + 16 * e][8 * w])[jq] = pack_bf2(gw[e][0], gw[e][1]);
         // one 16-byte row piece per lane: gr | gk, then gw

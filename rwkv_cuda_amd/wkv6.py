@@ -23,24 +23,29 @@ class WKV_6(torch.autograd.Function):
             require(r.numel() == B * T * C, "shape mismatch")
             ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
             ctx.flags = options.current_flags()
-            ctx.save_for_backward(r, k, v, w, u)
             y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
-            call("rwkv_wkv6raw_forward_ex", dev, B, T, C, H, r, k, v, w, u, y, ctx.flags)
+            # the forward keeps the state entering every 64th token for the backward's single reverse sweep (no bytes for
+            # head sizes and options that take the two-sweep kernels)
+            nsaved = _lib.load().rwkv_wkv6f_saved_bytes(B, T, C, H)
+            saved = torch.empty(nsaved, device=dev, dtype=torch.uint8)
+            call("rwkv_wkv6f_forward", dev, B, T, C, H, r, k, v, w, u, None, y, saved if nsaved else None, nsaved, ctx.flags)
+            ctx.save_for_backward(r, k, v, w, u, saved)
             return y
 
     @staticmethod
     def backward(ctx, gy):
         with torch.no_grad():
             B, T, C, H = ctx.B, ctx.T, ctx.C, ctx.H
-            r, k, v, w, u = ctx.saved_tensors
+            r, k, v, w, u, saved = ctx.saved_tensors
             gy = gy.contiguous()
             dev = check_tensors((gy,), torch.bfloat16, ("gy",))
             new = lambda *shape: torch.empty(shape, device=dev, dtype=torch.bfloat16)
             gr, gk, gv, gw = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C)
             gu = new(H, C // H)                               # summed over the batch by the library (:169)
-            nbytes = _lib.load().rwkv_wkv6f_backward_workspace_bytes(B, T, C, H)
+            nbytes = _lib.load().rwkv_wkv6f_backward_saved_workspace_bytes(B, T, C, H)
             ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
-            call("rwkv_wkv6f_backward", dev, B, T, C, H, r, k, v, w, u, None, gy, gr, gk, gv, gw, gu, None, ws, nbytes, ctx.flags)
+            call("rwkv_wkv6f_backward_saved", dev, B, T, C, H, r, k, v, w, u, None, gy, gr, gk, gv, gw, gu, None,
+                 saved if saved.numel() else None, saved.numel(), ws, nbytes, ctx.flags)
             return (None, None, None, None, gr, gk, gv, gw, gu)
 
 

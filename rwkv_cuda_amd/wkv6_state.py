@@ -21,26 +21,30 @@ class WKV_6STATE(torch.autograd.Function):
             require(r.numel() == B * T * C and s.numel() == B * H * (C // H) * (C // H), "shape mismatch")
             ctx.B, ctx.T, ctx.C, ctx.H = B, T, C, H
             ctx.flags = options.current_flags()
-            ctx.save_for_backward(r, k, v, w, u, s)
             y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
-            call("rwkv_wkv6state_forward_ex", dev, B, T, C, H, r, k, v, w, u, s, y, ctx.flags)
+            # the forward keeps the state entering every 64th token for the backward's single reverse sweep (no bytes for
+            # head sizes and options that take the two-sweep kernels)
+            nsaved = _lib.load().rwkv_wkv6f_saved_bytes(B, T, C, H)
+            saved = torch.empty(nsaved, device=dev, dtype=torch.uint8)
+            call("rwkv_wkv6f_forward", dev, B, T, C, H, r, k, v, w, u, s, y, saved if nsaved else None, nsaved, ctx.flags)
+            ctx.save_for_backward(r, k, v, w, u, s, saved)
             return y
 
     @staticmethod
     def backward(ctx, gy):
         with torch.no_grad():
             B, T, C, H = ctx.B, ctx.T, ctx.C, ctx.H
-            r, k, v, w, u, s = ctx.saved_tensors
+            r, k, v, w, u, s, saved = ctx.saved_tensors
             gy = gy.contiguous()
             dev = check_tensors((gy,), torch.bfloat16, ("gy",))
             new = lambda *shape: torch.empty(shape, device=dev, dtype=torch.bfloat16)
             gr, gk, gv, gw = new(B, T, C), new(B, T, C), new(B, T, C), new(B, T, C)
             gu = new(H, C // H)                               # summed over the batch by the library (:123)
             gs = new(B, H, C // H, C // H)
-            nbytes = _lib.load().rwkv_wkv6f_backward_workspace_bytes(B, T, C, H)
+            nbytes = _lib.load().rwkv_wkv6f_backward_saved_workspace_bytes(B, T, C, H)
             ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
-            call("rwkv_wkv6f_backward", dev, B, T, C, H, r, k, v, w, u, s, gy,
-                 gr, gk, gv, gw, gu, gs, ws, nbytes, ctx.flags)
+            call("rwkv_wkv6f_backward_saved", dev, B, T, C, H, r, k, v, w, u, s, gy,
+                 gr, gk, gv, gw, gu, gs, saved if saved.numel() else None, saved.numel(), ws, nbytes, ctx.flags)
             return (None, None, None, None, gr, gk, gv, gw, gu, gs)
 
 

@@ -1,0 +1,158 @@
+"""GPU parity of the wkv6 / wkv6_state pair that hands chunk states from the forward to a one-sweep backward
+(rwkv_wkv6f_forward + rwkv_wkv6f_backward_saved), through the C ABI, against the CPU oracle and against the two-sweep
+kernels.  The bar is the reference kernel's own error (fp32 emulation with its rounding points), as everywhere."""
+import pytest
+import torch
+
+from oracle import wkv56 as O
+from rwkv_cuda_amd import options, synth
+from rwkv_cuda_amd._call import call
+from _gpu_util import DEV, assert_no_worse, garbage
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+NAMES = ["y", "gr", "gk", "gv", "gw", "gu", "gs"]
+
+
+def run_pair(lib, B, T, H, r, k, v, w, u, s0, gy, flags=0, saved_fill=None):
+    """forward + backward through the C ABI; every output and the handed-over states start as garbage"""
+    C = H * 64
+    d = [x.to(DEV) if x is not None else None for x in (r, k, v, w, u, s0, gy)]
+    y = garbage((B, T, C), BF)
+    nsv = lib.rwkv_wkv6f_saved_bytes(B, T, C, H)
+    saved = torch.empty(nsv, device=DEV, dtype=torch.uint8)
+    if saved_fill is not None:
+        saved.fill_(saved_fill)
+    call("rwkv_wkv6f_forward", DEV, B, T, C, H, *d[:6], y, saved, nsv, flags)
+    gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
+    gu = garbage((H, 64), BF)
+    gs = garbage((B, H, 64, 64), BF) if s0 is not None else None
+    n = lib.rwkv_wkv6f_backward_saved_workspace_bytes(B, T, C, H)
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8).fill_(0x7f)
+    call("rwkv_wkv6f_backward_saved", DEV, B, T, C, H, *d[:6], d[6], gr, gk, gv, gw, gu, gs, saved, nsv, ws, n, flags)
+    torch.cuda.synchronize()
+    handed_back = int(ws[-B * H * 32:].view(torch.int32).ne(0).view(B * H, 8).any(1).sum())
+    return [y, gr, gk, gv, gw, gu] + ([gs] if s0 is not None else []), handed_back
+
+
+# (B, T, H, state): one chunk, a cut chunk, an odd and an even number of chunks, T = 1, many chunks
+SHAPES = [(1, 32, 1, False), (2, 50, 2, True), (1, 97, 3, True), (2, 64, 1, False), (3, 1, 1, True), (1, 7, 2, False),
+          (2, 96, 2, True), (1, 200, 1, False), (1, 1000, 2, True)]
+
+
+@pytest.mark.parametrize("B,T,H,state", SHAPES)
+def test_one_sweep_against_the_oracle(lib, B, T, H, state):
+    print(f"\nwkv6 one sweep B={B} T={T} H={H} state={state}", flush=True)
+    C = H * 64
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=300 + T, state=state)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    got, handed_back = run_pair(lib, B, T, H, r, k, v, w, u, s0, gy, saved_fill=0x7f)
+    assert handed_back == 0                                     # these decays stay inside the range of the mid-point factors
+    for name, a, e, g in zip(NAMES, ref, emu, got):
+        assert torch.isfinite(g.float()).all(), name
+        assert_no_worse(name, a, e, g)
+    gw = got[4].float()
+    assert float(gw[:, T - 1].abs().max()) == 0.0              # w_{T-1} feeds nothing
+    if not state:
+        assert float(gw[:, 0].abs().max()) == 0.0              # nothing to decay at t = 0 without an initial state
+
+
+def test_one_sweep_hands_strong_decays_to_the_two_sweep_kernels(lib):
+    """Decays so strong that a channel loses more than e^-60 over 16 tokens: those (batch, head) pairs are flagged by the
+    one-sweep kernel and redone by the two-sweep kernels, whose chunks have a step-by-step path; the others are not."""
+    B, T, H = 2, 100, 3
+    C = H * 64
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=316, state=True)
+    w = w.float()
+    w[:, 40:60, :64] = 2.5                                      # head 0 of both batch rows
+    w[1, 70:, 100] = 3.0                                        # one channel of (1, head 1), up to the last token
+    w = w.to(BF)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    got, handed_back = run_pair(lib, B, T, H, r, k, v, w, u, s0, gy)
+    assert handed_back == 3, handed_back                        # (0,0), (1,0), (1,1); head 2 and (0,1) stay
+    for name, a, e, g in zip(NAMES, ref, emu, got):
+        assert torch.isfinite(g.float()).all(), name
+        assert_no_worse(name, a, e, g)
+
+
+def test_one_sweep_agrees_with_the_two_sweep_kernels(lib):
+    """Same inputs through both backward paths of the library: the gradients differ by at most one bf16 unit of the
+    tensor's peak (they round the same fp32 quantities, formed in a different order)."""
+    B, T, H = 2, 333, 2
+    C = H * 64
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=317, state=True)
+    one, _ = run_pair(lib, B, T, H, r, k, v, w, u, s0, gy)
+    d = [x.to(DEV) for x in (r, k, v, w, u, s0, gy)]
+    y = garbage((B, T, C), BF)
+    call("rwkv_wkv6state_forward", DEV, B, T, C, H, *d[:6], y)
+    gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
+    gu, gs = garbage((H, 64), BF), garbage((B, H, 64, 64), BF)
+    n = lib.rwkv_wkv6f_backward_workspace_bytes(B, T, C, H)
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+    call("rwkv_wkv6f_backward", DEV, B, T, C, H, *d[:6], d[6], gr, gk, gv, gw, gu, gs, ws, n, 0)
+    torch.cuda.synchronize()
+    assert torch.equal(one[0], y)                              # the same forward kernel either way
+    for name, a, b in zip(NAMES[1:], one[1:], [gr, gk, gv, gw, gu, gs]):
+        diff = float((a.float() - b.float()).abs().max()) / float(b.float().abs().max())
+        print(f"  {name}: max difference {diff:.2e} of the peak", flush=True)
+        assert diff <= 2.0 ** -7, name
+
+
+def test_other_head_sizes_and_options_take_the_two_sweep_kernels(lib):
+    """With a head size other than 64 there is nothing to hand over (0 bytes) and the pair runs the row kernels; with the
+    sequential-sweeps option the handed-over buffer is ignored.  Results as good as ever."""
+    B, T, H, N = 2, 40, 2, 32
+    C = H * N
+    g = torch.Generator().manual_seed(5)
+    r, k, v = ((torch.randn(B, T, C, generator=g) * 0.5).to(BF) for _ in range(3))
+    w = (torch.randn(B, T, C, generator=g) * 0.7 - 0.6).to(BF)
+    u = (torch.randn(H, N, generator=g) * 0.3).to(BF)
+    gy = torch.randn(B, T, C, generator=g).to(BF)
+    assert lib.rwkv_wkv6f_saved_bytes(B, T, C, H) == 0
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy)
+    d = [x.to(DEV) for x in (r, k, v, w, u, gy)]
+    y = garbage((B, T, C), BF)
+    call("rwkv_wkv6f_forward", DEV, B, T, C, H, *d[:5], None, y, None, 0, 0)
+    gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
+    gu = garbage((H, N), BF)
+    n = lib.rwkv_wkv6f_backward_saved_workspace_bytes(B, T, C, H)
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+    call("rwkv_wkv6f_backward_saved", DEV, B, T, C, H, *d[:5], None, d[5], gr, gk, gv, gw, gu, None, None, 0, ws, n, 0)
+    torch.cuda.synchronize()
+    for name, a, e, got in zip(NAMES, ref, emu, [y, gr, gk, gv, gw, gu]):
+        assert_no_worse(name, a, e, got)
+    # head size 64 with the sequential sweeps: the states are not written and not read
+    B, T, H = 1, 70, 2
+    C = H * 64
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=318, state=True)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    got, _ = run_pair(lib, B, T, H, r, k, v, w, u, s0, gy, flags=options.FLAG_SWEEPS, saved_fill=0x7f)
+    for name, a, e, g in zip(NAMES, ref, emu, got):
+        assert_no_worse("sweeps " + name, a, e, g)
+
+
+def test_one_sweep_rejects_bad_arguments(lib):
+    B, T, H = 1, 64, 1
+    C = 64
+    r, k, v, w, u, gy, _ = (x.to(DEV) if x is not None else None for x in synth.wkv6_inputs(B, T, C, H, seed=1))
+    y = torch.empty((B, T, C), device=DEV, dtype=BF)
+    nsv = lib.rwkv_wkv6f_saved_bytes(B, T, C, H)
+    assert nsv == 64 * 64 * 4                                   # one segment of 64 tokens
+    saved = torch.empty(nsv, device=DEV, dtype=torch.uint8)
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda t: t.data_ptr()
+    assert lib.rwkv_wkv6f_forward(st, B, T, C, H, p(r), p(k), p(v), p(w), p(u), None, p(y), p(saved), nsv - 1, 0) == -4   # too small
+    assert lib.rwkv_wkv6f_forward(st, B, 0, C, H, p(r), p(k), p(v), p(w), p(u), None, p(y), p(saved), nsv, 0) == -1       # bad shape
+    g4 = [torch.empty((B, T, C), device=DEV, dtype=BF) for _ in range(4)]
+    gu = torch.empty((H, 64), device=DEV, dtype=BF)
+    n = lib.rwkv_wkv6f_backward_saved_workspace_bytes(B, T, C, H)
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+    args = [st, B, T, C, H, p(r), p(k), p(v), p(w), p(u), None, p(gy)] + [p(x) for x in g4] + [p(gu), None, p(saved), nsv, p(ws)]
+    assert lib.rwkv_wkv6f_backward_saved(*args, n - 1, 0) == -4                                                          # workspace too small
+    args[10] = p(torch.empty((B, H, 64, 64), device=DEV, dtype=BF))                                                      # a state without its gradient
+    assert lib.rwkv_wkv6f_backward_saved(*args, n, 0) == -2
+    torch.cuda.synchronize()
