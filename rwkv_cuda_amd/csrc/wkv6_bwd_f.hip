@@ -37,11 +37,16 @@
 namespace rwkv {
 namespace {
 
+typedef uint32_t lds_t;            // a byte address in the workgroup's LDS
 constexpr int NTG = 16 * 64;
-constexpr int CS = 72;             // row stride (dwords) of an fp32 [token][channel] array
+// Row strides (dwords) measured on the access patterns of this kernel: 36 serves the 8-byte operand reads in accumulator
+// order and the prep waves' 4-byte reads at twice the rate of 40, 68 serves the prep waves' reads of X and Z at five
+// times the rate of 72 (16-byte reads and the transposing reads do not care).
+constexpr int PS = 36;             // bf16 [token][channel] planes: 144 B
+constexpr int CS = 68;             // fp32 [token][channel] arrays: 272 B
 
 struct alignas(16) SlotG {
-    uint32_t RpH[L][OS], RpL[L][OS], KpH[L][OS], KpL[L][OS], V[L][OS], GY[L][OS];
+    uint32_t RpH[L][PS], RpL[L][PS], KpH[L][PS], KpL[L][PS], V[L][PS], GY[L][PS];
     float d1[N], d2[N], dec[N], l2[N];     // 2^{c_m}, 2^{c_L - c_m}, 2^{c_L}, cc_32 = c_L - c_m
     float ruk[8][L];                        // sum of r u k over the 8 channels of each prep wave
 };
@@ -56,27 +61,43 @@ struct alignas(16) SmemG {
     float pex[2][N];                        // P = sum_i dS S at the last two anchors
 };
 static_assert(sizeof(SmemG) <= 160 * 1024, "LDS");
+constexpr lds_t ROW_B = PS * 4, PLANE_B = L * ROW_B, TROW_B = AS * 4, XROW_B = CS * 4, XZ_B = L * XROW_B;
+constexpr lds_t O_RPH = 0, O_RPL = PLANE_B, O_KPH = 2 * PLANE_B, O_KPL = 3 * PLANE_B, O_V = 4 * PLANE_B, O_GY = 5 * PLANE_B;
+constexpr lds_t O_D1 = 6 * PLANE_B, O_D2 = O_D1 + 4 * N, O_DEC = O_D2 + 4 * N, O_L2 = O_DEC + 4 * N, O_RUK = O_L2 + 4 * N;
+constexpr lds_t SLOT_B = sizeof(SlotG), SLOT0 = offsetof(SmemG, slot);
+constexpr lds_t T_AH = 0, T_AL = L * TROW_B, T_BH = 2 * L * TROW_B, T_BL = 3 * L * TROW_B, TILE_B = sizeof(TilesG), TILE0 = offsetof(SmemG, tile);
+constexpr lds_t XZ0 = offsetof(SmemG, xz), VG0 = offsetof(SmemG, vg), PEX0 = offsetof(SmemG, pex);
+static_assert(offsetof(SlotG, GY) == O_GY && offsetof(SlotG, d1) == O_D1 && offsetof(SlotG, ruk) == O_RUK && offsetof(TilesG, BL) == T_BL, "layout");
 
+// LDS is addressed with explicit byte addresses: a few per-lane bases (made opaque to the optimiser once per iteration,
+// so that it does not keep dozens of base + constant sums in registers across the loop), a wave-uniform part that
+// changes with the chunk (slot, tile set, X / Z parity) and a constant that goes into the instruction.
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+template <class T> DEVINL T lds_ld(const lds_t a) { return *(const __attribute__((address_space(3))) T*)(a); }
+template <class T> DEVINL void lds_st(const lds_t a, const T v) { *(__attribute__((address_space(3))) T*)(a) = v; }
+DEVINL lds_t lds_of(const void* p) { return static_cast<lds_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) char*)p)); }
+DEVINL void opaque(lds_t& x) { asm volatile("" : "+v"(x)); }
 typedef short v4s __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef v4s __attribute__((address_space(3))) * lds_v4s_ptr;
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // Operand with the rows of an LDS matrix along K: slot (g, e) <-> row row0 + e (e = 0..7), lane l16 <-> column col + l16.
-// p points at element [row0][col] of a matrix of bf16 with `stride` dwords per row; row0 = 8 g for a 32-row contraction.
-DEVINL bf16x8 tr_pair(const uint32_t* p, const int stride, const int l16) {
-    const uint32_t* q = p + (l16 >> 2) * stride + 2 * (l16 & 3);
-    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(q));
-    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(q + 4 * stride));
-    const uint2 a = __builtin_bit_cast(uint2, lo), b = __builtin_bit_cast(uint2, hi);
-    return as_op(a.x, a.y, b.x, b.y);
+// a = address of element [row0 + (l16 >> 2)][col + 4 (l16 & 3)] of a bf16 matrix with rows of `row_bytes`; row0 = 8 g for
+// a 32-row contraction.
+DEVINL bf16x8 ld_tr(const lds_t a, const lds_t row_bytes) {
+    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(a));
+    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(a + 4 * row_bytes));
+    const u32x2 x = __builtin_bit_cast(u32x2, lo), y = __builtin_bit_cast(u32x2, hi);
+    return as_op(x[0], x[1], y[0], y[1]);
 }
 // Operand with channels along K in accumulator order: slot (g, e) <-> channel 32 ks + 16 (e >> 2) + 4 g + (e & 3).
-// row points at the first dword of a [token] row of a bf16 plane.
-DEVINL bf16x8 acc_order_op(const uint32_t* row, const int ks, const int g) {
-    const uint2 a = *reinterpret_cast<const uint2*>(row + 16 * ks + 2 * g);
-    const uint2 b = *reinterpret_cast<const uint2*>(row + 16 * ks + 8 + 2 * g);
-    return as_op(a.x, a.y, b.x, b.y);
+// a = address of channel 32 ks + 4 g of a [token] row of a bf16 plane.
+DEVINL bf16x8 ld_acc(const lds_t a) {
+    const u32x2 x = lds_ld<u32x2>(a), y = lds_ld<u32x2>(a + 32);
+    return as_op(x[0], x[1], y[0], y[1]);
 }
+DEVINL bf16x8 ld_op(const lds_t a) { return __builtin_bit_cast(bf16x8, lds_ld<u32x4>(a)); }
 // inclusive prefix sum over the 16 lanes of a row: lane l gets the sum of lanes 0..l
 DEVINL float row_prefix_sum(float x) {
     x = dpp_add<0x111, 0xf>(x);       // row_shr:1
@@ -109,12 +130,12 @@ struct ArgsG {
 };
 
 // state entering even chunk e of this (batch, head), in the layout of the SD waves: lane <-> key channel 16w + l16,
-// x[tile][v] <-> value channel 16 tile + 4g + v
-DEVINL void load_state(const float* __restrict__ p, f32x4 (&x)[4], const int g) {
+// x[tile][v] <-> value channel 16 tile + 4g + v.  p: the state (wave-uniform), lo = (4 g) * 64 + 16 w + l16.
+DEVINL void load_state(const float* __restrict__ p, const uint32_t lo, f32x4 (&x)[4]) {
 #pragma unroll
     for (int tl = 0; tl < 4; ++tl)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) x[tl][v] = p[(16 * tl + 4 * g + v) * N];
+        for (int v = 0; v < 4; ++v) x[tl][v] = p[lo + (16 * tl + v) * N];
 }
 
 // ---------------------------------------------------------------------------------------------------- P waves
@@ -157,8 +178,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         SlotG& O = S.slot[c % 3];
         const bool live = !decltype(PARTIAL)::value || c * L + rw < T;
         const u32x4 zero = {0u, 0u, 0u, 0u};
-        uint32_t* da = &O.RpH[rw][4 * w] + hl * (2 * L * OS);        // R' hi | K' hi
-        uint32_t* db = &O.RpL[rw][4 * w] + hl * (3 * L * OS);        // R' lo | V
+        uint32_t* da = &O.RpH[rw][4 * w] + hl * (2 * L * PS);        // R' hi | K' hi
+        uint32_t* db = &O.RpL[rw][4 * w] + hl * (3 * L * PS);        // R' lo | V
         *reinterpret_cast<u32x4*>(da) = live ? x.a : zero;
         *reinterpret_cast<u32x4*>(db) = (live || !hl) ? x.b : zero;  // w of a dead row is masked where the decay is formed
         if (!hl) *reinterpret_cast<u32x4*>(&O.GY[rw][4 * w]) = live ? x.c : zero;
@@ -319,12 +340,19 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
 // ---------------------------------------------------------------------------------------------------- SD waves
 template <int WMODE>
 DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t bh, const int n) {
-    // g, l16 and j are redefined behind an empty asm in every iteration: LDS addresses are then formed where they are
-    // used instead of being kept, dozens of them, in registers across the loop
-    int g = lane >> 4, l16 = lane & 15, j = 16 * w + l16;
+    const int g = lane >> 4, l16 = lane & 15, j = 16 * w + l16;
     const int nseg = (n + 1) / 2;
-    const float* __restrict__ sv = a.saved + bh * nseg * (N * N) + j;
+    const float* __restrict__ sv = a.saved + bh * nseg * (N * N);
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    const lds_t sb = lds_of(&S);
+    // per-lane address parts
+    uint32_t b_sv = 4 * g * N + j;                                              // [value channel 4 g][key channel j] of a saved state
+    lds_t b_acc = l16 * ROW_B + 8 * g;                                          // [token l16][channel 4 g] of a plane
+    lds_t b_tr = ((8 * g + (l16 >> 2)) * PS + 2 * (l16 & 3)) * 4;               // transposing read of a plane, rows 8 g ..
+    lds_t b_trt = ((8 * g + (l16 >> 2)) * AS + 2 * (l16 & 3)) * 4;              // the same of a tile
+    lds_t b_natt = l16 * TROW_B + 16 * g;                                       // [row l16][position 8 g] of a tile
+    lds_t b_xz = l16 * XROW_B + 16 * g;                                         // [token l16][channel 4 g] of X / Z
+    lds_t b_j = 4 * l16;
     f32x4 D[4] = {zero4, zero4, zero4, zero4};
     f32x4 Sa[4];                           // the saved state of the segment at hand (chunks 2 sg, 2 sg + 1)
 
@@ -332,17 +360,16 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
     // the batches apart): a wave then waits for LDS a few times per chunk instead of once per product.
     // X^T[j][t] = (S d1)^T GY^T + K'^T Bm^T for chunk c; S = Sa (even chunk) or one update of it (odd chunk)
     auto part_x = [&](const int c) __attribute__((always_inline)) {
-        const SlotG& O = S.slot[c % 3];
-        const TilesG& Tl = S.tile[c & 1];
+        const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B, xo = sb + XZ0 + (c & 1) * 2 * XZ_B + 64 * w;
         f32x4 Sc[4];
         if (c & 1) {
             // state entering the odd chunk: S dec + d2 V^T K' with the chunk below
-            const SlotG& Q = S.slot[(c - 1) % 3];
-            const float qdec = Q.dec[j], qd2 = Q.d2[j];
-            const bf16x8 qh = tr_pair(&Q.KpH[8 * g][8 * w], OS, l16), ql = tr_pair(&Q.KpL[8 * g][8 * w], OS, l16);
+            const lds_t qo = sb + SLOT0 + ((c - 1) % 3) * SLOT_B;
+            const float qdec = lds_ld<float>(qo + O_DEC + 64 * w + b_j), qd2 = lds_ld<float>(qo + O_D2 + 64 * w + b_j);
+            const bf16x8 qh = ld_tr(qo + O_KPH + 32 * w + b_tr, ROW_B), ql = ld_tr(qo + O_KPL + 32 * w + b_tr, ROW_B);
             bf16x8 vop[4];
 #pragma unroll
-            for (int tl = 0; tl < 4; ++tl) vop[tl] = tr_pair(&Q.V[8 * g][8 * tl], OS, l16);
+            for (int tl = 0; tl < 4; ++tl) vop[tl] = ld_tr(qo + O_V + 32 * tl + b_tr, ROW_B);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int tl = 0; tl < 4; ++tl) {
@@ -356,16 +383,16 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
             for (int tl = 0; tl < 4; ++tl) Sc[tl] = Sa[tl];
         }
         __builtin_amdgcn_sched_barrier(0);
-        const float d1 = O.d1[j];
+        const float d1 = lds_ld<float>(so + O_D1 + 64 * w + b_j);
         bf16x8 gop[2][2];
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) gop[tt][ks] = acc_order_op(&O.GY[16 * tt + l16][0], ks, g);
-        const bf16x8 kh = tr_pair(&O.KpH[8 * g][8 * w], OS, l16), kl = tr_pair(&O.KpL[8 * g][8 * w], OS, l16);
+            for (int ks = 0; ks < 2; ++ks) gop[tt][ks] = ld_acc(so + O_GY + tt * 16 * ROW_B + 64 * ks + b_acc);
+        const bf16x8 kh = ld_tr(so + O_KPH + 32 * w + b_tr, ROW_B), kl = ld_tr(so + O_KPL + 32 * w + b_tr, ROW_B);
         bf16x8 bh_[2], bl_[2];
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) { bh_[tt] = lds_op(&Tl.BH[16 * tt + l16][4 * g]); bl_[tt] = lds_op(&Tl.BL[16 * tt + l16][4 * g]); }
+        for (int tt = 0; tt < 2; ++tt) { bh_[tt] = ld_op(to + T_BH + tt * 16 * TROW_B + b_natt); bl_[tt] = ld_op(to + T_BL + tt * 16 * TROW_B + b_natt); }
         __builtin_amdgcn_sched_barrier(0);
         bf16x8 sh[2], sl[2];
         split16(Sc, d1, sh, sl);
@@ -384,30 +411,28 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
             X[tt] = mfma(kl, bh_[tt], X[tt]);
         }
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
-            *reinterpret_cast<float4*>(&S.xz[c & 1][0][16 * tt + l16][16 * w + 4 * g]) = make_float4(X[tt][0], X[tt][1], X[tt][2], X[tt][3]);
+        for (int tt = 0; tt < 2; ++tt) lds_st<f32x4>(xo + tt * 16 * XROW_B + b_xz, X[tt]);
     };
     // Z^T[j][s] = (dS d2)^T V^T + R'^T Bm, then dS <- dS dec + d1 GY^T R'
     auto part_z = [&](const int c) __attribute__((always_inline)) {
-        const SlotG& O = S.slot[c % 3];
-        const TilesG& Tl = S.tile[c & 1];
-        const float d1 = O.d1[j], d2 = O.d2[j], dec = O.dec[j];
+        const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B, xo = sb + XZ0 + (c & 1) * 2 * XZ_B + XZ_B + 64 * w;
+        const float d1 = lds_ld<float>(so + O_D1 + 64 * w + b_j), d2 = lds_ld<float>(so + O_D2 + 64 * w + b_j), dec = lds_ld<float>(so + O_DEC + 64 * w + b_j);
         bf16x8 vop[2][2];
 #pragma unroll
         for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) vop[tt][ks] = acc_order_op(&O.V[16 * tt + l16][0], ks, g);
-        const bf16x8 rh = tr_pair(&O.RpH[8 * g][8 * w], OS, l16), rl = tr_pair(&O.RpL[8 * g][8 * w], OS, l16);
+            for (int ks = 0; ks < 2; ++ks) vop[tt][ks] = ld_acc(so + O_V + tt * 16 * ROW_B + 64 * ks + b_acc);
+        const bf16x8 rh = ld_tr(so + O_RPH + 32 * w + b_tr, ROW_B), rl = ld_tr(so + O_RPL + 32 * w + b_tr, ROW_B);
         bf16x8 bh_[2], bl_[2];
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) { bh_[tt] = tr_pair(&Tl.BH[8 * g][8 * tt], AS, l16); bl_[tt] = tr_pair(&Tl.BL[8 * g][8 * tt], AS, l16); }
+        for (int tt = 0; tt < 2; ++tt) { bh_[tt] = ld_tr(to + T_BH + 32 * tt + b_trt, TROW_B); bl_[tt] = ld_tr(to + T_BL + 32 * tt + b_trt, TROW_B); }
         __builtin_amdgcn_sched_barrier(0);
         bf16x8 dh[2], dl[2];
         split16(D, d2, dh, dl);
         __builtin_amdgcn_sched_barrier(0);
         bf16x8 gop[4];
 #pragma unroll
-        for (int tl = 0; tl < 4; ++tl) gop[tl] = tr_pair(&O.GY[8 * g][8 * tl], OS, l16);
+        for (int tl = 0; tl < 4; ++tl) gop[tl] = ld_tr(so + O_GY + 32 * tl + b_tr, ROW_B);
         __builtin_amdgcn_sched_barrier(0);
         f32x4 Z[2] = {zero4, zero4};
 #pragma unroll
@@ -424,8 +449,7 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
             Z[tt] = mfma(rl, bh_[tt], Z[tt]);
         }
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
-            *reinterpret_cast<float4*>(&S.xz[c & 1][1][16 * tt + l16][16 * w + 4 * g]) = make_float4(Z[tt][0], Z[tt][1], Z[tt][2], Z[tt][3]);
+        for (int tt = 0; tt < 2; ++tt) lds_st<f32x4>(xo + tt * 16 * XROW_B + b_xz, Z[tt]);
 #pragma unroll
         for (int tl = 0; tl < 4; ++tl) {
             f32x4 U = mfma(gop[tl], rh, zero4);
@@ -435,12 +459,12 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
         }
     };
 
-    load_state(sv + static_cast<size_t>(nseg - 1) * (N * N), Sa, g);
+    load_state(sv + static_cast<size_t>(nseg - 1) * (N * N), b_sv, Sa);
     __syncthreads();                       // iterations 0 and 1: nothing prepared yet
     __syncthreads();
 #pragma unroll 1
     for (int c = n - 1; c >= 0; --c) {
-        asm volatile("" : "+v"(g), "+v"(l16), "+v"(j));
+        opaque(b_acc); opaque(b_tr); opaque(b_trt); opaque(b_natt); opaque(b_xz); opaque(b_j); opaque(b_sv);
         // Sa of an odd chunk was asked for at the end of the last iteration: what does not need it goes first
         part_z(c);
         __builtin_amdgcn_sched_barrier(0);
@@ -454,9 +478,9 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
 #pragma unroll
                 for (int v = 0; v < 4; ++v) p = fmaf(D[tl][v], Sa[tl][v], p);
             p = allreduce_rows(p);
-            if (g == 0) S.pex[(c >> 1) & 1][j] = p;
+            if (g == 0) lds_st<float>(sb + PEX0 + ((c >> 1) & 1) * (4 * N) + 64 * w + b_j, p);
             // the next segment's state (index clamped: the load is issued on every path, so that waits can count it)
-            load_state(sv + static_cast<size_t>(c >= 2 ? (c >> 1) - 1 : 0) * (N * N), Sa, g);
+            load_state(sv + static_cast<size_t>(c >= 2 ? (c >> 1) - 1 : 0) * (N * N), b_sv, Sa);
         }
         __syncthreads();
     }
@@ -469,26 +493,41 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
     }
 }
 
-// ---------------------------------------------------------------------------------------------------- EW waves
+// ---------------------------------------------------------------------------------------------------- E waves
 template <int WMODE>
 DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int n) {
-    int g = lane >> 4, l16 = lane & 15;    // redefined behind an empty asm in every iteration, see role_sd
+    const int g = lane >> 4, l16 = lane & 15;
     const int T = a.T, C = a.C;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    const lds_t sb = lds_of(&S);
+    lds_t b_acc = l16 * ROW_B + 8 * g;                                          // [token l16][channel 4 g] of a plane
+    lds_t b_nat = l16 * ROW_B + 16 * g;                                         // [token l16][channel 8 g] of a plane
+    lds_t b_tr = ((8 * g + (l16 >> 2)) * PS + 2 * (l16 & 3)) * 4;               // transposing read of a plane, rows 8 g ..
+    lds_t b_trt = ((8 * g + (l16 >> 2)) * AS + 2 * (l16 & 3)) * 4;              // the same of a tile
+    lds_t b_tw = l16 * TROW_B + 8 * g;                                          // [row l16][position 4 g] of a tile
+    lds_t b_g = 16 * g;                                                          // channel 4 g of a per-channel array
+    lds_t b_l = 4 * l16;
+    uint16_t* __restrict__ gvp = a.gv + base + 16 * w + 4 * g;
     f32x4 E[4] = {zero4, zero4, zero4, zero4};     // dS[i = 16w + l16][j = 16 tile + 4g + v]
 
     // causal tiles of chunk c (waves 0, 1, 2 -> quadrants (t, s) = (0,0) (1,0) (1,1)); accumulator rows are s, lanes t
     auto tiles = [&](const int c) __attribute__((always_inline)) {
-        const SlotG& O = S.slot[c % 3];
-        TilesG& Tl = S.tile[c & 1];
+        const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
         const int ta = (w == 0) ? 0 : 1, tb = (w == 2) ? 1 : 0;
+        const lds_t ra = so + ta * 16 * ROW_B + b_nat, rb = so + tb * 16 * ROW_B + b_nat;
         f32x4 a0 = zero4, a1 = zero4, bm = zero4;
         bf16x8 kh[2], kl[2], rh[2], rl[2], vo[2], go[2];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
-            kh[ks] = lds_op(&O.KpH[16 * tb + l16][16 * ks + 4 * g]); kl[ks] = lds_op(&O.KpL[16 * tb + l16][16 * ks + 4 * g]);
-            rh[ks] = lds_op(&O.RpH[16 * ta + l16][16 * ks + 4 * g]); rl[ks] = lds_op(&O.RpL[16 * ta + l16][16 * ks + 4 * g]);
-            vo[ks] = lds_op(&O.V[16 * tb + l16][16 * ks + 4 * g]); go[ks] = lds_op(&O.GY[16 * ta + l16][16 * ks + 4 * g]);
+            kh[ks] = ld_op(rb + O_KPH + 64 * ks); kl[ks] = ld_op(rb + O_KPL + 64 * ks);
+            rh[ks] = ld_op(ra + O_RPH + 64 * ks); rl[ks] = ld_op(ra + O_RPL + 64 * ks);
+            vo[ks] = ld_op(rb + O_V + 64 * ks); go[ks] = ld_op(ra + O_GY + 64 * ks);
+        }
+        float d = 0.f;
+        if (ta == tb) {
+            const lds_t ru = so + O_RUK + ta * 64 + b_l;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) d += lds_ld<float>(ru + q * (4 * L));
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -500,64 +539,59 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
         }
         f32x4 am = a0 + a1;                                    // [v]: s = 16 tb + 4g + v, t = 16 ta + l16
         if (ta == tb) {
-            const int t = 16 * ta + l16;
-            const float d = ((O.ruk[0][t] + O.ruk[1][t]) + (O.ruk[2][t] + O.ruk[3][t])) + ((O.ruk[4][t] + O.ruk[5][t]) + (O.ruk[6][t] + O.ruk[7][t]));
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int sl = 4 * g + v;
-                if (sl == l16) S.vg[c & 3][t] = bm[v];
+                if (sl == l16) lds_st<float>(sb + VG0 + (c & 3) * (4 * L) + ta * 64 + b_l, bm[v]);
                 am[v] = (sl < l16) ? am[v] : (sl == l16 ? d : 0.f);
                 bm[v] = (sl < l16) ? bm[v] : 0.f;
             }
         }
         const HL x0 = hilo2(am[0], am[1]), x1 = hilo2(am[2], am[3]), y0 = hilo2(bm[0], bm[1]), y1 = hilo2(bm[2], bm[3]);
-        *reinterpret_cast<uint2*>(&Tl.AH[16 * ta + l16][8 * tb + 2 * g]) = make_uint2(x0.h, x1.h);
-        *reinterpret_cast<uint2*>(&Tl.AL[16 * ta + l16][8 * tb + 2 * g]) = make_uint2(x0.l, x1.l);
-        *reinterpret_cast<uint2*>(&Tl.BH[16 * ta + l16][8 * tb + 2 * g]) = make_uint2(y0.h, y1.h);
-        *reinterpret_cast<uint2*>(&Tl.BL[16 * ta + l16][8 * tb + 2 * g]) = make_uint2(y0.l, y1.l);
+        const lds_t tw = to + ta * 16 * TROW_B + tb * 32 + b_tw;
+        lds_st<u32x2>(tw + T_AH, u32x2{x0.h, x1.h});
+        lds_st<u32x2>(tw + T_AL, u32x2{x0.l, x1.l});
+        lds_st<u32x2>(tw + T_BH, u32x2{y0.h, y1.h});
+        lds_st<u32x2>(tw + T_BL, u32x2{y0.l, y1.l});
     };
 
 #pragma unroll 1
     for (int it = 0; it <= n + 2; ++it) {
         const int c = n + 1 - it;
-        asm volatile("" : "+v"(g), "+v"(l16));
+        opaque(b_acc); opaque(b_nat); opaque(b_tr); opaque(b_trt); opaque(b_tw); opaque(b_g); opaque(b_l);
         if (it >= 2 && c >= 0) {
-            const SlotG& O = S.slot[c % 3];
-            const TilesG& Tl = S.tile[c & 1];
+            const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
             // Operands are fetched in batches, each issued as a whole before anything waits for it (the scheduling barriers
             // keep the batches apart): a wave then waits for LDS three times per chunk instead of once per product.
             // ------------------------------------------------------------ batch 1: d2 and K' (natural rows)
-            float4 dq[4];
+            f32x4 dq[4];
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                dq[2 * ks] = *reinterpret_cast<const float4*>(&O.d2[32 * ks + 4 * g]);
-                dq[2 * ks + 1] = *reinterpret_cast<const float4*>(&O.d2[32 * ks + 16 + 4 * g]);
-            }
+            for (int q = 0; q < 4; ++q) dq[q] = lds_ld<f32x4>(so + O_D2 + 64 * q + b_g);
             bf16x8 kh[2][2], kl[2][2];
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks) {
-                    kh[tt][ks] = acc_order_op(&O.KpH[16 * tt + l16][0], ks, g);
-                    kl[tt][ks] = acc_order_op(&O.KpL[16 * tt + l16][0], ks, g);
+                    kh[tt][ks] = ld_acc(so + O_KPH + tt * 16 * ROW_B + 64 * ks + b_acc);
+                    kl[tt][ks] = ld_acc(so + O_KPL + tt * 16 * ROW_B + 64 * ks + b_acc);
                 }
             __builtin_amdgcn_sched_barrier(0);
             // ------------------------------------------------------------ gv^T[i][s] = (dS d2) K'^T + GY^T A
             bf16x8 dh[2], dl[2];
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
-                const float4 p = dq[2 * ks], q = dq[2 * ks + 1];
-                const HL x0 = hilo2(E[2 * ks][0] * p.x, E[2 * ks][1] * p.y), x1 = hilo2(E[2 * ks][2] * p.z, E[2 * ks][3] * p.w);
-                const HL x2 = hilo2(E[2 * ks + 1][0] * q.x, E[2 * ks + 1][1] * q.y), x3 = hilo2(E[2 * ks + 1][2] * q.z, E[2 * ks + 1][3] * q.w);
+                const f32x4 p = dq[2 * ks], q = dq[2 * ks + 1];
+                const HL x0 = hilo2(E[2 * ks][0] * p[0], E[2 * ks][1] * p[1]), x1 = hilo2(E[2 * ks][2] * p[2], E[2 * ks][3] * p[3]);
+                const HL x2 = hilo2(E[2 * ks + 1][0] * q[0], E[2 * ks + 1][1] * q[1]), x3 = hilo2(E[2 * ks + 1][2] * q[2], E[2 * ks + 1][3] * q[3]);
                 dh[ks] = as_op(x0.h, x1.h, x2.h, x3.h);
                 dl[ks] = as_op(x0.l, x1.l, x2.l, x3.l);
             }
             __builtin_amdgcn_sched_barrier(0);
             // ------------------------------------------------------------ batch 2: gy and the A tile with the tokens along K
-            const bf16x8 gyo = tr_pair(&O.GY[8 * g][8 * w], OS, l16);       // lane = value channel 16w + l16, K = tokens
+            const bf16x8 gyo = ld_tr(so + O_GY + 32 * w + b_tr, ROW_B);        // lane = value channel 16w + l16, K = tokens
             bf16x8 ah[2], al[2];
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) { ah[tt] = tr_pair(&Tl.AH[8 * g][8 * tt], AS, l16); al[tt] = tr_pair(&Tl.AL[8 * g][8 * tt], AS, l16); }
+            for (int tt = 0; tt < 2; ++tt) { ah[tt] = ld_tr(to + T_AH + 32 * tt + b_trt, TROW_B); al[tt] = ld_tr(to + T_AL + 32 * tt + b_trt, TROW_B); }
             __builtin_amdgcn_sched_barrier(0);
             f32x4 G[2] = {zero4, zero4};
 #pragma unroll
@@ -569,10 +603,10 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                     G[tt] = mfma(dl[ks], kh[tt][ks], G[tt]);
                 }
             __builtin_amdgcn_sched_barrier(0);
-            // ------------------------------------------------------------ batch 3: R' with the tokens along K, dec, d1
+            // ------------------------------------------------------------ batch 3: R' with the tokens along K
             bf16x8 rh[4], rl[4];
 #pragma unroll
-            for (int tl = 0; tl < 4; ++tl) { rh[tl] = tr_pair(&O.RpH[8 * g][8 * tl], OS, l16); rl[tl] = tr_pair(&O.RpL[8 * g][8 * tl], OS, l16); }
+            for (int tl = 0; tl < 4; ++tl) { rh[tl] = ld_tr(so + O_RPH + 32 * tl + b_tr, ROW_B); rl[tl] = ld_tr(so + O_RPL + 32 * tl + b_tr, ROW_B); }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
@@ -590,16 +624,14 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
             for (int tt = 0; tt < 2; ++tt) {
                 const int tg = c * L + 16 * tt + l16;
                 if (tg < T)
-                    *reinterpret_cast<uint2*>(a.gv + base + static_cast<size_t>(tg) * C + 16 * w + 4 * g) =
-                        make_uint2(pack_bf2(G[tt][0], G[tt][1]), pack_bf2(G[tt][2], G[tt][3]));
+                    *reinterpret_cast<uint2*>(gvp + static_cast<uint32_t>(tg) * C) = make_uint2(pack_bf2(G[tt][0], G[tt][1]), pack_bf2(G[tt][2], G[tt][3]));
             }
             // ------------------------------------------------------------ dS^T <- dS^T dec + d1 R'^T GY
 #pragma unroll
             for (int tl = 0; tl < 4; ++tl) {
-                const float4 de = *reinterpret_cast<const float4*>(&O.dec[16 * tl + 4 * g]);
-                const float4 d1 = *reinterpret_cast<const float4*>(&O.d1[16 * tl + 4 * g]);
-                E[tl][0] = fmaf(E[tl][0], de.x, d1.x * U[tl][0]); E[tl][1] = fmaf(E[tl][1], de.y, d1.y * U[tl][1]);
-                E[tl][2] = fmaf(E[tl][2], de.z, d1.z * U[tl][2]); E[tl][3] = fmaf(E[tl][3], de.w, d1.w * U[tl][3]);
+                const f32x4 de = lds_ld<f32x4>(so + O_DEC + 64 * tl + b_g), d1 = lds_ld<f32x4>(so + O_D1 + 64 * tl + b_g);
+#pragma unroll
+                for (int v = 0; v < 4; ++v) E[tl][v] = fmaf(E[tl][v], de[v], d1[v] * U[tl][v]);
             }
         }
         __builtin_amdgcn_sched_barrier(0);
