@@ -38,7 +38,7 @@ FLAGS = 0                      # RWKV_FLAG_SWEEPS when --algo sweeps: passed per
 # by kernel label at the headline shape; None = not measured for the current kernels.
 TRAFFIC_MEASURED = {
     # profiles/wkv6_fused_kernels_B8_T4096_C2048.md  (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB)
-    "wkv6_fwd_ws (keeps states)": 537.2e6 + 402.7e6,
+    "wkv6_fwd_fused (keeps states)": 537.2e6 + 402.7e6,
     "wkv6_bwd_fused (+ gu batch sum)": 940.4e6 + 537.0e6,
     # profiles/wkv5_ws_kernels_B8_T4096_C2048.md
     "wkv6_fwd_ws<head decay>": 403e6 + 134e6,
@@ -128,7 +128,7 @@ def make_wkv6(dev, state):
 
     # algorithmic bytes per kernel: tensors it must read once + outputs it must write once, 2 B per element
     if ALGO == "chunked":
-        kernels = [("wkv6_fwd_ws (keeps states)", fwd, 10 * C * tok),                      # r k v w -> y
+        kernels = [("wkv6_fwd_fused (keeps states)", fwd, 10 * C * tok),                      # r k v w -> y
                    ("wkv6_bwd_fused (+ gu batch sum)", bwd_all, 18 * C * tok)]              # r k v w gy -> gr gk gv gw
     else:
         kernels = [("wkv_sweep<FWD>", fwd, 10 * C * tok),

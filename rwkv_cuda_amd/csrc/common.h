@@ -137,7 +137,11 @@ inline int launch_status() {
 // wkv6_chunk.hip: chunked MFMA kernels.  wmode: 1 = fp32 ew [B,T,C], 2 = raw bf16 w.
 int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                           const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
-                          const uint16_t* s0, uint16_t* y, float* saved = nullptr);
+                          const uint16_t* s0, uint16_t* y, float* saved = nullptr, const int* only_flagged = nullptr);
+// wkv6_fwd_f.hip: the forward that goes with wkv6_bwd_f.hip (raw bf16 decay, head size 64): y and the state entering
+// every second chunk; flags [B*H][8] names the (batch, head) pairs that have to be redone by the kernel above
+int launch_wkv6_fwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
+                          const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, float* saved, int* flags);
 int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                             const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
                             const uint16_t* s0, const uint16_t* gy, uint16_t* gr, uint16_t* gu, float* rdr,

@@ -1240,7 +1240,7 @@ bool fused_ok(int T, int C, int H, unsigned flags) {
 size_t rwkv_wkv6f_saved_bytes(int B, int T, int C, int H) {
     if (check_dims(B, T, C, H) != RWKV_OK || C != H * N || static_cast<long long>(T) * C >= (1LL << 30)) return 0;
     const size_t nchunks = (static_cast<size_t>(T) + 31) / 32, nseg = (nchunks + 1) / 2;
-    return static_cast<size_t>(B) * H * nseg * 64 * 64 * sizeof(float);
+    return static_cast<size_t>(B) * H * nseg * 64 * 64 * sizeof(float) + round16(static_cast<size_t>(B) * H * 8 * sizeof(int));
 }
 
 int rwkv_wkv6f_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
@@ -1255,7 +1255,13 @@ int rwkv_wkv6f_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16
         return launch_fwd<W_RAW>(static_cast<hipStream_t>(stream), B, a, flags);
     }
     if (saved_bytes < rwkv_wkv6f_saved_bytes(B, T, C, H) || !aligned16(saved)) return RWKV_ERR_WORKSPACE;
-    return launch_wkv6_fwd_chunk(static_cast<hipStream_t>(stream), W_RAW, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved));
+    // the states, then a word per prep wave of every (batch, head): set where a decay is too strong for the mid-point
+    // factors; those pairs are redone (y and states) by the kernel that has a step-by-step path, all others return at once
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    const size_t nflag = round16(static_cast<size_t>(B) * H * 8 * sizeof(int));
+    int* flg = reinterpret_cast<int*>(static_cast<char*>(saved) + (rwkv_wkv6f_saved_bytes(B, T, C, H) - nflag));
+    if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved), flg)) return e;
+    return launch_wkv6_fwd_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved), flg);
 }
 
 size_t rwkv_wkv6f_backward_saved_workspace_bytes(int B, int T, int C, int H) {

@@ -32,12 +32,11 @@
 //
 // A chunk in which some channel decays by more than e^-60 over either half cannot use the mid-point factors.  Such a
 // (batch, head) is flagged in `flags` and the caller reruns it with the two-sweep kernels, which have a step-by-step path.
-#include "wkv6_chunk.h"
+#include "wkv6_fused.h"
 
 namespace rwkv {
 namespace {
 
-typedef uint32_t lds_t;            // a byte address in the workgroup's LDS
 constexpr int NTG = 16 * 64;
 // Row strides (dwords) measured on the access patterns of this kernel: 36 serves the 8-byte operand reads in accumulator
 // order and the prep waves' 4-byte reads at twice the rate of 40, 68 serves the prep waves' reads of X and Z at five
@@ -69,56 +68,6 @@ constexpr lds_t T_AH = 0, T_AL = L * TROW_B, T_BH = 2 * L * TROW_B, T_BL = 3 * L
 constexpr lds_t XZ0 = offsetof(SmemG, xz), VG0 = offsetof(SmemG, vg), PEX0 = offsetof(SmemG, pex);
 static_assert(offsetof(SlotG, GY) == O_GY && offsetof(SlotG, d1) == O_D1 && offsetof(SlotG, ruk) == O_RUK && offsetof(TilesG, BL) == T_BL, "layout");
 
-// LDS is addressed with explicit byte addresses: a few per-lane bases (made opaque to the optimiser once per iteration,
-// so that it does not keep dozens of base + constant sums in registers across the loop), a wave-uniform part that
-// changes with the chunk (slot, tile set, X / Z parity) and a constant that goes into the instruction.
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-template <class T> DEVINL T lds_ld(const lds_t a) { return *(const __attribute__((address_space(3))) T*)(a); }
-template <class T> DEVINL void lds_st(const lds_t a, const T v) { *(__attribute__((address_space(3))) T*)(a) = v; }
-DEVINL lds_t lds_of(const void* p) { return static_cast<lds_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) char*)p)); }
-DEVINL void opaque(lds_t& x) { asm volatile("" : "+v"(x)); }
-typedef short v4s __attribute__((ext_vector_type(4)));
-typedef v4s __attribute__((address_space(3))) * lds_v4s_ptr;
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-// Operand with the rows of an LDS matrix along K: slot (g, e) <-> row row0 + e (e = 0..7), lane l16 <-> column col + l16.
-// a = address of element [row0 + (l16 >> 2)][col + 4 (l16 & 3)] of a bf16 matrix with rows of `row_bytes`; row0 = 8 g for
-// a 32-row contraction.
-DEVINL bf16x8 ld_tr(const lds_t a, const lds_t row_bytes) {
-    const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(a));
-    const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(a + 4 * row_bytes));
-    const u32x2 x = __builtin_bit_cast(u32x2, lo), y = __builtin_bit_cast(u32x2, hi);
-    return as_op(x[0], x[1], y[0], y[1]);
-}
-// Operand with channels along K in accumulator order: slot (g, e) <-> channel 32 ks + 16 (e >> 2) + 4 g + (e & 3).
-// a = address of channel 32 ks + 4 g of a [token] row of a bf16 plane.
-DEVINL bf16x8 ld_acc(const lds_t a) {
-    const u32x2 x = lds_ld<u32x2>(a), y = lds_ld<u32x2>(a + 32);
-    return as_op(x[0], x[1], y[0], y[1]);
-}
-DEVINL bf16x8 ld_op(const lds_t a) { return __builtin_bit_cast(bf16x8, lds_ld<u32x4>(a)); }
-// inclusive prefix sum over the 16 lanes of a row: lane l gets the sum of lanes 0..l
-DEVINL float row_prefix_sum(float x) {
-    x = dpp_add<0x111, 0xf>(x);       // row_shr:1
-    x = dpp_add<0x112, 0xf>(x);
-    x = dpp_add<0x114, 0xf>(x);
-    x = dpp_add<0x118, 0xf>(x);
-    return x;
-}
-// value of the next lane of the row (lane 15 gets 0)
-DEVINL float row_next(float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x101, 0xf, 0xf, true));
-}
-DEVINL void split16(const f32x4 (&x)[4], const float s, bf16x8 (&h)[2], bf16x8 (&l)[2]) {
-#pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-        const HL a = hilo2(x[2 * ks][0] * s, x[2 * ks][1] * s), b = hilo2(x[2 * ks][2] * s, x[2 * ks][3] * s);
-        const HL c = hilo2(x[2 * ks + 1][0] * s, x[2 * ks + 1][1] * s), d = hilo2(x[2 * ks + 1][2] * s, x[2 * ks + 1][3] * s);
-        h[ks] = as_op(a.h, b.h, c.h, d.h);
-        l[ks] = as_op(a.l, b.l, c.l, d.l);
-    }
-}
 
 struct ArgsG {
     int T, C, H;
@@ -141,7 +90,7 @@ DEVINL void load_state(const float* __restrict__ p, const uint32_t lo, f32x4 (&x
 // ---------------------------------------------------------------------------------------------------- P waves
 // wave w (0..7): channels 8w..8w+7; lane = 16 * (channel pair) + token: a thread has two channels of tokens tp and tp + 16
 template <int WMODE>
-DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n) {
+DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n, const int nit) {
     // jq, tp (and hl, rw below) are redefined behind an empty asm in every iteration, see role_sd
     int jq = lane >> 4, tp = lane & 15;
     const int ch0 = 8 * w + 2 * (lane >> 4);
@@ -175,8 +124,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     };
     // the pieces of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v and gy in place
     auto stage_in = [&](const int c, const Raw& x, auto PARTIAL) __attribute__((always_inline)) {
-        SlotG& O = S.slot[c % 3];
-        const bool live = !decltype(PARTIAL)::value || c * L + rw < T;
+        SlotG& O = S.slot[(c + 6) % 3];
+        const bool live = !decltype(PARTIAL)::value || (c >= 0 && c * L + rw < T);
         const u32x4 zero = {0u, 0u, 0u, 0u};
         uint32_t* da = &O.RpH[rw][4 * w] + hl * (2 * L * PS);        // R' hi | K' hi
         uint32_t* db = &O.RpL[rw][4 * w] + hl * (3 * L * PS);        // R' lo | V
@@ -193,14 +142,14 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
 
     auto prep = [&](const int c, Held& hd, auto PARTIAL) __attribute__((always_inline)) {
         const int ch = 8 * w + 2 * jq, cd = 4 * w + jq;        // cd: dword column of the pair in a bf16 plane
-        SlotG& O = S.slot[c % 3];
+        SlotG& O = S.slot[(c + 6) % 3];
         float lam[2][2], rf[2][2], kf[2][2];
         uint32_t xr[2], xk[2], xw[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) { xr[e] = O.RpH[tp + 16 * e][cd]; xk[e] = O.KpH[tp + 16 * e][cd]; xw[e] = O.RpL[tp + 16 * e][cd]; }
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const bool live = !decltype(PARTIAL)::value || c * L + tp + 16 * e < T;
+            const bool live = !decltype(PARTIAL)::value || (c >= 0 && c * L + tp + 16 * e < T);
             rf[e][0] = bf_lo(xr[e]); rf[e][1] = bf_hi(xr[e]);
             kf[e][0] = bf_lo(xk[e]); kf[e][1] = bf_hi(xk[e]);
             lam[e][0] = live ? -LOG2E * exp2_fast(LOG2E * bf_lo(xw[e])) : 0.f;
@@ -308,27 +257,31 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     const bool cut = (T % L) != 0;         // the last chunk is cut short
     const std::true_type part{};
     const std::false_type full{};
+    // in the order in which the loop consumes them: its waits are counted from the worst of all the ways into it
+    __builtin_amdgcn_sched_barrier(0);
     fetch(n - 1, ring[0]);
+    __builtin_amdgcn_sched_barrier(0);
     fetch(n >= 2 ? n - 2 : 0, ring[1]);
-    for (int it0 = 0; it0 <= n + 2; it0 += 2)
+    __builtin_amdgcn_sched_barrier(0);
+    // Two iterations per trip, no stage with loads or ring registers skipped: a way round one, or round the second half,
+    // would be one more way into the next wait, on which the registers it waits for are the newest loads (the count then
+    // covers everything).  Below chunk 0 the stages run on rows that all count as dead, into planes nobody reads any more
+    // (c < 0: the slot is that of chunk c + 3, of which only l2 is still needed, by this wave, before it is written).
+    for (int it0 = 0; it0 < nit; it0 += 2)
         static_for<2>([&](auto Z) {
             constexpr int z = decltype(Z)::value;
             const int it = it0 + z;
-            if (it <= n + 2) {
-                const int cp = n - 1 - it;
-                asm volatile("" : "+v"(jq), "+v"(tp), "+v"(hl), "+v"(rw));
-                // The same three loads in every iteration (chunk index clamped): the wait for a chunk's registers is then
-                // the count of loads issued after them on every path, and never has to cover the newest ones.
-                if (cp >= 0) { if (cut && it == 0) stage_in(cp, ring[z], part); else stage_in(cp, ring[z], full); }
-                __builtin_amdgcn_sched_barrier(0);
-                fetch(cp >= 2 ? cp - 2 : 0, ring[z]);
-                __builtin_amdgcn_sched_barrier(0);
-                if (it >= 3) { if (cut && it == 3) finish(cp + 3, hq[2], part); else finish(cp + 3, hq[2], full); }
-                __builtin_amdgcn_sched_barrier(0);
-                hq[2] = hq[1]; hq[1] = hq[0];
-                if (cp >= 0) { if (cut && it == 0) prep(cp, hq[0], part); else prep(cp, hq[0], full); }
-                __syncthreads();
-            }
+            const int cp = n - 1 - it;
+            asm volatile("" : "+v"(jq), "+v"(tp), "+v"(hl), "+v"(rw));
+            if ((cut && it == 0) || cp < 0) stage_in(cp, ring[z], part); else stage_in(cp, ring[z], full);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(cp >= 2 ? cp - 2 : 0, ring[z]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (it >= 3 && cp + 3 >= 0) { if (cut && it == 3) finish(cp + 3, hq[2], part); else finish(cp + 3, hq[2], full); }
+            __builtin_amdgcn_sched_barrier(0);
+            hq[2] = hq[1]; hq[1] = hq[0];
+            if ((cut && it == 0) || cp < 0) prep(cp, hq[0], part); else prep(cp, hq[0], full);
+            __syncthreads();
         });
     if (lane == 0) a.flags[bh * 8 + w] = any_exact ? 1 : 0;
     // gu of this batch row: sum over the tokens (lanes of a row)
@@ -339,7 +292,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
 
 // ---------------------------------------------------------------------------------------------------- SD waves
 template <int WMODE>
-DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t bh, const int n) {
+DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t bh, const int n, const int nit) {
     const int g = lane >> 4, l16 = lane & 15, j = 16 * w + l16;
     const int nseg = (n + 1) / 2;
     const float* __restrict__ sv = a.saved + bh * nseg * (N * N);
@@ -484,7 +437,7 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
         }
         __syncthreads();
     }
-    __syncthreads();                       // iteration n + 2: the P waves finish chunk 0
+    for (int it = n + 2; it < nit; ++it) __syncthreads();      // the P waves finish chunk 0
     if (a.gs != nullptr) {
 #pragma unroll
         for (int tl = 0; tl < 4; ++tl)
@@ -495,7 +448,7 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
 
 // ---------------------------------------------------------------------------------------------------- E waves
 template <int WMODE>
-DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int n) {
+DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int n, const int nit) {
     const int g = lane >> 4, l16 = lane & 15;
     const int T = a.T, C = a.C;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -556,7 +509,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
     };
 
 #pragma unroll 1
-    for (int it = 0; it <= n + 2; ++it) {
+    for (int it = 0; it < nit; ++it) {
         const int c = n + 1 - it;
         opaque(b_acc); opaque(b_nat); opaque(b_tr); opaque(b_trt); opaque(b_tw); opaque(b_g); opaque(b_l);
         if (it >= 2 && c >= 0) {
@@ -652,9 +605,10 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG a) {
     for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTG) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
-    if (wid < 8) role_prep<WMODE>(S, a, lane, wid, base, h, bh, n);
-    else if (wid < 12) role_sd<WMODE>(S, a, lane, w, bh, n);
-    else role_e<WMODE>(S, a, lane, w, base, n);
+    const int nit = (n + 4) & ~1;          // iterations of the pipeline: n + 3, made even
+    if (wid < 8) role_prep<WMODE>(S, a, lane, wid, base, h, bh, n, nit);
+    else if (wid < 12) role_sd<WMODE>(S, a, lane, w, bh, n, nit);
+    else role_e<WMODE>(S, a, lane, w, base, n, nit);
 }
 
 }  // namespace

@@ -64,6 +64,8 @@ struct ArgsC {
     // when not null: [B*H][ceil(chunks / 2)][64][64] fp32, the state entering every even chunk, [value][key], for the
     // one-sweep backward (wkv6_bwd_f.hip)
     float* saved;
+    // when not null: [B*H][8]; a workgroup runs only if one of its eight words is not zero (see ArgsB)
+    const int* only_flagged;
 };
 
 struct ArgsB {

@@ -483,6 +483,7 @@ __global__ __launch_bounds__(NTF) void wkv6_fwd_ws(const ArgsC a) {
     const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
     const size_t bh = static_cast<size_t>(b) * a.H + h;
     const int nchunks = (a.T + L - 1) / L;
+    if (skip_unflagged(a.only_flagged, blockIdx.x)) return;
     // positions of A that no tile ever writes (t < 16 <= s) must read as zero
     for (int i = tid; i < 2 * L * OS; i += NTF) { (&S.AmH[0][0][0])[i] = 0; (&S.AmL[0][0][0])[i] = 0; }
     if constexpr (SPLIT != 0) {
@@ -502,9 +503,10 @@ __global__ __launch_bounds__(NTF) void wkv6_fwd_ws(const ArgsC a) {
 
 int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                           const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
-                          const uint16_t* s0, uint16_t* y, float* saved) {
+                          const uint16_t* s0, uint16_t* y, float* saved, const int* only_flagged) {
     ArgsC a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y; a.saved = saved;
+    a.only_flagged = only_flagged;
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_fwd_ws<W_RAW>, dim3(B * H), dim3(NTF), 0, st, a);
     else if (wmode == W_EW) hipLaunchKernelGGL(wkv6_fwd_ws<W_EW>, dim3(B * H), dim3(NTF), 0, st, a);
     else hipLaunchKernelGGL(wkv6_fwd_ws<W_HEAD>, dim3(B * H), dim3(NTF), 0, st, a);

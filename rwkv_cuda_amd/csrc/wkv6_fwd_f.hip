@@ -1,0 +1,403 @@
+// wkv6 / wkv6_state forward (gfx950) that keeps the state entering every second chunk for the one-sweep backward
+// (wkv6_bwd_f.hip), built like that kernel: wave roles, operands from [token][channel] planes, one barrier per chunk.
+//
+// Formulas (wkv6_chunk.h for R', K', d1, d2, dec; chunk of L = 32 tokens, factors referred to its middle m = 16):
+//     A[t][s] = R'_t . K'_s (s < t),  A[t][t] = sum_j r u k
+//     y_t = (S d1) R'_t + sum_{s<=t} A[t][s] v_s              S <- S dec + d2 V^T K'
+//
+// One workgroup of 16 waves per (batch, head):
+//   P  (prep, 8 waves)  channels 8w..8w+7 of r, k, w, v for all 32 tokens of a chunk: lane = 16 * (channel pair) + token.
+//                       Writes the bf16 hi / lo planes of R', K' and plain v, the per-channel factors and the diagonal
+//                       of A; stores the finished y rows of the chunk three iterations back.
+//   S  (state, 4 waves) S[i][j], value channels i = 16w..: lane = i, registers = j.  y, the state update, the saved state.
+//   T  (tiles, 3 of 4 waves) the causal tile A of the next chunk, one 16 x 16 quadrant each; the fourth wave moves the
+//                       states to be saved from LDS to global memory.
+// Pipeline: in iteration `it` the P waves prepare chunk it, the T waves make the tile of chunk it-1, the S waves do the
+// products of chunk it-2 and the P waves store the y of chunk it-3.
+//
+// Global memory is touched 16 bytes per lane: a prep lane moves one row piece (its wave's 8 channels of one token) and
+// the pieces change lane order in LDS; y leaves through an LDS tile so that whole 128-byte rows are written.
+//
+// A chunk in which some channel decays by more than e^-60 over either half cannot use the mid-point factors.  Such a
+// (batch, head) is flagged in `flags` and the caller reruns it with wkv6_fwd_ws, which has a step-by-step path.
+#include "wkv6_fused.h"
+
+namespace rwkv {
+namespace {
+
+constexpr int NTQ = 16 * 64;
+constexpr int PS = 36;             // bf16 [token][channel] planes: 144 B per row (see wkv6_bwd_f.hip)
+constexpr int DEPTH = 4;           // chunks that the prep waves load ahead (a power of two)
+constexpr int SS = 68;             // fp32 [value][key] state: 272 B per row
+
+struct alignas(16) SlotQ {
+    uint32_t RpH[L][PS], RpL[L][PS], KpH[L][PS], KpL[L][PS], V[L][PS];
+    float d1[N], d2[N], dec[N];            // 2^{c_m}, 2^{c_L - c_m}, 2^{c_L}
+    float ruk[8][L];                        // sum of r u k over the 8 channels of each prep wave
+};
+struct alignas(16) TilesQ {
+    uint32_t AH[L][AS], AL[L][AS];         // [t][s] bf16 hi / lo
+};
+struct alignas(16) SmemQ {
+    SlotQ slot[3];
+    TilesQ tile[2];
+    uint32_t yb[2][L][PS];                  // y of the last two chunks, bf16 [token][channel]
+    float sst[N][SS];                       // the state entering an even chunk, on its way to global memory
+};
+constexpr lds_t ROW_B = PS * 4, PLANE_B = L * ROW_B, TROW_B = AS * 4;
+constexpr lds_t O_RPH = 0, O_RPL = PLANE_B, O_KPH = 2 * PLANE_B, O_KPL = 3 * PLANE_B, O_V = 4 * PLANE_B;
+constexpr lds_t O_D1 = 5 * PLANE_B, O_D2 = O_D1 + 4 * N, O_DEC = O_D2 + 4 * N, O_RUK = O_DEC + 4 * N;
+constexpr lds_t SLOT_B = sizeof(SlotQ), SLOT0 = offsetof(SmemQ, slot);
+constexpr lds_t T_AH = 0, T_AL = L * TROW_B, TILE_B = sizeof(TilesQ), TILE0 = offsetof(SmemQ, tile), YB0 = offsetof(SmemQ, yb), SST0 = offsetof(SmemQ, sst);
+static_assert(offsetof(SlotQ, V) == O_V && offsetof(SlotQ, d1) == O_D1 && offsetof(SlotQ, ruk) == O_RUK && offsetof(TilesQ, AL) == T_AL, "layout");
+
+struct ArgsQ {
+    int T, C, H;
+    const uint16_t *r, *k, *v, *w, *u, *s0;
+    uint16_t* y;
+    float* saved;                  // [B*H][ceil(n/2)][64][64]: the state entering every even chunk, [value][key]
+    int* flags;                    // [B*H][8]
+};
+
+// ---------------------------------------------------------------------------------------------------- P waves
+DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n, const int nit) {
+    int jq = lane >> 4, tp = lane & 15;                 // arithmetic: channel pair, token (and token + 16)
+    int hl = lane >> 5, rw = lane & 31;                 // memory: which tensor, which row of the chunk
+    int rw8 = lane;                                     // y: row 8 (w & 3) + lane / 8, piece lane % 8
+    const int ch0 = 8 * w + 2 * (lane >> 4);
+    const int hl0 = lane >> 5;
+    const int T = a.T, C = a.C;
+    const uint16_t* __restrict__ pA = (hl0 ? a.k : a.r) + base + 8 * w;      // r | k
+    const uint16_t* __restrict__ pB = (hl0 ? a.v : a.w) + base + 8 * w;      // w | v
+    float uj[2];
+    {
+        const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + ch0);
+        uj[0] = bf_lo(x); uj[1] = bf_hi(x);
+    }
+    struct Raw { u32x4 a, b; };
+    // Little's law sets the depth: 256 workgroups x 8 waves x 2 KB per chunk are 4 MB, the memory system answers after
+    // two to three microseconds under load, and a chunk is to take little more than one.
+    Raw ring[DEPTH];                       // DEPTH chunks ahead
+    auto fetch = [&](const int c, Raw& x) __attribute__((always_inline)) {
+        const int t = c * L + rw;
+        const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C;
+        x.a = *reinterpret_cast<const u32x4*>(pA + o);
+        x.b = *reinterpret_cast<const u32x4*>(pB + o);
+    };
+    // the pieces of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v in place
+    auto stage_in = [&](const int c, const Raw& x, auto PARTIAL) __attribute__((always_inline)) {
+        SlotQ& O = S.slot[c % 3];
+        const bool live = !decltype(PARTIAL)::value || c * L + rw < T;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        uint32_t* da = &O.RpH[rw][4 * w] + hl * (2 * L * PS);        // R' hi | K' hi
+        uint32_t* db = &O.RpL[rw][4 * w] + hl * (3 * L * PS);        // R' lo | V
+        *reinterpret_cast<u32x4*>(da) = live ? x.a : zero;
+        *reinterpret_cast<u32x4*>(db) = (live || !hl) ? x.b : zero;  // w of a dead row is masked where the decay is formed
+    };
+    bool any_exact = false;
+    auto prep = [&](const int c, auto PARTIAL) __attribute__((always_inline)) {
+        const int ch = 8 * w + 2 * jq, cd = 4 * w + jq;        // cd: dword column of the pair in a bf16 plane
+        SlotQ& O = S.slot[c % 3];
+        float lam[2][2], rf[2][2], kf[2][2], cc[2][2];
+        uint32_t xr[2], xk[2], xw[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) { xr[e] = O.RpH[tp + 16 * e][cd]; xk[e] = O.KpH[tp + 16 * e][cd]; xw[e] = O.RpL[tp + 16 * e][cd]; }
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const bool live = !decltype(PARTIAL)::value || c * L + tp + 16 * e < T;
+            rf[e][0] = bf_lo(xr[e]); rf[e][1] = bf_hi(xr[e]);
+            kf[e][0] = bf_lo(xk[e]); kf[e][1] = bf_hi(xk[e]);
+            lam[e][0] = live ? -LOG2E * exp2_fast(LOG2E * bf_lo(xw[e])) : 0.f;
+            lam[e][1] = live ? -LOG2E * exp2_fast(LOG2E * bf_hi(xw[e])) : 0.f;
+        }
+        float l1[2], l2[2];
+#pragma unroll
+        for (int z = 0; z < 2; ++z) {
+            const float s0 = row_suffix_sum(lam[0][z]);        // sum over tokens tp..15
+            const float p1 = row_prefix_sum(lam[1][z]);        // sum over tokens 16..16+tp
+            cc[0][z] = -s0;
+            cc[1][z] = p1 - lam[1][z];
+            l1[z] = bc<0>(s0);
+            l2[z] = bc<15>(p1);
+        }
+        {
+            const bool bad = (-l1[0] > RANGE_LIMIT * LOG2E) || (-l2[0] > RANGE_LIMIT * LOG2E) || (-l1[1] > RANGE_LIMIT * LOG2E) || (-l2[1] > RANGE_LIMIT * LOG2E);
+            any_exact = any_exact || (__ballot(bad) != 0ull);
+        }
+        if (tp == 0) {
+            const float a0 = exp2_fast(l1[0]), a1 = exp2_fast(l1[1]), b0 = exp2_fast(l2[0]), b1 = exp2_fast(l2[1]);
+            *reinterpret_cast<float2*>(&O.d1[ch]) = make_float2(a0, a1);
+            *reinterpret_cast<float2*>(&O.d2[ch]) = make_float2(b0, b1);
+            *reinterpret_cast<float2*>(&O.dec[ch]) = make_float2(a0 * b0, a1 * b1);
+        }
+        float ruk[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int t = tp + 16 * e;
+            const float rp0 = rf[e][0] * exp2_fast(cc[e][0]), rp1 = rf[e][1] * exp2_fast(cc[e][1]);
+            const float kp0 = kf[e][0] * exp2_fast(-(cc[e][0] + lam[e][0])), kp1 = kf[e][1] * exp2_fast(-(cc[e][1] + lam[e][1]));
+            ruk[e] = fmaf(rf[e][0] * uj[0], kf[e][0], rf[e][1] * uj[1] * kf[e][1]);
+            const HL r0 = hilo2(rp0, rp1), k0 = hilo2(kp0, kp1);
+            O.RpH[t][cd] = r0.h; O.RpL[t][cd] = r0.l;
+            O.KpH[t][cd] = k0.h; O.KpL[t][cd] = k0.l;
+        }
+        allreduce2_rows(ruk[0], ruk[1]);                       // sums over the four channel pairs of this wave
+        if (jq == 0) { O.ruk[w][tp] = ruk[0]; O.ruk[w][tp + 16] = ruk[1]; }
+    };
+    // The y rows of chunk c, left in LDS by the S waves in the last iteration: waves 0..3 store eight rows each, eight
+    // lanes per 128-byte row, so that the memory system sees whole lines and not the 16-byte pieces of the loads.
+    // (A store on every path, masked per lane, so that the waits for the prefetched inputs count the same on all of them.)
+    uint16_t* __restrict__ pY = a.y + base + 8 * (lane & 7);
+    auto store_y = [&](const int c, const bool on) __attribute__((always_inline)) {
+        const int row = 8 * (w & 3) + (rw8 >> 3);
+        const u32x4 o = *reinterpret_cast<const u32x4*>(&S.yb[c & 1][row][4 * (rw8 & 7)]);
+        const int tg = c * L + row;
+        if (on && w < 4 && tg < T) *reinterpret_cast<u32x4*>(pY + static_cast<uint32_t>(tg) * C) = o;
+    };
+
+    const std::true_type part{};           // only the last chunk can be cut short
+    const std::false_type full{};
+    // in the order in which the loop consumes them: its waits are counted from the worst of all the ways into it
+    static_for<DEPTH>([&](auto Z) {
+        constexpr int z = decltype(Z)::value;
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(z < n ? z : n - 1, ring[z]);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+    // DEPTH iterations per trip, nothing in them skipped: a way round a stage, or round the second half, would be one more
+    // way into the next wait, on which the registers it waits for are the newest loads (the count then covers everything).
+    // Past the last chunk the stages run on rows that all count as dead, into a slot nobody reads.
+    for (int it0 = 0; it0 < nit; it0 += DEPTH)
+        static_for<DEPTH>([&](auto Z) {
+            constexpr int z = decltype(Z)::value;
+            const int it = it0 + z;
+            asm volatile("" : "+v"(jq), "+v"(tp), "+v"(hl), "+v"(rw), "+v"(rw8));
+            if (it >= n - 1) stage_in(it, ring[z], part); else stage_in(it, ring[z], full);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(it + DEPTH < n ? it + DEPTH : n - 1, ring[z]);
+            __builtin_amdgcn_sched_barrier(0);
+            store_y(it >= 3 ? it - 3 : 0, it >= 3);
+            __builtin_amdgcn_sched_barrier(0);
+            if (it >= n - 1) prep(it, part); else prep(it, full);
+            __syncthreads();
+        });
+    if (lane == 0) a.flags[bh * 8 + w] = any_exact ? 1 : 0;
+}
+
+// ---------------------------------------------------------------------------------------------------- S waves
+DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, const size_t bh, const int n, const int nit) {
+    const int g = lane >> 4, l16 = lane & 15, i = 16 * w + l16;
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    const lds_t sb = lds_of(&S);
+    lds_t b_acc = l16 * ROW_B + 8 * g;                                          // [token l16][channel 4 g] of a plane
+    lds_t b_tr = ((8 * g + (l16 >> 2)) * PS + 2 * (l16 & 3)) * 4;               // transposing read of a plane, rows 8 g ..
+    lds_t b_natt = l16 * TROW_B + 16 * g;                                       // [row l16][position 8 g] of a tile
+    lds_t b_g = 16 * g + 4 * (l16 & 3);                                          // channel 4 g + (l16 & 3) of a per-channel array
+    const uint32_t b_sv = i * N + 4 * g;                                        // [value channel i][key channel 4 g] of a state
+    lds_t b_ss = (i * SS + 4 * g) * 4;                                          // the same in the LDS copy
+    f32x4 St[4];                           // S[i = 16w + l16][j = 16 tile + 4g + v]
+    if (a.s0 != nullptr) {
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) {
+            const uint2 x = *reinterpret_cast<const uint2*>(a.s0 + bh * (N * N) + b_sv + 16 * tl);
+            St[tl] = f32x4{bf_lo(x.x), bf_hi(x.x), bf_lo(x.y), bf_hi(x.y)};
+        }
+    } else {
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) St[tl] = zero4;
+    }
+    __syncthreads();                       // iterations 0 and 1: nothing prepared yet
+    __syncthreads();
+#pragma unroll 1
+    for (int c = 0; c < n; ++c) {
+        opaque(b_acc); opaque(b_tr); opaque(b_natt); opaque(b_g); opaque(b_ss);
+        const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
+        if (!(c & 1)) {
+            // The state entering an even chunk goes to LDS and from there, in the next iteration, to global memory through
+            // a wave that has nothing else to do: every workgroup writes its 16 KB at about the same moment, the memory
+            // system takes a while to accept such a burst, and a state wave that waited for that would hold up the chunk.
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl) lds_st<f32x4>(sb + SST0 + 64 * tl + b_ss, St[tl]);
+        }
+        // ------------------------------------------------------------ batch 1: d1 and R' (natural rows)
+        // per-channel factors: a lane holds the one of channel 16 tile + 4 g + (l16 & 3), a 4-byte read that all rows of
+        // four lanes share; the products below take lane v of the 16-lane row inside the multiply (row_newbcast)
+        float dq[4], de[4], d2[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            dq[q] = lds_ld<float>(so + O_D1 + 64 * q + b_g);
+            de[q] = lds_ld<float>(so + O_DEC + 64 * q + b_g);
+            d2[q] = lds_ld<float>(so + O_D2 + 64 * q + b_g);
+        }
+        bf16x8 rh[2][2], rl[2][2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                rh[tt][ks] = ld_acc(so + O_RPH + tt * 16 * ROW_B + 64 * ks + b_acc);
+                rl[tt][ks] = ld_acc(so + O_RPL + tt * 16 * ROW_B + 64 * ks + b_acc);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+        // ------------------------------------------------------------ y^T[i][t] = (S d1) R'^T + V^T A^T
+        bf16x8 sh[2], sl[2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            float p[4], q[4];
+            static_for<4>([&](auto V) {
+                constexpr int v = decltype(V)::value;
+                p[v] = St[2 * ks][v]; q[v] = St[2 * ks + 1][v];
+                mul_bc<v>(p[v], dq[2 * ks]); mul_bc<v>(q[v], dq[2 * ks + 1]);
+            });
+            const HL x0 = hilo2(p[0], p[1]), x1 = hilo2(p[2], p[3]), x2 = hilo2(q[0], q[1]), x3 = hilo2(q[2], q[3]);
+            sh[ks] = as_op(x0.h, x1.h, x2.h, x3.h);
+            sl[ks] = as_op(x0.l, x1.l, x2.l, x3.l);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // ------------------------------------------------------------ batch 2: v with the tokens along K, the A tile by rows
+        const bf16x8 vop = ld_tr(so + O_V + 32 * w + b_tr, ROW_B);              // lane = value channel 16w + l16, K = tokens
+        bf16x8 ah[2], al[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) { ah[tt] = ld_op(to + T_AH + tt * 16 * TROW_B + b_natt); al[tt] = ld_op(to + T_AL + tt * 16 * TROW_B + b_natt); }
+        __builtin_amdgcn_sched_barrier(0);
+        f32x4 Y[2] = {zero4, zero4};
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+                Y[tt] = mfma(sh[ks], rh[tt][ks], Y[tt]);
+                Y[tt] = mfma(sh[ks], rl[tt][ks], Y[tt]);
+                Y[tt] = mfma(sl[ks], rh[tt][ks], Y[tt]);
+            }
+        __builtin_amdgcn_sched_barrier(0);
+        // ------------------------------------------------------------ batch 3: K' with the tokens along K
+        bf16x8 kh[4], kl[4];
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) { kh[tl] = ld_tr(so + O_KPH + 32 * tl + b_tr, ROW_B); kl[tl] = ld_tr(so + O_KPL + 32 * tl + b_tr, ROW_B); }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+            Y[tt] = mfma(vop, ah[tt], Y[tt]);
+            Y[tt] = mfma(vop, al[tt], Y[tt]);
+        }
+        f32x4 U[4];
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) {
+            U[tl] = mfma(kh[tl], vop, zero4);
+            U[tl] = mfma(kl[tl], vop, U[tl]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // y: lane = token, four consecutive value channels in registers
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt)
+            lds_st<u32x2>(sb + YB0 + (c & 1) * PLANE_B + tt * 16 * ROW_B + 32 * w + b_acc, u32x2{pack_bf2(Y[tt][0], Y[tt][1]), pack_bf2(Y[tt][2], Y[tt][3])});
+        // ------------------------------------------------------------ S^T <- S^T dec + d2 K'^T V
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl)
+            static_for<4>([&](auto V) {
+                constexpr int v = decltype(V)::value;
+                float x = St[tl][v];
+                mul_bc<v>(x, de[tl]);
+                fmac_bc<v>(x, d2[tl], U[tl][v]);
+                St[tl][v] = x;
+            });
+        __syncthreads();
+    }
+    for (int it = n + 2; it < nit; ++it) __syncthreads();      // the P waves store the last y
+}
+
+// ---------------------------------------------------------------------------------------------------- T waves
+DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, const size_t bh, const int n, const int nit) {
+    const int g = lane >> 4, l16 = lane & 15;
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    const lds_t sb = lds_of(&S);
+    lds_t b_nat = l16 * ROW_B + 16 * g;                                         // [token l16][channel 8 g] of a plane
+    lds_t b_tw = l16 * TROW_B + 8 * g;                                          // [row l16][position 4 g] of a tile
+    lds_t b_l = 4 * l16;
+    // wave 0, 1, 2 -> quadrant (t, s) = (0,0) (1,0) (1,1); accumulator rows are s, lanes t
+    const int ta = (w == 0) ? 0 : 1, tb = (w == 2) ? 1 : 0;
+    // wave 3: the state that the S waves left in LDS in the last iteration; a lane moves 16 bytes of a row, 4 rows a time
+    lds_t b_sr = ((lane >> 4) * SS + 4 * (lane & 15)) * 4;
+    float* __restrict__ sv = a.saved + bh * ((n + 1) / 2) * (N * N) + (lane >> 4) * N + 4 * (lane & 15);
+    __syncthreads();                       // iteration 0
+#pragma unroll 1
+    for (int c = 0; c < nit - 1; ++c) {    // iteration c + 1
+        opaque(b_nat); opaque(b_tw); opaque(b_l); opaque(b_sr);
+        if (w == 3 && c >= 2 && c - 2 < n && !(c & 1)) {
+            float* dst = sv + static_cast<size_t>((c - 2) >> 1) * (N * N);
+#pragma unroll
+            for (int q = 0; q < 16; q += 4) {
+                f32x4 x[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) x[e] = lds_ld<f32x4>(sb + SST0 + (q + e) * (4 * SS * 4) + b_sr);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) *reinterpret_cast<f32x4*>(dst + (q + e) * (4 * N)) = x[e];
+            }
+        }
+        if (c < n && w < 3) {
+            const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
+            const lds_t ra = so + ta * 16 * ROW_B + b_nat, rb = so + tb * 16 * ROW_B + b_nat;
+            bf16x8 kh[2], kl[2], rh[2], rl[2];
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                kh[ks] = ld_op(rb + O_KPH + 64 * ks); kl[ks] = ld_op(rb + O_KPL + 64 * ks);
+                rh[ks] = ld_op(ra + O_RPH + 64 * ks); rl[ks] = ld_op(ra + O_RPL + 64 * ks);
+            }
+            float d = 0.f;
+            if (ta == tb) {
+                const lds_t ru = so + O_RUK + ta * 64 + b_l;
+#pragma unroll
+                for (int q = 0; q < 8; ++q) d += lds_ld<float>(ru + q * (4 * L));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            f32x4 a0 = zero4, a1 = zero4;
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                a0 = mfma(kh[ks], rh[ks], a0);
+                a1 = mfma(kh[ks], rl[ks], a1);
+                a1 = mfma(kl[ks], rh[ks], a1);
+            }
+            f32x4 am = a0 + a1;                                // [v]: s = 16 tb + 4g + v, t = 16 ta + l16
+            if (ta == tb) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int sl = 4 * g + v;
+                    am[v] = (sl < l16) ? am[v] : (sl == l16 ? d : 0.f);
+                }
+            }
+            const HL x0 = hilo2(am[0], am[1]), x1 = hilo2(am[2], am[3]);
+            const lds_t tw = to + ta * 16 * TROW_B + tb * 32 + b_tw;
+            lds_st<u32x2>(tw + T_AH, u32x2{x0.h, x1.h});
+            lds_st<u32x2>(tw + T_AL, u32x2{x0.l, x1.l});
+        }
+        __syncthreads();
+    }
+}
+
+__global__ __launch_bounds__(NTQ) void wkv6_fwd_fused(const ArgsQ a) {
+    __shared__ SmemQ S;
+    const int tid = threadIdx.x;
+    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
+    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
+    const size_t bh = static_cast<size_t>(b) * a.H + h;
+    const int n = (a.T + L - 1) / L;
+    // the quadrant t < 16 <= s of the tiles is never written and must read as zero
+    for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTQ) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
+    __syncthreads();
+    const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
+    const int nit = (n + 2 + DEPTH) & ~(DEPTH - 1);        // iterations of the pipeline: n + 3, in whole trips of the prep loop
+    if (wid < 8) role_prep(S, a, lane, wid, base, h, bh, n, nit);
+    else if (wid < 12) role_state(S, a, lane, w, bh, n, nit);
+    else role_tiles(S, a, lane, w, bh, n, nit);
+}
+
+}  // namespace
+
+int launch_wkv6_fwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
+                          const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, float* saved, int* flags) {
+    ArgsQ a{};
+    a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y; a.saved = saved; a.flags = flags;
+    hipLaunchKernelGGL(wkv6_fwd_fused, dim3(B * H), dim3(NTQ), 0, st, a);
+    return launch_status();
+}
+
+}  // namespace rwkv

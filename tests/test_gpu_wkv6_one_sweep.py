@@ -78,7 +78,7 @@ def test_one_sweep_hands_strong_decays_to_the_two_sweep_kernels(lib):
 
 
 def test_one_sweep_agrees_with_the_two_sweep_kernels(lib):
-    """Same inputs through both backward paths of the library: the gradients differ by at most one bf16 unit of the
+    """Same inputs through both pairs of kernels of the library: the results differ by at most one bf16 unit of the
     tensor's peak (they round the same fp32 quantities, formed in a different order)."""
     B, T, H = 2, 333, 2
     C = H * 64
@@ -93,8 +93,7 @@ def test_one_sweep_agrees_with_the_two_sweep_kernels(lib):
     ws = torch.empty(n, device=DEV, dtype=torch.uint8)
     call("rwkv_wkv6f_backward", DEV, B, T, C, H, *d[:6], d[6], gr, gk, gv, gw, gu, gs, ws, n, 0)
     torch.cuda.synchronize()
-    assert torch.equal(one[0], y)                              # the same forward kernel either way
-    for name, a, b in zip(NAMES[1:], one[1:], [gr, gk, gv, gw, gu, gs]):
+    for name, a, b in zip(NAMES, one, [y, gr, gk, gv, gw, gu, gs]):
         diff = float((a.float() - b.float()).abs().max()) / float(b.float().abs().max())
         print(f"  {name}: max difference {diff:.2e} of the peak", flush=True)
         assert diff <= 2.0 ** -7, name
@@ -141,7 +140,7 @@ def test_one_sweep_rejects_bad_arguments(lib):
     r, k, v, w, u, gy, _ = (x.to(DEV) if x is not None else None for x in synth.wkv6_inputs(B, T, C, H, seed=1))
     y = torch.empty((B, T, C), device=DEV, dtype=BF)
     nsv = lib.rwkv_wkv6f_saved_bytes(B, T, C, H)
-    assert nsv == 64 * 64 * 4                                   # one segment of 64 tokens
+    assert nsv == 64 * 64 * 4 + 32                              # one segment of 64 tokens, eight flag words
     saved = torch.empty(nsv, device=DEV, dtype=torch.uint8)
     st = torch.cuda.current_stream().cuda_stream
     p = lambda t: t.data_ptr()
