@@ -43,6 +43,7 @@ constexpr int NTG = 16 * 64;
 // times the rate of 72 (16-byte reads and the transposing reads do not care).
 constexpr int PS = 36;             // bf16 [token][channel] planes: 144 B
 constexpr int CS = 68;             // fp32 [token][channel] arrays: 272 B
+constexpr int TQ = 20;             // causal tiles [t][s], 32 bf16 and 16 bytes of padding: 80 B (16-byte reads of 16 rows hit all banks once)
 
 struct alignas(16) SlotG {
     uint32_t RpH[L][PS], RpL[L][PS], KpH[L][PS], KpL[L][PS], V[L][PS], GY[L][PS];
@@ -50,22 +51,24 @@ struct alignas(16) SlotG {
     float ruk[8][L];                        // sum of r u k over the 8 channels of each prep wave
 };
 struct alignas(16) TilesG {
-    uint32_t AH[L][AS], AL[L][AS], BH[L][AS], BL[L][AS];   // [t][s] bf16 hi / lo
+    uint32_t AH[L][TQ], AL[L][TQ], BH[L][TQ], BL[L][TQ];   // [t][s] bf16 hi / lo
 };
 struct alignas(16) SmemG {
     SlotG slot[3];
     TilesG tile[2];
     float xz[2][2][L][CS];                  // [chunk parity][X, Z][token][key channel]: from the SD waves to the P waves
-    float vg[4][L];                         // v_t . gy_t of the chunks in flight
+    float vg[3][L];                         // v_t . gy_t of the chunks in flight
     float pex[2][N];                        // P = sum_i dS S at the last two anchors
+    uint32_t out[4][L][PS];                 // gr, gk, gw, gv of one chunk, bf16 [token][channel], on their way to global memory
+    uint32_t met[3];                        // meeting counters: inputs staged, results written, gv taken
 };
 static_assert(sizeof(SmemG) <= 160 * 1024, "LDS");
-constexpr lds_t ROW_B = PS * 4, PLANE_B = L * ROW_B, TROW_B = AS * 4, XROW_B = CS * 4, XZ_B = L * XROW_B;
+constexpr lds_t ROW_B = PS * 4, PLANE_B = L * ROW_B, TROW_B = TQ * 4, XROW_B = CS * 4, XZ_B = L * XROW_B;
 constexpr lds_t O_RPH = 0, O_RPL = PLANE_B, O_KPH = 2 * PLANE_B, O_KPL = 3 * PLANE_B, O_V = 4 * PLANE_B, O_GY = 5 * PLANE_B;
 constexpr lds_t O_D1 = 6 * PLANE_B, O_D2 = O_D1 + 4 * N, O_DEC = O_D2 + 4 * N, O_L2 = O_DEC + 4 * N, O_RUK = O_L2 + 4 * N;
 constexpr lds_t SLOT_B = sizeof(SlotG), SLOT0 = offsetof(SmemG, slot);
 constexpr lds_t T_AH = 0, T_AL = L * TROW_B, T_BH = 2 * L * TROW_B, T_BL = 3 * L * TROW_B, TILE_B = sizeof(TilesG), TILE0 = offsetof(SmemG, tile);
-constexpr lds_t XZ0 = offsetof(SmemG, xz), VG0 = offsetof(SmemG, vg), PEX0 = offsetof(SmemG, pex);
+constexpr lds_t XZ0 = offsetof(SmemG, xz), VG0 = offsetof(SmemG, vg), PEX0 = offsetof(SmemG, pex), OUT0 = offsetof(SmemG, out);
 static_assert(offsetof(SlotG, GY) == O_GY && offsetof(SlotG, d1) == O_D1 && offsetof(SlotG, ruk) == O_RUK && offsetof(TilesG, BL) == T_BL, "layout");
 
 
@@ -95,19 +98,20 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     int jq = lane >> 4, tp = lane & 15;
     const int ch0 = 8 * w + 2 * (lane >> 4);
     const int T = a.T, C = a.C;
-    // Global memory is touched in another lane order than the arithmetic: a lane moves one 16-byte row piece (this wave's
-    // 8 channels of one token) of one tensor, so that a wave needs three loads and two stores per chunk instead of
-    // sixteen four-byte accesses to sixteen rows each.  The pieces cross to the arithmetic's lane order (and back)
-    // through this wave's own columns of LDS arrays that are free at that moment: the planes of the slot being
-    // prepared on the way in, the X / Z cells just consumed on the way out.  Only this wave touches those columns and
-    // LDS serves a wave's accesses in order, so no barrier is involved.
-    int hl = lane >> 5, rw = lane & 31;
-    const int hl0 = lane >> 5;
-    const uint16_t* __restrict__ pA = (hl0 ? a.k : a.r) + base + 8 * w;                                  // r | k
-    const uint16_t* __restrict__ pB = (hl0 ? a.v : static_cast<const uint16_t*>(a.w)) + base + 8 * w;   // w | v
-    const uint16_t* __restrict__ pC = a.gy + base + 8 * w;                                               // gy (both halves)
-    uint16_t* __restrict__ pS1 = (hl0 ? a.gk : a.gr) + base + 8 * w;                                     // gr | gk
-    uint16_t* __restrict__ pS2 = a.gw + base + 8 * w;                                                    // gw (first half)
+    // Global memory is touched in whole 128-byte rows, 16 bytes per lane and eight lanes per row: the memory system takes
+    // requests for pieces of a line, one from each of eight waves, at a much lower rate.  Per chunk a wave loads rows
+    // 8 (w & 3) .. +7 of two tensors (waves 0..3: r and w, waves 4..7: k and v) and rows 4 w .. +3 of gy, and stores rows
+    // 8 (w & 3) .. +7 of two (gr and gw, or gk and gv).  So a wave stages columns that other waves prepare, and stores
+    // columns that other waves have finished: the planes of the slot being prepared carry the inputs, `out` the results,
+    // and the prep waves meet (meet_signal / meet_wait) between writing and reading them.
+    int rq = lane >> 3, pc = lane & 7, rg = (lane & 31) >> 3;
+    const int wq = w & 3;
+    const bool lower = w < 4;
+    const uint16_t* __restrict__ pA = (lower ? a.r : a.k) + base + 8 * (lane & 7);                                  // r | k
+    const uint16_t* __restrict__ pB = (lower ? static_cast<const uint16_t*>(a.w) : a.v) + base + 8 * (lane & 7);   // w | v
+    const uint16_t* __restrict__ pC = a.gy + base + 8 * (lane & 7);
+    uint16_t* __restrict__ pS1 = (lower ? a.gr : a.gk) + base + 8 * (lane & 7);
+    uint16_t* __restrict__ pS2 = (lower ? a.gw : a.gv) + base + 8 * (lane & 7);
     float uj[2];
     {
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + ch0);
@@ -116,27 +120,29 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     struct Raw { u32x4 a, b, c; };
     Raw ring[2];                           // two chunks ahead
     auto fetch = [&](const int c, Raw& x) __attribute__((always_inline)) {
-        const int t = c * L + rw;
-        const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C;
+        const int t = c * L + 8 * wq + rq, tg = c * L + 4 * w + rg;
+        const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C, og = static_cast<uint32_t>(tg < T ? tg : T - 1) * C;
         x.a = *reinterpret_cast<const u32x4*>(pA + o);
         x.b = *reinterpret_cast<const u32x4*>(pB + o);
-        x.c = *reinterpret_cast<const u32x4*>(pC + o);
+        x.c = *reinterpret_cast<const u32x4*>(pC + og);    // (both halves of the wave ask for the same four rows)
     };
-    // the pieces of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v and gy in place
+    // the rows of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v and gy in place
     auto stage_in = [&](const int c, const Raw& x, auto PARTIAL) __attribute__((always_inline)) {
         SlotG& O = S.slot[(c + 6) % 3];
-        const bool live = !decltype(PARTIAL)::value || (c >= 0 && c * L + rw < T);
+        const int row = 8 * wq + rq, rowg = 4 * w + rg;
+        const bool live = !decltype(PARTIAL)::value || (c >= 0 && c * L + row < T);
+        const bool liveg = !decltype(PARTIAL)::value || (c >= 0 && c * L + rowg < T);
         const u32x4 zero = {0u, 0u, 0u, 0u};
-        uint32_t* da = &O.RpH[rw][4 * w] + hl * (2 * L * PS);        // R' hi | K' hi
-        uint32_t* db = &O.RpL[rw][4 * w] + hl * (3 * L * PS);        // R' lo | V
+        uint32_t* da = lower ? &O.RpH[row][4 * pc] : &O.KpH[row][4 * pc];
+        uint32_t* db = lower ? &O.RpL[row][4 * pc] : &O.V[row][4 * pc];
         *reinterpret_cast<u32x4*>(da) = live ? x.a : zero;
-        *reinterpret_cast<u32x4*>(db) = (live || !hl) ? x.b : zero;  // w of a dead row is masked where the decay is formed
-        if (!hl) *reinterpret_cast<u32x4*>(&O.GY[rw][4 * w]) = live ? x.c : zero;
+        *reinterpret_cast<u32x4*>(db) = (live || lower) ? x.b : zero;    // w of a dead row is masked where the decay is formed
+        if (lane < 32) *reinterpret_cast<u32x4*>(&O.GY[rowg][4 * pc]) = liveg ? x.c : zero;
     };
     // what the finishing of a chunk needs from its preparation, three iterations earlier
     struct Held { uint32_t r[2], k[2]; float cc[2][2]; };
     Held hq[3] = {};
-    bool any_exact = false;
+    bool any_exact = false, met_ok = true;
     float carry[2] = {0.f, 0.f}, gu_acc[2] = {0.f, 0.f};
     // Only the last chunk of the sequence can be cut short (PARTIAL): its rows past T carry no input and no decay.
 
@@ -204,7 +210,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             const float2 x2 = *reinterpret_cast<const float2*>(&S.xz[c & 1][0][t][ch]);
             const float2 z2 = *reinterpret_cast<const float2*>(&S.xz[c & 1][1][t][ch]);
             const float X[2] = {x2.x, x2.y}, Z[2] = {z2.x, z2.y};
-            const float vg = S.vg[c & 3][t];
+            const float vg = S.vg[c % 3][t];
             const float rf[2] = {bf_lo(hd.r[e]), bf_hi(hd.r[e])}, kf[2] = {bf_lo(hd.k[e]), bf_hi(hd.k[e])};
             float gr[2], gk[2];
 #pragma unroll
@@ -221,9 +227,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
                 gu_acc[z] = fmaf(rf[z] * kf[z], vg, gu_acc[z]);
                 lam[e][z] = gw_factor((ccn - cc) * LN2);
             }
-            // X and Z of this thread are in registers: their cells now carry the results to the lanes that store them
-            reinterpret_cast<uint32_t*>(&S.xz[c & 1][0][t][8 * w])[jq] = pack_bf2(gr[0], gr[1]);
-            reinterpret_cast<uint32_t*>(&S.xz[c & 1][0][t][8 * w + 4])[jq] = pack_bf2(gk[0], gk[1]);
+            S.out[0][t][4 * w + jq] = pack_bf2(gr[0], gr[1]);
+            S.out[1][t][4 * w + jq] = pack_bf2(gk[0], gk[1]);
         }
         float gw[2][2];
 #pragma unroll
@@ -242,15 +247,22 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         // without an initial state nothing has been accumulated before token 0: its decay has no effect at all
         if (a.gs == nullptr && c == 0 && tp == 0) { gw[0][0] = 0.f; gw[0][1] = 0.f; }
 #pragma unroll
-        for (int e = 0; e < 2; ++e) reinterpret_cast<uint32_t*>(&S.xz[c & 1][1][tp + 16 * e][8 * w])[jq] = pack_bf2(gw[e][0], gw[e][1]);
-        // one 16-byte row piece per lane: gr | gk, then gw
-        const u32x4 o1 = *reinterpret_cast<const u32x4*>(&S.xz[c & 1][0][rw][8 * w + 4 * hl]);
-        const u32x4 o2 = *reinterpret_cast<const u32x4*>(&S.xz[c & 1][1][rw][8 * w]);
-        const int tg = c * L + rw;
-        if (!decltype(PARTIAL)::value || tg < T) {
-            const uint32_t o = static_cast<uint32_t>(tg) * C;
-            *reinterpret_cast<u32x4*>(pS1 + o) = o1;
-            if (!hl) *reinterpret_cast<u32x4*>(pS2 + o) = o2;
+        for (int e = 0; e < 2; ++e) S.out[2][tp + 16 * e][4 * w + jq] = pack_bf2(gw[e][0], gw[e][1]);
+    };
+    // rows 8 (w & 3) .. +7 of the results of chunk c: gv, which the E waves left in the last iteration, at once (they
+    // wait for this before they write the next); the other three when all prep waves have finished their columns
+    auto store_gv = [&](const int c, const bool on) __attribute__((always_inline)) {
+        const int row = 8 * wq + rq, tg = c * L + row;
+        const u32x4 o = *reinterpret_cast<const u32x4*>(&S.out[3][row][4 * pc]);
+        if (on && !lower && tg < T) *reinterpret_cast<u32x4*>(pS2 + static_cast<uint32_t>(tg) * C) = o;
+    };
+    auto store_out = [&](const int c, const bool on) __attribute__((always_inline)) {
+        const int row = 8 * wq + rq, tg = c * L + row;
+        const u32x4 o1 = *reinterpret_cast<const u32x4*>(&S.out[lower ? 0 : 1][row][4 * pc]);
+        const u32x4 o2 = *reinterpret_cast<const u32x4*>(&S.out[2][row][4 * pc]);
+        if (on && tg < T) {
+            *reinterpret_cast<u32x4*>(pS1 + static_cast<uint32_t>(tg) * C) = o1;
+            if (lower) *reinterpret_cast<u32x4*>(pS2 + static_cast<uint32_t>(tg) * C) = o2;
         }
     };
 
@@ -272,18 +284,28 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             constexpr int z = decltype(Z)::value;
             const int it = it0 + z;
             const int cp = n - 1 - it;
-            asm volatile("" : "+v"(jq), "+v"(tp), "+v"(hl), "+v"(rw));
+            asm volatile("" : "+v"(jq), "+v"(tp), "+v"(rq), "+v"(pc), "+v"(rg));
+            const bool fin = it >= 3 && cp + 3 >= 0;               // chunk cp + 3 is finished and stored in this iteration
+            store_gv(fin ? cp + 3 : 0, fin);
+            meet_signal(&S.met[2], lane);
             if ((cut && it == 0) || cp < 0) stage_in(cp, ring[z], part); else stage_in(cp, ring[z], full);
+            meet_signal(&S.met[0], lane);
             __builtin_amdgcn_sched_barrier(0);
             fetch(cp >= 2 ? cp - 2 : 0, ring[z]);
             __builtin_amdgcn_sched_barrier(0);
-            if (it >= 3 && cp + 3 >= 0) { if (cut && it == 3) finish(cp + 3, hq[2], part); else finish(cp + 3, hq[2], full); }
+            if (fin) { if (cut && it == 3) finish(cp + 3, hq[2], part); else finish(cp + 3, hq[2], full); }
+            meet_signal(&S.met[1], lane);
             __builtin_amdgcn_sched_barrier(0);
             hq[2] = hq[1]; hq[1] = hq[0];
+            met_ok = meet_wait(&S.met[0], 8u * (it + 1)) && met_ok;        // all rows of chunk cp are staged
             if ((cut && it == 0) || cp < 0) prep(cp, hq[0], part); else prep(cp, hq[0], full);
+            __builtin_amdgcn_sched_barrier(0);
+            met_ok = meet_wait(&S.met[1], 8u * (it + 1)) && met_ok;        // all columns of chunk cp + 3 are finished
+            store_out(fin ? cp + 3 : 0, fin);
             __syncthreads();
         });
-    if (lane == 0) a.flags[bh * 8 + w] = any_exact ? 1 : 0;
+    // (a meeting that never completed, which the counting excludes, would leave this head to the two-sweep kernels)
+    if (lane == 0) a.flags[bh * 8 + w] = (any_exact || !met_ok) ? 1 : 0;
     // gu of this batch row: sum over the tokens (lanes of a row)
 #pragma unroll
     for (int z = 0; z < 2; ++z) gu_acc[z] = row_sum_to_last(gu_acc[z]);
@@ -302,7 +324,7 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
     uint32_t b_sv = 4 * g * N + j;                                              // [value channel 4 g][key channel j] of a saved state
     lds_t b_acc = l16 * ROW_B + 8 * g;                                          // [token l16][channel 4 g] of a plane
     lds_t b_tr = ((8 * g + (l16 >> 2)) * PS + 2 * (l16 & 3)) * 4;               // transposing read of a plane, rows 8 g ..
-    lds_t b_trt = ((8 * g + (l16 >> 2)) * AS + 2 * (l16 & 3)) * 4;              // the same of a tile
+    lds_t b_trt = ((8 * g + (l16 >> 2)) * TQ + 2 * (l16 & 3)) * 4;              // the same of a tile
     lds_t b_natt = l16 * TROW_B + 16 * g;                                       // [row l16][position 8 g] of a tile
     lds_t b_xz = l16 * XROW_B + 16 * g;                                         // [token l16][channel 4 g] of X / Z
     lds_t b_j = 4 * l16;
@@ -456,11 +478,10 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
     lds_t b_acc = l16 * ROW_B + 8 * g;                                          // [token l16][channel 4 g] of a plane
     lds_t b_nat = l16 * ROW_B + 16 * g;                                         // [token l16][channel 8 g] of a plane
     lds_t b_tr = ((8 * g + (l16 >> 2)) * PS + 2 * (l16 & 3)) * 4;               // transposing read of a plane, rows 8 g ..
-    lds_t b_trt = ((8 * g + (l16 >> 2)) * AS + 2 * (l16 & 3)) * 4;              // the same of a tile
+    lds_t b_trt = ((8 * g + (l16 >> 2)) * TQ + 2 * (l16 & 3)) * 4;              // the same of a tile
     lds_t b_tw = l16 * TROW_B + 8 * g;                                          // [row l16][position 4 g] of a tile
     lds_t b_g = 16 * g;                                                          // channel 4 g of a per-channel array
     lds_t b_l = 4 * l16;
-    uint16_t* __restrict__ gvp = a.gv + base + 16 * w + 4 * g;
     f32x4 E[4] = {zero4, zero4, zero4, zero4};     // dS[i = 16w + l16][j = 16 tile + 4g + v]
 
     // causal tiles of chunk c (waves 0, 1, 2 -> quadrants (t, s) = (0,0) (1,0) (1,1)); accumulator rows are s, lanes t
@@ -495,7 +516,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int sl = 4 * g + v;
-                if (sl == l16) lds_st<float>(sb + VG0 + (c & 3) * (4 * L) + ta * 64 + b_l, bm[v]);
+                if (sl == l16) lds_st<float>(sb + VG0 + (c % 3) * (4 * L) + ta * 64 + b_l, bm[v]);
                 am[v] = (sl < l16) ? am[v] : (sl == l16 ? d : 0.f);
                 bm[v] = (sl < l16) ? bm[v] : 0.f;
             }
@@ -573,12 +594,12 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                 U[tl] = mfma(rl[tl], gyo, U[tl]);
             }
             __builtin_amdgcn_sched_barrier(0);
+            // gv: lane = token, four consecutive value channels in registers; the prep waves store it in the next iteration,
+            // and have taken the last one out of `out` by now (they did that first thing in this iteration)
+            meet_wait(&S.met[2], 8u * (it + 1));
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
-                const int tg = c * L + 16 * tt + l16;
-                if (tg < T)
-                    *reinterpret_cast<uint2*>(gvp + static_cast<uint32_t>(tg) * C) = make_uint2(pack_bf2(G[tt][0], G[tt][1]), pack_bf2(G[tt][2], G[tt][3]));
-            }
+            for (int tt = 0; tt < 2; ++tt)
+                lds_st<u32x2>(sb + OUT0 + 3 * PLANE_B + tt * 16 * ROW_B + 32 * w + b_acc, u32x2{pack_bf2(G[tt][0], G[tt][1]), pack_bf2(G[tt][2], G[tt][3])});
             // ------------------------------------------------------------ dS^T <- dS^T dec + d1 R'^T GY
 #pragma unroll
             for (int tl = 0; tl < 4; ++tl) {
@@ -603,6 +624,7 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG a) {
     const int n = (a.T + L - 1) / L;
     // the quadrant t < 16 <= s of the tiles is never written and must read as zero
     for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTG) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
+    if (tid < 3) S.met[tid] = 0;
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
     const int nit = (n + 4) & ~1;          // iterations of the pipeline: n + 3, made even

@@ -58,5 +58,25 @@ DEVINL void split16(const f32x4 (&x)[4], const float s, bf16x8 (&h)[2], bf16x8 (
     }
 }
 
+// A meeting point for some of the waves of a workgroup (the hardware barrier takes all of them): each wave adds one to a
+// counter in LDS when its part of a staging area is written, and reads the area only when the counter says that all have.
+// LDS serves the requests of a wave in the order of issue, so whoever sees the count sees the data written before it.
+// The counter only grows: the k-th meeting of m waves is complete at k m.  The poll is bounded, so that a mistake in the
+// counting ends as a wrong result flagged to the caller and not as a hung GPU.
+DEVINL void meet_signal(uint32_t* cnt, const int lane) {
+    asm volatile("" ::: "memory");
+    if (lane == 0) __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+DEVINL bool meet_wait(uint32_t* cnt, const uint32_t target) {
+    bool ok = true;
+    int polls = 0;
+    while (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
+        if (++polls > (1 << 16)) { ok = false; break; }
+        __builtin_amdgcn_s_sleep(1);
+    }
+    asm volatile("" ::: "memory");
+    return ok;
+}
+
 }  // namespace
 }  // namespace rwkv

@@ -15,8 +15,8 @@
 // Pipeline: in iteration `it` the P waves prepare chunk it, the T waves make the tile of chunk it-1, the S waves do the
 // products of chunk it-2 and the P waves store the y of chunk it-3.
 //
-// Global memory is touched 16 bytes per lane: a prep lane moves one row piece (its wave's 8 channels of one token) and
-// the pieces change lane order in LDS; y leaves through an LDS tile so that whole 128-byte rows are written.
+// Global memory is touched in whole 128-byte rows, 16 bytes per lane: the inputs are staged in LDS by whichever prep wave
+// loaded them, and y leaves through an LDS tile.
 //
 // A chunk in which some channel decays by more than e^-60 over either half cannot use the mid-point factors.  Such a
 // (batch, head) is flagged in `flags` and the caller reruns it with wkv6_fwd_ws, which has a step-by-step path.
@@ -43,6 +43,7 @@ struct alignas(16) SmemQ {
     TilesQ tile[2];
     uint32_t yb[2][L][PS];                  // y of the last two chunks, bf16 [token][channel]
     float sst[N][SS];                       // the state entering an even chunk, on its way to global memory
+    uint32_t met;                           // meeting counter of the prep waves
 };
 constexpr lds_t ROW_B = PS * 4, PLANE_B = L * ROW_B, TROW_B = AS * 4;
 constexpr lds_t O_RPH = 0, O_RPL = PLANE_B, O_KPH = 2 * PLANE_B, O_KPL = 3 * PLANE_B, O_V = 4 * PLANE_B;
@@ -62,13 +63,17 @@ struct ArgsQ {
 // ---------------------------------------------------------------------------------------------------- P waves
 DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n, const int nit) {
     int jq = lane >> 4, tp = lane & 15;                 // arithmetic: channel pair, token (and token + 16)
-    int hl = lane >> 5, rw = lane & 31;                 // memory: which tensor, which row of the chunk
-    int rw8 = lane;                                     // y: row 8 (w & 3) + lane / 8, piece lane % 8
+    // Global memory is touched in whole 128-byte rows: eight lanes per row, eight rows per wave and instruction (waves
+    // 0..3: r and w, waves 4..7: k and v, rows 8 (w & 3) ..), because the memory system takes requests for pieces of
+    // a line, one from each of eight waves, at a much lower rate.  A wave thus stages columns that other waves prepare:
+    // the prep waves meet (meet_signal / meet_wait) between the two.
+    int rq = lane >> 3, pc = lane & 7;                  // memory: row 8 (w & 3) + rq of the chunk, piece pc of the row
     const int ch0 = 8 * w + 2 * (lane >> 4);
-    const int hl0 = lane >> 5;
     const int T = a.T, C = a.C;
-    const uint16_t* __restrict__ pA = (hl0 ? a.k : a.r) + base + 8 * w;      // r | k
-    const uint16_t* __restrict__ pB = (hl0 ? a.v : a.w) + base + 8 * w;      // w | v
+    const int wq = w & 3;
+    const bool lower = w < 4;
+    const uint16_t* __restrict__ pA = (lower ? a.r : a.k) + base + 8 * (lane & 7);      // r | k
+    const uint16_t* __restrict__ pB = (lower ? a.w : a.v) + base + 8 * (lane & 7);      // w | v
     float uj[2];
     {
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + ch0);
@@ -79,22 +84,24 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
     // two to three microseconds under load, and a chunk is to take little more than one.
     Raw ring[DEPTH];                       // DEPTH chunks ahead
     auto fetch = [&](const int c, Raw& x) __attribute__((always_inline)) {
-        const int t = c * L + rw;
+        const int t = c * L + 8 * wq + rq;
         const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C;
         x.a = *reinterpret_cast<const u32x4*>(pA + o);
         x.b = *reinterpret_cast<const u32x4*>(pB + o);
     };
-    // the pieces of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v in place
+    // the rows of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v in place
     auto stage_in = [&](const int c, const Raw& x, auto PARTIAL) __attribute__((always_inline)) {
         SlotQ& O = S.slot[c % 3];
-        const bool live = !decltype(PARTIAL)::value || c * L + rw < T;
+        const int row = 8 * wq + rq;
+        const bool live = !decltype(PARTIAL)::value || c * L + row < T;
         const u32x4 zero = {0u, 0u, 0u, 0u};
-        uint32_t* da = &O.RpH[rw][4 * w] + hl * (2 * L * PS);        // R' hi | K' hi
-        uint32_t* db = &O.RpL[rw][4 * w] + hl * (3 * L * PS);        // R' lo | V
+        uint32_t* da = lower ? &O.RpH[row][4 * pc] : &O.KpH[row][4 * pc];
+        uint32_t* db = lower ? &O.RpL[row][4 * pc] : &O.V[row][4 * pc];
         *reinterpret_cast<u32x4*>(da) = live ? x.a : zero;
-        *reinterpret_cast<u32x4*>(db) = (live || !hl) ? x.b : zero;  // w of a dead row is masked where the decay is formed
+        *reinterpret_cast<u32x4*>(db) = (live || lower) ? x.b : zero;    // w of a dead row is masked where the decay is formed
+        meet_signal(&S.met, lane);
     };
-    bool any_exact = false;
+    bool any_exact = false, met_ok = true;
     auto prep = [&](const int c, auto PARTIAL) __attribute__((always_inline)) {
         const int ch = 8 * w + 2 * jq, cd = 4 * w + jq;        // cd: dword column of the pair in a bf16 plane
         SlotQ& O = S.slot[c % 3];
@@ -149,10 +156,10 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
     // (A store on every path, masked per lane, so that the waits for the prefetched inputs count the same on all of them.)
     uint16_t* __restrict__ pY = a.y + base + 8 * (lane & 7);
     auto store_y = [&](const int c, const bool on) __attribute__((always_inline)) {
-        const int row = 8 * (w & 3) + (rw8 >> 3);
-        const u32x4 o = *reinterpret_cast<const u32x4*>(&S.yb[c & 1][row][4 * (rw8 & 7)]);
+        const int row = 8 * wq + rq;
+        const u32x4 o = *reinterpret_cast<const u32x4*>(&S.yb[c & 1][row][4 * pc]);
         const int tg = c * L + row;
-        if (on && w < 4 && tg < T) *reinterpret_cast<u32x4*>(pY + static_cast<uint32_t>(tg) * C) = o;
+        if (on && lower && tg < T) *reinterpret_cast<u32x4*>(pY + static_cast<uint32_t>(tg) * C) = o;
     };
 
     const std::true_type part{};           // only the last chunk can be cut short
@@ -171,17 +178,19 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
         static_for<DEPTH>([&](auto Z) {
             constexpr int z = decltype(Z)::value;
             const int it = it0 + z;
-            asm volatile("" : "+v"(jq), "+v"(tp), "+v"(hl), "+v"(rw), "+v"(rw8));
+            asm volatile("" : "+v"(jq), "+v"(tp), "+v"(rq), "+v"(pc));
             if (it >= n - 1) stage_in(it, ring[z], part); else stage_in(it, ring[z], full);
             __builtin_amdgcn_sched_barrier(0);
             fetch(it + DEPTH < n ? it + DEPTH : n - 1, ring[z]);
             __builtin_amdgcn_sched_barrier(0);
             store_y(it >= 3 ? it - 3 : 0, it >= 3);
             __builtin_amdgcn_sched_barrier(0);
+            met_ok = meet_wait(&S.met, 8u * (it + 1)) && met_ok;      // all eight waves have staged their rows of chunk it
             if (it >= n - 1) prep(it, part); else prep(it, full);
             __syncthreads();
         });
-    if (lane == 0) a.flags[bh * 8 + w] = any_exact ? 1 : 0;
+    // (a meeting that never completed, which the counting excludes, would leave the results of this head to the other kernel)
+    if (lane == 0) a.flags[bh * 8 + w] = (any_exact || !met_ok) ? 1 : 0;
 }
 
 // ---------------------------------------------------------------------------------------------------- S waves
@@ -382,6 +391,7 @@ __global__ __launch_bounds__(NTQ) void wkv6_fwd_fused(const ArgsQ a) {
     const int n = (a.T + L - 1) / L;
     // the quadrant t < 16 <= s of the tiles is never written and must read as zero
     for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTQ) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
+    if (tid == 0) S.met = 0;
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
     const int nit = (n + 2 + DEPTH) & ~(DEPTH - 1);        // iterations of the pipeline: n + 3, in whole trips of the prep loop
