@@ -43,6 +43,7 @@ constexpr int NTG = 16 * 64;
 // times the rate of 72 (16-byte reads and the transposing reads do not care).
 constexpr int PS = 36;             // bf16 [token][channel] planes: 144 B
 constexpr int CS = 68;             // fp32 [token][channel] arrays: 272 B
+constexpr int DEPTH = 2;           // chunks that the prep waves load ahead (a power of two; four would cost the prep waves spills)
 constexpr int TQ = 20;             // causal tiles [t][s], 32 bf16 and 16 bytes of padding: 80 B (16-byte reads of 16 rows hit all banks once)
 
 struct alignas(16) SlotG {
@@ -118,7 +119,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         uj[0] = bf_lo(x); uj[1] = bf_hi(x);
     }
     struct Raw { u32x4 a, b, c; };
-    Raw ring[2];                           // two chunks ahead
+    Raw ring[DEPTH];                       // DEPTH chunks ahead
     auto fetch = [&](const int c, Raw& x) __attribute__((always_inline)) {
         const int t = c * L + 8 * wq + rq, tg = c * L + 4 * w + rg;
         const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C, og = static_cast<uint32_t>(tg < T ? tg : T - 1) * C;
@@ -270,17 +271,18 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     const std::true_type part{};
     const std::false_type full{};
     // in the order in which the loop consumes them: its waits are counted from the worst of all the ways into it
+    static_for<DEPTH>([&](auto Z) {
+        constexpr int z = decltype(Z)::value;
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(n - 1 - z >= 0 ? n - 1 - z : 0, ring[z]);
+    });
     __builtin_amdgcn_sched_barrier(0);
-    fetch(n - 1, ring[0]);
-    __builtin_amdgcn_sched_barrier(0);
-    fetch(n >= 2 ? n - 2 : 0, ring[1]);
-    __builtin_amdgcn_sched_barrier(0);
-    // Two iterations per trip, no stage with loads or ring registers skipped: a way round one, or round the second half,
+    // DEPTH iterations per trip, no stage with loads or ring registers skipped: a way round one, or round the second half,
     // would be one more way into the next wait, on which the registers it waits for are the newest loads (the count then
     // covers everything).  Below chunk 0 the stages run on rows that all count as dead, into planes nobody reads any more
     // (c < 0: the slot is that of chunk c + 3, of which only l2 is still needed, by this wave, before it is written).
-    for (int it0 = 0; it0 < nit; it0 += 2)
-        static_for<2>([&](auto Z) {
+    for (int it0 = 0; it0 < nit; it0 += DEPTH)
+        static_for<DEPTH>([&](auto Z) {
             constexpr int z = decltype(Z)::value;
             const int it = it0 + z;
             const int cp = n - 1 - it;
@@ -291,7 +293,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             if ((cut && it == 0) || cp < 0) stage_in(cp, ring[z], part); else stage_in(cp, ring[z], full);
             meet_signal(&S.met[0], lane);
             __builtin_amdgcn_sched_barrier(0);
-            fetch(cp >= 2 ? cp - 2 : 0, ring[z]);
+            fetch(cp >= DEPTH ? cp - DEPTH : 0, ring[z]);
             __builtin_amdgcn_sched_barrier(0);
             if (fin) { if (cut && it == 3) finish(cp + 3, hq[2], part); else finish(cp + 3, hq[2], full); }
             meet_signal(&S.met[1], lane);
@@ -480,7 +482,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
     lds_t b_tr = ((8 * g + (l16 >> 2)) * PS + 2 * (l16 & 3)) * 4;               // transposing read of a plane, rows 8 g ..
     lds_t b_trt = ((8 * g + (l16 >> 2)) * TQ + 2 * (l16 & 3)) * 4;              // the same of a tile
     lds_t b_tw = l16 * TROW_B + 8 * g;                                          // [row l16][position 4 g] of a tile
-    lds_t b_g = 16 * g;                                                          // channel 4 g of a per-channel array
+    lds_t b_g = 16 * g + 4 * (l16 & 3);                                          // channel 4 g + (l16 & 3) of a per-channel array
     lds_t b_l = 4 * l16;
     f32x4 E[4] = {zero4, zero4, zero4, zero4};     // dS[i = 16w + l16][j = 16 tile + 4g + v]
 
@@ -538,9 +540,15 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
             // Operands are fetched in batches, each issued as a whole before anything waits for it (the scheduling barriers
             // keep the batches apart): a wave then waits for LDS three times per chunk instead of once per product.
             // ------------------------------------------------------------ batch 1: d2 and K' (natural rows)
-            f32x4 dq[4];
+            // per-channel factors: a lane holds the one of channel 16 tile + 4 g + (l16 & 3), a 4-byte read that rows of
+            // four lanes share; the products below take lane v of the 16-lane row inside the multiply (row_newbcast)
+            float dq[4], de[4], d1[4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) dq[q] = lds_ld<f32x4>(so + O_D2 + 64 * q + b_g);
+            for (int q = 0; q < 4; ++q) {
+                dq[q] = lds_ld<float>(so + O_D2 + 64 * q + b_g);
+                de[q] = lds_ld<float>(so + O_DEC + 64 * q + b_g);
+                d1[q] = lds_ld<float>(so + O_D1 + 64 * q + b_g);
+            }
             bf16x8 kh[2][2], kl[2][2];
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt)
@@ -554,9 +562,13 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
             bf16x8 dh[2], dl[2];
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
-                const f32x4 p = dq[2 * ks], q = dq[2 * ks + 1];
-                const HL x0 = hilo2(E[2 * ks][0] * p[0], E[2 * ks][1] * p[1]), x1 = hilo2(E[2 * ks][2] * p[2], E[2 * ks][3] * p[3]);
-                const HL x2 = hilo2(E[2 * ks + 1][0] * q[0], E[2 * ks + 1][1] * q[1]), x3 = hilo2(E[2 * ks + 1][2] * q[2], E[2 * ks + 1][3] * q[3]);
+                float p[4], q[4];
+                static_for<4>([&](auto V) {
+                    constexpr int v = decltype(V)::value;
+                    p[v] = E[2 * ks][v]; q[v] = E[2 * ks + 1][v];
+                    mul_bc<v>(p[v], dq[2 * ks]); mul_bc<v>(q[v], dq[2 * ks + 1]);
+                });
+                const HL x0 = hilo2(p[0], p[1]), x1 = hilo2(p[2], p[3]), x2 = hilo2(q[0], q[1]), x3 = hilo2(q[2], q[3]);
                 dh[ks] = as_op(x0.h, x1.h, x2.h, x3.h);
                 dl[ks] = as_op(x0.l, x1.l, x2.l, x3.l);
             }
@@ -602,11 +614,14 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                 lds_st<u32x2>(sb + OUT0 + 3 * PLANE_B + tt * 16 * ROW_B + 32 * w + b_acc, u32x2{pack_bf2(G[tt][0], G[tt][1]), pack_bf2(G[tt][2], G[tt][3])});
             // ------------------------------------------------------------ dS^T <- dS^T dec + d1 R'^T GY
 #pragma unroll
-            for (int tl = 0; tl < 4; ++tl) {
-                const f32x4 de = lds_ld<f32x4>(so + O_DEC + 64 * tl + b_g), d1 = lds_ld<f32x4>(so + O_D1 + 64 * tl + b_g);
-#pragma unroll
-                for (int v = 0; v < 4; ++v) E[tl][v] = fmaf(E[tl][v], de[v], d1[v] * U[tl][v]);
-            }
+            for (int tl = 0; tl < 4; ++tl)
+                static_for<4>([&](auto V) {
+                    constexpr int v = decltype(V)::value;
+                    float x = E[tl][v];
+                    mul_bc<v>(x, de[tl]);
+                    fmac_bc<v>(x, d1[tl], U[tl][v]);
+                    E[tl][v] = x;
+                });
         }
         __builtin_amdgcn_sched_barrier(0);
         if (it >= 1 && c - 1 >= 0 && w < 3) tiles(c - 1);
@@ -627,7 +642,7 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG a) {
     if (tid < 3) S.met[tid] = 0;
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
-    const int nit = (n + 4) & ~1;          // iterations of the pipeline: n + 3, made even
+    const int nit = (n + 2 + DEPTH) & ~(DEPTH - 1);        // iterations of the pipeline: n + 3, in whole trips of the prep loop
     if (wid < 8) role_prep<WMODE>(S, a, lane, wid, base, h, bh, n, nit);
     else if (wid < 12) role_sd<WMODE>(S, a, lane, w, bh, n, nit);
     else role_e<WMODE>(S, a, lane, w, base, n, nit);
