@@ -224,7 +224,19 @@ def wkv6_grads(B, T, C, H, r, k, v, w_raw, u, gy, s0=None, dtype=torch.float64, 
     return out
 
 
-def emulate_wkv5_bf16(B, T, C, H, r, k, v, w_raw, u, gy):
+def wkv_grads_by_hand(B, T, C, H, r, k, v, w_raw, u, gy, s0, dtype):
+    """y, gr, gk, gv, gw_raw [B,T,C], gu [B,H,N] (per batch row) and gs in `dtype`, by wkv_recurrent and
+    wkv_backward_hand instead of autograd: the same quantities at a third of the cost, for the long shapes."""
+    r_, k_, v_, w_, g_ = (x.to(dtype) for x in (r, k, v, w_raw, gy))
+    u_ = u.to(dtype)
+    s_ = None if s0 is None else s0.to(dtype)
+    dec = torch.exp(-torch.exp(w_))
+    y, _ = wkv_recurrent(B, T, C, H, r_, k_, v_, dec, u_, s_)
+    gr, gk, gv, G, gu, gs = wkv_backward_hand(B, T, C, H, r_, k_, v_, dec, u_, g_, s_)
+    return y, gr, gk, gv, -torch.exp(w_) * G, gu, gs
+
+
+def emulate_wkv5_bf16(B, T, C, H, r, k, v, w_raw, u, gy, hand=False):
     """Error bar for the bf16 wkv5 path: fp32 math on the bf16 inputs with the reference's
     rounding points -- y, gr, gk, gv stored as bf16 (wkv5_cuda_v1b.cu:59,105,174-175); gw, gu
     stored per batch as bf16 (:107,136) and summed over B by torch.sum on bf16
@@ -232,20 +244,27 @@ def emulate_wkv5_bf16(B, T, C, H, r, k, v, w_raw, u, gy):
     fp32 summation order and __expf are not modelled: their effect (~1e-7 relative) is far
     below the bf16 rounding that sets the bar."""
     f = torch.float32
-    y, gr, gk, gv, gw, gu = wkv5_grads(B, T, C, H, r, k, v, w_raw, u, gy, dtype=f, per_batch=True)
     rb = lambda x: x.to(torch.bfloat16)
+    if hand:
+        y, gr, gk, gv, gw, gu = wkv_grads_by_hand(B, T, C, H, r, k, v, w_raw.reshape(1, 1, C).expand(B, T, C), u, gy, None, f)[:6]
+        gw = gw.sum(1).reshape(B, H, C // H)                    # the decay of a head acts at every step
+    else:
+        y, gr, gk, gv, gw, gu = wkv5_grads(B, T, C, H, r, k, v, w_raw, u, gy, dtype=f, per_batch=True)
     gw = rb(gw).sum(0).reshape(H, C // H)
     gu = rb(gu).sum(0).reshape(H, C // H)
     return rb(y), rb(gr), rb(gk), rb(gv), gw, gu
 
 
-def emulate_wkv6_bf16(B, T, C, H, r, k, v, w_raw, u, gy, s0=None):
+def emulate_wkv6_bf16(B, T, C, H, r, k, v, w_raw, u, gy, s0=None, hand=False):
     """Error bar for the bf16 wkv6 / wkv6_state paths: fp32 math on bf16 inputs, outputs
     rounded where the reference kernels round -- y (wkv6state_cuda_v1a.cu:63), gr/gk/gv/gw
     (:119,143,166,251), per-batch gu as bf16 (:121) then torch.sum over B on bf16
     (wkv6_state/run.py:123), gs as bf16 (:187)."""
     f = torch.float32
-    out = wkv6_grads(B, T, C, H, r, k, v, w_raw, u, gy, s0=s0, dtype=f, per_batch=True)
+    if hand:
+        out = wkv_grads_by_hand(B, T, C, H, r, k, v, w_raw, u, gy, s0, f)
+    else:
+        out = wkv6_grads(B, T, C, H, r, k, v, w_raw, u, gy, s0=s0, dtype=f, per_batch=True)
     rb = lambda x: x.to(torch.bfloat16)
     y, gr, gk, gv, gw, gu = out[:6]
     res = [rb(y), rb(gr), rb(gk), rb(gv), rb(gw), rb(gu).sum(0).reshape(H, C // H)]

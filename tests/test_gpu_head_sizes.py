@@ -154,22 +154,21 @@ def test_wkv5_bf16_reference_default_shape_sampled_heads(lib):
     y.backward(gy.to(DEV))
     torch.cuda.synchronize()
     got_all = [y.detach()] + [x.grad for x in t]
-    for h in (3, 29):
-        print(f" head {h}", flush=True)
-        sl = slice(h * N, (h + 1) * N)
-        rr, kk, vv, gg = (x[:, :, sl].contiguous().double() for x in (r, k, v, gy))
-        uu, wr = u[h:h + 1].double(), w[h:h + 1].double()
-        dec = O.wkv6_decay(wr).reshape(1, 1, N).expand(B, T, N).contiguous()
-        yref, _ = O.wkv_recurrent(B, T, N, 1, rr, kk, vv, dec, uu)
-        gr, gk, gv, G, gu, _ = O.wkv_backward_hand(B, T, N, 1, rr, kk, vv, dec, uu, gg)
-        gw = (-torch.exp(wr) * G.sum((0, 1)).reshape(1, N))
-        ref = [yref, gr, gk, gv, gw, gu.sum(0)]
-        got = [got_all[0][:, :, sl], got_all[1][:, :, sl], got_all[2][:, :, sl], got_all[3][:, :, sl],
-               got_all[4][h:h + 1], got_all[5][h:h + 1]]
-        for name, a, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, got):
-            e = err_ratio(a, g.double().cpu())
-            print(f"  {name}: {e:.3e}", flush=True)
-            assert e < (4e-3 if name in ("gu", "gw") else 2.5e-3), (name, e)
+    # one head as a small problem: the fp64 oracle and the emulation of the reference kernel (fp32 math, its rounding
+    # points), both by the hand-derived backward
+    hs = [29]
+    n = N * len(hs)
+    ch = torch.cat([torch.arange(h * N, (h + 1) * N) for h in hs])
+    rr, kk, vv, gg = (x[:, :, ch].contiguous() for x in (r, k, v, gy))
+    uu, wr = u[hs].contiguous(), w[hs].contiguous()
+    ref = list(O.wkv_grads_by_hand(B, T, n, len(hs), rr, kk, vv, wr.reshape(1, 1, n).expand(B, T, n), uu, gg, None, torch.float64))[:6]
+    ref[4] = ref[4].sum((0, 1)).reshape(len(hs), N)
+    ref[5] = ref[5].sum(0)
+    emu = O.emulate_wkv5_bf16(B, T, n, len(hs), rr, kk, vv, wr, uu, gg, hand=True)
+    chd = ch.to(DEV)
+    got = [got_all[0][:, :, chd], got_all[1][:, :, chd], got_all[2][:, :, chd], got_all[3][:, :, chd], got_all[4][hs], got_all[5][hs]]
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, got):
+        assert_no_worse("wkv5 N=128 full size " + name, a, e, g)
 
 
 def _wkv5_c_abi(lib, B, T, C, H, r, k, v, w, u, gy, flags, with_forward_workspace):

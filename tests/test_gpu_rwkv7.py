@@ -71,11 +71,10 @@ def test_rwkv7_full_size_chain_equals_one_call(lib):
     h = 5
     sub = [args[0][:, h:h + 1]] + [x[:, :, h:h + 1] for x in args[1:8]] + [args[8][:, h:h + 1]]
     ref = O.backward_hand(*sub)
+    emu = O.emulate_bf16(*sub)
     got = [one[0][:, :, h:h + 1], one[1][:, h:h + 1], one[2][:, h:h + 1]] + [x[:, :, h:h + 1] for x in one[3:]]
-    for name, a, g in zip(NAMES, ref, got):
-        e = err_ratio(a, g.double().cpu())
-        print(f"  head {h} {name}: {e:.3e}", flush=True)
-        assert e < 3e-3, (name, e)
+    for name, a, e, g in zip(NAMES, ref, emu, got):
+        assert_no_worse(f"rwkv7 full size head {h} " + name, a, e, g)
 
 
 @pytest.mark.parametrize("B,T,H", [(2, 32, 2), (1, 48, 1)])
@@ -113,14 +112,15 @@ def test_rwkv7_state_only_and_stateless_ops(lib, B, T, H):
 
 
 def test_rwkv7_long_sequence_is_no_worse_than_the_reference_kernel(lib):
-    """T = 2048 on one head: the in-chunk inversion of the backward and the fp32 state must not lose accuracy with length."""
-    B, T, H = 1, 2048, 1
+    """T = 4096 on one head (the length of one call at the benchmark shape): the in-chunk inversion of the backward and the
+    fp32 state must not lose accuracy with length."""
+    B, T, H = 1, 4096, 1
     args = synth.rwkv7_inputs(B, T, H, 64, seed=34)
     ref = O.grads(*args)
     emu = O.emulate_bf16(*args)
     got = _run(args)
     for name, a, e, g in zip(NAMES, ref, emu, got):
-        assert_no_worse("rwkv7 T2048 " + name, a, e, g)
+        assert_no_worse("rwkv7 T4096 " + name, a, e, g)
 
 
 def _fp32_inputs(B, T, H, seed):

@@ -97,24 +97,20 @@ def test_wkv6_full_size_sampled_heads(lib):
     y.backward(gy.to(DEV))
     torch.cuda.synchronize()
     got_all = [y.detach()] + [x.grad for x in t]
-    for h in (0, 17, 31):
-        print(f" head {h}", flush=True)
-        sl = slice(h * 64, (h + 1) * 64)
-        rr, kk, vv, ww, gg = (x[:, :, sl].contiguous().double() for x in (r, k, v, w, gy))
-        uu = u[h:h + 1].double()
-        ss = s0[:, h:h + 1].double()
-        dec = O.wkv6_decay(ww)
-        yref, _ = O.wkv_recurrent(B, T, 64, 1, rr, kk, vv, dec, uu, ss)
-        gr, gk, gv, G, gu, gs = O.wkv_backward_hand(B, T, 64, 1, rr, kk, vv, dec, uu, gg, ss)
-        gw = -torch.exp(ww) * G
-        ref = [yref, gr, gk, gv, gw, gu.sum(0), gs]
-        got = [got_all[0][:, :, sl], got_all[1][:, :, sl], got_all[2][:, :, sl], got_all[3][:, :, sl],
-               got_all[4][:, :, sl], got_all[5][h:h + 1], got_all[6][:, h:h + 1]]
-        for name, a, g in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, got):
-            e = err_ratio(a, g.double().cpu())
-            print(f"  {name}: {e:.3e}", flush=True)
-            # pure bf16 output rounding is 1.7e-3; gu is a bf16 sum of 8 bf16 partials
-            assert e < (4e-3 if name == "gu" else 2.5e-3), (name, e)
+    # the sampled heads as one small problem of two heads: the fp64 oracle and the emulation of the reference kernel
+    # (fp32 math, its rounding points), both by the hand-derived backward, which costs a third of autograd at this length
+    hs = [0, 31]
+    ch = torch.cat([torch.arange(h * 64, (h + 1) * 64) for h in hs])
+    rr, kk, vv, ww, gg = (x[:, :, ch].contiguous() for x in (r, k, v, w, gy))
+    uu, ss = u[hs].contiguous(), s0[:, hs].contiguous()
+    ref = list(O.wkv_grads_by_hand(B, T, 64 * len(hs), len(hs), rr, kk, vv, ww, uu, gg, ss, torch.float64))
+    ref[5] = ref[5].sum(0)
+    emu = O.emulate_wkv6_bf16(B, T, 64 * len(hs), len(hs), rr, kk, vv, ww, uu, gg, s0=ss, hand=True)
+    chd = ch.to(DEV)
+    got = [got_all[0][:, :, chd], got_all[1][:, :, chd], got_all[2][:, :, chd], got_all[3][:, :, chd],
+           got_all[4][:, :, chd], got_all[5][hs], got_all[6][:, hs]]
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu", "gs"], ref, emu, got):
+        assert_no_worse("wkv6_state full size " + name, a, e, g)
 
 
 @pytest.mark.parametrize("entry", ["raw", "ew"])
@@ -138,23 +134,18 @@ def test_wkv6_stateless_full_size_sampled_heads(lib, entry):
     call(name_b, d[0].device, B, T, C, H, d[0], d[1], d[2], wd, d[4], d[5], gr, gk, gv, gw, gu, ws, n)
     torch.cuda.synchronize()
     assert float(gw[:, 0].float().abs().max()) == 0.0 and float(gw[:, T - 1].float().abs().max()) == 0.0
-    gu_sum = gu.float().sum(0).view(H, 64)
-    for h in (3, 28):
-        print(f" head {h}", flush=True)
-        sl = slice(h * 64, (h + 1) * 64)
-        rr, kk, vv, ww, gg = (x[:, :, sl].contiguous().double() for x in (r, k, v, w, gy))
-        uu = u[h:h + 1].double()
-        dec = O.wkv6_decay(ww)
-        yref, _ = O.wkv_recurrent(B, T, 64, 1, rr, kk, vv, dec, uu)
-        rgr, rgk, rgv, G, rgu, _ = O.wkv_backward_hand(B, T, 64, 1, rr, kk, vv, dec, uu, gg)
-        rgw = -torch.exp(ww) * G
-        ref = [yref, rgr, rgk, rgv, rgw, rgu.sum(0)]
-        got = [y[:, :, sl], gr[:, :, sl], gk[:, :, sl], gv[:, :, sl], gw[:, :, sl], gu_sum[h:h + 1]]
-        for name, a, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, got):
-            e = err_ratio(a, g.double().cpu())
-            print(f"  {name}: {e:.3e}", flush=True)
-            # pure bf16 output rounding is 1.7e-3; gu sums 8 bf16 per-batch partials
-            assert e < (4e-3 if name == "gu" else 2.5e-3), (name, e)
+    gu_sum = gu.sum(0).view(H, 64)                              # what the wrapper does: a bf16 sum of the per-batch rows
+    hs = [3, 28]
+    ch = torch.cat([torch.arange(h * 64, (h + 1) * 64) for h in hs])
+    rr, kk, vv, ww, gg = (x[:, :, ch].contiguous() for x in (r, k, v, w, gy))
+    uu = u[hs].contiguous()
+    ref = list(O.wkv_grads_by_hand(B, T, 64 * len(hs), len(hs), rr, kk, vv, ww, uu, gg, None, torch.float64))[:6]
+    ref[5] = ref[5].sum(0)
+    emu = O.emulate_wkv6_bf16(B, T, 64 * len(hs), len(hs), rr, kk, vv, ww, uu, gg, hand=True)
+    chd = ch.to(DEV)
+    got = [y[:, :, chd], gr[:, :, chd], gk[:, :, chd], gv[:, :, chd], gw[:, :, chd], gu_sum[hs]]
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, got):
+        assert_no_worse(f"wkv6 {entry} full size " + name, a, e, g)
 
 
 def test_wkv5_full_size_sampled_heads(lib):
@@ -168,23 +159,19 @@ def test_wkv5_full_size_sampled_heads(lib):
     y.backward(gy.to(DEV))
     torch.cuda.synchronize()
     got_all = [y.detach()] + [x.grad for x in t]
-    for h in (5, 30):
-        print(f" head {h}", flush=True)
-        sl = slice(h * 64, (h + 1) * 64)
-        rr, kk, vv, gg = (x[:, :, sl].contiguous().double() for x in (r, k, v, gy))
-        uu, wr = u[h:h + 1].double(), w[h:h + 1].double()
-        dec = O.wkv6_decay(wr).reshape(1, 1, 64).expand(B, T, 64).contiguous()    # exp(-exp(w_raw)) at every step
-        yref, _ = O.wkv_recurrent(B, T, 64, 1, rr, kk, vv, dec, uu)
-        gr, gk, gv, G, gu, _ = O.wkv_backward_hand(B, T, 64, 1, rr, kk, vv, dec, uu, gg)
-        gw = (-torch.exp(wr) * G.sum((0, 1)).reshape(1, 64))     # d/d w_raw, summed over batch and time
-        ref = [yref, gr, gk, gv, gw, gu.sum(0)]
-        got = [got_all[0][:, :, sl], got_all[1][:, :, sl], got_all[2][:, :, sl], got_all[3][:, :, sl],
-               got_all[4][h:h + 1], got_all[5][h:h + 1]]
-        for name, a, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, got):
-            e = err_ratio(a, g.double().cpu())
-            print(f"  {name}: {e:.3e}", flush=True)
-            # pure bf16 output rounding is 1.7e-3; gw and gu are bf16 sums of 8 bf16 per-batch partials
-            assert e < (4e-3 if name in ("gu", "gw") else 2.5e-3), (name, e)
+    hs = [5, 30]
+    ch = torch.cat([torch.arange(h * 64, (h + 1) * 64) for h in hs])
+    rr, kk, vv, gg = (x[:, :, ch].contiguous() for x in (r, k, v, gy))
+    uu, wr = u[hs].contiguous(), w[hs].contiguous()
+    n = 64 * len(hs)
+    ref = list(O.wkv_grads_by_hand(B, T, n, len(hs), rr, kk, vv, wr.reshape(1, 1, n).expand(B, T, n), uu, gg, None, torch.float64))[:6]
+    ref[4] = ref[4].sum((0, 1)).reshape(len(hs), 64)
+    ref[5] = ref[5].sum(0)
+    emu = O.emulate_wkv5_bf16(B, T, n, len(hs), rr, kk, vv, wr, uu, gg, hand=True)
+    chd = ch.to(DEV)
+    got = [got_all[0][:, :, chd], got_all[1][:, :, chd], got_all[2][:, :, chd], got_all[3][:, :, chd], got_all[4][hs], got_all[5][hs]]
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, got):
+        assert_no_worse("wkv5 full size " + name, a, e, g)
 
 
 def test_long_sequence_is_no_worse_than_the_reference_kernel(lib):

@@ -171,3 +171,26 @@ def test_error_bar_emulator_equals_the_reference_kernels_order_of_operations(see
         print(f"  {name}: proxy {ep:.4e}  kernel order {eq:.4e}  identical bf16 values {100 * same:.1f} %")
         assert abs(ep - eq) <= 0.02 * max(ep, eq), (name, ep, eq)
         assert same > 0.97, (name, same)
+
+
+def test_hand_derived_emulation_equals_the_autograd_one():
+    """The emulation of the reference kernels (the bar of the bf16 GPU tests) has a cheaper form for the long shapes, by
+    wkv_backward_hand instead of autograd: the same fp32 quantities up to the order of additions, so the same bf16 values
+    except where a rounding tie flips, and the same error against fp64 to four digits."""
+    from rwkv_cuda_amd import synth
+    from oracle import err_ratio
+    for B, T, H, state in [(2, 70, 2, True), (3, 33, 1, False)]:
+        C = 64 * H
+        r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=5, state=state)
+        ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+        a = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+        b = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0, hand=True)
+        for x, y, z in zip(ref, a, b):
+            assert abs(err_ratio(x, y.double()) - err_ratio(x, z.double())) < 2e-6
+            assert float((y.float() - z.float()).abs().max()) <= 2.0 ** -7 * float(y.float().abs().max())
+        r, k, v, w5, u, gy = synth.wkv5_inputs(B, T, C, H, seed=6)
+        ref = O.wkv5_grads(B, T, C, H, r, k, v, w5, u, gy)
+        a = O.emulate_wkv5_bf16(B, T, C, H, r, k, v, w5, u, gy)
+        b = O.emulate_wkv5_bf16(B, T, C, H, r, k, v, w5, u, gy, hand=True)
+        for x, y, z in zip(ref, a, b):
+            assert abs(err_ratio(x, y.double()) - err_ratio(x, z.double())) < 2e-6
