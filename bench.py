@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Headline benchmark: WKV6 bf16 forward+backward at B=8, T=4096, C=2048 (H=32, N=64) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wkv6|wkv6_state|wkv5|wkv5_n128|rwkv7|wkv4|wkv4_b32|timex|...]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload wkv6|wkv6_state|wkv6_b1|wkv5|wkv5_n128|rwkv7|wkv4|wkv4_b32|timex|...]
 
 A "step" is one forward + one backward of the operator over one batch of synthetic inputs that are
 already resident in HBM, through the same C-ABI calls and the same wrapper-side torch work
@@ -89,11 +89,11 @@ def time_gpu(fn, iters, warmup):
 # kernels: list of (label, fn, algorithmic_bytes) -- every kernel the step launches from the library
 # --------------------------------------------------------------------------------------------
 
-def make_wkv6(dev, state):
+def make_wkv6(dev, state, B=8):
     from rwkv_cuda_amd import _lib, synth
     from rwkv_cuda_amd._call import call
     lib = _lib.load()
-    B, T, H, N = 8, 4096, 32, 64
+    T, H, N = 4096, 32, 64
     C = H * N
     bf = torch.bfloat16
     r, k, v, w, u, gy, s0 = (x.to(dev) if x is not None else None for x in synth.wkv6_inputs(B, T, C, H, seed=42, state=state))
@@ -148,6 +148,22 @@ def make_wkv6(dev, state):
 
     cfg = {"workload": f"{name} bf16 fwd+bwd B{B} T{T} C{C} H{H} N{N}", "B": B, "T": T, "C": C, "H": H, "N": N,
            "algorithmic_bytes_per_token": 28 * C}
+    if B * H < 256 and ALGO == "chunked":
+        # fewer sequences than CUs: the library cuts them into blocks joined by a scan; the same step with one workgroup
+        # per sequence (RWKV_FLAG_WHOLE, 0x200) for comparison
+        def whole():
+            call("rwkv_wkv6f_forward", dev, B, T, C, H, r, k, v, w, u, s0, y, saved, nsaved, FLAGS | 0x200)
+            call("rwkv_wkv6f_backward_saved", dev, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu_sum, gs, saved, nsaved, ws, nbytes, FLAGS | 0x200)
+        for _ in range(5):
+            whole()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(50):
+            whole()
+        e1.record()
+        torch.cuda.synchronize()
+        cfg["ms_per_step_one_workgroup_per_sequence"] = round(e0.elapsed_time(e1) / 50, 4)
     return step, tok, kernels, cfg, cpu_baseline, 28 * C * tok
 
 
@@ -441,6 +457,7 @@ def make_timex(dev):
 WORKLOADS = {
     "wkv6": lambda dev: make_wkv6(dev, False),
     "wkv6_state": lambda dev: make_wkv6(dev, True),
+    "wkv6_b1": lambda dev: make_wkv6(dev, False, B=1),
     "wkv5": make_wkv5,
     "wkv5_n128": lambda dev: make_wkv5(dev, H=32, N=128),
     "wkv5_fp32": make_wkv5_fp32,
@@ -451,7 +468,7 @@ WORKLOADS = {
     "wkv4_b32": lambda dev: make_wkv4(dev, B=32, T=768),
     "timex": make_timex,
 }
-DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv5": "bf16", "wkv5_n128": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "wkv4_b32": "f32", "timex": "bf16x3 (every fp32 operand as three bf16 terms, fp32 accumulation)"}
+DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv6_b1": "bf16", "wkv5": "bf16", "wkv5_n128": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "wkv4_b32": "f32", "timex": "bf16x3 (every fp32 operand as three bf16 terms, fp32 accumulation)"}
 
 
 def main():
@@ -538,7 +555,7 @@ def main():
         if flops:                                # a kernel bound by the matrix cores, not by HBM
             per_kernel[-1].update(algorithmic_flops=flops[0], TFLOPs=round(flops[0] / (ms * 1e-3) / 1e12, 2))
     dom = max(per_kernel, key=lambda d: d["ms"])
-    traffic = TRAFFIC_MEASURED.get(dom["kernel"]) if ALGO == "chunked" else None
+    traffic = TRAFFIC_MEASURED.get(dom["kernel"]) if ALGO == "chunked" and args.workload != "wkv6_b1" else None   # counted at B = 8
     step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
     roofline = {"bound": "hbm", "kernel": dom["kernel"], "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(dom["GBps"] / HBM_PEAK_GBS, 4), "traffic": traffic,

@@ -70,6 +70,10 @@ int rwkv_hbm_probe(void* stream, int mode, const void* src, void* dst, size_t by
 #define RWKV_PASS_GK 4u
 #define RWKV_PASS_ALL 7u
 #define RWKV_FLAG_SWEEPS 0x100u
+/*   RWKV_FLAG_WHOLE  : rwkv_wkv6f_forward / rwkv_wkv6f_backward_saved keep one workgroup per (batch, head) also where
+ *                      B H is below the number of CUs (by default such shapes run as several blocks per sequence joined
+ *                      by a scan).  Forward and backward of one step must agree on it. */
+#define RWKV_FLAG_WHOLE 0x200u
 
 /* ---------------------------------------------------------------------------------------
  * RWKV-4 wkv, fp32.  Replaces cuda_forward / cuda_backward of wkv/cuda/wkv_op.cpp:3-4

@@ -898,6 +898,14 @@ __global__ __launch_bounds__(256) void bf16_batch_sum(int B, int C, const uint16
 }
 
 size_t round16(size_t x) { return (x + 15) & ~static_cast<size_t>(15); }
+// a fill kernel rather than hipMemsetAsync, which a caller's graph capture replays unreliably
+__global__ void zero_words_kernel(int* p, size_t n) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+void zero_words(hipStream_t st, int* p, size_t n) {
+    hipLaunchKernelGGL(zero_words_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, p, n);
+}
 
 // ---- wkv5 with heads of 128 channels on the matrix-core kernels: every head as four heads of 64, two launches per kernel,
 //      each leaving one fp32 term of every output element (see ArgsB in wkv6_chunk.h); the terms are added here
@@ -1237,10 +1245,33 @@ bool fused_ok(int T, int C, int H, unsigned flags) {
     return C == H * N && !(flags & (RWKV_FLAG_SWEEPS | RWKV_PASS_ALL)) && static_cast<long long>(T) * C < (1LL << 30);
 }
 
+// Fewer (batch, head) pairs than the chip has CUs: the sequences are cut into blocks of whole 64-token segments, as many
+// as it takes to give every CU a workgroup (and at least 128 tokens each, the pipeline needs a few chunks to fill).
+constexpr int NUM_CU = 256;
+int scan_blocks(int B, int T, int H, int* TB, unsigned flags = 0u) {
+    const long long bh = static_cast<long long>(B) * H;
+    const int seg = (T + 63) / 64;
+    long long want = NUM_CU / bh;
+    *TB = T;
+    if (want < 2 || seg < 4 || (flags & RWKV_FLAG_WHOLE)) return 1;
+    if (want > seg / 2) want = seg / 2;
+    const int per = static_cast<int>((seg + want - 1) / want);
+    *TB = per * 64;
+    return (T + *TB - 1) / *TB;
+}
+size_t saved_states_bytes(int B, int T, int H) {
+    const size_t nchunks = (static_cast<size_t>(T) + 31) / 32, nseg = (nchunks + 1) / 2;
+    return static_cast<size_t>(B) * H * nseg * 64 * 64 * sizeof(float);
+}
+size_t scan_scratch_bytes(int B, int T, int H) {           // local results and scanned states (fp32 [64][64]) and log decays per block
+    int TB;
+    const int NB = scan_blocks(B, T, H, &TB);
+    return NB <= 1 ? 0 : static_cast<size_t>(B) * H * NB * (2 * 64 * 64 + 64) * sizeof(float);
+}
+
 size_t rwkv_wkv6f_saved_bytes(int B, int T, int C, int H) {
     if (check_dims(B, T, C, H) != RWKV_OK || C != H * N || static_cast<long long>(T) * C >= (1LL << 30)) return 0;
-    const size_t nchunks = (static_cast<size_t>(T) + 31) / 32, nseg = (nchunks + 1) / 2;
-    return static_cast<size_t>(B) * H * nseg * 64 * 64 * sizeof(float) + round16(static_cast<size_t>(B) * H * 8 * sizeof(int));
+    return saved_states_bytes(B, T, H) + round16(static_cast<size_t>(B) * H * 8 * sizeof(int)) + scan_scratch_bytes(B, T, H);
 }
 
 int rwkv_wkv6f_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
@@ -1259,14 +1290,29 @@ int rwkv_wkv6f_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16
     // factors; those pairs are redone (y and states) by the kernel that has a step-by-step path, all others return at once
     const hipStream_t st = static_cast<hipStream_t>(stream);
     const size_t nflag = round16(static_cast<size_t>(B) * H * 8 * sizeof(int));
-    int* flg = reinterpret_cast<int*>(static_cast<char*>(saved) + (rwkv_wkv6f_saved_bytes(B, T, C, H) - nflag));
-    if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved), flg)) return e;
+    char* sb = static_cast<char*>(saved);
+    int* flg = reinterpret_cast<int*>(sb + saved_states_bytes(B, T, H));
+    int TB;
+    const int NB = scan_blocks(B, T, H, &TB, flags);
+    if (NB > 1) {
+        const size_t nq = static_cast<size_t>(B) * H * NB;
+        float* local = reinterpret_cast<float*>(sb + saved_states_bytes(B, T, H) + nflag);
+        float* s32 = local + nq * 64 * 64;
+        float* logdec = s32 + nq * 64 * 64;
+        zero_words(st, flg, static_cast<size_t>(B) * H * 8);
+        if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved), flg, NB, TB, local, logdec, s32)) return e;
+    } else if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved), flg)) return e;
     return launch_wkv6_fwd_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved), flg);
 }
 
 size_t rwkv_wkv6f_backward_saved_workspace_bytes(int B, int T, int C, int H) {
     const size_t n = rwkv_wkv6f_backward_workspace_bytes(B, T, C, H);
-    return n == 0 ? 0 : round16(n) + round16(static_cast<size_t>(B) * H * 8 * sizeof(int));
+    if (n == 0) return 0;
+    int TB;
+    const int NB = C == H * N ? scan_blocks(B, T, H, &TB) : 1;
+    // several blocks per sequence: the scan's scratch and gu per block and batch row in fp32
+    const size_t scan = NB <= 1 ? 0 : scan_scratch_bytes(B, T, H) + static_cast<size_t>(NB) * B * C * sizeof(float);
+    return round16(n) + round16(static_cast<size_t>(B) * H * 8 * sizeof(int)) + scan;
 }
 
 int rwkv_wkv6f_backward_saved(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
@@ -1288,7 +1334,18 @@ int rwkv_wkv6f_backward_saved(void* stream, int B, int T, int C, int H, const rw
     float* rdr = static_cast<float*>(workspace);
     uint16_t* pu = reinterpret_cast<uint16_t*>(wsb + n);                                  // per-batch gu
     int* flg = reinterpret_cast<int*>(wsb + round16(rwkv_wkv6f_backward_workspace_bytes(B, T, C, H)));
-    if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, pu, gs, static_cast<const float*>(saved), flg)) return e;
+    int TB;
+    const int NB = scan_blocks(B, T, H, &TB, flags);
+    if (NB > 1) {
+        const size_t nq = static_cast<size_t>(B) * H * NB;
+        float* local = reinterpret_cast<float*>(reinterpret_cast<char*>(flg) + round16(static_cast<size_t>(B) * H * 8 * sizeof(int)));
+        float* ds32 = local + nq * 64 * 64;
+        float* logdec = ds32 + nq * 64 * 64;
+        float* gu32 = logdec + nq * 64;
+        zero_words(st, flg, static_cast<size_t>(B) * H * 8);
+        if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, pu, gs, static_cast<const float*>(saved), flg,
+                                          NB, TB, local, logdec, ds32, gu32)) return e;
+    } else if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, pu, gs, static_cast<const float*>(saved), flg)) return e;
     // (batch, head) pairs with a decay the mid-point factors cannot carry: the two sweeps redo them, all others return at once
     if (int e = launch_wkv6_bwd_a_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, gy, gr, pu, rdr, flg)) return e;
     if (int e = launch_wkv6_bwd_b_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, gy, gk, gv, gw, gs, rdr, flg)) return e;

@@ -80,6 +80,16 @@ struct ArgsG {
     uint16_t *gr, *gk, *gv, *gw, *gu, *gs;
     const float* saved;            // [B*H][ceil(n/2)][64][64]: the forward state entering every even chunk
     int* flags;                    // [B*H][8]
+    // Sequences cut into NB blocks of TB tokens (a multiple of 64), one workgroup per (batch, head, block), see
+    // wkv6_fwd_f.hip.  LOCAL = true leaves in blk_ds the gradient state that a block builds from nothing, going down from
+    // its end, and in blk_decay the log2 of its total decay; wkv6_scan (reverse) turns these into the gradient state
+    // that enters every block from above (ds32); LOCAL = false then starts each block from there.
+    int NB, TB;
+    const float* ds32;             // [B*H][NB][64][64], [value][key], or null
+    float* blk_ds;                 // [B*H][NB][64][64]
+    float* blk_decay;              // [B*H][NB][64]
+    float* gu32;                   // NB > 1: gu of this (batch, head, block) in fp32 (the blocks are added before rounding)
+    bool first, above;             // this is block 0; there is a block above this one
 };
 
 // state entering even chunk e of this (batch, head), in the layout of the SD waves: lane <-> key channel 16w + l16,
@@ -93,7 +103,7 @@ DEVINL void load_state(const float* __restrict__ p, const uint32_t lo, f32x4 (&x
 
 // ---------------------------------------------------------------------------------------------------- P waves
 // wave w (0..7): channels 8w..8w+7; lane = 16 * (channel pair) + token: a thread has two channels of tokens tp and tp + 16
-template <int WMODE>
+template <int WMODE, bool LOCAL>
 DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n, const int nit) {
     // jq, tp (and hl, rw below) are redefined behind an empty asm in every iteration, see role_sd
     int jq = lane >> 4, tp = lane & 15;
@@ -144,6 +154,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     struct Held { uint32_t r[2], k[2]; float cc[2][2]; };
     Held hq[3] = {};
     bool any_exact = false, met_ok = true;
+    float logdec[2] = {0.f, 0.f};          // LOCAL: log2 of the decay over the whole block
     float carry[2] = {0.f, 0.f}, gu_acc[2] = {0.f, 0.f};
     // Only the last chunk of the sequence can be cut short (PARTIAL): its rows past T carry no input and no decay.
 
@@ -172,6 +183,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             hd.cc[1][z] = p1 - lam[1][z];
             l1[z] = bc<0>(s0);
             l2[z] = bc<15>(p1);
+            if constexpr (LOCAL) logdec[z] += l1[z] + l2[z];
         }
         {
             const bool bad = (-l1[0] > RANGE_LIMIT * LOG2E) || (-l2[0] > RANGE_LIMIT * LOG2E) || (-l1[1] > RANGE_LIMIT * LOG2E) || (-l2[1] > RANGE_LIMIT * LOG2E);
@@ -246,7 +258,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             carry[0] = p2.x; carry[1] = p2.y;
         }
         // without an initial state nothing has been accumulated before token 0: its decay has no effect at all
-        if (a.gs == nullptr && c == 0 && tp == 0) { gw[0][0] = 0.f; gw[0][1] = 0.f; }
+        if (a.gs == nullptr && a.first && c == 0 && tp == 0) { gw[0][0] = 0.f; gw[0][1] = 0.f; }
 #pragma unroll
         for (int e = 0; e < 2; ++e) S.out[2][tp + 16 * e][4 * w + jq] = pack_bf2(gw[e][0], gw[e][1]);
     };
@@ -287,39 +299,63 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             const int it = it0 + z;
             const int cp = n - 1 - it;
             asm volatile("" : "+v"(jq), "+v"(tp), "+v"(rq), "+v"(pc), "+v"(rg));
-            const bool fin = it >= 3 && cp + 3 >= 0;               // chunk cp + 3 is finished and stored in this iteration
-            store_gv(fin ? cp + 3 : 0, fin);
-            meet_signal(&S.met[2], lane);
+            const bool fin = !LOCAL && it >= 3 && cp + 3 >= 0;      // chunk cp + 3 is finished and stored in this iteration
+            if constexpr (!LOCAL) {
+                store_gv(fin ? cp + 3 : 0, fin);
+                meet_signal(&S.met[2], lane);
+            }
             if ((cut && it == 0) || cp < 0) stage_in(cp, ring[z], part); else stage_in(cp, ring[z], full);
             meet_signal(&S.met[0], lane);
             __builtin_amdgcn_sched_barrier(0);
             fetch(cp >= DEPTH ? cp - DEPTH : 0, ring[z]);
             __builtin_amdgcn_sched_barrier(0);
-            if (fin) { if (cut && it == 3) finish(cp + 3, hq[2], part); else finish(cp + 3, hq[2], full); }
-            meet_signal(&S.met[1], lane);
+            if constexpr (!LOCAL) {
+                if (it == 3 && a.above) {
+                    // P at the end of the block, from the gradient state that enters from above and the saved state there
+                    const float2 p2 = *reinterpret_cast<const float2*>(&S.pex[(n >> 1) & 1][8 * w + 2 * jq]);
+                    carry[0] = p2.x; carry[1] = p2.y;
+                }
+                if (fin) { if (cut && it == 3) finish(cp + 3, hq[2], part); else finish(cp + 3, hq[2], full); }
+                meet_signal(&S.met[1], lane);
+            }
             __builtin_amdgcn_sched_barrier(0);
             hq[2] = hq[1]; hq[1] = hq[0];
             met_ok = meet_wait(&S.met[0], 8u * (it + 1)) && met_ok;        // all rows of chunk cp are staged
             if ((cut && it == 0) || cp < 0) prep(cp, hq[0], part); else prep(cp, hq[0], full);
             __builtin_amdgcn_sched_barrier(0);
-            met_ok = meet_wait(&S.met[1], 8u * (it + 1)) && met_ok;        // all columns of chunk cp + 3 are finished
-            store_out(fin ? cp + 3 : 0, fin);
+            if constexpr (!LOCAL) {
+                met_ok = meet_wait(&S.met[1], 8u * (it + 1)) && met_ok;    // all columns of chunk cp + 3 are finished
+                store_out(fin ? cp + 3 : 0, fin);
+            }
             __syncthreads();
         });
     // (a meeting that never completed, which the counting excludes, would leave this head to the two-sweep kernels)
-    if (lane == 0) a.flags[bh * 8 + w] = (any_exact || !met_ok) ? 1 : 0;
-    // gu of this batch row: sum over the tokens (lanes of a row)
+    // (with several blocks per head the words are cleared by the caller and only ever set)
+    const bool flag = any_exact || !met_ok;
+    if (lane == 0 && (a.NB == 1 || flag)) a.flags[bh * 8 + w] = flag ? 1 : 0;
+    if constexpr (LOCAL) {
+        if (tp == 0) *reinterpret_cast<float2*>(a.blk_decay + ch0) = make_float2(logdec[0], logdec[1]);
+    } else {
+        // gu of this batch row (and block): sum over the tokens (lanes of a row)
 #pragma unroll
-    for (int z = 0; z < 2; ++z) gu_acc[z] = row_sum_to_last(gu_acc[z]);
-    if (tp == 15) *reinterpret_cast<uint32_t*>(a.gu + bh * N + ch0) = pack_bf2(gu_acc[0], gu_acc[1]);
+        for (int z = 0; z < 2; ++z) gu_acc[z] = row_sum_to_last(gu_acc[z]);
+        if (tp == 15) {
+            if (a.gu32 != nullptr) *reinterpret_cast<float2*>(a.gu32 + ch0) = make_float2(gu_acc[0], gu_acc[1]);
+            else *reinterpret_cast<uint32_t*>(a.gu + ch0) = pack_bf2(gu_acc[0], gu_acc[1]);
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------- SD waves
-template <int WMODE>
+template <int WMODE, bool LOCAL>
 DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t bh, const int n, const int nit) {
     const int g = lane >> 4, l16 = lane & 15, j = 16 * w + l16;
     const int nseg = (n + 1) / 2;
-    const float* __restrict__ sv = a.saved + bh * nseg * (N * N);
+    const float* __restrict__ sv = a.saved;                                     // the saved states of this block
+    if constexpr (LOCAL) {                 // only the E waves have work
+        for (int it = 0; it < nit; ++it) __syncthreads();
+        return;
+    }
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     const lds_t sb = lds_of(&S);
     // per-lane address parts
@@ -436,6 +472,20 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
         }
     };
 
+    if (a.ds32 != nullptr) {
+        load_state(a.ds32, b_sv, D);       // the gradient state that enters the block from above
+        if (a.above) {
+            // P there, with the forward state at the end of the block (the first saved state of the block above)
+            load_state(sv + static_cast<size_t>(n >> 1) * (N * N), b_sv, Sa);
+            float p = 0.f;
+#pragma unroll
+            for (int tl = 0; tl < 4; ++tl)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) p = fmaf(D[tl][v], Sa[tl][v], p);
+            p = allreduce_rows(p);
+            if (g == 0) lds_st<float>(sb + PEX0 + ((n >> 1) & 1) * (4 * N) + 64 * w + b_j, p);
+        }
+    }
     load_state(sv + static_cast<size_t>(nseg - 1) * (N * N), b_sv, Sa);
     __syncthreads();                       // iterations 0 and 1: nothing prepared yet
     __syncthreads();
@@ -462,7 +512,7 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
         __syncthreads();
     }
     for (int it = n + 2; it < nit; ++it) __syncthreads();      // the P waves finish chunk 0
-    if (a.gs != nullptr) {
+    if (a.gs != nullptr && a.first) {
 #pragma unroll
         for (int tl = 0; tl < 4; ++tl)
 #pragma unroll
@@ -471,7 +521,7 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
 }
 
 // ---------------------------------------------------------------------------------------------------- E waves
-template <int WMODE>
+template <int WMODE, bool LOCAL>
 DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int n, const int nit) {
     const int g = lane >> 4, l16 = lane & 15;
     const int T = a.T, C = a.C;
@@ -485,6 +535,11 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
     lds_t b_g = 16 * g + 4 * (l16 & 3);                                          // channel 4 g + (l16 & 3) of a per-channel array
     lds_t b_l = 4 * l16;
     f32x4 E[4] = {zero4, zero4, zero4, zero4};     // dS[i = 16w + l16][j = 16 tile + 4g + v]
+    const uint32_t b_e = (16 * w + l16) * N + 4 * g;                            // that element of a [value][key] state
+    if (!LOCAL && a.ds32 != nullptr) {
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) E[tl] = *reinterpret_cast<const f32x4*>(a.ds32 + b_e + 16 * tl);
+    }
 
     // causal tiles of chunk c (waves 0, 1, 2 -> quadrants (t, s) = (0,0) (1,0) (1,1)); accumulator rows are s, lanes t
     auto tiles = [&](const int c) __attribute__((always_inline)) {
@@ -549,9 +604,10 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                 de[q] = lds_ld<float>(so + O_DEC + 64 * q + b_g);
                 d1[q] = lds_ld<float>(so + O_D1 + 64 * q + b_g);
             }
+            // (LOCAL: only the gradient state is wanted, everything that serves gv is left out)
             bf16x8 kh[2][2], kl[2][2];
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
+            for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt)
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks) {
                     kh[tt][ks] = ld_acc(so + O_KPH + tt * 16 * ROW_B + 64 * ks + b_acc);
@@ -561,7 +617,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
             // ------------------------------------------------------------ gv^T[i][s] = (dS d2) K'^T + GY^T A
             bf16x8 dh[2], dl[2];
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
+            for (int ks = 0; ks < (LOCAL ? 0 : 2); ++ks) {
                 float p[4], q[4];
                 static_for<4>([&](auto V) {
                     constexpr int v = decltype(V)::value;
@@ -577,11 +633,11 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
             const bf16x8 gyo = ld_tr(so + O_GY + 32 * w + b_tr, ROW_B);        // lane = value channel 16w + l16, K = tokens
             bf16x8 ah[2], al[2];
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) { ah[tt] = ld_tr(to + T_AH + 32 * tt + b_trt, TROW_B); al[tt] = ld_tr(to + T_AL + 32 * tt + b_trt, TROW_B); }
+            for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt) { ah[tt] = ld_tr(to + T_AH + 32 * tt + b_trt, TROW_B); al[tt] = ld_tr(to + T_AL + 32 * tt + b_trt, TROW_B); }
             __builtin_amdgcn_sched_barrier(0);
             f32x4 G[2] = {zero4, zero4};
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
+            for (int ks = 0; ks < (LOCAL ? 0 : 2); ++ks)
 #pragma unroll
                 for (int tt = 0; tt < 2; ++tt) {
                     G[tt] = mfma(dh[ks], kh[tt][ks], G[tt]);
@@ -595,7 +651,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
             for (int tl = 0; tl < 4; ++tl) { rh[tl] = ld_tr(so + O_RPH + 32 * tl + b_tr, ROW_B); rl[tl] = ld_tr(so + O_RPL + 32 * tl + b_tr, ROW_B); }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt) {
+            for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt) {
                 G[tt] = mfma(gyo, ah[tt], G[tt]);
                 G[tt] = mfma(gyo, al[tt], G[tt]);
             }
@@ -608,9 +664,9 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
             __builtin_amdgcn_sched_barrier(0);
             // gv: lane = token, four consecutive value channels in registers; the prep waves store it in the next iteration,
             // and have taken the last one out of `out` by now (they did that first thing in this iteration)
-            meet_wait(&S.met[2], 8u * (it + 1));
+            if constexpr (!LOCAL) meet_wait(&S.met[2], 8u * (it + 1));
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
+            for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt)
                 lds_st<u32x2>(sb + OUT0 + 3 * PLANE_B + tt * 16 * ROW_B + 32 * w + b_acc, u32x2{pack_bf2(G[tt][0], G[tt][1]), pack_bf2(G[tt][2], G[tt][3])});
             // ------------------------------------------------------------ dS^T <- dS^T dec + d1 R'^T GY
 #pragma unroll
@@ -624,18 +680,36 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                 });
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (it >= 1 && c - 1 >= 0 && w < 3) tiles(c - 1);
+        if (!LOCAL && it >= 1 && c - 1 >= 0 && w < 3) tiles(c - 1);
         __syncthreads();
+    }
+    if constexpr (LOCAL) {
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) *reinterpret_cast<f32x4*>(a.blk_ds + b_e + 16 * tl) = E[tl];
     }
 }
 
-template <int WMODE>
-__global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG a) {
+template <int WMODE, bool LOCAL>
+__global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG arg) {
     __shared__ SmemG S;
     const int tid = threadIdx.x;
-    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
-    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
-    const size_t bh = static_cast<size_t>(b) * a.H + h;
+    // this workgroup's block of the sequence as a problem of its own
+    const int bhx = blockIdx.x / arg.NB, blk = blockIdx.x % arg.NB;
+    const int b = bhx / arg.H, h = bhx % arg.H;
+    const int t0 = blk * arg.TB;
+    const size_t base = (static_cast<size_t>(b) * arg.T + t0) * arg.C + static_cast<size_t>(h) * N;
+    const size_t bh = bhx, bq = bh * arg.NB + blk;
+    ArgsG a = arg;
+    a.T = arg.T - t0 < arg.TB ? arg.T - t0 : arg.TB;
+    const int nsegs = ((arg.T + L - 1) / L + 1) / 2;                // saved states of a whole sequence
+    a.saved = arg.saved + (bh * nsegs + t0 / (2 * L)) * (N * N);
+    a.first = blk == 0;
+    a.above = blk + 1 < arg.NB;
+    if (arg.ds32 != nullptr) a.ds32 = arg.ds32 + bq * (N * N);
+    if (arg.blk_ds != nullptr) { a.blk_ds = arg.blk_ds + bq * (N * N); a.blk_decay = arg.blk_decay + bq * N; }
+    // gu: a row per batch row [B][C], or per block and batch row [NB][B][C] in fp32
+    if (arg.gu32 != nullptr) a.gu32 = arg.gu32 + ((static_cast<size_t>(blk) * (gridDim.x / (arg.NB * arg.H)) + b) * arg.H + h) * N;
+    else a.gu = arg.gu + bh * N;
     const int n = (a.T + L - 1) / L;
     // the quadrant t < 16 <= s of the tiles is never written and must read as zero
     for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTG) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
@@ -643,20 +717,41 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG a) {
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
     const int nit = (n + 2 + DEPTH) & ~(DEPTH - 1);        // iterations of the pipeline: n + 3, in whole trips of the prep loop
-    if (wid < 8) role_prep<WMODE>(S, a, lane, wid, base, h, bh, n, nit);
-    else if (wid < 12) role_sd<WMODE>(S, a, lane, w, bh, n, nit);
-    else role_e<WMODE>(S, a, lane, w, base, n, nit);
+    if (wid < 8) role_prep<WMODE, LOCAL>(S, a, lane, wid, base, h, bh, n, nit);
+    else if (wid < 12) role_sd<WMODE, LOCAL>(S, a, lane, w, bh, n, nit);
+    else role_e<WMODE, LOCAL>(S, a, lane, w, base, n, nit);
+}
+
+// gu of a batch row from its blocks: out[b][c] = bf16(sum_blk part[blk][b][c])
+__global__ __launch_bounds__(256) void gu_block_sum(const int NB, const size_t n, const float* __restrict__ part, uint16_t* __restrict__ out) {
+    const size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i >= n) return;
+    float x = 0.f;
+    for (int blk = 0; blk < NB; ++blk) x += part[blk * n + i];
+    out[i] = f2bf(x);
 }
 
 }  // namespace
 
 int launch_wkv6_bwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
                           const uint16_t* w, const uint16_t* u, const uint16_t* gy, uint16_t* gr, uint16_t* gk, uint16_t* gv,
-                          uint16_t* gw, uint16_t* gu, uint16_t* gs, const float* saved, int* flags) {
+                          uint16_t* gw, uint16_t* gu, uint16_t* gs, const float* saved, int* flags,
+                          int NB, int TB, float* blk_ds, float* blk_decay, float* ds32, float* gu32) {
     ArgsG a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.gs = gs; a.saved = saved; a.flags = flags;
-    hipLaunchKernelGGL(wkv6_bwd_fused<W_RAW>, dim3(B * H), dim3(NTG), 0, st, a);
+    a.NB = 1; a.TB = T;
+    if (NB <= 1) {
+        hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, false>), dim3(B * H), dim3(NTG), 0, st, a);
+        return launch_status();
+    }
+    a.NB = NB; a.TB = TB; a.blk_ds = blk_ds; a.blk_decay = blk_decay;
+    hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, true>), dim3(B * H * NB), dim3(NTG), 0, st, a);
+    if (int e = launch_wkv6_scan_reverse(st, B * H, NB, blk_ds, blk_decay, ds32)) return e;
+    a.blk_ds = nullptr; a.blk_decay = nullptr; a.ds32 = ds32; a.gu32 = gu32;
+    hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, false>), dim3(B * H * NB), dim3(NTG), 0, st, a);
+    const size_t n = static_cast<size_t>(B) * C;
+    hipLaunchKernelGGL(gu_block_sum, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, NB, n, gu32, gu);
     return launch_status();
 }
 

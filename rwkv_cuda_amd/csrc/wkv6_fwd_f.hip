@@ -58,9 +58,18 @@ struct ArgsQ {
     uint16_t* y;
     float* saved;                  // [B*H][ceil(n/2)][64][64]: the state entering every even chunk, [value][key]
     int* flags;                    // [B*H][8]
+    // Sequences cut into NB blocks of TB tokens (a multiple of 64), one workgroup per (batch, head, block), for shapes with
+    // fewer (batch, head) pairs than the chip has CUs.  Three launches: LOCAL = true leaves in blk_state the state that a
+    // block builds from nothing and in blk_decay the log2 of its total decay per key channel; wkv6_scan turns these into
+    // the state entering every block (s32); LOCAL = false then starts each block from there.  NB = 1: one launch, TB = T.
+    int NB, TB;
+    const float* s32;              // [B*H][NB][64][64] or null
+    float* blk_state;              // [B*H][NB][64][64]
+    float* blk_decay;              // [B*H][NB][64]
 };
 
 // ---------------------------------------------------------------------------------------------------- P waves
+template <bool LOCAL>
 DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n, const int nit) {
     int jq = lane >> 4, tp = lane & 15;                 // arithmetic: channel pair, token (and token + 16)
     // Global memory is touched in whole 128-byte rows: eight lanes per row, eight rows per wave and instruction (waves
@@ -102,6 +111,7 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
         meet_signal(&S.met, lane);
     };
     bool any_exact = false, met_ok = true;
+    float logdec[2] = {0.f, 0.f};          // LOCAL: log2 of the decay over the whole block
     auto prep = [&](const int c, auto PARTIAL) __attribute__((always_inline)) {
         const int ch = 8 * w + 2 * jq, cd = 4 * w + jq;        // cd: dword column of the pair in a bf16 plane
         SlotQ& O = S.slot[c % 3];
@@ -126,6 +136,7 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
             cc[1][z] = p1 - lam[1][z];
             l1[z] = bc<0>(s0);
             l2[z] = bc<15>(p1);
+            if constexpr (LOCAL) logdec[z] += l1[z] + l2[z];
         }
         {
             const bool bad = (-l1[0] > RANGE_LIMIT * LOG2E) || (-l2[0] > RANGE_LIMIT * LOG2E) || (-l1[1] > RANGE_LIMIT * LOG2E) || (-l2[1] > RANGE_LIMIT * LOG2E);
@@ -183,17 +194,23 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
             __builtin_amdgcn_sched_barrier(0);
             fetch(it + DEPTH < n ? it + DEPTH : n - 1, ring[z]);
             __builtin_amdgcn_sched_barrier(0);
-            store_y(it >= 3 ? it - 3 : 0, it >= 3);
+            if constexpr (!LOCAL) store_y(it >= 3 ? it - 3 : 0, it >= 3);
             __builtin_amdgcn_sched_barrier(0);
             met_ok = meet_wait(&S.met, 8u * (it + 1)) && met_ok;      // all eight waves have staged their rows of chunk it
             if (it >= n - 1) prep(it, part); else prep(it, full);
             __syncthreads();
         });
     // (a meeting that never completed, which the counting excludes, would leave the results of this head to the other kernel)
-    if (lane == 0) a.flags[bh * 8 + w] = (any_exact || !met_ok) ? 1 : 0;
+    // (with several blocks per head the words are cleared by the caller and only ever set)
+    const bool flag = any_exact || !met_ok;
+    if (lane == 0 && (a.NB == 1 || flag)) a.flags[bh * 8 + w] = flag ? 1 : 0;
+    if constexpr (LOCAL) {
+        if (tp == 0) *reinterpret_cast<float2*>(a.blk_decay + ch0) = make_float2(logdec[0], logdec[1]);
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------- S waves
+template <bool LOCAL>
 DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, const size_t bh, const int n, const int nit) {
     const int g = lane >> 4, l16 = lane & 15, i = 16 * w + l16;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -205,7 +222,10 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
     const uint32_t b_sv = i * N + 4 * g;                                        // [value channel i][key channel 4 g] of a state
     lds_t b_ss = (i * SS + 4 * g) * 4;                                          // the same in the LDS copy
     f32x4 St[4];                           // S[i = 16w + l16][j = 16 tile + 4g + v]
-    if (a.s0 != nullptr) {
+    if (!LOCAL && a.s32 != nullptr) {
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) St[tl] = *reinterpret_cast<const f32x4*>(a.s32 + b_sv + 16 * tl);
+    } else if (!LOCAL && a.s0 != nullptr) {
 #pragma unroll
         for (int tl = 0; tl < 4; ++tl) {
             const uint2 x = *reinterpret_cast<const uint2*>(a.s0 + bh * (N * N) + b_sv + 16 * tl);
@@ -221,7 +241,7 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
     for (int c = 0; c < n; ++c) {
         opaque(b_acc); opaque(b_tr); opaque(b_natt); opaque(b_g); opaque(b_ss);
         const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
-        if (!(c & 1)) {
+        if (!LOCAL && !(c & 1)) {
             // The state entering an even chunk goes to LDS and from there, in the next iteration, to global memory through
             // a wave that has nothing else to do: every workgroup writes its 16 KB at about the same moment, the memory
             // system takes a while to accept such a burst, and a state wave that waited for that would hold up the chunk.
@@ -238,19 +258,22 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
             de[q] = lds_ld<float>(so + O_DEC + 64 * q + b_g);
             d2[q] = lds_ld<float>(so + O_D2 + 64 * q + b_g);
         }
+        // (LOCAL: only the state is wanted, everything that serves y is left out)
         bf16x8 rh[2][2], rl[2][2];
+        if constexpr (!LOCAL) {
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
+            for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                rh[tt][ks] = ld_acc(so + O_RPH + tt * 16 * ROW_B + 64 * ks + b_acc);
-                rl[tt][ks] = ld_acc(so + O_RPL + tt * 16 * ROW_B + 64 * ks + b_acc);
-            }
+                for (int ks = 0; ks < 2; ++ks) {
+                    rh[tt][ks] = ld_acc(so + O_RPH + tt * 16 * ROW_B + 64 * ks + b_acc);
+                    rl[tt][ks] = ld_acc(so + O_RPL + tt * 16 * ROW_B + 64 * ks + b_acc);
+                }
+        }
         __builtin_amdgcn_sched_barrier(0);
         // ------------------------------------------------------------ y^T[i][t] = (S d1) R'^T + V^T A^T
         bf16x8 sh[2], sl[2];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+        for (int ks = 0; ks < (LOCAL ? 0 : 2); ++ks) {
             float p[4], q[4];
             static_for<4>([&](auto V) {
                 constexpr int v = decltype(V)::value;
@@ -266,11 +289,11 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
         const bf16x8 vop = ld_tr(so + O_V + 32 * w + b_tr, ROW_B);              // lane = value channel 16w + l16, K = tokens
         bf16x8 ah[2], al[2];
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) { ah[tt] = ld_op(to + T_AH + tt * 16 * TROW_B + b_natt); al[tt] = ld_op(to + T_AL + tt * 16 * TROW_B + b_natt); }
+        for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt) { ah[tt] = ld_op(to + T_AH + tt * 16 * TROW_B + b_natt); al[tt] = ld_op(to + T_AL + tt * 16 * TROW_B + b_natt); }
         __builtin_amdgcn_sched_barrier(0);
         f32x4 Y[2] = {zero4, zero4};
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+        for (int ks = 0; ks < (LOCAL ? 0 : 2); ++ks)
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt) {
                 Y[tt] = mfma(sh[ks], rh[tt][ks], Y[tt]);
@@ -284,7 +307,7 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
         for (int tl = 0; tl < 4; ++tl) { kh[tl] = ld_tr(so + O_KPH + 32 * tl + b_tr, ROW_B); kl[tl] = ld_tr(so + O_KPL + 32 * tl + b_tr, ROW_B); }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
+        for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt) {
             Y[tt] = mfma(vop, ah[tt], Y[tt]);
             Y[tt] = mfma(vop, al[tt], Y[tt]);
         }
@@ -297,7 +320,7 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
         __builtin_amdgcn_sched_barrier(0);
         // y: lane = token, four consecutive value channels in registers
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt)
+        for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt)
             lds_st<u32x2>(sb + YB0 + (c & 1) * PLANE_B + tt * 16 * ROW_B + 32 * w + b_acc, u32x2{pack_bf2(Y[tt][0], Y[tt][1]), pack_bf2(Y[tt][2], Y[tt][3])});
         // ------------------------------------------------------------ S^T <- S^T dec + d2 K'^T V
 #pragma unroll
@@ -312,9 +335,14 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
         __syncthreads();
     }
     for (int it = n + 2; it < nit; ++it) __syncthreads();      // the P waves store the last y
+    if constexpr (LOCAL) {
+#pragma unroll
+        for (int tl = 0; tl < 4; ++tl) *reinterpret_cast<f32x4*>(a.blk_state + b_sv + 16 * tl) = St[tl];
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------- T waves
+template <bool LOCAL>
 DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, const size_t bh, const int n, const int nit) {
     const int g = lane >> 4, l16 = lane & 15;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -326,12 +354,12 @@ DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
     const int ta = (w == 0) ? 0 : 1, tb = (w == 2) ? 1 : 0;
     // wave 3: the state that the S waves left in LDS in the last iteration; a lane moves 16 bytes of a row, 4 rows a time
     lds_t b_sr = ((lane >> 4) * SS + 4 * (lane & 15)) * 4;
-    float* __restrict__ sv = a.saved + bh * ((n + 1) / 2) * (N * N) + (lane >> 4) * N + 4 * (lane & 15);
+    float* __restrict__ sv = a.saved + (lane >> 4) * N + 4 * (lane & 15);
     __syncthreads();                       // iteration 0
 #pragma unroll 1
     for (int c = 0; c < nit - 1; ++c) {    // iteration c + 1
         opaque(b_nat); opaque(b_tw); opaque(b_l); opaque(b_sr);
-        if (w == 3 && c >= 2 && c - 2 < n && !(c & 1)) {
+        if (!LOCAL && w == 3 && c >= 2 && c - 2 < n && !(c & 1)) {
             float* dst = sv + static_cast<size_t>((c - 2) >> 1) * (N * N);
 #pragma unroll
             for (int q = 0; q < 16; q += 4) {
@@ -342,7 +370,7 @@ DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
                 for (int e = 0; e < 4; ++e) *reinterpret_cast<f32x4*>(dst + (q + e) * (4 * N)) = x[e];
             }
         }
-        if (c < n && w < 3) {
+        if (!LOCAL && c < n && w < 3) {
             const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
             const lds_t ra = so + ta * 16 * ROW_B + b_nat, rb = so + tb * 16 * ROW_B + b_nat;
             bf16x8 kh[2], kl[2], rh[2], rl[2];
@@ -382,12 +410,22 @@ DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
     }
 }
 
-__global__ __launch_bounds__(NTQ) void wkv6_fwd_fused(const ArgsQ a) {
+template <bool LOCAL>
+__global__ __launch_bounds__(NTQ) void wkv6_fwd_fused(const ArgsQ arg) {
     __shared__ SmemQ S;
     const int tid = threadIdx.x;
-    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
-    const size_t base = static_cast<size_t>(b) * a.T * a.C + static_cast<size_t>(h) * N;
-    const size_t bh = static_cast<size_t>(b) * a.H + h;
+    // this workgroup's block of the sequence as a problem of its own
+    const int bhx = blockIdx.x / arg.NB, blk = blockIdx.x % arg.NB;
+    const int b = bhx / arg.H, h = bhx % arg.H;
+    const int t0 = blk * arg.TB;
+    const size_t base = (static_cast<size_t>(b) * arg.T + t0) * arg.C + static_cast<size_t>(h) * N;
+    const size_t bh = bhx, bq = bh * arg.NB + blk;
+    ArgsQ a = arg;
+    a.T = arg.T - t0 < arg.TB ? arg.T - t0 : arg.TB;
+    const int nseg = ((arg.T + L - 1) / L + 1) / 2;                 // saved states of a whole sequence
+    a.saved = arg.saved + (bh * nseg + t0 / (2 * L)) * (N * N);
+    if (arg.s32 != nullptr) a.s32 = arg.s32 + bq * (N * N);
+    if (arg.blk_state != nullptr) { a.blk_state = arg.blk_state + bq * (N * N); a.blk_decay = arg.blk_decay + bq * N; }
     const int n = (a.T + L - 1) / L;
     // the quadrant t < 16 <= s of the tiles is never written and must read as zero
     for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTQ) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
@@ -395,18 +433,55 @@ __global__ __launch_bounds__(NTQ) void wkv6_fwd_fused(const ArgsQ a) {
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
     const int nit = (n + 2 + DEPTH) & ~(DEPTH - 1);        // iterations of the pipeline: n + 3, in whole trips of the prep loop
-    if (wid < 8) role_prep(S, a, lane, wid, base, h, bh, n, nit);
-    else if (wid < 12) role_state(S, a, lane, w, bh, n, nit);
-    else role_tiles(S, a, lane, w, bh, n, nit);
+    if (wid < 8) role_prep<LOCAL>(S, a, lane, wid, base, h, bh, n, nit);
+    else if (wid < 12) role_state<LOCAL>(S, a, lane, w, bh, n, nit);
+    else role_tiles<LOCAL>(S, a, lane, w, bh, n, nit);
+}
+
+// States entering the blocks from the local results, one workgroup of 256 threads per (batch, head), 16 consecutive key
+// channels of one value channel per thread.  Forward (reverse = 0): S = s0; out[blk] = S; S <- S 2^logdec[blk] + local[blk].
+// Reverse: the same from the last block down, from zero: what enters a block from above.
+__global__ __launch_bounds__(256) void wkv6_scan(const float* __restrict__ local, const float* __restrict__ logdec, const uint16_t* __restrict__ s0,
+                                                 float* __restrict__ out, const int NB, const int reverse) {
+    const size_t bh = blockIdx.x;
+    const int e = threadIdx.x * 16, j0 = e % N;
+    float x[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) x[q] = (s0 != nullptr && !reverse) ? bf2f(s0[bh * (N * N) + e + q]) : 0.f;
+    for (int i = 0; i < NB; ++i) {
+        const int blk = reverse ? NB - 1 - i : i;
+        const size_t o = (bh * NB + blk) * (N * N) + e;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            out[o + q] = x[q];
+            x[q] = fmaf(x[q], exp2_fast(logdec[(bh * NB + blk) * N + j0 + q]), local[o + q]);
+        }
+    }
 }
 
 }  // namespace
 
 int launch_wkv6_fwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
-                          const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, float* saved, int* flags) {
+                          const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, float* saved, int* flags,
+                          int NB, int TB, float* blk_state, float* blk_decay, float* s32) {
     ArgsQ a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y; a.saved = saved; a.flags = flags;
-    hipLaunchKernelGGL(wkv6_fwd_fused, dim3(B * H), dim3(NTQ), 0, st, a);
+    a.NB = 1; a.TB = T;
+    if (NB <= 1) {
+        hipLaunchKernelGGL(wkv6_fwd_fused<false>, dim3(B * H), dim3(NTQ), 0, st, a);
+        return launch_status();
+    }
+    a.NB = NB; a.TB = TB; a.blk_state = blk_state; a.blk_decay = blk_decay;
+    hipLaunchKernelGGL(wkv6_fwd_fused<true>, dim3(B * H * NB), dim3(NTQ), 0, st, a);
+    hipLaunchKernelGGL(wkv6_scan, dim3(B * H), dim3(256), 0, st, blk_state, blk_decay, s0, s32, NB, 0);
+    a.blk_state = nullptr; a.blk_decay = nullptr; a.s32 = s32;
+    hipLaunchKernelGGL(wkv6_fwd_fused<false>, dim3(B * H * NB), dim3(NTQ), 0, st, a);
+    return launch_status();
+}
+
+// reverse scan for the backward (wkv6_bwd_f.hip): out[blk] = what enters block blk from above
+int launch_wkv6_scan_reverse(hipStream_t st, int BH, int NB, const float* local, const float* logdec, float* out) {
+    hipLaunchKernelGGL(wkv6_scan, dim3(BH), dim3(256), 0, st, local, logdec, static_cast<const uint16_t*>(nullptr), out, NB, 1);
     return launch_status();
 }
 

@@ -10,6 +10,7 @@ import threading
 
 PASS_GR, PASS_GV, PASS_GK, PASS_ALL = 1, 2, 4, 7
 FLAG_SWEEPS = 0x100
+FLAG_WHOLE = 0x200      # wkv6 one-sweep pair: one workgroup per sequence also for few sequences (no blocks, no scan)
 
 _tls = threading.local()
 

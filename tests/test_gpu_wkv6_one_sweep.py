@@ -31,13 +31,15 @@ def run_pair(lib, B, T, H, r, k, v, w, u, s0, gy, flags=0, saved_fill=None):
     ws = torch.empty(n, device=DEV, dtype=torch.uint8).fill_(0x7f)
     call("rwkv_wkv6f_backward_saved", DEV, B, T, C, H, *d[:6], d[6], gr, gk, gv, gw, gu, gs, saved, nsv, ws, n, flags)
     torch.cuda.synchronize()
-    handed_back = int(ws[-B * H * 32:].view(torch.int32).ne(0).view(B * H, 8).any(1).sum())
+    off = (lib.rwkv_wkv6f_backward_workspace_bytes(B, T, C, H) + 15) // 16 * 16     # the flag words follow the two-sweep workspace
+    handed_back = int(ws[off:off + B * H * 32].view(torch.int32).ne(0).view(B * H, 8).any(1).sum())
     return [y, gr, gk, gv, gw, gu] + ([gs] if s0 is not None else []), handed_back
 
 
 # (B, T, H, state): one chunk, a cut chunk, an odd and an even number of chunks, T = 1, many chunks
+# (from 256 tokens on these small batches run as several blocks per sequence: local states, a scan, the outputs)
 SHAPES = [(1, 32, 1, False), (2, 50, 2, True), (1, 97, 3, True), (2, 64, 1, False), (3, 1, 1, True), (1, 7, 2, False),
-          (2, 96, 2, True), (1, 200, 1, False), (1, 1000, 2, True)]
+          (2, 96, 2, True), (1, 200, 1, False), (1, 1000, 2, True), (1, 300, 2, True), (1, 257, 3, False), (2, 640, 1, True)]
 
 
 @pytest.mark.parametrize("B,T,H,state", SHAPES)
@@ -58,6 +60,38 @@ def test_one_sweep_against_the_oracle(lib, B, T, H, state):
         assert float(gw[:, 0].abs().max()) == 0.0              # nothing to decay at t = 0 without an initial state
 
 
+@pytest.mark.parametrize("B,H,state", [(1, 8, True), (2, 32, False)])
+def test_few_sequences_run_as_blocks_with_a_scan(lib, B, H, state):
+    """B H below the number of CUs at T = 4096: the sequences are cut into blocks (32 of 128 tokens at B1 H8, 4 of 1024 at
+    B2 H32), every block builds its state and gradient state from nothing, a scan hands each block what enters it, and the
+    outputs follow.  Two heads against the oracle on the bar of the reference kernel; the saved states say how it was cut."""
+    T, C = 4096, H * 64
+    print(f"\nwkv6 blocks B={B} H={H} state={state}", flush=True)
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=330 + H, state=state)
+    got, handed_back = run_pair(lib, B, T, H, r, k, v, w, u, s0, gy, saved_fill=0x7f)
+    assert handed_back == 0
+    assert lib.rwkv_wkv6f_saved_bytes(B, T, C, H) > B * H * 64 * (64 * 64 * 4) + B * H * 32      # room for the scan
+    hs = [1, H - 1]
+    ch = torch.cat([torch.arange(h * 64, (h + 1) * 64) for h in hs])
+    rr, kk, vv, ww, gg = (x[:, :, ch].contiguous() for x in (r, k, v, w, gy))
+    uu = u[hs].contiguous()
+    ss = s0[:, hs].contiguous() if state else None
+    ref = list(O.wkv_grads_by_hand(B, T, 128, 2, rr, kk, vv, ww, uu, gg, ss, torch.float64))
+    ref[5] = ref[5].sum(0)
+    emu = O.emulate_wkv6_bf16(B, T, 128, 2, rr, kk, vv, ww, uu, gg, s0=ss, hand=True)
+    chd = ch.to(DEV)
+    sub = [got[0][:, :, chd], got[1][:, :, chd], got[2][:, :, chd], got[3][:, :, chd], got[4][:, :, chd], got[5][hs]]
+    if state:
+        sub.append(got[6][:, hs])
+    for name, a, e, g in zip(NAMES, ref, emu, sub):
+        assert torch.isfinite(g.float()).all(), name
+        assert_no_worse(f"blocks B{B} H{H} " + name, a, e, g)
+    gw = got[4].float()
+    assert float(gw[:, T - 1].abs().max()) == 0.0
+    if not state:
+        assert float(gw[:, 0].abs().max()) == 0.0
+
+
 def test_one_sweep_hands_strong_decays_to_the_two_sweep_kernels(lib):
     """Decays so strong that a channel loses more than e^-60 over 16 tokens: those (batch, head) pairs are flagged by the
     one-sweep kernel and redone by the two-sweep kernels, whose chunks have a step-by-step path; the others are not."""
@@ -72,6 +106,23 @@ def test_one_sweep_hands_strong_decays_to_the_two_sweep_kernels(lib):
     emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
     got, handed_back = run_pair(lib, B, T, H, r, k, v, w, u, s0, gy)
     assert handed_back == 3, handed_back                        # (0,0), (1,0), (1,1); head 2 and (0,1) stay
+    for name, a, e, g in zip(NAMES, ref, emu, got):
+        assert torch.isfinite(g.float()).all(), name
+        assert_no_worse(name, a, e, g)
+
+
+def test_blocks_hand_strong_decays_back_too(lib):
+    """The same with sequences long enough to be cut into blocks: a flag raised by any block of a head hands the head back."""
+    B, T, H = 1, 700, 3
+    C = H * 64
+    r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=319, state=True)
+    w = w.float()
+    w[0, 400:430, 64:128] = 2.5                                 # head 1, inside one of the blocks
+    w = w.to(BF)
+    ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+    got, handed_back = run_pair(lib, B, T, H, r, k, v, w, u, s0, gy)
+    assert handed_back == 1, handed_back
     for name, a, e, g in zip(NAMES, ref, emu, got):
         assert torch.isfinite(g.float()).all(), name
         assert_no_worse(name, a, e, g)
