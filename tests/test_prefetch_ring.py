@@ -218,3 +218,81 @@ def test_no_compiler_vmem_inside_the_prefetching_loops(fname):
         for a, b in prefetching:
             bad = [l for l in lines[a:b + 1] if l.startswith("scratch_")]
             assert not bad, (name, bad)
+
+
+
+def _lambdas_over_raw(text):
+    """name -> body of every lambda of the prep role that takes a ring slot (`Raw& x`)."""
+    out = {}
+    for m in re.finditer(r"auto (\w+) = \[&\]\([^)]*Raw& x[^)]*\)", text):
+        out[m.group(1)] = _lambda_body(text, m.group(1))
+    return out
+
+
+@pytest.mark.parametrize("fname", sorted(KERNELS))
+def test_ring_registers_are_only_touched_by_their_loads_their_wait_and_their_readers(fname):
+    """The compiler takes the outputs of the asm loads as defined right after the asm statement: C++ that reads, copies or
+    assigns a loaded field of a ring slot between its `prefetch` and its `arrived` would touch a register whose load has
+    not landed, and neither the spill count nor the scratch scan would see the move.  On the source text:
+      * `prefetch` and `arrived` name the loaded fields inside asm statements only (outputs of the loads, "+v" operands of
+        the wait) and nothing else of a slot;
+      * the only other code that sees a slot are the reader lambdas scan / operands_a / operands_b, and the ring is never
+        copied, assigned or indexed outside calls of these five;
+      * in the main loop a slot is waited for before its first reader and reloaded after its last one (which slot that
+        is, and that the wait's count covers it, is the business of test_younger_counts_and_slot_contents)."""
+    text = _read(fname)
+    lam = _lambdas_over_raw(text)
+    assert set(lam) == {"prefetch", "arrived", "scan", "operands_a", "operands_b"}, sorted(lam)
+    loaded = set(re.findall(r'"=&v"\(x\.(\w+)\[', lam["prefetch"]))
+    assert {"r", "k", "v"} <= loaded, loaded
+    fields = set(re.search(r"struct Raw \{(.*?)\};", text, re.S).group(1).replace("[", " ").replace(";", " ").replace(",", " ").split())
+    assert loaded <= fields
+    for name in ("prefetch", "arrived"):
+        body = lam[name]
+        outside_asm = re.sub(r"asm volatile\(.*?\);", "", body, flags=re.S)
+        assert not re.search(r"\bx\.", outside_asm), (fname, name, "a slot is touched outside the asm statements")
+        for stmt in re.findall(r"asm volatile\((.*?)\);", body, re.S):
+            named = set(re.findall(r"x\.(\w+)", stmt))
+            assert named <= loaded, (fname, name, named - loaded)
+    # the wait names every loaded field of the mode it is compiled for ("+v": the compiler must treat them as redefined there)
+    for stmt in re.findall(r"asm volatile\((.*?)\);", lam["arrived"], re.S):
+        assert set(re.findall(r'"\+v"\(x\.(\w+)', stmt)) >= {"r", "k", "v"}, (fname, stmt)
+    # nobody else sees the ring
+    start = text.index("Raw ring[")
+    role_end = text.index("// ----------", start)
+    role = text[start:role_end]
+    for m in re.finditer(r"ring\[", role):
+        if role[m.start() - 4:m.start()] == "Raw ":
+            continue
+        stmt_start = max(role.rfind(";", 0, m.start()), role.rfind("{", 0, m.start()), role.rfind("}", 0, m.start())) + 1
+        stmt = role[stmt_start:role.index(";", m.start())]
+        assert re.search(r"\b(prefetch|arrived|scan|operands_a|operands_b)\(", stmt), (fname, stmt.strip())
+        assert not re.search(r"(^|[^=!<>])=[^=]", re.sub(r"\([^()]*\)", "", stmt).replace("exact_cur =", "").replace("exact_next =", "").replace("bool exact_cur", "").replace("bool exact_next", "")) \
+            or re.search(r"exact_(cur|next) = operands_a\(", stmt), (fname, stmt.strip())
+    assert not re.search(r"\bRaw\s+\w+\s*(=|\{|\()", role.replace("Raw ring[", "")), fname
+    # order inside one iteration of the main loop
+    loop = role[role.index("static_for<", role.index("for (int ib = 0")):]
+    at = {k: loop.index(k) for k in ("arrived(ring[(z + 2)", "scan(i + 2, ring[(z + 2)", "operands_a(i + 1, ring[(z + 1)", "operands_b(i + 1, ring[(z + 1)", "prefetch(i + 1 +")}
+    assert at["arrived(ring[(z + 2)"] < at["scan(i + 2, ring[(z + 2)"], fname                 # slot z + 2: waited for, then read
+    assert max(at["operands_a(i + 1, ring[(z + 1)"], at["operands_b(i + 1, ring[(z + 1)"]) < at["prefetch(i + 1 +"], fname   # slot z + 1: read, then reloaded
+    assert re.search(r"prefetch\(i \+ 1 \+ \w+, ring\[\(z \+ 1\)", loop), fname
+
+
+@pytest.mark.parametrize("fname", ["wkv6_fwd_f.hip", "wkv6_bwd_f.hip"])
+def test_one_sweep_kernels_leave_the_waits_to_the_compiler(fname):
+    """The one-sweep kernels prefetch with ordinary loads into ordinary variables: the compiler knows which registers are in
+    flight and places the waits itself, so there is no hand-counted wait to get wrong and no move it could place ahead of
+    one.  What they owe the compiler instead is a loop in which every stage runs in every iteration (its wait counts are
+    taken over all the ways into a wait): the prefetch, the staging and the stores sit outside any `if` of the prep loop
+    that depends on the iteration."""
+    text = _read(fname)
+    assert "asm volatile(\"global_load" not in text and "buffer_load" not in text
+    assert not re.search(r"s_waitcnt vmcnt", re.sub(r"//.*", "", text))
+    start = text.index("for (int it0 = 0; it0 < nit; it0 += DEPTH)")
+    loop = text[start:text.index("__syncthreads();", start)]
+    for call in re.findall(r"^\s*(?:if [^\n]*\))?\s*(fetch|stage_in)\(", loop, re.M):
+        pass
+    # fetch is unconditional; stage_in only chooses between its two forms
+    assert re.search(r"^\s+fetch\(", loop, re.M), fname
+    assert not re.search(r"if \([^\n]*\)\s*fetch\(", loop), fname
+    assert re.search(r"stage_in\([^;]*part\); else stage_in\([^;]*full\);", loop), fname
