@@ -50,6 +50,9 @@ const char* rwkv_strerror(int status);
 int rwkv_last_hip_error(void);
 /* ABI version of this header (bumped when a signature changes). */
 int rwkv_abi_version(void);
+/* The version this header describes: a client compiled against it (the torch shim, a cgo or ctypes binding) compares it
+ * with rwkv_abi_version() of the library it has loaded and refuses a mismatch. */
+#define RWKV_ABI_VERSION 4
 
 /* A measuring aid (no counterpart in the reference): one pass over `bytes` of device memory as a read-only stream
  * (mode 0: src is read, 16 bytes of dst may be written), a write-only stream (mode 1: dst) or a copy (mode 2), so that a
@@ -95,10 +98,12 @@ int rwkv_wkv4_backward(void* stream, int B, int T, int C,
 
 /* rwkv_wkv4_backward without a workspace argument and without any allocation.  It has no counterpart in the reference;
  * it is for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses
- * that forbid hipMalloc.  The backward's scratch (B*T*C floats, touched only beyond T = 32768) lives in a file-scope device array of the library,
- * rwkv_wkv4_backward_noalloc_max_elems() floats (8 MiB) that every GPU the library runs on holds until the process
- * ends; B*T*C beyond that returns RWKV_ERR_WORKSPACE.  All calls on one GPU share that one array: calls that overlap
- * in time on the same GPU (two streams, two threads) race; serialise them.  Results are those of rwkv_wkv4_backward. */
+ * that forbid hipMalloc.  Only the kernels for T > 32768 (or B > 65535) need scratch memory, B*T*C floats: it lives in
+ * a file-scope device array of the library, rwkv_wkv4_backward_noalloc_max_elems() floats (8 MiB) that every GPU the
+ * library runs on holds until the process ends, and for those shapes B*T*C beyond that returns RWKV_ERR_WORKSPACE.
+ * Shorter sequences use no scratch and have no size limit.  All calls on one GPU share the one array: calls that use it
+ * and overlap in time on the same GPU (two streams, two threads) race; serialise them.  Results are those of
+ * rwkv_wkv4_backward. */
 size_t rwkv_wkv4_backward_noalloc_max_elems(void);
 int rwkv_wkv4_backward_noalloc(void* stream, int B, int T, int C,
                                const float* w, const float* u, const float* k, const float* v, const float* gy,
@@ -356,8 +361,12 @@ int rwkv7_statepassing_backward(void* stream, int B, int T, int H,
                                 rwkv_bf16* da, rwkv_bf16* db);
 
 /* The state-passing op with the per-call flags word (RWKV_FLAG_SWEEPS: the step-by-step recurrence kernels instead of
- * the chunked matrix-core kernels; the two families lay `s` out differently, so a backward must be given the flags of
- * its forward).  Here s0 and sT (forward), dsT and ds0 (backward) may be NULL: a missing s0 / dsT is zero, a missing
+ * the chunked matrix-core kernels).  PAIRING RULE: the two families lay `s` out differently (the chunked kernels store
+ * the state entering each chunk, the step kernels, like the reference, the state leaving it) and `s` carries no tag, so a
+ * backward must be given the flags of the forward that wrote its `s` and `sa`.  The entry points without a flags word
+ * (rwkv7_*_forward / _backward, and through them the torch shim) are the chunked family: a forward_ex with
+ * RWKV_FLAG_SWEEPS followed by one of those backwards is undefined -- wrong gradients, no error.  The Python wrapper
+ * keeps the flags of the forward on the autograd context for this reason.  Here s0 and sT (forward), dsT and ds0 (backward) may be NULL: a missing s0 / dsT is zero, a missing
  * sT / ds0 is not written.  No counterpart in the reference. */
 int rwkv7_statepassing_forward_ex(void* stream, int B, int T, int H,
                                   const float* s0, const rwkv_bf16* r, const rwkv_bf16* w, const rwkv_bf16* k,

@@ -80,6 +80,11 @@ def load():
     spec = importlib.util.spec_from_loader(NAME, loader)
     mod = importlib.util.module_from_spec(spec)
     loader.exec_module(mod)
+    # a shim built against another version of the C ABI would resolve its symbols lazily and fail, or misbehave, at call time
+    have, want = getattr(mod, "abi_version", None), _lib.load().rwkv_abi_version()
+    if have != want:
+        raise RuntimeError(f"{SO_PATH} was built against ABI version {have}, librwkv_hip.so is version {want}: "
+                           "rebuild it (rwkv_cuda_amd.binding.build())")
     sys.modules[NAME] = mod
     _ext = mod
     return mod

@@ -59,6 +59,6 @@ const char* rwkv_strerror(int status) {
 
 int rwkv_last_hip_error(void) { return rwkv::g_last_hip_error; }
 
-int rwkv_abi_version(void) { return 3; }
+int rwkv_abi_version(void) { return RWKV_ABI_VERSION; }
 
 }  // extern "C"

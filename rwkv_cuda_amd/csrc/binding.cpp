@@ -18,6 +18,9 @@
 // TORCH_CHECK instead of being cast blindly; work is enqueued on the current HIP stream of the tensors' device instead of
 // the legacy default stream; the scratch some backwards need is taken from torch's caching allocator here (the C ABI
 // itself never allocates).  No arithmetic happens in this file.
+#include <limits>
+#include <initializer_list>
+#include <utility>
 #include <torch/extension.h>
 // PyTorch on ROCm presents HIP devices under the device type "cuda"; these are its stream and guard for that arrangement
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
@@ -48,6 +51,13 @@ struct Checker {
     }
 };
 
+// The C ABI takes its sizes as int: a value outside (0, INT_MAX] would be narrowed silently, and the workspace-size queries
+// run before any tensor is checked against it.
+void dims_ok(const char* op, std::initializer_list<std::pair<const char*, int64_t>> dims) {
+    for (const auto& d : dims)
+        TORCH_CHECK(d.second > 0 && d.second <= std::numeric_limits<int>::max(), op, ": ", d.first, " = ", d.second, " is outside 1 .. 2147483647");
+}
+
 template <typename T> T* ptr(const Tensor& t) { return static_cast<T*>(t.data_ptr()); }
 rwkv_bf16* bp(const Tensor& t) { return static_cast<rwkv_bf16*>(t.data_ptr()); }
 float* fp(const Tensor& t) { return static_cast<float*>(t.data_ptr()); }
@@ -62,6 +72,7 @@ constexpr auto F32 = torch::kFloat32;
 // --------------------------------------------------------------------------------------------- wkv (RWKV-4)
 void wkv_forward(int64_t B, int64_t T, int64_t C, Tensor& w, Tensor& u, Tensor& k, Tensor& v, Tensor& y) {
     const Checker chk{k, "wkv.forward"};
+    dims_ok("wkv.forward", {{"B", B}, {"T", T}, {"C", C}});
     chk(w, F32, C, "w"); chk(u, F32, C, "u"); chk(k, F32, B * T * C, "k"); chk(v, F32, B * T * C, "v"); chk(y, F32, B * T * C, "y");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(k.device());
     ok(rwkv_wkv4_forward(stream_of(k), B, T, C, fp(w), fp(u), fp(k), fp(v), fp(y)), "wkv.forward");
@@ -69,6 +80,7 @@ void wkv_forward(int64_t B, int64_t T, int64_t C, Tensor& w, Tensor& u, Tensor& 
 void wkv_backward(int64_t B, int64_t T, int64_t C, Tensor& w, Tensor& u, Tensor& k, Tensor& v, Tensor& gy, Tensor& gw,
                   Tensor& gu, Tensor& gk, Tensor& gv) {
     const Checker chk{k, "wkv.backward"};
+    dims_ok("wkv.backward", {{"B", B}, {"T", T}, {"C", C}});
     chk(w, F32, C, "w"); chk(u, F32, C, "u"); chk(k, F32, B * T * C, "k"); chk(v, F32, B * T * C, "v"); chk(gy, F32, B * T * C, "gy");
     chk(gw, F32, B * C, "gw"); chk(gu, F32, B * C, "gu"); chk(gk, F32, B * T * C, "gk"); chk(gv, F32, B * T * C, "gv");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(k.device());
@@ -81,12 +93,14 @@ void wkv_backward(int64_t B, int64_t T, int64_t C, Tensor& w, Tensor& u, Tensor&
 // --------------------------------------------------------------------------------------------- timex (depthwise_conv1d)
 void timex_forward(Tensor& w, const Tensor& k, Tensor& x, double eps, int64_t B, int64_t C, int64_t T) {
     const Checker chk{k, "timex.forward"};
+    dims_ok("timex.forward", {{"B", B}, {"C", C}, {"T", T}});
     chk(w, F32, C * T, "w"); chk(k, F32, B * C * T, "k"); chk(x, F32, B * C * T, "x");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(k.device());
     ok(rwkv_timex_forward(stream_of(k), fp(w), fp(k), fp(x), static_cast<float>(eps), B, C, T), "timex.forward");
 }
 void timex_backward(Tensor& w, const Tensor& k, const Tensor& gwk, Tensor& gw, Tensor& gk, int64_t B, int64_t C, int64_t T) {
     const Checker chk{k, "timex.backward"};
+    dims_ok("timex.backward", {{"B", B}, {"C", C}, {"T", T}});
     chk(w, F32, C * T, "w"); chk(k, F32, B * C * T, "k"); chk(gwk, F32, B * C * T, "gwk"); chk(gw, F32, B * C * T, "gw"); chk(gk, F32, B * C * T, "gk");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(k.device());
     ok(rwkv_timex_backward(stream_of(k), fp(w), fp(k), fp(gwk), fp(gw), fp(gk), B, C, T), "timex.backward");
@@ -95,6 +109,7 @@ void timex_backward(Tensor& w, const Tensor& k, const Tensor& gwk, Tensor& gw, T
 // --------------------------------------------------------------------------------------------- wkv5 (bf16 or fp32 I/O)
 void wkv5_forward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor& k, Tensor& v, Tensor& w, Tensor& u, Tensor& y) {
     const Checker chk{r, "wkv5.forward"};
+    dims_ok("wkv5.forward", {{"B", B}, {"T", T}, {"C", C}, {"H", H}});
     const auto dt = r.scalar_type();
     TORCH_CHECK(dt == BF || dt == F32, "wkv5.forward: r must be bfloat16 or float32");
     chk(r, dt, B * T * C, "r"); chk(k, dt, B * T * C, "k"); chk(v, dt, B * T * C, "v"); chk(w, F32, C, "w"); chk(u, dt, C, "u"); chk(y, dt, B * T * C, "y");
@@ -110,6 +125,7 @@ void wkv5_forward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor&
 void wkv5_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor& k, Tensor& v, Tensor& w, Tensor& ww, Tensor& u,
                    Tensor& gy, Tensor& gr, Tensor& gk, Tensor& gv, Tensor& gw, Tensor& gu) {
     const Checker chk{r, "wkv5.backward"};
+    dims_ok("wkv5.backward", {{"B", B}, {"T", T}, {"C", C}, {"H", H}});
     const auto dt = r.scalar_type();
     TORCH_CHECK(dt == BF || dt == F32, "wkv5.backward: r must be bfloat16 or float32");
     chk(r, dt, B * T * C, "r"); chk(k, dt, B * T * C, "k"); chk(v, dt, B * T * C, "v"); chk(w, F32, C, "w"); chk(ww, F32, C, "ww");
@@ -132,6 +148,7 @@ void wkv5_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor
 void wkv5a_forward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor& k, Tensor& v, Tensor& w1, Tensor& u1, Tensor& w2,
                    Tensor& u2, Tensor& y) {
     const Checker chk{r, "wkv5a.forward"};
+    dims_ok("wkv5a.forward", {{"B", B}, {"T", T}, {"C", C}, {"H", H}});
     chk(r, F32, B * T * C, "r"); chk(k, F32, B * T * C, "k"); chk(v, F32, B * T * C, "v"); chk(y, F32, B * T * C, "y");
     chk(w1, F32, C, "w1"); chk(u1, F32, C, "u1"); chk(w2, F32, C, "w2"); chk(u2, F32, C, "u2");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(r.device());
@@ -141,6 +158,7 @@ void wkv5a_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tenso
                     Tensor& w2, Tensor& ww2, Tensor& u2, Tensor& gy, Tensor& gr, Tensor& gk, Tensor& gv, Tensor& gw1, Tensor& gu1,
                     Tensor& gw2, Tensor& gu2) {
     const Checker chk{r, "wkv5a.backward"};
+    dims_ok("wkv5a.backward", {{"B", B}, {"T", T}, {"C", C}, {"H", H}});
     chk(r, F32, B * T * C, "r"); chk(k, F32, B * T * C, "k"); chk(v, F32, B * T * C, "v"); chk(gy, F32, B * T * C, "gy");
     chk(gr, F32, B * T * C, "gr"); chk(gk, F32, B * T * C, "gk"); chk(gv, F32, B * T * C, "gv");
     for (const Tensor* t : {&w1, &ww1, &u1, &w2, &ww2, &u2}) chk(*t, F32, C, "a per-head parameter");
@@ -153,6 +171,7 @@ void wkv5a_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tenso
 // --------------------------------------------------------------------------------------------- wkv6 (fp32 ew)
 void wkv6_forward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor& k, Tensor& v, Tensor& w, Tensor& u, Tensor& y) {
     const Checker chk{r, "wkv6.forward"};
+    dims_ok("wkv6.forward", {{"B", B}, {"T", T}, {"C", C}, {"H", H}});
     chk(r, BF, B * T * C, "r"); chk(k, BF, B * T * C, "k"); chk(v, BF, B * T * C, "v"); chk(w, F32, B * T * C, "w"); chk(u, BF, C, "u");
     chk(y, BF, B * T * C, "y");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(r.device());
@@ -161,6 +180,7 @@ void wkv6_forward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor&
 void wkv6_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor& k, Tensor& v, Tensor& w, Tensor& u, Tensor& gy,
                    Tensor& gr, Tensor& gk, Tensor& gv, Tensor& gw, Tensor& gu) {
     const Checker chk{r, "wkv6.backward"};
+    dims_ok("wkv6.backward", {{"B", B}, {"T", T}, {"C", C}, {"H", H}});
     chk(r, BF, B * T * C, "r"); chk(k, BF, B * T * C, "k"); chk(v, BF, B * T * C, "v"); chk(w, F32, B * T * C, "w"); chk(u, BF, C, "u");
     chk(gy, BF, B * T * C, "gy"); chk(gr, BF, B * T * C, "gr"); chk(gk, BF, B * T * C, "gk"); chk(gv, BF, B * T * C, "gv");
     chk(gw, BF, B * T * C, "gw"); chk(gu, BF, B * C, "gu");
@@ -175,6 +195,7 @@ void wkv6_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor
 // --------------------------------------------------------------------------------------------- wkv6b (wkv6_state)
 void wkv6b_forward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor& k, Tensor& v, Tensor& w, Tensor& u, Tensor& s, Tensor& y) {
     const Checker chk{r, "wkv6b.forward"};
+    dims_ok("wkv6b.forward", {{"B", B}, {"T", T}, {"C", C}, {"H", H}});
     chk(r, BF, B * T * C, "r"); chk(k, BF, B * T * C, "k"); chk(v, BF, B * T * C, "v"); chk(w, BF, B * T * C, "w"); chk(u, BF, C, "u");
     chk(s, BF, B * C * (C / H), "s"); chk(y, BF, B * T * C, "y");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(r.device());
@@ -183,6 +204,7 @@ void wkv6b_forward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor
 void wkv6b_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tensor& k, Tensor& v, Tensor& w, Tensor& u, Tensor& s,
                     Tensor& gy, Tensor& gr, Tensor& gk, Tensor& gv, Tensor& gw, Tensor& gu, Tensor& gs) {
     const Checker chk{r, "wkv6b.backward"};
+    dims_ok("wkv6b.backward", {{"B", B}, {"T", T}, {"C", C}, {"H", H}});
     chk(r, BF, B * T * C, "r"); chk(k, BF, B * T * C, "k"); chk(v, BF, B * T * C, "v"); chk(w, BF, B * T * C, "w"); chk(u, BF, C, "u");
     chk(s, BF, B * C * (C / H), "s"); chk(gy, BF, B * T * C, "gy"); chk(gr, BF, B * T * C, "gr"); chk(gk, BF, B * T * C, "gk");
     chk(gv, BF, B * T * C, "gv"); chk(gw, BF, B * T * C, "gw"); chk(gu, BF, B * C, "gu"); chk(gs, BF, B * C * (C / H), "gs");
@@ -198,8 +220,9 @@ void wkv6b_backward(int64_t B, int64_t T, int64_t C, int64_t H, Tensor& r, Tenso
 struct Dims7 { int B, T, H; int64_t btc, state, ckpt; };
 Dims7 dims7(const Tensor& r, const char* op) {
     TORCH_CHECK(r.dim() == 4 && r.size(3) == 64, op, ": r must be [B,T,H,64]");
+    dims_ok(op, {{"B", r.size(0)}, {"T", r.size(1)}, {"H", r.size(2)}});
     Dims7 d;
-    d.B = r.size(0); d.T = r.size(1); d.H = r.size(2);
+    d.B = static_cast<int>(r.size(0)); d.T = static_cast<int>(r.size(1)); d.H = static_cast<int>(r.size(2));
     d.btc = r.numel(); d.state = static_cast<int64_t>(d.B) * d.H * 64 * 64; d.ckpt = d.state * (d.T / RWKV7_CHUNK_LEN);
     return d;
 }
@@ -292,6 +315,8 @@ void r7_backward(Tensor& r, Tensor& w, Tensor& k, Tensor& v, Tensor& a, Tensor& 
 // One Python extension module with a submodule per reference extension: `ext.wkv6state.forward(...)` is what
 // `wkv6state_cuda.forward(...)` is in wkv6_state/run.py:77,103.
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+    // the ABI this shim was compiled against; binding.load() compares it with the library's
+    m.attr("abi_version") = RWKV_ABI_VERSION;
     auto sub = [&](const char* name, auto fwd, auto bwd) {
         auto s = m.def_submodule(name);
         s.def("forward", fwd);

@@ -970,6 +970,12 @@ void launch4_bwd(hipStream_t st, int B, int T, int C, const float* w, const floa
     }
 }
 
+// the forms of launch4_bwd that take the workspace `ze` (the plain kernel and the one for very long sequences)
+bool bwd_uses_workspace(int B, int T) {
+    const int S = (T + NSEG - 1) / NSEG;
+    return B > 65535 || (S > 16 && T > BLK_T * BLK_MAX);
+}
+
 int check4(int B, int T, int C) {
     if (B <= 0 || T <= 0 || C <= 0) return RWKV_ERR_SHAPE;
     if (static_cast<long long>(B) * C > 0x7fffffffLL) return RWKV_ERR_SHAPE;
@@ -1066,11 +1072,17 @@ size_t rwkv_wkv4_backward_noalloc_max_elems(void) { return NOALLOC_MAX_FLOATS; }
 int rwkv_wkv4_backward_noalloc(void* stream, int B, int T, int C, const float* w, const float* u, const float* k,
                                const float* v, const float* gy, float* gw, float* gu, float* gk, float* gv) {
     if (int e = check4(B, T, C)) return e;
-    if (static_cast<unsigned long long>(B) * T * C > NOALLOC_MAX_FLOATS) return RWKV_ERR_WORKSPACE;
+    if (int e = check_ptrs({w, u, k, v, gy, gw, gu, gk, gv})) return e;
     float* ws = nullptr;
-    if (int e = scratch_of_current_device(&ws)) return e;
-    // every element of the scratch that the kernels read they have written earlier in the same launch: nothing to clear
-    return rwkv_wkv4_backward(stream, B, T, C, w, u, k, v, gy, gw, gu, gk, gv, ws, static_cast<size_t>(B) * T * C * sizeof(float));
+    // The kernels for T up to 32768 keep their intermediates in registers and LDS; only the plain kernel (B above 65535)
+    // and the one for longer sequences write B T C floats to a workspace, and only those shapes are bounded by the scratch.
+    if (bwd_uses_workspace(B, T)) {
+        if (static_cast<unsigned long long>(B) * T * C > NOALLOC_MAX_FLOATS) return RWKV_ERR_WORKSPACE;
+        // every element of the scratch that the kernels read they have written earlier in the same launch: nothing to clear
+        if (int e = scratch_of_current_device(&ws)) return e;
+    }
+    launch4_bwd<false>(static_cast<hipStream_t>(stream), B, T, C, w, u, k, v, gy, gw, gu, gk, gv, ws);
+    return launch_status();
 }
 
 }  // extern "C"

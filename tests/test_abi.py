@@ -27,7 +27,7 @@ def test_header_and_bindings_agree(lib):
 
 
 def test_status_text(lib):
-    assert lib.rwkv_abi_version() == 3
+    assert lib.rwkv_abi_version() == 4
     assert lib.rwkv_strerror(0) == b"ok"
     for code in (-1, -2, -3, -4, -5, -99):
         assert len(lib.rwkv_strerror(code)) > 0

@@ -200,3 +200,12 @@ def test_shim_rejects_wrong_dtype_and_cpu_tensors(ext):
     c = torch.zeros(4)
     with pytest.raises(RuntimeError, match="HIP device"):
         torch.ops.wkv.forward(1, 1, 4, c, c, c, c, c)
+
+
+def test_shim_is_built_against_the_loaded_abi_and_refuses_sizes_beyond_int(lib, ext):
+    assert ext.abi_version == lib.rwkv_abi_version()
+    x = torch.zeros(16, device=DEV, dtype=torch.float32)
+    with pytest.raises(RuntimeError, match="outside 1 .. 2147483647"):
+        ext.wkv.forward(2 ** 31, 1, 1, x, x, x, x, x)               # would be narrowed to a negative int
+    with pytest.raises(RuntimeError, match="outside 1 .. 2147483647"):
+        ext.wkv6.forward(1, 0, 64, 1, x, x, x, x, x, x)

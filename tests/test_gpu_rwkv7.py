@@ -181,3 +181,22 @@ def test_rwkv7_fp32_mode_siblings(lib):
     for name, a_, e, g in zip(NAMES, ref, emu, got):
         if g is not None:
             assert_fp32_mode("fp32 stateless op " + name, a_, e, g)
+
+
+def test_rwkv7_backward_uses_the_kernel_family_of_its_forward(lib):
+    """The two kernel families lay the checkpoint tensor `s` out differently and nothing in it says which one wrote it: a
+    backward must run with the flags of its forward.  The wrapper keeps them on the autograd context, so a forward issued
+    inside `algorithm("sweeps")` gets the step kernels' backward even when autograd runs it after the block has ended."""
+    B, T, H = 2, 48, 2
+    args = synth.rwkv7_inputs(B, T, H, 64, seed=35)
+    ref, emu = O.grads(*args), O.emulate_bf16(*args)
+    s0, r, w, k, v, a, b, dy, dsT = args
+    t = [x.to(DEV).requires_grad_(True) for x in (s0, r, w, k, v, a, b)]
+    with options.algorithm("sweeps"):
+        y, S = R.RWKV7_STATE_PASSING_CLAMPW_CUDA(t[0], *(x.contiguous().view(B, T, H * 64) for x in t[1:]))
+    assert options.current_flags() == 0                            # the block has ended: the default family is current again
+    torch.autograd.backward([y, S], [dy.to(DEV).view(B, T, H * 64), dsT.to(DEV)])
+    torch.cuda.synchronize()
+    got = [y.detach().view(B, T, H, 64), S.detach()] + [x.grad for x in t]
+    for name, a_, e, g in zip(NAMES, ref, emu, got):
+        assert_no_worse("sweeps forward, backward after the block: " + name, a_, e, g)

@@ -41,8 +41,17 @@ def test_noalloc_equals_workspace_entry_point_twice(lib):
             assert torch.equal(a, g), name                         # same kernels, same order of operations: bit-identical
 
 
-def test_noalloc_rejects_sizes_beyond_its_scratch(lib):
-    B, T, C = 4, 1024, 768                                         # 3 145 728 elements > 2 097 152
+def test_noalloc_limit_applies_only_where_the_scratch_is_used(lib):
+    """Sequences up to 32768 tokens run on kernels that keep their intermediates on the chip: no scratch, no limit (the
+    reference's own shapes B32 T768 C768 and B4 T1024 C768 are above 2^21 elements).  Beyond that length the kernel parks
+    B T C floats in the scratch, and a shape that does not fit is refused."""
+    for B, T, C, seed in ((32, 768, 768, 9), (4, 1024, 768, 10)):
+        assert B * T * C > lib.rwkv_wkv4_backward_noalloc_max_elems()
+        print(f"\nwkv4 noalloc, no scratch needed: B={B} T={T} C={C}", flush=True)
+        ref, got = _both(lib, B, T, C, seed)
+        for name, a, g in zip(("gw", "gu", "gk", "gv"), ref, got):
+            assert torch.equal(a, g), name
+    B, T, C = 2, 40000, 64                                         # 5 120 000 elements > 2 097 152, and T > 32768
     z = torch.zeros(16, device=DEV, dtype=torch.float32)
     status = lib.rwkv_wkv4_backward_noalloc(None, B, T, C, *([z.data_ptr()] * 9))
     assert status == -4
