@@ -67,7 +67,7 @@ def test_bad_arguments_are_rejected_without_a_launch(lib):
     assert lib.rwkv_wkv5a_backward(None, 2, 8, 128, 2, *([p] * 16), p + 4) == -3
     assert lib.rwkv_wkv4_backward(None, 1, 4, 4, *([p] * 9), None, 0) == -4
     # the entry point that allocates nothing rejects sizes beyond its built-in scratch before it touches the device
-    assert lib.rwkv_wkv4_backward_noalloc(None, 4, 1024, 768, *([p] * 9)) == -4
+    assert lib.rwkv_wkv4_backward_noalloc(None, 2, 40000, 64, *([p] * 9)) == -4      # T > 32768: the kernel that uses the scratch
     # per-call flags: same validation as the plain entry points
     assert lib.rwkv_wkv6state_backward_ex(None, 2, 8, 128, 2, *([p] * 13), None, 0, 0x100) == -4
     assert lib.rwkv_wkv6raw_forward_ex(None, 1, 8, 130, 1, p, p, p, p, p, p, 0) == -1
