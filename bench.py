@@ -189,9 +189,22 @@ def make_wkv5(dev, H=32, N=64):
     ew = (-torch.exp(w.float())).contiguous()
     eew = torch.exp(ew).contiguous()
 
+    one_sweep = N == 64 and ALGO == "chunked"
+    if one_sweep:
+        nsaved = lib.rwkv_wkv5s_saved_bytes(B, T, C, H)
+        saved = torch.empty(nsaved, device=dev, dtype=torch.uint8)
+        sbytes = lib.rwkv_wkv5s_backward_workspace_bytes(B, T, C, H)
+        sws = torch.empty(sbytes, device=dev, dtype=torch.uint8)
+    fwd1 = lambda: call("rwkv_wkv5s_forward", dev, B, T, C, H, r, k, v, w, u, y, decay, saved, nsaved, FLAGS)
+    bwd1 = lambda: call("rwkv_wkv5s_backward", dev, B, T, C, H, r, k, v, w, decay, u, gy, gr, gk, gv, gw_sum, gu_sum, saved, nsaved, sws, sbytes, FLAGS)
+
     def step():
         # what WKV_5.forward / backward do; the decay transforms (wkv5_bf16/run.py:63-64) and the sums over the batch
-        # (:86-87) run inside the library
+        # (:86-87) run inside the library.  Head size 64: one forward and one reverse sweep (the kernels of wkv6).
+        if one_sweep:
+            fwd1()
+            bwd1()
+            return
         call("rwkv_wkv5raw_forward_ws", dev, B, T, C, H, r, k, v, w, u, y, decay, fws, fbytes, FLAGS)
         call("rwkv_wkv5raw_backward", dev, B, T, C, H, r, k, v, decay, u, gy, gr, gk, gv, gw_sum, gu_sum, ws, nbytes, FLAGS)
 
@@ -200,7 +213,10 @@ def make_wkv5(dev, H=32, N=64):
             call("rwkv_wkv5_backward_ex", dev, B, T, C, H, r, k, v, eew, ew, u, gy, gr, gk, gv, gw, gu, ws, nbytes, mask | FLAGS)
         return run
 
-    if N == 64:
+    if one_sweep:
+        kernels = [("wkv6_fwd_fused<head decay> (keeps states)", fwd1, 8 * C * tok),       # r k v -> y
+                   ("wkv6_bwd_fused<head decay> (+ batch sums)", bwd1, 14 * C * tok)]      # r k v gy -> gr gk gv
+    elif N == 64:
         kernels = [("wkv6_fwd_ws<head decay>", lambda: call("rwkv_wkv5_forward_ex", dev, B, T, C, H, r, k, v, eew, u, y, FLAGS), 8 * C * tok),
                    ("wkv6_bwd_a_ws<head decay>", bwd(1), 10 * C * tok),           # r k v gy -> gr (+ fp32 workspace)
                    ("wkv6_bwd_b_ws<head decay>", bwd(4), 12 * C * tok)]           # r k v gy -> gk gv

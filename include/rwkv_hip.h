@@ -312,6 +312,23 @@ int rwkv_wkv6f_backward_saved(void* stream, int B, int T, int C, int H,
                               rwkv_bf16* gs, const void* saved, size_t saved_bytes,
                               void* workspace, size_t workspace_bytes, unsigned flags);
 
+/* The same pair for wkv5 at head size 64 (no counterpart in the reference; what WKV_5 of wkv5_bf16/run.py:44-88 does in
+ * two calls, its wrapper's decay transforms and sums included): raw bf16 w[H,N] in, y out, `decay` = [eew | ew] (2 C
+ * floats) left by the forward for the backward, gw, gu [H,N] summed over time and batch out.  The decay of a channel
+ * stands in for every token's decay in the kernels of rwkv_wkv6f_*, and its gradient is added up over the tokens inside
+ * the kernel.  Other head sizes, RWKV_FLAG_SWEEPS / RWKV_PASS_* or saved = NULL: rwkv_wkv5raw_forward / _backward. */
+size_t rwkv_wkv5s_saved_bytes(int B, int T, int C, int H);
+int rwkv_wkv5s_forward(void* stream, int B, int T, int C, int H,
+                       const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                       const rwkv_bf16* w_raw, const rwkv_bf16* u, rwkv_bf16* y, float* decay,
+                       void* saved, size_t saved_bytes, unsigned flags);
+size_t rwkv_wkv5s_backward_workspace_bytes(int B, int T, int C, int H);
+int rwkv_wkv5s_backward(void* stream, int B, int T, int C, int H,
+                        const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                        const rwkv_bf16* w_raw, const float* decay, const rwkv_bf16* u, const rwkv_bf16* gy,
+                        rwkv_bf16* gr, rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu,
+                        const void* saved, size_t saved_bytes, void* workspace, size_t workspace_bytes, unsigned flags);
+
 /* ---------------------------------------------------------------------------------------
  * RWKV-6 wkv with initial state.  Replaces cuda_forward / cuda_backward of
  * wkv6_state/cuda/wkv6state_op.cpp:5-6 (kernels: wkv6state_cuda_v1a.cu:6-308).

@@ -144,6 +144,10 @@ SIGNATURES = {
     "rwkv_wkv6f_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 7 + [_P, _Z, _U]),
     "rwkv_wkv6f_backward_saved_workspace_bytes": (_Z, [_I, _I, _I, _I]),
     "rwkv_wkv6f_backward_saved": (_I, [_P, _I, _I, _I, _I] + [_P] * 13 + [_P, _Z, _P, _Z, _U]),
+    "rwkv_wkv5s_saved_bytes": (_Z, [_I, _I, _I, _I]),
+    "rwkv_wkv5s_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 7 + [_P, _Z, _U]),
+    "rwkv_wkv5s_backward_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "rwkv_wkv5s_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_P, _Z, _P, _Z, _U]),
     "rwkv_wkv5f32_forward": (_I, [_P, _I, _I, _I, _I] + [_P] * 6),
     "rwkv_wkv5f32_backward": (_I, [_P, _I, _I, _I, _I] + [_P] * 12),
     "rwkv_wkv5f32_backward_ex": (_I, [_P, _I, _I, _I, _I] + [_P] * 12 + [_U]),

@@ -144,7 +144,8 @@ int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H,
 // (blk_state, s32: [B*H*NB][64][64] floats each, blk_decay: [B*H*NB][64]; flags cleared by the caller)
 int launch_wkv6_fwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
                           const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, float* saved, int* flags,
-                          int NB = 1, int TB = 0, float* blk_state = nullptr, float* blk_decay = nullptr, float* s32 = nullptr);
+                          int NB = 1, int TB = 0, float* blk_state = nullptr, float* blk_decay = nullptr, float* s32 = nullptr,
+                          bool head_decay = false);
 int launch_wkv6_scan_reverse(hipStream_t st, int BH, int NB, const float* local, const float* logdec, float* out);
 int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                             const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
@@ -160,7 +161,8 @@ int launch_wkv6_bwd_fused(hipStream_t st, int B, int T, int C, int H, const uint
                           const uint16_t* w, const uint16_t* u, const uint16_t* gy, uint16_t* gr, uint16_t* gk, uint16_t* gv,
                           uint16_t* gw, uint16_t* gu, uint16_t* gs, const float* saved, int* flags,
                           int NB = 1, int TB = 0, float* blk_ds = nullptr, float* blk_decay = nullptr, float* ds32 = nullptr,
-                          float* gu32 = nullptr);
+                          float* gu32 = nullptr, uint16_t* gwp = nullptr, float* gw32 = nullptr);
+// gwp != nullptr: wkv5 (w is the raw decay per channel [H][64]; its gradient per batch row goes to gwp [B][C], gw is not written)
 // wkv5 with heads of 128 channels as four heads of 64 (see ArgsB in wkv6_chunk.h): one launch of each kernel per value
 // of `cross`.  Forward and first sweep: the first launch (cross = 0) leaves fp32 terms, the second adds them to its own
 // and writes the bf16 outputs.  Second sweep: both launches leave fp32 terms (its waves have no registers to spare for

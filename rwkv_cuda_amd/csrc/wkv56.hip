@@ -1354,6 +1354,85 @@ int rwkv_wkv6f_backward_saved(void* stream, int B, int T, int C, int H, const rw
     return launch_status();
 }
 
+// ---- wkv5 (head size 64) on the one-sweep pair: the raw decay of a channel stands in for every token's, its gradient is
+//      summed over the tokens inside the kernel.  `decay` = [eew | ew] is made for the kernels that redo flagged heads.
+size_t rwkv_wkv5s_saved_bytes(int B, int T, int C, int H) { return rwkv_wkv6f_saved_bytes(B, T, C, H); }
+
+int rwkv_wkv5s_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                       const rwkv_bf16* w_raw, const rwkv_bf16* u, rwkv_bf16* y, float* decay, void* saved, size_t saved_bytes,
+                       unsigned flags) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (int e = check_ptrs({r, k, v, w_raw, u, y, decay}, C == H * N)) return e;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(wkv5_decay_transform, dim3((C + 255) / 256), dim3(256), 0, st, C, w_raw, decay);
+    if (!fused_ok(T, C, H, flags) || saved == nullptr) return rwkv_wkv5_forward_ex(stream, B, T, C, H, r, k, v, decay, u, y, flags);
+    if (saved_bytes < rwkv_wkv5s_saved_bytes(B, T, C, H) || !aligned16(saved)) return RWKV_ERR_WORKSPACE;
+    const size_t nflag = round16(static_cast<size_t>(B) * H * 8 * sizeof(int));
+    char* sb = static_cast<char*>(saved);
+    int* flg = reinterpret_cast<int*>(sb + saved_states_bytes(B, T, H));
+    int TB;
+    const int NB = scan_blocks(B, T, H, &TB, flags);
+    if (NB > 1) {
+        const size_t nq = static_cast<size_t>(B) * H * NB;
+        float* local = reinterpret_cast<float*>(sb + saved_states_bytes(B, T, H) + nflag);
+        float* s32 = local + nq * 64 * 64;
+        float* logdec = s32 + nq * 64 * 64;
+        zero_words(st, flg, static_cast<size_t>(B) * H * 8);
+        if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w_raw, u, nullptr, y, static_cast<float*>(saved), flg, NB, TB, local, logdec, s32, true)) return e;
+    } else if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w_raw, u, nullptr, y, static_cast<float*>(saved), flg, 1, 0, nullptr, nullptr, nullptr, true)) return e;
+    return launch_wkv6_fwd_chunk(st, W_HEAD, B, T, C, H, r, k, v, decay, u, nullptr, y, static_cast<float*>(saved), flg);
+}
+
+size_t rwkv_wkv5s_backward_workspace_bytes(int B, int T, int C, int H) {
+    const size_t n = rwkv_wkv5raw_backward_workspace_bytes(B, T, C, H);
+    if (n == 0) return 0;
+    int TB;
+    const int NB = C == H * N ? scan_blocks(B, T, H, &TB) : 1;
+    // several blocks per sequence: the scan's scratch and gw, gu per block and batch row in fp32
+    const size_t scan = NB <= 1 ? 0 : scan_scratch_bytes(B, T, H) + 2 * static_cast<size_t>(NB) * B * C * sizeof(float);
+    return round16(n) + round16(static_cast<size_t>(B) * H * 8 * sizeof(int)) + scan;
+}
+
+int rwkv_wkv5s_backward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k, const rwkv_bf16* v,
+                        const rwkv_bf16* w_raw, const float* decay, const rwkv_bf16* u, const rwkv_bf16* gy, rwkv_bf16* gr,
+                        rwkv_bf16* gk, rwkv_bf16* gv, rwkv_bf16* gw, rwkv_bf16* gu, const void* saved, size_t saved_bytes,
+                        void* workspace, size_t workspace_bytes, unsigned flags) {
+    if (int e = check_dims(B, T, C, H)) return e;
+    if (workspace == nullptr || workspace_bytes < rwkv_wkv5s_backward_workspace_bytes(B, T, C, H) || !aligned16(workspace))
+        return RWKV_ERR_WORKSPACE;
+    if (!fused_ok(T, C, H, flags) || saved == nullptr)
+        return rwkv_wkv5raw_backward(stream, B, T, C, H, r, k, v, decay, u, gy, gr, gk, gv, gw, gu, workspace, workspace_bytes, flags);
+    if (int e = check_ptrs({r, k, v, w_raw, decay, u, gy, gr, gk, gv, gw, gu})) return e;
+    if (saved_bytes < rwkv_wkv5s_saved_bytes(B, T, C, H) || !aligned16(saved)) return RWKV_ERR_WORKSPACE;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
+    char* wsb = static_cast<char*>(workspace);
+    const size_t n = round16(rwkv_wkv5_backward_workspace_bytes(B, T, C, H));
+    float* rdr = static_cast<float*>(workspace);
+    uint16_t* pw = reinterpret_cast<uint16_t*>(wsb + n);                                  // per-batch gw, then per-batch gu
+    uint16_t* pu = pw + static_cast<size_t>(B) * C;
+    int* flg = reinterpret_cast<int*>(wsb + round16(rwkv_wkv5raw_backward_workspace_bytes(B, T, C, H)));
+    int TB;
+    const int NB = scan_blocks(B, T, H, &TB, flags);
+    if (NB > 1) {
+        const size_t nq = static_cast<size_t>(B) * H * NB;
+        float* local = reinterpret_cast<float*>(reinterpret_cast<char*>(flg) + round16(static_cast<size_t>(B) * H * 8 * sizeof(int)));
+        float* ds32 = local + nq * 64 * 64;
+        float* logdec = ds32 + nq * 64 * 64;
+        float* gu32 = logdec + nq * 64;
+        float* gw32 = gu32 + static_cast<size_t>(NB) * B * C;
+        zero_words(st, flg, static_cast<size_t>(B) * H * 8);
+        if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w_raw, u, gy, gr, gk, gv, nullptr, pu, nullptr, static_cast<const float*>(saved), flg,
+                                          NB, TB, local, logdec, ds32, gu32, pw, gw32)) return e;
+    } else if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w_raw, u, gy, gr, gk, gv, nullptr, pu, nullptr, static_cast<const float*>(saved), flg,
+                                             1, 0, nullptr, nullptr, nullptr, nullptr, pw, nullptr)) return e;
+    // heads whose decay the mid-point factors cannot carry: the two sweeps redo them (their per-batch gw, gu rows included)
+    const float* ew = decay + C;
+    if (int e = launch_wkv6_bwd_a_chunk(st, W_HEAD, B, T, C, H, r, k, v, ew, u, nullptr, gy, gr, pu, rdr, flg)) return e;
+    if (int e = launch_wkv6_bwd_b_chunk(st, W_HEAD, B, T, C, H, r, k, v, ew, u, nullptr, gy, gk, gv, pw, nullptr, rdr, flg)) return e;
+    hipLaunchKernelGGL(bf16_batch_sum, dim3((C + 255) / 256), dim3(256), 0, st, B, C, pw, gw, pu, gu);
+    return launch_status();
+}
+
 // ---- the reference-signature entry points: default kernels, every pass
 int rwkv_wkv5_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16* r, const rwkv_bf16* k,
                       const rwkv_bf16* v, const float* eew, const rwkv_bf16* u, rwkv_bf16* y) {

@@ -90,6 +90,11 @@ struct ArgsG {
     float* blk_decay;              // [B*H][NB][64]
     float* gu32;                   // NB > 1: gu of this (batch, head, block) in fp32 (the blocks are added before rounding)
     bool first, above;             // this is block 0; there is a block above this one
+    // wkv5: w is one raw decay per channel, [H][64], and its gradient is summed over the tokens: a row per batch row in
+    // gwp (bf16 [B][C]) or, with NB > 1, per block and batch row in gw32 (fp32 [NB][B][C]); gw is not written
+    bool head_decay;
+    uint16_t* gwp;
+    float* gw32;
 };
 
 // state entering even chunk e of this (batch, head), in the layout of the SD waves: lane <-> key channel 16w + l16,
@@ -119,7 +124,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     const int wq = w & 3;
     const bool lower = w < 4;
     const uint16_t* __restrict__ pA = (lower ? a.r : a.k) + base + 8 * (lane & 7);                                  // r | k
-    const uint16_t* __restrict__ pB = (lower ? static_cast<const uint16_t*>(a.w) : a.v) + base + 8 * (lane & 7);   // w | v
+    const uint16_t* __restrict__ pB = (lower ? (a.head_decay ? static_cast<const uint16_t*>(a.w) + h * N : static_cast<const uint16_t*>(a.w) + base) : a.v + base) + 8 * (lane & 7);   // w | v
+    const uint32_t bmask = (lower && a.head_decay) ? 0u : ~0u;          // wkv5: the decay row of the head at every token
     const uint16_t* __restrict__ pC = a.gy + base + 8 * (lane & 7);
     uint16_t* __restrict__ pS1 = (lower ? a.gr : a.gk) + base + 8 * (lane & 7);
     uint16_t* __restrict__ pS2 = (lower ? a.gw : a.gv) + base + 8 * (lane & 7);
@@ -134,7 +140,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         const int t = c * L + 8 * wq + rq, tg = c * L + 4 * w + rg;
         const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C, og = static_cast<uint32_t>(tg < T ? tg : T - 1) * C;
         x.a = *reinterpret_cast<const u32x4*>(pA + o);
-        x.b = *reinterpret_cast<const u32x4*>(pB + o);
+        x.b = *reinterpret_cast<const u32x4*>(pB + (o & bmask));
         x.c = *reinterpret_cast<const u32x4*>(pC + og);    // (both halves of the wave ask for the same four rows)
     };
     // the rows of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v and gy in place
@@ -155,7 +161,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     Held hq[3] = {};
     bool any_exact = false, met_ok = true;
     float logdec[2] = {0.f, 0.f};          // LOCAL: log2 of the decay over the whole block
-    float carry[2] = {0.f, 0.f}, gu_acc[2] = {0.f, 0.f};
+    float carry[2] = {0.f, 0.f}, gu_acc[2] = {0.f, 0.f}, gw_acc[2] = {0.f, 0.f};
     // Only the last chunk of the sequence can be cut short (PARTIAL): its rows past T carry no input and no decay.
 
     auto prep = [&](const int c, Held& hd, auto PARTIAL) __attribute__((always_inline)) {
@@ -259,8 +265,12 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         }
         // without an initial state nothing has been accumulated before token 0: its decay has no effect at all
         if (a.gs == nullptr && a.first && c == 0 && tp == 0) { gw[0][0] = 0.f; gw[0][1] = 0.f; }
+        if (a.head_decay) {
+            gw_acc[0] += gw[0][0] + gw[1][0]; gw_acc[1] += gw[0][1] + gw[1][1];
+        } else {
 #pragma unroll
-        for (int e = 0; e < 2; ++e) S.out[2][tp + 16 * e][4 * w + jq] = pack_bf2(gw[e][0], gw[e][1]);
+            for (int e = 0; e < 2; ++e) S.out[2][tp + 16 * e][4 * w + jq] = pack_bf2(gw[e][0], gw[e][1]);
+        }
     };
     // rows 8 (w & 3) .. +7 of the results of chunk c: gv, which the E waves left in the last iteration, at once (they
     // wait for this before they write the next); the other three when all prep waves have finished their columns
@@ -275,7 +285,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         const u32x4 o2 = *reinterpret_cast<const u32x4*>(&S.out[2][row][4 * pc]);
         if (on && tg < T) {
             *reinterpret_cast<u32x4*>(pS1 + static_cast<uint32_t>(tg) * C) = o1;
-            if (lower) *reinterpret_cast<u32x4*>(pS2 + static_cast<uint32_t>(tg) * C) = o2;
+            if (lower && !a.head_decay) *reinterpret_cast<u32x4*>(pS2 + static_cast<uint32_t>(tg) * C) = o2;
         }
     };
 
@@ -342,6 +352,14 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         if (tp == 15) {
             if (a.gu32 != nullptr) *reinterpret_cast<float2*>(a.gu32 + ch0) = make_float2(gu_acc[0], gu_acc[1]);
             else *reinterpret_cast<uint32_t*>(a.gu + ch0) = pack_bf2(gu_acc[0], gu_acc[1]);
+        }
+        if (a.head_decay) {
+#pragma unroll
+            for (int z = 0; z < 2; ++z) gw_acc[z] = row_sum_to_last(gw_acc[z]);
+            if (tp == 15) {
+                if (a.gw32 != nullptr) *reinterpret_cast<float2*>(a.gw32 + ch0) = make_float2(gw_acc[0], gw_acc[1]);
+                else *reinterpret_cast<uint32_t*>(a.gwp + ch0) = pack_bf2(gw_acc[0], gw_acc[1]);
+            }
         }
     }
 }
@@ -710,6 +728,8 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG arg) {
     // gu: a row per batch row [B][C], or per block and batch row [NB][B][C] in fp32
     if (arg.gu32 != nullptr) a.gu32 = arg.gu32 + ((static_cast<size_t>(blk) * (gridDim.x / (arg.NB * arg.H)) + b) * arg.H + h) * N;
     else a.gu = arg.gu + bh * N;
+    if (arg.gw32 != nullptr) a.gw32 = arg.gw32 + ((static_cast<size_t>(blk) * (gridDim.x / (arg.NB * arg.H)) + b) * arg.H + h) * N;
+    else if (arg.gwp != nullptr) a.gwp = arg.gwp + bh * N;
     const int n = (a.T + L - 1) / L;
     // the quadrant t < 16 <= s of the tiles is never written and must read as zero
     for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTG) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
@@ -736,8 +756,9 @@ __global__ __launch_bounds__(256) void gu_block_sum(const int NB, const size_t n
 int launch_wkv6_bwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
                           const uint16_t* w, const uint16_t* u, const uint16_t* gy, uint16_t* gr, uint16_t* gk, uint16_t* gv,
                           uint16_t* gw, uint16_t* gu, uint16_t* gs, const float* saved, int* flags,
-                          int NB, int TB, float* blk_ds, float* blk_decay, float* ds32, float* gu32) {
+                          int NB, int TB, float* blk_ds, float* blk_decay, float* ds32, float* gu32, uint16_t* gwp, float* gw32) {
     ArgsG a{};
+    a.head_decay = gwp != nullptr; a.gwp = gwp;
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.gs = gs; a.saved = saved; a.flags = flags;
     a.NB = 1; a.TB = T;
@@ -749,9 +770,11 @@ int launch_wkv6_bwd_fused(hipStream_t st, int B, int T, int C, int H, const uint
     hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, true>), dim3(B * H * NB), dim3(NTG), 0, st, a);
     if (int e = launch_wkv6_scan_reverse(st, B * H, NB, blk_ds, blk_decay, ds32)) return e;
     a.blk_ds = nullptr; a.blk_decay = nullptr; a.ds32 = ds32; a.gu32 = gu32;
+    if (gwp != nullptr) a.gw32 = gw32;
     hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, false>), dim3(B * H * NB), dim3(NTG), 0, st, a);
     const size_t n = static_cast<size_t>(B) * C;
     hipLaunchKernelGGL(gu_block_sum, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, NB, n, gu32, gu);
+    if (gwp != nullptr) hipLaunchKernelGGL(gu_block_sum, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, NB, n, gw32, gwp);
     return launch_status();
 }
 

@@ -66,6 +66,7 @@ struct ArgsQ {
     const float* s32;              // [B*H][NB][64][64] or null
     float* blk_state;              // [B*H][NB][64][64]
     float* blk_decay;              // [B*H][NB][64]
+    bool head_decay;               // wkv5: w is one raw decay per channel, [H][64], the same at every token
 };
 
 // ---------------------------------------------------------------------------------------------------- P waves
@@ -82,7 +83,9 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
     const int wq = w & 3;
     const bool lower = w < 4;
     const uint16_t* __restrict__ pA = (lower ? a.r : a.k) + base + 8 * (lane & 7);      // r | k
-    const uint16_t* __restrict__ pB = (lower ? a.w : a.v) + base + 8 * (lane & 7);      // w | v
+    // wkv5: the decay row of the head stands in for every token's (the loads stay, they hit the cache)
+    const uint16_t* __restrict__ pB = (lower ? (a.head_decay ? a.w + h * N : a.w + base) : a.v + base) + 8 * (lane & 7);   // w | v
+    const uint32_t bmask = (lower && a.head_decay) ? 0u : ~0u;
     float uj[2];
     {
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + ch0);
@@ -96,7 +99,7 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
         const int t = c * L + 8 * wq + rq;
         const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C;
         x.a = *reinterpret_cast<const u32x4*>(pA + o);
-        x.b = *reinterpret_cast<const u32x4*>(pB + o);
+        x.b = *reinterpret_cast<const u32x4*>(pB + (o & bmask));
     };
     // the rows of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v in place
     auto stage_in = [&](const int c, const Raw& x, auto PARTIAL) __attribute__((always_inline)) {
@@ -463,8 +466,9 @@ __global__ __launch_bounds__(256) void wkv6_scan(const float* __restrict__ local
 
 int launch_wkv6_fwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
                           const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, float* saved, int* flags,
-                          int NB, int TB, float* blk_state, float* blk_decay, float* s32) {
+                          int NB, int TB, float* blk_state, float* blk_decay, float* s32, bool head_decay) {
     ArgsQ a{};
+    a.head_decay = head_decay;
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y; a.saved = saved; a.flags = flags;
     a.NB = 1; a.TB = T;
     if (NB <= 1) {

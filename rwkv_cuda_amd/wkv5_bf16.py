@@ -24,10 +24,20 @@ class WKV_5(torch.autograd.Function):
             # ew = -exp(w.float()), eew = exp(ew) (:63-64) are made by the library into `decay` = [eew | ew]
             decay = torch.empty(2 * C, device=dev, dtype=torch.float32)
             y = torch.empty((B, T, C), device=dev, dtype=torch.bfloat16)
+            lib = _lib.load()
+            nsaved = lib.rwkv_wkv5s_saved_bytes(B, T, C, H) if C == H * HEAD_SIZE else 0
+            if nsaved > 0:
+                # head size 64: one forward and one reverse sweep; the forward keeps the state entering every 64th token
+                saved = torch.empty(nsaved, device=dev, dtype=torch.uint8)
+                call("rwkv_wkv5s_forward", dev, B, T, C, H, r, k, v, w, u, y, decay, saved, nsaved, ctx.flags)
+                ctx.nsaved = nsaved
+                ctx.save_for_backward(r, k, v, decay, u, w, saved)
+                return y
             # heads of 128 channels run as four heads of 64 whose fp32 terms need scratch; every other size needs none
-            nbytes = _lib.load().rwkv_wkv5_forward_workspace_bytes(B, T, C, H)
+            nbytes = lib.rwkv_wkv5_forward_workspace_bytes(B, T, C, H)
             ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
             call("rwkv_wkv5raw_forward_ws", dev, B, T, C, H, r, k, v, w, u, y, decay, ws, nbytes, ctx.flags)
+            ctx.nsaved = 0
             ctx.save_for_backward(r, k, v, decay, u)
             return y
 
@@ -35,12 +45,18 @@ class WKV_5(torch.autograd.Function):
     def backward(ctx, gy):
         with torch.no_grad():
             B, T, C, H = ctx.B, ctx.T, ctx.C, ctx.H
-            r, k, v, decay, u = ctx.saved_tensors
+            r, k, v, decay, u = ctx.saved_tensors[:5]
             gy = gy.contiguous()
             dev = check_tensors((gy,), torch.bfloat16, ("gy",))
             new = lambda *shape: torch.empty(shape, device=dev, dtype=torch.bfloat16)
             gr, gk, gv = new(B, T, C), new(B, T, C), new(B, T, C)
             gw, gu = new(H, C // H), new(H, C // H)           # summed over the batch by the library (:86-87)
+            if ctx.nsaved > 0:
+                w, saved = ctx.saved_tensors[5:]
+                nbytes = _lib.load().rwkv_wkv5s_backward_workspace_bytes(B, T, C, H)
+                ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
+                call("rwkv_wkv5s_backward", dev, B, T, C, H, r, k, v, w, decay, u, gy, gr, gk, gv, gw, gu, saved, ctx.nsaved, ws, nbytes, ctx.flags)
+                return (None, None, None, None, gr, gk, gv, gw, gu)
             nbytes = _lib.load().rwkv_wkv5raw_backward_workspace_bytes(B, T, C, H)
             ws = torch.empty(nbytes, device=dev, dtype=torch.uint8)
             call("rwkv_wkv5raw_backward", dev, B, T, C, H, r, k, v, decay, u, gy, gr, gk, gv, gw, gu, ws, nbytes, ctx.flags)

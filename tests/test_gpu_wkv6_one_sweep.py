@@ -206,3 +206,38 @@ def test_one_sweep_rejects_bad_arguments(lib):
     args[10] = p(torch.empty((B, H, 64, 64), device=DEV, dtype=BF))                                                      # a state without its gradient
     assert lib.rwkv_wkv6f_backward_saved(*args, n, 0) == -2
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("B,T,H", [(2, 50, 2), (1, 700, 3), (3, 64, 1), (1, 4096, 2)])
+def test_wkv5_on_the_one_sweep_pair(lib, B, T, H):
+    """wkv5 at head size 64 through rwkv_wkv5s_forward / rwkv_wkv5s_backward: the raw decay of a channel stands in for every
+    token's, gw is summed over the tokens inside the kernel and over the batch after it ((1, 700, 3) and (1, 4096, 2) run
+    as blocks with a scan)."""
+    print(f"\nwkv5 one sweep B={B} T={T} H={H}", flush=True)
+    C = H * 64
+    r, k, v, w, u, gy = synth.wkv5_inputs(B, T, C, H, seed=340 + T)
+    ref = O.wkv5_grads(B, T, C, H, r, k, v, w, u, gy) if T < 2000 else None
+    if ref is None:
+        ref = list(O.wkv_grads_by_hand(B, T, C, H, r, k, v, w.reshape(1, 1, C).expand(B, T, C), u, gy, None, torch.float64))[:6]
+        ref[4] = ref[4].sum((0, 1)).reshape(H, 64)
+        ref[5] = ref[5].sum(0)
+    emu = O.emulate_wkv5_bf16(B, T, C, H, r, k, v, w, u, gy, hand=T >= 2000)
+    d = [x.to(DEV) for x in (r, k, v, w, u, gy)]
+    y = garbage((B, T, C), BF)
+    decay = torch.empty(2 * C, device=DEV, dtype=torch.float32)
+    nsv = lib.rwkv_wkv5s_saved_bytes(B, T, C, H)
+    saved = torch.empty(nsv, device=DEV, dtype=torch.uint8).fill_(0x7f)
+    call("rwkv_wkv5s_forward", DEV, B, T, C, H, *d[:5], y, decay, saved, nsv, 0)
+    gr, gk, gv = (garbage((B, T, C), BF) for _ in range(3))
+    gw, gu = garbage((H, 64), BF), garbage((H, 64), BF)
+    n = lib.rwkv_wkv5s_backward_workspace_bytes(B, T, C, H)
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8).fill_(0x7f)
+    call("rwkv_wkv5s_backward", DEV, B, T, C, H, d[0], d[1], d[2], d[3], decay, d[4], d[5], gr, gk, gv, gw, gu, saved, nsv, ws, n, 0)
+    torch.cuda.synchronize()
+    for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y, gr, gk, gv, gw, gu]):
+        assert torch.isfinite(g.float()).all(), name
+        assert_no_worse("wkv5 " + name, a, e, g)
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda t: t.data_ptr()
+    assert lib.rwkv_wkv5s_forward(st, B, T, C, H, p(d[0]), p(d[1]), p(d[2]), p(d[3]), p(d[4]), p(y), p(decay), p(saved), nsv - 1, 0) == -4
+    torch.cuda.synchronize()
