@@ -241,3 +241,31 @@ def test_wkv5_on_the_one_sweep_pair(lib, B, T, H):
     p = lambda t: t.data_ptr()
     assert lib.rwkv_wkv5s_forward(st, B, T, C, H, p(d[0]), p(d[1]), p(d[2]), p(d[3]), p(d[4]), p(y), p(decay), p(saved), nsv - 1, 0) == -4
     torch.cuda.synchronize()
+
+
+def test_random_shapes_states_and_decays(lib):
+    """Twenty seeded random cases of the wkv6 pair: batch 1..3, heads 1..3, T up to 900 (cut chunks, odd chunk counts, one to
+    seven blocks, a cut last block), with or without a state, a third of them with a stretch of strong decays somewhere
+    (inside a block, across a block boundary, in the cut chunk)."""
+    g = torch.Generator().manual_seed(2024)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    for case in range(20):
+        B, H, T = ri(1, 3), ri(1, 3), ri(1, 900)
+        state = bool(ri(0, 1))
+        C = H * 64
+        r, k, v, w, u, gy, s0 = synth.wkv6_inputs(B, T, C, H, seed=400 + case, state=state)
+        strong = case % 3 == 0 and T > 40
+        if strong:
+            t0 = ri(0, T - 20)
+            h = ri(0, H - 1)
+            w = w.float()
+            w[ri(0, B - 1), t0:t0 + 20, 64 * h:64 * h + ri(1, 64)] = 2.5
+            w = w.to(BF)
+        print(f"\ncase {case}: B={B} T={T} H={H} state={state} strong={strong}", flush=True)
+        ref = O.wkv6_grads(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+        emu = O.emulate_wkv6_bf16(B, T, C, H, r, k, v, w, u, gy, s0=s0)
+        got, handed_back = run_pair(lib, B, T, H, r, k, v, w, u, s0, gy, saved_fill=0x7f)
+        assert handed_back == (1 if strong else 0), (case, handed_back)
+        for name, a, e, x in zip(NAMES, ref, emu, got):
+            assert torch.isfinite(x.float()).all(), (case, name)
+            assert_no_worse(f"case {case} {name}", a, e, x)
