@@ -48,7 +48,7 @@ constexpr int TQ = 20;             // causal tiles [t][s], 32 bf16 and 16 bytes 
 
 struct alignas(16) SlotG {
     uint32_t RpH[L][PS], RpL[L][PS], KpH[L][PS], KpL[L][PS], V[L][PS], GY[L][PS];
-    float d1[N], d2[N], dec[N], l2[N];     // 2^{c_m}, 2^{c_L - c_m}, 2^{c_L}, cc_32 = c_L - c_m
+    float d1[N], d2[N], dec[N];            // 2^{c_m}, 2^{c_L - c_m}, 2^{c_L}
     float ruk[8][L];                        // sum of r u k over the 8 channels of each prep wave
 };
 struct alignas(16) TilesG {
@@ -66,7 +66,7 @@ struct alignas(16) SmemG {
 static_assert(sizeof(SmemG) <= 160 * 1024, "LDS");
 constexpr lds_t ROW_B = PS * 4, PLANE_B = L * ROW_B, TROW_B = TQ * 4, XROW_B = CS * 4, XZ_B = L * XROW_B;
 constexpr lds_t O_RPH = 0, O_RPL = PLANE_B, O_KPH = 2 * PLANE_B, O_KPL = 3 * PLANE_B, O_V = 4 * PLANE_B, O_GY = 5 * PLANE_B;
-constexpr lds_t O_D1 = 6 * PLANE_B, O_D2 = O_D1 + 4 * N, O_DEC = O_D2 + 4 * N, O_L2 = O_DEC + 4 * N, O_RUK = O_L2 + 4 * N;
+constexpr lds_t O_D1 = 6 * PLANE_B, O_D2 = O_D1 + 4 * N, O_DEC = O_D2 + 4 * N, O_RUK = O_DEC + 4 * N;
 constexpr lds_t SLOT_B = sizeof(SlotG), SLOT0 = offsetof(SmemG, slot);
 constexpr lds_t T_AH = 0, T_AL = L * TROW_B, T_BH = 2 * L * TROW_B, T_BL = 3 * L * TROW_B, TILE_B = sizeof(TilesG), TILE0 = offsetof(SmemG, tile);
 constexpr lds_t XZ0 = offsetof(SmemG, xz), VG0 = offsetof(SmemG, vg), PEX0 = offsetof(SmemG, pex), OUT0 = offsetof(SmemG, out);
@@ -157,7 +157,9 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         if (lane < 32) *reinterpret_cast<u32x4*>(&O.GY[rowg][4 * pc]) = liveg ? x.c : zero;
     };
     // what the finishing of a chunk needs from its preparation, three iterations earlier
-    struct Held { uint32_t r[2], k[2]; float cc[2][2]; };
+    // (r, k as loaded; ea = 2^{cc_t}, eb = 2^{-cc_{t+1}}, the factors of R' and K'; lf = d ln w / d w_raw, the decay gradient's factor:
+    //  keeping the factors costs twelve registers per chunk in flight and saves the finishing two exponentials per element)
+    struct Held { uint32_t r[2], k[2]; float ea[2][2], eb[2][2], lf[2][2]; };
     Held hq[3] = {};
     bool any_exact = false, met_ok = true;
     float logdec[2] = {0.f, 0.f};          // LOCAL: log2 of the decay over the whole block
@@ -167,7 +169,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     auto prep = [&](const int c, Held& hd, auto PARTIAL) __attribute__((always_inline)) {
         const int ch = 8 * w + 2 * jq, cd = 4 * w + jq;        // cd: dword column of the pair in a bf16 plane
         SlotG& O = S.slot[(c + 6) % 3];
-        float lam[2][2], rf[2][2], kf[2][2];
+        float lam[2][2], rf[2][2], kf[2][2], cc[2][2];
         uint32_t xr[2], xk[2], xw[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) { xr[e] = O.RpH[tp + 16 * e][cd]; xk[e] = O.KpH[tp + 16 * e][cd]; xw[e] = O.RpL[tp + 16 * e][cd]; }
@@ -185,8 +187,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         for (int z = 0; z < 2; ++z) {
             const float s0 = row_suffix_sum(lam[0][z]);        // sum over tokens tp..15
             const float p1 = row_prefix_sum(lam[1][z]);        // sum over tokens 16..16+tp
-            hd.cc[0][z] = -s0;
-            hd.cc[1][z] = p1 - lam[1][z];
+            cc[0][z] = -s0;
+            cc[1][z] = p1 - lam[1][z];
             l1[z] = bc<0>(s0);
             l2[z] = bc<15>(p1);
             if constexpr (LOCAL) logdec[z] += l1[z] + l2[z];
@@ -200,14 +202,19 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             *reinterpret_cast<float2*>(&O.d1[ch]) = make_float2(a0, a1);
             *reinterpret_cast<float2*>(&O.d2[ch]) = make_float2(b0, b1);
             *reinterpret_cast<float2*>(&O.dec[ch]) = make_float2(a0 * b0, a1 * b1);
-            *reinterpret_cast<float2*>(&O.l2[ch]) = make_float2(l2[0], l2[1]);
         }
         float ruk[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int t = tp + 16 * e;
-            const float rp0 = rf[e][0] * exp2_fast(hd.cc[e][0]), rp1 = rf[e][1] * exp2_fast(hd.cc[e][1]);
-            const float kp0 = kf[e][0] * exp2_fast(-(hd.cc[e][0] + lam[e][0])), kp1 = kf[e][1] * exp2_fast(-(hd.cc[e][1] + lam[e][1]));
+#pragma unroll
+            for (int z = 0; z < 2; ++z) {
+                hd.ea[e][z] = exp2_fast(cc[e][z]);
+                hd.eb[e][z] = exp2_fast(-(cc[e][z] + lam[e][z]));
+                hd.lf[e][z] = gw_factor(lam[e][z] * LN2);
+            }
+            const float rp0 = rf[e][0] * hd.ea[e][0], rp1 = rf[e][1] * hd.ea[e][1];
+            const float kp0 = kf[e][0] * hd.eb[e][0], kp1 = kf[e][1] * hd.eb[e][1];
             ruk[e] = fmaf(rf[e][0] * uj[0], kf[e][0], rf[e][1] * uj[1] * kf[e][1]);
             const HL r0 = hilo2(rp0, rp1), k0 = hilo2(kp0, kp1);
             O.RpH[t][cd] = r0.h; O.RpL[t][cd] = r0.l;
@@ -220,9 +227,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     // gr, gk, gw of chunk c from X, Z (left by the SD waves in the last iteration) and what prep kept
     auto finish = [&](const int c, const Held& hd, auto PARTIAL) __attribute__((always_inline)) {
         const int ch = 8 * w + 2 * jq;
-        const float2 e2 = *reinterpret_cast<const float2*>(&S.slot[c % 3].l2[ch]);
-        const float l2v[2] = {e2.x, e2.y};
-        float q[2][2], kdk[2][2], lam[2][2];
+        float q[2][2], kdk[2][2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const int t = tp + 16 * e, tg = c * L + t;
@@ -234,17 +239,13 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             float gr[2], gk[2];
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
-                const float cc = hd.cc[e][z];
-                const float nx = row_next(cc);
-                const float ccn = tp == 15 ? (e ? l2v[z] : 0.f) : nx;
-                const float drp = exp2_fast(cc) * X[z], dkp = exp2_fast(-ccn) * Z[z];
+                const float drp = hd.ea[e][z] * X[z], dkp = hd.eb[e][z] * Z[z];
                 const float uvg = uj[z] * vg;
                 gr[z] = fmaf(uvg, kf[z], drp);
                 gk[z] = fmaf(uvg, rf[z], dkp);
                 kdk[e][z] = kf[z] * dkp;
                 q[e][z] = fmaf(rf[z], drp, -kdk[e][z]);
                 gu_acc[z] = fmaf(rf[z] * kf[z], vg, gu_acc[z]);
-                lam[e][z] = gw_factor((ccn - cc) * LN2);
             }
             S.out[0][t][4 * w + jq] = pack_bf2(gr[0], gr[1]);
             S.out[1][t][4 * w + jq] = pack_bf2(gk[0], gk[1]);
@@ -254,8 +255,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         for (int z = 0; z < 2; ++z) {
             const float s1 = row_suffix_sum(q[1][z]) + carry[z];           // P_t of the second half
             const float s0 = row_suffix_sum(q[0][z]) + bc<0>(s1);
-            gw[1][z] = lam[1][z] * ((s1 - q[1][z]) - kdk[1][z]);          // lam (P_{t+1} - k dk')
-            gw[0][z] = lam[0][z] * ((s0 - q[0][z]) - kdk[0][z]);
+            gw[1][z] = hd.lf[1][z] * ((s1 - q[1][z]) - kdk[1][z]);        // lam (P_{t+1} - k dk')
+            gw[0][z] = hd.lf[0][z] * ((s0 - q[0][z]) - kdk[0][z]);
             carry[z] = bc<0>(s0);
         }
         if (!(c & 1)) {
@@ -301,8 +302,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     __builtin_amdgcn_sched_barrier(0);
     // DEPTH iterations per trip, no stage with loads or ring registers skipped: a way round one, or round the second half,
     // would be one more way into the next wait, on which the registers it waits for are the newest loads (the count then
-    // covers everything).  Below chunk 0 the stages run on rows that all count as dead, into planes nobody reads any more
-    // (c < 0: the slot is that of chunk c + 3, of which only l2 is still needed, by this wave, before it is written).
+    // covers everything).  Below chunk 0 the stages run on rows that all count as dead, into the planes of a slot that
+    // nobody reads any more (c < 0: the slot of chunk c + 3, whose products were done in the iteration before).
     for (int it0 = 0; it0 < nit; it0 += DEPTH)
         static_for<DEPTH>([&](auto Z) {
             constexpr int z = decltype(Z)::value;
