@@ -434,6 +434,34 @@ def make_wkv4(dev, B=4, T=512):
         return B * T / dt / 1e6, f"wkv4 fwd+bwd, grouped F.conv1d formulation, fp32, full B{B} T{T} C{C} ({dt:.1f} s)"
 
     cfg = {"workload": f"wkv4 fp32 fwd+bwd B{B} T{T} C{C}", "B": B, "T": T, "C": C, "algorithmic_bytes_per_token": 32 * C}
+    # The step is three launches of 4 to 17 us: at this size the gaps between launches are a third of it.  A caller who
+    # replays the step from a HIP graph does not pay them; the same step captured once and replayed, for comparison
+    # (no entry point allocates, synchronises or records a memset, so the calls capture as they are).
+    try:
+        step()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            step()                                         # warm the stream
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                for _ in range(10):
+                    step()
+        torch.cuda.current_stream().wait_stream(side)
+        for _ in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(30):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        cfg["ms_per_step_replayed_from_a_hip_graph"] = round(e0.elapsed_time(e1) / 300, 5)
+    except Exception as exc:                               # graphs are an extra: never let them fail the benchmark
+        cfg["ms_per_step_replayed_from_a_hip_graph"] = f"not measured: {type(exc).__name__}"
     return step, tok, kernels, cfg, cpu_baseline, 32 * C * tok
 
 
