@@ -269,3 +269,46 @@ def test_random_shapes_states_and_decays(lib):
         for name, a, e, x in zip(NAMES, ref, emu, got):
             assert torch.isfinite(x.float()).all(), (case, name)
             assert_no_worse(f"case {case} {name}", a, e, x)
+
+
+def test_the_pair_replays_from_a_hip_graph(lib):
+    """Forward and backward of a step captured once and replayed: no entry point allocates, synchronises or records a
+    memset (the flag words of the block form are cleared by a fill kernel), so replays give the eager results every time,
+    also with the program's own work and synchronisations between them.  A shape that runs as blocks with a scan."""
+    B, T, H = 1, 512, 4
+    C = H * 64
+    r, k, v, w, u, gy, s0 = (x.to(DEV) if x is not None else None for x in synth.wkv6_inputs(B, T, C, H, seed=350, state=True))
+    y = garbage((B, T, C), BF)
+    gr, gk, gv, gw = (garbage((B, T, C), BF) for _ in range(4))
+    gu, gs = garbage((H, 64), BF), garbage((B, H, 64, 64), BF)
+    nsv = lib.rwkv_wkv6f_saved_bytes(B, T, C, H)
+    saved = torch.empty(nsv, device=DEV, dtype=torch.uint8)
+    n = lib.rwkv_wkv6f_backward_saved_workspace_bytes(B, T, C, H)
+    ws = torch.empty(n, device=DEV, dtype=torch.uint8)
+
+    def step():
+        call("rwkv_wkv6f_forward", DEV, B, T, C, H, r, k, v, w, u, s0, y, saved, nsv, 0)
+        call("rwkv_wkv6f_backward_saved", DEV, B, T, C, H, r, k, v, w, u, s0, gy, gr, gk, gv, gw, gu, gs, saved, nsv, ws, n, 0)
+
+    step()
+    torch.cuda.synchronize()
+    eager = [x.clone() for x in (y, gr, gk, gv, gw, gu, gs)]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        step()
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(4):
+        for x in (y, gr, gk, gv, gw, gu, gs):
+            x.fill_(float("nan"))
+        saved.fill_(0x7f)
+        ws.fill_(0x7f)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(NAMES, eager, (y, gr, gk, gv, gw, gu, gs)):
+            assert torch.equal(a, b), (rep, name)
