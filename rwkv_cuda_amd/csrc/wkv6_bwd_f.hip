@@ -560,18 +560,18 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
         for (int tl = 0; tl < 4; ++tl) E[tl] = *reinterpret_cast<const f32x4*>(a.ds32 + b_e + 16 * tl);
     }
 
-    // causal tiles of chunk c (waves 0, 1, 2 -> quadrants (t, s) = (0,0) (1,0) (1,1)); accumulator rows are s, lanes t
-    auto tiles = [&](const int c) __attribute__((always_inline)) {
+    // causal tiles of chunk c, quadrants (t, s) = (0,0) (1,0) (1,1); accumulator rows are s, lanes t.  A = tril(K' R'^T) with
+    // the bonus on the diagonal, Bm = tril_strict(V GY^T) (its diagonal goes to vg).  Waves 0 and 2 form the A tile of a
+    // diagonal quadrant each, wave 1 both tiles of the full quadrant, wave 3 the Bm tiles of the two diagonal quadrants.
+    auto tile_a = [&](const int c, const int ta, const int tb) __attribute__((always_inline)) {
         const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
-        const int ta = (w == 0) ? 0 : 1, tb = (w == 2) ? 1 : 0;
         const lds_t ra = so + ta * 16 * ROW_B + b_nat, rb = so + tb * 16 * ROW_B + b_nat;
-        f32x4 a0 = zero4, a1 = zero4, bm = zero4;
-        bf16x8 kh[2], kl[2], rh[2], rl[2], vo[2], go[2];
+        f32x4 a0 = zero4, a1 = zero4;
+        bf16x8 kh[2], kl[2], rh[2], rl[2];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
             kh[ks] = ld_op(rb + O_KPH + 64 * ks); kl[ks] = ld_op(rb + O_KPL + 64 * ks);
             rh[ks] = ld_op(ra + O_RPH + 64 * ks); rl[ks] = ld_op(ra + O_RPL + 64 * ks);
-            vo[ks] = ld_op(rb + O_V + 64 * ks); go[ks] = ld_op(ra + O_GY + 64 * ks);
         }
         float d = 0.f;
         if (ta == tb) {
@@ -585,24 +585,48 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
             a0 = mfma(kh[ks], rh[ks], a0);
             a1 = mfma(kh[ks], rl[ks], a1);
             a1 = mfma(kl[ks], rh[ks], a1);
-            bm = mfma(vo[ks], go[ks], bm);
         }
         f32x4 am = a0 + a1;                                    // [v]: s = 16 tb + 4g + v, t = 16 ta + l16
         if (ta == tb) {
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int sl = 4 * g + v;
-                if (sl == l16) lds_st<float>(sb + VG0 + (c % 3) * (4 * L) + ta * 64 + b_l, bm[v]);
                 am[v] = (sl < l16) ? am[v] : (sl == l16 ? d : 0.f);
-                bm[v] = (sl < l16) ? bm[v] : 0.f;
             }
         }
-        const HL x0 = hilo2(am[0], am[1]), x1 = hilo2(am[2], am[3]), y0 = hilo2(bm[0], bm[1]), y1 = hilo2(bm[2], bm[3]);
+        const HL x0 = hilo2(am[0], am[1]), x1 = hilo2(am[2], am[3]);
         const lds_t tw = to + ta * 16 * TROW_B + tb * 32 + b_tw;
         lds_st<u32x2>(tw + T_AH, u32x2{x0.h, x1.h});
         lds_st<u32x2>(tw + T_AL, u32x2{x0.l, x1.l});
+    };
+    auto tile_b = [&](const int c, const int ta, const int tb) __attribute__((always_inline)) {
+        const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
+        const lds_t ra = so + ta * 16 * ROW_B + b_nat, rb = so + tb * 16 * ROW_B + b_nat;
+        f32x4 bm = zero4;
+        bf16x8 vo[2], go[2];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) { vo[ks] = ld_op(rb + O_V + 64 * ks); go[ks] = ld_op(ra + O_GY + 64 * ks); }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) bm = mfma(vo[ks], go[ks], bm);
+        if (ta == tb) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int sl = 4 * g + v;
+                if (sl == l16) lds_st<float>(sb + VG0 + (c % 3) * (4 * L) + ta * 64 + b_l, bm[v]);
+                bm[v] = (sl < l16) ? bm[v] : 0.f;
+            }
+        }
+        const HL y0 = hilo2(bm[0], bm[1]), y1 = hilo2(bm[2], bm[3]);
+        const lds_t tw = to + ta * 16 * TROW_B + tb * 32 + b_tw;
         lds_st<u32x2>(tw + T_BH, u32x2{y0.h, y1.h});
         lds_st<u32x2>(tw + T_BL, u32x2{y0.l, y1.l});
+    };
+    auto tiles = [&](const int c) __attribute__((always_inline)) {
+        if (w == 0) tile_a(c, 0, 0);
+        else if (w == 2) tile_a(c, 1, 1);
+        else if (w == 1) { tile_a(c, 1, 0); tile_b(c, 1, 0); }
+        else { tile_b(c, 0, 0); tile_b(c, 1, 1); }
     };
 
 #pragma unroll 1
@@ -699,7 +723,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                 });
         }
         __builtin_amdgcn_sched_barrier(0);
-        if (!LOCAL && it >= 1 && c - 1 >= 0 && w < 3) tiles(c - 1);
+        if (!LOCAL && it >= 1 && c - 1 >= 0) tiles(c - 1);
         __syncthreads();
     }
     if constexpr (LOCAL) {
@@ -740,7 +764,14 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG arg) {
     const int nit = (n + 2 + DEPTH) & ~(DEPTH - 1);        // iterations of the pipeline: n + 3, in whole trips of the prep loop
     if (wid < 8) role_prep<WMODE, LOCAL>(S, a, lane, wid, base, h, bh, n, nit);
     else if (wid < 12) role_sd<WMODE, LOCAL>(S, a, lane, w, bh, n, nit);
-    else role_e<WMODE, LOCAL>(S, a, lane, w, base, n, nit);
+    else {
+        // The dS waves carry the recurrence and issue little; left at the default priority they are the youngest waves of
+        // their SIMDs, get the issue slots that the others leave, and the whole workgroup waits for them at every barrier
+        // (measured: 5 % of their time at the barrier against 22..37 % for the others).  Ahead of the others they cost those
+        // almost nothing.  (Raising the X/Z waves as well starves the prep waves: slower.)
+        __builtin_amdgcn_s_setprio(2);
+        role_e<WMODE, LOCAL>(S, a, lane, w, base, n, nit);
+    }
 }
 
 // gu of a batch row from its blocks: out[b][c] = bf16(sum_blk part[blk][b][c])
