@@ -43,7 +43,10 @@ constexpr int NTG = 16 * 64;
 // times the rate of 72 (16-byte reads and the transposing reads do not care).
 constexpr int PS = 36;             // bf16 [token][channel] planes: 144 B
 constexpr int CS = 68;             // fp32 [token][channel] arrays: 272 B
-constexpr int DEPTH = 2;           // chunks that the prep waves load ahead (a power of two; four would cost the prep waves spills)
+constexpr int DEPTH = 2;           // chunks that the prep waves load ahead (four would cost the prep waves spills)
+constexpr int KEPT = 3;            // iterations between the preparation of a chunk and its finishing
+constexpr int TRIP = 6;            // iterations per trip of the prep loop: a multiple of both, so that the registers of the
+                                   // loads in flight and of what is kept for the finishing have fixed names (no copies)
 constexpr int TQ = 20;             // causal tiles [t][s], 32 bf16 and 16 bytes of padding: 80 B (16-byte reads of 16 rows hit all banks once)
 
 struct alignas(16) SlotG {
@@ -55,13 +58,14 @@ struct alignas(16) TilesG {
     uint32_t AH[L][TQ], AL[L][TQ], BH[L][TQ], BL[L][TQ];   // [t][s] bf16 hi / lo
 };
 struct alignas(16) SmemG {
+    // (the small arrays come first: below 64 KB their addresses are a lane offset plus a constant inside the instruction)
+    uint32_t out[4][L][PS];                 // gr, gk, gw, gv of one chunk, bf16 [token][channel], on their way to global memory
+    float vg[3][L];                         // v_t . gy_t of the chunks in flight
+    float pex[2][N];                        // P = sum_i dS S at the last two anchors
+    uint32_t met[4];                        // meeting counters: inputs staged, results written, gv taken
     SlotG slot[3];
     TilesG tile[2];
     float xz[2][2][L][CS];                  // [chunk parity][X, Z][token][key channel]: from the SD waves to the P waves
-    float vg[3][L];                         // v_t . gy_t of the chunks in flight
-    float pex[2][N];                        // P = sum_i dS S at the last two anchors
-    uint32_t out[4][L][PS];                 // gr, gk, gw, gv of one chunk, bf16 [token][channel], on their way to global memory
-    uint32_t met[3];                        // meeting counters: inputs staged, results written, gv taken
 };
 static_assert(sizeof(SmemG) <= 160 * 1024, "LDS");
 constexpr lds_t ROW_B = PS * 4, PLANE_B = L * ROW_B, TROW_B = TQ * 4, XROW_B = CS * 4, XZ_B = L * XROW_B;
@@ -98,12 +102,15 @@ struct ArgsG {
 };
 
 // state entering even chunk e of this (batch, head), in the layout of the SD waves: lane <-> key channel 16w + l16,
-// x[tile][v] <-> value channel 16 tile + 4g + v.  p: the state (wave-uniform), lo = (4 g) * 64 + 16 w + l16.
+// x[tile][v] <-> value channel 16 tile + 4g + v.  p: the state (wave-uniform), lo = byte offset of [4 g][16 w + l16].
+// (a uniform base per tile, one 32-bit lane offset and constants: sixteen loads without any address arithmetic)
 DEVINL void load_state(const float* __restrict__ p, const uint32_t lo, f32x4 (&x)[4]) {
 #pragma unroll
-    for (int tl = 0; tl < 4; ++tl)
+    for (int tl = 0; tl < 4; ++tl) {
+        const char* q = reinterpret_cast<const char*>(p + 16 * tl * N) + lo;
 #pragma unroll
-        for (int v = 0; v < 4; ++v) x[tl][v] = p[lo + (16 * tl + v) * N];
+        for (int v = 0; v < 4; ++v) x[tl][v] = *reinterpret_cast<const float*>(q + v * (4 * N));
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------- P waves
@@ -123,12 +130,26 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     int rq = lane >> 3, pc = lane & 7, rg = (lane & 31) >> 3;
     const int wq = w & 3;
     const bool lower = w < 4;
-    const uint16_t* __restrict__ pA = (lower ? a.r : a.k) + base + 8 * (lane & 7);                                  // r | k
-    const uint16_t* __restrict__ pB = (lower ? (a.head_decay ? static_cast<const uint16_t*>(a.w) + h * N : static_cast<const uint16_t*>(a.w) + base) : a.v + base) + 8 * (lane & 7);   // w | v
-    const uint32_t bmask = (lower && a.head_decay) ? 0u : ~0u;          // wkv5: the decay row of the head at every token
-    const uint16_t* __restrict__ pC = a.gy + base + 8 * (lane & 7);
-    uint16_t* __restrict__ pS1 = (lower ? a.gr : a.gk) + base + 8 * (lane & 7);
-    uint16_t* __restrict__ pS2 = (lower ? a.gw : a.gv) + base + 8 * (lane & 7);
+    // LDS is addressed as in the other roles: uniform bases plus a few per-lane byte offsets, constants in the instruction
+    const lds_t sb = lds_of(&S);
+    lds_t b_row = (8 * wq + rq) * ROW_B + 16 * pc;                    // [row 8 wq + rq][16 bytes pc] of a plane (staging, stores)
+    lds_t b_rowg = (4 * w + rg) * ROW_B + 16 * pc;                    // the same for the rows of gy
+    lds_t b_tp = tp * ROW_B + 4 * (4 * w + jq);                       // [token tp][channel pair 4 w + jq] of a plane
+    lds_t b_ch = 4 * (8 * w + 2 * jq);                                // channel 8 w + 2 jq of a per-channel array
+    lds_t b_l = 4 * tp;                                               // token tp of a per-token array
+    lds_t b_x = tp * XROW_B + 4 * (8 * w + 2 * jq);                   // [token tp][channel 8 w + 2 jq] of X / Z
+    // global addresses: a wave-uniform base and a 32-bit byte offset per lane (row of the chunk + 16 bytes of the row), to
+    // which a chunk adds a uniform term; rows past the end of the sequence are clamped to the last one
+    const char* __restrict__ pA = reinterpret_cast<const char*>((lower ? a.r : a.k) + base);                         // r | k
+    const char* __restrict__ pB = reinterpret_cast<const char*>(lower ? (a.head_decay ? static_cast<const uint16_t*>(a.w) + h * N : static_cast<const uint16_t*>(a.w) + base) : a.v + base);   // w | v
+    const uint32_t bmask = (lower && a.head_decay) ? 127u : ~0u;        // wkv5: the decay row of the head at every token
+    const char* __restrict__ pC = reinterpret_cast<const char*>(a.gy + base);
+    char* __restrict__ pS1 = reinterpret_cast<char*>((lower ? a.gr : a.gk) + base);
+    char* __restrict__ pS2 = reinterpret_cast<char*>((lower ? a.gw : a.gv) + base);
+    const uint32_t row_b = 2u * static_cast<uint32_t>(a.C);                                     // bytes from a token to the next
+    uint32_t offA = (8 * (w & 3) + (lane >> 3)) * row_b + 16 * (lane & 7);                      // rows 8 (w & 3) .. +7
+    uint32_t offG = (4 * w + ((lane & 31) >> 3)) * row_b + 16 * (lane & 7);                     // rows 4 w .. +3
+    const uint32_t lastA = static_cast<uint32_t>(a.T - 1) * row_b + 16 * (lane & 7);
     float uj[2];
     {
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + ch0);
@@ -137,24 +158,23 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     struct Raw { u32x4 a, b, c; };
     Raw ring[DEPTH];                       // DEPTH chunks ahead
     auto fetch = [&](const int c, Raw& x) __attribute__((always_inline)) {
-        const int t = c * L + 8 * wq + rq, tg = c * L + 4 * w + rg;
-        const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C, og = static_cast<uint32_t>(tg < T ? tg : T - 1) * C;
+        const uint32_t cb = static_cast<uint32_t>(c * L) * row_b;
+        const uint32_t o = min(cb + offA, lastA), og = min(cb + offG, lastA);
         x.a = *reinterpret_cast<const u32x4*>(pA + o);
         x.b = *reinterpret_cast<const u32x4*>(pB + (o & bmask));
         x.c = *reinterpret_cast<const u32x4*>(pC + og);    // (both halves of the wave ask for the same four rows)
     };
     // the rows of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v and gy in place
     auto stage_in = [&](const int c, const Raw& x, auto PARTIAL) __attribute__((always_inline)) {
-        SlotG& O = S.slot[(c + 6) % 3];
+        const lds_t so = uniform_base(sb + SLOT0 + ((c + 9) % 3) * SLOT_B);
         const int row = 8 * wq + rq, rowg = 4 * w + rg;
         const bool live = !decltype(PARTIAL)::value || (c >= 0 && c * L + row < T);
         const bool liveg = !decltype(PARTIAL)::value || (c >= 0 && c * L + rowg < T);
         const u32x4 zero = {0u, 0u, 0u, 0u};
-        uint32_t* da = lower ? &O.RpH[row][4 * pc] : &O.KpH[row][4 * pc];
-        uint32_t* db = lower ? &O.RpL[row][4 * pc] : &O.V[row][4 * pc];
-        *reinterpret_cast<u32x4*>(da) = live ? x.a : zero;
-        *reinterpret_cast<u32x4*>(db) = (live || lower) ? x.b : zero;    // w of a dead row is masked where the decay is formed
-        if (lane < 32) *reinterpret_cast<u32x4*>(&O.GY[rowg][4 * pc]) = liveg ? x.c : zero;
+        const lds_t da = so + (lower ? O_RPH : O_KPH) + b_row, db = so + (lower ? O_RPL : O_V) + b_row;
+        lds_st<u32x4>(da, live ? x.a : zero);
+        lds_st<u32x4>(db, (live || lower) ? x.b : zero);                 // w of a dead row is masked where the decay is formed
+        if (lane < 32) lds_st<u32x4>(so + O_GY + b_rowg, liveg ? x.c : zero);
     };
     // what the finishing of a chunk needs from its preparation, three iterations earlier
     // (r, k as loaded; ea = 2^{cc_t}, eb = 2^{-cc_{t+1}}, the factors of R' and K'; lf = d ln w / d w_raw, the decay gradient's factor:
@@ -167,12 +187,15 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     // Only the last chunk of the sequence can be cut short (PARTIAL): its rows past T carry no input and no decay.
 
     auto prep = [&](const int c, Held& hd, auto PARTIAL) __attribute__((always_inline)) {
-        const int ch = 8 * w + 2 * jq, cd = 4 * w + jq;        // cd: dword column of the pair in a bf16 plane
-        SlotG& O = S.slot[(c + 6) % 3];
+        const lds_t so = uniform_base(sb + SLOT0 + ((c + 9) % 3) * SLOT_B);
         float lam[2][2], rf[2][2], kf[2][2], cc[2][2];
         uint32_t xr[2], xk[2], xw[2];
 #pragma unroll
-        for (int e = 0; e < 2; ++e) { xr[e] = O.RpH[tp + 16 * e][cd]; xk[e] = O.KpH[tp + 16 * e][cd]; xw[e] = O.RpL[tp + 16 * e][cd]; }
+        for (int e = 0; e < 2; ++e) {
+            xr[e] = lds_ld<uint32_t>(so + O_RPH + e * 16 * ROW_B + b_tp);
+            xk[e] = lds_ld<uint32_t>(so + O_KPH + e * 16 * ROW_B + b_tp);
+            xw[e] = lds_ld<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp);
+        }
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const bool live = !decltype(PARTIAL)::value || (c >= 0 && c * L + tp + 16 * e < T);
@@ -199,14 +222,13 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         }
         if (tp == 0) {
             const float a0 = exp2_fast(l1[0]), a1 = exp2_fast(l1[1]), b0 = exp2_fast(l2[0]), b1 = exp2_fast(l2[1]);
-            *reinterpret_cast<float2*>(&O.d1[ch]) = make_float2(a0, a1);
-            *reinterpret_cast<float2*>(&O.d2[ch]) = make_float2(b0, b1);
-            *reinterpret_cast<float2*>(&O.dec[ch]) = make_float2(a0 * b0, a1 * b1);
+            lds_st<f32x2>(so + O_D1 + b_ch, f32x2{a0, a1});
+            lds_st<f32x2>(so + O_D2 + b_ch, f32x2{b0, b1});
+            lds_st<f32x2>(so + O_DEC + b_ch, f32x2{a0 * b0, a1 * b1});
         }
         float ruk[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const int t = tp + 16 * e;
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
                 hd.ea[e][z] = exp2_fast(cc[e][z]);
@@ -216,25 +238,24 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             const float rp0 = rf[e][0] * hd.ea[e][0], rp1 = rf[e][1] * hd.ea[e][1];
             const float kp0 = kf[e][0] * hd.eb[e][0], kp1 = kf[e][1] * hd.eb[e][1];
             ruk[e] = fmaf(rf[e][0] * uj[0], kf[e][0], rf[e][1] * uj[1] * kf[e][1]);
-            const HL r0 = hilo2(rp0, rp1), k0 = hilo2(kp0, kp1);
-            O.RpH[t][cd] = r0.h; O.RpL[t][cd] = r0.l;
-            O.KpH[t][cd] = k0.h; O.KpL[t][cd] = k0.l;
+            const HL r0 = hilo2k(rp0, rp1), k0 = hilo2k(kp0, kp1);
+            lds_st<uint32_t>(so + O_RPH + e * 16 * ROW_B + b_tp, r0.h); lds_st<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp, r0.l);
+            lds_st<uint32_t>(so + O_KPH + e * 16 * ROW_B + b_tp, k0.h); lds_st<uint32_t>(so + O_KPL + e * 16 * ROW_B + b_tp, k0.l);
         }
         allreduce2_rows(ruk[0], ruk[1]);                       // sums over the four channel pairs of this wave
-        if (jq == 0) { O.ruk[w][tp] = ruk[0]; O.ruk[w][tp + 16] = ruk[1]; }
+        if (jq == 0) { lds_st<float>(so + O_RUK + w * (4 * L) + b_l, ruk[0]); lds_st<float>(so + O_RUK + w * (4 * L) + 64 + b_l, ruk[1]); }
     };
 
     // gr, gk, gw of chunk c from X, Z (left by the SD waves in the last iteration) and what prep kept
     auto finish = [&](const int c, const Held& hd, auto PARTIAL) __attribute__((always_inline)) {
-        const int ch = 8 * w + 2 * jq;
+        const lds_t xo = uniform_base(sb + XZ0 + (c & 1) * 2 * XZ_B), vo = uniform_base(sb + VG0 + (c % 3) * (4 * L));
         float q[2][2], kdk[2][2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const int t = tp + 16 * e, tg = c * L + t;
-            const float2 x2 = *reinterpret_cast<const float2*>(&S.xz[c & 1][0][t][ch]);
-            const float2 z2 = *reinterpret_cast<const float2*>(&S.xz[c & 1][1][t][ch]);
+            const f32x2 x2 = lds_ld<f32x2>(xo + e * 16 * XROW_B + b_x);
+            const f32x2 z2 = lds_ld<f32x2>(xo + XZ_B + e * 16 * XROW_B + b_x);
             const float X[2] = {x2.x, x2.y}, Z[2] = {z2.x, z2.y};
-            const float vg = S.vg[c % 3][t];
+            const float vg = lds_ld<float>(vo + 64 * e + b_l);
             const float rf[2] = {bf_lo(hd.r[e]), bf_hi(hd.r[e])}, kf[2] = {bf_lo(hd.k[e]), bf_hi(hd.k[e])};
             float gr[2], gk[2];
 #pragma unroll
@@ -247,8 +268,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
                 q[e][z] = fmaf(rf[z], drp, -kdk[e][z]);
                 gu_acc[z] = fmaf(rf[z] * kf[z], vg, gu_acc[z]);
             }
-            S.out[0][t][4 * w + jq] = pack_bf2(gr[0], gr[1]);
-            S.out[1][t][4 * w + jq] = pack_bf2(gk[0], gk[1]);
+            lds_st<uint32_t>(sb + OUT0 + e * 16 * ROW_B + b_tp, pack_bf2(gr[0], gr[1]));
+            lds_st<uint32_t>(sb + OUT0 + PLANE_B + e * 16 * ROW_B + b_tp, pack_bf2(gk[0], gk[1]));
         }
         float gw[2][2];
 #pragma unroll
@@ -261,7 +282,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         }
         if (!(c & 1)) {
             // the chunk began at an anchor: from here on P counts from its exact value there
-            const float2 p2 = *reinterpret_cast<const float2*>(&S.pex[(c >> 1) & 1][ch]);
+            const f32x2 p2 = lds_ld<f32x2>(sb + PEX0 + ((c >> 1) & 1) * (4 * N) + b_ch);
             carry[0] = p2.x; carry[1] = p2.y;
         }
         // without an initial state nothing has been accumulated before token 0: its decay has no effect at all
@@ -270,23 +291,24 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             gw_acc[0] += gw[0][0] + gw[1][0]; gw_acc[1] += gw[0][1] + gw[1][1];
         } else {
 #pragma unroll
-            for (int e = 0; e < 2; ++e) S.out[2][tp + 16 * e][4 * w + jq] = pack_bf2(gw[e][0], gw[e][1]);
+            for (int e = 0; e < 2; ++e) lds_st<uint32_t>(sb + OUT0 + 2 * PLANE_B + e * 16 * ROW_B + b_tp, pack_bf2(gw[e][0], gw[e][1]));
         }
     };
     // rows 8 (w & 3) .. +7 of the results of chunk c: gv, which the E waves left in the last iteration, at once (they
     // wait for this before they write the next); the other three when all prep waves have finished their columns
     auto store_gv = [&](const int c, const bool on) __attribute__((always_inline)) {
         const int row = 8 * wq + rq, tg = c * L + row;
-        const u32x4 o = *reinterpret_cast<const u32x4*>(&S.out[3][row][4 * pc]);
-        if (on && !lower && tg < T) *reinterpret_cast<u32x4*>(pS2 + static_cast<uint32_t>(tg) * C) = o;
+        const u32x4 o = lds_ld<u32x4>(sb + OUT0 + 3 * PLANE_B + b_row);
+        if (on && !lower && tg < T) *reinterpret_cast<u32x4*>(pS2 + (static_cast<uint32_t>(c * L) * row_b + offA)) = o;
     };
     auto store_out = [&](const int c, const bool on) __attribute__((always_inline)) {
         const int row = 8 * wq + rq, tg = c * L + row;
-        const u32x4 o1 = *reinterpret_cast<const u32x4*>(&S.out[lower ? 0 : 1][row][4 * pc]);
-        const u32x4 o2 = *reinterpret_cast<const u32x4*>(&S.out[2][row][4 * pc]);
+        const u32x4 o1 = lds_ld<u32x4>(sb + OUT0 + (lower ? 0 : PLANE_B) + b_row);
+        const u32x4 o2 = lds_ld<u32x4>(sb + OUT0 + 2 * PLANE_B + b_row);
         if (on && tg < T) {
-            *reinterpret_cast<u32x4*>(pS1 + static_cast<uint32_t>(tg) * C) = o1;
-            if (lower && !a.head_decay) *reinterpret_cast<u32x4*>(pS2 + static_cast<uint32_t>(tg) * C) = o2;
+            const uint32_t ob = static_cast<uint32_t>(c * L) * row_b + offA;
+            *reinterpret_cast<u32x4*>(pS1 + ob) = o1;
+            if (lower && !a.head_decay) *reinterpret_cast<u32x4*>(pS2 + ob) = o2;
         }
     };
 
@@ -304,12 +326,13 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     // would be one more way into the next wait, on which the registers it waits for are the newest loads (the count then
     // covers everything).  Below chunk 0 the stages run on rows that all count as dead, into the planes of a slot that
     // nobody reads any more (c < 0: the slot of chunk c + 3, whose products were done in the iteration before).
-    for (int it0 = 0; it0 < nit; it0 += DEPTH)
-        static_for<DEPTH>([&](auto Z) {
-            constexpr int z = decltype(Z)::value;
-            const int it = it0 + z;
+    for (int it0 = 0; it0 < nit; it0 += TRIP)
+        static_for<TRIP>([&](auto Z) {
+            constexpr int z = decltype(Z)::value % DEPTH, zk = decltype(Z)::value % KEPT;
+            const int it = it0 + decltype(Z)::value;
             const int cp = n - 1 - it;
-            asm volatile("" : "+v"(jq), "+v"(tp), "+v"(rq), "+v"(pc), "+v"(rg));
+            asm volatile("" : "+v"(jq), "+v"(tp), "+v"(rq), "+v"(pc), "+v"(rg), "+v"(offA), "+v"(offG));
+            opaque(b_row); opaque(b_rowg); opaque(b_tp); opaque(b_ch); opaque(b_l); opaque(b_x);
             const bool fin = !LOCAL && it >= 3 && cp + 3 >= 0;      // chunk cp + 3 is finished and stored in this iteration
             if constexpr (!LOCAL) {
                 store_gv(fin ? cp + 3 : 0, fin);
@@ -323,16 +346,15 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             if constexpr (!LOCAL) {
                 if (it == 3 && a.above) {
                     // P at the end of the block, from the gradient state that enters from above and the saved state there
-                    const float2 p2 = *reinterpret_cast<const float2*>(&S.pex[(n >> 1) & 1][8 * w + 2 * jq]);
+                    const f32x2 p2 = lds_ld<f32x2>(sb + PEX0 + ((n >> 1) & 1) * (4 * N) + b_ch);
                     carry[0] = p2.x; carry[1] = p2.y;
                 }
-                if (fin) { if (cut && it == 3) finish(cp + 3, hq[2], part); else finish(cp + 3, hq[2], full); }
+                if (fin) { if (cut && it == 3) finish(cp + 3, hq[zk], part); else finish(cp + 3, hq[zk], full); }
                 meet_signal(&S.met[1], lane);
             }
             __builtin_amdgcn_sched_barrier(0);
-            hq[2] = hq[1]; hq[1] = hq[0];
             met_ok = meet_wait(&S.met[0], 8u * (it + 1)) && met_ok;        // all rows of chunk cp are staged
-            if ((cut && it == 0) || cp < 0) prep(cp, hq[0], part); else prep(cp, hq[0], full);
+            if ((cut && it == 0) || cp < 0) prep(cp, hq[zk], part); else prep(cp, hq[zk], full);
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (!LOCAL) {
                 met_ok = meet_wait(&S.met[1], 8u * (it + 1)) && met_ok;    // all columns of chunk cp + 3 are finished
@@ -378,7 +400,7 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     const lds_t sb = lds_of(&S);
     // per-lane address parts
-    uint32_t b_sv = 4 * g * N + j;                                              // [value channel 4 g][key channel j] of a saved state
+    uint32_t b_sv = 4 * (4 * g * N + j);                                        // [value channel 4 g][key channel j] of a saved state (bytes)
     lds_t b_acc = l16 * ROW_B + 8 * g;                                          // [token l16][channel 4 g] of a plane
     lds_t b_tr = ((8 * g + (l16 >> 2)) * PS + 2 * (l16 & 3)) * 4;               // transposing read of a plane, rows 8 g ..
     lds_t b_trt = ((8 * g + (l16 >> 2)) * TQ + 2 * (l16 & 3)) * 4;              // the same of a tile
@@ -392,11 +414,11 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
     // the batches apart): a wave then waits for LDS a few times per chunk instead of once per product.
     // X^T[j][t] = (S d1)^T GY^T + K'^T Bm^T for chunk c; S = Sa (even chunk) or one update of it (odd chunk)
     auto part_x = [&](const int c) __attribute__((always_inline)) {
-        const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B, xo = sb + XZ0 + (c & 1) * 2 * XZ_B + 64 * w;
+        const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B), to = uniform_base(sb + TILE0 + (c & 1) * TILE_B), xo = uniform_base(sb + XZ0 + (c & 1) * 2 * XZ_B + 64 * w);
         f32x4 Sc[4];
         if (c & 1) {
             // state entering the odd chunk: S dec + d2 V^T K' with the chunk below
-            const lds_t qo = sb + SLOT0 + ((c - 1) % 3) * SLOT_B;
+            const lds_t qo = uniform_base(sb + SLOT0 + ((c - 1) % 3) * SLOT_B);
             const float qdec = lds_ld<float>(qo + O_DEC + 64 * w + b_j), qd2 = lds_ld<float>(qo + O_D2 + 64 * w + b_j);
             const bf16x8 qh = ld_tr(qo + O_KPH + 32 * w + b_tr, ROW_B), ql = ld_tr(qo + O_KPL + 32 * w + b_tr, ROW_B);
             bf16x8 vop[4];
@@ -447,7 +469,7 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
     };
     // Z^T[j][s] = (dS d2)^T V^T + R'^T Bm, then dS <- dS dec + d1 GY^T R'
     auto part_z = [&](const int c) __attribute__((always_inline)) {
-        const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B, xo = sb + XZ0 + (c & 1) * 2 * XZ_B + XZ_B + 64 * w;
+        const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B), to = uniform_base(sb + TILE0 + (c & 1) * TILE_B), xo = uniform_base(sb + XZ0 + (c & 1) * 2 * XZ_B + XZ_B + 64 * w);
         const float d1 = lds_ld<float>(so + O_D1 + 64 * w + b_j), d2 = lds_ld<float>(so + O_D2 + 64 * w + b_j), dec = lds_ld<float>(so + O_DEC + 64 * w + b_j);
         bf16x8 vop[2][2];
 #pragma unroll
@@ -594,7 +616,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                 am[v] = (sl < l16) ? am[v] : (sl == l16 ? d : 0.f);
             }
         }
-        const HL x0 = hilo2(am[0], am[1]), x1 = hilo2(am[2], am[3]);
+        const HL x0 = hilo2k(am[0], am[1]), x1 = hilo2k(am[2], am[3]);
         const lds_t tw = to + ta * 16 * TROW_B + tb * 32 + b_tw;
         lds_st<u32x2>(tw + T_AH, u32x2{x0.h, x1.h});
         lds_st<u32x2>(tw + T_AL, u32x2{x0.l, x1.l});
@@ -617,7 +639,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                 bm[v] = (sl < l16) ? bm[v] : 0.f;
             }
         }
-        const HL y0 = hilo2(bm[0], bm[1]), y1 = hilo2(bm[2], bm[3]);
+        const HL y0 = hilo2k(bm[0], bm[1]), y1 = hilo2k(bm[2], bm[3]);
         const lds_t tw = to + ta * 16 * TROW_B + tb * 32 + b_tw;
         lds_st<u32x2>(tw + T_BH, u32x2{y0.h, y1.h});
         lds_st<u32x2>(tw + T_BL, u32x2{y0.l, y1.l});
@@ -667,7 +689,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                     p[v] = E[2 * ks][v]; q[v] = E[2 * ks + 1][v];
                     mul_bc<v>(p[v], dq[2 * ks]); mul_bc<v>(q[v], dq[2 * ks + 1]);
                 });
-                const HL x0 = hilo2(p[0], p[1]), x1 = hilo2(p[2], p[3]), x2 = hilo2(q[0], q[1]), x3 = hilo2(q[2], q[3]);
+                const HL x0 = hilo2k(p[0], p[1]), x1 = hilo2k(p[2], p[3]), x2 = hilo2k(q[0], q[1]), x3 = hilo2k(q[2], q[3]);
                 dh[ks] = as_op(x0.h, x1.h, x2.h, x3.h);
                 dl[ks] = as_op(x0.l, x1.l, x2.l, x3.l);
             }
@@ -761,7 +783,7 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG arg) {
     if (tid < 3) S.met[tid] = 0;
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
-    const int nit = (n + 2 + DEPTH) & ~(DEPTH - 1);        // iterations of the pipeline: n + 3, in whole trips of the prep loop
+    const int nit = (n + 3 + TRIP - 1) / TRIP * TRIP;      // iterations of the pipeline: n + 3, in whole trips of the prep loop
     if (wid < 8) role_prep<WMODE, LOCAL>(S, a, lane, wid, base, h, bh, n, nit);
     else if (wid < 12) role_sd<WMODE, LOCAL>(S, a, lane, w, bh, n, nit);
     else {

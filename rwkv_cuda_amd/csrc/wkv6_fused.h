@@ -16,6 +16,10 @@ template <class T> DEVINL T lds_ld(const lds_t a) { return *(const __attribute__
 template <class T> DEVINL void lds_st(const lds_t a, const T v) { *(__attribute__((address_space(3))) T*)(a) = v; }
 DEVINL lds_t lds_of(const void* p) { return static_cast<lds_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) char*)p)); }
 DEVINL void opaque(lds_t& x) { asm volatile("" : "+v"(x)); }
+// a wave-uniform base (a slot, a tile) behind an empty asm: left to itself the compiler merges "(c % 3) * size" of two
+// chunks into one induction variable plus constants, some of them negative, and a negative constant cannot ride in the
+// offset field of an LDS instruction: every such read then costs an add
+DEVINL lds_t uniform_base(lds_t x) { asm volatile("" : "+s"(x)); return x; }
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef v4s __attribute__((address_space(3))) * lds_v4s_ptr;
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -48,11 +52,20 @@ DEVINL float row_prefix_sum(float x) {
 DEVINL float row_next(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x101, 0xf, 0xf, true));
 }
+// hilo2 with the pair of hi parts behind an empty asm (otherwise the compiler converts the first element once more by
+// itself to get its rounded value back: one more instruction per pair)
+DEVINL HL hilo2k(float a, float b) {
+    HL r;
+    r.h = cvt2(a, b);
+    asm("" : "+v"(r.h));
+    r.l = cvt2(a - __uint_as_float(r.h << 16), b - __uint_as_float(r.h & 0xffff0000u));
+    return r;
+}
 DEVINL void split16(const f32x4 (&x)[4], const float s, bf16x8 (&h)[2], bf16x8 (&l)[2]) {
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-        const HL a = hilo2(x[2 * ks][0] * s, x[2 * ks][1] * s), b = hilo2(x[2 * ks][2] * s, x[2 * ks][3] * s);
-        const HL c = hilo2(x[2 * ks + 1][0] * s, x[2 * ks + 1][1] * s), d = hilo2(x[2 * ks + 1][2] * s, x[2 * ks + 1][3] * s);
+        const HL a = hilo2k(x[2 * ks][0] * s, x[2 * ks][1] * s), b = hilo2k(x[2 * ks][2] * s, x[2 * ks][3] * s);
+        const HL c = hilo2k(x[2 * ks + 1][0] * s, x[2 * ks + 1][1] * s), d = hilo2k(x[2 * ks + 1][2] * s, x[2 * ks + 1][3] * s);
         h[ks] = as_op(a.h, b.h, c.h, d.h);
         l[ks] = as_op(a.l, b.l, c.l, d.l);
     }

@@ -158,7 +158,7 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
             const float rp0 = rf[e][0] * exp2_fast(cc[e][0]), rp1 = rf[e][1] * exp2_fast(cc[e][1]);
             const float kp0 = kf[e][0] * exp2_fast(-(cc[e][0] + lam[e][0])), kp1 = kf[e][1] * exp2_fast(-(cc[e][1] + lam[e][1]));
             ruk[e] = fmaf(rf[e][0] * uj[0], kf[e][0], rf[e][1] * uj[1] * kf[e][1]);
-            const HL r0 = hilo2(rp0, rp1), k0 = hilo2(kp0, kp1);
+            const HL r0 = hilo2k(rp0, rp1), k0 = hilo2k(kp0, kp1);
             O.RpH[t][cd] = r0.h; O.RpL[t][cd] = r0.l;
             O.KpH[t][cd] = k0.h; O.KpL[t][cd] = k0.l;
         }
@@ -283,7 +283,7 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
                 p[v] = St[2 * ks][v]; q[v] = St[2 * ks + 1][v];
                 mul_bc<v>(p[v], dq[2 * ks]); mul_bc<v>(q[v], dq[2 * ks + 1]);
             });
-            const HL x0 = hilo2(p[0], p[1]), x1 = hilo2(p[2], p[3]), x2 = hilo2(q[0], q[1]), x3 = hilo2(q[2], q[3]);
+            const HL x0 = hilo2k(p[0], p[1]), x1 = hilo2k(p[2], p[3]), x2 = hilo2k(q[0], q[1]), x3 = hilo2k(q[2], q[3]);
             sh[ks] = as_op(x0.h, x1.h, x2.h, x3.h);
             sl[ks] = as_op(x0.l, x1.l, x2.l, x3.l);
         }
@@ -404,7 +404,7 @@ DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
                     am[v] = (sl < l16) ? am[v] : (sl == l16 ? d : 0.f);
                 }
             }
-            const HL x0 = hilo2(am[0], am[1]), x1 = hilo2(am[2], am[3]);
+            const HL x0 = hilo2k(am[0], am[1]), x1 = hilo2k(am[2], am[3]);
             const lds_t tw = to + ta * 16 * TROW_B + tb * 32 + b_tw;
             lds_st<u32x2>(tw + T_AH, u32x2{x0.h, x1.h});
             lds_st<u32x2>(tw + T_AL, u32x2{x0.l, x1.l});
