@@ -586,7 +586,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
     // the bonus on the diagonal, Bm = tril_strict(V GY^T) (its diagonal goes to vg).  Waves 0 and 2 form the A tile of a
     // diagonal quadrant each, wave 1 both tiles of the full quadrant, wave 3 the Bm tiles of the two diagonal quadrants.
     auto tile_a = [&](const int c, const int ta, const int tb) __attribute__((always_inline)) {
-        const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
+        const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B), to = uniform_base(sb + TILE0 + (c & 1) * TILE_B);
         const lds_t ra = so + ta * 16 * ROW_B + b_nat, rb = so + tb * 16 * ROW_B + b_nat;
         f32x4 a0 = zero4, a1 = zero4;
         bf16x8 kh[2], kl[2], rh[2], rl[2];
@@ -622,7 +622,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
         lds_st<u32x2>(tw + T_AL, u32x2{x0.l, x1.l});
     };
     auto tile_b = [&](const int c, const int ta, const int tb) __attribute__((always_inline)) {
-        const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
+        const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B), to = uniform_base(sb + TILE0 + (c & 1) * TILE_B);
         const lds_t ra = so + ta * 16 * ROW_B + b_nat, rb = so + tb * 16 * ROW_B + b_nat;
         f32x4 bm = zero4;
         bf16x8 vo[2], go[2];
@@ -656,7 +656,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
         const int c = n + 1 - it;
         opaque(b_acc); opaque(b_nat); opaque(b_tr); opaque(b_trt); opaque(b_tw); opaque(b_g); opaque(b_l);
         if (it >= 2 && c >= 0) {
-            const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
+            const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B), to = uniform_base(sb + TILE0 + (c & 1) * TILE_B);
             // Operands are fetched in batches, each issued as a whole before anything waits for it (the scheduling barriers
             // keep the batches apart): a wave then waits for LDS three times per chunk instead of once per product.
             // ------------------------------------------------------------ batch 1: d2 and K' (natural rows)

@@ -77,8 +77,10 @@ DEVINL void split16(const f32x4 (&x)[4], const float s, bf16x8 (&h)[2], bf16x8 (
 // The counter only grows: the k-th meeting of m waves is complete at k m.  The poll is bounded, so that a mistake in the
 // counting ends as a wrong result flagged to the caller and not as a hung GPU.
 DEVINL void meet_signal(uint32_t* cnt, const int lane) {
+    // (the add is written out: the compiler's own lowering of an atomic counts the active lanes first, five vector
+    //  instructions for a wave in which one lane is active by construction; nothing is returned, so no wait depends on it)
     asm volatile("" ::: "memory");
-    if (lane == 0) __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (lane == 0) asm volatile("ds_add_u32 %0, %1" : : "v"(lds_of(cnt)), "v"(1u) : "memory");
 }
 DEVINL bool meet_wait(uint32_t* cnt, const uint32_t target) {
     bool ok = true;
