@@ -39,11 +39,12 @@ struct alignas(16) TilesQ {
     uint32_t AH[L][AS], AL[L][AS];         // [t][s] bf16 hi / lo
 };
 struct alignas(16) SmemQ {
-    SlotQ slot[3];
-    TilesQ tile[2];
+    // (the small arrays come first: below 64 KB their addresses are a lane offset plus a constant inside the instruction)
     uint32_t yb[2][L][PS];                  // y of the last two chunks, bf16 [token][channel]
     float sst[N][SS];                       // the state entering an even chunk, on its way to global memory
-    uint32_t met;                           // meeting counter of the prep waves
+    uint32_t met[4];                        // [0]: meeting counter of the prep waves
+    SlotQ slot[3];
+    TilesQ tile[2];
 };
 constexpr lds_t ROW_B = PS * 4, PLANE_B = L * ROW_B, TROW_B = AS * 4;
 constexpr lds_t O_RPH = 0, O_RPL = PLANE_B, O_KPH = 2 * PLANE_B, O_KPL = 3 * PLANE_B, O_V = 4 * PLANE_B;
@@ -82,10 +83,21 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
     const int T = a.T, C = a.C;
     const int wq = w & 3;
     const bool lower = w < 4;
-    const uint16_t* __restrict__ pA = (lower ? a.r : a.k) + base + 8 * (lane & 7);      // r | k
+    // global addresses: a wave-uniform base and a 32-bit byte offset per lane (row of the chunk + 16 bytes of the row), to
+    // which a chunk adds a uniform term; rows past the end of the sequence are clamped to the last one
+    const char* __restrict__ pA = reinterpret_cast<const char*>((lower ? a.r : a.k) + base);      // r | k
     // wkv5: the decay row of the head stands in for every token's (the loads stay, they hit the cache)
-    const uint16_t* __restrict__ pB = (lower ? (a.head_decay ? a.w + h * N : a.w + base) : a.v + base) + 8 * (lane & 7);   // w | v
-    const uint32_t bmask = (lower && a.head_decay) ? 0u : ~0u;
+    const char* __restrict__ pB = reinterpret_cast<const char*>(lower ? (a.head_decay ? a.w + h * N : a.w + base) : a.v + base);   // w | v
+    const uint32_t bmask = (lower && a.head_decay) ? 127u : ~0u;
+    const uint32_t row_b = 2u * static_cast<uint32_t>(a.C);                                     // bytes from a token to the next
+    uint32_t offA = (8 * (w & 3) + (lane >> 3)) * row_b + 16 * (lane & 7);                      // rows 8 (w & 3) .. +7
+    const uint32_t lastA = static_cast<uint32_t>(a.T - 1) * row_b + 16 * (lane & 7);
+    // LDS: uniform bases plus a few per-lane byte offsets, constants in the instruction
+    const lds_t sb = lds_of(&S);
+    lds_t b_row = (8 * (w & 3) + (lane >> 3)) * ROW_B + 16 * (lane & 7);  // [row 8 wq + rq][16 bytes pc] of a plane (staging, stores)
+    lds_t b_tp = (lane & 15) * ROW_B + 4 * (4 * w + (lane >> 4));         // [token tp][channel pair 4 w + jq] of a plane
+    lds_t b_ch = 4 * (8 * w + 2 * (lane >> 4));                           // channel 8 w + 2 jq of a per-channel array
+    lds_t b_l = 4 * (lane & 15);                                          // token tp of a per-token array
     float uj[2];
     {
         const uint32_t x = *reinterpret_cast<const uint32_t*>(a.u + h * N + ch0);
@@ -96,32 +108,32 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
     // two to three microseconds under load, and a chunk is to take little more than one.
     Raw ring[DEPTH];                       // DEPTH chunks ahead
     auto fetch = [&](const int c, Raw& x) __attribute__((always_inline)) {
-        const int t = c * L + 8 * wq + rq;
-        const uint32_t o = static_cast<uint32_t>(t < T ? t : T - 1) * C;
+        const uint32_t o = min(static_cast<uint32_t>(c * L) * row_b + offA, lastA);
         x.a = *reinterpret_cast<const u32x4*>(pA + o);
         x.b = *reinterpret_cast<const u32x4*>(pB + (o & bmask));
     };
     // the rows of chunk c into the slot: r, k, w where the R' hi, K' hi, R' lo planes will be (staging), v in place
     auto stage_in = [&](const int c, const Raw& x, auto PARTIAL) __attribute__((always_inline)) {
-        SlotQ& O = S.slot[c % 3];
+        const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B);
         const int row = 8 * wq + rq;
         const bool live = !decltype(PARTIAL)::value || c * L + row < T;
         const u32x4 zero = {0u, 0u, 0u, 0u};
-        uint32_t* da = lower ? &O.RpH[row][4 * pc] : &O.KpH[row][4 * pc];
-        uint32_t* db = lower ? &O.RpL[row][4 * pc] : &O.V[row][4 * pc];
-        *reinterpret_cast<u32x4*>(da) = live ? x.a : zero;
-        *reinterpret_cast<u32x4*>(db) = (live || lower) ? x.b : zero;    // w of a dead row is masked where the decay is formed
-        meet_signal(&S.met, lane);
+        lds_st<u32x4>(so + (lower ? O_RPH : O_KPH) + b_row, live ? x.a : zero);
+        lds_st<u32x4>(so + (lower ? O_RPL : O_V) + b_row, (live || lower) ? x.b : zero);    // w of a dead row is masked where the decay is formed
+        meet_signal(&S.met[0], lane);
     };
     bool any_exact = false, met_ok = true;
     float logdec[2] = {0.f, 0.f};          // LOCAL: log2 of the decay over the whole block
     auto prep = [&](const int c, auto PARTIAL) __attribute__((always_inline)) {
-        const int ch = 8 * w + 2 * jq, cd = 4 * w + jq;        // cd: dword column of the pair in a bf16 plane
-        SlotQ& O = S.slot[c % 3];
+        const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B);
         float lam[2][2], rf[2][2], kf[2][2], cc[2][2];
         uint32_t xr[2], xk[2], xw[2];
 #pragma unroll
-        for (int e = 0; e < 2; ++e) { xr[e] = O.RpH[tp + 16 * e][cd]; xk[e] = O.KpH[tp + 16 * e][cd]; xw[e] = O.RpL[tp + 16 * e][cd]; }
+        for (int e = 0; e < 2; ++e) {
+            xr[e] = lds_ld<uint32_t>(so + O_RPH + e * 16 * ROW_B + b_tp);
+            xk[e] = lds_ld<uint32_t>(so + O_KPH + e * 16 * ROW_B + b_tp);
+            xw[e] = lds_ld<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp);
+        }
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const bool live = !decltype(PARTIAL)::value || c * L + tp + 16 * e < T;
@@ -147,33 +159,32 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
         }
         if (tp == 0) {
             const float a0 = exp2_fast(l1[0]), a1 = exp2_fast(l1[1]), b0 = exp2_fast(l2[0]), b1 = exp2_fast(l2[1]);
-            *reinterpret_cast<float2*>(&O.d1[ch]) = make_float2(a0, a1);
-            *reinterpret_cast<float2*>(&O.d2[ch]) = make_float2(b0, b1);
-            *reinterpret_cast<float2*>(&O.dec[ch]) = make_float2(a0 * b0, a1 * b1);
+            lds_st<f32x2>(so + O_D1 + b_ch, f32x2{a0, a1});
+            lds_st<f32x2>(so + O_D2 + b_ch, f32x2{b0, b1});
+            lds_st<f32x2>(so + O_DEC + b_ch, f32x2{a0 * b0, a1 * b1});
         }
         float ruk[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const int t = tp + 16 * e;
             const float rp0 = rf[e][0] * exp2_fast(cc[e][0]), rp1 = rf[e][1] * exp2_fast(cc[e][1]);
             const float kp0 = kf[e][0] * exp2_fast(-(cc[e][0] + lam[e][0])), kp1 = kf[e][1] * exp2_fast(-(cc[e][1] + lam[e][1]));
             ruk[e] = fmaf(rf[e][0] * uj[0], kf[e][0], rf[e][1] * uj[1] * kf[e][1]);
             const HL r0 = hilo2k(rp0, rp1), k0 = hilo2k(kp0, kp1);
-            O.RpH[t][cd] = r0.h; O.RpL[t][cd] = r0.l;
-            O.KpH[t][cd] = k0.h; O.KpL[t][cd] = k0.l;
+            lds_st<uint32_t>(so + O_RPH + e * 16 * ROW_B + b_tp, r0.h); lds_st<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp, r0.l);
+            lds_st<uint32_t>(so + O_KPH + e * 16 * ROW_B + b_tp, k0.h); lds_st<uint32_t>(so + O_KPL + e * 16 * ROW_B + b_tp, k0.l);
         }
         allreduce2_rows(ruk[0], ruk[1]);                       // sums over the four channel pairs of this wave
-        if (jq == 0) { O.ruk[w][tp] = ruk[0]; O.ruk[w][tp + 16] = ruk[1]; }
+        if (jq == 0) { lds_st<float>(so + O_RUK + w * (4 * L) + b_l, ruk[0]); lds_st<float>(so + O_RUK + w * (4 * L) + 64 + b_l, ruk[1]); }
     };
     // The y rows of chunk c, left in LDS by the S waves in the last iteration: waves 0..3 store eight rows each, eight
     // lanes per 128-byte row, so that the memory system sees whole lines and not the 16-byte pieces of the loads.
     // (A store on every path, masked per lane, so that the waits for the prefetched inputs count the same on all of them.)
-    uint16_t* __restrict__ pY = a.y + base + 8 * (lane & 7);
+    char* __restrict__ pY = reinterpret_cast<char*>(a.y + base);
     auto store_y = [&](const int c, const bool on) __attribute__((always_inline)) {
         const int row = 8 * wq + rq;
-        const u32x4 o = *reinterpret_cast<const u32x4*>(&S.yb[c & 1][row][4 * pc]);
+        const u32x4 o = lds_ld<u32x4>(sb + YB0 + (c & 1) * PLANE_B + b_row);
         const int tg = c * L + row;
-        if (on && lower && tg < T) *reinterpret_cast<u32x4*>(pY + static_cast<uint32_t>(tg) * C) = o;
+        if (on && lower && tg < T) *reinterpret_cast<u32x4*>(pY + (static_cast<uint32_t>(c * L) * row_b + offA)) = o;
     };
 
     const std::true_type part{};           // only the last chunk can be cut short
@@ -192,14 +203,15 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
         static_for<DEPTH>([&](auto Z) {
             constexpr int z = decltype(Z)::value;
             const int it = it0 + z;
-            asm volatile("" : "+v"(jq), "+v"(tp), "+v"(rq), "+v"(pc));
+            asm volatile("" : "+v"(jq), "+v"(tp), "+v"(rq), "+v"(pc), "+v"(offA));
+            opaque(b_row); opaque(b_tp); opaque(b_ch); opaque(b_l);
             if (it >= n - 1) stage_in(it, ring[z], part); else stage_in(it, ring[z], full);
             __builtin_amdgcn_sched_barrier(0);
             fetch(it + DEPTH < n ? it + DEPTH : n - 1, ring[z]);
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (!LOCAL) store_y(it >= 3 ? it - 3 : 0, it >= 3);
             __builtin_amdgcn_sched_barrier(0);
-            met_ok = meet_wait(&S.met, 8u * (it + 1)) && met_ok;      // all eight waves have staged their rows of chunk it
+            met_ok = meet_wait(&S.met[0], 8u * (it + 1)) && met_ok;      // all eight waves have staged their rows of chunk it
             if (it >= n - 1) prep(it, part); else prep(it, full);
             __syncthreads();
         });
@@ -243,7 +255,7 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
 #pragma unroll 1
     for (int c = 0; c < n; ++c) {
         opaque(b_acc); opaque(b_tr); opaque(b_natt); opaque(b_g); opaque(b_ss);
-        const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
+        const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B), to = uniform_base(sb + TILE0 + (c & 1) * TILE_B);
         if (!LOCAL && !(c & 1)) {
             // The state entering an even chunk goes to LDS and from there, in the next iteration, to global memory through
             // a wave that has nothing else to do: every workgroup writes its 16 KB at about the same moment, the memory
@@ -374,7 +386,7 @@ DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
             }
         }
         if (!LOCAL && c < n && w < 3) {
-            const lds_t so = sb + SLOT0 + (c % 3) * SLOT_B, to = sb + TILE0 + (c & 1) * TILE_B;
+            const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B), to = uniform_base(sb + TILE0 + (c & 1) * TILE_B);
             const lds_t ra = so + ta * 16 * ROW_B + b_nat, rb = so + tb * 16 * ROW_B + b_nat;
             bf16x8 kh[2], kl[2], rh[2], rl[2];
 #pragma unroll
@@ -432,7 +444,7 @@ __global__ __launch_bounds__(NTQ) void wkv6_fwd_fused(const ArgsQ arg) {
     const int n = (a.T + L - 1) / L;
     // the quadrant t < 16 <= s of the tiles is never written and must read as zero
     for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTQ) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
-    if (tid == 0) S.met = 0;
+    if (tid == 0) S.met[0] = 0;
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
     const int nit = (n + 2 + DEPTH) & ~(DEPTH - 1);        // iterations of the pipeline: n + 3, in whole trips of the prep loop
