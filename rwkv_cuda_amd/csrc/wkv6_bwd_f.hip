@@ -144,8 +144,6 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     const char* __restrict__ pB = reinterpret_cast<const char*>(lower ? (a.head_decay ? static_cast<const uint16_t*>(a.w) + h * N : static_cast<const uint16_t*>(a.w) + base) : a.v + base);   // w | v
     const uint32_t bmask = (lower && a.head_decay) ? 127u : ~0u;        // wkv5: the decay row of the head at every token
     const char* __restrict__ pC = reinterpret_cast<const char*>(a.gy + base);
-    char* __restrict__ pS1 = reinterpret_cast<char*>((lower ? a.gr : a.gk) + base);
-    char* __restrict__ pS2 = reinterpret_cast<char*>((lower ? a.gw : a.gv) + base);
     const uint32_t row_b = 2u * static_cast<uint32_t>(a.C);                                     // bytes from a token to the next
     uint32_t offA = (8 * (w & 3) + (lane >> 3)) * row_b + 16 * (lane & 7);                      // rows 8 (w & 3) .. +7
     uint32_t offG = (4 * w + ((lane & 31) >> 3)) * row_b + 16 * (lane & 7);                     // rows 4 w .. +3
@@ -227,6 +225,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             lds_st<f32x2>(so + O_DEC + b_ch, f32x2{a0 * b0, a1 * b1});
         }
         float ruk[2];
+        HL r0[2], k0[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
 #pragma unroll
@@ -238,10 +237,13 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             const float rp0 = rf[e][0] * hd.ea[e][0], rp1 = rf[e][1] * hd.ea[e][1];
             const float kp0 = kf[e][0] * hd.eb[e][0], kp1 = kf[e][1] * hd.eb[e][1];
             ruk[e] = fmaf(rf[e][0] * uj[0], kf[e][0], rf[e][1] * uj[1] * kf[e][1]);
-            const HL r0 = hilo2k(rp0, rp1), k0 = hilo2k(kp0, kp1);
-            lds_st<uint32_t>(so + O_RPH + e * 16 * ROW_B + b_tp, r0.h); lds_st<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp, r0.l);
-            lds_st<uint32_t>(so + O_KPH + e * 16 * ROW_B + b_tp, k0.h); lds_st<uint32_t>(so + O_KPL + e * 16 * ROW_B + b_tp, k0.l);
+            r0[e] = hilo2k(rp0, rp1); k0[e] = hilo2k(kp0, kp1);
         }
+        // (the stores side by side, with no load between them: the compiler then pairs them, two planes or two rows an instruction)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) { lds_st<uint32_t>(so + O_RPH + e * 16 * ROW_B + b_tp, r0[e].h); lds_st<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp, r0[e].l); }
+#pragma unroll
+        for (int e = 0; e < 2; ++e) { lds_st<uint32_t>(so + O_KPH + e * 16 * ROW_B + b_tp, k0[e].h); lds_st<uint32_t>(so + O_KPL + e * 16 * ROW_B + b_tp, k0[e].l); }
         allreduce2_rows(ruk[0], ruk[1]);                       // sums over the four channel pairs of this wave
         if (jq == 0) { lds_st<float>(so + O_RUK + w * (4 * L) + b_l, ruk[0]); lds_st<float>(so + O_RUK + w * (4 * L) + 64 + b_l, ruk[1]); }
     };
@@ -250,6 +252,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     auto finish = [&](const int c, const Held& hd, auto PARTIAL) __attribute__((always_inline)) {
         const lds_t xo = uniform_base(sb + XZ0 + (c & 1) * 2 * XZ_B), vo = uniform_base(sb + VG0 + (c % 3) * (4 * L));
         float q[2][2], kdk[2][2];
+        uint32_t ogr[2], ogk[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const f32x2 x2 = lds_ld<f32x2>(xo + e * 16 * XROW_B + b_x);
@@ -268,9 +271,10 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
                 q[e][z] = fmaf(rf[z], drp, -kdk[e][z]);
                 gu_acc[z] = fmaf(rf[z] * kf[z], vg, gu_acc[z]);
             }
-            lds_st<uint32_t>(sb + OUT0 + e * 16 * ROW_B + b_tp, pack_bf2(gr[0], gr[1]));
-            lds_st<uint32_t>(sb + OUT0 + PLANE_B + e * 16 * ROW_B + b_tp, pack_bf2(gk[0], gk[1]));
+            ogr[e] = pack_bf2(gr[0], gr[1]); ogk[e] = pack_bf2(gk[0], gk[1]);
         }
+#pragma unroll
+        for (int e = 0; e < 2; ++e) { lds_st<uint32_t>(sb + OUT0 + e * 16 * ROW_B + b_tp, ogr[e]); lds_st<uint32_t>(sb + OUT0 + PLANE_B + e * 16 * ROW_B + b_tp, ogk[e]); }
         float gw[2][2];
 #pragma unroll
         for (int z = 0; z < 2; ++z) {
@@ -294,24 +298,6 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             for (int e = 0; e < 2; ++e) lds_st<uint32_t>(sb + OUT0 + 2 * PLANE_B + e * 16 * ROW_B + b_tp, pack_bf2(gw[e][0], gw[e][1]));
         }
     };
-    // rows 8 (w & 3) .. +7 of the results of chunk c: gv, which the E waves left in the last iteration, at once (they
-    // wait for this before they write the next); the other three when all prep waves have finished their columns
-    auto store_gv = [&](const int c, const bool on) __attribute__((always_inline)) {
-        const int row = 8 * wq + rq, tg = c * L + row;
-        const u32x4 o = lds_ld<u32x4>(sb + OUT0 + 3 * PLANE_B + b_row);
-        if (on && !lower && tg < T) *reinterpret_cast<u32x4*>(pS2 + (static_cast<uint32_t>(c * L) * row_b + offA)) = o;
-    };
-    auto store_out = [&](const int c, const bool on) __attribute__((always_inline)) {
-        const int row = 8 * wq + rq, tg = c * L + row;
-        const u32x4 o1 = lds_ld<u32x4>(sb + OUT0 + (lower ? 0 : PLANE_B) + b_row);
-        const u32x4 o2 = lds_ld<u32x4>(sb + OUT0 + 2 * PLANE_B + b_row);
-        if (on && tg < T) {
-            const uint32_t ob = static_cast<uint32_t>(c * L) * row_b + offA;
-            *reinterpret_cast<u32x4*>(pS1 + ob) = o1;
-            if (lower && !a.head_decay) *reinterpret_cast<u32x4*>(pS2 + ob) = o2;
-        }
-    };
-
     const bool cut = (T % L) != 0;         // the last chunk is cut short
     const std::true_type part{};
     const std::false_type full{};
@@ -333,11 +319,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             const int cp = n - 1 - it;
             asm volatile("" : "+v"(jq), "+v"(tp), "+v"(rq), "+v"(pc), "+v"(rg), "+v"(offA), "+v"(offG));
             opaque(b_row); opaque(b_rowg); opaque(b_tp); opaque(b_ch); opaque(b_l); opaque(b_x);
-            const bool fin = !LOCAL && it >= 3 && cp + 3 >= 0;      // chunk cp + 3 is finished and stored in this iteration
-            if constexpr (!LOCAL) {
-                store_gv(fin ? cp + 3 : 0, fin);
-                meet_signal(&S.met[2], lane);
-            }
+            const bool fin = !LOCAL && it >= 3 && cp + 3 >= 0;      // chunk cp + 3 is finished in this iteration
             if ((cut && it == 0) || cp < 0) stage_in(cp, ring[z], part); else stage_in(cp, ring[z], full);
             meet_signal(&S.met[0], lane);
             __builtin_amdgcn_sched_barrier(0);
@@ -355,16 +337,12 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             __builtin_amdgcn_sched_barrier(0);
             met_ok = meet_wait(&S.met[0], 8u * (it + 1)) && met_ok;        // all rows of chunk cp are staged
             if ((cut && it == 0) || cp < 0) prep(cp, hq[zk], part); else prep(cp, hq[zk], full);
-            __builtin_amdgcn_sched_barrier(0);
-            if constexpr (!LOCAL) {
-                met_ok = meet_wait(&S.met[1], 8u * (it + 1)) && met_ok;    // all columns of chunk cp + 3 are finished
-                store_out(fin ? cp + 3 : 0, fin);
-            }
             __syncthreads();
         });
     // (a meeting that never completed, which the counting excludes, would leave this head to the two-sweep kernels)
     // (with several blocks per head the words are cleared by the caller and only ever set)
-    const bool flag = any_exact || !met_ok;
+    // (S.met[3]: a meeting of the E waves that never completed; written before the last barrier)
+    const bool flag = any_exact || !met_ok || S.met[3] != 0;
     if (lane == 0 && (a.NB == 1 || flag)) a.flags[bh * 8 + w] = flag ? 1 : 0;
     if constexpr (LOCAL) {
         if (tp == 0) *reinterpret_cast<float2*>(a.blk_decay + ch0) = make_float2(logdec[0], logdec[1]);
@@ -575,6 +553,17 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
     lds_t b_tw = l16 * TROW_B + 8 * g;                                          // [row l16][position 4 g] of a tile
     lds_t b_g = 16 * g + 4 * (l16 & 3);                                          // channel 4 g + (l16 & 3) of a per-channel array
     lds_t b_l = 4 * l16;
+    // The E waves also carry the results to global memory, in whole 128-byte rows (eight lanes a row, rows 8 w .. +7 of each
+    // of the four tensors per wave): the prep waves leave gr, gk, gw of a chunk in `out`, the E waves gv, and meetings
+    // (meet_signal / meet_wait) stand between the writing and the reading of a plane.
+    lds_t b_row = (8 * w + (lane >> 3)) * ROW_B + 16 * (lane & 7);
+    const uint32_t row_b = 2u * static_cast<uint32_t>(C);
+    uint32_t offA = (8 * w + (lane >> 3)) * row_b + 16 * (lane & 7);
+    char* __restrict__ pgr = reinterpret_cast<char*>(a.gr + base);
+    char* __restrict__ pgk = reinterpret_cast<char*>(a.gk + base);
+    char* __restrict__ pgv = reinterpret_cast<char*>(a.gv + base);
+    char* __restrict__ pgw = reinterpret_cast<char*>(a.gw + base);
+    bool met_ok = true;
     f32x4 E[4] = {zero4, zero4, zero4, zero4};     // dS[i = 16w + l16][j = 16 tile + 4g + v]
     const uint32_t b_e = (16 * w + l16) * N + 4 * g;                            // that element of a [value][key] state
     if (!LOCAL && a.ds32 != nullptr) {
@@ -654,7 +643,8 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
 #pragma unroll 1
     for (int it = 0; it < nit; ++it) {
         const int c = n + 1 - it;
-        opaque(b_acc); opaque(b_nat); opaque(b_tr); opaque(b_trt); opaque(b_tw); opaque(b_g); opaque(b_l);
+        opaque(b_acc); opaque(b_nat); opaque(b_tr); opaque(b_trt); opaque(b_tw); opaque(b_g); opaque(b_l); opaque(b_row);
+        asm volatile("" : "+v"(offA));
         if (it >= 2 && c >= 0) {
             const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B), to = uniform_base(sb + TILE0 + (c & 1) * TILE_B);
             // Operands are fetched in batches, each issued as a whole before anything waits for it (the scheduling barriers
@@ -727,9 +717,8 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                 U[tl] = mfma(rl[tl], gyo, U[tl]);
             }
             __builtin_amdgcn_sched_barrier(0);
-            // gv: lane = token, four consecutive value channels in registers; the prep waves store it in the next iteration,
-            // and have taken the last one out of `out` by now (they did that first thing in this iteration)
-            if constexpr (!LOCAL) meet_wait(&S.met[2], 8u * (it + 1));
+            // gv: lane = token, four consecutive value channels in registers (the rows of the last chunk were taken out of
+            // `out` before the barrier)
 #pragma unroll
             for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt)
                 lds_st<u32x2>(sb + OUT0 + 3 * PLANE_B + tt * 16 * ROW_B + 32 * w + b_acc, u32x2{pack_bf2(G[tt][0], G[tt][1]), pack_bf2(G[tt][2], G[tt][3])});
@@ -745,7 +734,28 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                 });
         }
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!LOCAL) {
+            // gv of chunk c, when all four E waves have written their channels
+            meet_signal(&S.met[2], lane);
+            met_ok = meet_wait(&S.met[2], 4u * (it + 1)) && met_ok;
+            const u32x4 o = lds_ld<u32x4>(sb + OUT0 + 3 * PLANE_B + b_row);
+            if (it >= 2 && c >= 0 && c * L + 8 * w + (lane >> 3) < T) *reinterpret_cast<u32x4*>(pgv + (static_cast<uint32_t>(c * L) * row_b + offA)) = o;
+        }
+        __builtin_amdgcn_sched_barrier(0);
         if (!LOCAL && it >= 1 && c - 1 >= 0) tiles(c - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!LOCAL) {
+            // gr, gk, gw of chunk c + 1, when all eight prep waves have finished their columns
+            met_ok = meet_wait(&S.met[1], 8u * (it + 1)) && met_ok;
+            const u32x4 o0 = lds_ld<u32x4>(sb + OUT0 + b_row), o1 = lds_ld<u32x4>(sb + OUT0 + PLANE_B + b_row), o2 = lds_ld<u32x4>(sb + OUT0 + 2 * PLANE_B + b_row);
+            if (it >= 3 && c + 1 >= 0 && (c + 1) * L + 8 * w + (lane >> 3) < T) {
+                const uint32_t ob = static_cast<uint32_t>((c + 1) * L) * row_b + offA;
+                *reinterpret_cast<u32x4*>(pgr + ob) = o0;
+                *reinterpret_cast<u32x4*>(pgk + ob) = o1;
+                if (!a.head_decay) *reinterpret_cast<u32x4*>(pgw + ob) = o2;
+            }
+        }
+        if (!met_ok && lane == 0) S.met[3] = 1;        // (the prep waves read it after the last barrier and flag the head)
         __syncthreads();
     }
     if constexpr (LOCAL) {
@@ -780,7 +790,7 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG arg) {
     const int n = (a.T + L - 1) / L;
     // the quadrant t < 16 <= s of the tiles is never written and must read as zero
     for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTG) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
-    if (tid < 3) S.met[tid] = 0;
+    if (tid < 4) S.met[tid] = 0;
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
     const int nit = (n + 3 + TRIP - 1) / TRIP * TRIP;      // iterations of the pipeline: n + 3, in whole trips of the prep loop

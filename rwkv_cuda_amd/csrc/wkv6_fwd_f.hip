@@ -164,15 +164,19 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
             lds_st<f32x2>(so + O_DEC + b_ch, f32x2{a0 * b0, a1 * b1});
         }
         float ruk[2];
+        HL r0[2], k0[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const float rp0 = rf[e][0] * exp2_fast(cc[e][0]), rp1 = rf[e][1] * exp2_fast(cc[e][1]);
             const float kp0 = kf[e][0] * exp2_fast(-(cc[e][0] + lam[e][0])), kp1 = kf[e][1] * exp2_fast(-(cc[e][1] + lam[e][1]));
             ruk[e] = fmaf(rf[e][0] * uj[0], kf[e][0], rf[e][1] * uj[1] * kf[e][1]);
-            const HL r0 = hilo2k(rp0, rp1), k0 = hilo2k(kp0, kp1);
-            lds_st<uint32_t>(so + O_RPH + e * 16 * ROW_B + b_tp, r0.h); lds_st<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp, r0.l);
-            lds_st<uint32_t>(so + O_KPH + e * 16 * ROW_B + b_tp, k0.h); lds_st<uint32_t>(so + O_KPL + e * 16 * ROW_B + b_tp, k0.l);
+            r0[e] = hilo2k(rp0, rp1); k0[e] = hilo2k(kp0, kp1);
         }
+        // (the stores side by side, with no load between them: the compiler then pairs them, two planes or two rows an instruction)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) { lds_st<uint32_t>(so + O_RPH + e * 16 * ROW_B + b_tp, r0[e].h); lds_st<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp, r0[e].l); }
+#pragma unroll
+        for (int e = 0; e < 2; ++e) { lds_st<uint32_t>(so + O_KPH + e * 16 * ROW_B + b_tp, k0[e].h); lds_st<uint32_t>(so + O_KPL + e * 16 * ROW_B + b_tp, k0[e].l); }
         allreduce2_rows(ruk[0], ruk[1]);                       // sums over the four channel pairs of this wave
         if (jq == 0) { lds_st<float>(so + O_RUK + w * (4 * L) + b_l, ruk[0]); lds_st<float>(so + O_RUK + w * (4 * L) + 64 + b_l, ruk[1]); }
     };
