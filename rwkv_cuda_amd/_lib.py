@@ -39,7 +39,7 @@ HIPCC_FLAGS = [
 # The wkv4 kernels that hold a segment's inputs in registers exist to avoid memory round trips: a spill defeats them.
 # The one-sweep backward lets the compiler count its waits: a spill inside its loops would put scratch traffic between a
 # prefetch and its use.  What it spills today are values that are only needed after the loops (indices of the gs store).
-SPILL_LIMIT = {"wkv6_bwd_fused": 5, "wkv6_fwd_fused": 0, "wkv6_fwd_ws": 0, "wkv6_bwd_a_ws": 0, "wkv6_bwd_b_wsILi0E": 3, "wkv6_bwd_b_wsILi1E": 1, "wkv6_bwd_b_wsILi2E": 1,
+SPILL_LIMIT = {"wkv6_bwd_fused": 0, "wkv6_fwd_fused": 0, "wkv6_fwd_ws": 0, "wkv6_bwd_a_ws": 0, "wkv6_bwd_b_wsILi0E": 3, "wkv6_bwd_b_wsILi1E": 1, "wkv6_bwd_b_wsILi2E": 1,
                "wkv_rows": 0, "wkv4_fwd_reg": 0, "wkv4_bwd_reg": 0}
 
 _lib = None

@@ -256,6 +256,25 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
     }
     __syncthreads();                       // iterations 0 and 1: nothing prepared yet
     __syncthreads();
+    // d1 and R' of a chunk have been in LDS for a whole iteration when its turn comes: they are asked for at the end of
+    // the chunk before, so that the scaling of the state can start right behind the barrier
+    float dq[4];
+    bf16x8 rh[2][2], rl[2][2];
+    auto ahead = [&](const int c) __attribute__((always_inline)) {
+        const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) dq[q] = lds_ld<float>(so + O_D1 + 64 * q + b_g);
+        if constexpr (!LOCAL) {
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks) {
+                    rh[tt][ks] = ld_acc(so + O_RPH + tt * 16 * ROW_B + 64 * ks + b_acc);
+                    rl[tt][ks] = ld_acc(so + O_RPL + tt * 16 * ROW_B + 64 * ks + b_acc);
+                }
+        }
+    };
+    ahead(0);
 #pragma unroll 1
     for (int c = 0; c < n; ++c) {
         opaque(b_acc); opaque(b_tr); opaque(b_natt); opaque(b_g); opaque(b_ss);
@@ -267,27 +286,21 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
 #pragma unroll
             for (int tl = 0; tl < 4; ++tl) lds_st<f32x4>(sb + SST0 + 64 * tl + b_ss, St[tl]);
         }
-        // ------------------------------------------------------------ batch 1: d1 and R' (natural rows)
+        // ------------------------------------------------------------ batch 1: d1, R' (natural rows), v and the A tile
         // per-channel factors: a lane holds the one of channel 16 tile + 4 g + (l16 & 3), a 4-byte read that all rows of
         // four lanes share; the products below take lane v of the 16-lane row inside the multiply (row_newbcast)
-        float dq[4], de[4], d2[4];
+        float de[4], d2[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            dq[q] = lds_ld<float>(so + O_D1 + 64 * q + b_g);
             de[q] = lds_ld<float>(so + O_DEC + 64 * q + b_g);
             d2[q] = lds_ld<float>(so + O_D2 + 64 * q + b_g);
         }
         // (LOCAL: only the state is wanted, everything that serves y is left out)
-        bf16x8 rh[2][2], rl[2][2];
-        if constexpr (!LOCAL) {
+        // (v with the tokens along K and the A tile by rows as well: they arrive while the state is scaled and split)
+        const bf16x8 vop = ld_tr(so + O_V + 32 * w + b_tr, ROW_B);              // lane = value channel 16w + l16, K = tokens
+        bf16x8 ah[2], al[2];
 #pragma unroll
-            for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks) {
-                    rh[tt][ks] = ld_acc(so + O_RPH + tt * 16 * ROW_B + 64 * ks + b_acc);
-                    rl[tt][ks] = ld_acc(so + O_RPL + tt * 16 * ROW_B + 64 * ks + b_acc);
-                }
-        }
+        for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt) { ah[tt] = ld_op(to + T_AH + tt * 16 * TROW_B + b_natt); al[tt] = ld_op(to + T_AL + tt * 16 * TROW_B + b_natt); }
         __builtin_amdgcn_sched_barrier(0);
         // ------------------------------------------------------------ y^T[i][t] = (S d1) R'^T + V^T A^T
         bf16x8 sh[2], sl[2];
@@ -303,12 +316,6 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
             sh[ks] = as_op(x0.h, x1.h, x2.h, x3.h);
             sl[ks] = as_op(x0.l, x1.l, x2.l, x3.l);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        // ------------------------------------------------------------ batch 2: v with the tokens along K, the A tile by rows
-        const bf16x8 vop = ld_tr(so + O_V + 32 * w + b_tr, ROW_B);              // lane = value channel 16w + l16, K = tokens
-        bf16x8 ah[2], al[2];
-#pragma unroll
-        for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt) { ah[tt] = ld_op(to + T_AH + tt * 16 * TROW_B + b_natt); al[tt] = ld_op(to + T_AL + tt * 16 * TROW_B + b_natt); }
         __builtin_amdgcn_sched_barrier(0);
         f32x4 Y[2] = {zero4, zero4};
 #pragma unroll
@@ -336,6 +343,8 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
             U[tl] = mfma(kh[tl], vop, zero4);
             U[tl] = mfma(kl[tl], vop, U[tl]);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        ahead(c + 1);                      // (past the last chunk: a slot that holds something, read for nothing)
         __builtin_amdgcn_sched_barrier(0);
         // y: lane = token, four consecutive value channels in registers
 #pragma unroll
