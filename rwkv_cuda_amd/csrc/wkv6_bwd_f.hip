@@ -141,8 +141,11 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     // global addresses: a wave-uniform base and a 32-bit byte offset per lane (row of the chunk + 16 bytes of the row), to
     // which a chunk adds a uniform term; rows past the end of the sequence are clamped to the last one
     const char* __restrict__ pA = reinterpret_cast<const char*>((lower ? a.r : a.k) + base);                         // r | k
-    const char* __restrict__ pB = reinterpret_cast<const char*>(lower ? (a.head_decay ? static_cast<const uint16_t*>(a.w) + h * N : static_cast<const uint16_t*>(a.w) + base) : a.v + base);   // w | v
-    const uint32_t bmask = (lower && a.head_decay) ? 127u : ~0u;        // wkv5: the decay row of the head at every token
+    constexpr bool HD = WMODE == W_HEAD;   // wkv5: one decay per channel, the same at every token
+    // (HD: the r waves keep their second load, of the head's decay row at every token - a cache hit - so that all prep waves
+    //  run the same loads and the waits count the same; the decay itself is read once, below)
+    const char* __restrict__ pB = reinterpret_cast<const char*>(lower ? (HD ? static_cast<const uint16_t*>(a.w) + h * N : static_cast<const uint16_t*>(a.w) + base) : a.v + base);   // w | v
+    const uint32_t bmask = (lower && HD) ? 127u : ~0u;
     const char* __restrict__ pC = reinterpret_cast<const char*>(a.gy + base);
     const uint32_t row_b = 2u * static_cast<uint32_t>(a.C);                                     // bytes from a token to the next
     uint32_t offA = (8 * (w & 3) + (lane >> 3)) * row_b + 16 * (lane & 7);                      // rows 8 (w & 3) .. +7
@@ -171,7 +174,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         const u32x4 zero = {0u, 0u, 0u, 0u};
         const lds_t da = so + (lower ? O_RPH : O_KPH) + b_row, db = so + (lower ? O_RPL : O_V) + b_row;
         lds_st<u32x4>(da, live ? x.a : zero);
-        lds_st<u32x4>(db, (live || lower) ? x.b : zero);                 // w of a dead row is masked where the decay is formed
+        if (!(HD && lower)) lds_st<u32x4>(db, (live || lower) ? x.b : zero);    // w of a dead row is masked where the decay is formed
         if (lane < 32) lds_st<u32x4>(so + O_GY + b_rowg, liveg ? x.c : zero);
     };
     // what the finishing of a chunk needs from its preparation, three iterations earlier
@@ -182,44 +185,85 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
     bool any_exact = false, met_ok = true;
     float logdec[2] = {0.f, 0.f};          // LOCAL: log2 of the decay over the whole block
     float carry[2] = {0.f, 0.f}, gu_acc[2] = {0.f, 0.f}, gw_acc[2] = {0.f, 0.f};
+    // HD: the factors of every whole chunk are the same: the sums along time are products, the exponentials are taken once
+    float lamc[2] = {0.f, 0.f}, eac[2][2] = {}, ebc[2][2] = {}, dc[2] = {0.f, 0.f}, lfc[2] = {0.f, 0.f};
+    if constexpr (HD) {
+        const uint32_t x = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(a.w) + h * N + ch0);
+        lamc[0] = -LOG2E * exp2_fast(LOG2E * bf_lo(x)); lamc[1] = -LOG2E * exp2_fast(LOG2E * bf_hi(x));
+#pragma unroll
+        for (int z = 0; z < 2; ++z) {
+            const float cc0 = -static_cast<float>(16 - tp) * lamc[z], cc1 = static_cast<float>(tp) * lamc[z];
+            eac[0][z] = exp2_fast(cc0); eac[1][z] = exp2_fast(cc1);
+            ebc[0][z] = exp2_fast(-(cc0 + lamc[z])); ebc[1][z] = exp2_fast(-(cc1 + lamc[z]));
+            dc[z] = exp2_fast(16.f * lamc[z]);              // d1 = d2: the decay over half a chunk
+            lfc[z] = gw_factor(lamc[z] * LN2);
+        }
+        const bool bad = (-16.f * lamc[0] > RANGE_LIMIT * LOG2E) || (-16.f * lamc[1] > RANGE_LIMIT * LOG2E);
+        any_exact = __ballot(bad) != 0ull;
+    }
     // Only the last chunk of the sequence can be cut short (PARTIAL): its rows past T carry no input and no decay.
 
     auto prep = [&](const int c, Held& hd, auto PARTIAL) __attribute__((always_inline)) {
         const lds_t so = uniform_base(sb + SLOT0 + ((c + 9) % 3) * SLOT_B);
-        float lam[2][2], rf[2][2], kf[2][2], cc[2][2];
-        uint32_t xr[2], xk[2], xw[2];
+        constexpr bool CONST = HD && !decltype(PARTIAL)::value;      // a whole chunk of a constant decay
+        float lam[2][2], rf[2][2], kf[2][2], ea[2][2], eb[2][2];
+        uint32_t xr[2], xk[2], xw[2] = {0u, 0u};
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             xr[e] = lds_ld<uint32_t>(so + O_RPH + e * 16 * ROW_B + b_tp);
             xk[e] = lds_ld<uint32_t>(so + O_KPH + e * 16 * ROW_B + b_tp);
-            xw[e] = lds_ld<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp);
+            if constexpr (!HD) xw[e] = lds_ld<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp);
         }
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const bool live = !decltype(PARTIAL)::value || (c >= 0 && c * L + tp + 16 * e < T);
             rf[e][0] = bf_lo(xr[e]); rf[e][1] = bf_hi(xr[e]);
             kf[e][0] = bf_lo(xk[e]); kf[e][1] = bf_hi(xk[e]);
-            lam[e][0] = live ? -LOG2E * exp2_fast(LOG2E * bf_lo(xw[e])) : 0.f;
-            lam[e][1] = live ? -LOG2E * exp2_fast(LOG2E * bf_hi(xw[e])) : 0.f;
             hd.r[e] = xr[e]; hd.k[e] = xk[e];
         }
-        float l1[2], l2[2];
+        float a0, a1, b0, b1;
+        if constexpr (CONST) {
+            // (the finishing takes the constant factors too: nothing but r and k is kept)
 #pragma unroll
-        for (int z = 0; z < 2; ++z) {
-            const float s0 = row_suffix_sum(lam[0][z]);        // sum over tokens tp..15
-            const float p1 = row_prefix_sum(lam[1][z]);        // sum over tokens 16..16+tp
-            cc[0][z] = -s0;
-            cc[1][z] = p1 - lam[1][z];
-            l1[z] = bc<0>(s0);
-            l2[z] = bc<15>(p1);
-            if constexpr (LOCAL) logdec[z] += l1[z] + l2[z];
-        }
-        {
-            const bool bad = (-l1[0] > RANGE_LIMIT * LOG2E) || (-l2[0] > RANGE_LIMIT * LOG2E) || (-l1[1] > RANGE_LIMIT * LOG2E) || (-l2[1] > RANGE_LIMIT * LOG2E);
-            any_exact = any_exact || (__ballot(bad) != 0ull);
+            for (int e = 0; e < 2; ++e)
+#pragma unroll
+                for (int z = 0; z < 2; ++z) { ea[e][z] = eac[e][z]; eb[e][z] = ebc[e][z]; }
+            a0 = dc[0]; a1 = dc[1]; b0 = dc[0]; b1 = dc[1];
+            if constexpr (LOCAL) { logdec[0] += 32.f * lamc[0]; logdec[1] += 32.f * lamc[1]; }
+        } else {
+            float cc[2][2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const bool live = !decltype(PARTIAL)::value || (c >= 0 && c * L + tp + 16 * e < T);
+                lam[e][0] = live ? (HD ? lamc[0] : -LOG2E * exp2_fast(LOG2E * bf_lo(xw[e]))) : 0.f;
+                lam[e][1] = live ? (HD ? lamc[1] : -LOG2E * exp2_fast(LOG2E * bf_hi(xw[e]))) : 0.f;
+            }
+            float l1[2], l2[2];
+#pragma unroll
+            for (int z = 0; z < 2; ++z) {
+                const float s0 = row_suffix_sum(lam[0][z]);        // sum over tokens tp..15
+                const float p1 = row_prefix_sum(lam[1][z]);        // sum over tokens 16..16+tp
+                cc[0][z] = -s0;
+                cc[1][z] = p1 - lam[1][z];
+                l1[z] = bc<0>(s0);
+                l2[z] = bc<15>(p1);
+                if constexpr (LOCAL) logdec[z] += l1[z] + l2[z];
+            }
+            {
+                const bool bad = (-l1[0] > RANGE_LIMIT * LOG2E) || (-l2[0] > RANGE_LIMIT * LOG2E) || (-l1[1] > RANGE_LIMIT * LOG2E) || (-l2[1] > RANGE_LIMIT * LOG2E);
+                any_exact = any_exact || (__ballot(bad) != 0ull);
+            }
+            a0 = exp2_fast(l1[0]); a1 = exp2_fast(l1[1]); b0 = exp2_fast(l2[0]); b1 = exp2_fast(l2[1]);
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+#pragma unroll
+                for (int z = 0; z < 2; ++z) {
+                    ea[e][z] = exp2_fast(cc[e][z]);
+                    eb[e][z] = exp2_fast(-(cc[e][z] + lam[e][z]));
+                    hd.ea[e][z] = ea[e][z]; hd.eb[e][z] = eb[e][z];
+                    hd.lf[e][z] = gw_factor(lam[e][z] * LN2);
+                }
         }
         if (tp == 0) {
-            const float a0 = exp2_fast(l1[0]), a1 = exp2_fast(l1[1]), b0 = exp2_fast(l2[0]), b1 = exp2_fast(l2[1]);
             lds_st<f32x2>(so + O_D1 + b_ch, f32x2{a0, a1});
             lds_st<f32x2>(so + O_D2 + b_ch, f32x2{b0, b1});
             lds_st<f32x2>(so + O_DEC + b_ch, f32x2{a0 * b0, a1 * b1});
@@ -228,14 +272,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         HL r0[2], k0[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-#pragma unroll
-            for (int z = 0; z < 2; ++z) {
-                hd.ea[e][z] = exp2_fast(cc[e][z]);
-                hd.eb[e][z] = exp2_fast(-(cc[e][z] + lam[e][z]));
-                hd.lf[e][z] = gw_factor(lam[e][z] * LN2);
-            }
-            const float rp0 = rf[e][0] * hd.ea[e][0], rp1 = rf[e][1] * hd.ea[e][1];
-            const float kp0 = kf[e][0] * hd.eb[e][0], kp1 = kf[e][1] * hd.eb[e][1];
+            const float rp0 = rf[e][0] * ea[e][0], rp1 = rf[e][1] * ea[e][1];
+            const float kp0 = kf[e][0] * eb[e][0], kp1 = kf[e][1] * eb[e][1];
             ruk[e] = fmaf(rf[e][0] * uj[0], kf[e][0], rf[e][1] * uj[1] * kf[e][1]);
             r0[e] = hilo2k(rp0, rp1); k0[e] = hilo2k(kp0, kp1);
         }
@@ -250,6 +288,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
 
     // gr, gk, gw of chunk c from X, Z (left by the SD waves in the last iteration) and what prep kept
     auto finish = [&](const int c, const Held& hd, auto PARTIAL) __attribute__((always_inline)) {
+        constexpr bool CONSTF = HD && !decltype(PARTIAL)::value;
         const lds_t xo = uniform_base(sb + XZ0 + (c & 1) * 2 * XZ_B), vo = uniform_base(sb + VG0 + (c % 3) * (4 * L));
         float q[2][2], kdk[2][2];
         uint32_t ogr[2], ogk[2];
@@ -263,7 +302,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             float gr[2], gk[2];
 #pragma unroll
             for (int z = 0; z < 2; ++z) {
-                const float drp = hd.ea[e][z] * X[z], dkp = hd.eb[e][z] * Z[z];
+                const float drp = (CONSTF ? eac[e][z] : hd.ea[e][z]) * X[z], dkp = (CONSTF ? ebc[e][z] : hd.eb[e][z]) * Z[z];
                 const float uvg = uj[z] * vg;
                 gr[z] = fmaf(uvg, kf[z], drp);
                 gk[z] = fmaf(uvg, rf[z], dkp);
@@ -280,8 +319,8 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         for (int z = 0; z < 2; ++z) {
             const float s1 = row_suffix_sum(q[1][z]) + carry[z];           // P_t of the second half
             const float s0 = row_suffix_sum(q[0][z]) + bc<0>(s1);
-            gw[1][z] = hd.lf[1][z] * ((s1 - q[1][z]) - kdk[1][z]);        // lam (P_{t+1} - k dk')
-            gw[0][z] = hd.lf[0][z] * ((s0 - q[0][z]) - kdk[0][z]);
+            gw[1][z] = (CONSTF ? lfc[z] : hd.lf[1][z]) * ((s1 - q[1][z]) - kdk[1][z]);        // lam (P_{t+1} - k dk')
+            gw[0][z] = (CONSTF ? lfc[z] : hd.lf[0][z]) * ((s0 - q[0][z]) - kdk[0][z]);
             carry[z] = bc<0>(s0);
         }
         if (!(c & 1)) {
@@ -291,7 +330,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
         }
         // without an initial state nothing has been accumulated before token 0: its decay has no effect at all
         if (a.gs == nullptr && a.first && c == 0 && tp == 0) { gw[0][0] = 0.f; gw[0][1] = 0.f; }
-        if (a.head_decay) {
+        if (HD) {
             gw_acc[0] += gw[0][0] + gw[1][0]; gw_acc[1] += gw[0][1] + gw[1][1];
         } else {
 #pragma unroll
@@ -354,7 +393,7 @@ DEVINL void role_prep(SmemG& S, const ArgsG& a, const int lane, const int w, con
             if (a.gu32 != nullptr) *reinterpret_cast<float2*>(a.gu32 + ch0) = make_float2(gu_acc[0], gu_acc[1]);
             else *reinterpret_cast<uint32_t*>(a.gu + ch0) = pack_bf2(gu_acc[0], gu_acc[1]);
         }
-        if (a.head_decay) {
+        if (HD) {
 #pragma unroll
             for (int z = 0; z < 2; ++z) gw_acc[z] = row_sum_to_last(gw_acc[z]);
             if (tp == 15) {
@@ -542,6 +581,7 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
 // ---------------------------------------------------------------------------------------------------- E waves
 template <int WMODE, bool LOCAL>
 DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t base, const int n, const int nit) {
+    constexpr bool HD = WMODE == W_HEAD;
     const int g = lane >> 4, l16 = lane & 15;
     const int T = a.T, C = a.C;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -752,7 +792,7 @@ DEVINL void role_e(SmemG& S, const ArgsG& a, const int lane, const int w, const 
                 const uint32_t ob = static_cast<uint32_t>((c + 1) * L) * row_b + offA;
                 *reinterpret_cast<u32x4*>(pgr + ob) = o0;
                 *reinterpret_cast<u32x4*>(pgk + ob) = o1;
-                if (!a.head_decay) *reinterpret_cast<u32x4*>(pgw + ob) = o2;
+                if (!HD) *reinterpret_cast<u32x4*>(pgw + ob) = o2;
             }
         }
         if (!met_ok && lane == 0) S.met[3] = 1;        // (the prep waves read it after the last barrier and flag the head)
@@ -826,16 +866,20 @@ int launch_wkv6_bwd_fused(hipStream_t st, int B, int T, int C, int H, const uint
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu; a.gs = gs; a.saved = saved; a.flags = flags;
     a.NB = 1; a.TB = T;
+    const bool hd = a.head_decay;
     if (NB <= 1) {
-        hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, false>), dim3(B * H), dim3(NTG), 0, st, a);
+        if (hd) hipLaunchKernelGGL((wkv6_bwd_fused<W_HEAD, false>), dim3(B * H), dim3(NTG), 0, st, a);
+        else hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, false>), dim3(B * H), dim3(NTG), 0, st, a);
         return launch_status();
     }
     a.NB = NB; a.TB = TB; a.blk_ds = blk_ds; a.blk_decay = blk_decay;
-    hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, true>), dim3(B * H * NB), dim3(NTG), 0, st, a);
+    if (hd) hipLaunchKernelGGL((wkv6_bwd_fused<W_HEAD, true>), dim3(B * H * NB), dim3(NTG), 0, st, a);
+    else hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, true>), dim3(B * H * NB), dim3(NTG), 0, st, a);
     if (int e = launch_wkv6_scan_reverse(st, B * H, NB, blk_ds, blk_decay, ds32)) return e;
     a.blk_ds = nullptr; a.blk_decay = nullptr; a.ds32 = ds32; a.gu32 = gu32;
     if (gwp != nullptr) a.gw32 = gw32;
-    hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, false>), dim3(B * H * NB), dim3(NTG), 0, st, a);
+    if (hd) hipLaunchKernelGGL((wkv6_bwd_fused<W_HEAD, false>), dim3(B * H * NB), dim3(NTG), 0, st, a);
+    else hipLaunchKernelGGL((wkv6_bwd_fused<W_RAW, false>), dim3(B * H * NB), dim3(NTG), 0, st, a);
     const size_t n = static_cast<size_t>(B) * C;
     hipLaunchKernelGGL(gu_block_sum, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, NB, n, gu32, gu);
     if (gwp != nullptr) hipLaunchKernelGGL(gu_block_sum, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, st, NB, n, gw32, gwp);

@@ -71,7 +71,7 @@ struct ArgsQ {
 };
 
 // ---------------------------------------------------------------------------------------------------- P waves
-template <bool LOCAL>
+template <bool LOCAL, bool HD>
 DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, const size_t base, const int h, const size_t bh, const int n, const int nit) {
     int jq = lane >> 4, tp = lane & 15;                 // arithmetic: channel pair, token (and token + 16)
     // Global memory is touched in whole 128-byte rows: eight lanes per row, eight rows per wave and instruction (waves
@@ -87,8 +87,10 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
     // which a chunk adds a uniform term; rows past the end of the sequence are clamped to the last one
     const char* __restrict__ pA = reinterpret_cast<const char*>((lower ? a.r : a.k) + base);      // r | k
     // wkv5: the decay row of the head stands in for every token's (the loads stay, they hit the cache)
-    const char* __restrict__ pB = reinterpret_cast<const char*>(lower ? (a.head_decay ? a.w + h * N : a.w + base) : a.v + base);   // w | v
-    const uint32_t bmask = (lower && a.head_decay) ? 127u : ~0u;
+    // (HD: the decay is one value per channel and read once below; the r waves keep their second load, of the head's decay
+    //  row at every token - a cache hit - so that all prep waves run the same loads and the waits count the same)
+    const char* __restrict__ pB = reinterpret_cast<const char*>(lower ? (HD ? a.w + h * N : a.w + base) : a.v + base);   // w | v
+    const uint32_t bmask = (HD && lower) ? 127u : ~0u;
     const uint32_t row_b = 2u * static_cast<uint32_t>(a.C);                                     // bytes from a token to the next
     uint32_t offA = (8 * (w & 3) + (lane >> 3)) * row_b + 16 * (lane & 7);                      // rows 8 (w & 3) .. +7
     const uint32_t lastA = static_cast<uint32_t>(a.T - 1) * row_b + 16 * (lane & 7);
@@ -119,46 +121,81 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
         const bool live = !decltype(PARTIAL)::value || c * L + row < T;
         const u32x4 zero = {0u, 0u, 0u, 0u};
         lds_st<u32x4>(so + (lower ? O_RPH : O_KPH) + b_row, live ? x.a : zero);
-        lds_st<u32x4>(so + (lower ? O_RPL : O_V) + b_row, (live || lower) ? x.b : zero);    // w of a dead row is masked where the decay is formed
+        if (!(HD && lower)) lds_st<u32x4>(so + (lower ? O_RPL : O_V) + b_row, (live || lower) ? x.b : zero);    // w of a dead row is masked where the decay is formed
         meet_signal(&S.met[0], lane);
     };
     bool any_exact = false, met_ok = true;
     float logdec[2] = {0.f, 0.f};          // LOCAL: log2 of the decay over the whole block
+    // HD (wkv5): the decay of a channel is the same at every token, and so are the factors of every whole chunk: the sums
+    // along time are products, the exponentials are taken once
+    float lamc[2] = {0.f, 0.f}, eac[2][2] = {}, ebc[2][2] = {}, dc[2] = {0.f, 0.f};
+    if constexpr (HD) {
+        const uint32_t x = *reinterpret_cast<const uint32_t*>(a.w + h * N + ch0);
+        lamc[0] = -LOG2E * exp2_fast(LOG2E * bf_lo(x)); lamc[1] = -LOG2E * exp2_fast(LOG2E * bf_hi(x));
+#pragma unroll
+        for (int z = 0; z < 2; ++z) {
+            const float cc0 = -static_cast<float>(16 - tp) * lamc[z], cc1 = static_cast<float>(tp) * lamc[z];
+            eac[0][z] = exp2_fast(cc0); eac[1][z] = exp2_fast(cc1);
+            ebc[0][z] = exp2_fast(-(cc0 + lamc[z])); ebc[1][z] = exp2_fast(-(cc1 + lamc[z]));
+            dc[z] = exp2_fast(16.f * lamc[z]);              // d1 = d2: the decay over half a chunk
+        }
+        const bool bad = (-16.f * lamc[0] > RANGE_LIMIT * LOG2E) || (-16.f * lamc[1] > RANGE_LIMIT * LOG2E);
+        any_exact = __ballot(bad) != 0ull;
+    }
     auto prep = [&](const int c, auto PARTIAL) __attribute__((always_inline)) {
         const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B);
-        float lam[2][2], rf[2][2], kf[2][2], cc[2][2];
-        uint32_t xr[2], xk[2], xw[2];
+        constexpr bool CONST = HD && !decltype(PARTIAL)::value;      // a whole chunk of a constant decay
+        float lam[2][2], rf[2][2], kf[2][2], ea[2][2], eb[2][2];
+        uint32_t xr[2], xk[2], xw[2] = {0u, 0u};
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             xr[e] = lds_ld<uint32_t>(so + O_RPH + e * 16 * ROW_B + b_tp);
             xk[e] = lds_ld<uint32_t>(so + O_KPH + e * 16 * ROW_B + b_tp);
-            xw[e] = lds_ld<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp);
+            if constexpr (!HD) xw[e] = lds_ld<uint32_t>(so + O_RPL + e * 16 * ROW_B + b_tp);
         }
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const bool live = !decltype(PARTIAL)::value || c * L + tp + 16 * e < T;
             rf[e][0] = bf_lo(xr[e]); rf[e][1] = bf_hi(xr[e]);
             kf[e][0] = bf_lo(xk[e]); kf[e][1] = bf_hi(xk[e]);
-            lam[e][0] = live ? -LOG2E * exp2_fast(LOG2E * bf_lo(xw[e])) : 0.f;
-            lam[e][1] = live ? -LOG2E * exp2_fast(LOG2E * bf_hi(xw[e])) : 0.f;
         }
-        float l1[2], l2[2];
+        float a0, a1, b0, b1;
+        if constexpr (CONST) {
 #pragma unroll
-        for (int z = 0; z < 2; ++z) {
-            const float s0 = row_suffix_sum(lam[0][z]);        // sum over tokens tp..15
-            const float p1 = row_prefix_sum(lam[1][z]);        // sum over tokens 16..16+tp
-            cc[0][z] = -s0;
-            cc[1][z] = p1 - lam[1][z];
-            l1[z] = bc<0>(s0);
-            l2[z] = bc<15>(p1);
-            if constexpr (LOCAL) logdec[z] += l1[z] + l2[z];
-        }
-        {
-            const bool bad = (-l1[0] > RANGE_LIMIT * LOG2E) || (-l2[0] > RANGE_LIMIT * LOG2E) || (-l1[1] > RANGE_LIMIT * LOG2E) || (-l2[1] > RANGE_LIMIT * LOG2E);
-            any_exact = any_exact || (__ballot(bad) != 0ull);
+            for (int e = 0; e < 2; ++e)
+#pragma unroll
+                for (int z = 0; z < 2; ++z) { ea[e][z] = eac[e][z]; eb[e][z] = ebc[e][z]; }
+            a0 = dc[0]; a1 = dc[1]; b0 = dc[0]; b1 = dc[1];
+            if constexpr (LOCAL) { logdec[0] += 32.f * lamc[0]; logdec[1] += 32.f * lamc[1]; }
+        } else {
+            float cc[2][2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const bool live = !decltype(PARTIAL)::value || c * L + tp + 16 * e < T;
+                lam[e][0] = live ? (HD ? lamc[0] : -LOG2E * exp2_fast(LOG2E * bf_lo(xw[e]))) : 0.f;
+                lam[e][1] = live ? (HD ? lamc[1] : -LOG2E * exp2_fast(LOG2E * bf_hi(xw[e]))) : 0.f;
+            }
+            float l1[2], l2[2];
+#pragma unroll
+            for (int z = 0; z < 2; ++z) {
+                const float s0 = row_suffix_sum(lam[0][z]);        // sum over tokens tp..15
+                const float p1 = row_prefix_sum(lam[1][z]);        // sum over tokens 16..16+tp
+                cc[0][z] = -s0;
+                cc[1][z] = p1 - lam[1][z];
+                l1[z] = bc<0>(s0);
+                l2[z] = bc<15>(p1);
+                if constexpr (LOCAL) logdec[z] += l1[z] + l2[z];
+            }
+            {
+                const bool bad = (-l1[0] > RANGE_LIMIT * LOG2E) || (-l2[0] > RANGE_LIMIT * LOG2E) || (-l1[1] > RANGE_LIMIT * LOG2E) || (-l2[1] > RANGE_LIMIT * LOG2E);
+                any_exact = any_exact || (__ballot(bad) != 0ull);
+            }
+            a0 = exp2_fast(l1[0]); a1 = exp2_fast(l1[1]); b0 = exp2_fast(l2[0]); b1 = exp2_fast(l2[1]);
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+#pragma unroll
+                for (int z = 0; z < 2; ++z) { ea[e][z] = exp2_fast(cc[e][z]); eb[e][z] = exp2_fast(-(cc[e][z] + lam[e][z])); }
         }
         if (tp == 0) {
-            const float a0 = exp2_fast(l1[0]), a1 = exp2_fast(l1[1]), b0 = exp2_fast(l2[0]), b1 = exp2_fast(l2[1]);
             lds_st<f32x2>(so + O_D1 + b_ch, f32x2{a0, a1});
             lds_st<f32x2>(so + O_D2 + b_ch, f32x2{b0, b1});
             lds_st<f32x2>(so + O_DEC + b_ch, f32x2{a0 * b0, a1 * b1});
@@ -167,8 +204,8 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
         HL r0[2], k0[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-            const float rp0 = rf[e][0] * exp2_fast(cc[e][0]), rp1 = rf[e][1] * exp2_fast(cc[e][1]);
-            const float kp0 = kf[e][0] * exp2_fast(-(cc[e][0] + lam[e][0])), kp1 = kf[e][1] * exp2_fast(-(cc[e][1] + lam[e][1]));
+            const float rp0 = rf[e][0] * ea[e][0], rp1 = rf[e][1] * ea[e][1];
+            const float kp0 = kf[e][0] * eb[e][0], kp1 = kf[e][1] * eb[e][1];
             ruk[e] = fmaf(rf[e][0] * uj[0], kf[e][0], rf[e][1] * uj[1] * kf[e][1]);
             r0[e] = hilo2k(rp0, rp1); k0[e] = hilo2k(kp0, kp1);
         }
@@ -438,7 +475,7 @@ DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
     }
 }
 
-template <bool LOCAL>
+template <bool LOCAL, bool HD>
 __global__ __launch_bounds__(NTQ) void wkv6_fwd_fused(const ArgsQ arg) {
     __shared__ SmemQ S;
     const int tid = threadIdx.x;
@@ -461,7 +498,7 @@ __global__ __launch_bounds__(NTQ) void wkv6_fwd_fused(const ArgsQ arg) {
     __syncthreads();
     const int wid = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, w = wid & 3;
     const int nit = (n + 2 + DEPTH) & ~(DEPTH - 1);        // iterations of the pipeline: n + 3, in whole trips of the prep loop
-    if (wid < 8) role_prep<LOCAL>(S, a, lane, wid, base, h, bh, n, nit);
+    if (wid < 8) role_prep<LOCAL, HD>(S, a, lane, wid, base, h, bh, n, nit);
     else if (wid < 12) role_state<LOCAL>(S, a, lane, w, bh, n, nit);
     else role_tiles<LOCAL>(S, a, lane, w, bh, n, nit);
 }
@@ -497,14 +534,17 @@ int launch_wkv6_fwd_fused(hipStream_t st, int B, int T, int C, int H, const uint
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y; a.saved = saved; a.flags = flags;
     a.NB = 1; a.TB = T;
     if (NB <= 1) {
-        hipLaunchKernelGGL(wkv6_fwd_fused<false>, dim3(B * H), dim3(NTQ), 0, st, a);
+        if (head_decay) hipLaunchKernelGGL((wkv6_fwd_fused<false, true>), dim3(B * H), dim3(NTQ), 0, st, a);
+        else hipLaunchKernelGGL((wkv6_fwd_fused<false, false>), dim3(B * H), dim3(NTQ), 0, st, a);
         return launch_status();
     }
     a.NB = NB; a.TB = TB; a.blk_state = blk_state; a.blk_decay = blk_decay;
-    hipLaunchKernelGGL(wkv6_fwd_fused<true>, dim3(B * H * NB), dim3(NTQ), 0, st, a);
+    if (head_decay) hipLaunchKernelGGL((wkv6_fwd_fused<true, true>), dim3(B * H * NB), dim3(NTQ), 0, st, a);
+    else hipLaunchKernelGGL((wkv6_fwd_fused<true, false>), dim3(B * H * NB), dim3(NTQ), 0, st, a);
     hipLaunchKernelGGL(wkv6_scan, dim3(B * H), dim3(256), 0, st, blk_state, blk_decay, s0, s32, NB, 0);
     a.blk_state = nullptr; a.blk_decay = nullptr; a.s32 = s32;
-    hipLaunchKernelGGL(wkv6_fwd_fused<false>, dim3(B * H * NB), dim3(NTQ), 0, st, a);
+    if (head_decay) hipLaunchKernelGGL((wkv6_fwd_fused<false, true>), dim3(B * H * NB), dim3(NTQ), 0, st, a);
+    else hipLaunchKernelGGL((wkv6_fwd_fused<false, false>), dim3(B * H * NB), dim3(NTQ), 0, st, a);
     return launch_status();
 }
 
