@@ -19,7 +19,7 @@ DEVINL void opaque(lds_t& x) { asm volatile("" : "+v"(x)); }
 // a wave-uniform base (a slot, a tile) behind an empty asm: left to itself the compiler merges "(c % 3) * size" of two
 // chunks into one induction variable plus constants, some of them negative, and a negative constant cannot ride in the
 // offset field of an LDS instruction: every such read then costs an add
-DEVINL lds_t uniform_base(lds_t x) { asm volatile("" : "+s"(x)); return x; }
+DEVINL lds_t uniform_base(lds_t x) { x = __builtin_amdgcn_readfirstlane(x); asm volatile("" : "+s"(x)); return x; }
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef v4s __attribute__((address_space(3))) * lds_v4s_ptr;
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
