@@ -145,7 +145,7 @@ int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H,
 int launch_wkv6_fwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
                           const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, float* saved, int* flags,
                           int NB = 1, int TB = 0, float* blk_state = nullptr, float* blk_decay = nullptr, float* s32 = nullptr,
-                          bool head_decay = false);
+                          float* decay_out = nullptr);
 int launch_wkv6_scan_reverse(hipStream_t st, int BH, int NB, const float* local, const float* logdec, float* out);
 int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                             const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,

@@ -1364,8 +1364,11 @@ int rwkv_wkv5s_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16
     if (int e = check_dims(B, T, C, H)) return e;
     if (int e = check_ptrs({r, k, v, w_raw, u, y, decay}, C == H * N)) return e;
     const hipStream_t st = static_cast<hipStream_t>(stream);
-    hipLaunchKernelGGL(wkv5_decay_transform, dim3((C + 255) / 256), dim3(256), 0, st, C, w_raw, decay);
-    if (!fused_ok(T, C, H, flags) || saved == nullptr) return rwkv_wkv5_forward_ex(stream, B, T, C, H, r, k, v, decay, u, y, flags);
+    if (!fused_ok(T, C, H, flags) || saved == nullptr) {
+        hipLaunchKernelGGL(wkv5_decay_transform, dim3((C + 255) / 256), dim3(256), 0, st, C, w_raw, decay);
+        return rwkv_wkv5_forward_ex(stream, B, T, C, H, r, k, v, decay, u, y, flags);
+    }
+    // (the one-sweep kernel writes `decay` itself: its workgroups of batch row 0 hold every channel's raw value)
     if (saved_bytes < rwkv_wkv5s_saved_bytes(B, T, C, H) || !aligned16(saved)) return RWKV_ERR_WORKSPACE;
     const size_t nflag = round16(static_cast<size_t>(B) * H * 8 * sizeof(int));
     char* sb = static_cast<char*>(saved);
@@ -1378,8 +1381,8 @@ int rwkv_wkv5s_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16
         float* s32 = local + nq * 64 * 64;
         float* logdec = s32 + nq * 64 * 64;
         zero_words(st, flg, static_cast<size_t>(B) * H * 8);
-        if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w_raw, u, nullptr, y, static_cast<float*>(saved), flg, NB, TB, local, logdec, s32, true)) return e;
-    } else if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w_raw, u, nullptr, y, static_cast<float*>(saved), flg, 1, 0, nullptr, nullptr, nullptr, true)) return e;
+        if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w_raw, u, nullptr, y, static_cast<float*>(saved), flg, NB, TB, local, logdec, s32, decay)) return e;
+    } else if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w_raw, u, nullptr, y, static_cast<float*>(saved), flg, 1, 0, nullptr, nullptr, nullptr, decay)) return e;
     return launch_wkv6_fwd_chunk(st, W_HEAD, B, T, C, H, r, k, v, decay, u, nullptr, y, static_cast<float*>(saved), flg);
 }
 

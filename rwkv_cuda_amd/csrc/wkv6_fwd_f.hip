@@ -68,6 +68,8 @@ struct ArgsQ {
     float* blk_state;              // [B*H][NB][64][64]
     float* blk_decay;              // [B*H][NB][64]
     bool head_decay;               // wkv5: w is one raw decay per channel, [H][64], the same at every token
+    float* decay_out;              // wkv5: [2][C] fp32, exp(-exp(w)) and -exp(w), left for the two-sweep kernels and the backward
+    bool first_row;                // this workgroup has batch row 0 (and block 0): it writes decay_out
 };
 
 // ---------------------------------------------------------------------------------------------------- P waves
@@ -141,6 +143,12 @@ DEVINL void role_prep(SmemQ& S, const ArgsQ& a, const int lane, const int w, con
         }
         const bool bad = (-16.f * lamc[0] > RANGE_LIMIT * LOG2E) || (-16.f * lamc[1] > RANGE_LIMIT * LOG2E);
         any_exact = __ballot(bad) != 0ull;
+        if (!LOCAL && a.first_row && tp == 0) {
+            // the wrapper-side transform of wkv5_bf16/run.py:63-64, for whoever needs the decay in that form afterwards
+            const float e0 = -expf(bf_lo(x)), e1 = -expf(bf_hi(x));
+            *reinterpret_cast<float2*>(a.decay_out + h * N + ch0) = make_float2(expf(e0), expf(e1));
+            *reinterpret_cast<float2*>(a.decay_out + a.C + h * N + ch0) = make_float2(e0, e1);
+        }
     }
     auto prep = [&](const int c, auto PARTIAL) __attribute__((always_inline)) {
         const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B);
@@ -491,6 +499,7 @@ __global__ __launch_bounds__(NTQ) void wkv6_fwd_fused(const ArgsQ arg) {
     a.saved = arg.saved + (bh * nseg + t0 / (2 * L)) * (N * N);
     if (arg.s32 != nullptr) a.s32 = arg.s32 + bq * (N * N);
     if (arg.blk_state != nullptr) { a.blk_state = arg.blk_state + bq * (N * N); a.blk_decay = arg.blk_decay + bq * N; }
+    a.first_row = b == 0 && blk == 0;
     const int n = (a.T + L - 1) / L;
     // the quadrant t < 16 <= s of the tiles is never written and must read as zero
     for (int i = tid; i < static_cast<int>(sizeof(S.tile) / 4); i += NTQ) reinterpret_cast<uint32_t*>(&S.tile[0])[i] = 0;
@@ -528,9 +537,10 @@ __global__ __launch_bounds__(256) void wkv6_scan(const float* __restrict__ local
 
 int launch_wkv6_fwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
                           const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, float* saved, int* flags,
-                          int NB, int TB, float* blk_state, float* blk_decay, float* s32, bool head_decay) {
+                          int NB, int TB, float* blk_state, float* blk_decay, float* s32, float* decay_out) {
     ArgsQ a{};
-    a.head_decay = head_decay;
+    const bool head_decay = decay_out != nullptr;
+    a.head_decay = head_decay; a.decay_out = decay_out;
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y; a.saved = saved; a.flags = flags;
     a.NB = 1; a.TB = T;
     if (NB <= 1) {

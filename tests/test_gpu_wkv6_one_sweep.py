@@ -224,10 +224,13 @@ def test_wkv5_on_the_one_sweep_pair(lib, B, T, H):
     emu = O.emulate_wkv5_bf16(B, T, C, H, r, k, v, w, u, gy, hand=T >= 2000)
     d = [x.to(DEV) for x in (r, k, v, w, u, gy)]
     y = garbage((B, T, C), BF)
-    decay = torch.empty(2 * C, device=DEV, dtype=torch.float32)
+    decay = torch.full((2 * C,), float("nan"), device=DEV, dtype=torch.float32)
     nsv = lib.rwkv_wkv5s_saved_bytes(B, T, C, H)
     saved = torch.empty(nsv, device=DEV, dtype=torch.uint8).fill_(0x7f)
     call("rwkv_wkv5s_forward", DEV, B, T, C, H, *d[:5], y, decay, saved, nsv, 0)
+    # the forward leaves the wrapper-side transform of the decay (wkv5_bf16/run.py:63-64) for the backward
+    ew = -torch.exp(w.double().reshape(-1))
+    assert torch.allclose(decay[C:].cpu().double(), ew, rtol=2e-6, atol=0) and torch.allclose(decay[:C].cpu().double(), torch.exp(ew), rtol=2e-6, atol=0)
     gr, gk, gv = (garbage((B, T, C), BF) for _ in range(3))
     gw, gu = garbage((H, 64), BF), garbage((H, 64), BF)
     n = lib.rwkv_wkv5s_backward_workspace_bytes(B, T, C, H)
