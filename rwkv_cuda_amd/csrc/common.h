@@ -154,7 +154,8 @@ int launch_wkv6_bwd_a_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
 int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                             const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
                             const uint16_t* s0, const uint16_t* gy, uint16_t* gk, uint16_t* gv, uint16_t* gw,
-                            uint16_t* gs, const float* rdr, const int* only_flagged = nullptr);
+                            uint16_t* gs, const float* rdr, const int* only_flagged = nullptr,
+                            const uint16_t* sum_in = nullptr, uint16_t* sum_out = nullptr);
 // wkv6_bwd_f.hip: the whole backward in one reverse sweep from the states the forward saved (raw bf16 decay);
 // flags [B*H][8] names the (batch, head) pairs that have to be redone by the two sweeps above
 int launch_wkv6_bwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,

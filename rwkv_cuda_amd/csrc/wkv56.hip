@@ -1348,10 +1348,9 @@ int rwkv_wkv6f_backward_saved(void* stream, int B, int T, int C, int H, const rw
     } else if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, pu, gs, static_cast<const float*>(saved), flg)) return e;
     // (batch, head) pairs with a decay the mid-point factors cannot carry: the two sweeps redo them, all others return at once
     if (int e = launch_wkv6_bwd_a_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, gy, gr, pu, rdr, flg)) return e;
-    if (int e = launch_wkv6_bwd_b_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, gy, gk, gv, gw, gs, rdr, flg)) return e;
-    hipLaunchKernelGGL(bf16_batch_sum, dim3((C + 255) / 256), dim3(256), 0, st, B, C, pu, gu,
-                       static_cast<const uint16_t*>(nullptr), static_cast<uint16_t*>(nullptr));
-    return launch_status();
+    // (the second sweep's workgroups of batch row 0 first add the per-batch gu rows up: they are complete by then, and a
+    //  launch of its own for that costs as much as any other, about 5 us)
+    return launch_wkv6_bwd_b_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, gy, gk, gv, gw, gs, rdr, flg, pu, gu);
 }
 
 // ---- wkv5 (head size 64) on the one-sweep pair: the raw decay of a channel stands in for every token's, its gradient is

@@ -661,6 +661,12 @@ DEVINL void bwd_state_e(SmemB2& S, const ArgsB& a, const int tid, const size_t b
 template <int WMODE, bool SPLIT = false>
 __global__ __launch_bounds__(NTB) void wkv6_bwd_b_ws(const ArgsB a) {
     __shared__ SmemB2 S;
+    if (a.sum_out != nullptr && blockIdx.x < static_cast<unsigned>(a.H) && threadIdx.x < N) {
+        const int c = blockIdx.x * N + threadIdx.x;
+        float x = 0.f;
+        for (int b = 0; b < a.sum_B; ++b) x += bf2f(a.sum_in[static_cast<size_t>(b) * a.C + c]);
+        a.sum_out[c] = f2bf(x);
+    }
     if (skip_unflagged(a.only_flagged, blockIdx.x)) return;
     const int tid = threadIdx.x;
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
@@ -689,8 +695,9 @@ __global__ __launch_bounds__(NTB) void wkv6_bwd_b_ws(const ArgsB a) {
 int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                             const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
                             const uint16_t* s0, const uint16_t* gy, uint16_t* gk, uint16_t* gv, uint16_t* gw,
-                            uint16_t* gs, const float* rdr, const int* only_flagged) {
+                            uint16_t* gs, const float* rdr, const int* only_flagged, const uint16_t* sum_in, uint16_t* sum_out) {
     ArgsB a{};
+    a.sum_in = sum_in; a.sum_out = sum_out; a.sum_B = B;
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.gy = gy;
     a.gk = gk; a.gv = gv; a.gw = gw; a.gs = gs; a.rdr = const_cast<float*>(rdr); a.only_flagged = only_flagged;
     if (wmode == W_RAW) hipLaunchKernelGGL(wkv6_bwd_b_ws<W_RAW>, dim3(B * H), dim3(NTB), 0, st, a);

@@ -80,6 +80,12 @@ struct ArgsB {
     // when not null: [B*H][8]; a workgroup runs only if one of its eight words is not zero (the (batch, head) pairs that
     // the one-sweep backward has handed back)
     const int* only_flagged;
+    // when not null (sweep B only): out[c] = bf16(sum_b float(in[b][c])), the sum of per-batch-row partials over the batch
+    // (torch.sum(gu, 0) of the wrapper), done by the workgroups of batch row 0 before anything else.  `in` must be
+    // complete when the kernel starts: sweep B does not write it.
+    const uint16_t* sum_in;
+    uint16_t* sum_out;
+    int sum_B;
 };
 DEVINL bool skip_unflagged(const int* f, const int bh) {
     if (f == nullptr) return false;
