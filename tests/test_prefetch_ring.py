@@ -288,7 +288,14 @@ def test_one_sweep_kernels_leave_the_waits_to_the_compiler(fname):
     text = _read(fname)
     assert "asm volatile(\"global_load" not in text and "buffer_load" not in text
     assert not re.search(r"s_waitcnt vmcnt", re.sub(r"//.*", "", text))
-    start = text.index("for (int it0 = 0; it0 < nit; it0 += DEPTH)")
+    m = re.search(r"for \(int it0 = 0; it0 < nit; it0 \+= (DEPTH|TRIP)\)", text)
+    start = m.start()
+    if m.group(1) == "TRIP":
+        # a trip of the loop is a whole number of turns of the prefetch ring and of the registers kept for the finishing:
+        # both are indexed by compile-time constants, so nothing in flight is ever copied
+        depth, kept, trip = (int(re.search(rf"constexpr int {n} = (\d+);", text).group(1)) for n in ("DEPTH", "KEPT", "TRIP"))
+        assert trip % depth == 0 and trip % kept == 0
+        assert "static_for<TRIP>" in text and "% DEPTH" in text and "% KEPT" in text
     loop = text[start:text.index("__syncthreads();", start)]
     for call in re.findall(r"^\s*(?:if [^\n]*\))?\s*(fetch|stage_in)\(", loop, re.M):
         pass
