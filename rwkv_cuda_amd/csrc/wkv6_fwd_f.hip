@@ -420,7 +420,7 @@ DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
     const int g = lane >> 4, l16 = lane & 15;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     const lds_t sb = lds_of(&S);
-    lds_t b_nat = l16 * ROW_B + 16 * g;                                         // [token l16][channel 8 g] of a plane
+    lds_t b_nat = l16 * ROW_B + 8 * g;                                          // [token l16][channel 4 g] of a plane
     lds_t b_tw = l16 * TROW_B + 8 * g;                                          // [row l16][position 4 g] of a tile
     lds_t b_l = 4 * l16;
     // wave 0, 1, 2 -> quadrant (t, s) = (0,0) (1,0) (1,1); accumulator rows are s, lanes t
@@ -445,12 +445,14 @@ DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
         }
         if (!LOCAL && c < n && w < 3) {
             const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B), to = uniform_base(sb + TILE0 + (c & 1) * TILE_B);
+            // (in accumulator order, two 8-byte pieces: any order of the channels serves a contraction over them, and these
+            //  reads run at the LDS's rate where 16-byte reads of rows take 1.6 x as long)
             const lds_t ra = so + ta * 16 * ROW_B + b_nat, rb = so + tb * 16 * ROW_B + b_nat;
             bf16x8 kh[2], kl[2], rh[2], rl[2];
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
-                kh[ks] = ld_op(rb + O_KPH + 64 * ks); kl[ks] = ld_op(rb + O_KPL + 64 * ks);
-                rh[ks] = ld_op(ra + O_RPH + 64 * ks); rl[ks] = ld_op(ra + O_RPL + 64 * ks);
+                kh[ks] = ld_acc(rb + O_KPH + 64 * ks); kl[ks] = ld_acc(rb + O_KPL + 64 * ks);
+                rh[ks] = ld_acc(ra + O_RPH + 64 * ks); rl[ks] = ld_acc(ra + O_RPL + 64 * ks);
             }
             float d = 0.f;
             if (ta == tb) {
