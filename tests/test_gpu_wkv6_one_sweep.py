@@ -208,14 +208,19 @@ def test_one_sweep_rejects_bad_arguments(lib):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("B,T,H", [(2, 50, 2), (1, 700, 3), (3, 64, 1), (1, 4096, 2)])
-def test_wkv5_on_the_one_sweep_pair(lib, B, T, H):
+@pytest.mark.parametrize("B,T,H,fast", [(2, 50, 2, False), (1, 700, 3, False), (3, 64, 1, False), (1, 4096, 2, False), (2, 100, 3, True), (1, 300, 2, True)])
+def test_wkv5_on_the_one_sweep_pair(lib, B, T, H, fast):
     """wkv5 at head size 64 through rwkv_wkv5s_forward / rwkv_wkv5s_backward: the raw decay of a channel stands in for every
-    token's, gw is summed over the tokens inside the kernel and over the batch after it ((1, 700, 3) and (1, 4096, 2) run
-    as blocks with a scan)."""
-    print(f"\nwkv5 one sweep B={B} T={T} H={H}", flush=True)
+    token's, gw is summed over the tokens inside the kernel and over the batch after it ((1, 700, 3), (1, 4096, 2) and
+    (1, 300, 2) run as blocks with a scan).  fast: one channel of head 1 decays by more than e^-60 over 16 tokens, so the
+    kernels hand that head (its per-batch gw, gu rows included) to the two-sweep kernels."""
+    print(f"\nwkv5 one sweep B={B} T={T} H={H} fast={fast}", flush=True)
     C = H * 64
     r, k, v, w, u, gy = synth.wkv5_inputs(B, T, C, H, seed=340 + T)
+    if fast:
+        w = w.float()
+        w.view(-1)[64 + 17] = 1.5                                # exp(1.5) = 4.48 per token: e^-72 over 16 tokens
+        w = w.to(BF)
     ref = O.wkv5_grads(B, T, C, H, r, k, v, w, u, gy) if T < 2000 else None
     if ref is None:
         ref = list(O.wkv_grads_by_hand(B, T, C, H, r, k, v, w.reshape(1, 1, C).expand(B, T, C), u, gy, None, torch.float64))[:6]
@@ -237,6 +242,10 @@ def test_wkv5_on_the_one_sweep_pair(lib, B, T, H):
     ws = torch.empty(n, device=DEV, dtype=torch.uint8).fill_(0x7f)
     call("rwkv_wkv5s_backward", DEV, B, T, C, H, d[0], d[1], d[2], d[3], decay, d[4], d[5], gr, gk, gv, gw, gu, saved, nsv, ws, n, 0)
     torch.cuda.synchronize()
+    # the words in which the kernels flag the (batch, head) pairs they hand back, after the two-sweep kernels' own workspace
+    off = (lib.rwkv_wkv5raw_backward_workspace_bytes(B, T, C, H) + 15) // 16 * 16
+    flags = ws[off:off + B * H * 8 * 4].view(torch.int32).view(B * H, 8)
+    assert int((flags != 0).any(1).sum()) == (B if fast else 0)
     for name, a, e, g in zip(["y", "gr", "gk", "gv", "gw", "gu"], ref, emu, [y, gr, gk, gv, gw, gu]):
         assert torch.isfinite(g.float()).all(), name
         assert_no_worse("wkv5 " + name, a, e, g)
