@@ -331,8 +331,8 @@ __global__ __launch_bounds__(NT, 2) void rwkv7c_fwd(const Args7c p) {
 //                of the contractions over the value channel, U dS and V dS, next to S0 of the chunk loaded from `s` in the same
 //                layout (dW S0, dY S0); they make dA', dR', dB', dK' (register v <-> token 4 g + v, lane <-> key channel), scale
 //                them, scan the decay gradient and park the results; they run one phase behind the A waves.
-//   waves 8..11 ("P"): fetch the next chunk's seven input rows and `sa`, convert them, build the operand planes
-//                (double-buffered) and store the finished gradient rows (LDS-staged, whole rows).
+//   waves 8..11 ("P"): fetch the seven input rows and `sa` two chunks ahead, convert them and build the operand planes
+//                (double-buffered).  The finished gradient rows leave LDS-staged, as whole rows, through A waves 2 and 3.
 // The gradient state is therefore kept twice (both copies get the same update); nothing is transposed through LDS.
 constexpr int NTB = 12 * 64;       // waves 0..3 role A, 4..7 role B, 8..11 role P
 
@@ -379,7 +379,8 @@ DEVINL void causal_tile(const float (*X)[PS], const float (*Y)[PS], float (*Tl)[
 //          phase 1                          | phase 2                                   | phase 3
 //   A:     tile, M, tile-free parts of (i)   | dU, dW, dV, state update of (i)           | dAB, dAK of (i)
 //   B:     tile parts + epilogue of (i - 1)  | dY S0, U dS, V dS, dRB, dRK of (i)        | dW S0, state update of (i)
-//   P:     raw inputs -> decay sums (i + 1)  | row stores (i - 1); factors, planes (i+1) | -
+//   P:     raw inputs -> decay sums (i + 1)  | factors, planes (i + 1)                   | -
+// (the rows of visit i - 1 leave in phase 3, through the two A waves that have no tile there)
 
 // ---- role P: elementwise preparation (lane = channel, tokens 4 wp + e) one visit ahead, and the row-wise output stores
 struct Prep7 { uint32_t nx[7][4]; float nsa[4]; };
@@ -451,31 +452,39 @@ DEVINL void bwd_store_rows(const SmemCB& S, int vbuf, const Args7c& p, size_t ro
 }
 DEVINL void bwd_role_p(SmemCB& S, const Args7c& p, int tid, int w, size_t tok0, int nch, int H, int h) {
     const int lane = tid & 63, wp = w - 8, tp = tid - 8 * 64;
-    Prep7 x;
+    // Raw rows are asked for two visits before they are converted (one visit, of which only two phases lie between the
+    // request and the use, is less than the memory system takes under load: the A and B waves then waited for the P waves
+    // at two of the three barriers of every visit).  Two register sets take turns; the chunk index is clamped instead of
+    // the request being skipped, so that every visit issues the same loads and the waits count the same.
+    Prep7 x[2];
     Conv7 y;
-    bwd_fetch(p, x, tok0 + static_cast<size_t>(nch - 1) * CL, wp, lane, H, h);
-    bwd_convert(S.pl[0], x, y, wp, lane);            // visit 0, before the loop
-    if (nch > 1) bwd_fetch(p, x, tok0 + static_cast<size_t>(nch - 2) * CL, wp, lane, H, h);
+    auto row_of = [&](int visit) { const int c = nch - 1 - visit; return tok0 + static_cast<size_t>(c > 0 ? c : 0) * CL; };
+    bwd_fetch(p, x[0], row_of(0), wp, lane, H, h);
+    bwd_fetch(p, x[1], row_of(1), wp, lane, H, h);
+    bwd_convert(S.pl[0], x[0], y, wp, lane);          // visit 0, before the loop
+    bwd_fetch(p, x[0], row_of(2), wp, lane, H, h);
     __syncthreads();
     bwd_planes(S.pl[0], y, wp, lane);
     __syncthreads();
-    for (int i = 0; i < nch; ++i) {                  // visit i is chunk nch - 1 - i
+    auto visit = [&](const int i, auto Z) __attribute__((always_inline)) {     // visit i is chunk nch - 1 - i
+        constexpr int z = decltype(Z)::value;        // the set that holds visit i + 1
         const bool next = i + 1 < nch;
-        if (next) {
-            bwd_convert(S.pl[(i + 1) & 1], x, y, wp, lane);
-            if (i + 2 < nch) bwd_fetch(p, x, tok0 + static_cast<size_t>(nch - 3 - i) * CL, wp, lane, H, h);
-        }
+        if (next) bwd_convert(S.pl[(i + 1) & 1], x[z], y, wp, lane);
+        bwd_fetch(p, x[z], row_of(i + 3), wp, lane, H, h);
         __syncthreads();
-        if (i > 0) bwd_store_rows(S, (i - 1) & 1, p, tok0 + static_cast<size_t>(nch - i) * CL, tp, H, h);
         if (next) bwd_planes(S.pl[(i + 1) & 1], y, wp, lane);
         __syncthreads();
         __syncthreads();
+    };
+    for (int i = 0; i < nch; i += 2) {
+        visit(i, std::integral_constant<int, 1>{});
+        if (i + 1 < nch) visit(i + 1, std::integral_constant<int, 0>{});
     }
     __syncthreads();                                 // role B finishes the last chunk
     bwd_store_rows(S, (nch - 1) & 1, p, tok0, tp, H, h);
 }
 
-DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, int nch) {
+DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, int nch, size_t tok0, int H, int h) {
     const int lane = tid & 63, q = w & 3, l16 = lane & 15, g = lane >> 4;
     const int own = 16 * q + l16;                    // value channel i of this lane's column
     f32x4 dS[4];                                     // dS[i = own][j = 16 jt + 4 g + v]
@@ -539,6 +548,14 @@ DEVINL void bwd_role_a(SmemCB& S, const Args7c& p, int tid, int w, size_t bh, in
         __syncthreads();
         // ---------------------------------------------------------------- phase 3: dAB, dAK (they need dW)
         if (q < 2) causal_tile(S.dW, q == 0 ? O.U : O.V, q == 0 ? S.dAB : S.dAK, true, l16, g);
+        else if (i > 0) {
+            // The two waves without a tile here carry the finished rows of the visit before to global memory (parked by the
+            // B waves in phase 1, dv by this role one visit earlier; both stay as they are until the next visit): the P
+            // waves, for which this was a third of a phase that everybody waits for, keep to loads.
+            const int tp = tid - 2 * 64;
+            bwd_store_rows(S, (i - 1) & 1, p, tok0 + static_cast<size_t>(nch - i) * CL, tp, H, h);
+            bwd_store_rows(S, (i - 1) & 1, p, tok0 + static_cast<size_t>(nch - i) * CL, tp + 128, H, h);
+        }
         __syncthreads();
     }
     __syncthreads();
@@ -695,7 +712,7 @@ __global__ __launch_bounds__(NTB, 3) void rwkv7c_bwd(const Args7c p) {
     const size_t bh = static_cast<size_t>(b) * p.H + h;
     const size_t tok0 = static_cast<size_t>(b) * p.T;
     const int nch = p.T / CL;
-    if (w < 4) bwd_role_a(S, p, tid, w, bh, nch);
+    if (w < 4) bwd_role_a(S, p, tid, w, bh, nch, tok0, p.H, h);
     else if (w < 8) bwd_role_b(S, p, tid, w, bh, nch);
     else bwd_role_p(S, p, tid, w, tok0, nch, p.H, h);
 }
