@@ -116,6 +116,7 @@ DEVINL float exp_acc(float x) {
 // Every exponent is formed as a direct sum of the lam between the token and its reference point (never as a difference of
 // two long cumulative sums), so its absolute error -- the factor's relative error -- scales with the exponent itself.
 struct Factors { float ea[4], er[4], eb[4], es[4], ee[4]; };   // e^{c_t - c_m}, e^{c_{t+1} - c_m}, e^{c_m - c_{t+1}}, e^{c_t}, e^{c_L - c_{t+1}}
+template <int E0 = 0, int E1 = 4>
 DEVINL Factors chunk_factors(const float (&lam)[4], const float (*part)[N], int q, int j, float& cm_out, float& cl_out) {
     const float p0 = part[0][j], p1 = part[1][j], p2 = part[2][j], p3 = part[3][j];
     const float cm = p0 + p1, cl = (p0 + p1) + (p2 + p3);
@@ -129,9 +130,9 @@ DEVINL Factors chunk_factors(const float (&lam)[4], const float (*part)[N], int 
     for (int e = 0; e < 4; ++e) pre[e + 1] = pre[e] + lam[e];
 #pragma unroll
     for (int e = 3; e >= 0; --e) suf[e] = suf[e + 1] + lam[e];
-    Factors f;
+    Factors f = {};
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = E0; e < E1; ++e) {                // (the exponentials of the tokens asked for; the sums above are cheap)
         // c_t - c_m and c_{t+1} - c_m
         const float xt = q < 2 ? -(suf[e] + gap) : gap + pre[e];
         const float xn = q < 2 ? -(suf[e + 1] + gap) : gap + pre[e + 1];
@@ -412,12 +413,13 @@ DEVINL void bwd_convert(PlanesB& O, const Prep7& x, Conv7& y, int wp, int lane) 
     O.part[wp][lane] = W_SCALE * ((y.sg[0] + y.sg[1]) + (y.sg[2] + y.sg[3]));
 }
 // second half (after a barrier): the in-chunk factors and every plane
+template <int E0 = 0, int E1 = 4>
 DEVINL void bwd_planes(PlanesB& O, const Conv7& y, int wp, int lane) {
     float cm, cl;
     const float lam[4] = {W_SCALE * y.sg[0], W_SCALE * y.sg[1], W_SCALE * y.sg[2], W_SCALE * y.sg[3]};
-    const Factors f = chunk_factors(lam, O.part, wp, lane, cm, cl);
+    const Factors f = chunk_factors<E0, E1>(lam, O.part, wp, lane, cm, cl);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = E0; e < E1; ++e) {
         const int t = 4 * wp + e;
         auto in = [&](int k) __attribute__((always_inline)) { return (e & 1) ? bf_hi(y.pk[k][e >> 1]) : bf_lo(y.pk[k][e >> 1]); };
         const float rr = in(0), kk = in(1), vv = in(2), aa = in(3), bb = in(4), gg = in(5);
@@ -436,7 +438,7 @@ DEVINL void bwd_planes(PlanesB& O, const Conv7& y, int wp, int lane) {
         O.ER[t][lane] = f.er[e];
         O.DWF[t][lane] = W_SCALE * y.sg[e] * (1.f - y.sg[e]);
     }
-    if (wp == 0) { O.d1[lane] = exp_acc(cm); O.d2[lane] = exp_acc(cl - cm); O.dec[lane] = exp_acc(cl); }
+    if (E0 == 0 && wp == 0) { O.d1[lane] = exp_acc(cm); O.d2[lane] = exp_acc(cl - cm); O.dec[lane] = exp_acc(cl); }
 }
 // da dr db dk dw (and dv) of one chunk leave their parking places as whole rows (256 threads, four channels each)
 DEVINL void bwd_store_rows(const SmemCB& S, int vbuf, const Args7c& p, size_t row0, int tp, int H, int h) {
@@ -472,8 +474,11 @@ DEVINL void bwd_role_p(SmemCB& S, const Args7c& p, int tid, int w, size_t tok0, 
         if (next) bwd_convert(S.pl[(i + 1) & 1], x[z], y, wp, lane);
         bwd_fetch(p, x[z], row_of(i + 3), wp, lane, H, h);
         __syncthreads();
-        if (next) bwd_planes(S.pl[(i + 1) & 1], y, wp, lane);
+        // the planes of two of this wave's four tokens in phase 2, the other two in phase 3, in which these waves used to idle
+        // while everybody waited for them in phase 2 (nothing reads these planes before the next visit)
+        if (next) bwd_planes<0, 2>(S.pl[(i + 1) & 1], y, wp, lane);
         __syncthreads();
+        if (next) bwd_planes<2, 4>(S.pl[(i + 1) & 1], y, wp, lane);
         __syncthreads();
     };
     for (int i = 0; i < nch; i += 2) {
