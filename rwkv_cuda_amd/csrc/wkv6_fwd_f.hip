@@ -301,10 +301,21 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
     }
     __syncthreads();                       // iterations 0 and 1: nothing prepared yet
     __syncthreads();
-    // d1 and R' of a chunk have been in LDS for a whole iteration when its turn comes: they are asked for at the end of
-    // the chunk before, so that the scaling of the state can start right behind the barrier
-    float dq[4];
-    bf16x8 rh[2][2], rl[2][2];
+    // The factors, R' and v of a chunk have been in LDS for a whole iteration when its turn comes: they are asked for at
+    // the end of the chunk before, so that the scaling of the state and the first products can start right behind the
+    // barrier, when every wave of the workgroup is asking the LDS for something (only the A tile is made that late).
+    float dq[4], de[4], d2[4];
+    bf16x8 rh[2][2], rl[2][2], vop;
+    // (in two parts, each where the registers it fills have had their last use in the current chunk)
+    auto ahead_late = [&](const int c) __attribute__((always_inline)) {
+        const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            de[q] = lds_ld<float>(so + O_DEC + 64 * q + b_g);
+            d2[q] = lds_ld<float>(so + O_D2 + 64 * q + b_g);
+        }
+        vop = ld_tr(so + O_V + 32 * w + b_tr, ROW_B);                           // lane = value channel 16w + l16, K = tokens
+    };
     auto ahead = [&](const int c) __attribute__((always_inline)) {
         const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B);
 #pragma unroll
@@ -320,6 +331,7 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
         }
     };
     ahead(0);
+    ahead_late(0);
 #pragma unroll 1
     for (int c = 0; c < n; ++c) {
         opaque(b_acc); opaque(b_tr); opaque(b_natt); opaque(b_g); opaque(b_ss);
@@ -334,15 +346,8 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
         // ------------------------------------------------------------ batch 1: d1, R' (natural rows), v and the A tile
         // per-channel factors: a lane holds the one of channel 16 tile + 4 g + (l16 & 3), a 4-byte read that all rows of
         // four lanes share; the products below take lane v of the 16-lane row inside the multiply (row_newbcast)
-        float de[4], d2[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            de[q] = lds_ld<float>(so + O_DEC + 64 * q + b_g);
-            d2[q] = lds_ld<float>(so + O_D2 + 64 * q + b_g);
-        }
         // (LOCAL: only the state is wanted, everything that serves y is left out)
-        // (v with the tokens along K and the A tile by rows as well: they arrive while the state is scaled and split)
-        const bf16x8 vop = ld_tr(so + O_V + 32 * w + b_tr, ROW_B);              // lane = value channel 16w + l16, K = tokens
+        // (the A tile by rows: it arrives while the state is scaled and split)
         bf16x8 ah[2], al[2];
 #pragma unroll
         for (int tt = 0; tt < (LOCAL ? 0 : 2); ++tt) { ah[tt] = ld_op(to + T_AH + tt * 16 * TROW_B + b_natt); al[tt] = ld_op(to + T_AL + tt * 16 * TROW_B + b_natt); }
@@ -405,6 +410,8 @@ DEVINL void role_state(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
                 fmac_bc<v>(x, d2[tl], U[tl][v]);
                 St[tl][v] = x;
             });
+        __builtin_amdgcn_sched_barrier(0);
+        ahead_late(c + 1);
         __syncthreads();
     }
     for (int it = n + 2; it < nit; ++it) __syncthreads();      // the P waves store the last y
