@@ -38,11 +38,11 @@ FLAGS = 0                      # RWKV_FLAG_SWEEPS when --algo sweeps: passed per
 # by kernel label at the headline shape; None = not measured for the current kernels.
 TRAFFIC_MEASURED = {
     # profiles/wkv6_fused_kernels_B8_T4096_C2048.md  (FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB)
-    "wkv6_fwd_fused (keeps states)": 537.2e6 + 402.7e6,
-    "wkv6_bwd_fused (+ gu batch sum)": 940.6e6 + 537.7e6,
+    "wkv6_fwd_fused (keeps states)": 537.2e6 + 335.6e6,
+    "wkv6_bwd_fused (+ gu batch sum)": 872.9e6 + 536.9e6,
     # profiles/wkv5_fused_kernels_B8_T4096_C2048.md
-    "wkv6_fwd_fused<head decay> (keeps states)": 403.0e6 + 402.7e6,
-    "wkv6_bwd_fused<head decay> (+ batch sums)": 807.2e6 + 404.7e6,
+    "wkv6_fwd_fused<head decay> (keeps states)": 402.9e6 + 335.6e6,
+    "wkv6_bwd_fused<head decay> (+ batch sums)": 738.7e6 + 402.7e6,
     # profiles/wkv5_ws_kernels_B8_T4096_C2048.md
     "wkv6_fwd_ws<head decay>": 403e6 + 134e6,
     "wkv6_bwd_a_ws<head decay>": 548e6 + 533e6,

@@ -291,8 +291,8 @@ int rwkv_wkv6f_backward(void* stream, int B, int T, int C, int H,
                         rwkv_bf16* gs, void* workspace, size_t workspace_bytes, unsigned flags);
 
 /* WKV_6 (s = gs = NULL) and WKV_6STATE with states handed from the forward to the backward.  The forward also writes,
- * into `saved` (rwkv_wkv6f_saved_bytes; fp32 [B*H][ceil(T/64)][64][64]), the state entering every 64th token; the backward
- * reads them and produces every gradient in ONE reverse sweep instead of two sweeps and an fp32 [B,T,C] hand-over.  The
+ * into `saved` (rwkv_wkv6f_saved_bytes; [B*H][ceil(T/64)] states of 64 x 64 values in 12 KB each: fp32 rounded to 24
+ * bits, in an order private to the two kernels), the state entering every 64th token; the backward reads them and produces every gradient in ONE reverse sweep instead of two sweeps and an fp32 [B,T,C] hand-over.  The
  * reference's wkv6 operators keep nothing between their two calls; the precedents are its rwkv7 forward, which keeps `s`
  * and `sa` for its backward (rwkv7_statepassing_clampw.cu:67-73), and wkv5_bf16/cuda/wkv5_cuda_v3.cu:12-30 (chunk states).
  * Results are those of the pair above to the rounding of the outputs.  With another head size than 64, or with

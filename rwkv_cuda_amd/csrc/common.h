@@ -137,13 +137,13 @@ inline int launch_status() {
 // wkv6_chunk.hip: chunked MFMA kernels.  wmode: 1 = fp32 ew [B,T,C], 2 = raw bf16 w.
 int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                           const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
-                          const uint16_t* s0, uint16_t* y, float* saved = nullptr, const int* only_flagged = nullptr);
+                          const uint16_t* s0, uint16_t* y, char* saved = nullptr, const int* only_flagged = nullptr);
 // wkv6_fwd_f.hip: the forward that goes with wkv6_bwd_f.hip (raw bf16 decay, head size 64): y and the state entering
 // every second chunk; flags [B*H][8] names the (batch, head) pairs that have to be redone by the kernel above
 // NB > 1: the sequences in NB blocks of TB tokens, one workgroup per (batch, head, block): local states, a scan, the outputs
 // (blk_state, s32: [B*H*NB][64][64] floats each, blk_decay: [B*H*NB][64]; flags cleared by the caller)
 int launch_wkv6_fwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
-                          const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, float* saved, int* flags,
+                          const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, char* saved, int* flags,
                           int NB = 1, int TB = 0, float* blk_state = nullptr, float* blk_decay = nullptr, float* s32 = nullptr,
                           float* decay_out = nullptr);
 int launch_wkv6_scan_reverse(hipStream_t st, int BH, int NB, const float* local, const float* logdec, float* out);
@@ -160,7 +160,7 @@ int launch_wkv6_bwd_b_chunk(hipStream_t st, int wmode, int B, int T, int C, int 
 // flags [B*H][8] names the (batch, head) pairs that have to be redone by the two sweeps above
 int launch_wkv6_bwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
                           const uint16_t* w, const uint16_t* u, const uint16_t* gy, uint16_t* gr, uint16_t* gk, uint16_t* gv,
-                          uint16_t* gw, uint16_t* gu, uint16_t* gs, const float* saved, int* flags,
+                          uint16_t* gw, uint16_t* gu, uint16_t* gs, const char* saved, int* flags,
                           int NB = 1, int TB = 0, float* blk_ds = nullptr, float* blk_decay = nullptr, float* ds32 = nullptr,
                           float* gu32 = nullptr, uint16_t* gwp = nullptr, float* gw32 = nullptr);
 // gwp != nullptr: wkv5 (w is the raw decay per channel [H][64]; its gradient per batch row goes to gwp [B][C], gw is not written)

@@ -1261,7 +1261,7 @@ int scan_blocks(int B, int T, int H, int* TB, unsigned flags = 0u) {
 }
 size_t saved_states_bytes(int B, int T, int H) {
     const size_t nchunks = (static_cast<size_t>(T) + 31) / 32, nseg = (nchunks + 1) / 2;
-    return static_cast<size_t>(B) * H * nseg * 64 * 64 * sizeof(float);
+    return static_cast<size_t>(B) * H * nseg * 64 * 64 * 3;          // 24 bits per value (SAVED_STATE_B, wkv6_chunk.h)
 }
 size_t scan_scratch_bytes(int B, int T, int H) {           // local results and scanned states (fp32 [64][64]) and log decays per block
     int TB;
@@ -1300,9 +1300,9 @@ int rwkv_wkv6f_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16
         float* s32 = local + nq * 64 * 64;
         float* logdec = s32 + nq * 64 * 64;
         zero_words(st, flg, static_cast<size_t>(B) * H * 8);
-        if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved), flg, NB, TB, local, logdec, s32)) return e;
-    } else if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved), flg)) return e;
-    return launch_wkv6_fwd_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, y, static_cast<float*>(saved), flg);
+        if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w, u, s, y, static_cast<char*>(saved), flg, NB, TB, local, logdec, s32)) return e;
+    } else if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w, u, s, y, static_cast<char*>(saved), flg)) return e;
+    return launch_wkv6_fwd_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, y, static_cast<char*>(saved), flg);
 }
 
 size_t rwkv_wkv6f_backward_saved_workspace_bytes(int B, int T, int C, int H) {
@@ -1343,9 +1343,9 @@ int rwkv_wkv6f_backward_saved(void* stream, int B, int T, int C, int H, const rw
         float* logdec = ds32 + nq * 64 * 64;
         float* gu32 = logdec + nq * 64;
         zero_words(st, flg, static_cast<size_t>(B) * H * 8);
-        if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, pu, gs, static_cast<const float*>(saved), flg,
+        if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, pu, gs, static_cast<const char*>(saved), flg,
                                           NB, TB, local, logdec, ds32, gu32)) return e;
-    } else if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, pu, gs, static_cast<const float*>(saved), flg)) return e;
+    } else if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, pu, gs, static_cast<const char*>(saved), flg)) return e;
     // (batch, head) pairs with a decay the mid-point factors cannot carry: the two sweeps redo them, all others return at once
     if (int e = launch_wkv6_bwd_a_chunk(st, W_RAW, B, T, C, H, r, k, v, w, u, s, gy, gr, pu, rdr, flg)) return e;
     // (the second sweep's workgroups of batch row 0 first add the per-batch gu rows up: they are complete by then, and a
@@ -1380,9 +1380,9 @@ int rwkv_wkv5s_forward(void* stream, int B, int T, int C, int H, const rwkv_bf16
         float* s32 = local + nq * 64 * 64;
         float* logdec = s32 + nq * 64 * 64;
         zero_words(st, flg, static_cast<size_t>(B) * H * 8);
-        if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w_raw, u, nullptr, y, static_cast<float*>(saved), flg, NB, TB, local, logdec, s32, decay)) return e;
-    } else if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w_raw, u, nullptr, y, static_cast<float*>(saved), flg, 1, 0, nullptr, nullptr, nullptr, decay)) return e;
-    return launch_wkv6_fwd_chunk(st, W_HEAD, B, T, C, H, r, k, v, decay, u, nullptr, y, static_cast<float*>(saved), flg);
+        if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w_raw, u, nullptr, y, static_cast<char*>(saved), flg, NB, TB, local, logdec, s32, decay)) return e;
+    } else if (int e = launch_wkv6_fwd_fused(st, B, T, C, H, r, k, v, w_raw, u, nullptr, y, static_cast<char*>(saved), flg, 1, 0, nullptr, nullptr, nullptr, decay)) return e;
+    return launch_wkv6_fwd_chunk(st, W_HEAD, B, T, C, H, r, k, v, decay, u, nullptr, y, static_cast<char*>(saved), flg);
 }
 
 size_t rwkv_wkv5s_backward_workspace_bytes(int B, int T, int C, int H) {
@@ -1423,9 +1423,9 @@ int rwkv_wkv5s_backward(void* stream, int B, int T, int C, int H, const rwkv_bf1
         float* gu32 = logdec + nq * 64;
         float* gw32 = gu32 + static_cast<size_t>(NB) * B * C;
         zero_words(st, flg, static_cast<size_t>(B) * H * 8);
-        if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w_raw, u, gy, gr, gk, gv, nullptr, pu, nullptr, static_cast<const float*>(saved), flg,
+        if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w_raw, u, gy, gr, gk, gv, nullptr, pu, nullptr, static_cast<const char*>(saved), flg,
                                           NB, TB, local, logdec, ds32, gu32, pw, gw32)) return e;
-    } else if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w_raw, u, gy, gr, gk, gv, nullptr, pu, nullptr, static_cast<const float*>(saved), flg,
+    } else if (int e = launch_wkv6_bwd_fused(st, B, T, C, H, r, k, v, w_raw, u, gy, gr, gk, gv, nullptr, pu, nullptr, static_cast<const char*>(saved), flg,
                                              1, 0, nullptr, nullptr, nullptr, nullptr, pw, nullptr)) return e;
     // heads whose decay the mid-point factors cannot carry: the two sweeps redo them (their per-batch gw, gu rows included)
     const float* ew = decay + C;

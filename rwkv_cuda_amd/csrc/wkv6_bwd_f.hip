@@ -82,7 +82,7 @@ struct ArgsG {
     const uint16_t *r, *k, *v, *u, *gy;
     const void* w;
     uint16_t *gr, *gk, *gv, *gw, *gu, *gs;
-    const float* saved;            // [B*H][ceil(n/2)][64][64]: the forward state entering every even chunk
+    const char* saved;             // [B*H][ceil(n/2)] saved states (SAVED_STATE_B bytes each): the forward state entering every even chunk
     int* flags;                    // [B*H][8]
     // Sequences cut into NB blocks of TB tokens (a multiple of 64), one workgroup per (batch, head, block), see
     // wkv6_fwd_f.hip.  LOCAL = true leaves in blk_ds the gradient state that a block builds from nothing, going down from
@@ -110,6 +110,26 @@ DEVINL void load_state(const float* __restrict__ p, const uint32_t lo, f32x4 (&x
         const char* q = reinterpret_cast<const char*>(p + 16 * tl * N) + lo;
 #pragma unroll
         for (int v = 0; v < 4; ++v) x[tl][v] = *reinterpret_cast<const float*>(q + v * (4 * N));
+    }
+}
+
+// A saved state (format: wkv6_chunk.h) in the same layout, for SD wave w: three 16-byte loads per lane (p: the state,
+// wave-uniform; lo = 16 * lane), kept as loaded while they are in flight and expanded where the state is first needed.
+struct SavedRaw { u32x4 ha, hb, lo; };
+DEVINL void fetch_saved(const char* __restrict__ p, const int w, const uint32_t lo, SavedRaw& q) {
+    const char* hi = p + 2048 * w, *lw = p + SAVED_LO_B + 1024 * w;
+    q.ha = *reinterpret_cast<const u32x4*>(hi + lo);
+    q.hb = *reinterpret_cast<const u32x4*>(hi + 1024 + lo);
+    q.lo = *reinterpret_cast<const u32x4*>(lw + lo);
+}
+DEVINL void expand_saved(const SavedRaw& q, f32x4 (&x)[4]) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        // bytes 3, 2: the element's upper half; byte 1: its low byte; byte 0: zero
+        constexpr uint32_t ZERO = 0x0cu;
+        const uint32_t sel = ((5u + 2u * (e & 1)) << 24) | ((4u + 2u * (e & 1)) << 16) | (static_cast<uint32_t>(e & 3) << 8) | ZERO;
+        const uint32_t h = e < 8 ? q.ha[(e & 7) >> 1] : q.hb[(e & 7) >> 1];
+        x[e >> 2][e & 3] = __uint_as_float(__builtin_amdgcn_perm(h, q.lo[e >> 2], sel));
     }
 }
 
@@ -409,7 +429,7 @@ template <int WMODE, bool LOCAL>
 DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const size_t bh, const int n, const int nit) {
     const int g = lane >> 4, l16 = lane & 15, j = 16 * w + l16;
     const int nseg = (n + 1) / 2;
-    const float* __restrict__ sv = a.saved;                                     // the saved states of this block
+    const char* __restrict__ sv = a.saved;                                      // the saved states of this block
     if constexpr (LOCAL) {                 // only the E waves have work
         for (int it = 0; it < nit; ++it) __syncthreads();
         return;
@@ -417,7 +437,8 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     const lds_t sb = lds_of(&S);
     // per-lane address parts
-    uint32_t b_sv = 4 * (4 * g * N + j);                                        // [value channel 4 g][key channel j] of a saved state (bytes)
+    uint32_t b_sv = 4 * (4 * g * N + j);                                        // [value channel 4 g][key channel j] of an fp32 state (bytes)
+    uint32_t b_q = 16 * lane;                                                   // this lane's pieces of a saved state
     lds_t b_acc = l16 * ROW_B + 8 * g;                                          // [token l16][channel 4 g] of a plane
     lds_t b_tr = ((8 * g + (l16 >> 2)) * PS + 2 * (l16 & 3)) * 4;               // transposing read of a plane, rows 8 g ..
     lds_t b_trt = ((8 * g + (l16 >> 2)) * TQ + 2 * (l16 & 3)) * 4;              // the same of a tile
@@ -425,14 +446,17 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
     lds_t b_xz = l16 * XROW_B + 16 * g;                                         // [token l16][channel 4 g] of X / Z
     lds_t b_j = 4 * l16;
     f32x4 D[4] = {zero4, zero4, zero4, zero4};
-    f32x4 Sa[4];                           // the saved state of the segment at hand (chunks 2 sg, 2 sg + 1)
+    SavedRaw Sq;                           // the saved state of the segment at hand (chunks 2 sg, 2 sg + 1), as loaded: twelve
+                                           // registers instead of sixteen, expanded where a chunk uses it
+    float pa = 0.f;                        // P = sum_i dS S of an even chunk, this lane's part
 
     // Operands are fetched in batches, each issued as a whole before anything waits for it (the scheduling barriers keep
     // the batches apart): a wave then waits for LDS a few times per chunk instead of once per product.
     // X^T[j][t] = (S d1)^T GY^T + K'^T Bm^T for chunk c; S = Sa (even chunk) or one update of it (odd chunk)
     auto part_x = [&](const int c) __attribute__((always_inline)) {
         const lds_t so = uniform_base(sb + SLOT0 + (c % 3) * SLOT_B), to = uniform_base(sb + TILE0 + (c & 1) * TILE_B), xo = uniform_base(sb + XZ0 + (c & 1) * 2 * XZ_B + 64 * w);
-        f32x4 Sc[4];
+        f32x4 Sc[4], Sa[4];
+        expand_saved(Sq, Sa);
         if (c & 1) {
             // state entering the odd chunk: S dec + d2 V^T K' with the chunk below
             const lds_t qo = uniform_base(sb + SLOT0 + ((c - 1) % 3) * SLOT_B);
@@ -450,8 +474,14 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
                 for (int v = 0; v < 4; ++v) Sc[tl][v] = fmaf(Sa[tl][v], qdec, qd2 * U[v]);
             }
         } else {
+            // anchor: P = sum_i dS S with the saved state entering this chunk (D has taken the chunk in already)
+            pa = 0.f;
 #pragma unroll
-            for (int tl = 0; tl < 4; ++tl) Sc[tl] = Sa[tl];
+            for (int tl = 0; tl < 4; ++tl) {
+                Sc[tl] = Sa[tl];
+#pragma unroll
+                for (int v = 0; v < 4; ++v) pa = fmaf(D[tl][v], Sa[tl][v], pa);
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         const float d1 = lds_ld<float>(so + O_D1 + 64 * w + b_j);
@@ -534,7 +564,9 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
         load_state(a.ds32, b_sv, D);       // the gradient state that enters the block from above
         if (a.above) {
             // P there, with the forward state at the end of the block (the first saved state of the block above)
-            load_state(sv + static_cast<size_t>(n >> 1) * (N * N), b_sv, Sa);
+            fetch_saved(sv + static_cast<size_t>(n >> 1) * SAVED_STATE_B, w, b_q, Sq);
+            f32x4 Sa[4];
+            expand_saved(Sq, Sa);
             float p = 0.f;
 #pragma unroll
             for (int tl = 0; tl < 4; ++tl)
@@ -544,28 +576,22 @@ DEVINL void role_sd(SmemG& S, const ArgsG& a, const int lane, const int w, const
             if (g == 0) lds_st<float>(sb + PEX0 + ((n >> 1) & 1) * (4 * N) + 64 * w + b_j, p);
         }
     }
-    load_state(sv + static_cast<size_t>(nseg - 1) * (N * N), b_sv, Sa);
+    fetch_saved(sv + static_cast<size_t>(nseg - 1) * SAVED_STATE_B, w, b_q, Sq);
     __syncthreads();                       // iterations 0 and 1: nothing prepared yet
     __syncthreads();
 #pragma unroll 1
     for (int c = n - 1; c >= 0; --c) {
-        opaque(b_acc); opaque(b_tr); opaque(b_trt); opaque(b_natt); opaque(b_xz); opaque(b_j); opaque(b_sv);
-        // Sa of an odd chunk was asked for at the end of the last iteration: what does not need it goes first
+        opaque(b_acc); opaque(b_tr); opaque(b_trt); opaque(b_natt); opaque(b_xz); opaque(b_j); opaque(b_q);
+        // the state of an odd chunk's segment was asked for at the end of the last iteration: what does not need it goes first
         part_z(c);
         __builtin_amdgcn_sched_barrier(0);
         part_x(c);
         __builtin_amdgcn_sched_barrier(0);
         if (!(c & 1)) {
-            // anchor: P = sum_i dS S with the saved state entering this chunk
-            float p = 0.f;
-#pragma unroll
-            for (int tl = 0; tl < 4; ++tl)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) p = fmaf(D[tl][v], Sa[tl][v], p);
-            p = allreduce_rows(p);
+            const float p = allreduce_rows(pa);
             if (g == 0) lds_st<float>(sb + PEX0 + ((c >> 1) & 1) * (4 * N) + 64 * w + b_j, p);
             // the next segment's state (index clamped: the load is issued on every path, so that waits can count it)
-            load_state(sv + static_cast<size_t>(c >= 2 ? (c >> 1) - 1 : 0) * (N * N), b_sv, Sa);
+            fetch_saved(sv + static_cast<size_t>(c >= 2 ? (c >> 1) - 1 : 0) * SAVED_STATE_B, w, b_q, Sq);
         }
         __syncthreads();
     }
@@ -817,7 +843,7 @@ __global__ __launch_bounds__(NTG) void wkv6_bwd_fused(const ArgsG arg) {
     ArgsG a = arg;
     a.T = arg.T - t0 < arg.TB ? arg.T - t0 : arg.TB;
     const int nsegs = ((arg.T + L - 1) / L + 1) / 2;                // saved states of a whole sequence
-    a.saved = arg.saved + (bh * nsegs + t0 / (2 * L)) * (N * N);
+    a.saved = arg.saved + (bh * nsegs + t0 / (2 * L)) * SAVED_STATE_B;
     a.first = blk == 0;
     a.above = blk + 1 < arg.NB;
     if (arg.ds32 != nullptr) a.ds32 = arg.ds32 + bq * (N * N);
@@ -859,7 +885,7 @@ __global__ __launch_bounds__(256) void gu_block_sum(const int NB, const size_t n
 
 int launch_wkv6_bwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
                           const uint16_t* w, const uint16_t* u, const uint16_t* gy, uint16_t* gr, uint16_t* gk, uint16_t* gv,
-                          uint16_t* gw, uint16_t* gu, uint16_t* gs, const float* saved, int* flags,
+                          uint16_t* gw, uint16_t* gu, uint16_t* gs, const char* saved, int* flags,
                           int NB, int TB, float* blk_ds, float* blk_decay, float* ds32, float* gu32, uint16_t* gwp, float* gw32) {
     ArgsG a{};
     a.head_decay = gwp != nullptr; a.gwp = gwp;

@@ -50,6 +50,27 @@ constexpr float LOG2E = 1.44269504088896340736f;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
+// A state that the forward saves for the one-sweep backward (wkv6_fwd_f.hip -> wkv6_bwd_f.hip; the two-sweep forward
+// writes it for the heads it redoes): 64 x 64 values of 24 bits -- fp32 rounded to 16 significant bits, which is what the
+// backward's hi/lo bf16 operands keep of it anyway -- in 12 KB instead of 16: first the upper 16 bits of every value
+// (8 KB), then the next 8 bits (4 KB), both in the order in which the backward's state waves take them.  Value channel i,
+// key channel j: wave j / 16, lane 16 ((i / 4) % 4) + j % 16, element e = 4 (i / 16) + i % 4; a lane's sixteen elements
+// are 16 bytes of upper halves for e < 8, 16 bytes for e >= 8 (1 KB further on) and 16 low bytes.
+constexpr int SAVED_LO_B = 2 * N * N, SAVED_STATE_B = 3 * N * N;
+DEVINL uint32_t saved_round(const float x) { return __float_as_uint(x) + 0x80u; }    // bits 31..8 are what is kept
+// x: value channel i, key channels j .. j + 3 (j a multiple of 4: neighbours in a group of sixteen keys lie 16 bytes apart)
+DEVINL void saved_put4(char* state, const int i, const int j, const f32x4 x) {
+    const int w = j >> 4, lane = 16 * ((i >> 2) & 3) + (j & 15), e = 4 * (i >> 4) + (i & 3);
+    char* hi = state + ((2 * w + (e >> 3)) * 64 + lane) * 16 + 2 * (e & 7);
+    char* lo = state + SAVED_LO_B + (w * 64 + lane) * 16 + e;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const uint32_t q = saved_round(x[d]);
+        *reinterpret_cast<uint16_t*>(hi + 16 * d) = static_cast<uint16_t>(q >> 16);
+        *reinterpret_cast<uint8_t*>(lo + 16 * d) = static_cast<uint8_t>(q >> 8);
+    }
+}
+
 enum { W_HEAD = 0, W_EW = 1, W_RAW = 2 };   // wkv5: fp32 [H,N] (forward: decay eew, backward: ew = log decay);
                                              // wkv6: fp32 ew = -exp(w_raw) [B,T,C];  wkv6_state: raw bf16 w [B,T,C]
 
@@ -61,9 +82,9 @@ struct ArgsC {
     // SPLIT kernels only (see below)
     int cross;
     float* y32;
-    // when not null: [B*H][ceil(chunks / 2)][64][64] fp32, the state entering every even chunk, [value][key], for the
-    // one-sweep backward (wkv6_bwd_f.hip)
-    float* saved;
+    // when not null: [B*H][ceil(chunks / 2)] saved states (SAVED_STATE_B bytes each), the state entering every even chunk,
+    // for the one-sweep backward (wkv6_bwd_f.hip)
+    char* saved;
     // when not null: [B*H][8]; a workgroup runs only if one of its eight words is not zero (see ArgsB)
     const int* only_flagged;
 };

@@ -392,9 +392,9 @@ DEVINL void fwd_state(SmemF& S, const ArgsC& a, const int tid, const size_t base
         fetch_term(i);                                 // used by finish(i), one iteration from here
         if constexpr (SPLIT == 0) {
             if (a.saved != nullptr && !(i & 1)) {      // the state entering every even chunk, for the one-sweep backward
-                float* dst = a.saved + ((bh * ((nchunks + 1) / 2) + (i >> 1)) * N + i_own) * N + j0[0];
-                *reinterpret_cast<float4*>(dst) = make_float4(D[0][0], D[0][1], D[0][2], D[0][3]);
-                *reinterpret_cast<float4*>(dst + 4) = make_float4(D[1][0], D[1][1], D[1][2], D[1][3]);
+                char* dst = a.saved + (bh * ((nchunks + 1) / 2) + (i >> 1)) * SAVED_STATE_B;
+                saved_put4(dst, i_own, j0[0], D[0]);
+                saved_put4(dst, i_own, j0[1], D[1]);
             }
         }
         if (!exact) {
@@ -503,7 +503,7 @@ __global__ __launch_bounds__(NTF) void wkv6_fwd_ws(const ArgsC a) {
 
 int launch_wkv6_fwd_chunk(hipStream_t st, int wmode, int B, int T, int C, int H, const uint16_t* r,
                           const uint16_t* k, const uint16_t* v, const void* w, const uint16_t* u,
-                          const uint16_t* s0, uint16_t* y, float* saved, const int* only_flagged) {
+                          const uint16_t* s0, uint16_t* y, char* saved, const int* only_flagged) {
     ArgsC a{};
     a.T = T; a.C = C; a.H = H; a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.y = y; a.saved = saved;
     a.only_flagged = only_flagged;

@@ -57,7 +57,7 @@ struct ArgsQ {
     int T, C, H;
     const uint16_t *r, *k, *v, *w, *u, *s0;
     uint16_t* y;
-    float* saved;                  // [B*H][ceil(n/2)][64][64]: the state entering every even chunk, [value][key]
+    char* saved;                   // [B*H][ceil(n/2)] saved states (SAVED_STATE_B bytes each): the state entering every even chunk
     int* flags;                    // [B*H][8]
     // Sequences cut into NB blocks of TB tokens (a multiple of 64), one workgroup per (batch, head, block), for shapes with
     // fewer (batch, head) pairs than the chip has CUs.  Three launches: LOCAL = true leaves in blk_state the state that a
@@ -432,22 +432,36 @@ DEVINL void role_tiles(SmemQ& S, const ArgsQ& a, const int lane, const int w, co
     lds_t b_l = 4 * l16;
     // wave 0, 1, 2 -> quadrant (t, s) = (0,0) (1,0) (1,1); accumulator rows are s, lanes t
     const int ta = (w == 0) ? 0 : 1, tb = (w == 2) ? 1 : 0;
-    // wave 3: the state that the S waves left in LDS in the last iteration; a lane moves 16 bytes of a row, 4 rows a time
-    lds_t b_sr = ((lane >> 4) * SS + 4 * (lane & 15)) * 4;
-    float* __restrict__ sv = a.saved + (lane >> 4) * N + 4 * (lane & 15);
+    // wave 3: the state that the S waves left in LDS in the last iteration, into the saved-state format (wkv6_chunk.h): in
+    // step wq the lane gathers the sixteen elements of lane `lane` of the backward's state wave wq (value channels
+    // 16 (e / 4) + 4 g + e % 4 of key channel 16 wq + l16: 4-byte reads, a bank per lane) and stores 3 x 16 bytes
+    lds_t b_sr = (4 * g * SS + l16) * 4;
+    char* __restrict__ sv = a.saved + 16 * lane;
     __syncthreads();                       // iteration 0
 #pragma unroll 1
     for (int c = 0; c < nit - 1; ++c) {    // iteration c + 1
         opaque(b_nat); opaque(b_tw); opaque(b_l); opaque(b_sr);
         if (!LOCAL && w == 3 && c >= 2 && c - 2 < n && !(c & 1)) {
-            float* dst = sv + static_cast<size_t>((c - 2) >> 1) * (N * N);
+            char* dst = sv + static_cast<size_t>((c - 2) >> 1) * SAVED_STATE_B;
 #pragma unroll
-            for (int q = 0; q < 16; q += 4) {
-                f32x4 x[4];
+            for (int wq = 0; wq < 4; ++wq) {
+                uint32_t x[16];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) x[e] = lds_ld<f32x4>(sb + SST0 + (q + e) * (4 * SS * 4) + b_sr);
+                for (int e = 0; e < 16; ++e)
+                    x[e] = saved_round(lds_ld<float>(sb + SST0 + ((16 * (e >> 2) + (e & 3)) * SS + 16 * wq) * 4 + b_sr));
+                u32x4 hi[2], lo;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) *reinterpret_cast<f32x4*>(dst + (q + e) * (4 * N)) = x[e];
+                for (int q = 0; q < 4; ++q) {
+                    // byte selectors: 0..3 from the second operand, 4..7 from the first
+                    hi[0][q] = __builtin_amdgcn_perm(x[2 * q + 1], x[2 * q], 0x07060302u);
+                    hi[1][q] = __builtin_amdgcn_perm(x[8 + 2 * q + 1], x[8 + 2 * q], 0x07060302u);
+                    const uint32_t p01 = __builtin_amdgcn_perm(x[4 * q + 1], x[4 * q], 0x0c0c0501u);
+                    const uint32_t p23 = __builtin_amdgcn_perm(x[4 * q + 3], x[4 * q + 2], 0x0c0c0501u);
+                    lo[q] = __builtin_amdgcn_perm(p23, p01, 0x05040100u);
+                }
+                *reinterpret_cast<u32x4*>(dst + wq * 2048) = hi[0];
+                *reinterpret_cast<u32x4*>(dst + wq * 2048 + 1024) = hi[1];
+                *reinterpret_cast<u32x4*>(dst + SAVED_LO_B + wq * 1024) = lo;
             }
         }
         if (!LOCAL && c < n && w < 3) {
@@ -505,7 +519,7 @@ __global__ __launch_bounds__(NTQ) void wkv6_fwd_fused(const ArgsQ arg) {
     ArgsQ a = arg;
     a.T = arg.T - t0 < arg.TB ? arg.T - t0 : arg.TB;
     const int nseg = ((arg.T + L - 1) / L + 1) / 2;                 // saved states of a whole sequence
-    a.saved = arg.saved + (bh * nseg + t0 / (2 * L)) * (N * N);
+    a.saved = arg.saved + (bh * nseg + t0 / (2 * L)) * SAVED_STATE_B;
     if (arg.s32 != nullptr) a.s32 = arg.s32 + bq * (N * N);
     if (arg.blk_state != nullptr) { a.blk_state = arg.blk_state + bq * (N * N); a.blk_decay = arg.blk_decay + bq * N; }
     a.first_row = b == 0 && blk == 0;
@@ -545,7 +559,7 @@ __global__ __launch_bounds__(256) void wkv6_scan(const float* __restrict__ local
 }  // namespace
 
 int launch_wkv6_fwd_fused(hipStream_t st, int B, int T, int C, int H, const uint16_t* r, const uint16_t* k, const uint16_t* v,
-                          const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, float* saved, int* flags,
+                          const uint16_t* w, const uint16_t* u, const uint16_t* s0, uint16_t* y, char* saved, int* flags,
                           int NB, int TB, float* blk_state, float* blk_decay, float* s32, float* decay_out) {
     ArgsQ a{};
     const bool head_decay = decay_out != nullptr;
