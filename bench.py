@@ -26,10 +26,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X published HBM3E bandwidth
 FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X published dense fp32 matrix rate
-BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 matrix rate
-# depthwise_conv1d up to T = 768 forms every fp32 product from six bf16 matrix products (three bf16 terms per operand):
-# its ceiling in algorithmic (fp32) flops is a sixth of the bf16 rate
-BF3_PRODUCTS = 6
+F16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X published dense fp16 (and bf16) matrix rate
+# depthwise_conv1d up to T = 1024 forms every fp32 product from three fp16 matrix products (two fp16 terms per operand):
+# its ceiling in algorithmic (fp32) flops is a third of the fp16 rate
+H2_PRODUCTS = 3
 PREWARM_S = 0.3                # seconds of untimed load before the warmup steps (clock ramp)
 ALGO = "chunked"
 FLAGS = 0                      # RWKV_FLAG_SWEEPS when --algo sweeps: passed per call to the *_ex entry points
@@ -63,9 +63,9 @@ TRAFFIC_MEASURED = {
     # profiles/wkv4_reg_kernels_B32_T768_C768.md
     "wkv4_fwd_reg B32 T768": 152.5e6 + 78.4e6,
     "wkv4_bwd_reg + wkv4_batch_sum B32 T768": 227.2e6 + 151.7e6,
-    # profiles/timex_bf3_kernels_B32_C768_T768.md
-    "timex_conv_bf3 (forward)": 78.0e6 + 75.5e6,
-    "timex backward (timex_conv_bf3 + timex_gw_sum_bf3)": (78.0e6 + 75.5e6) + (151.2e6 + 2.4e6),
+    # profiles/timex_h2_kernels_B32_C768_T768.md
+    "timex_conv_h2 (forward)": 78.0e6 + 75.5e6,
+    "timex backward (timex_conv_h2 + timex_gw_sum_h2)": (78.0e6 + 75.5e6) + (151.2e6 + 2.4e6),
 }
 
 
@@ -481,11 +481,12 @@ def make_timex(dev):
 
     fwd_bytes = (C * T + 2 * B * C * T) * 4
     bwd_bytes = (2 * C * T + 3 * B * C * T) * 4
-    # The direct convolution does T (T + 1) / 2 multiply-adds per row and output array, in fp32: 64 flop per byte at
-    # T = 768, three times the ratio of the fp32 matrix peak to the HBM peak, so these kernels are bound by the former.
+    # The direct convolution does T (T + 1) / 2 multiply-adds per row and output array, in fp32: 95 flop per byte in the
+    # forward and 125 in the backward at T = 768, against a ridge of 104 (a third of the fp16 matrix rate over the HBM
+    # peak): the kernels sit at the ridge, and the matrix rate is the bound that is reported.
     conv_flops = B * C * T * (T + 1)
-    kernels = [("timex_conv_bf3 (forward)", lambda: call("rwkv_timex_forward", dev, w, k, x, 0.0, B, C, T), fwd_bytes, conv_flops),
-               ("timex backward (timex_conv_bf3 + timex_gw_sum_bf3)",
+    kernels = [("timex_conv_h2 (forward)", lambda: call("rwkv_timex_forward", dev, w, k, x, 0.0, B, C, T), fwd_bytes, conv_flops),
+               ("timex backward (timex_conv_h2 + timex_gw_sum_h2)",
                 lambda: call("rwkv_timex_backward_sum", dev, w, k, g, gw, gk, B, C, T), bwd_bytes, 2 * conv_flops)]
 
     def cpu_baseline(bs=4):
@@ -515,7 +516,7 @@ WORKLOADS = {
     "wkv4_b32": lambda dev: make_wkv4(dev, B=32, T=768),
     "timex": make_timex,
 }
-DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv6_b1": "bf16", "wkv5": "bf16", "wkv5_n128": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "wkv4_b32": "f32", "timex": "bf16x3 (every fp32 operand as three bf16 terms, fp32 accumulation)"}
+DTYPES = {"wkv6": "bf16", "wkv6_state": "bf16", "wkv6_b1": "bf16", "wkv5": "bf16", "wkv5_n128": "bf16", "wkv5_fp32": "f32", "wkv5a": "f32", "rwkv7": "bf16", "rwkv7_fp32": "f32", "wkv4": "f32", "wkv4_b32": "f32", "timex": "f16x2 (every fp32 operand as two fp16 terms, fp32 accumulation)"}
 
 
 def main():
@@ -613,9 +614,9 @@ def main():
                 "whole_step_frac_of_copy": round(step_gbps / copy_gbps, 4),
                 "hbm_read_GBps": round(read_gbps, 1), "hbm_write_GBps": round(write_gbps, 1)}
     if "TFLOPs" in dom:
-        peak = BF16_MFMA_PEAK_TFLOPS / BF3_PRODUCTS
+        peak = F16_MFMA_PEAK_TFLOPS / H2_PRODUCTS
         roofline = {"bound": "mfma", "kernel": dom["kernel"], "achieved": dom["TFLOPs"], "peak": round(peak, 1),
-                    "peak_is": "bf16 dense 2500 TFLOP/s / 6 bf16 products per fp32 product",
+                    "peak_is": "fp16 dense 2500 TFLOP/s / 3 fp16 products per fp32 product",
                     "unit": "TFLOP/s", "frac": round(dom["TFLOPs"] / peak, 4),
                     "frac_of_fp32_matrix_peak": round(dom["TFLOPs"] / FP32_MFMA_PEAK_TFLOPS, 4), "traffic": traffic,
                     "traffic_over_algorithmic": round(traffic / dom["algorithmic_bytes"], 3) if traffic else None,

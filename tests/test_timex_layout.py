@@ -1,6 +1,6 @@
-"""CPU: the LDS layout of the depthwise_conv1d kernels that use three-term bf16 products (csrc/timex.hip).
+"""CPU: the LDS layout of the depthwise_conv1d kernels that use two-term fp16 products (csrc/timex.hip).
 
-Those kernels fill the LDS to within a few KB of its 160 KiB and read the Toeplitz operand through two shifted copies of a
+Those kernels fill most of the 160 KiB of LDS and read the Toeplitz operand through two shifted copies of a
 line, one element past the last tap being a legal read.  The constants are taken from the source text and the index
 ranges are walked for every T the kernels accept: every read and write must stay inside its array, every multi-byte
 access must be aligned as the instruction needs, and the window a lane reads must be the taps the product needs."""
@@ -27,12 +27,12 @@ def _affine(fn):
     return int(m.group(1))
 
 
-T_MAX3 = _const("T_BF3_MAX")
+T_MAX3 = _const("T_H2_MAX")
 MROWS = _const("MROWS")
-GB3_ROWS = _const("GB3_ROWS")
-ROW_PAD = _affine("bf3_row_stride")
-_m = re.search(r"inline int bf3_line_len\(int T\) \{ return T \+ \(\(T & 32\) \? (\d+) : (\d+)\); \}", SRC)
-assert _m, "bf3_line_len"
+GH2_ROWS = _const("GH2_ROWS")
+ROW_PAD = _affine("h2_row_stride")
+_m = re.search(r"inline int h2_line_len\(int T\) \{ return T \+ \(\(T & 32\) \? (\d+) : (\d+)\); \}", SRC)
+assert _m, "h2_line_len"
 
 
 def line_len(T):
@@ -45,15 +45,16 @@ TS = [t for t in range(32, T_MAX3 + 1, 32)]
 @pytest.mark.parametrize("T", TS)
 def test_conv_planes_fit_and_are_aligned(T):
     rs, xl = T + ROW_PAD, line_len(T)
-    total = (3 * MROWS * rs + 6 * xl) * 2
+    total = (2 * MROWS * rs + 4 * xl) * 2 + 16 * 4            # two planes of rows, two planes x two copies of the line, the maxima
     assert total <= LDS_BYTES, (T, total)
+    assert ((2 * MROWS * rs + 4 * xl) * 2) % 4 == 0            # the maxima are floats
     assert (rs * 2) % 16 == 0                       # a lane's eight slots of a row: one aligned 16-byte read
-    assert (3 * MROWS * rs * 2) % 4 == 0 and (xl * 2) % 4 == 0     # the line copies start on dwords
+    assert (2 * MROWS * rs * 2) % 4 == 0 and (xl * 2) % 4 == 0     # the line copies start on dwords
     # the second copy sits 16 banks (of 4 bytes) away from the first, modulo 32 banks
     assert (xl // 2) % 32 == 16
 
 
-@pytest.mark.parametrize("T", [32, 64, 96, 384, 736, 768])
+@pytest.mark.parametrize("T", [32, 64, 96, 384, 736, 768, 992, 1024])
 @pytest.mark.parametrize("mirror", [False, True])
 def test_conv_tap_windows(T, mirror):
     """line[] as the kernel fills it, the two copies, and the window of every (output tile, input tile, lane, K block)."""
@@ -89,8 +90,15 @@ def test_conv_tap_windows(T, mirror):
 
 @pytest.mark.parametrize("T", TS)
 def test_gradient_planes_fit(T):
-    total = 6 * T * GB3_ROWS * 2 + 2 * T * 4
+    total = 4 * T * GH2_ROWS * 2 + (2 * T + 16) * 4 + 32 * GH2_ROWS * 2
     assert total <= LDS_BYTES, (T, total)
+    # the product loop fetches one tile pair past the last one: lag tile d, pair n = T/32 - d, of the last plane
+    nt, plane = T // 32, T * GH2_ROWS
+    for d in range(nt):
+        n = nt - d
+        last_g = ((32 * (d + n) + 31) * GH2_ROWS + 8 + 7 + plane) * 2 + 1                  # last byte read from the g planes
+        last_k = (2 * plane + (32 * n + 31) * GH2_ROWS + 8 + 7 + plane) * 2 + 1            # ... from the k planes
+        assert max(last_g, last_k) < total, (T, d)
     # the rotated cells of a group of four steps are a permutation, and a lane's read covers its own step
     for q in range(T // 4):
         assert sorted((e + q) & 3 for e in range(4)) == [0, 1, 2, 3]
