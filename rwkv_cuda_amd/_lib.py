@@ -37,10 +37,12 @@ HIPCC_FLAGS = [
 # The row-per-thread kernels for other head sizes (wkv_rows) keep a whole state row in registers; an instantiation that
 # no longer fits gave wrong results on the GPU (fp32 decay-gradient sweep at 128), so none may spill.
 # The wkv4 kernels that hold a segment's inputs in registers exist to avoid memory round trips: a spill defeats them.
+# The depthwise_conv1d matrix-core kernels hold the next unit's rows in registers across their product loops, which run at
+# the register limit: a spill there is scratch traffic in the innermost loop.
 # The one-sweep kernels let the compiler count their waits: a spill inside their loops would put scratch traffic between a
 # prefetch and its use (and a forward variant that spilled eleven registers gave wrong results): none may spill.
 SPILL_LIMIT = {"wkv6_bwd_fused": 0, "wkv6_fwd_fused": 0, "wkv6_fwd_ws": 0, "wkv6_bwd_a_ws": 0, "wkv6_bwd_b_wsILi0E": 3, "wkv6_bwd_b_wsILi1E": 1, "wkv6_bwd_b_wsILi2E": 1,
-               "wkv_rows": 0, "wkv4_fwd_reg": 0, "wkv4_bwd_reg": 0}
+               "wkv_rows": 0, "wkv4_fwd_reg": 0, "wkv4_bwd_reg": 0, "timex_conv_h2": 0, "timex_gw_sum_h2": 0}
 
 _lib = None
 

@@ -109,8 +109,8 @@ __global__ __launch_bounds__(1024) void timex_gw(const float* __restrict__ k, co
 // product of the lower-triangular Toeplitz matrix W[t][u] = wr[t-u] with the [T x 32] block of inputs, on 32 x 32 matrix
 // instructions (accumulator register v of lane l: row 8 (v/4) + 4 (l>>5) + (v&3), column l & 31).  The kernel row is
 // followed by zeros, so a tap of negative lag reads 0 and the diagonal block needs no mask.  Output tile o of 32 time
-// steps sums over input tiles 0..o (mirror: o..T/32-1); wave p takes tiles p and T/32-1-p (and p + 8, ...), which
-// balances the triangle.  256 persistent workgroups; a unit is one channel x 32 batch rows, and the next unit's rows are
+// steps sums over input tiles 0..o (mirror: o..T/32-1); the tiles are dealt to the eight waves so that their loads are
+// about equal.  256 persistent workgroups; a unit is one channel x 32 batch rows, and the next unit's rows are
 // loaded into registers under the products of the current one.
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr int MROWS = 32;              // batch rows per workgroup = columns of the product
@@ -139,7 +139,7 @@ constexpr int NCU = 256;               // workgroups of the persistent kernels: 
 // LDS: 2 x 32 x (T + 16) x 2 + 4 x (T + 96) x 2 + 64 bytes = 142 144 of 163 840 at T = 1024, the longest T this form takes.
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 constexpr int T_H2_MAX = 1024;
-constexpr int PFQ3 = MROWS * (T_H2_MAX / 4) / TXT;     // 16-byte pieces of a unit's rows per thread, at the longest T
+constexpr int T_H2_MID = 768;          // up to here a lane holds 3 pieces (16 bytes each) of each of its four rows while they are in flight, beyond 4
 __host__ __device__ inline int h2_row_stride(int T) { return T + 16; }           // elements; (T + 16) / 2 dwords = 8 or 24 mod 32
 __host__ __device__ inline int h2_line_len(int T) { return T + ((T & 32) ? 64 : 96); }    // half of it = 16 mod 32 dwords: the shifted copy sits 16 banks away
 __host__ __device__ inline size_t h2_lds_bytes(int T) {
@@ -153,6 +153,21 @@ DEVINL H2 split2(float x) {
     H2 r;
     r.h = __builtin_bit_cast(uint16_t, h);
     r.l = __builtin_bit_cast(uint16_t, l);
+    return r;
+}
+// the same for four elements times a power of two (the scaling is exact, so the remainder may be formed from x up in one
+// fused operation): four multiplications, four fused multiply-adds and four packed conversions
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+struct H2x4 { uint2 h, l; };
+DEVINL H2x4 split2x4(const float4& v, const float up) {
+    const f32x2 a = {v.x * up, v.y * up}, b = {v.z * up, v.w * up};
+    const f16x2 ha = __builtin_convertvector(a, f16x2), hb = __builtin_convertvector(b, f16x2);
+    const f32x2 ra = a - __builtin_convertvector(ha, f32x2), rb = b - __builtin_convertvector(hb, f32x2);
+    const f16x2 la = __builtin_convertvector(ra, f16x2), lb = __builtin_convertvector(rb, f16x2);
+    H2x4 r;
+    r.h = make_uint2(__builtin_bit_cast(uint32_t, ha), __builtin_bit_cast(uint32_t, hb));
+    r.l = make_uint2(__builtin_bit_cast(uint32_t, la), __builtin_bit_cast(uint32_t, lb));
     return r;
 }
 // 2^s with m 2^s in [2^14, 2^15) for a magnitude m (s = 0 for zero, subnormal or infinite m), and 2^-s
@@ -174,7 +189,8 @@ DEVINL float wave_max(float m) {
 }
 DEVINL float max_abs4(float m, const float4& v) { return fmaxf(fmaxf(m, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w))); }
 
-template <bool MIRROR>
+// NI: 16-byte pieces of a row per lane, 64 lanes a row: 3 up to T = 768, 4 beyond
+template <bool MIRROR, int NI>
 __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w, const float* __restrict__ in,
                                                       float* __restrict__ out, float eps, int B, int C, int T) {
     extern __shared__ float lds[];
@@ -182,33 +198,34 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
     uint16_t* rp = reinterpret_cast<uint16_t*>(lds);                    // [2][32][rs]
     uint16_t* al = rp + 2 * MROWS * rs;                                 // [2 planes][2 copies][xl]
     float* red = reinterpret_cast<float*>(al + 4 * xl);                 // [2][8]: every wave's largest magnitude of the rows / of the kernel row
-    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ln = lane & 31, kh = lane >> 5;
-    const int q4n = T >> 2, total = MROWS * q4n, nt = T >> 5;
+    const int q4n = T >> 2, nt = T >> 5;
     const int nbg = (B + MROWS - 1) / MROWS, nunits = C * nbg;
-    float4 x[PFQ3];
+    // Staging: wave wv takes rows 4 wv .. 4 wv + 3 of the unit, lane l the 16-byte pieces l, l + 64, ... of each: a row's
+    // address is wave-uniform, the rest is the lane number times 16 and a constant, in global memory and in LDS alike.
+    float4 x[4][NI];
     float wr[2];
-    // piece s of this thread is 16-byte piece idx = s TXT + tid of the unit's rows, (row, piece in the row) = (idx / q4n,
-    // idx % q4n): one division here, then steps of TXT
-    const int r_first = tid / q4n, q_first = tid - r_first * q4n, r_step = TXT / q4n, q_step = TXT - r_step * q4n;
     auto fetch_unit = [&](const int unit) __attribute__((always_inline)) {
         const int c = unit / nbg, b0 = (unit - c * nbg) * MROWS;
-        int r = r_first, q4 = q_first;
 #pragma unroll
-        for (int s = 0; s < PFQ3; ++s) {
-            const bool live = s * TXT + tid < total && b0 + r < B;
-            x[s] = *reinterpret_cast<const float4*>(in + (static_cast<size_t>(live ? b0 + r : b0) * C + c) * T + (live ? 4 * q4 : 0));
-            r += r_step; q4 += q_step;
-            if (q4 >= q4n) { q4 -= q4n; ++r; }
+        for (int rr = 0; rr < 4; ++rr) {
+            // (a row past the batch is read as the batch's last row and counts as zero later)
+            const int b = min(b0 + 4 * wv + rr, B - 1);
+            const float* row = in + (static_cast<size_t>(b) * C + c) * T;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) x[rr][i] = *reinterpret_cast<const float4*>(row + 4 * min(lane + 64 * i, q4n - 1));
         }
 #pragma unroll
         for (int s = 0; s < 2; ++s) wr[s] = w[static_cast<size_t>(c) * T + min(s * TXT + tid, T - 1)];
     };
-    // the largest magnitudes of the unit, this wave's part (pieces past the unit's end repeat real elements of the unit)
+    // the largest magnitudes of the unit, this wave's part (pieces past a row's end repeat its last piece)
     auto unit_max = [&]() __attribute__((always_inline)) {
         float mx = 0.f;
 #pragma unroll
-        for (int s = 0; s < PFQ3; ++s) mx = max_abs4(mx, x[s]);
+        for (int rr = 0; rr < 4; ++rr)
+#pragma unroll
+            for (int i = 0; i < NI; ++i) mx = max_abs4(mx, x[rr][i]);
         mx = wave_max(mx);
         const float mw = wave_max(fmaxf(fabsf(wr[0]), fabsf(wr[1])));
         if (lane == 0) { red[wv] = mx; red[8 + wv] = mw; }
@@ -221,18 +238,19 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
         for (int i = 0; i < TXW; ++i) { mx = fmaxf(mx, red[i]); mw = fmaxf(mw, red[8 + i]); }
         const Pow2 sx = scale_for(mx), sw = scale_for(mw);
         unscale = sx.down * sw.down;
-        int r = r_first, q4 = q_first;
 #pragma unroll
-        for (int s = 0; s < PFQ3; ++s) {
-            if (s * TXT + tid < total) {
-                const float4 v = b0 + r < B ? x[s] : make_float4(0.f, 0.f, 0.f, 0.f);
-                const H2 a0 = split2(v.x * sx.up), a1 = split2(v.y * sx.up), a2 = split2(v.z * sx.up), a3 = split2(v.w * sx.up);
-                uint16_t* d = rp + r * rs + 4 * q4;
-                *reinterpret_cast<uint2*>(d) = make_uint2(a0.h | (static_cast<uint32_t>(a1.h) << 16), a2.h | (static_cast<uint32_t>(a3.h) << 16));
-                *reinterpret_cast<uint2*>(d + MROWS * rs) = make_uint2(a0.l | (static_cast<uint32_t>(a1.l) << 16), a2.l | (static_cast<uint32_t>(a3.l) << 16));
+        for (int rr = 0; rr < 4; ++rr) {
+            const int r = 4 * wv + rr;
+            const float up = b0 + r < B ? sx.up : 0.f;
+            uint16_t* d = rp + r * rs + 4 * lane;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                if (lane + 64 * i < q4n) {
+                    const H2x4 y = split2x4(x[rr][i], up);
+                    *reinterpret_cast<uint2*>(d + 256 * i) = y.h;
+                    *reinterpret_cast<uint2*>(d + 256 * i + MROWS * rs) = y.l;
+                }
             }
-            r += r_step; q4 += q_step;
-            if (q4 >= q4n) { q4 -= q4n; ++r; }
         }
         // tap tau of the kernel row sits at line position tau (forward) or 31 + (T - 1 - tau) (mirror); the rest is zero
 #pragma unroll
@@ -264,61 +282,107 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
         store_unit(unit);
         __syncthreads();
         if (unit + static_cast<int>(gridDim.x) < nunits) fetch_unit(unit + gridDim.x);
-        for (int p = wv; 2 * p < nt; p += TXW) {
+        // Output tile ot sums over ot + 1 input tiles (mirror: T/32 - ot).  A wave works on two neighbouring output tiles at a
+        // time, because they share operands: a step is 16 input steps (K = 16), and with
+        //   forward: row t = 32 ot + ln, slot u: tap T-1-(t-u)            -> line[T-1-32 ot-ln + u],  rows[u]
+        //   mirror : row u = 32 ot + ln, slot t: lag 32 (it-ot) + slot-ln -> line[31-ln + 32 (it-ot) + slot],  rows[32 ot + slot]
+        // step j of both tiles takes the same rows (forward) or the same taps (mirror), and the other operand of the
+        // shorter tile at step j is that of the longer one (forward: tile ot + 1, mirror: tile ot) at step j + 2.  So a
+        // step reads one operand of each kind from LDS (4 KB per wave) for six matrix instructions instead of three: the
+        // "carried" operand C(j) enters the shorter tile at once and the longer tile two steps later, from registers.
+        // The pairs are dealt to the waves in the order of decreasing work, back and forth (waves 0..7, then 7..0, ...).
+        const int npairs = (nt + 1) >> 1;
 #pragma unroll 1
-            for (int side = 0; side < 2; ++side) {
-                const int ot = side == 0 ? p : nt - 1 - p;
-                if (side == 1 && ot == p) break;
-                f32x16 acc, acc1;                              // two chains: consecutive MFMAs are independent
+        for (int rd = 0; rd * TXW < npairs; ++rd) {
+            {
+                const int ts = rd * TXW + ((rd & 1) ? TXW - 1 - wv : wv);
+                if (ts >= npairs) break;
+                const int m = MIRROR ? ts : npairs - 1 - ts;
+                // the longer tile and the shorter one (absent when T/32 is odd and this is the last tile)
+                const bool both = 2 * m + 1 < nt;
+                const int tl = MIRROR ? 2 * m : (both ? 2 * m + 1 : 2 * m), tsh = MIRROR ? 2 * m + 1 : 2 * m;
+                const int n_long = 2 * (MIRROR ? nt - tl : tl + 1), n_short = n_long - 2;
+                f32x16 accl, accs;                             // the two tiles' instructions alternate: consecutive ones are independent
 #pragma unroll
-                for (int v = 0; v < 16; ++v) { acc[v] = 0.f; acc1[v] = 0.f; }
-                const int n_in = MIRROR ? nt - ot : ot + 1;
-                // A step is 16 input steps: the three products of one K block.  From one step to the next both operands move on
-                // by 16 elements: the tap window because the lag falls by 16 (forward) or grows by 16 (mirror) together with
-                // the slot base, the rows because the input step does.
-                //   forward: row t = 32 ot + ln, slot u: tap T-1-(t-u)            -> line[T-1-32 ot-ln + u]
-                //   mirror : row u = 32 ot + ln, slot t: lag 32 (it-ot) + slot-ln -> line[31-ln + 32 (it-ot) + slot]
-                const int start0 = (MIRROR ? 31 - ln : T - 1 - 32 * ot - ln) + 8 * kh;
+                for (int v = 0; v < 16; ++v) { accl[v] = 0.f; accs[v] = 0.f; }
+                const int start0 = (MIRROR ? 31 - ln : T - 1 - 32 * tl - ln) + 8 * kh;
                 const uint32_t* ap0 = reinterpret_cast<const uint32_t*>(al + (start0 & 1) * xl) + (start0 >> 1);
-                const uint16_t* bp0 = rp + ln * rs + (MIRROR ? 32 * ot : 0) + 8 * kh;
-                auto fetch = [&](int j2, f16x8 (&fa)[2], f16x8 (&fb)[2]) __attribute__((always_inline)) {
+                const uint16_t* bp0 = rp + ln * rs + (MIRROR ? 32 * tl : 0) + 8 * kh;
+                auto taps = [&](int j, f16x8 (&f)[2]) __attribute__((always_inline)) {
 #pragma unroll
                     for (int pq = 0; pq < 2; ++pq) {
-                        const uint32_t* a4 = ap0 + 8 * j2 + pq * xl;   // a plane is 2 xl elements = xl dwords
-                        fa[pq] = __builtin_bit_cast(f16x8, make_uint4(a4[0], a4[1], a4[2], a4[3]));
-                        fb[pq] = __builtin_bit_cast(f16x8, *reinterpret_cast<const uint4*>(bp0 + 16 * j2 + pq * MROWS * rs));
+                        const uint32_t* a4 = ap0 + 8 * j + pq * xl;    // a plane is 2 xl elements = xl dwords
+                        f[pq] = __builtin_bit_cast(f16x8, make_uint4(a4[0], a4[1], a4[2], a4[3]));
                     }
                 };
-                // (the large term goes to one accumulator, the two small ones to the other)
-                auto products = [&](const f16x8 (&fa)[2], const f16x8 (&fb)[2]) __attribute__((always_inline)) {
-                    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[0], fb[0], acc, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[0], fb[1], acc1, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[1], fb[0], acc1, 0, 0, 0);
+                auto rows = [&](int j, f16x8 (&f)[2]) __attribute__((always_inline)) {
+#pragma unroll
+                    for (int pq = 0; pq < 2; ++pq) f[pq] = __builtin_bit_cast(f16x8, *reinterpret_cast<const uint4*>(bp0 + 16 * j + pq * MROWS * rs));
                 };
-                // two register sets take turns; the step after the last one is fetched too and never used (it lies inside
-                // the workgroup's LDS: the line has at least 64 spare elements, the rows are followed by the line)
-                f16x8 a[2], b[2], a2[2], b2[2];
-                fetch(0, a, b);
-                // (the fences keep the reads of the next step in front of the products of this one: left to itself the
-                // scheduler sinks them behind the products and then waits for them at once)
-                for (int j2 = 0; j2 < 2 * n_in; j2 += 2) {
-                    fetch(j2 + 1, a2, b2);
-                    __builtin_amdgcn_sched_barrier(0);
-                    products(a, b);
-                    __builtin_amdgcn_sched_barrier(0);
-                    fetch(j2 + 2, a, b);
-                    __builtin_amdgcn_sched_barrier(0);
-                    products(a2, b2);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+                auto carried = [&](int j, f16x8 (&f)[2]) __attribute__((always_inline)) { if constexpr (MIRROR) rows(j, f); else taps(j, f); };
+                auto shared = [&](int j, f16x8 (&f)[2]) __attribute__((always_inline)) { if constexpr (MIRROR) taps(j, f); else rows(j, f); };
+                // term number `term` of the product of a carried and a shared operand: h h', h l', l h'
+                auto product = [&](f32x16& acc, const int term, const f16x8 (&cc)[2], const f16x8 (&sh)[2]) __attribute__((always_inline)) {
+                    const f16x8 (&fa)[2] = MIRROR ? sh : cc;
+                    const f16x8 (&fb)[2] = MIRROR ? cc : sh;
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[term == 2 ? 1 : 0], fb[term == 1 ? 1 : 0], acc, 0, 0, 0);
+                };
+                // (a last tile without a partner computes a second tile all the same and does not store it)
+                auto step = [&](const f16x8 (&cl)[2], const f16x8 (&cs)[2], const f16x8 (&sh)[2]) __attribute__((always_inline)) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[v] = fmaf(acc[v] + acc1[v], unscale, MIRROR ? 0.f : eps);
-                if (b0 + ln < B) {
-                    float* o = out + (static_cast<size_t>(b0 + ln) * C + c) * T + 32 * ot + 4 * kh;
+                    for (int term = 0; term < 3; ++term) { product(accl, term, cl, sh); product(accs, term, cs, sh); }
+                };
+                // Two pairs of carried operands, P and Q, change roles every two steps (the longer tile reads what the shorter
+                // one read two steps earlier), the shared operand alternates between two sets: no register is ever copied.
+                // Every read is issued one step ahead; the fences keep it in front of the products of the current step.
+                // (C(j) is asked for up to j = n_long - 1 only, S(j) likewise: nothing outside the tiles' own steps is read.)
+                f16x8 P[2][2], Q[2][2], se[2], so[2];
+                carried(0, P[0]); carried(1, P[1]); carried(n_long > 2 ? 2 : 1, Q[0]); shared(0, se);
+                int j = 0;
+                for (;;) {
+                    if (j >= n_short) break;
+                    carried(j + 3, Q[1]); shared(j + 1, so);
+                    __builtin_amdgcn_sched_barrier(0);
+                    step(P[0], Q[0], se);
+                    __builtin_amdgcn_sched_barrier(0);
+                    carried(min(j + 4, n_long - 1), P[0]); shared(j + 2, se);
+                    __builtin_amdgcn_sched_barrier(0);
+                    step(P[1], Q[1], so);
+                    __builtin_amdgcn_sched_barrier(0);
+                    j += 2;
+                    if (j >= n_short) {                         // (leave with the longer tile's operands in P, as the other way out does)
 #pragma unroll
-                    for (int v4 = 0; v4 < 4; ++v4)
-                        *reinterpret_cast<float4*>(o + 8 * v4) = make_float4(acc[4 * v4], acc[4 * v4 + 1], acc[4 * v4 + 2], acc[4 * v4 + 3]);
+                        for (int q = 0; q < 2; ++q) { P[0][q] = Q[0][q]; P[1][q] = Q[1][q]; }
+                        break;
+                    }
+                    carried(j + 3, P[1]); shared(j + 1, so);
+                    __builtin_amdgcn_sched_barrier(0);
+                    step(Q[0], P[0], se);
+                    __builtin_amdgcn_sched_barrier(0);
+                    carried(min(j + 4, n_long - 1), Q[0]); shared(j + 2, se);
+                    __builtin_amdgcn_sched_barrier(0);
+                    step(Q[1], P[1], so);
+                    __builtin_amdgcn_sched_barrier(0);
+                    j += 2;
                 }
+                // the last two steps belong to the longer tile alone
+                shared(n_short + 1, so);
+#pragma unroll
+                for (int term = 0; term < 3; ++term) product(accl, term, P[0], se);
+#pragma unroll
+                for (int term = 0; term < 3; ++term) product(accl, term, P[1], so);
+                auto put_tile = [&](f32x16& acc, const int ot) __attribute__((always_inline)) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[v] = fmaf(acc[v], unscale, MIRROR ? 0.f : eps);
+                    if (b0 + ln < B) {
+                        float* o = out + (static_cast<size_t>(b0 + ln) * C + c) * T + 32 * ot + 4 * kh;
+#pragma unroll
+                        for (int v4 = 0; v4 < 4; ++v4)
+                            *reinterpret_cast<float4*>(o + 8 * v4) = make_float4(acc[4 * v4], acc[4 * v4 + 1], acc[4 * v4 + 2], acc[4 * v4 + 3]);
+                    }
+                };
+                put_tile(accl, tl);
+                if (both) put_tile(accs, tsh);
             }
         }
         __syncthreads();               // every wave is done with this unit's rows
@@ -329,7 +393,7 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
 // sub-diagonal of M = G^T K (contraction over the batch), with the two-term fp16 products of timex_conv_h2.  Batch rows
 // are staged 16 at a time (a pass; both tensors scaled by a power of two of their own per pass): one
 // v_mfma_f32_32x32x16_f16 block per pair of tiles and product.  A wave owns whole lag tiles d (all tile pairs
-// (tt, tt-d) accumulate into the same registers; d and T/32-1-d together balance the triangle); no atomics, every fp32
+// (tt, tt-d) accumulate into the same registers); no atomics, every fp32
 // sum in a fixed order.  Both operands hold eight consecutive batch rows per lane, so the planes are kept transposed,
 // [step][16 rows] fp16: 32 bytes per step, and the 64 lanes of an operand read cover one contiguous KiB.
 // A finished tile's diagonals are summed in registers: lane p of a half-wave collects, for every row t it holds, the
@@ -419,11 +483,12 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__
         store_unit(u);
         __syncthreads();
         if (u + 1 < nmine) fetch_unit(u + 1);
-        for (int p = wv; 2 * p < nt; p += TXW) {
+        // (lag tile d has T/32 - d tile pairs: dealt to the waves like the output tiles of timex_conv_h2)
 #pragma unroll 1
-            for (int side = 0; side < 2; ++side) {
-                const int d = side == 0 ? p : nt - 1 - p;
-                if (side == 1 && d == p) break;
+        for (int rd = 0; rd * TXW < nt; ++rd) {
+            {
+                const int d = rd * TXW + ((rd & 1) ? TXW - 1 - wv : wv);
+                if (d >= nt) break;
                 f32x16 acc0, acc1;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.f;
@@ -519,9 +584,9 @@ using namespace rwkv;
 int launch_gk(void* stream, const float* w, const float* gwk, float* gk, int B, int C, int T) {
     if (use_mfma(B, T)) {
         const size_t lds = h2_lds_bytes(T);
-        if (int e = raise_lds_limit(timex_conv_h2<true>, lds)) return e;
-        hipLaunchKernelGGL(timex_conv_h2<true>, dim3(conv_grid(B, C)), dim3(TXT), lds,
-                           static_cast<hipStream_t>(stream), w, gwk, gk, 0.0f, B, C, T);
+        auto kernel = T <= T_H2_MID ? timex_conv_h2<true, T_H2_MID / 256> : timex_conv_h2<true, T_H2_MAX / 256>;
+        if (int e = raise_lds_limit(kernel, lds)) return e;
+        hipLaunchKernelGGL(kernel, dim3(conv_grid(B, C)), dim3(TXT), lds, static_cast<hipStream_t>(stream), w, gwk, gk, 0.0f, B, C, T);
     } else {
         const size_t lds = (static_cast<size_t>(BB + 1) * T + 4) * sizeof(float);
         if (int e = raise_lds_limit(timex_conv<true>, lds)) return e;
@@ -538,9 +603,9 @@ int rwkv_timex_forward(void* stream, const float* w, const float* k, float* x, f
     if (int e = check_ptrs({w, k, x})) return e;
     if (use_mfma(B, T)) {
         const size_t lds = h2_lds_bytes(T);
-        if (int e = raise_lds_limit(timex_conv_h2<false>, lds)) return e;
-        hipLaunchKernelGGL(timex_conv_h2<false>, dim3(conv_grid(B, C)), dim3(TXT), lds,
-                           static_cast<hipStream_t>(stream), w, k, x, eps, B, C, T);
+        auto kernel = T <= T_H2_MID ? timex_conv_h2<false, T_H2_MID / 256> : timex_conv_h2<false, T_H2_MAX / 256>;
+        if (int e = raise_lds_limit(kernel, lds)) return e;
+        hipLaunchKernelGGL(kernel, dim3(conv_grid(B, C)), dim3(TXT), lds, static_cast<hipStream_t>(stream), w, k, x, eps, B, C, T);
         return launch_status();
     }
     const size_t lds = (static_cast<size_t>(BB + 1) * T + 4) * sizeof(float);
