@@ -392,84 +392,110 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
 // Kernel gradient summed over the batch: gws[c][T-1-lag] = sum_b sum_t g[b,c,t] k[b,c,t-lag], i.e. the sum of the lag-th
 // sub-diagonal of M = G^T K (contraction over the batch), with the two-term fp16 products of timex_conv_h2.  Batch rows
 // are staged 16 at a time (a pass; both tensors scaled by a power of two of their own per pass): one
-// v_mfma_f32_32x32x16_f16 block per pair of tiles and product.  A wave owns whole lag tiles d (all tile pairs
-// (tt, tt-d) accumulate into the same registers); no atomics, every fp32
-// sum in a fixed order.  Both operands hold eight consecutive batch rows per lane, so the planes are kept transposed,
-// [step][16 rows] fp16: 32 bytes per step, and the 64 lanes of an operand read cover one contiguous KiB.
+// v_mfma_f32_32x32x16_f16 block per pair of tiles and product, K = the 16 batch rows.  A wave owns whole lag tiles d (all
+// tile pairs (d + i, i) accumulate into the same registers); no atomics, every fp32 sum in a fixed order.
+// The planes keep the tensors' own layout, [16 rows][T + 8] fp16 (staged like the convolution's rows: a wave takes two
+// rows of each tensor, wave-uniform row addresses, 8-byte LDS stores).  Both operands need the batch rows along K and a
+// lane per step: ds_read_b64_tr_b16 delivers exactly that -- within 16 lanes, four rows of 16 consecutive steps come back
+// with a lane per step and the four rows in its registers; two such reads are a lane's eight K slots.
+// Two neighbouring lag tiles per wave at a time: tile pair i of lag tile d + 1 takes the same k tile as pair i of lag
+// tile d, and its g tile is the one that lag tile d takes at pair i + 1.  So a pair reads one g tile and one k tile
+// from LDS for six matrix instructions; the g operand enters lag tile d + 1 at once and lag tile d one pair later.
 // A finished tile's diagonals are summed in registers: lane p of a half-wave collects, for every row t it holds, the
 // element of column (t - p) mod 32 (one ds_bpermute per accumulator register), which belongs to diagonal p if t >= p and
 // to diagonal p - 32 otherwise.
-// LDS: 2 x 2 x T x 32 + 2 T x 4 + 64 bytes + one tile of slack = 140 352 at T = 1024.
+// LDS: 2 x 2 x 16 x (T + 8) x 2 + 2 T x 4 + 64 bytes = 140 352 at T = 1024.
 constexpr int GH2_ROWS = 16;
-constexpr int GH2_SLACK = 32 * GH2_ROWS * 2;       // bytes: the product loop reads one tile past the last plane (and never uses it)
-__host__ __device__ inline size_t gw_h2_lds_bytes(int T) { return 4 * static_cast<size_t>(T) * GH2_ROWS * sizeof(uint16_t) + (2 * static_cast<size_t>(T) + 16) * sizeof(float) + GH2_SLACK; }
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef v4s __attribute__((address_space(3))) * lds_v4s_ptr;
+__host__ __device__ inline int gw_row_stride(int T) { return T + 8; }              // elements: rows stay 16-byte aligned
+__host__ __device__ inline size_t gw_h2_lds_bytes(int T) {
+    return 4 * static_cast<size_t>(GH2_ROWS) * gw_row_stride(T) * sizeof(uint16_t) + (2 * static_cast<size_t>(T) + 16) * sizeof(float);
+}
 
+// NI: 16-byte pieces of a row per lane, 64 lanes a row: 3 up to T = 768, 4 beyond
+template <int NI>
 __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__ k, const float* __restrict__ g,
                                                         float* __restrict__ gws, int B, int C, int T) {
     extern __shared__ float lds[];
-    uint16_t* gp = reinterpret_cast<uint16_t*>(lds);           // [2][T][16]
-    uint16_t* kp = gp + 2 * T * GH2_ROWS;                      // [2][T][16]
-    float* diag = reinterpret_cast<float*>(kp + 2 * T * GH2_ROWS);   // [T/32 lag tiles][64]: entry l of tile d is the sum for lag 32 d + l - 31
+    const int rsg = gw_row_stride(T);
+    const int plane = GH2_ROWS * rsg;                          // elements
+    uint16_t* gp = reinterpret_cast<uint16_t*>(lds);           // [2][16][rsg]
+    uint16_t* kp = gp + 2 * plane;                             // [2][16][rsg]
+    float* diag = reinterpret_cast<float*>(kp + 2 * plane);    // [T/32 lag tiles][64]: entry l of tile d is the sum for lag 32 d + l - 31
     float* red = diag + 2 * T;                                 // [2][8]: every wave's largest magnitude of g / of k in this pass
-    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    const int ln = lane & 31, kh = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ln = lane & 31, kh = lane >> 5, l16 = lane & 15;
     const int nt = T >> 5, q4n = T >> 2;
-    const int plane = T * GH2_ROWS;                            // elements
-
-    // Staging: thread (row r = tid & 15, piece q = tid >> 4, + 32 per round) reads 16 bytes of its row.  The bank of a
-    // step's cell depends on the step within its group of four and on the row only, so the cells of a group are stored
-    // rotated by the group number: step 4 q + e sits in cell 4 q + ((e + q) & 3), and the lanes of a store instruction
-    // (one e, many q) spread over all banks.  A reading lane applies the same rotation to its step, once.
-    constexpr int PF = GH2_ROWS * (T_H2_MAX / 4) / TXT;        // pieces per thread and tensor: 8
     const int npass = (B + GH2_ROWS - 1) / GH2_ROWS;
     const int nmine = (C > static_cast<int>(blockIdx.x) ? (C - 1 - static_cast<int>(blockIdx.x)) / static_cast<int>(gridDim.x) + 1 : 0) * npass;
-    const int r_own = tid & 15, q_own = tid >> 4;
-    float4 xg[PF], xk[PF];
+    // Staging: wave wv takes rows 2 wv and 2 wv + 1 of the pass, of both tensors; lane l the 16-byte pieces l, l + 64, ...
+    float4 xg[2][NI], xk[2][NI];
     auto fetch_unit = [&](const int u) __attribute__((always_inline)) {
         const int c = blockIdx.x + (u / npass) * gridDim.x, b0 = (u % npass) * GH2_ROWS;
 #pragma unroll
-        for (int s = 0; s < PF; ++s) {
-            const int q4 = s * 32 + q_own;
-            const bool live = q4 < q4n && b0 + r_own < B;
-            const size_t off = (static_cast<size_t>(live ? b0 + r_own : b0) * C + c) * T + (live ? 4 * q4 : 0);
-            xg[s] = *reinterpret_cast<const float4*>(g + off);
-            xk[s] = *reinterpret_cast<const float4*>(k + off);
-        }
-    };
-    auto put = [&](uint16_t* dst, const float4& x4, const int q4, const float up) __attribute__((always_inline)) {
-        const float xs[4] = {x4.x * up, x4.y * up, x4.z * up, x4.w * up};      // (up = 0 for a row past the batch)
+        for (int rr = 0; rr < 2; ++rr) {
+            // (a row past the batch is read as the batch's last row and counts as zero later)
+            const size_t row = (static_cast<size_t>(min(b0 + 2 * wv + rr, B - 1)) * C + c) * T;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const H2 y = split2(xs[e]);
-            uint16_t* d = dst + (4 * q4 + ((e + q4) & 3)) * GH2_ROWS + r_own;
-            d[0] = y.h; d[plane] = y.l;
+            for (int i = 0; i < NI; ++i) {
+                const int q4 = min(lane + 64 * i, q4n - 1);
+                xg[rr][i] = *reinterpret_cast<const float4*>(g + row + 4 * q4);
+                xk[rr][i] = *reinterpret_cast<const float4*>(k + row + 4 * q4);
+            }
         }
     };
-    // the largest magnitudes of the pass, this wave's part (pieces past the pass's end repeat real elements of it)
+    // the largest magnitudes of the pass, this wave's part (pieces past a row's end repeat its last piece)
     auto unit_max = [&]() __attribute__((always_inline)) {
         float mg = 0.f, mk = 0.f;
 #pragma unroll
-        for (int s = 0; s < PF; ++s) { mg = max_abs4(mg, xg[s]); mk = max_abs4(mk, xk[s]); }
+        for (int rr = 0; rr < 2; ++rr)
+#pragma unroll
+            for (int i = 0; i < NI; ++i) { mg = max_abs4(mg, xg[rr][i]); mk = max_abs4(mk, xk[rr][i]); }
         mg = wave_max(mg); mk = wave_max(mk);
         if (lane == 0) { red[wv] = mg; red[8 + wv] = mk; }
     };
     float unscale = 1.f;
     auto store_unit = [&](const int u) __attribute__((always_inline)) {
         const int b0 = (u % npass) * GH2_ROWS;
-        const bool real = b0 + r_own < B;
         float mg = 0.f, mk = 0.f;
 #pragma unroll
         for (int i = 0; i < TXW; ++i) { mg = fmaxf(mg, red[i]); mk = fmaxf(mk, red[8 + i]); }
         const Pow2 sg = scale_for(mg), sk = scale_for(mk);
         unscale = sg.down * sk.down;
-        // (the piece number is made opaque here: otherwise the LDS addresses of all 64 stores are computed once, outside
-        //  the loop over the units, and held in registers that the product loop needs)
-        int q_here = q_own;
-        asm volatile("" : "+v"(q_here));
 #pragma unroll
-        for (int s = 0; s < PF; ++s) {
-            const int q4 = s * 32 + q_here;
-            if (q4 < q4n) { put(gp, xg[s], q4, real ? sg.up : 0.f); put(kp, xk[s], q4, real ? sk.up : 0.f); }
+        for (int rr = 0; rr < 2; ++rr) {
+            const int r = 2 * wv + rr;
+            const bool real = b0 + r < B;
+            const float ug = real ? sg.up : 0.f, uk = real ? sk.up : 0.f;
+            uint16_t* dg = gp + r * rsg + 4 * lane;
+            uint16_t* dk = kp + r * rsg + 4 * lane;
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                if (lane + 64 * i < q4n) {
+                    const H2x4 yg = split2x4(xg[rr][i], ug), yk = split2x4(xk[rr][i], uk);
+                    *reinterpret_cast<uint2*>(dg + 256 * i) = yg.h;
+                    *reinterpret_cast<uint2*>(dg + 256 * i + plane) = yg.l;
+                    *reinterpret_cast<uint2*>(dk + 256 * i) = yk.h;
+                    *reinterpret_cast<uint2*>(dk + 256 * i + plane) = yk.l;
+                }
+            }
+        }
+    };
+    // operand of tile tt of a tensor: lane (ln, kh) <-> step 32 tt + ln, K slot 8 kh + e <-> batch row 8 kh + e.  Within its
+    // group of 16 lanes a lane points at [row 8 kh + (l16 >> 2)][step 32 tt + 16 (ln >> 4) + 4 (l16 & 3)]; the second read
+    // is four rows further on.
+    const uint32_t tr0 = static_cast<uint32_t>(reinterpret_cast<uintptr_t>((const __attribute__((address_space(3))) char*)gp))
+                       + 2u * static_cast<uint32_t>((8 * kh + (l16 >> 2)) * rsg + 16 * (ln >> 4) + 4 * (l16 & 3));
+    const uint32_t k_off = 2u * 2u * static_cast<uint32_t>(plane), row4 = 2u * 4u * static_cast<uint32_t>(rsg), pl_b = 2u * static_cast<uint32_t>(plane);
+    auto operand = [&](const uint32_t base, const int tt, f16x8 (&f)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int pq = 0; pq < 2; ++pq) {
+            const uint32_t a = base + 64u * static_cast<uint32_t>(tt) + pq * pl_b;
+            const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(a));
+            const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s_ptr)(a + row4));
+            const uint2 x = __builtin_bit_cast(uint2, lo), y = __builtin_bit_cast(uint2, hi);
+            f[pq] = __builtin_bit_cast(f16x8, make_uint4(x.x, x.y, y.x, y.y));
         }
     };
     if (nmine > 0) fetch_unit(0);
@@ -483,61 +509,69 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__
         store_unit(u);
         __syncthreads();
         if (u + 1 < nmine) fetch_unit(u + 1);
-        // (lag tile d has T/32 - d tile pairs: dealt to the waves like the output tiles of timex_conv_h2)
+        // lag tile d has T/32 - d tile pairs; the lag tiles go to the waves two at a time (2 m, 2 m + 1), in the order of
+        // decreasing work, back and forth (waves 0..7, then 7..0, ...)
+        const int npairs = (nt + 1) >> 1;
 #pragma unroll 1
-        for (int rd = 0; rd * TXW < nt; ++rd) {
-            {
-                const int d = rd * TXW + ((rd & 1) ? TXW - 1 - wv : wv);
-                if (d >= nt) break;
-                f32x16 acc0, acc1;
+        for (int rd = 0; rd * TXW < npairs; ++rd) {
+            const int m = rd * TXW + ((rd & 1) ? TXW - 1 - wv : wv);
+            if (m >= npairs) break;
+            const int dl = 2 * m, n = nt - dl;                 // the longer lag tile and its tile pairs; the shorter one, dl + 1, has n - 1
+            f32x16 accl, accs;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc0[v] = acc1[v] = 0.f;
-                // tile tt of g against tile tt - d of k: both move on by one tile (32 steps of 32 bytes) per iteration
-                const int cell = (ln & ~3) | (((ln & 3) + (ln >> 2)) & 3);     // where step ln of a tile sits (8 groups per tile)
-                const uint16_t* ga0 = gp + (32 * d + cell) * GH2_ROWS + 8 * kh;
-                const uint16_t* kb0 = kp + cell * GH2_ROWS + 8 * kh;
-                auto fetch = [&](int i, f16x8 (&fa)[2], f16x8 (&fb)[2]) __attribute__((always_inline)) {
+            for (int v = 0; v < 16; ++v) { accl[v] = 0.f; accs[v] = 0.f; }
+            // term number `term` of the product of a g and a k operand: h h', h l', l h'
+            auto product = [&](f32x16& acc, const int term, const f16x8 (&fa)[2], const f16x8 (&fb)[2]) __attribute__((always_inline)) {
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[term == 2 ? 1 : 0], fb[term == 1 ? 1 : 0], acc, 0, 0, 0);
+            };
+            auto both = [&](const f16x8 (&al_)[2], const f16x8 (&as_)[2], const f16x8 (&fb)[2]) __attribute__((always_inline)) {
 #pragma unroll
-                    for (int pq = 0; pq < 2; ++pq) {
-                        fa[pq] = __builtin_bit_cast(f16x8, *reinterpret_cast<const uint4*>(ga0 + i * 32 * GH2_ROWS + pq * plane));
-                        fb[pq] = __builtin_bit_cast(f16x8, *reinterpret_cast<const uint4*>(kb0 + i * 32 * GH2_ROWS + pq * plane));
-                    }
-                };
-                auto products = [&](const f16x8 (&fa)[2], const f16x8 (&fb)[2]) __attribute__((always_inline)) {
-                    acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[0], fb[0], acc0, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[0], fb[1], acc1, 0, 0, 0);
-                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[1], fb[0], acc1, 0, 0, 0);
-                };
-                const int n = nt - d;                          // tile pairs of this lag tile
-                // two register sets take turns; the pair after the last one is fetched too and never used (it lies inside the
-                // workgroup's LDS: the k planes follow the g planes, diag, the maxima and a tile of slack follow the k planes)
-                f16x8 a[2], b[2], a2[2], b2[2];
-                fetch(0, a, b);
-                for (int i = 0; i < n; i += 2) {
-                    fetch(i + 1, a2, b2);
-                    __builtin_amdgcn_sched_barrier(0);
-                    products(a, b);
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (i + 1 < n) {
-                        fetch(i + 2, a, b);
-                        __builtin_amdgcn_sched_barrier(0);
-                        products(a2, b2);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-                // accumulator v: t = 8 (v/4) + 4 kh + (v&3), u = ln, of tiles d apart
+                for (int term = 0; term < 3; ++term) product(accl, term, al_, fb);
+#pragma unroll
+                for (int term = 0; term < 3; ++term) product(accs, term, as_, fb);
+            };
+            auto last = [&](const f16x8 (&al_)[2], const f16x8 (&fb)[2]) __attribute__((always_inline)) {
+#pragma unroll
+                for (int term = 0; term < 3; ++term) product(accl, term, al_, fb);
+            };
+            // Pair i: the longer lag tile takes g tile dl + i, the shorter one g tile dl + 1 + i, both k tile i.  Two sets of g
+            // operands change roles every pair, two sets of k operands alternate; a set is read again as soon as its last
+            // product has been issued, one pair ahead of its use.
+            f16x8 P[2], Q[2], be[2], bo[2];
+            operand(tr0, dl, P); operand(tr0 + k_off, 0, be); operand(tr0, min(dl + 1, nt - 1), Q);
+            int i = 0;
+            for (;;) {
+                if (i >= n - 1) { last(P, be); break; }
+                operand(tr0 + k_off, i + 1, bo);
+                __builtin_amdgcn_sched_barrier(0);
+                both(P, Q, be);
+                __builtin_amdgcn_sched_barrier(0);
+                operand(tr0, min(dl + 2 + i, nt - 1), P);
+                ++i;
+                if (i >= n - 1) { last(Q, bo); break; }
+                operand(tr0 + k_off, i + 1, be);
+                __builtin_amdgcn_sched_barrier(0);
+                both(Q, P, bo);
+                __builtin_amdgcn_sched_barrier(0);
+                operand(tr0, min(dl + 2 + i, nt - 1), Q);
+                ++i;
+            }
+            // accumulator v: t = 8 (v/4) + 4 kh + (v&3), u = ln, of tiles d apart
+            auto diagonals = [&](const f32x16& acc, const int d) __attribute__((always_inline)) {
                 float pos = 0.f, neg = 0.f;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int t = 8 * (v >> 2) + 4 * kh + (v & 3);
-                    const float y = __shfl(acc0[v] + acc1[v], (kh << 5) | ((t - ln) & 31), 64);
+                    const float y = __shfl(acc[v], (kh << 5) | ((t - ln) & 31), 64);
                     if (t >= ln) pos += y; else neg += y;
                 }
                 pos += __shfl_xor(pos, 32, 64);
                 neg += __shfl_xor(neg, 32, 64);
                 if (kh == 0) diag[64 * d + 31 + ln] += pos * unscale;    // lag tile d belongs to this wave alone
                 else if (ln >= 1) diag[64 * d + ln - 1] += neg * unscale;
-            }
+            };
+            diagonals(accl, dl);
+            if (dl + 1 < nt) diagonals(accs, dl + 1);
         }
         __syncthreads();
         if (pass == npass - 1) {
@@ -634,8 +668,9 @@ int rwkv_timex_backward_sum(void* stream, const float* w, const float* k, const 
     if (int e = launch_gk(stream, w, gwk, gk, B, C, T)) return e;
     // (any batch size: a pass takes 16 rows, rows past the batch count as zero)
     const size_t lds_gw = gw_h2_lds_bytes(T);
-    if (int e = raise_lds_limit(timex_gw_sum_h2, lds_gw)) return e;
-    hipLaunchKernelGGL(timex_gw_sum_h2, dim3(C < NCU ? C : NCU), dim3(TXT), lds_gw, static_cast<hipStream_t>(stream), k, gwk, gw_sum, B, C, T);
+    auto kernel = T <= T_H2_MID ? timex_gw_sum_h2<T_H2_MID / 256> : timex_gw_sum_h2<T_H2_MAX / 256>;
+    if (int e = raise_lds_limit(kernel, lds_gw)) return e;
+    hipLaunchKernelGGL(kernel, dim3(C < NCU ? C : NCU), dim3(TXT), lds_gw, static_cast<hipStream_t>(stream), k, gwk, gw_sum, B, C, T);
     return launch_status();
 }
 

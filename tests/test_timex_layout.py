@@ -88,26 +88,32 @@ def test_conv_tap_windows(T, mirror):
                         assert got[i] == want, (T, mirror, ot, j2, ln, kh, i)
 
 
+GW_PAD = _affine("gw_row_stride")
+
+
 @pytest.mark.parametrize("T", TS)
 def test_gradient_planes_fit(T):
-    total = 4 * T * GH2_ROWS * 2 + (2 * T + 16) * 4 + 32 * GH2_ROWS * 2
+    """Planes [2 tensors][2 terms][16 rows][T + pad] fp16, the diagonal sums, the maxima; 8-byte stores of a lane's four
+    steps and the two transposing reads of an operand (rows 8 kh + (l16 >> 2) and four further on, 8 bytes at step
+    32 tile + 16 (ln >> 4) + 4 (l16 & 3)) stay inside their plane and are aligned."""
+    rsg = T + GW_PAD
+    plane = GH2_ROWS * rsg
+    total = 4 * plane * 2 + (2 * T + 16) * 4
     assert total <= LDS_BYTES, (T, total)
-    # the product loop fetches one tile pair past the last one: lag tile d, pair n = T/32 - d, of the last plane
-    nt, plane = T // 32, T * GH2_ROWS
-    for d in range(nt):
-        n = nt - d
-        last_g = ((32 * (d + n) + 31) * GH2_ROWS + 8 + 7 + plane) * 2 + 1                  # last byte read from the g planes
-        last_k = (2 * plane + (32 * n + 31) * GH2_ROWS + 8 + 7 + plane) * 2 + 1            # ... from the k planes
-        assert max(last_g, last_k) < total, (T, d)
-    # the rotated cells of a group of four steps are a permutation, and a lane's read covers its own step
-    for q in range(T // 4):
-        assert sorted((e + q) & 3 for e in range(4)) == [0, 1, 2, 3]
+    assert (rsg * 2) % 8 == 0 and (4 * plane * 2) % 4 == 0
     for tile in range(T // 32):
-        for ln in range(32):
-            cell = (ln & ~3) | (((ln & 3) + (ln >> 2)) & 3)
-            t = 32 * tile + ln
-            q, e = t >> 2, t & 3
-            assert 32 * tile + cell == 4 * q + ((e + q) & 3)
+        for lane in range(64):
+            ln, kh, l16 = lane & 31, lane >> 5, lane & 15
+            for extra in (0, 4):
+                row = 8 * kh + (l16 >> 2) + extra
+                step = 32 * tile + 16 * (ln >> 4) + 4 * (l16 & 3)
+                assert row < GH2_ROWS and step + 3 < T
+                assert ((row * rsg + step) * 2) % 8 == 0
+    # a lane's eight K slots are the batch rows 8 kh .. 8 kh + 7 of step 32 tile + ln: the 16 lanes of a group ask for four
+    # rows x 16 steps, and lane l16 gets step 16 (ln >> 4) + l16 of each
+    for lane in range(64):
+        ln, l16 = lane & 31, lane & 15
+        assert 16 * (ln >> 4) + l16 == ln
 
 
 def test_diagonal_sums_in_registers():
