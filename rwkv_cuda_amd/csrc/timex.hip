@@ -338,9 +338,10 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
                 // (C(j) is asked for up to j = n_long - 1 only, S(j) likewise: nothing outside the tiles' own steps is read.)
                 f16x8 P[2][2], Q[2][2], se[2], so[2];
                 carried(0, P[0]); carried(1, P[1]); carried(n_long > 2 ? 2 : 1, Q[0]); shared(0, se);
-                int j = 0;
-                for (;;) {
-                    if (j >= n_short) break;
+                // (one way into every loop body and one way out: with an exit in the middle of a body the compiler keeps two
+                //  versions of the accumulators and copies all 32 registers between them in every round, after waiting for
+                //  the matrix pipeline to drain)
+                auto block_pq = [&](const int j) __attribute__((always_inline)) {      // steps j, j + 1: longer tile from P, shorter from Q
                     carried(j + 3, Q[1]); shared(j + 1, so);
                     __builtin_amdgcn_sched_barrier(0);
                     step(P[0], Q[0], se);
@@ -349,12 +350,8 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
                     __builtin_amdgcn_sched_barrier(0);
                     step(P[1], Q[1], so);
                     __builtin_amdgcn_sched_barrier(0);
-                    j += 2;
-                    if (j >= n_short) {                         // (leave with the longer tile's operands in P, as the other way out does)
-#pragma unroll
-                        for (int q = 0; q < 2; ++q) { P[0][q] = Q[0][q]; P[1][q] = Q[1][q]; }
-                        break;
-                    }
+                };
+                auto block_qp = [&](const int j) __attribute__((always_inline)) {      // the same with the roles of P and Q exchanged
                     carried(j + 3, P[1]); shared(j + 1, so);
                     __builtin_amdgcn_sched_barrier(0);
                     step(Q[0], P[0], se);
@@ -363,7 +360,13 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
                     __builtin_amdgcn_sched_barrier(0);
                     step(Q[1], P[1], so);
                     __builtin_amdgcn_sched_barrier(0);
-                    j += 2;
+                };
+                int j = 0;
+                for (; j + 4 <= n_short; j += 4) { block_pq(j); block_qp(j + 2); }
+                if (j < n_short) {                              // (two steps left: afterwards the longer tile's operands are in Q)
+                    block_pq(j);
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) { P[0][q] = Q[0][q]; P[1][q] = Q[1][q]; }
                 }
                 // the last two steps belong to the longer tile alone
                 shared(n_short + 1, so);
@@ -525,10 +528,10 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__
                 acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[term == 2 ? 1 : 0], fb[term == 1 ? 1 : 0], acc, 0, 0, 0);
             };
             auto both = [&](const f16x8 (&al_)[2], const f16x8 (&as_)[2], const f16x8 (&fb)[2]) __attribute__((always_inline)) {
-#pragma unroll
-                for (int term = 0; term < 3; ++term) product(accl, term, al_, fb);
-#pragma unroll
-                for (int term = 0; term < 3; ++term) product(accs, term, as_, fb);
+                // (the longer tile's first two terms go first: the shorter tile's g operand is the read issued last)
+                product(accl, 0, al_, fb); product(accl, 1, al_, fb);
+                product(accs, 0, as_, fb); product(accl, 2, al_, fb);
+                product(accs, 1, as_, fb); product(accs, 2, as_, fb);
             };
             auto last = [&](const f16x8 (&al_)[2], const f16x8 (&fb)[2]) __attribute__((always_inline)) {
 #pragma unroll
@@ -539,23 +542,27 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__
             // product has been issued, one pair ahead of its use.
             f16x8 P[2], Q[2], be[2], bo[2];
             operand(tr0, dl, P); operand(tr0 + k_off, 0, be); operand(tr0, min(dl + 1, nt - 1), Q);
+            // (one way into the loop body and one way out, see timex_conv_h2)
             int i = 0;
-            for (;;) {
-                if (i >= n - 1) { last(P, be); break; }
+            for (; i + 2 <= n - 1; i += 2) {
                 operand(tr0 + k_off, i + 1, bo);
                 __builtin_amdgcn_sched_barrier(0);
                 both(P, Q, be);
                 __builtin_amdgcn_sched_barrier(0);
                 operand(tr0, min(dl + 2 + i, nt - 1), P);
-                ++i;
-                if (i >= n - 1) { last(Q, bo); break; }
-                operand(tr0 + k_off, i + 1, be);
+                operand(tr0 + k_off, i + 2, be);
                 __builtin_amdgcn_sched_barrier(0);
                 both(Q, P, bo);
                 __builtin_amdgcn_sched_barrier(0);
-                operand(tr0, min(dl + 2 + i, nt - 1), Q);
-                ++i;
+                operand(tr0, min(dl + 3 + i, nt - 1), Q);
             }
+            if (i < n - 1) {                                    // one pair with both tiles left, then the longer tile's last pair
+                operand(tr0 + k_off, i + 1, bo);
+                __builtin_amdgcn_sched_barrier(0);
+                both(P, Q, be);
+                __builtin_amdgcn_sched_barrier(0);
+                last(Q, bo);
+            } else last(P, be);
             // accumulator v: t = 8 (v/4) + 4 kh + (v&3), u = ln, of tiles d apart
             auto diagonals = [&](const f32x16& acc, const int d) __attribute__((always_inline)) {
                 float pos = 0.f, neg = 0.f;
