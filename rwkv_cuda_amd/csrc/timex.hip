@@ -434,18 +434,19 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__
     const int nmine = (C > static_cast<int>(blockIdx.x) ? (C - 1 - static_cast<int>(blockIdx.x)) / static_cast<int>(gridDim.x) + 1 : 0) * npass;
     // Staging: wave wv takes rows 2 wv and 2 wv + 1 of the pass, of both tensors; lane l the 16-byte pieces l, l + 64, ...
     float4 xg[2][NI], xk[2][NI];
-    auto fetch_unit = [&](const int u) __attribute__((always_inline)) {
-        const int c = blockIdx.x + (u / npass) * gridDim.x, b0 = (u % npass) * GH2_ROWS;
+    // (in NI parts, piece i of both rows and both tensors each: asked for all at once by every workgroup of the chip at the
+    //  same moment, the loads queue up in the memory system and the waves stall issuing them while the matrix cores wait;
+    //  the parts are spread over the products of the pass before)
+    const int nblk = gridDim.x;
+    auto fetch_part = [&](const int u, const int i) __attribute__((always_inline)) {
+        const int c = blockIdx.x + (u / npass) * nblk, b0 = (u % npass) * GH2_ROWS;
+        const int q4 = min(lane + 64 * i, q4n - 1);
 #pragma unroll
         for (int rr = 0; rr < 2; ++rr) {
             // (a row past the batch is read as the batch's last row and counts as zero later)
             const size_t row = (static_cast<size_t>(min(b0 + 2 * wv + rr, B - 1)) * C + c) * T;
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                const int q4 = min(lane + 64 * i, q4n - 1);
-                xg[rr][i] = *reinterpret_cast<const float4*>(g + row + 4 * q4);
-                xk[rr][i] = *reinterpret_cast<const float4*>(k + row + 4 * q4);
-            }
+            xg[rr][i] = *reinterpret_cast<const float4*>(g + row + 4 * q4);
+            xk[rr][i] = *reinterpret_cast<const float4*>(k + row + 4 * q4);
         }
     };
     // the largest magnitudes of the pass, this wave's part (pieces past a row's end repeat its last piece)
@@ -501,7 +502,11 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__
             f[pq] = __builtin_bit_cast(f16x8, make_uint4(x.x, x.y, y.x, y.y));
         }
     };
-    if (nmine > 0) fetch_unit(0);
+    if (nmine > 0) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) fetch_part(0, i);
+    }
+    static_assert(T_H2_MAX / 64 <= 2 * TXW, "a wave takes at most two pairs of lag tiles per pass");
 
     for (int u = 0; u < nmine; ++u) {
         const int pass = u % npass;
@@ -511,14 +516,12 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__
         __syncthreads();
         store_unit(u);
         __syncthreads();
-        if (u + 1 < nmine) fetch_unit(u + 1);
+        const bool more = u + 1 < nmine;
+        if (more) fetch_part(u + 1, 0);
         // lag tile d has T/32 - d tile pairs; the lag tiles go to the waves two at a time (2 m, 2 m + 1), in the order of
-        // decreasing work, back and forth (waves 0..7, then 7..0, ...)
+        // decreasing work, back and forth (waves 0..7, then 7..0): at most two pairs a wave
         const int npairs = (nt + 1) >> 1;
-#pragma unroll 1
-        for (int rd = 0; rd * TXW < npairs; ++rd) {
-            const int m = rd * TXW + ((rd & 1) ? TXW - 1 - wv : wv);
-            if (m >= npairs) break;
+        auto do_pair = [&](const int m, auto&& halfway) __attribute__((always_inline)) {
             const int dl = 2 * m, n = nt - dl;                 // the longer lag tile and its tile pairs; the shorter one, dl + 1, has n - 1
             f32x16 accl, accs;
 #pragma unroll
@@ -543,8 +546,7 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__
             f16x8 P[2], Q[2], be[2], bo[2];
             operand(tr0, dl, P); operand(tr0 + k_off, 0, be); operand(tr0, min(dl + 1, nt - 1), Q);
             // (one way into the loop body and one way out, see timex_conv_h2)
-            int i = 0;
-            for (; i + 2 <= n - 1; i += 2) {
+            auto two_pairs = [&](const int i) __attribute__((always_inline)) {
                 operand(tr0 + k_off, i + 1, bo);
                 __builtin_amdgcn_sched_barrier(0);
                 both(P, Q, be);
@@ -555,7 +557,12 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__
                 both(Q, P, bo);
                 __builtin_amdgcn_sched_barrier(0);
                 operand(tr0, min(dl + 3 + i, nt - 1), Q);
-            }
+            };
+            int i = 0;
+            const int half = ((n - 1) >> 1) & ~1;
+            for (; i < half; i += 2) two_pairs(i);
+            halfway();
+            for (; i + 2 <= n - 1; i += 2) two_pairs(i);
             if (i < n - 1) {                                    // one pair with both tiles left, then the longer tile's last pair
                 operand(tr0 + k_off, i + 1, bo);
                 __builtin_amdgcn_sched_barrier(0);
@@ -579,7 +586,12 @@ __global__ __launch_bounds__(TXT) void timex_gw_sum_h2(const float* __restrict__
             };
             diagonals(accl, dl);
             if (dl + 1 < nt) diagonals(accs, dl + 1);
-        }
+        };
+        if (wv < npairs) do_pair(wv, [&]() __attribute__((always_inline)) { if (more) fetch_part(u + 1, 1); });
+        else if (more) fetch_part(u + 1, 1);
+        if (more) fetch_part(u + 1, 2);
+        if (2 * TXW - 1 - wv < npairs) do_pair(2 * TXW - 1 - wv, []() __attribute__((always_inline)) {});
+        if constexpr (NI > 3) { if (more) fetch_part(u + 1, 3); }
         __syncthreads();
         if (pass == npass - 1) {
             const int c = blockIdx.x + (u / npass) * gridDim.x;
