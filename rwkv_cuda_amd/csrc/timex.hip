@@ -397,7 +397,7 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
 // are staged 16 at a time (a pass; both tensors scaled by a power of two of their own per pass): one
 // v_mfma_f32_32x32x16_f16 block per pair of tiles and product, K = the 16 batch rows.  A wave owns whole lag tiles d (all
 // tile pairs (d + i, i) accumulate into the same registers); no atomics, every fp32 sum in a fixed order.
-// The planes keep the tensors' own layout, [16 rows][T + 8] fp16 (staged like the convolution's rows: a wave takes two
+// The planes keep the tensors' own layout, [16 rows][T + 16 .. 112] fp16 (staged like the convolution's rows: a wave takes two
 // rows of each tensor, wave-uniform row addresses, 8-byte LDS stores).  Both operands need the batch rows along K and a
 // lane per step: ds_read_b64_tr_b16 delivers exactly that -- within 16 lanes, four rows of 16 consecutive steps come back
 // with a lane per step and the four rows in its registers; two such reads are a lane's eight K slots.
@@ -407,11 +407,13 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
 // A finished tile's diagonals are summed in registers: lane p of a half-wave collects, for every row t it holds, the
 // element of column (t - p) mod 32 (one ds_bpermute per accumulator register), which belongs to diagonal p if t >= p and
 // to diagonal p - 32 otherwise.
-// LDS: 2 x 2 x 16 x (T + 8) x 2 + 2 T x 4 + 64 bytes = 140 352 at T = 1024.
+// LDS: 2 x 2 x 16 x (T + 16) x 2 + 2 T x 4 + 64 bytes = 141 376 at T = 1024.
 constexpr int GH2_ROWS = 16;
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef v4s __attribute__((address_space(3))) * lds_v4s_ptr;
-__host__ __device__ inline int gw_row_stride(int T) { return T + 8; }              // elements: rows stay 16-byte aligned
+// elements; = 16 mod 128, i.e. 8 banks mod 64: the 16 lanes of a transposing read take four rows x four 8-byte pieces, and
+// with rows 8 banks apart the sixteen pieces fall on different banks
+__host__ __device__ inline int gw_row_stride(int T) { return T + ((144 - (T & 127)) & 127); }
 __host__ __device__ inline size_t gw_h2_lds_bytes(int T) {
     return 4 * static_cast<size_t>(GH2_ROWS) * gw_row_stride(T) * sizeof(uint16_t) + (2 * static_cast<size_t>(T) + 16) * sizeof(float);
 }

@@ -88,7 +88,12 @@ def test_conv_tap_windows(T, mirror):
                         assert got[i] == want, (T, mirror, ot, j2, ln, kh, i)
 
 
-GW_PAD = _affine("gw_row_stride")
+_g = re.search(r"inline int gw_row_stride\(int T\) \{ return T \+ \(\((\d+) - \(T & 127\)\) & 127\); \}", SRC)
+assert _g, "gw_row_stride"
+
+
+def gw_row_stride(T):
+    return T + ((int(_g.group(1)) - (T & 127)) & 127)
 
 
 @pytest.mark.parametrize("T", TS)
@@ -96,7 +101,8 @@ def test_gradient_planes_fit(T):
     """Planes [2 tensors][2 terms][16 rows][T + pad] fp16, the diagonal sums, the maxima; 8-byte stores of a lane's four
     steps and the two transposing reads of an operand (rows 8 kh + (l16 >> 2) and four further on, 8 bytes at step
     32 tile + 16 (ln >> 4) + 4 (l16 & 3)) stay inside their plane and are aligned."""
-    rsg = T + GW_PAD
+    rsg = gw_row_stride(T)
+    assert rsg >= T + 8
     plane = GH2_ROWS * rsg
     total = 4 * plane * 2 + (2 * T + 16) * 4
     assert total <= LDS_BYTES, (T, total)
@@ -109,6 +115,13 @@ def test_gradient_planes_fit(T):
                 step = 32 * tile + 16 * (ln >> 4) + 4 * (l16 & 3)
                 assert row < GH2_ROWS and step + 3 < T
                 assert ((row * rsg + step) * 2) % 8 == 0
+    # the sixteen 8-byte pieces that the 16 lanes of a group read at once fall on different banks (64 banks of 4 bytes)
+    for kh in range(2):
+        banks = set()
+        for l16 in range(16):
+            a = ((8 * kh + (l16 >> 2)) * rsg + 4 * (l16 & 3)) * 2
+            banks.update({(a // 4) % 64, (a // 4 + 1) % 64})
+        assert len(banks) == 32, (T, kh)
     # a lane's eight K slots are the batch rows 8 kh .. 8 kh + 7 of step 32 tile + ln: the 16 lanes of a group ask for four
     # rows x 16 steps, and lane l16 gets step 16 (ln >> 4) + l16 of each
     for lane in range(64):
