@@ -206,18 +206,22 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
     // address is wave-uniform, the rest is the lane number times 16 and a constant, in global memory and in LDS alike.
     float4 x[4][NI];
     float wr[2];
-    auto fetch_unit = [&](const int unit) __attribute__((always_inline)) {
+    // (in NI parts, piece i of the four rows each, the kernel row with part 0: asked for all at once by every workgroup of
+    //  the chip at the same moment, the loads queue up in the memory system and the waves stall issuing them; the parts
+    //  are spread over the products of the unit before)
+    auto fetch_part = [&](const int unit, const int i) __attribute__((always_inline)) {
         const int c = unit / nbg, b0 = (unit - c * nbg) * MROWS;
+        const int q4 = min(lane + 64 * i, q4n - 1);
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
             // (a row past the batch is read as the batch's last row and counts as zero later)
             const int b = min(b0 + 4 * wv + rr, B - 1);
-            const float* row = in + (static_cast<size_t>(b) * C + c) * T;
-#pragma unroll
-            for (int i = 0; i < NI; ++i) x[rr][i] = *reinterpret_cast<const float4*>(row + 4 * min(lane + 64 * i, q4n - 1));
+            x[rr][i] = *reinterpret_cast<const float4*>(in + (static_cast<size_t>(b) * C + c) * T + 4 * q4);
         }
+        if (i == 0) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s) wr[s] = w[static_cast<size_t>(c) * T + min(s * TXT + tid, T - 1)];
+            for (int s = 0; s < 2; ++s) wr[s] = w[static_cast<size_t>(c) * T + min(s * TXT + tid, T - 1)];
+        }
     };
     // the largest magnitudes of the unit, this wave's part (pieces past a row's end repeat its last piece)
     auto unit_max = [&]() __attribute__((always_inline)) {
@@ -273,7 +277,11 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
     for (int i = tid; i < 4 * xl; i += TXT) al[i] = 0;
     __syncthreads();
     int unit = blockIdx.x;
-    if (unit < nunits) fetch_unit(unit);
+    if (unit < nunits) {
+#pragma unroll
+        for (int i = 0; i < NI; ++i) fetch_part(unit, i);
+    }
+    static_assert(T_H2_MAX / 64 <= 2 * TXW, "a wave takes at most two pairs of tiles per unit");
 
     for (; unit < nunits; unit += gridDim.x) {
         const int c = unit / nbg, b0 = (unit - c * nbg) * MROWS;
@@ -281,7 +289,9 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
         __syncthreads();
         store_unit(unit);
         __syncthreads();
-        if (unit + static_cast<int>(gridDim.x) < nunits) fetch_unit(unit + gridDim.x);
+        const int next = unit + static_cast<int>(gridDim.x);
+        const bool more = next < nunits;
+        if (more) fetch_part(next, 0);
         // Output tile ot sums over ot + 1 input tiles (mirror: T/32 - ot).  A wave works on two neighbouring output tiles at a
         // time, because they share operands: a step is 16 input steps (K = 16), and with
         //   forward: row t = 32 ot + ln, slot u: tap T-1-(t-u)            -> line[T-1-32 ot-ln + u],  rows[u]
@@ -290,13 +300,11 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
         // shorter tile at step j is that of the longer one (forward: tile ot + 1, mirror: tile ot) at step j + 2.  So a
         // step reads one operand of each kind from LDS (4 KB per wave) for six matrix instructions instead of three: the
         // "carried" operand C(j) enters the shorter tile at once and the longer tile two steps later, from registers.
-        // The pairs are dealt to the waves in the order of decreasing work, back and forth (waves 0..7, then 7..0, ...).
+        // The pairs are dealt to the waves in the order of decreasing work, back and forth (waves 0..7, then 7..0): at most
+        // two pairs a wave.
         const int npairs = (nt + 1) >> 1;
-#pragma unroll 1
-        for (int rd = 0; rd * TXW < npairs; ++rd) {
+        auto do_pair = [&](const int ts, auto&& halfway) __attribute__((always_inline)) {
             {
-                const int ts = rd * TXW + ((rd & 1) ? TXW - 1 - wv : wv);
-                if (ts >= npairs) break;
                 const int m = MIRROR ? ts : npairs - 1 - ts;
                 // the longer tile and the shorter one (absent when T/32 is odd and this is the last tile)
                 const bool both = 2 * m + 1 < nt;
@@ -362,6 +370,9 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
                     __builtin_amdgcn_sched_barrier(0);
                 };
                 int j = 0;
+                const int half = (n_short >> 1) & ~3;
+                for (; j < half; j += 4) { block_pq(j); block_qp(j + 2); }
+                halfway();
                 for (; j + 4 <= n_short; j += 4) { block_pq(j); block_qp(j + 2); }
                 if (j < n_short) {                              // (two steps left: afterwards the longer tile's operands are in Q)
                     block_pq(j);
@@ -387,7 +398,12 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
                 put_tile(accl, tl);
                 if (both) put_tile(accs, tsh);
             }
-        }
+        };
+        if (wv < npairs) do_pair(wv, [&]() __attribute__((always_inline)) { if (more) fetch_part(next, 1); });
+        else if (more) fetch_part(next, 1);
+        if (more) fetch_part(next, 2);
+        if (2 * TXW - 1 - wv < npairs) do_pair(2 * TXW - 1 - wv, []() __attribute__((always_inline)) {});
+        if constexpr (NI > 3) { if (more) fetch_part(next, 3); }
         __syncthreads();               // every wave is done with this unit's rows
     }
 }
