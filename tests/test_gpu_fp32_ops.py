@@ -96,7 +96,8 @@ def test_wkv4_extreme_k_stays_finite(lib):
 # T % 32 == 0 up to 1024 with 8 or more batch rows runs on the matrix cores with two-term fp16 products (one tile, a
 # ragged last group of 32 rows, a last pass of one row for the batch-summed gradient, the longest T)
 @pytest.mark.parametrize("B,C,T", [(3, 5, 64), (9, 2, 4), (40, 3, 96), (17, 2, 1024), (32, 768, 768), (3, 2, 1100), (2, 3, 4096),
-                                   (8, 3, 32), (9, 2, 64), (33, 2, 736), (17, 5, 768), (48, 2, 128), (16, 1, 800)])
+                                   (8, 3, 32), (9, 2, 64), (33, 2, 736), (17, 5, 768), (48, 2, 128), (16, 1, 800),
+                                   (9, 3, 992), (40, 2, 1024), (8, 2, 96), (70, 1, 160)])
 def test_timex(lib, B, C, T):
     print(f"\ntimex B={B} C={C} T={T}", flush=True)
     w, k, g = synth.timex_inputs(B, C, T, seed=23)
