@@ -347,7 +347,7 @@ __global__ __launch_bounds__(TXT) void timex_conv_h2(const float* __restrict__ w
                 f16x8 P[2][2], Q[2][2], se[2], so[2];
                 carried(0, P[0]); carried(1, P[1]); carried(n_long > 2 ? 2 : 1, Q[0]); shared(0, se);
                 // (one way into every loop body and one way out: with an exit in the middle of a body the compiler keeps two
-                //  versions of the accumulators and copies all 32 registers between them in every round, after waiting for
+                //  versions of the accumulators and copies all 32 registers between them in every pass of the loop, after waiting for
                 //  the matrix pipeline to drain)
                 auto block_pq = [&](const int j) __attribute__((always_inline)) {      // steps j, j + 1: longer tile from P, shorter from Q
                     carried(j + 3, Q[1]); shared(j + 1, so);
